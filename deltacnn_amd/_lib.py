@@ -1,0 +1,77 @@
+"""ctypes binding of libdeltacnn_hip.so (declared in include/deltacnn_hip.h).
+
+The library is the only compute path of this package: if it is missing, loading
+raises instead of falling back to anything else.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdeltacnn_hip.so")
+
+DC_F32, DC_F16 = 0, 1
+ERROR_NAMES = {0: "DC_OK", -1: "DC_ERR_DTYPE", -2: "DC_ERR_SHAPE", -3: "DC_ERR_UNSUPPORTED",
+               -4: "DC_ERR_NULL", -5: "DC_ERR_ALIGN", -6: "DC_ERR_LAUNCH"}
+
+
+class Geometry(ctypes.Structure):
+    """struct dc_geometry."""
+    _fields_ = [(n, c_int32) for n in (
+        "batch", "in_h", "in_w", "in_c", "out_h", "out_w", "out_c", "kernel_h", "kernel_w",
+        "stride_h", "stride_w", "dilation_h", "dilation_w", "pad_top", "pad_left", "pad_bottom",
+        "pad_right", "groups")]
+
+
+_P = c_void_p
+_G = POINTER(Geometry)
+_SIGNATURES = {
+    "dc_version": (c_char_p, []),
+    "dc_last_error": (c_char_p, []),
+    "dc_sparsify": (c_int, [_P, _P, _P, _P, c_float, c_int32, c_int32, c_int, _P]),
+    "dc_activate_truncate": (c_int, [_P, _P, _P, _P, c_float, c_int, c_int, c_int32, c_int32, c_int, _P]),
+    "dc_conv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),
+    "dc_conv_act": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_float, c_int, c_int, c_int, _P]),
+    "dc_packed_filter_bytes": (c_int64, [_G, c_int, c_int]),
+    "dc_pack_filter": (c_int, [_G, _P, _P, c_int, c_int, _P]),
+    "dc_deconv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),
+    "dc_pool": (c_int, [_G, _P, _P, _P, _P, _P, c_int, c_int, _P]),
+    "dc_add": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_float, c_float, c_int, c_int, c_int32, c_int32, c_int, _P]),
+    "dc_add_to_dense": (c_int, [_P, _P, _P, c_int, c_int32, c_int32, c_int, _P]),
+    "dc_upsample": (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int32, c_int32, c_int32, c_int, _P]),
+    "dc_concat": (c_int, [_P, _P, _P, _P, _P, _P, c_int32, c_int32, c_int32, c_int, _P]),
+    "dc_mul_add": (c_int, [_P, _P, _P, _P, _P, _P, c_int32, c_int32, c_int, _P]),
+}
+
+_lib = None
+
+
+class DeltaCNNError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"{ERROR_NAMES.get(code, code)}: {message}")
+        self.code = code
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python deltacnn_amd/csrc/build.py` "
+            "(hipcc --offload-arch=gfx950). There is no fallback path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(code: int) -> None:
+    if code != 0:
+        raise DeltaCNNError(code, load().dc_last_error().decode())

@@ -1,0 +1,132 @@
+// Shared device helpers and the internal launch interface of libdeltacnn_hip.so.
+// gfx950 only: wavefronts are 64 lanes wide and every kernel here relies on that.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/deltacnn_hip.h"
+
+namespace dc {
+
+constexpr int WAVE = 64;
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+// N elements of T moved with one naturally aligned load / store.
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Vec {
+    T v[N];
+};
+
+template <typename T, int N>
+__device__ __forceinline__ Vec<T, N> vload(const T *p) {
+    return *reinterpret_cast<const Vec<T, N> *>(p);
+}
+template <typename T, int N>
+__device__ __forceinline__ void vstore(T *p, const Vec<T, N> &x) {
+    *reinterpret_cast<Vec<T, N> *>(p) = x;
+}
+
+// Elements per 16-byte vector.
+template <typename T>
+struct Vec16 {
+    static constexpr int N = 16 / sizeof(T);
+};
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
+
+__device__ __forceinline__ uint64_t ballot(bool p) { return __ballot(p); }
+
+// Does any lane of this lane's aligned group of `g` lanes (g a power of two) hold `p`?
+__device__ __forceinline__ bool group_any(bool p, int g) {
+    uint64_t b = ballot(p);
+    if (g >= WAVE) return b != 0;
+    int lo = lane_id() & ~(g - 1);
+    return ((b >> lo) & ((1ull << g) - 1ull)) != 0;
+}
+
+// Rank of this lane among the lanes with `p` set, and their count.
+__device__ __forceinline__ int wave_rank(bool p, int &count) {
+    uint64_t b = ballot(p);
+    count = __popcll(b);
+    return __popcll(b & ((1ull << lane_id()) - 1ull));
+}
+
+// Activation functions, one IEEE operation at a time in the tensor's own type so that
+// results are bit-identical to evaluating the same expression op by op on the host.
+template <typename T>
+__device__ __forceinline__ T act_apply(T x, int act) {
+    switch (act) {
+        case DC_ACT_RELU: return x < T(0) ? T(0) : x;
+        case DC_ACT_RELU6: return x < T(0) ? T(0) : (x > T(6) ? T(6) : x);
+        case DC_ACT_LEAKY: return x < T(0) ? x * T(0.1f) : x;
+        case DC_ACT_SIGMOID: return T(1.0f / (1.0f + __expf(-float(x))));
+        case DC_ACT_SWISH: return T(float(x) / (1.0f + __expf(-float(x))));
+        default: return x;
+    }
+}
+
+// Fused multiply-add with a single rounding in the operand type.
+__device__ __forceinline__ float fma_t(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ half_t fma_t(half_t a, half_t b, half_t c) {
+    return __builtin_fmaf16(a, b, c);
+}
+
+template <typename T>
+__device__ __forceinline__ T tabs(T x) {
+    return x < T(0) ? -x : x;
+}
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline int pow2_ceil(int v) {
+    int p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+
+// ---- launch interface (one function per operator; arguments already validated) ----
+hipError_t launch_sparsify(const void *in, void *prev, void *delta, int32_t *mask, float thr,
+                           int32_t P, int32_t C, int dtype, hipStream_t s);
+hipError_t launch_activate_truncate(void *delta, void *prev, void *trunc, int32_t *mask, float thr,
+                                    int act, int mode, int32_t P, int32_t C, int dtype,
+                                    hipStream_t s);
+hipError_t launch_add(const void *a, const void *b, void *prev, void *out, const int32_t *ma,
+                      const int32_t *mb, int32_t *mo, float wa, float wb, int act, int dense_out,
+                      int32_t P, int32_t C, int dtype, hipStream_t s);
+hipError_t launch_add_to_dense(void *a, void *b, const int32_t *ma, int act, int32_t P, int32_t C,
+                               int dtype, hipStream_t s);
+hipError_t launch_upsample(const void *in, void *out, const int32_t *mi, int32_t *mo, int32_t B,
+                           int32_t H, int32_t W, int32_t C, int32_t scale, int dtype,
+                           hipStream_t s);
+hipError_t launch_concat(const void *a, const void *b, void *out, const int32_t *ma,
+                         const int32_t *mb, int32_t *mo, int32_t P, int32_t Ca, int32_t Cb,
+                         int dtype, hipStream_t s);
+hipError_t launch_mul_add(const void *in, const int32_t *mask, void *out, int32_t *mo,
+                          const void *scale, const void *bias, int32_t P, int32_t C, int dtype,
+                          hipStream_t s);
+
+struct ActEpilogue {  // optional activation/truncation fused behind a convolution
+    void *prev;
+    void *trunc;
+    float thr;
+    int act;
+    int mode;
+};
+
+hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
+                       const void *packed, const void *bias, void *out, const int32_t *mask,
+                       int32_t *out_mask, int dtype, bool transposed, const ActEpilogue *epi,
+                       hipStream_t s);
+hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *packed, int dtype,
+                              bool transposed, hipStream_t s);
+int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed);
+hipError_t launch_pool(const dc_geometry &g, const void *in, const void *prev, void *out,
+                       const int32_t *mask, int32_t *out_mask, int mode, int dtype, hipStream_t s);
+
+}  // namespace dc

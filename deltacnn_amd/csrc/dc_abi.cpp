@@ -1,0 +1,332 @@
+// extern "C" surface of libdeltacnn_hip.so: argument validation, error reporting, dispatch.
+// Every check runs before the first HIP call, so bad arguments are reported without a GPU.
+#include <cstdarg>
+#include <cstdio>
+
+#include "common.hpp"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int finish(hipError_t e, const char *what) {
+    if (e == hipSuccess) return DC_OK;
+    return fail(DC_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+inline size_t esize(int dtype) { return dtype == DC_F32 ? 4 : 2; }
+
+#define DC_REQUIRE_DTYPE(fn) \
+    if (dtype != DC_F32 && dtype != DC_F16) return fail(DC_ERR_DTYPE, fn ": unsupported dtype %d", dtype)
+#define DC_REQUIRE_PTR(fn, p) \
+    if ((p) == nullptr) return fail(DC_ERR_NULL, fn ": " #p " is NULL")
+#define DC_REQUIRE_ALIGNED(fn, p, a) \
+    if ((p) != nullptr && (reinterpret_cast<uintptr_t>(p) % (a)) != 0) \
+        return fail(DC_ERR_ALIGN, fn ": " #p " is not aligned to %d bytes", int(a))
+
+int check_pc(const char *fn, int32_t pixels, int32_t channels) {
+    if (pixels <= 0 || channels <= 0)
+        return fail(DC_ERR_SHAPE, "%s: pixels=%d channels=%d must be positive", fn, pixels, channels);
+    if ((int64_t)pixels * channels >= (int64_t)1 << 40)
+        return fail(DC_ERR_SHAPE, "%s: tensor too large", fn);
+    if (pixels > (1 << 29))
+        return fail(DC_ERR_SHAPE, "%s: pixels=%d exceeds 2^29", fn, pixels);
+    return DC_OK;
+}
+
+int check_geometry(const char *fn, const dc_geometry *g, bool transposed, bool pooling) {
+    if (g == nullptr) return fail(DC_ERR_NULL, "%s: geometry is NULL", fn);
+    if (g->batch <= 0 || g->in_h <= 0 || g->in_w <= 0 || g->in_c <= 0 || g->out_h <= 0 ||
+        g->out_w <= 0 || g->out_c <= 0)
+        return fail(DC_ERR_SHAPE, "%s: non-positive dimension", fn);
+    if (g->in_h > 32767 || g->in_w > 32767 || g->out_h > 32767 || g->out_w > 32767 ||
+        g->batch > 65535)
+        return fail(DC_ERR_SHAPE, "%s: spatial dimension exceeds 32767 or batch exceeds 65535", fn);
+    if ((int64_t)g->batch * g->in_h * g->in_w > (1 << 29) ||
+        (int64_t)g->batch * g->out_h * g->out_w > (1 << 29))
+        return fail(DC_ERR_SHAPE, "%s: more than 2^29 pixels", fn);
+    if (g->kernel_h <= 0 || g->kernel_w <= 0 || g->stride_h <= 0 || g->stride_w <= 0 ||
+        g->dilation_h <= 0 || g->dilation_w <= 0)
+        return fail(DC_ERR_SHAPE, "%s: kernel, stride and dilation must be positive", fn);
+    if (g->pad_top < 0 || g->pad_left < 0 || g->pad_bottom < 0 || g->pad_right < 0)
+        return fail(DC_ERR_SHAPE, "%s: negative padding", fn);
+    int eh, ew;
+    if (transposed) {
+        if (g->pad_top != g->pad_bottom || g->pad_left != g->pad_right)
+            return fail(DC_ERR_UNSUPPORTED, "%s: transposed convolution needs symmetric padding", fn);
+        eh = (g->in_h - 1) * g->stride_h - 2 * g->pad_top + g->dilation_h * (g->kernel_h - 1) + 1;
+        ew = (g->in_w - 1) * g->stride_w - 2 * g->pad_left + g->dilation_w * (g->kernel_w - 1) + 1;
+    } else {
+        int nh = g->in_h + g->pad_top + g->pad_bottom - g->dilation_h * (g->kernel_h - 1) - 1;
+        int nw = g->in_w + g->pad_left + g->pad_right - g->dilation_w * (g->kernel_w - 1) - 1;
+        if (nh < 0 || nw < 0) return fail(DC_ERR_SHAPE, "%s: window larger than padded input", fn);
+        eh = nh / g->stride_h + 1;
+        ew = nw / g->stride_w + 1;
+    }
+    if (eh != g->out_h || ew != g->out_w)
+        return fail(DC_ERR_SHAPE, "%s: output %dx%d does not match geometry (expected %dx%d)", fn,
+                    g->out_h, g->out_w, eh, ew);
+    if (pooling) {
+        if (g->in_c != g->out_c) return fail(DC_ERR_SHAPE, "%s: pooling keeps the channel count", fn);
+        return DC_OK;
+    }
+    if (g->groups <= 0 || g->in_c % g->groups != 0 || g->out_c % g->groups != 0)
+        return fail(DC_ERR_SHAPE, "%s: groups=%d does not divide channels %d -> %d", fn, g->groups,
+                    g->in_c, g->out_c);
+    return DC_OK;
+}
+
+int check_conv(const char *fn, const dc_geometry *g, const void *input, const void *filter,
+               const void *out, const int32_t *mask, const int32_t *out_mask, int dtype,
+               bool transposed) {
+    if (dtype != DC_F32 && dtype != DC_F16) return fail(DC_ERR_DTYPE, "%s: unsupported dtype %d", fn, dtype);
+    int rc = check_geometry(fn, g, transposed, false);
+    if (rc != DC_OK) return rc;
+    if (!input || !filter || !out || !mask || !out_mask)
+        return fail(DC_ERR_NULL, "%s: input, filter, out, mask and out_mask are required", fn);
+    const bool depthwise = g->groups == g->in_c && g->groups == g->out_c;
+    if (transposed && g->groups != 1)
+        return fail(DC_ERR_UNSUPPORTED, "%s: transposed convolution supports groups == 1 only", fn);
+    if (dtype == DC_F16 && g->groups != 1 && !depthwise)
+        return fail(DC_ERR_UNSUPPORTED,
+                    "%s: fp16 grouped convolution needs groups == 1 or depthwise (the reference "
+                    "fp16 filter layout is only defined for those)", fn);
+    size_t es = esize(dtype);
+    if (reinterpret_cast<uintptr_t>(input) % es || reinterpret_cast<uintptr_t>(filter) % es ||
+        reinterpret_cast<uintptr_t>(out) % es || reinterpret_cast<uintptr_t>(mask) % 4 ||
+        reinterpret_cast<uintptr_t>(out_mask) % 4)
+        return fail(DC_ERR_ALIGN, "%s: pointer not aligned to its element size", fn);
+    return DC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *dc_version(void) { return "deltacnn-hip 0.1 (gfx950)"; }
+
+const char *dc_last_error(void) { return g_error; }
+
+int dc_sparsify(const void *input, void *prev_input, void *delta, int32_t *mask, float threshold,
+                int32_t pixels, int32_t channels, int dtype, void *stream) {
+    DC_REQUIRE_DTYPE("dc_sparsify");
+    int rc = check_pc("dc_sparsify", pixels, channels);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_PTR("dc_sparsify", input);
+    DC_REQUIRE_PTR("dc_sparsify", prev_input);
+    DC_REQUIRE_PTR("dc_sparsify", delta);
+    DC_REQUIRE_PTR("dc_sparsify", mask);
+    DC_REQUIRE_ALIGNED("dc_sparsify", input, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_sparsify", prev_input, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_sparsify", delta, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_sparsify", mask, 4);
+    return finish(dc::launch_sparsify(input, prev_input, delta, mask, threshold, pixels, channels,
+                                      dtype, (hipStream_t)stream), "dc_sparsify");
+}
+
+int dc_activate_truncate(void *delta, void *prev_input, void *truncated, int32_t *mask,
+                         float threshold, int activation, int truncation_mode, int32_t pixels,
+                         int32_t channels, int dtype, void *stream) {
+    DC_REQUIRE_DTYPE("dc_activate_truncate");
+    int rc = check_pc("dc_activate_truncate", pixels, channels);
+    if (rc != DC_OK) return rc;
+    if (activation > DC_ACT_SWISH)
+        return fail(DC_ERR_UNSUPPORTED, "dc_activate_truncate: activation id %d", activation);
+    if (truncation_mode > DC_TRUNC_RMS)
+        return fail(DC_ERR_UNSUPPORTED, "dc_activate_truncate: truncation mode %d", truncation_mode);
+    DC_REQUIRE_PTR("dc_activate_truncate", delta);
+    DC_REQUIRE_PTR("dc_activate_truncate", prev_input);
+    DC_REQUIRE_PTR("dc_activate_truncate", mask);
+    if (truncation_mode >= 0) DC_REQUIRE_PTR("dc_activate_truncate", truncated);
+    DC_REQUIRE_ALIGNED("dc_activate_truncate", delta, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_activate_truncate", prev_input, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_activate_truncate", truncated, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_activate_truncate", mask, 4);
+    return finish(dc::launch_activate_truncate(delta, prev_input, truncated, mask, threshold,
+                                               activation, truncation_mode, pixels, channels,
+                                               dtype, (hipStream_t)stream), "dc_activate_truncate");
+}
+
+int dc_conv(const dc_geometry *g, const void *input, const void *filter, const void *packed_filter,
+            const void *bias, void *out, const int32_t *mask, int32_t *out_mask, int dtype,
+            void *stream) {
+    int rc = check_conv("dc_conv", g, input, filter, out, mask, out_mask, dtype, false);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_ALIGNED("dc_conv", packed_filter, 16);
+    return finish(dc::launch_conv(*g, input, filter, packed_filter, bias, out, mask, out_mask,
+                                  dtype, false, nullptr, (hipStream_t)stream), "dc_conv");
+}
+
+int dc_conv_act(const dc_geometry *g, const void *input, const void *filter,
+                const void *packed_filter, const void *bias, void *out, const int32_t *mask,
+                int32_t *out_mask, void *prev_out, void *truncated, float threshold, int activation,
+                int truncation_mode, int dtype, void *stream) {
+    int rc = check_conv("dc_conv_act", g, input, filter, out, mask, out_mask, dtype, false);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_ALIGNED("dc_conv_act", packed_filter, 16);
+    DC_REQUIRE_PTR("dc_conv_act", prev_out);
+    if (truncation_mode >= 0) DC_REQUIRE_PTR("dc_conv_act", truncated);
+    if (activation > DC_ACT_SWISH || truncation_mode > DC_TRUNC_RMS)
+        return fail(DC_ERR_UNSUPPORTED, "dc_conv_act: activation %d / truncation mode %d",
+                    activation, truncation_mode);
+    dc::ActEpilogue epi{prev_out, truncated, threshold, activation, truncation_mode};
+    return finish(dc::launch_conv(*g, input, filter, packed_filter, bias, out, mask, out_mask,
+                                  dtype, false, &epi, (hipStream_t)stream), "dc_conv_act");
+}
+
+int64_t dc_packed_filter_bytes(const dc_geometry *g, int dtype, int transposed) {
+    if (g == nullptr || g->in_c <= 0 || g->out_c <= 0 || g->kernel_h <= 0 || g->kernel_w <= 0 ||
+        g->groups <= 0)
+        return 0;
+    return dc::packed_filter_bytes(*g, dtype, transposed != 0);
+}
+
+int dc_pack_filter(const dc_geometry *g, const void *filter, void *packed_filter, int dtype,
+                   int transposed, void *stream) {
+    DC_REQUIRE_DTYPE("dc_pack_filter");
+    if (g == nullptr) return fail(DC_ERR_NULL, "dc_pack_filter: geometry is NULL");
+    if (dc_packed_filter_bytes(g, dtype, transposed) == 0)
+        return fail(DC_ERR_UNSUPPORTED, "dc_pack_filter: this convolution has no packed form");
+    DC_REQUIRE_PTR("dc_pack_filter", filter);
+    DC_REQUIRE_PTR("dc_pack_filter", packed_filter);
+    DC_REQUIRE_ALIGNED("dc_pack_filter", filter, 2);
+    DC_REQUIRE_ALIGNED("dc_pack_filter", packed_filter, 16);
+    return finish(dc::launch_pack_filter(*g, filter, packed_filter, dtype, transposed != 0,
+                                         (hipStream_t)stream), "dc_pack_filter");
+}
+
+int dc_deconv(const dc_geometry *g, const void *input, const void *filter,
+              const void *packed_filter, const void *bias, void *out, const int32_t *mask,
+              int32_t *out_mask, int dtype, void *stream) {
+    int rc = check_conv("dc_deconv", g, input, filter, out, mask, out_mask, dtype, true);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_ALIGNED("dc_deconv", packed_filter, 16);
+    return finish(dc::launch_conv(*g, input, filter, packed_filter, bias, out, mask, out_mask,
+                                  dtype, true, nullptr, (hipStream_t)stream), "dc_deconv");
+}
+
+int dc_pool(const dc_geometry *g, const void *input, const void *prev_input, void *out,
+            const int32_t *mask, int32_t *out_mask, int pooling_mode, int dtype, void *stream) {
+    DC_REQUIRE_DTYPE("dc_pool");
+    int rc = check_geometry("dc_pool", g, false, true);
+    if (rc != DC_OK) return rc;
+    if (pooling_mode != DC_POOL_MAX && pooling_mode != DC_POOL_AVG)
+        return fail(DC_ERR_UNSUPPORTED, "dc_pool: pooling mode %d", pooling_mode);
+    DC_REQUIRE_PTR("dc_pool", input);
+    DC_REQUIRE_PTR("dc_pool", out);
+    DC_REQUIRE_PTR("dc_pool", mask);
+    DC_REQUIRE_PTR("dc_pool", out_mask);
+    if (pooling_mode == DC_POOL_MAX) DC_REQUIRE_PTR("dc_pool", prev_input);
+    DC_REQUIRE_ALIGNED("dc_pool", input, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_pool", prev_input, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_pool", out, (g->out_h == 1 && g->out_w == 1) ? 4 : esize(dtype));
+    return finish(dc::launch_pool(*g, input, prev_input, out, mask, out_mask, pooling_mode, dtype,
+                                  (hipStream_t)stream), "dc_pool");
+}
+
+int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_t *mask_a,
+           const int32_t *mask_b, int32_t *mask_out, float weight_a, float weight_b, int activation,
+           int dense_out, int32_t pixels, int32_t channels, int dtype, void *stream) {
+    DC_REQUIRE_DTYPE("dc_add");
+    int rc = check_pc("dc_add", pixels, channels);
+    if (rc != DC_OK) return rc;
+    if (activation > DC_ACT_SWISH) return fail(DC_ERR_UNSUPPORTED, "dc_add: activation id %d", activation);
+    DC_REQUIRE_PTR("dc_add", a);
+    DC_REQUIRE_PTR("dc_add", b);
+    DC_REQUIRE_PTR("dc_add", out);
+    DC_REQUIRE_PTR("dc_add", mask_a);
+    DC_REQUIRE_PTR("dc_add", mask_b);
+    if (!dense_out) DC_REQUIRE_PTR("dc_add", mask_out);
+    if (dense_out || activation > 0) DC_REQUIRE_PTR("dc_add", prev_out);
+    DC_REQUIRE_ALIGNED("dc_add", a, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_add", b, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_add", out, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_add", prev_out, esize(dtype));
+    return finish(dc::launch_add(a, b, prev_out, out, mask_a, mask_b, mask_out, weight_a, weight_b,
+                                 activation, dense_out, pixels, channels, dtype,
+                                 (hipStream_t)stream), "dc_add");
+}
+
+int dc_add_to_dense(void *a, void *b, const int32_t *mask_a, int activation, int32_t pixels,
+                    int32_t channels, int dtype, void *stream) {
+    DC_REQUIRE_DTYPE("dc_add_to_dense");
+    int rc = check_pc("dc_add_to_dense", pixels, channels);
+    if (rc != DC_OK) return rc;
+    if (activation > DC_ACT_SWISH)
+        return fail(DC_ERR_UNSUPPORTED, "dc_add_to_dense: activation id %d", activation);
+    DC_REQUIRE_PTR("dc_add_to_dense", a);
+    DC_REQUIRE_PTR("dc_add_to_dense", b);
+    DC_REQUIRE_PTR("dc_add_to_dense", mask_a);
+    DC_REQUIRE_ALIGNED("dc_add_to_dense", a, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_add_to_dense", b, esize(dtype));
+    return finish(dc::launch_add_to_dense(a, b, mask_a, activation, pixels, channels, dtype,
+                                          (hipStream_t)stream), "dc_add_to_dense");
+}
+
+int dc_upsample(const void *input, void *out, const int32_t *mask_in, int32_t *mask_out,
+                int32_t batch, int32_t in_h, int32_t in_w, int32_t channels, int32_t scale,
+                int dtype, void *stream) {
+    DC_REQUIRE_DTYPE("dc_upsample");
+    if (batch <= 0 || in_h <= 0 || in_w <= 0 || channels <= 0 || scale <= 0)
+        return fail(DC_ERR_SHAPE, "dc_upsample: non-positive dimension");
+    if ((int64_t)batch * in_h * in_w * scale * scale > (1 << 29))
+        return fail(DC_ERR_SHAPE, "dc_upsample: more than 2^29 output pixels");
+    DC_REQUIRE_PTR("dc_upsample", input);
+    DC_REQUIRE_PTR("dc_upsample", out);
+    DC_REQUIRE_PTR("dc_upsample", mask_in);
+    DC_REQUIRE_PTR("dc_upsample", mask_out);
+    DC_REQUIRE_ALIGNED("dc_upsample", input, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_upsample", out, esize(dtype));
+    return finish(dc::launch_upsample(input, out, mask_in, mask_out, batch, in_h, in_w, channels,
+                                      scale, dtype, (hipStream_t)stream), "dc_upsample");
+}
+
+int dc_concat(const void *a, const void *b, void *out, const int32_t *mask_a, const int32_t *mask_b,
+              int32_t *mask_out, int32_t pixels, int32_t channels_a, int32_t channels_b, int dtype,
+              void *stream) {
+    DC_REQUIRE_DTYPE("dc_concat");
+    int rc = check_pc("dc_concat", pixels, channels_a);
+    if (rc != DC_OK) return rc;
+    rc = check_pc("dc_concat", pixels, channels_b);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_PTR("dc_concat", a);
+    DC_REQUIRE_PTR("dc_concat", b);
+    DC_REQUIRE_PTR("dc_concat", out);
+    DC_REQUIRE_PTR("dc_concat", mask_a);
+    DC_REQUIRE_PTR("dc_concat", mask_b);
+    DC_REQUIRE_PTR("dc_concat", mask_out);
+    DC_REQUIRE_ALIGNED("dc_concat", a, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_concat", b, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_concat", out, esize(dtype));
+    return finish(dc::launch_concat(a, b, out, mask_a, mask_b, mask_out, pixels, channels_a,
+                                    channels_b, dtype, (hipStream_t)stream), "dc_concat");
+}
+
+int dc_mul_add(const void *input, const int32_t *mask, void *out, int32_t *mask_out,
+               const void *scale, const void *bias, int32_t pixels, int32_t channels, int dtype,
+               void *stream) {
+    DC_REQUIRE_DTYPE("dc_mul_add");
+    int rc = check_pc("dc_mul_add", pixels, channels);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_PTR("dc_mul_add", input);
+    DC_REQUIRE_PTR("dc_mul_add", mask);
+    DC_REQUIRE_PTR("dc_mul_add", out);
+    DC_REQUIRE_PTR("dc_mul_add", mask_out);
+    DC_REQUIRE_PTR("dc_mul_add", scale);
+    DC_REQUIRE_ALIGNED("dc_mul_add", input, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_mul_add", out, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_mul_add", scale, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_mul_add", bias, esize(dtype));
+    return finish(dc::launch_mul_add(input, mask, out, mask_out, scale, bias, pixels, channels,
+                                     dtype, (hipStream_t)stream), "dc_mul_add");
+}
+
+}  // extern "C"

@@ -1,0 +1,715 @@
+// Bandwidth-bound per-pixel operators of the delta path: sparsify, activation + truncation,
+// densify, add, add-to-dense, nearest upsample, concatenate, per-channel scale/offset.
+//
+// Common shape: features are NHWC, so a pixel is a contiguous row of C values.  A pixel is
+// handled by an aligned group of G lanes (G a power of two, chosen on the host so that a
+// group covers the row with 16-byte vectors); a wavefront therefore handles 64/G pixels at a
+// time.  Operators that only touch active pixels first compact the active pixels of the
+// wavefront's 64 candidates (one coalesced mask load + ballot + popcount rank) into an LDS
+// list, so lanes are not wasted on inactive pixels at low update density.
+//
+// Compiled with -ffp-contract=off: every arithmetic operation rounds on its own, in the
+// tensor's own type, which is what makes masks reproducible bit for bit.
+#include "common.hpp"
+
+namespace dc {
+namespace {
+
+constexpr int MAXW = 4;  // wavefronts per workgroup (blockDim.x <= 256)
+
+// Compact the active pixels of this wavefront's 64 candidates and run `f(pixel, group_lane,
+// valid)` for each of them, 64/G pixels per step.  Every lane of the workgroup must call
+// this (it contains a workgroup barrier).  `f` is called by all lanes of a step; lanes whose
+// group has no pixel get valid == false.
+template <typename F>
+__device__ __forceinline__ void for_each_active(bool active, int px, int G, F f) {
+    __shared__ int s_list[MAXW][WAVE];
+    const int wave = threadIdx.x / WAVE;
+    int n;
+    int rank = wave_rank(active, n);
+    if (active) s_list[wave][rank] = px;
+    __syncthreads();
+    const int per_step = WAVE / G;
+    const int grp = lane_id() / G;
+    const int gl = lane_id() & (G - 1);
+    for (int base = 0; base < n; base += per_step) {
+        int idx = base + grp;
+        bool valid = idx < n;
+        int p = valid ? s_list[wave][idx] : 0;
+        f(p, gl, valid);
+    }
+}
+
+// ------------------------------------------------------------------------------- sparsify
+// delta = in - prev; the pixel is active if any channel passes the compare (`ge`: >= instead
+// of >, the fp16 even-C rule); active pixels write delta and prev := in for all channels.
+template <typename T, int ITERS>
+__global__ void __launch_bounds__(256)
+sparsify_vec_kernel(const T *__restrict__ in, T *__restrict__ prev, T *__restrict__ delta,
+                    int32_t *__restrict__ mask, float thr_f, int P, int C, int G, bool ge) {
+    constexpr int N = Vec16<T>::N;
+    const T thr = T(thr_f);
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int p = gid / G;
+    const int gl = gid & (G - 1);
+    const bool valid = p < P;
+    Vec<T, N> x[ITERS], d[ITERS];
+    bool hit = false;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        int c = (it * G + gl) * N;
+        if (valid && c < C) {
+            size_t off = (size_t)p * C + c;
+            x[it] = vload<T, N>(in + off);
+            Vec<T, N> q = vload<T, N>(prev + off);
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                d[it].v[j] = x[it].v[j] - q.v[j];
+                T a = tabs(d[it].v[j]);
+                hit |= ge ? !(a < thr) : (a > thr);
+            }
+        }
+    }
+    const bool any = group_any(hit, G);
+    if (valid && any) {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            int c = (it * G + gl) * N;
+            if (c < C) {
+                size_t off = (size_t)p * C + c;
+                vstore<T, N>(delta + off, d[it]);
+                vstore<T, N>(prev + off, x[it]);
+            }
+        }
+    }
+    if (valid && gl == 0) mask[p] = any ? 1 : 0;
+}
+
+// Any C / alignment: scalar, two passes (scan, then recompute and write).
+template <typename T>
+__global__ void __launch_bounds__(256)
+sparsify_gen_kernel(const T *__restrict__ in, T *__restrict__ prev, T *__restrict__ delta,
+                    int32_t *__restrict__ mask, float thr_f, int P, int C, int G, bool ge) {
+    const T thr = T(thr_f);
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int p = gid / G;
+    const int gl = gid & (G - 1);
+    const bool valid = p < P;
+    bool hit = false;
+    if (valid) {
+        for (int c = gl; c < C; c += G) {
+            size_t off = (size_t)p * C + c;
+            T a = tabs(T(in[off] - prev[off]));
+            hit |= ge ? !(a < thr) : (a > thr);
+        }
+    }
+    const bool any = group_any(hit, G);
+    if (valid && any) {
+        for (int c = gl; c < C; c += G) {
+            size_t off = (size_t)p * C + c;
+            T xi = in[off];
+            delta[off] = xi - prev[off];
+            prev[off] = xi;
+        }
+    }
+    if (valid && gl == 0) mask[p] = any ? 1 : 0;
+}
+
+// ----------------------------------------------------------------- activation + truncation
+// Per active pixel: T = trunc + delta; S = T + prev; D = act(S) - act(prev).
+// keep (max: any |D| > thr; norm: sqrt(sum D^2) > thr; rms: sqrt(sum D^2 / C) > thr):
+//   prev = S, delta = D, trunc = 0;   otherwise trunc = T and the mask word is cleared.
+__device__ __forceinline__ float group_sum(float v, int G) {
+    for (int o = 1; o < G; o <<= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+
+template <typename T, int ITERS, int ACT>
+__global__ void __launch_bounds__(256)
+act_trunc_vec_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict__ trunc,
+                     int32_t *__restrict__ mask, float thr_f, int mode, int P, int C, int G) {
+    constexpr int N = Vec16<T>::N;
+    const T thr = T(thr_f);
+    const int px = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool active = px < P && mask[px] != 0;
+    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
+        Vec<T, N> t[ITERS], s[ITERS], d[ITERS];
+        bool hit = false;
+        float sq = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            int c = (it * G + gl) * N;
+            if (valid && c < C) {
+                size_t off = (size_t)p * C + c;
+                Vec<T, N> dl = vload<T, N>(delta + off);
+                Vec<T, N> q = vload<T, N>(prev + off);
+                Vec<T, N> tr = vload<T, N>(trunc + off);
+#pragma unroll
+                for (int j = 0; j < N; ++j) {
+                    t[it].v[j] = tr.v[j] + dl.v[j];
+                    s[it].v[j] = t[it].v[j] + q.v[j];
+                    d[it].v[j] = act_apply<T>(s[it].v[j], ACT) - act_apply<T>(q.v[j], ACT);
+                    hit |= tabs(d[it].v[j]) > thr;
+                    sq += float(d[it].v[j]) * float(d[it].v[j]);
+                }
+            }
+        }
+        bool keep;
+        if (mode == DC_TRUNC_MAX) {
+            keep = group_any(hit, G);
+        } else {
+            sq = group_sum(sq, G);
+            if (mode == DC_TRUNC_RMS) sq /= float(C);
+            keep = sqrtf(sq) > float(thr);
+        }
+        if (valid) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                int c = (it * G + gl) * N;
+                if (c < C) {
+                    size_t off = (size_t)p * C + c;
+                    if (keep) {
+                        Vec<T, N> z;
+#pragma unroll
+                        for (int j = 0; j < N; ++j) z.v[j] = T(0);
+                        vstore<T, N>(prev + off, s[it]);
+                        vstore<T, N>(delta + off, d[it]);
+                        vstore<T, N>(trunc + off, z);
+                    } else {
+                        vstore<T, N>(trunc + off, t[it]);
+                    }
+                }
+            }
+            if (!keep && gl == 0) mask[p] = 0;
+        }
+    });
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+act_trunc_gen_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict__ trunc,
+                     int32_t *__restrict__ mask, float thr_f, int act, int mode, int P, int C,
+                     int G) {
+    const T thr = T(thr_f);
+    const int px = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool active = px < P && mask[px] != 0;
+    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
+        bool hit = false;
+        float sq = 0.f;
+        if (valid) {
+            for (int c = gl; c < C; c += G) {
+                size_t off = (size_t)p * C + c;
+                T q = prev[off];
+                T t = trunc[off] + delta[off];
+                T s = t + q;
+                T d = act_apply<T>(s, act) - act_apply<T>(q, act);
+                hit |= tabs(d) > thr;
+                sq += float(d) * float(d);
+            }
+        }
+        bool keep;
+        if (mode == DC_TRUNC_MAX) {
+            keep = group_any(hit, G);
+        } else {
+            sq = group_sum(sq, G);
+            if (mode == DC_TRUNC_RMS) sq /= float(C);
+            keep = sqrtf(sq) > float(thr);
+        }
+        if (valid) {
+            for (int c = gl; c < C; c += G) {
+                size_t off = (size_t)p * C + c;
+                T q = prev[off];
+                T t = trunc[off] + delta[off];
+                if (keep) {
+                    T s = t + q;
+                    prev[off] = s;
+                    delta[off] = act_apply<T>(s, act) - act_apply<T>(q, act);
+                    trunc[off] = T(0);
+                } else {
+                    trunc[off] = t;
+                }
+            }
+            if (!keep && gl == 0) mask[p] = 0;
+        }
+    });
+}
+
+// -------------------------------------------------------------------------------- densify
+// Truncation mode < 0: prev += delta on active pixels; a non-linear activation also rewrites
+// delta = act(prev_new) - act(prev_old).
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+accumulate_kernel(T *__restrict__ delta, T *__restrict__ prev, const int32_t *__restrict__ mask,
+                  int act, int P, int C, int G) {
+    const int px = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool active = px < P && mask[px] != 0;
+    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
+        if (!valid) return;
+        for (int c = gl * N; c < C; c += G * N) {
+            size_t off = (size_t)p * C + c;
+            Vec<T, N> dl = vload<T, N>(delta + off);
+            Vec<T, N> q = vload<T, N>(prev + off);
+            Vec<T, N> s;
+#pragma unroll
+            for (int j = 0; j < N; ++j) s.v[j] = dl.v[j] + q.v[j];
+            vstore<T, N>(prev + off, s);
+            if (act > 0) {
+#pragma unroll
+                for (int j = 0; j < N; ++j)
+                    dl.v[j] = act_apply<T>(s.v[j], act) - act_apply<T>(q.v[j], act);
+                vstore<T, N>(delta + off, dl);
+            }
+        }
+    });
+}
+
+// ------------------------------------------------------------------------------------ add
+// s = wa*a*[Ma]; s = fma(b, wb, s)*[Mb]; mask_out = Ma | Mb (written for every pixel).
+// act > 0: prev += s, out = act(prev_new) - act(prev_old).
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+add_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ prev,
+           T *__restrict__ out, const int32_t *__restrict__ ma, const int32_t *__restrict__ mb,
+           int32_t *__restrict__ mo, float wa_f, float wb_f, int act, int P, int C, int G) {
+    const T wa = T(wa_f), wb = T(wb_f);
+    const int px = blockIdx.x * blockDim.x + threadIdx.x;
+    int flags = 0;
+    if (px < P) {
+        flags = (ma[px] != 0 ? 1 : 0) | (mb[px] != 0 ? 2 : 0);
+        mo[px] = flags != 0 ? 1 : 0;
+    }
+    // the pixel index and its two activity bits travel together through the compaction
+    for_each_active(flags != 0, px * 4 + flags, G, [&](int code, int gl, bool valid) {
+        if (!valid) return;
+        const int p = code >> 2;
+        const bool aa = code & 1, ab = code & 2;
+        for (int c = gl * N; c < C; c += G * N) {
+            size_t off = (size_t)p * C + c;
+            Vec<T, N> s;
+#pragma unroll
+            for (int j = 0; j < N; ++j) s.v[j] = T(0);
+            if (aa) {
+                Vec<T, N> va = vload<T, N>(a + off);
+#pragma unroll
+                for (int j = 0; j < N; ++j) s.v[j] = va.v[j] * wa;
+            }
+            if (ab) {
+                Vec<T, N> vb = vload<T, N>(b + off);
+#pragma unroll
+                for (int j = 0; j < N; ++j) s.v[j] = fma_t(vb.v[j], wb, s.v[j]);
+            }
+            if (act > 0) {
+                Vec<T, N> q = vload<T, N>(prev + off);
+                Vec<T, N> n;
+#pragma unroll
+                for (int j = 0; j < N; ++j) {
+                    n.v[j] = s.v[j] + q.v[j];
+                    s.v[j] = act_apply<T>(n.v[j], act) - act_apply<T>(q.v[j], act);
+                }
+                vstore<T, N>(prev + off, n);
+            }
+            vstore<T, N>(out + off, s);
+        }
+    });
+}
+
+// dense_out: prev += s on active pixels, out = act(prev) for every pixel.
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+add_dense_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ prev,
+                 T *__restrict__ out, const int32_t *__restrict__ ma,
+                 const int32_t *__restrict__ mb, float wa_f, float wb_f, int act, int P, int C,
+                 int G) {
+    const T wa = T(wa_f), wb = T(wb_f);
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int p = gid / G;
+    const int gl = gid & (G - 1);
+    if (p >= P) return;
+    const bool aa = ma[p] != 0, ab = mb[p] != 0;
+    for (int c = gl * N; c < C; c += G * N) {
+        size_t off = (size_t)p * C + c;
+        Vec<T, N> q = vload<T, N>(prev + off);
+        if (aa || ab) {
+            Vec<T, N> s;
+#pragma unroll
+            for (int j = 0; j < N; ++j) s.v[j] = T(0);
+            if (aa) {
+                Vec<T, N> va = vload<T, N>(a + off);
+#pragma unroll
+                for (int j = 0; j < N; ++j) s.v[j] = va.v[j] * wa;
+            }
+            if (ab) {
+                Vec<T, N> vb = vload<T, N>(b + off);
+#pragma unroll
+                for (int j = 0; j < N; ++j) s.v[j] = fma_t(vb.v[j], wb, s.v[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < N; ++j) q.v[j] = s.v[j] + q.v[j];
+            vstore<T, N>(prev + off, q);
+        }
+#pragma unroll
+        for (int j = 0; j < N; ++j) q.v[j] = act_apply<T>(q.v[j], act);
+        vstore<T, N>(out + off, q);
+    }
+}
+
+// --------------------------------------------------------------------------- add to dense
+// b[px] += a[px] on active pixels.
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+add_to_dense_kernel(const T *__restrict__ a, T *__restrict__ b, const int32_t *__restrict__ ma,
+                    int P, int C, int G) {
+    const int px = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool active = px < P && ma[px] != 0;
+    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
+        if (!valid) return;
+        for (int c = gl * N; c < C; c += G * N) {
+            size_t off = (size_t)p * C + c;
+            Vec<T, N> va = vload<T, N>(a + off);
+            Vec<T, N> vb = vload<T, N>(b + off);
+#pragma unroll
+            for (int j = 0; j < N; ++j) vb.v[j] = vb.v[j] + va.v[j];
+            vstore<T, N>(b + off, vb);
+        }
+    });
+}
+
+// With an activation the operator turns `a` into a dense output: b += a on active pixels,
+// then a = act(b) on every pixel.
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+add_to_dense_act_kernel(T *__restrict__ a, T *__restrict__ b, const int32_t *__restrict__ ma,
+                        int act, int P, int C, int G) {
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int p = gid / G;
+    const int gl = gid & (G - 1);
+    if (p >= P) return;
+    const bool active = ma[p] != 0;
+    for (int c = gl * N; c < C; c += G * N) {
+        size_t off = (size_t)p * C + c;
+        Vec<T, N> vb = vload<T, N>(b + off);
+        if (active) {
+            Vec<T, N> va = vload<T, N>(a + off);
+#pragma unroll
+            for (int j = 0; j < N; ++j) vb.v[j] = vb.v[j] + va.v[j];
+            vstore<T, N>(b + off, vb);
+        }
+#pragma unroll
+        for (int j = 0; j < N; ++j) vb.v[j] = act_apply<T>(vb.v[j], act);
+        vstore<T, N>(a + off, vb);
+    }
+}
+
+// ------------------------------------------------------------------------------- upsample
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+upsample_kernel(const T *__restrict__ in, T *__restrict__ out, const int32_t *__restrict__ mi,
+                int32_t *__restrict__ mo, int B, int H, int W, int C, int S, int G) {
+    const int P = B * H * W;
+    const int px = blockIdx.x * blockDim.x + threadIdx.x;
+    const int Wo = W * S;
+    bool active = false;
+    if (px < P) {
+        active = mi[px] != 0;
+        int row = px / W, x = px - row * W;  // row = b*H + y
+        for (int i = 0; i < S * S; ++i)
+            mo[(size_t)(row * S + i / S) * Wo + x * S + i % S] = active ? 1 : 0;
+    }
+    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
+        if (!valid) return;
+        int row = p / W, x = p - row * W;
+        for (int c = gl * N; c < C; c += G * N) {
+            Vec<T, N> v = vload<T, N>(in + (size_t)p * C + c);
+            for (int i = 0; i < S * S; ++i) {
+                size_t op = (size_t)(row * S + i / S) * Wo + x * S + i % S;
+                vstore<T, N>(out + op * C + c, v);
+            }
+        }
+    });
+}
+
+// ---------------------------------------------------------------------------- concatenate
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+concat_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ out,
+              const int32_t *__restrict__ ma, const int32_t *__restrict__ mb,
+              int32_t *__restrict__ mo, int P, int Ca, int Cb, int G) {
+    const int px = blockIdx.x * blockDim.x + threadIdx.x;
+    int flags = 0;
+    if (px < P) {
+        flags = (ma[px] != 0 ? 1 : 0) | (mb[px] != 0 ? 2 : 0);
+        mo[px] = flags != 0 ? 1 : 0;
+    }
+    for_each_active(flags != 0, px * 4 + flags, G, [&](int code, int gl, bool valid) {
+        if (!valid) return;
+        const int p = code >> 2;
+        const bool aa = code & 1, ab = code & 2;
+        T *o = out + (size_t)p * (Ca + Cb);
+        Vec<T, N> z;
+#pragma unroll
+        for (int j = 0; j < N; ++j) z.v[j] = T(0);
+        for (int c = gl * N; c < Ca; c += G * N)
+            vstore<T, N>(o + c, aa ? vload<T, N>(a + (size_t)p * Ca + c) : z);
+        for (int c = gl * N; c < Cb; c += G * N)
+            vstore<T, N>(o + Ca + c, ab ? vload<T, N>(b + (size_t)p * Cb + c) : z);
+    });
+}
+
+// -------------------------------------------------------------------------------- mul_add
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+mul_add_kernel(const T *__restrict__ in, const int32_t *__restrict__ mask, T *__restrict__ out,
+               int32_t *__restrict__ mo, const T *__restrict__ scale,
+               const T *__restrict__ bias, int P, int C, int G) {
+    const int px = blockIdx.x * blockDim.x + threadIdx.x;
+    bool active = false;
+    if (px < P) {
+        active = mask[px] != 0;
+        if (mo != mask) mo[px] = active ? 1 : 0;
+    }
+    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
+        if (!valid) return;
+        for (int c = gl * N; c < C; c += G * N) {
+            size_t off = (size_t)p * C + c;
+            Vec<T, N> v = vload<T, N>(in + off);
+            Vec<T, N> sc = vload<T, N>(scale + c);
+            if (bias != nullptr) {
+                Vec<T, N> bi = vload<T, N>(bias + c);
+#pragma unroll
+                for (int j = 0; j < N; ++j)
+                    v.v[j] = fma_t(v.v[j], sc.v[j], bi.v[j]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < N; ++j) v.v[j] = v.v[j] * sc.v[j];
+            }
+            vstore<T, N>(out + off, v);
+        }
+    });
+}
+
+// ---------------------------------------------------------------------------- host helpers
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Lanes per pixel for `nvec` vectors per row when a lane may hold up to `max_iters` of them.
+inline int group_lanes(int nvec, int max_iters) {
+    int g = pow2_ceil(ceil_div(nvec, max_iters));
+    return g > WAVE ? WAVE : g;
+}
+
+inline int block_for(int64_t threads) { return threads >= (1 << 16) ? 256 : 64; }
+
+template <typename T>
+bool can_vec(int C, std::initializer_list<const void *> ptrs) {
+    if (C % Vec16<T>::N != 0) return false;
+    for (const void *p : ptrs)
+        if (p != nullptr && !aligned16(p)) return false;
+    return true;
+}
+
+template <typename T>
+hipError_t sparsify_t(const T *in, T *prev, T *delta, int32_t *mask, float thr, int P, int C,
+                      bool ge, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    if (can_vec<T>(C, {in, prev, delta}) && C / N <= WAVE * 4) {
+        int nvec = C / N;
+        int G = group_lanes(nvec, 4);
+        int iters = ceil_div(nvec, G);
+        int64_t threads = (int64_t)P * G;
+        int blk = block_for(threads);
+        dim3 grid((unsigned)ceil_div64(threads, blk));
+        switch (iters) {
+            case 1: sparsify_vec_kernel<T, 1><<<grid, blk, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
+            case 2: sparsify_vec_kernel<T, 2><<<grid, blk, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
+            default: sparsify_vec_kernel<T, 4><<<grid, blk, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
+        }
+    } else {
+        int G = group_lanes(C, 4);
+        int64_t threads = (int64_t)P * G;
+        int blk = block_for(threads);
+        sparsify_gen_kernel<T><<<dim3((unsigned)ceil_div64(threads, blk)), blk, 0, s>>>(
+            in, prev, delta, mask, thr, P, C, G, ge);
+    }
+    return hipGetLastError();
+}
+
+template <typename T, int ITERS>
+void act_trunc_launch(dim3 grid, int blk, hipStream_t s, T *delta, T *prev, T *trunc,
+                      int32_t *mask, float thr, int act, int mode, int P, int C, int G) {
+#define DC_AT(A) act_trunc_vec_kernel<T, ITERS, A><<<grid, blk, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, G)
+    switch (act) {
+        case DC_ACT_RELU: DC_AT(DC_ACT_RELU); break;
+        case DC_ACT_RELU6: DC_AT(DC_ACT_RELU6); break;
+        case DC_ACT_LEAKY: DC_AT(DC_ACT_LEAKY); break;
+        case DC_ACT_SIGMOID: DC_AT(DC_ACT_SIGMOID); break;
+        case DC_ACT_SWISH: DC_AT(DC_ACT_SWISH); break;
+        default: DC_AT(DC_ACT_LINEAR); break;
+    }
+#undef DC_AT
+}
+
+template <typename T>
+hipError_t act_trunc_t(T *delta, T *prev, T *trunc, int32_t *mask, float thr, int act, int mode,
+                       int P, int C, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    if (act < 0) act = 0;
+    int blk = block_for(P);
+    dim3 grid((unsigned)ceil_div(P, blk));
+    if (mode < 0) {
+        if (can_vec<T>(C, {delta, prev})) {
+            int G = group_lanes(C / N, 1);
+            accumulate_kernel<T, N><<<grid, blk, 0, s>>>(delta, prev, mask, act, P, C, G);
+        } else {
+            int G = group_lanes(C, 1);
+            accumulate_kernel<T, 1><<<grid, blk, 0, s>>>(delta, prev, mask, act, P, C, G);
+        }
+        return hipGetLastError();
+    }
+    if (can_vec<T>(C, {delta, prev, trunc}) && C / N <= WAVE * 4) {
+        int nvec = C / N;
+        int G = group_lanes(nvec, 4);
+        int iters = ceil_div(nvec, G);
+        switch (iters) {
+            case 1: act_trunc_launch<T, 1>(grid, blk, s, delta, prev, trunc, mask, thr, act, mode, P, C, G); break;
+            case 2: act_trunc_launch<T, 2>(grid, blk, s, delta, prev, trunc, mask, thr, act, mode, P, C, G); break;
+            default: act_trunc_launch<T, 4>(grid, blk, s, delta, prev, trunc, mask, thr, act, mode, P, C, G); break;
+        }
+    } else {
+        int G = group_lanes(C, 1);
+        act_trunc_gen_kernel<T><<<grid, blk, 0, s>>>(delta, prev, trunc, mask, thr, act, mode, P, C, G);
+    }
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t add_t(const T *a, const T *b, T *prev, T *out, const int32_t *ma, const int32_t *mb,
+                 int32_t *mo, float wa, float wb, int act, bool dense_out, int P, int C,
+                 hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    if (act < 0) act = 0;
+    const bool vec = can_vec<T>(C, {a, b, prev, out});
+    const int G = group_lanes(vec ? C / N : C, 1);
+    if (dense_out) {
+        int64_t threads = (int64_t)P * G;
+        int blk = block_for(threads);
+        dim3 grid((unsigned)ceil_div64(threads, blk));
+        if (vec) add_dense_kernel<T, N><<<grid, blk, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, G);
+        else add_dense_kernel<T, 1><<<grid, blk, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, G);
+    } else {
+        int blk = block_for(P);
+        dim3 grid((unsigned)ceil_div(P, blk));
+        if (vec) add_kernel<T, N><<<grid, blk, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, G);
+        else add_kernel<T, 1><<<grid, blk, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, G);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_sparsify(const void *in, void *prev, void *delta, int32_t *mask, float thr,
+                           int32_t P, int32_t C, int dtype, hipStream_t s) {
+    if (dtype == DC_F32)
+        return sparsify_t<float>((const float *)in, (float *)prev, (float *)delta, mask, thr, P, C, false, s);
+    return sparsify_t<half_t>((const half_t *)in, (half_t *)prev, (half_t *)delta, mask, thr, P, C,
+                              C % 2 == 0, s);
+}
+
+hipError_t launch_activate_truncate(void *delta, void *prev, void *trunc, int32_t *mask, float thr,
+                                    int act, int mode, int32_t P, int32_t C, int dtype,
+                                    hipStream_t s) {
+    if (dtype == DC_F32)
+        return act_trunc_t<float>((float *)delta, (float *)prev, (float *)trunc, mask, thr, act, mode, P, C, s);
+    return act_trunc_t<half_t>((half_t *)delta, (half_t *)prev, (half_t *)trunc, mask, thr, act, mode, P, C, s);
+}
+
+hipError_t launch_add(const void *a, const void *b, void *prev, void *out, const int32_t *ma,
+                      const int32_t *mb, int32_t *mo, float wa, float wb, int act, int dense_out,
+                      int32_t P, int32_t C, int dtype, hipStream_t s) {
+    if (dtype == DC_F32)
+        return add_t<float>((const float *)a, (const float *)b, (float *)prev, (float *)out, ma, mb, mo, wa, wb, act, dense_out != 0, P, C, s);
+    return add_t<half_t>((const half_t *)a, (const half_t *)b, (half_t *)prev, (half_t *)out, ma, mb, mo, wa, wb, act, dense_out != 0, P, C, s);
+}
+
+namespace {
+template <typename T>
+hipError_t add_to_dense_t(T *a, T *b, const int32_t *ma, int act, int P, int C, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    const bool vec = can_vec<T>(C, {a, b});
+    const int G = group_lanes(vec ? C / N : C, 1);
+    if (act > 0) {
+        int64_t threads = (int64_t)P * G;
+        int blk = block_for(threads);
+        dim3 grid((unsigned)ceil_div64(threads, blk));
+        if (vec) add_to_dense_act_kernel<T, N><<<grid, blk, 0, s>>>(a, b, ma, act, P, C, G);
+        else add_to_dense_act_kernel<T, 1><<<grid, blk, 0, s>>>(a, b, ma, act, P, C, G);
+        return hipGetLastError();
+    }
+    int blk = block_for(P);
+    dim3 grid((unsigned)ceil_div(P, blk));
+    if (vec) add_to_dense_kernel<T, N><<<grid, blk, 0, s>>>(a, b, ma, P, C, G);
+    else add_to_dense_kernel<T, 1><<<grid, blk, 0, s>>>(a, b, ma, P, C, G);
+    return hipGetLastError();
+}
+template <typename T>
+hipError_t upsample_t(const T *in, T *out, const int32_t *mi, int32_t *mo, int B, int H, int W,
+                      int C, int S, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    int P = B * H * W;
+    int blk = block_for(P);
+    dim3 grid((unsigned)ceil_div(P, blk));
+    if (can_vec<T>(C, {in, out})) upsample_kernel<T, N><<<grid, blk, 0, s>>>(in, out, mi, mo, B, H, W, C, S, group_lanes(C / N, 1));
+    else upsample_kernel<T, 1><<<grid, blk, 0, s>>>(in, out, mi, mo, B, H, W, C, S, group_lanes(C, 1));
+    return hipGetLastError();
+}
+template <typename T>
+hipError_t concat_t(const T *a, const T *b, T *out, const int32_t *ma, const int32_t *mb,
+                    int32_t *mo, int P, int Ca, int Cb, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    int blk = block_for(P);
+    dim3 grid((unsigned)ceil_div(P, blk));
+    int Cm = Ca > Cb ? Ca : Cb;
+    if (Ca % N == 0 && Cb % N == 0 && can_vec<T>(Ca, {a, b, out}))
+        concat_kernel<T, N><<<grid, blk, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, group_lanes(Cm / N, 1));
+    else
+        concat_kernel<T, 1><<<grid, blk, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, group_lanes(Cm, 1));
+    return hipGetLastError();
+}
+template <typename T>
+hipError_t mul_add_t(const T *in, const int32_t *mask, T *out, int32_t *mo, const T *scale,
+                     const T *bias, int P, int C, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    int blk = block_for(P);
+    dim3 grid((unsigned)ceil_div(P, blk));
+    if (can_vec<T>(C, {in, out, scale, bias})) mul_add_kernel<T, N><<<grid, blk, 0, s>>>(in, mask, out, mo, scale, bias, P, C, group_lanes(C / N, 1));
+    else mul_add_kernel<T, 1><<<grid, blk, 0, s>>>(in, mask, out, mo, scale, bias, P, C, group_lanes(C, 1));
+    return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_add_to_dense(void *a, void *b, const int32_t *ma, int act, int32_t P, int32_t C,
+                               int dtype, hipStream_t s) {
+    if (dtype == DC_F32) return add_to_dense_t<float>((float *)a, (float *)b, ma, act, P, C, s);
+    return add_to_dense_t<half_t>((half_t *)a, (half_t *)b, ma, act, P, C, s);
+}
+
+hipError_t launch_upsample(const void *in, void *out, const int32_t *mi, int32_t *mo, int32_t B,
+                           int32_t H, int32_t W, int32_t C, int32_t scale, int dtype,
+                           hipStream_t s) {
+    if (dtype == DC_F32) return upsample_t<float>((const float *)in, (float *)out, mi, mo, B, H, W, C, scale, s);
+    return upsample_t<half_t>((const half_t *)in, (half_t *)out, mi, mo, B, H, W, C, scale, s);
+}
+
+hipError_t launch_concat(const void *a, const void *b, void *out, const int32_t *ma,
+                         const int32_t *mb, int32_t *mo, int32_t P, int32_t Ca, int32_t Cb,
+                         int dtype, hipStream_t s) {
+    if (dtype == DC_F32) return concat_t<float>((const float *)a, (const float *)b, (float *)out, ma, mb, mo, P, Ca, Cb, s);
+    return concat_t<half_t>((const half_t *)a, (const half_t *)b, (half_t *)out, ma, mb, mo, P, Ca, Cb, s);
+}
+
+hipError_t launch_mul_add(const void *in, const int32_t *mask, void *out, int32_t *mo,
+                          const void *scale, const void *bias, int32_t P, int32_t C, int dtype,
+                          hipStream_t s) {
+    if (dtype == DC_F32) return mul_add_t<float>((const float *)in, mask, (float *)out, mo, (const float *)scale, (const float *)bias, P, C, s);
+    return mul_add_t<half_t>((const half_t *)in, mask, (half_t *)out, mo, (const half_t *)scale, (const half_t *)bias, P, C, s);
+}
+
+}  // namespace dc

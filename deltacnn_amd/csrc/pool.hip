@@ -1,0 +1,216 @@
+// Delta pooling.
+//   max: out = max_w(prev + M*delta) - max_w(prev) over in-bounds window pixels
+//   avg: out = sum_w M*delta / (Kh*Kw)
+// Arithmetic is fp32 for both tensor types with one rounding on store.
+//
+// pool_window_kernel  8x8 output tile per workgroup, mask dilation + compaction as for the
+//                     convolutions; each compacted pixel is then handled by a group of G lanes
+//                     that run along the channels with 16-byte vectors
+// pool_global_kernel  1x1 output (float32 [B][C]); every workgroup owns a slice of channels
+//                     and walks all input pixels, so the sum has a fixed order and needs no
+//                     atomics
+#include "tile.hpp"
+
+namespace dc {
+namespace {
+
+struct PoolQ {          // the literal zero that joins the maximum for bottom / right padding
+    int zero_bottom;    // rows >= Hi inside the bottom padding when pad_top != pad_bottom
+    int zero_right;     // columns >= Wi inside the right padding when pad_left != pad_right
+    int pb, pr;
+};
+
+template <typename T, int N, bool MAX>
+__global__ void __launch_bounds__(256)
+pool_window_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restrict__ prev,
+                   T *__restrict__ out, const int32_t *__restrict__ mask,
+                   int32_t *__restrict__ out_mask, int G) {
+    __shared__ int s_list[TILE_PX];
+    __shared__ int s_n;
+    const int b = blockIdx.z;
+    const int n = tile_mask_phase<false>(p, mask, out_mask, b, blockIdx.y * TILE,
+                                         blockIdx.x * TILE, true, s_list, &s_n);
+    if (n == 0) return;
+    const int C = p.Ci;
+    const int grp = threadIdx.x / G, gl = threadIdx.x & (G - 1), groups = 256 / G;
+    const T *inb = in + (size_t)b * p.Hi * p.Wi * C;
+    const T *pvb = MAX ? prev + (size_t)b * p.Hi * p.Wi * C : nullptr;
+    const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
+    for (int idx = grp; idx < n; idx += groups) {
+        const int code = s_list[idx];
+        const int oy = code >> 16, ox = code & 0xffff;
+        for (int c = gl * N; c < C; c += G * N) {
+            float hi[N], hp[N];
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                hi[j] = MAX ? -INFINITY : 0.f;
+                hp[j] = -INFINITY;
+            }
+            for (int ky = 0; ky < p.Kh; ++ky) {
+                const int iy = oy * p.sh - p.pt + ky * p.dh;
+                if (iy < 0) continue;
+                if (iy >= p.Hi) {
+                    if (MAX && q.zero_bottom && iy < p.Hi + q.pb) {
+#pragma unroll
+                        for (int j = 0; j < N; ++j) {
+                            hi[j] = fmaxf(hi[j], 0.f);
+                            hp[j] = fmaxf(hp[j], 0.f);
+                        }
+                    }
+                    continue;
+                }
+                for (int kx = 0; kx < p.Kw; ++kx) {
+                    const int ix = ox * p.sw - p.pl + kx * p.dw;
+                    if (ix < 0) continue;
+                    if (ix >= p.Wi) {
+                        if (MAX && q.zero_right && ix < p.Wi + q.pr) {
+#pragma unroll
+                            for (int j = 0; j < N; ++j) {
+                                hi[j] = fmaxf(hi[j], 0.f);
+                                hp[j] = fmaxf(hp[j], 0.f);
+                            }
+                        }
+                        continue;
+                    }
+                    const int ip = iy * p.Wi + ix;
+                    const bool act = mb[ip] != 0;
+                    if (!MAX && !act) continue;
+                    Vec<T, N> d;
+#pragma unroll
+                    for (int j = 0; j < N; ++j) d.v[j] = T(0);
+                    if (act) d = vload<T, N>(inb + (size_t)ip * C + c);
+                    if (MAX) {
+                        Vec<T, N> pv = vload<T, N>(pvb + (size_t)ip * C + c);
+#pragma unroll
+                        for (int j = 0; j < N; ++j) {
+                            float pf = float(pv.v[j]);
+                            hi[j] = fmaxf(hi[j], float(d.v[j]) + pf);
+                            hp[j] = fmaxf(hp[j], pf);
+                        }
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < N; ++j) hi[j] += float(d.v[j]);
+                    }
+                }
+            }
+            Vec<T, N> r;
+            const float area = float(p.Kh * p.Kw);
+#pragma unroll
+            for (int j = 0; j < N; ++j) r.v[j] = MAX ? T(hi[j] - hp[j]) : T(hi[j] / area);
+            vstore<T, N>(out + (((size_t)b * p.Ho + oy) * p.Wo + ox) * C + c, r);
+        }
+    }
+}
+
+// 1x1 output: grid (channel slices, batch); a workgroup's 4 wavefronts stride over the window
+// taps, each lane owns one channel, partial results meet in LDS.
+template <typename T, bool MAX>
+__global__ void __launch_bounds__(256)
+pool_global_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restrict__ prev,
+                   float *__restrict__ out, const int32_t *__restrict__ mask,
+                   int32_t *__restrict__ out_mask) {
+    __shared__ float s_hi[4][WAVE], s_hp[4][WAVE];
+    __shared__ int s_any[4];
+    const int b = blockIdx.y;
+    const int C = p.Ci;
+    const int c = blockIdx.x * WAVE + lane_id();
+    const int wave = threadIdx.x / WAVE;
+    const int npx = p.Hi * p.Wi;
+    const int K2 = p.Kh * p.Kw;
+    const T *inb = in + (size_t)b * npx * C;
+    const T *pvb = MAX ? prev + (size_t)b * npx * C : nullptr;
+    const int32_t *mb = mask + (size_t)b * npx;
+    float hi = MAX ? -INFINITY : 0.f, hp = -INFINITY;
+    int any = 0;
+    for (int tap = wave; tap < K2; tap += 4) {
+        const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
+        const int iy = ky * p.dh - p.pt, ix = kx * p.dw - p.pl;
+        if (iy < 0 || ix < 0) continue;
+        if (iy >= p.Hi || ix >= p.Wi) {
+            const bool zero = iy >= p.Hi ? (q.zero_bottom && iy < p.Hi + q.pb)
+                                         : (q.zero_right && ix < p.Wi + q.pr);
+            if (MAX && zero) {
+                hi = fmaxf(hi, 0.f);
+                hp = fmaxf(hp, 0.f);
+            }
+            continue;
+        }
+        const int ip = iy * p.Wi + ix;
+        const bool act = mb[ip] != 0;  // wave-uniform
+        any |= act ? 1 : 0;
+        if (c >= C) continue;
+        if (MAX) {
+            float pf = float(pvb[(size_t)ip * C + c]);
+            float d = act ? float(inb[(size_t)ip * C + c]) : 0.f;
+            hi = fmaxf(hi, d + pf);
+            hp = fmaxf(hp, pf);
+        } else if (act) {
+            hi += float(inb[(size_t)ip * C + c]);
+        }
+    }
+    s_hi[wave][lane_id()] = hi;
+    s_hp[wave][lane_id()] = hp;
+    if (lane_id() == 0) s_any[wave] = any;
+    __syncthreads();
+    if (wave == 0) {
+        for (int w = 1; w < 4; ++w) {
+            if (MAX) {
+                hi = fmaxf(hi, s_hi[w][lane_id()]);
+                hp = fmaxf(hp, s_hp[w][lane_id()]);
+            } else {
+                hi += s_hi[w][lane_id()];
+            }
+            any |= s_any[w];
+        }
+        if (c < C) out[(size_t)b * C + c] = any ? (MAX ? hi - hp : hi / float(K2)) : 0.f;
+        if (blockIdx.x == 0 && lane_id() == 0 && out_mask != nullptr) out_mask[b] = any;
+    }
+}
+
+template <typename T>
+hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, const int32_t *mask,
+                  int32_t *out_mask, int mode, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    ConvP p;
+    p.B = g.batch; p.Hi = g.in_h; p.Wi = g.in_w; p.Ci = g.in_c;
+    p.Ho = g.out_h; p.Wo = g.out_w; p.Co = g.in_c;
+    p.Kh = g.kernel_h; p.Kw = g.kernel_w; p.sh = g.stride_h; p.sw = g.stride_w;
+    p.dh = g.dilation_h; p.dw = g.dilation_w; p.pt = g.pad_top; p.pl = g.pad_left;
+    p.ci_g = p.co_g = 1; p.w_co = 0; p.swz = 0;
+    PoolQ q;
+    q.pb = g.pad_bottom; q.pr = g.pad_right;
+    q.zero_bottom = g.pad_top != g.pad_bottom;
+    q.zero_right = g.pad_left != g.pad_right;
+    if (g.out_h == 1 && g.out_w == 1) {
+        dim3 grid(ceil_div(g.in_c, WAVE), g.batch);
+        if (mode == DC_POOL_MAX)
+            pool_global_kernel<T, true><<<grid, 256, 0, s>>>(p, q, in, prev, (float *)out, mask, out_mask);
+        else
+            pool_global_kernel<T, false><<<grid, 256, 0, s>>>(p, q, in, prev, (float *)out, mask, out_mask);
+        return hipGetLastError();
+    }
+    dim3 grid(ceil_div(g.out_w, TILE), ceil_div(g.out_h, TILE), g.batch);
+    const bool vec = g.in_c % N == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
+                     ((uintptr_t)prev & 15) == 0;
+    int G = pow2_ceil(vec ? g.in_c / N : g.in_c);
+    if (G > WAVE) G = WAVE;
+#define DC_POOL(NN, MX) pool_window_kernel<T, NN, MX><<<grid, 256, 0, s>>>(p, q, in, prev, (T *)out, mask, out_mask, G)
+    if (mode == DC_POOL_MAX) {
+        if (vec) DC_POOL(N, true); else DC_POOL(1, true);
+    } else {
+        if (vec) DC_POOL(N, false); else DC_POOL(1, false);
+    }
+#undef DC_POOL
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_pool(const dc_geometry &g, const void *in, const void *prev, void *out,
+                       const int32_t *mask, int32_t *out_mask, int mode, int dtype, hipStream_t s) {
+    if (dtype == DC_F32)
+        return pool_t<float>(g, (const float *)in, (const float *)prev, out, mask, out_mask, mode, s);
+    return pool_t<half_t>(g, (const half_t *)in, (const half_t *)prev, out, mask, out_mask, mode, s);
+}
+
+}  // namespace dc

@@ -1,0 +1,289 @@
+"""Functional wrappers over libdeltacnn_hip.so with the names, argument order and defaults
+of the reference's ``src/deltacnn/cuda_kernels.py``: shape arithmetic, output allocation
+(NHWC / ``torch.channels_last`` features, int32 ``[B,1,H,W]`` masks) and the C-ABI call on
+torch's current stream.  Tensors are borrowed for the asynchronous launch; nothing
+synchronises.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+from ._lib import DC_F16, DC_F32, Geometry
+
+_DTYPES = {torch.float32: DC_F32, torch.float16: DC_F16}
+
+
+def _dtype(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise _lib.DeltaCNNError(-1, f"unsupported dtype {t.dtype} (float32 and float16 only)")
+
+
+def _nhwc(t: torch.Tensor, name: str) -> torch.Tensor:
+    """The kernels index features as [B][H][W][C]; refuse anything else instead of guessing."""
+    if t.dim() != 4 or not t.is_contiguous(memory_format=torch.channels_last):
+        raise _lib.DeltaCNNError(-2, f"{name} must be a 4-d channels_last tensor, got shape "
+                                     f"{tuple(t.shape)} strides {t.stride()}")
+    if not t.is_cuda:
+        raise _lib.DeltaCNNError(-4, f"{name} must live on the GPU")
+    return t
+
+
+def _mask(m: torch.Tensor, name: str) -> torch.Tensor:
+    if m.dtype != torch.int32 or not m.is_cuda or not (m.is_contiguous() or m.is_contiguous(
+            memory_format=torch.channels_last)):
+        raise _lib.DeltaCNNError(-2, f"{name} must be a dense int32 GPU tensor")
+    return m
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _pixels(t: torch.Tensor) -> int:
+    return t.shape[0] * t.shape[2] * t.shape[3]
+
+
+def _pad4(padding: Sequence[int]):
+    """(top, bottom, left, right), cuda_kernels.py:21-26."""
+    if len(padding) == 2:
+        return padding[0], padding[0], padding[1], padding[1]
+    if len(padding) == 4:
+        return tuple(padding)
+    raise ValueError("Padding must be iterable of size 2 or 4")
+
+
+def new_features(b, c, h, w, dtype, device) -> torch.Tensor:
+    return torch.empty((b, c, h, w), dtype=dtype, device=device, memory_format=torch.channels_last)
+
+
+def new_mask(b, h, w, device) -> torch.Tensor:
+    return torch.empty((b, 1, h, w), dtype=torch.int32, device=device)
+
+
+def conv_geometry(x_shape, kernel, c_out, stride, padding, dilation, groups, transposed=False,
+                  out_hw=None) -> Geometry:
+    b, c_in, h, w = x_shape
+    t, bt, l, r = _pad4(padding)
+    if out_hw is None:
+        if transposed:
+            oh = (h - 1) * stride[0] - 2 * t + dilation[0] * (kernel[0] - 1) + 1
+            ow = (w - 1) * stride[1] - 2 * l + dilation[1] * (kernel[1] - 1) + 1
+        else:
+            oh = (h + t + bt - dilation[0] * (kernel[0] - 1) - 1) // stride[0] + 1
+            ow = (w + l + r - dilation[1] * (kernel[1] - 1) - 1) // stride[1] + 1
+    else:
+        oh, ow = out_hw
+    return Geometry(b, h, w, c_in, oh, ow, c_out, kernel[0], kernel[1], stride[0], stride[1],
+                    dilation[0], dilation[1], t, l, bt, r, groups)
+
+
+def _conv_like(transposed, x, filter, mask, bias, stride, padding, dilation, groups, c_out,
+               create_out_mask, out_mask, out_shape, packed_filter, out, geometry, epilogue=None):
+    lib = _lib.load()
+    _nhwc(x, "x")
+    if mask is None:
+        raise _lib.DeltaCNNError(-4, "the delta kernels need an update mask (mask=None is the "
+                                     "dense path of the reference and is not part of this library)")
+    _mask(mask, "mask")
+    out_c = filter.shape[3] if c_out is None else c_out
+    g = geometry
+    if g is None:
+        hw = tuple(out_shape) if out_shape is not None and len(out_shape) == 2 else None
+        g = conv_geometry(x.shape, (filter.shape[1], filter.shape[2]), out_c, stride, padding,
+                          dilation, groups, transposed, hw)
+        if isinstance(out_shape, list) and len(out_shape) == 0:
+            out_shape.extend([g.out_h, g.out_w])
+    if out is None:
+        out = new_features(g.batch, out_c, g.out_h, g.out_w, x.dtype, x.device)
+    if out_mask is None:
+        out_mask = new_mask(g.batch, g.out_h, g.out_w, x.device)
+    dt = _dtype(x)
+    if epilogue is not None:
+        prev, trunc, thr, act, mode = epilogue
+        rc = lib.dc_conv_act(g, x.data_ptr(), filter.data_ptr(), _ptr(packed_filter), _ptr(bias),
+                             out.data_ptr(), mask.data_ptr(), out_mask.data_ptr(), prev.data_ptr(),
+                             _ptr(trunc), thr, act, mode, dt, _stream())
+    else:
+        fn = lib.dc_deconv if transposed else lib.dc_conv
+        rc = fn(g, x.data_ptr(), filter.data_ptr(), _ptr(packed_filter), _ptr(bias), out.data_ptr(),
+                mask.data_ptr(), out_mask.data_ptr(), dt, _stream())
+    _lib.check(rc)
+    if create_out_mask:
+        return out, out_mask
+    return out
+
+
+def sparse_conv(x, filter, mask=None, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
+                groups=1, c_out: int = None, create_out_mask=False, sub_tile_sparsity=True,
+                out_mask=None, out_shape=None, *, packed_filter=None, out=None, geometry=None):
+    """cuda_kernels.py:13-45.  ``filter`` is in the layout of ``process_filters()``.
+
+    Keyword-only extras: ``packed_filter`` (from :func:`pack_filter`) selects the MFMA
+    kernels, ``out`` / ``geometry`` let a layer reuse its buffers.
+    """
+    return _conv_like(False, x, filter, mask, bias, stride, padding, dilation, groups, c_out,
+                      create_out_mask, out_mask, out_shape, packed_filter, out, geometry)
+
+
+def sparse_conv_activation(x, filter, mask, bias, prev_out, truncated, threshold, activation,
+                           truncation_mode, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
+                           groups=1, c_out=None, *, packed_filter=None, out=None, out_mask=None,
+                           geometry=None):
+    """``sparse_conv`` followed by ``sparse_activation`` on its output in one library call."""
+    return _conv_like(False, x, filter, mask, bias, stride, padding, dilation, groups, c_out, True,
+                      out_mask, None, packed_filter, out, geometry,
+                      (prev_out, truncated, float(threshold), int(activation), int(truncation_mode)))
+
+
+def sparse_deconv(x, filter, mask=None, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
+                  groups=1, c_out: int = None, create_out_mask=False, sub_tile_sparsity=True,
+                  out_mask=None, out_shape=None, *, packed_filter=None, out=None, geometry=None):
+    """cuda_kernels.py:47-78."""
+    if len(padding) != 2:
+        raise ValueError("Padding must be iterable of size 2")
+    return _conv_like(True, x, filter, mask, bias, stride, padding, dilation, groups, c_out,
+                      create_out_mask, out_mask, out_shape, packed_filter, out, geometry)
+
+
+def pack_filter(filter: torch.Tensor, c_in: int, c_out: int, groups: int = 1,
+                transposed: bool = False) -> Optional[torch.Tensor]:
+    """One-time relayout of a processed fp16 filter for the MFMA kernels; None if the shape
+    has no packed form (fp32, grouped, Cin % 8 != 0)."""
+    lib = _lib.load()
+    if filter.dtype != torch.float16:
+        return None
+    g = Geometry(1, 1, 1, c_in, 1, 1, c_out, filter.shape[1], filter.shape[2], 1, 1, 1, 1, 0, 0, 0,
+                 0, groups)
+    nbytes = lib.dc_packed_filter_bytes(g, DC_F16, int(transposed))
+    if nbytes == 0:
+        return None
+    packed = torch.empty(nbytes // 2, dtype=torch.float16, device=filter.device)
+    _lib.check(lib.dc_pack_filter(g, filter.data_ptr(), packed.data_ptr(), DC_F16, int(transposed),
+                                  _stream()))
+    return packed
+
+
+def sparse_pooling(x, prev_x, kernel_size, mask=None, stride=(1, 1), padding=(0, 0),
+                   dilation=(1, 1), create_out_mask=True, sub_tile_sparsity=True, out_mask=None,
+                   pooling_mode_int=0, out_shape=None, *, out=None):
+    """cuda_kernels.py:80-129.  A 1x1 output is accumulated in a float32 buffer and cast
+    back to the input dtype afterwards (:101-124)."""
+    lib = _lib.load()
+    _nhwc(x, "x")
+    if mask is None:
+        raise _lib.DeltaCNNError(-4, "sparse_pooling needs an update mask")
+    hw = tuple(out_shape) if out_shape is not None and len(out_shape) == 2 else None
+    g = conv_geometry(x.shape, kernel_size, x.shape[1], stride, padding, dilation, 1, False, hw)
+    if isinstance(out_shape, list) and len(out_shape) == 0:
+        out_shape.extend([g.out_h, g.out_w])
+    is_global = g.out_h == 1 and g.out_w == 1
+    if out is None:
+        odt = torch.float32 if is_global else x.dtype
+        out = new_features(g.batch, x.shape[1], g.out_h, g.out_w, odt, x.device)
+    if out_mask is None:
+        out_mask = new_mask(g.batch, g.out_h, g.out_w, x.device)
+    _lib.check(lib.dc_pool(g, x.data_ptr(), _ptr(prev_x), out.data_ptr(), _mask(mask, "mask").data_ptr(),
+                           out_mask.data_ptr(), int(pooling_mode_int), _dtype(x), _stream()))
+    if out.dtype != x.dtype:
+        out = out.to(dtype=x.dtype)
+    if create_out_mask:
+        return out, out_mask
+    return out
+
+
+def sparse_activation(x, prev_x, truncated, mask, threshold, activation, truncation_mode):
+    """cuda_kernels.py:132-133; in place on ``x``, ``prev_x``, ``truncated`` and ``mask``."""
+    lib = _lib.load()
+    _nhwc(x, "x")
+    _lib.check(lib.dc_activate_truncate(x.data_ptr(), prev_x.data_ptr(), _ptr(truncated),
+                                        _mask(mask, "mask").data_ptr(), float(threshold),
+                                        int(activation), int(truncation_mode), _pixels(x),
+                                        x.shape[1], _dtype(x), _stream()))
+
+
+def sparsify(input, prev_in, delta, mask, threshold):
+    """cuda_kernels.py:136-137."""
+    lib = _lib.load()
+    _nhwc(input, "input")
+    _nhwc(delta, "delta")
+    _lib.check(lib.dc_sparsify(input.data_ptr(), prev_in.data_ptr(), delta.data_ptr(),
+                               _mask(mask, "mask").data_ptr(), float(threshold), _pixels(input),
+                               input.shape[1], _dtype(input), _stream()))
+
+
+def sparse_add_tensors(a, b, prev_out, out, mask_a, mask_b, mask_out, weight_a, weight_b,
+                       activation, dense_out):
+    """cuda_kernels.py:140-141."""
+    lib = _lib.load()
+    _nhwc(a, "a")
+    _nhwc(b, "b")
+    if a.shape != b.shape:
+        raise _lib.DeltaCNNError(-2, f"shape mismatch {tuple(a.shape)} vs {tuple(b.shape)}")
+    _lib.check(lib.dc_add(a.data_ptr(), b.data_ptr(), _ptr(prev_out), out.data_ptr(),
+                          _mask(mask_a, "mask_a").data_ptr(), _mask(mask_b, "mask_b").data_ptr(),
+                          _ptr(mask_out), float(weight_a), float(weight_b), int(activation),
+                          int(bool(dense_out)), _pixels(a), a.shape[1], _dtype(a), _stream()))
+
+
+def sparse_add_to_dense_tensor(a, b, mask_a, activation=0):
+    """cuda_kernels.py:144-145: ``b[px] += a[px]`` on active pixels."""
+    lib = _lib.load()
+    _nhwc(a, "a")
+    _lib.check(lib.dc_add_to_dense(a.data_ptr(), b.data_ptr(), _mask(mask_a, "mask_a").data_ptr(),
+                                   int(activation), _pixels(a), a.shape[1], _dtype(a), _stream()))
+
+
+def sparse_mul_add(x, x_mask, out, out_mask, scale, bias):
+    """cuda_kernels.py:148-149: per-channel ``x*scale (+bias)`` on active pixels."""
+    lib = _lib.load()
+    _nhwc(x, "x")
+    scale = scale.reshape(-1).to(x.dtype).contiguous()
+    bias = None if bias is None else bias.reshape(-1).to(x.dtype).contiguous()
+    _lib.check(lib.dc_mul_add(x.data_ptr(), _mask(x_mask, "x_mask").data_ptr(), out.data_ptr(),
+                              out_mask.data_ptr(), scale.data_ptr(), _ptr(bias), _pixels(x),
+                              x.shape[1], _dtype(x), _stream()))
+
+
+def sparse_upsample(input, mask_in, scale, out=None):
+    """cuda_kernels.py:152-167."""
+    lib = _lib.load()
+    _nhwc(input, "input")
+    b, c, h, w = input.shape
+    scale = int(scale)
+    if out is None:
+        out_t = new_features(b, c, h * scale, w * scale, input.dtype, input.device)
+        mask_out = new_mask(b, h * scale, w * scale, input.device)
+    else:
+        out_t, mask_out = out
+    _lib.check(lib.dc_upsample(input.data_ptr(), out_t.data_ptr(), _mask(mask_in, "mask_in").data_ptr(),
+                               mask_out.data_ptr(), b, h, w, c, scale, _dtype(input), _stream()))
+    return out_t, mask_out
+
+
+def sparse_concatenate(a, b, out=None):
+    """cuda_kernels.py:170-185."""
+    lib = _lib.load()
+    a, mask_a = a
+    b, mask_b = b
+    _nhwc(a, "a")
+    _nhwc(b, "b")
+    if out is None:
+        out_t = new_features(a.shape[0], a.shape[1] + b.shape[1], a.shape[2], a.shape[3], a.dtype,
+                             a.device)
+        mask_out = new_mask(a.shape[0], a.shape[2], a.shape[3], a.device)
+    else:
+        out_t, mask_out = out
+    _lib.check(lib.dc_concat(a.data_ptr(), b.data_ptr(), out_t.data_ptr(),
+                             _mask(mask_a, "mask_a").data_ptr(), _mask(mask_b, "mask_b").data_ptr(),
+                             mask_out.data_ptr(), _pixels(a), a.shape[1], b.shape[1], _dtype(a),
+                             _stream()))
+    return out_t, mask_out

@@ -1,0 +1,155 @@
+/*
+ * deltacnn_hip.h -- C ABI of libdeltacnn_hip.so: DeltaCNN's sparse delta-propagation
+ * operators as hand-written gfx950 (MI355X) HIP kernels.
+ *
+ * Every entry point replaces one function of the reference's pybind11 module
+ * `deltacnn.cuda` (src/cuda/conv_torch_wrapper.cpp:640-655).  Conventions:
+ *
+ *   - feature tensors are NHWC (torch.channels_last) device pointers, element type
+ *     given by `dtype` (DC_F32 or DC_F16); masks are dense int32 [B*H*W] device
+ *     pointers, a pixel is active iff its word != 0
+ *   - the library never allocates, frees or retains memory; pointers are borrowed
+ *     for the duration of the asynchronous launch on `stream` (a hipStream_t, NULL =
+ *     default stream); no entry point synchronises
+ *   - values of inactive pixels are never read; outputs are written only for pixels
+ *     whose output mask is 1 (the reference additionally writes the inactive pixels
+ *     of partially active tiles, conv_kernel.cu:348-356; nothing downstream reads them)
+ *   - return value: DC_OK or a negative dc_status; dc_last_error() gives the message
+ *     of the calling thread's last failure.  All argument checks run before the first
+ *     HIP call, so they can be exercised without a GPU.
+ */
+#ifndef DELTACNN_HIP_H
+#define DELTACNN_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum dc_status {
+    DC_OK = 0,
+    DC_ERR_DTYPE = -1,       /* dtype not DC_F32 / DC_F16 */
+    DC_ERR_SHAPE = -2,       /* non-positive or inconsistent dimensions */
+    DC_ERR_UNSUPPORTED = -3, /* valid but not implemented configuration */
+    DC_ERR_NULL = -4,        /* required pointer is NULL */
+    DC_ERR_ALIGN = -5,       /* pointer not aligned to its element / vector size */
+    DC_ERR_LAUNCH = -6       /* HIP reported a launch error */
+} dc_status;
+
+enum { DC_F32 = 0, DC_F16 = 1 };
+
+/* activation ids of convert_activation_string (sparse_layers.py:20-34); <= 0 is linear */
+enum { DC_ACT_LINEAR = 0, DC_ACT_RELU = 1, DC_ACT_RELU6 = 2, DC_ACT_LEAKY = 3,
+       DC_ACT_SIGMOID = 4, DC_ACT_SWISH = 5 };
+
+/* DCTruncation (sparse_layers.py:102-106) */
+enum { DC_TRUNC_NONE = -1, DC_TRUNC_MAX = 0, DC_TRUNC_NORM = 1, DC_TRUNC_RMS = 2 };
+
+/* pooling_mode of sparse_pooling_wrapper_masked (conv_torch_wrapper.cpp:213-226) */
+enum { DC_POOL_MAX = 0, DC_POOL_AVG = 1 };
+
+/* Geometry of a (transposed) convolution or pooling window.  Mirrors the reference's
+ * Dimensions + ConvConfig structs (src/cuda/common.cuh:12-35) with 32-bit fields and
+ * padding in (top, left, bottom, right) order like conv_torch_wrapper.cpp:43-53. */
+typedef struct dc_geometry {
+    int32_t batch;
+    int32_t in_h, in_w, in_c;
+    int32_t out_h, out_w, out_c;
+    int32_t kernel_h, kernel_w;
+    int32_t stride_h, stride_w;
+    int32_t dilation_h, dilation_w;
+    int32_t pad_top, pad_left, pad_bottom, pad_right;
+    int32_t groups;
+} dc_geometry;
+
+const char *dc_version(void);
+const char *dc_last_error(void);
+
+/* Replaces deltacnn_prepare_diff_mask_wrapper (conv_torch_wrapper.cpp:347-384).
+ * delta = input - prev_input; active pixels get delta and prev_input := input on all
+ * channels; mask is written for every pixel. */
+int dc_sparsify(const void *input, void *prev_input, void *delta, int32_t *mask,
+                float threshold, int32_t pixels, int32_t channels, int dtype, void *stream);
+
+/* Replaces deltacnn_activate_truncate (conv_torch_wrapper.cpp:295-344).  In place on delta,
+ * prev_input, truncated and mask.  truncation_mode < 0 accumulates delta into prev_input
+ * (densify); `truncated` may then be NULL. */
+int dc_activate_truncate(void *delta, void *prev_input, void *truncated, int32_t *mask,
+                         float threshold, int activation, int truncation_mode,
+                         int32_t pixels, int32_t channels, int dtype, void *stream);
+
+/* Replaces sparse_conv_bias_wrapper_masked (conv_torch_wrapper.cpp:62-134).
+ * `filter` is in the reference layout produced by process_filters(): fp32
+ * [Cin/g][Kh][Kw][Cout]; fp16 the same with Cin and Cout padded to even and the 2x2
+ * channel-pair swizzle of filter_conversion.py:13-38 (depthwise: unpadded, unswizzled).
+ * `packed_filter` (optional, may be NULL) is the output of dc_pack_filter for the same
+ * filter; when given, eligible shapes run on the MFMA kernels.
+ * `bias` may be NULL.  groups must be 1 or in_c == out_c (depthwise). */
+int dc_conv(const dc_geometry *g, const void *input, const void *filter,
+            const void *packed_filter, const void *bias, void *out, const int32_t *mask,
+            int32_t *out_mask, int dtype, void *stream);
+
+/* Fused conv + activation/truncation epilogue: dc_conv followed by dc_activate_truncate on
+ * the conv output, in one launch where one workgroup owns all output channels of its
+ * pixels.  No counterpart in the reference (it launches the two kernels separately,
+ * sparse_layers.py:636-638); results are identical to the two-call sequence. */
+int dc_conv_act(const dc_geometry *g, const void *input, const void *filter,
+                const void *packed_filter, const void *bias, void *out, const int32_t *mask,
+                int32_t *out_mask, void *prev_out, void *truncated, float threshold,
+                int activation, int truncation_mode, int dtype, void *stream);
+
+/* Number of bytes dc_pack_filter writes for this geometry (0 if the shape has no packed
+ * form).  One-time weight relayout for the MFMA kernels: [Cout pad 16][Kh][Kw][Cin pad 32]
+ * fp16, un-swizzled. */
+int64_t dc_packed_filter_bytes(const dc_geometry *g, int dtype, int transposed);
+int dc_pack_filter(const dc_geometry *g, const void *filter, void *packed_filter, int dtype,
+                   int transposed, void *stream);
+
+/* Replaces sparse_deconv_bias_wrapper_masked (conv_torch_wrapper.cpp:136-210).  `filter`
+ * layout [Cin][Kh][Kw][Cout] (fp16: padded + swizzled as for dc_conv).  Any kernel size /
+ * stride with groups == 1 (the reference supports only k4s2 and k6s4,
+ * deconv_kernel.cu:857,872). */
+int dc_deconv(const dc_geometry *g, const void *input, const void *filter,
+              const void *packed_filter, const void *bias, void *out, const int32_t *mask,
+              int32_t *out_mask, int dtype, void *stream);
+
+/* Replaces sparse_pooling_wrapper_masked (conv_torch_wrapper.cpp:213-293).  `prev_input` is
+ * required for DC_POOL_MAX.  When out_h == out_w == 1, `out` is float32 [B][C]
+ * irrespective of dtype (cuda_kernels.py:101-109) and is fully overwritten. */
+int dc_pool(const dc_geometry *g, const void *input, const void *prev_input, void *out,
+            const int32_t *mask, int32_t *out_mask, int pooling_mode, int dtype, void *stream);
+
+/* Replaces sparse_add_tensors_wrapper (conv_torch_wrapper.cpp:387-444). */
+int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_t *mask_a,
+           const int32_t *mask_b, int32_t *mask_out, float weight_a, float weight_b,
+           int activation, int dense_out, int32_t pixels, int32_t channels, int dtype,
+           void *stream);
+
+/* Replaces sparse_add_to_dense_tensor_wrapper (conv_torch_wrapper.cpp:447-482):
+ * b[px] += a[px] on active pixels.  With activation > 0 it also writes a = act(b) on every
+ * pixel (the USE_ACTIVATION variant, other_nn_layers.cu:1731-1957). */
+int dc_add_to_dense(void *a, void *b, const int32_t *mask_a, int activation, int32_t pixels,
+                    int32_t channels, int dtype, void *stream);
+
+/* Replaces sparse_upsample_wrapper (conv_torch_wrapper.cpp:484-522): nearest upsample by an
+ * integer factor. */
+int dc_upsample(const void *input, void *out, const int32_t *mask_in, int32_t *mask_out,
+                int32_t batch, int32_t in_h, int32_t in_w, int32_t channels, int32_t scale,
+                int dtype, void *stream);
+
+/* Replaces sparse_concatenate_wrapper (conv_torch_wrapper.cpp:524-567). */
+int dc_concat(const void *a, const void *b, void *out, const int32_t *mask_a,
+              const int32_t *mask_b, int32_t *mask_out, int32_t pixels, int32_t channels_a,
+              int32_t channels_b, int dtype, void *stream);
+
+/* Replaces sparse_mul_add_wrapper (conv_torch_wrapper.cpp:569-630): out = in*scale (+bias)
+ * per channel on active pixels; mask_out := mask when they are distinct buffers. */
+int dc_mul_add(const void *input, const int32_t *mask, void *out, int32_t *mask_out,
+               const void *scale, const void *bias, int32_t pixels, int32_t channels,
+               int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DELTACNN_HIP_H */

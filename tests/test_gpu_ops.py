@@ -1,0 +1,428 @@
+"""Operator-level parity: every C-ABI operator against the CPU oracle on identical seeded
+inputs.  Masks and pixel sets must match exactly; elementwise operators must match bit for
+bit; contractions within 1e-4 relative (fp32) / 2e-2 absolute (fp16).  Inactive pixels of
+every delta input are NaN-poisoned, so a kernel that reads them cannot pass.
+"""
+import pytest
+import torch
+
+from oracle import delta_ops as ops
+from util import DEV, assert_masked_close, assert_masked_equal, cl, poison, rand_mask
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16]
+CHANNELS = [1, 3, 4, 8, 16, 31, 32, 33, 64, 96, 130, 256, 960, 1280, 2100]
+
+
+def hk():
+    import deltacnn_amd.hip_kernels as m
+    return m
+
+
+def _gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ------------------------------------------------------------------------------- sparsify
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", CHANNELS)
+def test_sparsify(lib, dtype, C):
+    g = _gen(100 + C)
+    B, H, W = 2, 13, 9
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+    x = prev.clone()
+    upd = rand_mask(g, B, H, W, 0.3) != 0
+    x = torch.where(upd, (x.float() + torch.randn(B, C, H, W, generator=g) * 0.5).to(dtype), x)
+    # ties: a pixel whose largest |difference| equals the threshold exactly
+    thr = 0.25
+    x[0, :, 0, 0] = prev[0, :, 0, 0]
+    x[0, 0, 0, 0] = 1.0
+    prev[0, 0, 0, 0] = 0.75
+    want_prev = prev.clone()
+    want_delta, want_mask = ops.sparsify(x, want_prev, thr)
+
+    d_prev, d_x = cl(prev), cl(x)
+    d_delta = torch.full_like(d_x, float("nan"))
+    d_mask = torch.full((B, 1, H, W), -7, dtype=torch.int32, device=DEV)
+    hk().sparsify(d_x, d_prev, d_delta, d_mask, thr)
+    assert torch.equal(d_mask.cpu(), want_mask)
+    assert_masked_equal(d_delta, want_delta, want_mask, "delta")
+    assert torch.equal(d_prev.cpu(), want_prev)
+    # inactive pixels of delta are not written
+    assert bool(d_delta.cpu()[(want_mask == 0).expand_as(want_delta)].isnan().all())
+
+
+# ------------------------------------------------------------------ activation + truncation
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", CHANNELS)
+@pytest.mark.parametrize("act", [1, 2, 3])
+def test_activate_truncate_max(lib, dtype, C, act):
+    g = _gen(200 + C + act)
+    B, H, W = 2, 11, 7
+    mask = rand_mask(g, B, H, W, 0.5)
+    scale = 3.0 if act == 2 else 1.0
+    prev = (torch.randn(B, C, H, W, generator=g) * scale).to(dtype)
+    trunc = (torch.randn(B, C, H, W, generator=g) * 0.005).to(dtype)
+    big = rand_mask(g, B, H, W, 0.5).float()
+    delta = (torch.randn(B, C, H, W, generator=g) * (0.005 + 0.5 * big)).to(dtype)
+    thr = 0.1
+    w_delta, w_prev, w_trunc, w_mask = delta.clone(), prev.clone(), trunc.clone(), mask.clone()
+    ops.activate_truncate(w_delta, w_prev, w_trunc, w_mask, thr, act, 0)
+    assert 0 < int(w_mask.sum()) < int(mask.sum())
+
+    d_delta, d_prev, d_trunc, d_mask = cl(poison(delta, mask)), cl(prev), cl(trunc), cl(mask)
+    hk().sparse_activation(d_delta, d_prev, d_trunc, d_mask, thr, act, 0)
+    assert torch.equal(d_mask.cpu(), w_mask)
+    assert_masked_equal(d_delta, w_delta, w_mask, "delta")
+    assert torch.equal(d_prev.cpu(), w_prev)
+    assert torch.equal(d_trunc.cpu(), w_trunc)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("act", [4, 5])
+def test_activate_truncate_transcendental(lib, dtype, act):
+    """sigmoid / swish go through exp: tolerance instead of bit equality, ties excluded."""
+    g = _gen(300 + act)
+    B, C, H, W = 1, 24, 9, 9
+    mask = rand_mask(g, B, H, W, 0.6)
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+    trunc = torch.zeros(B, C, H, W).to(dtype)
+    big = rand_mask(g, B, H, W, 0.5).float()
+    delta = (torch.randn(B, C, H, W, generator=g) * (0.001 + 2.0 * big)).to(dtype)
+    thr = 0.05
+    w_delta, w_prev, w_trunc, w_mask = delta.clone(), prev.clone(), trunc.clone(), mask.clone()
+    ops.activate_truncate(w_delta, w_prev, w_trunc, w_mask, thr, act, 0)
+    d_delta, d_prev, d_trunc, d_mask = cl(poison(delta, mask)), cl(prev), cl(trunc), cl(mask)
+    hk().sparse_activation(d_delta, d_prev, d_trunc, d_mask, thr, act, 0)
+    assert torch.equal(d_mask.cpu(), w_mask)
+    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    assert_masked_close(d_delta, w_delta, w_mask, tol, tol, "delta")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mode", [1, 2])
+@pytest.mark.parametrize("C", [8, 33, 96])
+def test_activate_truncate_norm_modes(lib, dtype, mode, C):
+    """norm / rms: pixels are either far above or far below the threshold."""
+    g = _gen(400 + mode + C)
+    B, H, W = 1, 10, 10
+    mask = rand_mask(g, B, H, W, 0.7)
+    prev = (torch.rand(B, C, H, W, generator=g) + 0.5).to(dtype)
+    trunc = torch.zeros(B, C, H, W).to(dtype)
+    big = rand_mask(g, B, H, W, 0.5).float()
+    delta = ((torch.rand(B, C, H, W, generator=g) + 0.5) * (1e-4 + 0.5 * big)).to(dtype)
+    thr = 0.2
+    w = [delta.clone(), prev.clone(), trunc.clone(), mask.clone()]
+    ops.activate_truncate(*w, thr, 1, mode)
+    d = [cl(poison(delta, mask)), cl(prev), cl(trunc), cl(mask)]
+    hk().sparse_activation(*d, thr, 1, mode)
+    assert torch.equal(d[3].cpu(), w[3])
+    assert_masked_equal(d[0], w[0], w[3], "delta")
+    assert torch.equal(d[1].cpu(), w[1])
+    assert torch.equal(d[2].cpu(), w[2])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [3, 17, 80, 84, 1280])
+@pytest.mark.parametrize("act", [-1, 1])
+def test_densify_accumulate(lib, dtype, C, act):
+    g = _gen(500 + C)
+    B, H, W = 2, 8, 12
+    mask = rand_mask(g, B, H, W, 0.4)
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+    delta = torch.randn(B, C, H, W, generator=g).to(dtype)
+    w_delta, w_prev = delta.clone(), prev.clone()
+    ops.activate_truncate(w_delta, w_prev, None, mask, -1, act, -1)
+    d_delta, d_prev, d_mask = cl(poison(delta, mask)), cl(prev), cl(mask)
+    hk().sparse_activation(d_delta, d_prev, None, d_mask, -1, act, -1)
+    assert torch.equal(d_prev.cpu(), w_prev)
+    assert_masked_equal(d_delta, w_delta, mask, "delta")
+    assert torch.equal(d_mask.cpu(), mask)
+
+
+# ------------------------------------------------------------------------------------ add
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [3, 16, 24, 33, 160, 2100])
+@pytest.mark.parametrize("act,dense_out", [(-1, False), (1, False), (-1, True), (2, True)])
+@pytest.mark.parametrize("weights", [(1.0, 1.0), (0.5, -1.25)])
+def test_add(lib, dtype, C, act, dense_out, weights):
+    g = _gen(600 + C)
+    B, H, W = 2, 9, 10
+    ma, mb = rand_mask(g, B, H, W, 0.4), rand_mask(g, B, H, W, 0.3)
+    a = torch.randn(B, C, H, W, generator=g).to(dtype)
+    b = torch.randn(B, C, H, W, generator=g).to(dtype)
+    need_prev = dense_out or act > 0
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype) if need_prev else None
+    w_prev = prev.clone() if need_prev else None
+    w_out, w_mask = ops.add(a, ma, b, mb, w_prev, weights[0], weights[1], act, dense_out)
+
+    d_prev = cl(prev) if need_prev else None
+    d_out = torch.full((B, C, H, W), float("nan"), dtype=dtype, device=DEV).contiguous(
+        memory_format=torch.channels_last)
+    d_mo = torch.full((B, 1, H, W), -3, dtype=torch.int32, device=DEV)
+    hk().sparse_add_tensors(cl(poison(a, ma)), cl(poison(b, mb)), d_prev, d_out, cl(ma), cl(mb), d_mo,
+                            weights[0], weights[1], act, dense_out)
+    if dense_out:
+        assert torch.equal(d_out.cpu(), w_out)
+    else:
+        assert torch.equal(d_mo.cpu(), w_mask)
+        assert_masked_equal(d_out, w_out, w_mask, "out")
+    if need_prev:
+        assert torch.equal(d_prev.cpu(), w_prev)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [5, 64])
+@pytest.mark.parametrize("act", [0, 1])
+def test_add_to_dense(lib, dtype, C, act):
+    g = _gen(700 + C)
+    B, H, W = 1, 7, 9
+    ma = rand_mask(g, B, H, W, 0.4)
+    a = torch.randn(B, C, H, W, generator=g).to(dtype)
+    b = torch.randn(B, C, H, W, generator=g).to(dtype)
+    w_b = b.clone()
+    ops.add_to_dense(a, w_b, ma)
+    d_a, d_b = cl(poison(a, ma)), cl(b)
+    hk().sparse_add_to_dense_tensor(d_a, d_b, cl(ma), act)
+    assert torch.equal(d_b.cpu(), w_b)
+    if act:
+        assert torch.equal(d_a.cpu(), ops.activation(w_b, act))
+
+
+# ------------------------------------------------------------------------------------ conv
+CONVS = [
+    # Cin, Cout, K, stride, padding, dilation, groups, H, W
+    (3, 16, 3, 1, 1, 1, 1, 17, 13),
+    (16, 32, 3, 1, 1, 1, 1, 16, 16),
+    (3, 32, 3, 2, 1, 1, 1, 33, 31),
+    (32, 32, 3, 1, 1, 1, 32, 15, 18),       # depthwise
+    (96, 96, 3, 2, 1, 1, 96, 19, 17),       # depthwise stride 2
+    (24, 24, 5, 1, 2, 1, 24, 12, 12),       # depthwise 5x5
+    (16, 96, 1, 1, 0, 1, 1, 14, 14),
+    (96, 24, 1, 1, 0, 1, 1, 9, 20),
+    (144, 32, 1, 1, 0, 1, 1, 7, 7),
+    (64, 64, 1, 2, 0, 1, 1, 11, 11),        # 1x1 stride 2 samples the mask
+    (32, 48, 3, 1, 2, 2, 1, 14, 15),        # dilation 2
+    (8, 8, 5, 2, 2, 1, 1, 13, 13),
+    (8, 16, 7, 1, 3, 1, 1, 12, 10),         # 7x7 stride 1 (not dispatched by the reference)
+    (3, 8, 7, 2, 3, 1, 1, 20, 22),
+    (16, 16, 3, 1, (0, 1, 1, 0), 1, 1, 9, 9),   # (top, bottom, left, right)
+    (40, 24, (1, 3), (1, 2), (0, 1), 1, 1, 8, 16),
+    (12, 18, 3, 1, 1, 1, 3, 8, 8),          # general groups (fp32 only)
+    (5, 7, 3, 1, 1, 1, 1, 9, 9),            # odd channels: fp16 padding rows/cols of the swizzle
+]
+
+
+def _pair(v):
+    return (v, v) if isinstance(v, int) else tuple(v)
+
+
+def _conv_case(dtype, cfg, seed, density, transposed=False):
+    from deltacnn_amd.filter_conversion import convert_filter_out_channels_last, convert_half_filter
+    Cin, Cout, K, s, p, d, groups, H, W = cfg
+    K, s, d = _pair(K), _pair(s), _pair(d)
+    p = _pair(p)
+    g = _gen(seed)
+    B = 2
+    mask = rand_mask(g, B, H, W, density)
+    x = torch.randn(B, Cin, H, W, generator=g).to(dtype)
+    if transposed:
+        wt = (torch.randn(Cin, Cout // groups, *K, generator=g) / (Cin * K[0] * K[1]) ** 0.5).to(dtype)
+    else:
+        wt = (torch.randn(Cout, Cin // groups, *K, generator=g) / (Cin // groups * K[0] * K[1]) ** 0.5).to(dtype)
+    bias = torch.randn(Cout, generator=g).to(dtype)
+    dw = groups == Cin == Cout and groups > 1
+    if dtype == torch.float16:
+        filt = convert_half_filter(wt, pixel_wise=dw, transposed=transposed)
+    else:
+        filt = convert_filter_out_channels_last(wt, transposed=transposed)
+    return x, mask, wt, bias, filt, (K, s, p, d, groups)
+
+
+def _check_conv(dtype, got, want, want_mask):
+    if dtype == torch.float32:
+        assert_masked_close(got, want, want_mask, 1e-4, 1e-5, "out")
+    else:
+        assert_masked_close(got, want, want_mask, 0, 2e-2, "out")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", CONVS, ids=lambda c: "-".join(str(v).replace(" ", "") for v in c))
+@pytest.mark.parametrize("density", [0.05, 0.5, 1.0])
+@pytest.mark.parametrize("use_bias", [False, True])
+@pytest.mark.parametrize("packed", [False, True])
+def test_conv(lib, dtype, cfg, density, use_bias, packed):
+    groups, Cin, Cout = cfg[6], cfg[0], cfg[1]
+    general_groups = groups > 1 and not (groups == Cin == Cout)
+    if general_groups and dtype == torch.float16:
+        pytest.skip("fp16 filter layout is defined for groups == 1 and depthwise only")
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 800 + Cin + Cout, density)
+    want, want_mask = ops.conv(x, mask, wt, bias if use_bias else None, s, p, d, groups)
+    d_filt = filt.to(DEV)
+    pk = None
+    if packed:
+        pk = hk().pack_filter(d_filt, Cin, Cout, groups)
+        if pk is None:
+            pytest.skip("no packed form for this shape")
+    out, om = hk().sparse_conv(cl(poison(x, mask)), d_filt, cl(mask), bias.to(DEV) if use_bias else None,
+                               s, p, d, groups, c_out=Cout, create_out_mask=True, packed_filter=pk)
+    assert out.shape == want.shape
+    assert torch.equal(om.cpu(), want_mask)
+    _check_conv(dtype, out, want, want_mask)
+
+
+DECONVS = [
+    (16, 8, 4, 2, 1, 1, 1, 9, 11),     # k4 s2 p1 (reference config)
+    (8, 8, 6, 4, 1, 1, 1, 6, 7),       # k6 s4 p1 (reference config)
+    (24, 16, 2, 2, 0, 1, 1, 7, 7),
+    (8, 12, 3, 1, 1, 1, 1, 8, 9),
+    (5, 3, 4, 2, 1, 1, 1, 6, 6),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", DECONVS, ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("density", [0.1, 1.0])
+@pytest.mark.parametrize("packed", [False, True])
+def test_deconv(lib, dtype, cfg, density, packed):
+    Cin, Cout = cfg[0], cfg[1]
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 900 + Cin, density, True)
+    want, want_mask = ops.deconv(x, mask, wt, bias, s, p, d, groups)
+    d_filt = filt.to(DEV)
+    pk = None
+    if packed:
+        pk = hk().pack_filter(d_filt, Cin, Cout, groups, transposed=True)
+        if pk is None:
+            pytest.skip("no packed form for this shape")
+    out, om = hk().sparse_deconv(cl(poison(x, mask)), d_filt, cl(mask), bias.to(DEV), s, p, d, groups,
+                                 c_out=Cout, create_out_mask=True, packed_filter=pk)
+    assert out.shape == want.shape
+    assert torch.equal(om.cpu(), want_mask)
+    _check_conv(dtype, out, want, want_mask)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_conv_activation_fused(lib, dtype):
+    """dc_conv_act == dc_conv followed by dc_activate_truncate."""
+    cfg = (32, 64, 1, 1, 0, 1, 1, 12, 12)
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 77, 0.4)
+    g = _gen(78)
+    x = (x.float() * (0.01 + rand_mask(g, 2, 12, 12, 0.5).float())).to(dtype)  # small and large updates
+    prev = torch.randn(2, 64, 12, 12, generator=g).to(dtype)
+    trunc = (torch.randn(2, 64, 12, 12, generator=g) * 0.01).to(dtype)
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, 32, 64, 1)
+    dx, dm = cl(poison(x, mask)), cl(mask)
+    out1, om1 = hk().sparse_conv(dx, d_filt, dm, None, s, p, d, groups, c_out=64, create_out_mask=True,
+                                 packed_filter=pk)
+    p1, t1 = cl(prev), cl(trunc)
+    hk().sparse_activation(out1, p1, t1, om1, 0.3, 2, 0)
+    p2, t2 = cl(prev), cl(trunc)
+    out2, om2 = hk().sparse_conv_activation(dx, d_filt, dm, None, p2, t2, 0.3, 2, 0, s, p, d, groups, 64,
+                                            packed_filter=pk)
+    assert torch.equal(om1, om2)
+    assert 0 < int(om1.sum()) < int(mask.sum())
+    assert torch.equal(p1, p2) and torch.equal(t1, t2)
+    assert_masked_equal(out2, out1.cpu(), om1.cpu(), "out")
+
+
+# --------------------------------------------------------------------------------- pooling
+POOLS = [
+    # C, K, stride, padding, dilation, H, W
+    (16, 2, 2, 0, 1, 12, 14),
+    (32, 3, 2, 1, 1, 13, 13),
+    (5, 3, 1, 1, 1, 9, 8),
+    (8, 2, 2, (0, 1, 0, 1), 1, 9, 9),     # asymmetric: zero joins the maximum
+    (24, 3, 1, 2, 2, 10, 10),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", POOLS, ids=lambda c: "-".join(str(v).replace(" ", "") for v in c))
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("density", [0.1, 0.6])
+def test_pool(lib, dtype, cfg, mode, density):
+    C, K, s, p, d, H, W = cfg
+    K, s, d, p = _pair(K), _pair(s), _pair(d), _pair(p)
+    g = _gen(1000 + C)
+    B = 2
+    mask = rand_mask(g, B, H, W, density)
+    x = torch.randn(B, C, H, W, generator=g).to(dtype)
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+    want, want_mask = ops.pool(x, prev if mode == 0 else None, mask, K, s, p, d, mode)
+    out, om = hk().sparse_pooling(cl(poison(x, mask)), cl(prev) if mode == 0 else None, K, cl(mask), s, p, d,
+                                  pooling_mode_int=mode)
+    assert torch.equal(om.cpu(), want_mask)
+    assert_masked_equal(out, want, want_mask, "out")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("C,H,W", [(1280, 7, 7), (17, 5, 9), (64, 16, 16)])
+@pytest.mark.parametrize("density", [0.0, 0.2, 1.0])
+def test_pool_global(lib, dtype, mode, C, H, W, density):
+    g = _gen(1100 + C)
+    B = 2
+    mask = rand_mask(g, B, H, W, density)
+    x = torch.randn(B, C, H, W, generator=g).to(dtype)
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+    want, want_mask = ops.pool(x, prev if mode == 0 else None, mask, (H, W), (1, 1), (0, 0), (1, 1), mode)
+    out, om = hk().sparse_pooling(cl(poison(x, mask)), cl(prev) if mode == 0 else None, (H, W), cl(mask),
+                                  pooling_mode_int=mode)
+    assert out.dtype == dtype and out.shape == (B, C, 1, 1)
+    assert torch.equal(om.cpu(), want_mask)
+    # the average is a float sum over up to H*W values in a different order than the oracle's
+    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    assert_masked_close(out, want, want_mask, tol, tol, "out")
+
+
+# ------------------------------------------------------------- upsample / concat / mul_add
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [3, 32, 72])
+@pytest.mark.parametrize("scale", [2, 4, 8])
+def test_upsample(lib, dtype, C, scale):
+    g = _gen(1200 + C)
+    B, H, W = 2, 6, 5
+    mask = rand_mask(g, B, H, W, 0.4)
+    x = torch.randn(B, C, H, W, generator=g).to(dtype)
+    want, want_mask = ops.upsample(x, mask, scale)
+    out, om = hk().sparse_upsample(cl(poison(x, mask)), cl(mask), scale)
+    assert torch.equal(om.cpu(), want_mask)
+    assert_masked_equal(out, want, want_mask, "out")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Ca,Cb", [(3, 5), (16, 32), (64, 24), (8, 3)])
+def test_concat(lib, dtype, Ca, Cb):
+    g = _gen(1300 + Ca)
+    B, H, W = 2, 7, 6
+    ma, mb = rand_mask(g, B, H, W, 0.4), rand_mask(g, B, H, W, 0.4)
+    a = torch.randn(B, Ca, H, W, generator=g).to(dtype)
+    b = torch.randn(B, Cb, H, W, generator=g).to(dtype)
+    want, want_mask = ops.concatenate(a, ma, b, mb)
+    out, om = hk().sparse_concatenate((cl(poison(a, ma)), cl(ma)), (cl(poison(b, mb)), cl(mb)))
+    assert torch.equal(om.cpu(), want_mask)
+    assert_masked_equal(out, want, want_mask, "out")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [3, 32, 100])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_mul_add(lib, dtype, C, with_bias):
+    g = _gen(1400 + C)
+    B, H, W = 2, 7, 6
+    mask = rand_mask(g, B, H, W, 0.5)
+    x = torch.randn(B, C, H, W, generator=g).to(dtype)
+    scale = torch.randn(C, generator=g).to(dtype)
+    bias = torch.randn(C, generator=g).to(dtype) if with_bias else None
+    want, want_mask = ops.mul_add(x, mask, scale, bias)
+    d_x, d_m = cl(poison(x, mask)), cl(mask)
+    out = torch.full_like(d_x, float("nan"))
+    om = torch.zeros_like(d_m)
+    hk().sparse_mul_add(d_x, d_m, out, om, scale.to(DEV), None if bias is None else bias.to(DEV))
+    assert torch.equal(om.cpu(), want_mask)
+    if dtype == torch.float32 and with_bias:
+        assert_masked_close(out, want, want_mask, 1e-6, 1e-6, "out")  # fma vs mul+add in fp64
+    else:
+        assert_masked_equal(out, want, want_mask, "out")
