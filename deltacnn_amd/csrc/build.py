@@ -46,7 +46,13 @@ def build(force: bool = False, verbose: bool = True) -> str:
     def run(cmd):
         if verbose:
             print(" ".join(cmd), flush=True)
-        subprocess.run(cmd, check=True)
+        r = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+        # the host pass does not know the device-only target feature; that line is harmless
+        err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+        if err.strip():
+            print(err, file=sys.stderr, flush=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed ({r.returncode}): {' '.join(cmd)}")
 
     with ThreadPoolExecutor(max_workers=min(4, max(1, len(jobs)))) as ex:
         list(ex.map(run, jobs))

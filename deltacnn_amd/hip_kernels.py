@@ -15,6 +15,23 @@ from ._lib import DC_F16, DC_F32, Geometry
 
 _DTYPES = {torch.float32: DC_F32, torch.float16: DC_F16}
 
+# Optional per-call tracer (see deltacnn_amd/trace.py): when set, every library call goes
+# through ``tracer.run(op, fn, args, meta)`` which brackets it with events and records the
+# shapes and mask populations that the algorithmic byte counts are computed from.
+_TRACER = None
+
+
+def set_tracer(tracer) -> None:
+    global _TRACER
+    _TRACER = tracer
+
+
+def _call(op, fn, args, **meta):
+    if _TRACER is None:
+        _lib.check(fn(*args))
+    else:
+        _lib.check(_TRACER.run(op, fn, args, meta))
+
 
 def _dtype(t: torch.Tensor) -> int:
     try:
@@ -107,16 +124,18 @@ def _conv_like(transposed, x, filter, mask, bias, stride, padding, dilation, gro
     if out_mask is None:
         out_mask = new_mask(g.batch, g.out_h, g.out_w, x.device)
     dt = _dtype(x)
+    meta = dict(g=g, esize=x.element_size(), in_mask=mask, out_mask=out_mask,
+                mfma=packed_filter is not None)
     if epilogue is not None:
         prev, trunc, thr, act, mode = epilogue
-        rc = lib.dc_conv_act(g, x.data_ptr(), filter.data_ptr(), _ptr(packed_filter), _ptr(bias),
-                             out.data_ptr(), mask.data_ptr(), out_mask.data_ptr(), prev.data_ptr(),
-                             _ptr(trunc), thr, act, mode, dt, _stream())
+        _call("conv_act", lib.dc_conv_act,
+              (g, x.data_ptr(), filter.data_ptr(), _ptr(packed_filter), _ptr(bias), out.data_ptr(),
+               mask.data_ptr(), out_mask.data_ptr(), prev.data_ptr(), _ptr(trunc), thr, act, mode,
+               dt, _stream()), **meta)
     else:
-        fn = lib.dc_deconv if transposed else lib.dc_conv
-        rc = fn(g, x.data_ptr(), filter.data_ptr(), _ptr(packed_filter), _ptr(bias), out.data_ptr(),
-                mask.data_ptr(), out_mask.data_ptr(), dt, _stream())
-    _lib.check(rc)
+        _call("deconv" if transposed else "conv", lib.dc_deconv if transposed else lib.dc_conv,
+              (g, x.data_ptr(), filter.data_ptr(), _ptr(packed_filter), _ptr(bias), out.data_ptr(),
+               mask.data_ptr(), out_mask.data_ptr(), dt, _stream()), **meta)
     if create_out_mask:
         return out, out_mask
     return out
@@ -191,8 +210,10 @@ def sparse_pooling(x, prev_x, kernel_size, mask=None, stride=(1, 1), padding=(0,
         out = new_features(g.batch, x.shape[1], g.out_h, g.out_w, odt, x.device)
     if out_mask is None:
         out_mask = new_mask(g.batch, g.out_h, g.out_w, x.device)
-    _lib.check(lib.dc_pool(g, x.data_ptr(), _ptr(prev_x), out.data_ptr(), _mask(mask, "mask").data_ptr(),
-                           out_mask.data_ptr(), int(pooling_mode_int), _dtype(x), _stream()))
+    _call("pool", lib.dc_pool,
+          (g, x.data_ptr(), _ptr(prev_x), out.data_ptr(), _mask(mask, "mask").data_ptr(),
+           out_mask.data_ptr(), int(pooling_mode_int), _dtype(x), _stream()),
+          g=g, esize=x.element_size(), in_mask=mask, out_mask=out_mask, mode=int(pooling_mode_int))
     if out.dtype != x.dtype:
         out = out.to(dtype=x.dtype)
     if create_out_mask:
@@ -204,10 +225,11 @@ def sparse_activation(x, prev_x, truncated, mask, threshold, activation, truncat
     """cuda_kernels.py:132-133; in place on ``x``, ``prev_x``, ``truncated`` and ``mask``."""
     lib = _lib.load()
     _nhwc(x, "x")
-    _lib.check(lib.dc_activate_truncate(x.data_ptr(), prev_x.data_ptr(), _ptr(truncated),
-                                        _mask(mask, "mask").data_ptr(), float(threshold),
-                                        int(activation), int(truncation_mode), _pixels(x),
-                                        x.shape[1], _dtype(x), _stream()))
+    _call("densify" if truncation_mode < 0 else "activate_truncate", lib.dc_activate_truncate,
+          (x.data_ptr(), prev_x.data_ptr(), _ptr(truncated), _mask(mask, "mask").data_ptr(),
+           float(threshold), int(activation), int(truncation_mode), _pixels(x), x.shape[1],
+           _dtype(x), _stream()),
+          P=_pixels(x), C=x.shape[1], esize=x.element_size(), in_mask=mask, out_mask=mask)
 
 
 def sparsify(input, prev_in, delta, mask, threshold):
@@ -215,9 +237,10 @@ def sparsify(input, prev_in, delta, mask, threshold):
     lib = _lib.load()
     _nhwc(input, "input")
     _nhwc(delta, "delta")
-    _lib.check(lib.dc_sparsify(input.data_ptr(), prev_in.data_ptr(), delta.data_ptr(),
-                               _mask(mask, "mask").data_ptr(), float(threshold), _pixels(input),
-                               input.shape[1], _dtype(input), _stream()))
+    _call("sparsify", lib.dc_sparsify,
+          (input.data_ptr(), prev_in.data_ptr(), delta.data_ptr(), _mask(mask, "mask").data_ptr(),
+           float(threshold), _pixels(input), input.shape[1], _dtype(input), _stream()),
+          P=_pixels(input), C=input.shape[1], esize=input.element_size(), out_mask=mask)
 
 
 def sparse_add_tensors(a, b, prev_out, out, mask_a, mask_b, mask_out, weight_a, weight_b,
@@ -228,18 +251,24 @@ def sparse_add_tensors(a, b, prev_out, out, mask_a, mask_b, mask_out, weight_a, 
     _nhwc(b, "b")
     if a.shape != b.shape:
         raise _lib.DeltaCNNError(-2, f"shape mismatch {tuple(a.shape)} vs {tuple(b.shape)}")
-    _lib.check(lib.dc_add(a.data_ptr(), b.data_ptr(), _ptr(prev_out), out.data_ptr(),
-                          _mask(mask_a, "mask_a").data_ptr(), _mask(mask_b, "mask_b").data_ptr(),
-                          _ptr(mask_out), float(weight_a), float(weight_b), int(activation),
-                          int(bool(dense_out)), _pixels(a), a.shape[1], _dtype(a), _stream()))
+    _call("add", lib.dc_add,
+          (a.data_ptr(), b.data_ptr(), _ptr(prev_out), out.data_ptr(),
+           _mask(mask_a, "mask_a").data_ptr(), _mask(mask_b, "mask_b").data_ptr(), _ptr(mask_out),
+           float(weight_a), float(weight_b), int(activation), int(bool(dense_out)), _pixels(a),
+           a.shape[1], _dtype(a), _stream()),
+          P=_pixels(a), C=a.shape[1], esize=a.element_size(), in_mask=mask_a, in_mask_b=mask_b,
+          out_mask=None if dense_out else mask_out, with_prev=prev_out is not None,
+          dense_out=bool(dense_out))
 
 
 def sparse_add_to_dense_tensor(a, b, mask_a, activation=0):
     """cuda_kernels.py:144-145: ``b[px] += a[px]`` on active pixels."""
     lib = _lib.load()
     _nhwc(a, "a")
-    _lib.check(lib.dc_add_to_dense(a.data_ptr(), b.data_ptr(), _mask(mask_a, "mask_a").data_ptr(),
-                                   int(activation), _pixels(a), a.shape[1], _dtype(a), _stream()))
+    _call("add_to_dense", lib.dc_add_to_dense,
+          (a.data_ptr(), b.data_ptr(), _mask(mask_a, "mask_a").data_ptr(), int(activation),
+           _pixels(a), a.shape[1], _dtype(a), _stream()),
+          P=_pixels(a), C=a.shape[1], esize=a.element_size(), in_mask=mask_a)
 
 
 def sparse_mul_add(x, x_mask, out, out_mask, scale, bias):
@@ -248,9 +277,10 @@ def sparse_mul_add(x, x_mask, out, out_mask, scale, bias):
     _nhwc(x, "x")
     scale = scale.reshape(-1).to(x.dtype).contiguous()
     bias = None if bias is None else bias.reshape(-1).to(x.dtype).contiguous()
-    _lib.check(lib.dc_mul_add(x.data_ptr(), _mask(x_mask, "x_mask").data_ptr(), out.data_ptr(),
-                              out_mask.data_ptr(), scale.data_ptr(), _ptr(bias), _pixels(x),
-                              x.shape[1], _dtype(x), _stream()))
+    _call("mul_add", lib.dc_mul_add,
+          (x.data_ptr(), _mask(x_mask, "x_mask").data_ptr(), out.data_ptr(), out_mask.data_ptr(),
+           scale.data_ptr(), _ptr(bias), _pixels(x), x.shape[1], _dtype(x), _stream()),
+          P=_pixels(x), C=x.shape[1], esize=x.element_size(), in_mask=x_mask)
 
 
 def sparse_upsample(input, mask_in, scale, out=None):
@@ -264,8 +294,10 @@ def sparse_upsample(input, mask_in, scale, out=None):
         mask_out = new_mask(b, h * scale, w * scale, input.device)
     else:
         out_t, mask_out = out
-    _lib.check(lib.dc_upsample(input.data_ptr(), out_t.data_ptr(), _mask(mask_in, "mask_in").data_ptr(),
-                               mask_out.data_ptr(), b, h, w, c, scale, _dtype(input), _stream()))
+    _call("upsample", lib.dc_upsample,
+          (input.data_ptr(), out_t.data_ptr(), _mask(mask_in, "mask_in").data_ptr(),
+           mask_out.data_ptr(), b, h, w, c, scale, _dtype(input), _stream()),
+          P=b * h * w, C=c, esize=input.element_size(), in_mask=mask_in, scale=scale)
     return out_t, mask_out
 
 
@@ -282,8 +314,10 @@ def sparse_concatenate(a, b, out=None):
         mask_out = new_mask(a.shape[0], a.shape[2], a.shape[3], a.device)
     else:
         out_t, mask_out = out
-    _lib.check(lib.dc_concat(a.data_ptr(), b.data_ptr(), out_t.data_ptr(),
-                             _mask(mask_a, "mask_a").data_ptr(), _mask(mask_b, "mask_b").data_ptr(),
-                             mask_out.data_ptr(), _pixels(a), a.shape[1], b.shape[1], _dtype(a),
-                             _stream()))
+    _call("concat", lib.dc_concat,
+          (a.data_ptr(), b.data_ptr(), out_t.data_ptr(), _mask(mask_a, "mask_a").data_ptr(),
+           _mask(mask_b, "mask_b").data_ptr(), mask_out.data_ptr(), _pixels(a), a.shape[1],
+           b.shape[1], _dtype(a), _stream()),
+          P=_pixels(a), C=a.shape[1], Cb=b.shape[1], esize=a.element_size(), in_mask=mask_a,
+          in_mask_b=mask_b, out_mask=mask_out)
     return out_t, mask_out

@@ -230,7 +230,7 @@ class _DeltaConvBase:
             plan["out_mask"] = hk.new_mask(g.batch, g.out_h, g.out_w, x.device)
         return plan
 
-    def _forward_delta_conv(self, input, first_iter):
+    def _prepare(self, input):
         if type(input) == Tensor:
             raise TypeError("the deltacnn backend propagates (delta, mask) tuples: put a "
                             "DCSparsify in front of the first convolution")
@@ -241,7 +241,6 @@ class _DeltaConvBase:
         if self._plan is None or self._plan["shape"] != tuple(x.shape) or self._plan["dtype"] != x.dtype:
             self._plan = self._make_plan(x)
             self.in_shape = x.shape
-        plan = self._plan
         if self._packed is None:
             self._packed = hk.pack_filter(self.weight.data, self.in_channels, self.out_channels,
                                           self.groups, self._transposed)
@@ -250,23 +249,31 @@ class _DeltaConvBase:
         packed = self._packed if self._packed is not False else None
         bias = self.bias if self.frame_idx <= 0 else None
         pad = self.padding4 if getattr(self, "padding4", None) is not None else self.padding
+        return x, mask, self._plan, packed, bias, pad
+
+    def conv_delta(self, input):
+        """The convolution alone: ``(delta, mask) -> (out, out_mask)`` without the layer's
+        activation / densify stage (bias is applied while ``frame_idx <= 0``)."""
+        x, mask, plan, packed, bias, pad = self._prepare(input)
+        fn = hk.sparse_deconv if self._transposed else hk.sparse_conv
+        return fn(x=x, filter=self.weight, mask=mask, bias=bias, stride=self.stride, padding=pad,
+                  dilation=self.dilation, groups=self.groups, c_out=self.out_channels,
+                  create_out_mask=True, out_mask=plan["out_mask"], packed_filter=packed,
+                  out=plan["out"], geometry=plan["g"])
+
+    def _forward_delta_conv(self, input, first_iter):
         act = self.activation_layer
         fuse = (act is not None and not act.first_iter and not self._transposed
                 and DCConv2d.fuse_activation and act.inplace)
         if fuse:
             # activation/truncation runs as the epilogue of the convolution call
-            out, out_mask = hk.sparse_conv_activation(
+            x, mask, plan, packed, bias, pad = self._prepare(input)
+            return hk.sparse_conv_activation(
                 x, self.weight, mask, bias, act.prev_out, act.out_truncated,
                 DCThreshold.get(act), act.activation_int, act.truncation_mode.value, self.stride,
                 pad, self.dilation, self.groups, self.out_channels, packed_filter=packed,
                 out=plan["out"], out_mask=plan["out_mask"], geometry=plan["g"])
-            return out, out_mask
-        fn = hk.sparse_deconv if self._transposed else hk.sparse_conv
-        out, out_mask = fn(x=x, filter=self.weight, mask=mask, bias=bias, stride=self.stride,
-                           padding=pad, dilation=self.dilation, groups=self.groups,
-                           c_out=self.out_channels, create_out_mask=True,
-                           out_mask=plan["out_mask"], packed_filter=packed, out=plan["out"],
-                           geometry=plan["g"])
+        out, out_mask = self.conv_delta(input)
         if self.dense_out:
             return self.densify_layer((out, out_mask))
         if act is not None:

@@ -1,0 +1,149 @@
+"""Per-call tracer for the delta operators: durations from stream events and ALGORITHMIC
+byte / flop counts from the shapes and the measured mask populations.
+
+Algorithmic traffic is the minimum a delta operator has to move (s = bytes per element,
+m = 4-byte mask word, P pixels, n_x = number of active pixels of mask x):
+
+  sparsify           R = 2*P*C*s                          W = 2*n_out*C*s + P*m
+  activate_truncate  R = P*m + n_in*3*C*s                 W = n_out*3*C*s + (n_in-n_out)*(C*s + m)
+  densify            R = P*m + n*2*C*s                    W = n*C*s
+  add                R = 2*P*m + (n_a+n_b)*C*s [+n_out*C*s]  W = n_out*C*s [+n_out*C*s] + P*m
+  conv / deconv      R = P_in*m + n_in*Cin*s + K*K*(Cin/g)*Cout*s   W = n_out*Cout*s + P_out*m
+                     flops = 2*(Cin/g)*Cout*N_pairs, N_pairs = sum over updated outputs of the
+                     active inputs in their window (computed exactly from the masks)
+  pool               R = P_in*m + n_in*C*s (x2 for max)   W = n_out*C*s + P_out*m
+  add_to_dense       R = P*m + 2*n*C*s                    W = n*C*s
+  upsample           R = P*m + n*C*s                      W = S*S*(n*C*s + P*m)
+  concat             R = 2*P*m + (n_a*Ca + n_b*Cb)*s      W = n_out*(Ca+Cb)*s + P*m
+  mul_add            R = P*m + n*C*s + C*s                W = n*C*s
+"""
+from __future__ import annotations
+
+from collections import defaultdict
+
+import torch
+import torch.nn.functional as F
+
+
+class Tracer:
+    """Install with ``hip_kernels.set_tracer(t)``; run frames eagerly; ``t.finish()``."""
+
+    def __init__(self, count_pairs: bool = True):
+        self.records = []
+        self.count_pairs = count_pairs
+
+    @staticmethod
+    def _count(mask):
+        return None if mask is None else (mask != 0).sum()
+
+    def run(self, op, fn, args, meta):
+        rec = {"op": op, "meta": meta}
+        rec["n_in"] = self._count(meta.get("in_mask"))
+        rec["n_in_b"] = self._count(meta.get("in_mask_b"))
+        if self.count_pairs and op in ("conv", "deconv", "conv_act"):
+            rec["pairs"] = self._pairs(meta["g"], meta["in_mask"], op == "deconv")
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        rc = fn(*args)
+        end.record()
+        rec["events"] = (start, end)
+        rec["n_out"] = self._count(meta.get("out_mask"))
+        self.records.append(rec)
+        return rc
+
+    @staticmethod
+    def _pairs(g, mask, transposed):
+        """N_pairs: number of (updated output pixel, active input pixel in its window) pairs.
+        Every active input pixel reaches each output pixel of its footprint, and each of
+        those outputs is updated, so N_pairs = sum over taps of the shifted mask."""
+        m = (mask != 0).float()
+        ones = torch.ones(1, 1, g.kernel_h, g.kernel_w, device=m.device)
+        if transposed:
+            cnt = F.conv_transpose2d(m, ones, stride=(g.stride_h, g.stride_w), padding=(g.pad_top, g.pad_left),
+                                     dilation=(g.dilation_h, g.dilation_w))
+        else:
+            mp = F.pad(m, (g.pad_left, g.pad_right, g.pad_top, g.pad_bottom))
+            cnt = F.conv2d(mp, ones, stride=(g.stride_h, g.stride_w), dilation=(g.dilation_h, g.dilation_w))
+        return cnt.sum()
+
+    def finish(self):
+        """Synchronise and turn the records into dicts with ``ms``, ``bytes``, ``flops``."""
+        torch.cuda.synchronize()
+        out = []
+        for r in self.records:
+            meta, op = r["meta"], r["op"]
+            n_in = None if r["n_in"] is None else int(r["n_in"])
+            n_in_b = None if r["n_in_b"] is None else int(r["n_in_b"])
+            n_out = None if r["n_out"] is None else int(r["n_out"])
+            s, m = meta["esize"], 4
+            flops = 0
+            if op in ("conv", "deconv", "conv_act"):
+                g = meta["g"]
+                p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
+                wbytes = g.kernel_h * g.kernel_w * (g.in_c // g.groups) * g.out_c * s
+                rd = p_in * m + n_in * g.in_c * s + wbytes
+                wr = n_out * g.out_c * s + p_out * m
+                if "pairs" in r:
+                    flops = 2 * (g.in_c // g.groups) * g.out_c * int(r["pairs"])
+                dw = g.groups > 1
+                kind = ("dw" if dw else "pw" if g.kernel_h == 1 and g.kernel_w == 1 else "kxk")
+                name = f"{op}_{kind}{'_mfma' if meta.get('mfma') and not dw else ''}"
+                shape = f"{g.in_c}->{g.out_c} k{g.kernel_h} s{g.stride_h} @{g.in_h}x{g.in_w}"
+                dens = (n_in / p_in, n_out / p_out)
+            elif op == "pool":
+                g = meta["g"]
+                p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
+                rd = p_in * m + n_in * g.in_c * s * (2 if meta["mode"] == 0 else 1)
+                wr = n_out * g.in_c * s + p_out * m
+                name, shape = "pool", f"C{g.in_c} k{g.kernel_h} @{g.in_h}x{g.in_w}"
+                dens = (n_in / p_in, n_out / p_out)
+            else:
+                P, C = meta["P"], meta["C"]
+                name, shape = op, f"C{C} P{P}"
+                if op == "sparsify":
+                    rd, wr = 2 * P * C * s, 2 * n_out * C * s + P * m
+                    dens = (1.0, n_out / P)
+                elif op == "activate_truncate":
+                    rd = P * m + n_in * 3 * C * s
+                    wr = n_out * 3 * C * s + (n_in - n_out) * (C * s + m)
+                    dens = (n_in / P, n_out / P)
+                elif op == "densify":
+                    rd, wr = P * m + n_in * 2 * C * s, n_in * C * s
+                    dens = (n_in / P, n_in / P)
+                elif op == "add":
+                    n_o = n_out if n_out is not None else P
+                    extra = n_o * C * s if meta["with_prev"] else 0
+                    rd = 2 * P * m + (n_in + n_in_b) * C * s + extra
+                    wr = n_o * C * s + extra + P * m
+                    dens = ((n_in + n_in_b) / (2 * P), n_o / P)
+                elif op == "add_to_dense":
+                    rd, wr = P * m + 2 * n_in * C * s, n_in * C * s
+                    dens = (n_in / P, n_in / P)
+                elif op == "upsample":
+                    sc = meta["scale"] ** 2
+                    rd, wr = P * m + n_in * C * s, sc * (n_in * C * s + P * m)
+                    dens = (n_in / P, n_in / P)
+                elif op == "concat":
+                    cb = meta["Cb"]
+                    rd = 2 * P * m + (n_in * C + n_in_b * cb) * s
+                    wr = n_out * (C + cb) * s + P * m
+                    dens = ((n_in + n_in_b) / (2 * P), n_out / P)
+                else:  # mul_add
+                    rd, wr = P * m + n_in * C * s + C * s, n_in * C * s
+                    dens = (n_in / P, n_in / P)
+            out.append({"kernel": name, "shape": shape, "ms": r["events"][0].elapsed_time(r["events"][1]),
+                        "bytes": rd + wr, "flops": flops, "density_in": dens[0], "density_out": dens[1]})
+        self.records = []
+        return out
+
+
+def summarise(rows):
+    """Aggregate trace rows per kernel class: launches, total ms, bytes, flops."""
+    agg = defaultdict(lambda: {"launches": 0, "ms": 0.0, "bytes": 0, "flops": 0})
+    for r in rows:
+        a = agg[r["kernel"]]
+        a["launches"] += 1
+        a["ms"] += r["ms"]
+        a["bytes"] += r["bytes"]
+        a["flops"] += r["flops"]
+    return dict(agg)
