@@ -13,6 +13,7 @@
 //                     [Cout][tap][Cin]) and columns = compacted pixels (NHWC rows), so both
 //                     operands are 16-byte row loads and the accumulator tile stores 4
 //                     consecutive channels per lane
+#include "epilogue.hpp"
 #include "tile.hpp"
 
 namespace dc {
@@ -74,7 +75,7 @@ conv_direct_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
                         float w = float(filter[((size_t)(cg ^ wsw) * K2 + tap) * p.w_co + co]);
 #pragma unroll
                         for (int j = 0; j < PB; ++j)
-                            if (ip[j] >= 0) acc[j] += float(inb[(size_t)ip[j] * p.Ci + cin0 + cg]) * w;
+                            if (ip[j] >= 0) acc[j] = __builtin_fmaf(float(inb[(size_t)ip[j] * p.Ci + cin0 + cg]), w, acc[j]);
                     }
                 }
             }
@@ -87,18 +88,129 @@ conv_direct_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
     }
 }
 
+// ------------------------------------------------------------------------------- depthwise
+// One group of G lanes per OUTPUT pixel (grid = pixels x G): the group ballots the input mask
+// over the window into a tap bit set (the dilated output mask is "any bit set"), then walks
+// only the active taps with 16-byte channel vectors.  With ACT >= 0 the activation/truncation
+// of the layer runs on the accumulators as an epilogue, so the convolution output never makes
+// a round trip through memory and one launch is saved per layer.
+struct EpiP {
+    void *prev;
+    void *trunc;
+    float thr;
+    int mode;
+};
+
+template <typename T, int ITERS, int ACT>
+__global__ void __launch_bounds__(256)
+conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
+               const T *__restrict__ bias, T *__restrict__ out, const int32_t *__restrict__ mask,
+               int32_t *__restrict__ out_mask, EpiP epi, int lg) {
+    constexpr int N = Vec16<T>::N;
+    const int G = 1 << lg;
+    const int C = p.Ci;
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int po = gid >> lg, gl = gid & (G - 1);
+    const int P_out = p.B * p.Ho * p.Wo;
+    const bool valid = po < P_out;
+    const int b = po / (p.Ho * p.Wo);
+    const int r = po - b * p.Ho * p.Wo;
+    const int oy = r / p.Wo, ox = r - oy * p.Wo;
+    const int K2 = p.Kh * p.Kw;
+    const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
+    const int glo = lane_id() & ~(G - 1);
+    const uint64_t gmask = G >= WAVE ? ~0ull : ((1ull << G) - 1ull);
+
+    uint64_t taps = 0;
+    for (int j = 0; j < K2; j += G) {
+        const int t = j + gl;
+        bool m = false;
+        if (valid && t < K2) {
+            const int ky = t / p.Kw, kx = t - ky * p.Kw;
+            const int iy = oy * p.sh - p.pt + ky * p.dh, ix = ox * p.sw - p.pl + kx * p.dw;
+            if (iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi) m = mb[iy * p.Wi + ix] != 0;
+        }
+        taps |= ((ballot(m) >> glo) & gmask) << j;
+    }
+    const bool active = valid && taps != 0;
+    if (valid && gl == 0) out_mask[po] = active ? 1 : 0;
+    if (ballot(active) == 0) return;
+
+    float acc[ITERS][N];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int j = 0; j < N; ++j) acc[it][j] = 0.f;
+    if (active) {
+        const T *inb = in + (size_t)b * p.Hi * p.Wi * C;
+        for (int t = 0; t < K2; ++t) {
+            if (!((taps >> t) & 1ull)) continue;
+            const int ky = t / p.Kw, kx = t - ky * p.Kw;
+            const int iy = oy * p.sh - p.pt + ky * p.dh, ix = ox * p.sw - p.pl + kx * p.dw;
+            const T *xr = inb + (size_t)(iy * p.Wi + ix) * C;
+            const T *wr = filter + (size_t)t * C;
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int c = (it * G + gl) * N;
+                if (c < C) {
+                    const Vec<T, N> x = vload<T, N>(xr + c);
+                    const Vec<T, N> w = vload<T, N>(wr + c);
+#pragma unroll
+                    for (int j = 0; j < N; ++j)
+                        acc[it][j] = __builtin_fmaf(float(x.v[j]), float(w.v[j]), acc[it][j]);
+                }
+            }
+        }
+    }
+    Vec<T, N> dl[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int c = (it * G + gl) * N;
+        if (active && c < C) {
+            if (bias != nullptr) {
+                const Vec<T, N> bv = vload<T, N>(bias + c);
+#pragma unroll
+                for (int j = 0; j < N; ++j) acc[it][j] += float(bv.v[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < N; ++j) dl[it].v[j] = T(acc[it][j]);
+        }
+    }
+    if (ACT < 0) {
+        if (active) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int c = (it * G + gl) * N;
+                if (c < C) vstore<T, N>(out + (size_t)po * C + c, dl[it]);
+            }
+        }
+    } else {
+        act_trunc_pixel<T, ITERS, (ACT < 0 ? 0 : ACT)>(dl, active, (size_t)po, gl, G, C, out,
+                                                         (T *)epi.prev, (T *)epi.trunc, out_mask,
+                                                         T(epi.thr), epi.mode);
+    }
+}
+
 // ------------------------------------------------------------------------------------ MFMA
-// One work item = one 16(channels) x 16(pixels) accumulator tile with the full reduction over
-// taps and input channels; the items of a workgroup (channel tiles of its channel block x
-// pixel sub-tiles of its compacted list) are dealt round-robin to its four wavefronts.
-template <bool TR>
+// Implicit GEMM on v_mfma_f32_16x16x32_f16: rows = 16 output channels (packed filter rows),
+// columns = 16 compacted pixels (NHWC input rows), reduction over (tap, input channel) in
+// steps of 32.  A wavefront keeps up to four pixel sub-tiles (64 pixels) in accumulators, so a
+// filter fragment is loaded once per step and reused four times.
+//   KSPLIT = false: the four wavefronts of a workgroup take four different channel tiles.
+//   KSPLIT = true : the workgroup owns one channel tile and its wavefronts split the reduction
+//                   steps round-robin; partial accumulators meet in LDS.  This is what keeps
+//                   deep layers with tiny maps (7x7 x 960 channels) from being one long serial
+//                   chain in a handful of wavefronts.
+template <bool TR, bool KSPLIT>
 __global__ void __launch_bounds__(256)
 conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                  const half_t *__restrict__ bias, half_t *__restrict__ out,
                  const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, int co_blocks,
-                 int co_tiles_per_block, int ci_p) {
+                 int ci_p) {
+    constexpr int NT = 4;
     __shared__ int s_list[TILE_PX];
     __shared__ int s_n;
+    __shared__ float4_t s_red[KSPLIT ? 4 * NT * WAVE : 1];
     const int b = blockIdx.z / co_blocks;
     const int cb = blockIdx.z % co_blocks;
     const int n = tile_mask_phase<TR>(p, mask, out_mask, b, blockIdx.y * TILE, blockIdx.x * TILE,
@@ -106,63 +218,115 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
     if (n == 0) return;
 
     const int wave = threadIdx.x / WAVE, lane = lane_id();
-    const int l16 = lane & 15, kq = lane >> 4;  // row/column inside the tile, k-quarter
+    const int l16 = lane & 15, kq = lane >> 4;  // row / column inside a tile, k-quarter
     const int K2 = p.Kh * p.Kw;
     const int n_tiles = (n + 15) >> 4;
     const int co_tiles = (p.Co + 15) >> 4;
-    const int ct0 = cb * co_tiles_per_block;
-    const int ct_end = min(ct0 + co_tiles_per_block, co_tiles);
-    const int items = (ct_end - ct0) * n_tiles;
+    const int ct = KSPLIT ? cb : cb * 4 + wave;
+    if (!KSPLIT && ct >= co_tiles) return;
     const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
     const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
     const bool pointwise = !TR && K2 == 1 && p.sh == 1 && p.sw == 1 && p.pt == 0 && p.pl == 0;
 
-    for (int item = wave; item < items; item += 4) {
-        const int ct = ct0 + item / n_tiles, nt = item % n_tiles;
+    int oy[NT], ox[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
         const int pix = nt * 16 + l16;
         const int code = pix < n ? s_list[pix] : -1;
-        const int oy = code >> 16, ox = code & 0xffff;
-        const half_t *wrow = wp + (size_t)(ct * 16 + l16) * K2 * ci_p + kq * 8;
-        float4_t acc = {0.f, 0.f, 0.f, 0.f};
-        for (int ky = 0; ky < p.Kh; ++ky) {
-            for (int kx = 0; kx < p.Kw; ++kx) {
+        oy[nt] = code < 0 ? -1 : code >> 16;
+        ox[nt] = code & 0xffff;
+    }
+    float4_t acc[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const half_t *wrow = wp + (size_t)(ct * 16 + l16) * K2 * ci_p + kq * 8;
+    const int ksteps = ci_p >> 5;
+    const int total = K2 * ksteps;
+    const int kvalid = kq * 8;  // this lane's channel offset inside a 32-wide step
+    int cur_tap = -1;
+    const half_t *xrow[NT];
+    bool xok[NT];
+    bool tap_used = false;
+    for (int s = KSPLIT ? wave : 0; s < total; s += KSPLIT ? 4 : 1) {
+        const int tap = s / ksteps;
+        const int k0 = (s - tap * ksteps) << 5;
+        if (tap != cur_tap) {
+            cur_tap = tap;
+            const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
+            bool any = false;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
                 int ipix = -1;
-                if (code >= 0) {
+                if (oy[nt] >= 0) {
                     if (pointwise) {
-                        ipix = oy * p.Wi + ox;
+                        ipix = oy[nt] * p.Wi + ox[nt];
                     } else {
                         int iy, ix;
-                        if (tap_src<TR>(oy, ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
-                            tap_src<TR>(ox, kx, p.sw, p.dw, p.pl, p.Wi, ix) &&
+                        if (tap_src<TR>(oy[nt], ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
+                            tap_src<TR>(ox[nt], kx, p.sw, p.dw, p.pl, p.Wi, ix) &&
                             mb[iy * p.Wi + ix] != 0)
                             ipix = iy * p.Wi + ix;
                     }
                 }
-                if (ballot(ipix >= 0) == 0) continue;  // no pixel of this sub-tile uses the tap
-                const half_t *xrow = inb + (size_t)(ipix < 0 ? 0 : ipix) * p.Ci + kq * 8;
-                const half_t *wt = wrow + (size_t)(ky * p.Kw + kx) * ci_p;
-                for (int k0 = 0; k0 < ci_p; k0 += 32) {
-                    half8_t a = *reinterpret_cast<const half8_t *>(wt + k0);
-                    half8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
-                    if (ipix >= 0 && k0 + kq * 8 < p.Ci) x = *reinterpret_cast<const half8_t *>(xrow + k0);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, x, acc, 0, 0, 0);
-                }
+                xok[nt] = ipix >= 0;
+                any |= xok[nt];
+                xrow[nt] = inb + (size_t)(ipix < 0 ? 0 : ipix) * p.Ci + kvalid;
+            }
+            tap_used = ballot(any) != 0;  // does any pixel of this tile use the tap at all?
+        }
+        if (!tap_used) continue;
+        const half8_t a = *reinterpret_cast<const half8_t *>(wrow + (size_t)tap * ci_p + k0);
+        const bool kin = k0 + kvalid < p.Ci;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            if (nt < n_tiles) {
+                half8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (xok[nt] && kin) x = *reinterpret_cast<const half8_t *>(xrow[nt] + k0);
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, x, acc[nt], 0, 0, 0);
             }
         }
-        // lane holds channels ct*16 + kq*4 + {0..3} of pixel `pix`
-        if (code >= 0) {
-            const int co = ct * 16 + kq * 4;
-            half_t *o = out + (((size_t)b * p.Ho + oy) * p.Wo + ox) * p.Co + co;
-            if (co + 3 < p.Co && (p.Co & 3) == 0) {
-                half4_t r;
+    }
+
+    if (KSPLIT) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) r[i] = half_t(acc[i] + (bias ? float(bias[co + i]) : 0.f));
-                *reinterpret_cast<half4_t *>(o) = r;
-            } else {
+        for (int nt = 0; nt < NT; ++nt)
+            if (nt < n_tiles) s_red[(wave * NT + nt) * WAVE + lane] = acc[nt];
+        __syncthreads();
+        // wavefront w finishes pixel sub-tile w
+        if (wave >= n_tiles) return;
+        float4_t sum = s_red[(0 * NT + wave) * WAVE + lane];
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (co + i < p.Co) o[i] = half_t(acc[i] + (bias ? float(bias[co + i]) : 0.f));
-            }
+        for (int w = 1; w < 4; ++w) {
+            const float4_t v = s_red[(w * NT + wave) * WAVE + lane];
+            sum += v;
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            if (nt == wave) acc[nt] = sum;
+    }
+    // lane holds channels ct*16 + kq*4 + {0..3} of pixel (nt, l16)
+    const int co = ct * 16 + kq * 4;
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias != nullptr) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (co + i < p.Co) bv[i] = float(bias[co + i]);
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        if (nt >= n_tiles || oy[nt] < 0) continue;
+        if (KSPLIT && nt != wave) continue;
+        half_t *o = out + (((size_t)b * p.Ho + oy[nt]) * p.Wo + ox[nt]) * p.Co + co;
+        if (co + 3 < p.Co && (p.Co & 3) == 0) {
+            half4_t r;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) r[i] = half_t(acc[nt][i] + bv[i]);
+            *reinterpret_cast<half4_t *>(o) = r;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (co + i < p.Co) o[i] = half_t(acc[nt][i] + bv[i]);
         }
     }
 }
@@ -225,22 +389,77 @@ hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *pa
     return hipGetLastError();
 }
 
+namespace {
+
+template <typename T, int ITERS>
+void dw_launch(dim3 grid, hipStream_t s, int act, const ConvP &p, const T *in, const T *filter,
+               const T *bias, T *out, const int32_t *mask, int32_t *out_mask, EpiP e, int lg) {
+#define DC_DW(A) conv_dw_kernel<T, ITERS, A><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg)
+    switch (act) {
+        case DC_ACT_LINEAR: DC_DW(DC_ACT_LINEAR); break;
+        case DC_ACT_RELU: DC_DW(DC_ACT_RELU); break;
+        case DC_ACT_RELU6: DC_DW(DC_ACT_RELU6); break;
+        case DC_ACT_LEAKY: DC_DW(DC_ACT_LEAKY); break;
+        case DC_ACT_SIGMOID: DC_DW(DC_ACT_SIGMOID); break;
+        case DC_ACT_SWISH: DC_DW(DC_ACT_SWISH); break;
+        default: DC_DW(-1); break;
+    }
+#undef DC_DW
+}
+
+// Depthwise fast path; returns false if the shape does not qualify.
+template <typename T>
+bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *filter,
+                   const T *bias, T *out, const int32_t *mask, int32_t *out_mask,
+                   const ActEpilogue *epi, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    const auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (g.groups != g.in_c || g.groups != g.out_c || g.groups == 1) return false;
+    if (g.in_c % N != 0 || g.kernel_h * g.kernel_w > 64 || g.in_c / N > WAVE * 4) return false;
+    if (!al(in) || !al(filter) || !al(out) || (bias && !al(bias))) return false;
+    if (epi && (!al(epi->prev) || (epi->trunc && !al(epi->trunc)) || epi->mode < 0)) return false;
+    const int64_t P_out = (int64_t)g.batch * g.out_h * g.out_w;
+    const int nvec = g.in_c / N;
+    const int G = pick_group(nvec, P_out, 4);
+    const int iters = ceil_div(nvec, G);
+    dim3 grid((unsigned)ceil_div64(P_out * G, 256));
+    EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f,
+           epi ? epi->mode : 0};
+    const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
+    const int lg = log2i(G);
+    switch (iters) {
+        case 1: dw_launch<T, 1>(grid, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
+        case 2: dw_launch<T, 2>(grid, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
+        default: dw_launch<T, 4>(grid, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
+    }
+    return true;
+}
+
+}  // namespace
+
 hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                        const void *packed, const void *bias, void *out, const int32_t *mask,
                        int32_t *out_mask, int dtype, bool transposed, const ActEpilogue *epi,
                        hipStream_t s) {
     ConvP p = make_params(g, dtype);
     const int tx = ceil_div(g.out_w, TILE), ty = ceil_div(g.out_h, TILE);
+    if (!transposed) {
+        const bool done = dtype == DC_F32
+            ? try_depthwise<float>(g, p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, epi, s)
+            : try_depthwise<half_t>(g, p, (const half_t *)in, (const half_t *)filter, (const half_t *)bias, (half_t *)out, mask, out_mask, epi, s);
+        if (done) return hipGetLastError();
+    }
     if (packed != nullptr && mfma_eligible(g, dtype)) {
         const int co_tiles = ceil_div(g.out_c, 16);
-        const int tiles_per_block = 4;  // one channel tile per wavefront and pixel sub-tile
-        const int co_blocks = ceil_div(co_tiles, tiles_per_block);
-        dim3 grid(tx, ty, g.batch * co_blocks);
         const int ci_p = round_up(g.in_c, 32);
-        if (transposed)
-            conv_mfma_kernel<true><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, co_blocks, tiles_per_block, ci_p);
-        else
-            conv_mfma_kernel<false><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, co_blocks, tiles_per_block, ci_p);
+        const int steps = g.kernel_h * g.kernel_w * (ci_p / 32);
+        const bool ksplit = steps >= 8;
+        const int co_blocks = ksplit ? co_tiles : ceil_div(co_tiles, 4);
+        dim3 grid(tx, ty, g.batch * co_blocks);
+#define DC_MFMA(TRF, KS) conv_mfma_kernel<TRF, KS><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, co_blocks, ci_p)
+        if (transposed) { if (ksplit) DC_MFMA(true, true); else DC_MFMA(true, false); }
+        else { if (ksplit) DC_MFMA(false, true); else DC_MFMA(false, false); }
+#undef DC_MFMA
     } else {
         dim3 grid(tx, ty, g.batch);
         int COT = pow2_ceil(g.out_c);

@@ -3,41 +3,24 @@
 //
 // Common shape: features are NHWC, so a pixel is a contiguous row of C values.  A pixel is
 // handled by an aligned group of G lanes (G a power of two, chosen on the host so that a
-// group covers the row with 16-byte vectors); a wavefront therefore handles 64/G pixels at a
-// time.  Operators that only touch active pixels first compact the active pixels of the
-// wavefront's 64 candidates (one coalesced mask load + ballot + popcount rank) into an LDS
-// list, so lanes are not wasted on inactive pixels at low update density.
+// group covers the row with 16-byte vectors); a wavefront therefore handles 64/G pixels and
+// the grid has one group per pixel.  Groups of inactive pixels read their mask word and
+// leave; per-pixel decisions are group-wide ballots.  One group per pixel (instead of a loop
+// over pixels inside a wavefront) keeps small feature maps -- a 7x7 map is 49 pixels -- spread
+// over many wavefronts, which is what matters at batch 1.
 //
 // Compiled with -ffp-contract=off: every arithmetic operation rounds on its own, in the
 // tensor's own type, which is what makes masks reproducible bit for bit.
-#include "common.hpp"
+#include "epilogue.hpp"
 
 namespace dc {
 namespace {
 
-constexpr int MAXW = 4;  // wavefronts per workgroup (blockDim.x <= 256)
-
-// Compact the active pixels of this wavefront's 64 candidates and run `f(pixel, group_lane,
-// valid)` for each of them, 64/G pixels per step.  Every lane of the workgroup must call
-// this (it contains a workgroup barrier).  `f` is called by all lanes of a step; lanes whose
-// group has no pixel get valid == false.
-template <typename F>
-__device__ __forceinline__ void for_each_active(bool active, int px, int G, F f) {
-    __shared__ int s_list[MAXW][WAVE];
-    const int wave = threadIdx.x / WAVE;
-    int n;
-    int rank = wave_rank(active, n);
-    if (active) s_list[wave][rank] = px;
-    __syncthreads();
-    const int per_step = WAVE / G;
-    const int grp = lane_id() / G;
-    const int gl = lane_id() & (G - 1);
-    for (int base = 0; base < n; base += per_step) {
-        int idx = base + grp;
-        bool valid = idx < n;
-        int p = valid ? s_list[wave][idx] : 0;
-        f(p, gl, valid);
-    }
+// Pixel and lane-in-group of this thread for groups of G = 1 << lg lanes.
+__device__ __forceinline__ void group_coords(int lg, int &p, int &gl) {
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    p = gid >> lg;
+    gl = gid & ((1 << lg) - 1);
 }
 
 // ------------------------------------------------------------------------------- sparsify
@@ -116,122 +99,75 @@ sparsify_gen_kernel(const T *__restrict__ in, T *__restrict__ prev, T *__restric
 }
 
 // ----------------------------------------------------------------- activation + truncation
-// Per active pixel: T = trunc + delta; S = T + prev; D = act(S) - act(prev).
-// keep (max: any |D| > thr; norm: sqrt(sum D^2) > thr; rms: sqrt(sum D^2 / C) > thr):
-//   prev = S, delta = D, trunc = 0;   otherwise trunc = T and the mask word is cleared.
-__device__ __forceinline__ float group_sum(float v, int G) {
-    for (int o = 1; o < G; o <<= 1) v += __shfl_xor(v, o, WAVE);
-    return v;
-}
-
 template <typename T, int ITERS, int ACT>
 __global__ void __launch_bounds__(256)
 act_trunc_vec_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict__ trunc,
-                     int32_t *__restrict__ mask, float thr_f, int mode, int P, int C, int G) {
+                     int32_t *__restrict__ mask, float thr_f, int mode, int P, int C, int lg) {
     constexpr int N = Vec16<T>::N;
-    const T thr = T(thr_f);
-    const int px = blockIdx.x * blockDim.x + threadIdx.x;
-    const bool active = px < P && mask[px] != 0;
-    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
-        Vec<T, N> t[ITERS], s[ITERS], d[ITERS];
-        bool hit = false;
-        float sq = 0.f;
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
+    const bool valid = p < P && mask[p] != 0;
+    if (ballot(valid) == 0) return;
+    Vec<T, N> dl[ITERS];
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            int c = (it * G + gl) * N;
-            if (valid && c < C) {
-                size_t off = (size_t)p * C + c;
-                Vec<T, N> dl = vload<T, N>(delta + off);
-                Vec<T, N> q = vload<T, N>(prev + off);
-                Vec<T, N> tr = vload<T, N>(trunc + off);
-#pragma unroll
-                for (int j = 0; j < N; ++j) {
-                    t[it].v[j] = tr.v[j] + dl.v[j];
-                    s[it].v[j] = t[it].v[j] + q.v[j];
-                    d[it].v[j] = act_apply<T>(s[it].v[j], ACT) - act_apply<T>(q.v[j], ACT);
-                    hit |= tabs(d[it].v[j]) > thr;
-                    sq += float(d[it].v[j]) * float(d[it].v[j]);
-                }
-            }
-        }
-        bool keep;
-        if (mode == DC_TRUNC_MAX) {
-            keep = group_any(hit, G);
-        } else {
-            sq = group_sum(sq, G);
-            if (mode == DC_TRUNC_RMS) sq /= float(C);
-            keep = sqrtf(sq) > float(thr);
-        }
-        if (valid) {
-#pragma unroll
-            for (int it = 0; it < ITERS; ++it) {
-                int c = (it * G + gl) * N;
-                if (c < C) {
-                    size_t off = (size_t)p * C + c;
-                    if (keep) {
-                        Vec<T, N> z;
-#pragma unroll
-                        for (int j = 0; j < N; ++j) z.v[j] = T(0);
-                        vstore<T, N>(prev + off, s[it]);
-                        vstore<T, N>(delta + off, d[it]);
-                        vstore<T, N>(trunc + off, z);
-                    } else {
-                        vstore<T, N>(trunc + off, t[it]);
-                    }
-                }
-            }
-            if (!keep && gl == 0) mask[p] = 0;
-        }
-    });
+    for (int it = 0; it < ITERS; ++it) {
+        const int c = (it * G + gl) * N;
+        if (valid && c < C) dl[it] = vload<T, N>(delta + (size_t)p * C + c);
+    }
+    act_trunc_pixel<T, ITERS, ACT>(dl, valid, (size_t)p, gl, G, C, delta, prev, trunc, mask,
+                                   T(thr_f), mode);
 }
 
+// Any C / alignment: scalar, two passes (decide, then recompute and write).
 template <typename T>
 __global__ void __launch_bounds__(256)
 act_trunc_gen_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict__ trunc,
                      int32_t *__restrict__ mask, float thr_f, int act, int mode, int P, int C,
-                     int G) {
+                     int lg) {
     const T thr = T(thr_f);
-    const int px = blockIdx.x * blockDim.x + threadIdx.x;
-    const bool active = px < P && mask[px] != 0;
-    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
-        bool hit = false;
-        float sq = 0.f;
-        if (valid) {
-            for (int c = gl; c < C; c += G) {
-                size_t off = (size_t)p * C + c;
-                T q = prev[off];
-                T t = trunc[off] + delta[off];
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
+    const bool valid = p < P && mask[p] != 0;
+    if (ballot(valid) == 0) return;
+    bool hit = false;
+    float sq = 0.f;
+    if (valid) {
+        for (int c = gl; c < C; c += G) {
+            size_t off = (size_t)p * C + c;
+            T q = prev[off];
+            T t = trunc[off] + delta[off];
+            T s = t + q;
+            T d = act_apply<T>(s, act) - act_apply<T>(q, act);
+            hit |= tabs(d) > thr;
+            sq += float(d) * float(d);
+        }
+    }
+    bool keep;
+    if (mode == DC_TRUNC_MAX) {
+        keep = group_any(hit, G);
+    } else {
+        sq = group_sum(sq, G);
+        if (mode == DC_TRUNC_RMS) sq /= float(C);
+        keep = sqrtf(sq) > float(thr);
+    }
+    if (valid) {
+        for (int c = gl; c < C; c += G) {
+            size_t off = (size_t)p * C + c;
+            T q = prev[off];
+            T t = trunc[off] + delta[off];
+            if (keep) {
                 T s = t + q;
-                T d = act_apply<T>(s, act) - act_apply<T>(q, act);
-                hit |= tabs(d) > thr;
-                sq += float(d) * float(d);
+                prev[off] = s;
+                delta[off] = act_apply<T>(s, act) - act_apply<T>(q, act);
+                trunc[off] = T(0);
+            } else {
+                trunc[off] = t;
             }
         }
-        bool keep;
-        if (mode == DC_TRUNC_MAX) {
-            keep = group_any(hit, G);
-        } else {
-            sq = group_sum(sq, G);
-            if (mode == DC_TRUNC_RMS) sq /= float(C);
-            keep = sqrtf(sq) > float(thr);
-        }
-        if (valid) {
-            for (int c = gl; c < C; c += G) {
-                size_t off = (size_t)p * C + c;
-                T q = prev[off];
-                T t = trunc[off] + delta[off];
-                if (keep) {
-                    T s = t + q;
-                    prev[off] = s;
-                    delta[off] = act_apply<T>(s, act) - act_apply<T>(q, act);
-                    trunc[off] = T(0);
-                } else {
-                    trunc[off] = t;
-                }
-            }
-            if (!keep && gl == 0) mask[p] = 0;
-        }
-    });
+        if (!keep && gl == 0) mask[p] = 0;
+    }
 }
 
 // -------------------------------------------------------------------------------- densify
@@ -240,27 +176,26 @@ act_trunc_gen_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict_
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
 accumulate_kernel(T *__restrict__ delta, T *__restrict__ prev, const int32_t *__restrict__ mask,
-                  int act, int P, int C, int G) {
-    const int px = blockIdx.x * blockDim.x + threadIdx.x;
-    const bool active = px < P && mask[px] != 0;
-    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
-        if (!valid) return;
-        for (int c = gl * N; c < C; c += G * N) {
-            size_t off = (size_t)p * C + c;
-            Vec<T, N> dl = vload<T, N>(delta + off);
-            Vec<T, N> q = vload<T, N>(prev + off);
-            Vec<T, N> s;
+                  int act, int P, int C, int lg) {
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
+    if (p >= P || mask[p] == 0) return;
+    for (int c = gl * N; c < C; c += G * N) {
+        size_t off = (size_t)p * C + c;
+        Vec<T, N> dl = vload<T, N>(delta + off);
+        Vec<T, N> q = vload<T, N>(prev + off);
+        Vec<T, N> s;
 #pragma unroll
-            for (int j = 0; j < N; ++j) s.v[j] = dl.v[j] + q.v[j];
-            vstore<T, N>(prev + off, s);
-            if (act > 0) {
+        for (int j = 0; j < N; ++j) s.v[j] = dl.v[j] + q.v[j];
+        vstore<T, N>(prev + off, s);
+        if (act > 0) {
 #pragma unroll
-                for (int j = 0; j < N; ++j)
-                    dl.v[j] = act_apply<T>(s.v[j], act) - act_apply<T>(q.v[j], act);
-                vstore<T, N>(delta + off, dl);
-            }
+            for (int j = 0; j < N; ++j)
+                dl.v[j] = act_apply<T>(s.v[j], act) - act_apply<T>(q.v[j], act);
+            vstore<T, N>(delta + off, dl);
         }
-    });
+    }
 }
 
 // ------------------------------------------------------------------------------------ add
@@ -270,47 +205,42 @@ template <typename T, int N>
 __global__ void __launch_bounds__(256)
 add_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ prev,
            T *__restrict__ out, const int32_t *__restrict__ ma, const int32_t *__restrict__ mb,
-           int32_t *__restrict__ mo, float wa_f, float wb_f, int act, int P, int C, int G) {
+           int32_t *__restrict__ mo, float wa_f, float wb_f, int act, int P, int C, int lg) {
     const T wa = T(wa_f), wb = T(wb_f);
-    const int px = blockIdx.x * blockDim.x + threadIdx.x;
-    int flags = 0;
-    if (px < P) {
-        flags = (ma[px] != 0 ? 1 : 0) | (mb[px] != 0 ? 2 : 0);
-        mo[px] = flags != 0 ? 1 : 0;
-    }
-    // the pixel index and its two activity bits travel together through the compaction
-    for_each_active(flags != 0, px * 4 + flags, G, [&](int code, int gl, bool valid) {
-        if (!valid) return;
-        const int p = code >> 2;
-        const bool aa = code & 1, ab = code & 2;
-        for (int c = gl * N; c < C; c += G * N) {
-            size_t off = (size_t)p * C + c;
-            Vec<T, N> s;
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
+    if (p >= P) return;
+    const bool aa = ma[p] != 0, ab = mb[p] != 0;
+    if (gl == 0) mo[p] = (aa || ab) ? 1 : 0;
+    if (!(aa || ab)) return;
+    for (int c = gl * N; c < C; c += G * N) {
+        size_t off = (size_t)p * C + c;
+        Vec<T, N> s;
 #pragma unroll
-            for (int j = 0; j < N; ++j) s.v[j] = T(0);
-            if (aa) {
-                Vec<T, N> va = vload<T, N>(a + off);
+        for (int j = 0; j < N; ++j) s.v[j] = T(0);
+        if (aa) {
+            Vec<T, N> va = vload<T, N>(a + off);
 #pragma unroll
-                for (int j = 0; j < N; ++j) s.v[j] = va.v[j] * wa;
-            }
-            if (ab) {
-                Vec<T, N> vb = vload<T, N>(b + off);
-#pragma unroll
-                for (int j = 0; j < N; ++j) s.v[j] = fma_t(vb.v[j], wb, s.v[j]);
-            }
-            if (act > 0) {
-                Vec<T, N> q = vload<T, N>(prev + off);
-                Vec<T, N> n;
-#pragma unroll
-                for (int j = 0; j < N; ++j) {
-                    n.v[j] = s.v[j] + q.v[j];
-                    s.v[j] = act_apply<T>(n.v[j], act) - act_apply<T>(q.v[j], act);
-                }
-                vstore<T, N>(prev + off, n);
-            }
-            vstore<T, N>(out + off, s);
+            for (int j = 0; j < N; ++j) s.v[j] = va.v[j] * wa;
         }
-    });
+        if (ab) {
+            Vec<T, N> vb = vload<T, N>(b + off);
+#pragma unroll
+            for (int j = 0; j < N; ++j) s.v[j] = fma_t(vb.v[j], wb, s.v[j]);
+        }
+        if (act > 0) {
+            Vec<T, N> q = vload<T, N>(prev + off);
+            Vec<T, N> n;
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                n.v[j] = s.v[j] + q.v[j];
+                s.v[j] = act_apply<T>(n.v[j], act) - act_apply<T>(q.v[j], act);
+            }
+            vstore<T, N>(prev + off, n);
+        }
+        vstore<T, N>(out + off, s);
+    }
 }
 
 // dense_out: prev += s on active pixels, out = act(prev) for every pixel.
@@ -319,11 +249,11 @@ __global__ void __launch_bounds__(256)
 add_dense_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ prev,
                  T *__restrict__ out, const int32_t *__restrict__ ma,
                  const int32_t *__restrict__ mb, float wa_f, float wb_f, int act, int P, int C,
-                 int G) {
+                 int lg) {
     const T wa = T(wa_f), wb = T(wb_f);
-    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
-    const int p = gid / G;
-    const int gl = gid & (G - 1);
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
     if (p >= P) return;
     const bool aa = ma[p] != 0, ab = mb[p] != 0;
     for (int c = gl * N; c < C; c += G * N) {
@@ -358,20 +288,19 @@ add_dense_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
 add_to_dense_kernel(const T *__restrict__ a, T *__restrict__ b, const int32_t *__restrict__ ma,
-                    int P, int C, int G) {
-    const int px = blockIdx.x * blockDim.x + threadIdx.x;
-    const bool active = px < P && ma[px] != 0;
-    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
-        if (!valid) return;
-        for (int c = gl * N; c < C; c += G * N) {
-            size_t off = (size_t)p * C + c;
-            Vec<T, N> va = vload<T, N>(a + off);
-            Vec<T, N> vb = vload<T, N>(b + off);
+                    int P, int C, int lg) {
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
+    if (p >= P || ma[p] == 0) return;
+    for (int c = gl * N; c < C; c += G * N) {
+        size_t off = (size_t)p * C + c;
+        Vec<T, N> va = vload<T, N>(a + off);
+        Vec<T, N> vb = vload<T, N>(b + off);
 #pragma unroll
-            for (int j = 0; j < N; ++j) vb.v[j] = vb.v[j] + va.v[j];
-            vstore<T, N>(b + off, vb);
-        }
-    });
+        for (int j = 0; j < N; ++j) vb.v[j] = vb.v[j] + va.v[j];
+        vstore<T, N>(b + off, vb);
+    }
 }
 
 // With an activation the operator turns `a` into a dense output: b += a on active pixels,
@@ -379,10 +308,10 @@ add_to_dense_kernel(const T *__restrict__ a, T *__restrict__ b, const int32_t *_
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
 add_to_dense_act_kernel(T *__restrict__ a, T *__restrict__ b, const int32_t *__restrict__ ma,
-                        int act, int P, int C, int G) {
-    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
-    const int p = gid / G;
-    const int gl = gid & (G - 1);
+                        int act, int P, int C, int lg) {
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
     if (p >= P) return;
     const bool active = ma[p] != 0;
     for (int c = gl * N; c < C; c += G * N) {
@@ -404,28 +333,25 @@ add_to_dense_act_kernel(T *__restrict__ a, T *__restrict__ b, const int32_t *__r
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
 upsample_kernel(const T *__restrict__ in, T *__restrict__ out, const int32_t *__restrict__ mi,
-                int32_t *__restrict__ mo, int B, int H, int W, int C, int S, int G) {
+                int32_t *__restrict__ mo, int B, int H, int W, int C, int S, int lg) {
     const int P = B * H * W;
-    const int px = blockIdx.x * blockDim.x + threadIdx.x;
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
+    if (p >= P) return;
     const int Wo = W * S;
-    bool active = false;
-    if (px < P) {
-        active = mi[px] != 0;
-        int row = px / W, x = px - row * W;  // row = b*H + y
-        for (int i = 0; i < S * S; ++i)
-            mo[(size_t)(row * S + i / S) * Wo + x * S + i % S] = active ? 1 : 0;
-    }
-    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
-        if (!valid) return;
-        int row = p / W, x = p - row * W;
-        for (int c = gl * N; c < C; c += G * N) {
-            Vec<T, N> v = vload<T, N>(in + (size_t)p * C + c);
-            for (int i = 0; i < S * S; ++i) {
-                size_t op = (size_t)(row * S + i / S) * Wo + x * S + i % S;
-                vstore<T, N>(out + op * C + c, v);
-            }
+    const bool active = mi[p] != 0;
+    const int row = p / W, x = p - row * W;  // row = b*H + y
+    for (int i = gl; i < S * S; i += G)
+        mo[(size_t)(row * S + i / S) * Wo + x * S + i % S] = active ? 1 : 0;
+    if (!active) return;
+    for (int c = gl * N; c < C; c += G * N) {
+        Vec<T, N> v = vload<T, N>(in + (size_t)p * C + c);
+        for (int i = 0; i < S * S; ++i) {
+            size_t op = (size_t)(row * S + i / S) * Wo + x * S + i % S;
+            vstore<T, N>(out + op * C + c, v);
         }
-    });
+    }
 }
 
 // ---------------------------------------------------------------------------- concatenate
@@ -433,26 +359,22 @@ template <typename T, int N>
 __global__ void __launch_bounds__(256)
 concat_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ out,
               const int32_t *__restrict__ ma, const int32_t *__restrict__ mb,
-              int32_t *__restrict__ mo, int P, int Ca, int Cb, int G) {
-    const int px = blockIdx.x * blockDim.x + threadIdx.x;
-    int flags = 0;
-    if (px < P) {
-        flags = (ma[px] != 0 ? 1 : 0) | (mb[px] != 0 ? 2 : 0);
-        mo[px] = flags != 0 ? 1 : 0;
-    }
-    for_each_active(flags != 0, px * 4 + flags, G, [&](int code, int gl, bool valid) {
-        if (!valid) return;
-        const int p = code >> 2;
-        const bool aa = code & 1, ab = code & 2;
-        T *o = out + (size_t)p * (Ca + Cb);
-        Vec<T, N> z;
+              int32_t *__restrict__ mo, int P, int Ca, int Cb, int lg) {
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
+    if (p >= P) return;
+    const bool aa = ma[p] != 0, ab = mb[p] != 0;
+    if (gl == 0) mo[p] = (aa || ab) ? 1 : 0;
+    if (!(aa || ab)) return;
+    T *o = out + (size_t)p * (Ca + Cb);
+    Vec<T, N> z;
 #pragma unroll
-        for (int j = 0; j < N; ++j) z.v[j] = T(0);
-        for (int c = gl * N; c < Ca; c += G * N)
-            vstore<T, N>(o + c, aa ? vload<T, N>(a + (size_t)p * Ca + c) : z);
-        for (int c = gl * N; c < Cb; c += G * N)
-            vstore<T, N>(o + Ca + c, ab ? vload<T, N>(b + (size_t)p * Cb + c) : z);
-    });
+    for (int j = 0; j < N; ++j) z.v[j] = T(0);
+    for (int c = gl * N; c < Ca; c += G * N)
+        vstore<T, N>(o + c, aa ? vload<T, N>(a + (size_t)p * Ca + c) : z);
+    for (int c = gl * N; c < Cb; c += G * N)
+        vstore<T, N>(o + Ca + c, ab ? vload<T, N>(b + (size_t)p * Cb + c) : z);
 }
 
 // -------------------------------------------------------------------------------- mul_add
@@ -460,43 +382,32 @@ template <typename T, int N>
 __global__ void __launch_bounds__(256)
 mul_add_kernel(const T *__restrict__ in, const int32_t *__restrict__ mask, T *__restrict__ out,
                int32_t *__restrict__ mo, const T *__restrict__ scale,
-               const T *__restrict__ bias, int P, int C, int G) {
-    const int px = blockIdx.x * blockDim.x + threadIdx.x;
-    bool active = false;
-    if (px < P) {
-        active = mask[px] != 0;
-        if (mo != mask) mo[px] = active ? 1 : 0;
-    }
-    for_each_active(active, px, G, [&](int p, int gl, bool valid) {
-        if (!valid) return;
-        for (int c = gl * N; c < C; c += G * N) {
-            size_t off = (size_t)p * C + c;
-            Vec<T, N> v = vload<T, N>(in + off);
-            Vec<T, N> sc = vload<T, N>(scale + c);
-            if (bias != nullptr) {
-                Vec<T, N> bi = vload<T, N>(bias + c);
+               const T *__restrict__ bias, int P, int C, int lg) {
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
+    if (p >= P) return;
+    const bool active = mask[p] != 0;
+    if (mo != mask && gl == 0) mo[p] = active ? 1 : 0;
+    if (!active) return;
+    for (int c = gl * N; c < C; c += G * N) {
+        size_t off = (size_t)p * C + c;
+        Vec<T, N> v = vload<T, N>(in + off);
+        Vec<T, N> sc = vload<T, N>(scale + c);
+        if (bias != nullptr) {
+            Vec<T, N> bi = vload<T, N>(bias + c);
 #pragma unroll
-                for (int j = 0; j < N; ++j)
-                    v.v[j] = fma_t(v.v[j], sc.v[j], bi.v[j]);
-            } else {
+            for (int j = 0; j < N; ++j) v.v[j] = fma_t(v.v[j], sc.v[j], bi.v[j]);
+        } else {
 #pragma unroll
-                for (int j = 0; j < N; ++j) v.v[j] = v.v[j] * sc.v[j];
-            }
-            vstore<T, N>(out + off, v);
+            for (int j = 0; j < N; ++j) v.v[j] = v.v[j] * sc.v[j];
         }
-    });
+        vstore<T, N>(out + off, v);
+    }
 }
 
 // ---------------------------------------------------------------------------- host helpers
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
-// Lanes per pixel for `nvec` vectors per row when a lane may hold up to `max_iters` of them.
-inline int group_lanes(int nvec, int max_iters) {
-    int g = pow2_ceil(ceil_div(nvec, max_iters));
-    return g > WAVE ? WAVE : g;
-}
-
-inline int block_for(int64_t threads) { return threads >= (1 << 16) ? 256 : 64; }
 
 template <typename T>
 bool can_vec(int C, std::initializer_list<const void *> ptrs) {
@@ -506,36 +417,39 @@ bool can_vec(int C, std::initializer_list<const void *> ptrs) {
     return true;
 }
 
+// Launch shape for one group of G lanes per pixel.
+struct GroupLaunch {
+    int lg;
+    dim3 grid;
+    GroupLaunch(int64_t pixels, int G) : lg(log2i(G)), grid((unsigned)ceil_div64(pixels * G, 256)) {}
+};
+
 template <typename T>
 hipError_t sparsify_t(const T *in, T *prev, T *delta, int32_t *mask, float thr, int P, int C,
                       bool ge, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
     if (can_vec<T>(C, {in, prev, delta}) && C / N <= WAVE * 4) {
         int nvec = C / N;
-        int G = group_lanes(nvec, 4);
+        int G = pick_group(nvec, P, 4);
         int iters = ceil_div(nvec, G);
-        int64_t threads = (int64_t)P * G;
-        int blk = block_for(threads);
-        dim3 grid((unsigned)ceil_div64(threads, blk));
+        GroupLaunch L(P, G);
         switch (iters) {
-            case 1: sparsify_vec_kernel<T, 1><<<grid, blk, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
-            case 2: sparsify_vec_kernel<T, 2><<<grid, blk, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
-            default: sparsify_vec_kernel<T, 4><<<grid, blk, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
+            case 1: sparsify_vec_kernel<T, 1><<<L.grid, 256, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
+            case 2: sparsify_vec_kernel<T, 2><<<L.grid, 256, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
+            default: sparsify_vec_kernel<T, 4><<<L.grid, 256, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
         }
     } else {
         int G = group_lanes(C, 4);
-        int64_t threads = (int64_t)P * G;
-        int blk = block_for(threads);
-        sparsify_gen_kernel<T><<<dim3((unsigned)ceil_div64(threads, blk)), blk, 0, s>>>(
-            in, prev, delta, mask, thr, P, C, G, ge);
+        GroupLaunch L(P, G);
+        sparsify_gen_kernel<T><<<L.grid, 256, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge);
     }
     return hipGetLastError();
 }
 
 template <typename T, int ITERS>
-void act_trunc_launch(dim3 grid, int blk, hipStream_t s, T *delta, T *prev, T *trunc,
-                      int32_t *mask, float thr, int act, int mode, int P, int C, int G) {
-#define DC_AT(A) act_trunc_vec_kernel<T, ITERS, A><<<grid, blk, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, G)
+void act_trunc_launch(dim3 grid, hipStream_t s, T *delta, T *prev, T *trunc, int32_t *mask,
+                      float thr, int act, int mode, int P, int C, int lg) {
+#define DC_AT(A) act_trunc_vec_kernel<T, ITERS, A><<<grid, 256, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, lg)
     switch (act) {
         case DC_ACT_RELU: DC_AT(DC_ACT_RELU); break;
         case DC_ACT_RELU6: DC_AT(DC_ACT_RELU6); break;
@@ -552,30 +466,29 @@ hipError_t act_trunc_t(T *delta, T *prev, T *trunc, int32_t *mask, float thr, in
                        int P, int C, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
     if (act < 0) act = 0;
-    int blk = block_for(P);
-    dim3 grid((unsigned)ceil_div(P, blk));
     if (mode < 0) {
         if (can_vec<T>(C, {delta, prev})) {
-            int G = group_lanes(C / N, 1);
-            accumulate_kernel<T, N><<<grid, blk, 0, s>>>(delta, prev, mask, act, P, C, G);
+            GroupLaunch L(P, pick_group(C / N, P, 4));
+            accumulate_kernel<T, N><<<L.grid, 256, 0, s>>>(delta, prev, mask, act, P, C, L.lg);
         } else {
-            int G = group_lanes(C, 1);
-            accumulate_kernel<T, 1><<<grid, blk, 0, s>>>(delta, prev, mask, act, P, C, G);
+            GroupLaunch L(P, group_lanes(C, 1));
+            accumulate_kernel<T, 1><<<L.grid, 256, 0, s>>>(delta, prev, mask, act, P, C, L.lg);
         }
         return hipGetLastError();
     }
     if (can_vec<T>(C, {delta, prev, trunc}) && C / N <= WAVE * 4) {
         int nvec = C / N;
-        int G = group_lanes(nvec, 4);
+        int G = pick_group(nvec, P, 4);
         int iters = ceil_div(nvec, G);
+        GroupLaunch L(P, G);
         switch (iters) {
-            case 1: act_trunc_launch<T, 1>(grid, blk, s, delta, prev, trunc, mask, thr, act, mode, P, C, G); break;
-            case 2: act_trunc_launch<T, 2>(grid, blk, s, delta, prev, trunc, mask, thr, act, mode, P, C, G); break;
-            default: act_trunc_launch<T, 4>(grid, blk, s, delta, prev, trunc, mask, thr, act, mode, P, C, G); break;
+            case 1: act_trunc_launch<T, 1>(L.grid, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;
+            case 2: act_trunc_launch<T, 2>(L.grid, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;
+            default: act_trunc_launch<T, 4>(L.grid, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;
         }
     } else {
-        int G = group_lanes(C, 1);
-        act_trunc_gen_kernel<T><<<grid, blk, 0, s>>>(delta, prev, trunc, mask, thr, act, mode, P, C, G);
+        GroupLaunch L(P, group_lanes(C, 1));
+        act_trunc_gen_kernel<T><<<L.grid, 256, 0, s>>>(delta, prev, trunc, mask, thr, act, mode, P, C, L.lg);
     }
     return hipGetLastError();
 }
@@ -587,18 +500,13 @@ hipError_t add_t(const T *a, const T *b, T *prev, T *out, const int32_t *ma, con
     constexpr int N = Vec16<T>::N;
     if (act < 0) act = 0;
     const bool vec = can_vec<T>(C, {a, b, prev, out});
-    const int G = group_lanes(vec ? C / N : C, 1);
+    GroupLaunch L(P, vec ? pick_group(C / N, P, 4) : group_lanes(C, 1));
     if (dense_out) {
-        int64_t threads = (int64_t)P * G;
-        int blk = block_for(threads);
-        dim3 grid((unsigned)ceil_div64(threads, blk));
-        if (vec) add_dense_kernel<T, N><<<grid, blk, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, G);
-        else add_dense_kernel<T, 1><<<grid, blk, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, G);
+        if (vec) add_dense_kernel<T, N><<<L.grid, 256, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, L.lg);
+        else add_dense_kernel<T, 1><<<L.grid, 256, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, L.lg);
     } else {
-        int blk = block_for(P);
-        dim3 grid((unsigned)ceil_div(P, blk));
-        if (vec) add_kernel<T, N><<<grid, blk, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, G);
-        else add_kernel<T, 1><<<grid, blk, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, G);
+        if (vec) add_kernel<T, N><<<L.grid, 256, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, L.lg);
+        else add_kernel<T, 1><<<L.grid, 256, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, L.lg);
     }
     return hipGetLastError();
 }
@@ -634,19 +542,14 @@ template <typename T>
 hipError_t add_to_dense_t(T *a, T *b, const int32_t *ma, int act, int P, int C, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
     const bool vec = can_vec<T>(C, {a, b});
-    const int G = group_lanes(vec ? C / N : C, 1);
+    GroupLaunch L(P, vec ? pick_group(C / N, P, 4) : group_lanes(C, 1));
     if (act > 0) {
-        int64_t threads = (int64_t)P * G;
-        int blk = block_for(threads);
-        dim3 grid((unsigned)ceil_div64(threads, blk));
-        if (vec) add_to_dense_act_kernel<T, N><<<grid, blk, 0, s>>>(a, b, ma, act, P, C, G);
-        else add_to_dense_act_kernel<T, 1><<<grid, blk, 0, s>>>(a, b, ma, act, P, C, G);
-        return hipGetLastError();
+        if (vec) add_to_dense_act_kernel<T, N><<<L.grid, 256, 0, s>>>(a, b, ma, act, P, C, L.lg);
+        else add_to_dense_act_kernel<T, 1><<<L.grid, 256, 0, s>>>(a, b, ma, act, P, C, L.lg);
+    } else {
+        if (vec) add_to_dense_kernel<T, N><<<L.grid, 256, 0, s>>>(a, b, ma, P, C, L.lg);
+        else add_to_dense_kernel<T, 1><<<L.grid, 256, 0, s>>>(a, b, ma, P, C, L.lg);
     }
-    int blk = block_for(P);
-    dim3 grid((unsigned)ceil_div(P, blk));
-    if (vec) add_to_dense_kernel<T, N><<<grid, blk, 0, s>>>(a, b, ma, P, C, G);
-    else add_to_dense_kernel<T, 1><<<grid, blk, 0, s>>>(a, b, ma, P, C, G);
     return hipGetLastError();
 }
 template <typename T>
@@ -654,33 +557,40 @@ hipError_t upsample_t(const T *in, T *out, const int32_t *mi, int32_t *mo, int B
                       int C, int S, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
     int P = B * H * W;
-    int blk = block_for(P);
-    dim3 grid((unsigned)ceil_div(P, blk));
-    if (can_vec<T>(C, {in, out})) upsample_kernel<T, N><<<grid, blk, 0, s>>>(in, out, mi, mo, B, H, W, C, S, group_lanes(C / N, 1));
-    else upsample_kernel<T, 1><<<grid, blk, 0, s>>>(in, out, mi, mo, B, H, W, C, S, group_lanes(C, 1));
+    if (can_vec<T>(C, {in, out})) {
+        GroupLaunch L(P, pick_group(C / N, P, 4));
+        upsample_kernel<T, N><<<L.grid, 256, 0, s>>>(in, out, mi, mo, B, H, W, C, S, L.lg);
+    } else {
+        GroupLaunch L(P, group_lanes(C, 1));
+        upsample_kernel<T, 1><<<L.grid, 256, 0, s>>>(in, out, mi, mo, B, H, W, C, S, L.lg);
+    }
     return hipGetLastError();
 }
 template <typename T>
 hipError_t concat_t(const T *a, const T *b, T *out, const int32_t *ma, const int32_t *mb,
                     int32_t *mo, int P, int Ca, int Cb, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
-    int blk = block_for(P);
-    dim3 grid((unsigned)ceil_div(P, blk));
     int Cm = Ca > Cb ? Ca : Cb;
-    if (Ca % N == 0 && Cb % N == 0 && can_vec<T>(Ca, {a, b, out}))
-        concat_kernel<T, N><<<grid, blk, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, group_lanes(Cm / N, 1));
-    else
-        concat_kernel<T, 1><<<grid, blk, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, group_lanes(Cm, 1));
+    if (Ca % N == 0 && Cb % N == 0 && can_vec<T>(Ca, {a, b, out})) {
+        GroupLaunch L(P, pick_group(Cm / N, P, 4));
+        concat_kernel<T, N><<<L.grid, 256, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, L.lg);
+    } else {
+        GroupLaunch L(P, group_lanes(Cm, 1));
+        concat_kernel<T, 1><<<L.grid, 256, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, L.lg);
+    }
     return hipGetLastError();
 }
 template <typename T>
 hipError_t mul_add_t(const T *in, const int32_t *mask, T *out, int32_t *mo, const T *scale,
                      const T *bias, int P, int C, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
-    int blk = block_for(P);
-    dim3 grid((unsigned)ceil_div(P, blk));
-    if (can_vec<T>(C, {in, out, scale, bias})) mul_add_kernel<T, N><<<grid, blk, 0, s>>>(in, mask, out, mo, scale, bias, P, C, group_lanes(C / N, 1));
-    else mul_add_kernel<T, 1><<<grid, blk, 0, s>>>(in, mask, out, mo, scale, bias, P, C, group_lanes(C, 1));
+    if (can_vec<T>(C, {in, out, scale, bias})) {
+        GroupLaunch L(P, pick_group(C / N, P, 4));
+        mul_add_kernel<T, N><<<L.grid, 256, 0, s>>>(in, mask, out, mo, scale, bias, P, C, L.lg);
+    } else {
+        GroupLaunch L(P, group_lanes(C, 1));
+        mul_add_kernel<T, 1><<<L.grid, 256, 0, s>>>(in, mask, out, mo, scale, bias, P, C, L.lg);
+    }
     return hipGetLastError();
 }
 }  // namespace
