@@ -59,14 +59,26 @@ __device__ __forceinline__ int wave_rank(bool p, int &count) {
 
 // Activation functions, one IEEE operation at a time in the tensor's own type so that
 // results are bit-identical to evaluating the same expression op by op on the host.
+// sigmoid / swish through fp32 exp.  Kept out of line, conversion included: when these are
+// inlined into unrolled vector loops the compiler folds the surrounding negations into packed
+// two-float operations that this target (packed fp32 ops disabled) cannot select.
+__device__ __attribute__((noinline)) float sigmoid_t(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __attribute__((noinline)) float swish_t(float x) { return x * (1.0f / (1.0f + expf(-x))); }
+__device__ __attribute__((noinline)) half_t sigmoid_t(half_t x) {
+    return half_t(1.0f / (1.0f + expf(-float(x))));
+}
+__device__ __attribute__((noinline)) half_t swish_t(half_t x) {
+    return half_t(float(x) * (1.0f / (1.0f + expf(-float(x)))));
+}
+
 template <typename T>
 __device__ __forceinline__ T act_apply(T x, int act) {
     switch (act) {
         case DC_ACT_RELU: return x < T(0) ? T(0) : x;
         case DC_ACT_RELU6: return x < T(0) ? T(0) : (x > T(6) ? T(6) : x);
         case DC_ACT_LEAKY: return x < T(0) ? x * T(0.1f) : x;
-        case DC_ACT_SIGMOID: return T(1.0f / (1.0f + __expf(-float(x))));
-        case DC_ACT_SWISH: return T(float(x) / (1.0f + __expf(-float(x))));
+        case DC_ACT_SIGMOID: return sigmoid_t(x);
+        case DC_ACT_SWISH: return swish_t(x);
         default: return x;
     }
 }
@@ -77,10 +89,8 @@ __device__ __forceinline__ half_t fma_t(half_t a, half_t b, half_t c) {
     return __builtin_fmaf16(a, b, c);
 }
 
-template <typename T>
-__device__ __forceinline__ T tabs(T x) {
-    return x < T(0) ? -x : x;
-}
+__device__ __forceinline__ float tabs(float x) { return __builtin_fabsf(x); }
+__device__ __forceinline__ half_t tabs(half_t x) { return __builtin_fabsf16(x); }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }

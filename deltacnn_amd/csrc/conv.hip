@@ -101,7 +101,7 @@ struct EpiP {
     int mode;
 };
 
-template <typename T, int ITERS, int ACT>
+template <typename T, int ITERS, int ACT, bool K3>
 __global__ void __launch_bounds__(256)
 conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
                const T *__restrict__ bias, T *__restrict__ out, const int32_t *__restrict__ mask,
@@ -136,6 +136,12 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
     if (valid && gl == 0) out_mask[po] = active ? 1 : 0;
     if (ballot(active) == 0) return;
 
+    // cached state of the epilogue: requested now so that it arrives while the taps are summed
+    Vec<T, N> q[ITERS], tr[ITERS];
+    if (ACT >= 0)
+        load_state<T, ITERS>(q, tr, active, (size_t)po, gl, G, C, (const T *)epi.prev,
+                             (const T *)epi.trunc);
+
     float acc[ITERS][N];
 #pragma unroll
     for (int it = 0; it < ITERS; ++it)
@@ -143,21 +149,51 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
         for (int j = 0; j < N; ++j) acc[it][j] = 0.f;
     if (active) {
         const T *inb = in + (size_t)b * p.Hi * p.Wi * C;
-        for (int t = 0; t < K2; ++t) {
-            if (!((taps >> t) & 1ull)) continue;
-            const int ky = t / p.Kw, kx = t - ky * p.Kw;
-            const int iy = oy * p.sh - p.pt + ky * p.dh, ix = ox * p.sw - p.pl + kx * p.dw;
-            const T *xr = inb + (size_t)(iy * p.Wi + ix) * C;
-            const T *wr = filter + (size_t)t * C;
+        if (K3 && ITERS <= 2) {
+            // 3x3: all tap loads are issued before the first multiply (one memory round trip)
+            Vec<T, N> x[9][ITERS], w[9][ITERS];
 #pragma unroll
-            for (int it = 0; it < ITERS; ++it) {
-                const int c = (it * G + gl) * N;
-                if (c < C) {
-                    const Vec<T, N> x = vload<T, N>(xr + c);
-                    const Vec<T, N> w = vload<T, N>(wr + c);
+            for (int t = 0; t < 9; ++t) {
+                const bool on = (taps >> t) & 1ull;
+                const int ky = t / 3, kx = t - ky * 3;
+                const int iy = oy * p.sh - p.pt + ky * p.dh, ix = ox * p.sw - p.pl + kx * p.dw;
+                const T *xr = inb + (size_t)(iy * p.Wi + ix) * C;
+#pragma unroll
+                for (int it = 0; it < ITERS; ++it) {
+                    const int c = (it * G + gl) * N;
+                    if (on && c < C) {
+                        x[t][it] = vload<T, N>(xr + c);
+                        w[t][it] = vload<T, N>(filter + (size_t)t * C + c);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < N; ++j) x[t][it].v[j] = w[t][it].v[j] = T(0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < 9; ++t)
+#pragma unroll
+                for (int it = 0; it < ITERS; ++it)
 #pragma unroll
                     for (int j = 0; j < N; ++j)
-                        acc[it][j] = __builtin_fmaf(float(x.v[j]), float(w.v[j]), acc[it][j]);
+                        acc[it][j] = __builtin_fmaf(float(x[t][it].v[j]), float(w[t][it].v[j]), acc[it][j]);
+        } else {
+            for (int t = 0; t < K2; ++t) {
+                if (!((taps >> t) & 1ull)) continue;
+                const int ky = t / p.Kw, kx = t - ky * p.Kw;
+                const int iy = oy * p.sh - p.pt + ky * p.dh, ix = ox * p.sw - p.pl + kx * p.dw;
+                const T *xr = inb + (size_t)(iy * p.Wi + ix) * C;
+                const T *wr = filter + (size_t)t * C;
+#pragma unroll
+                for (int it = 0; it < ITERS; ++it) {
+                    const int c = (it * G + gl) * N;
+                    if (c < C) {
+                        const Vec<T, N> x = vload<T, N>(xr + c);
+                        const Vec<T, N> w = vload<T, N>(wr + c);
+#pragma unroll
+                        for (int j = 0; j < N; ++j)
+                            acc[it][j] = __builtin_fmaf(float(x.v[j]), float(w.v[j]), acc[it][j]);
+                    }
                 }
             }
         }
@@ -185,9 +221,100 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
             }
         }
     } else {
-        act_trunc_pixel<T, ITERS, (ACT < 0 ? 0 : ACT)>(dl, active, (size_t)po, gl, G, C, out,
+        act_trunc_pixel<T, ITERS, (ACT < 0 ? 0 : ACT)>(dl, q, tr, active, (size_t)po, gl, G, C, out,
                                                          (T *)epi.prev, (T *)epi.trunc, out_mask,
                                                          T(epi.thr), epi.mode);
+    }
+}
+
+// ------------------------------------------------------------------ few input channels
+// Network stems (RGB input): groups == 1, Cin <= 4.  Same one-group-per-output-pixel shape as
+// the depthwise kernel; a lane owns N consecutive output channels, input values are scalar
+// broadcasts.  fp16 filters are read in the reference layout directly: for an even channel
+// offset the even outputs sit in row ci and the odd ones in row ci ^ 1 of the swizzle.
+template <typename T, int ACT>
+__global__ void __launch_bounds__(256)
+conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
+                   const T *__restrict__ bias, T *__restrict__ out,
+                   const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, EpiP epi,
+                   int lg) {
+    constexpr int N = Vec16<T>::N;
+    constexpr int MAXCI = 4;
+    const int G = 1 << lg;
+    const int C = p.Co;
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int po = gid >> lg, gl = gid & (G - 1);
+    const int P_out = p.B * p.Ho * p.Wo;
+    const bool valid = po < P_out;
+    const int b = po / (p.Ho * p.Wo);
+    const int r = po - b * p.Ho * p.Wo;
+    const int oy = r / p.Wo, ox = r - oy * p.Wo;
+    const int K2 = p.Kh * p.Kw;
+    const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
+    const int glo = lane_id() & ~(G - 1);
+    const uint64_t gmask = G >= WAVE ? ~0ull : ((1ull << G) - 1ull);
+
+    uint64_t taps = 0;
+    for (int j = 0; j < K2; j += G) {
+        const int t = j + gl;
+        bool m = false;
+        if (valid && t < K2) {
+            const int ky = t / p.Kw, kx = t - ky * p.Kw;
+            const int iy = oy * p.sh - p.pt + ky * p.dh, ix = ox * p.sw - p.pl + kx * p.dw;
+            if (iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi) m = mb[iy * p.Wi + ix] != 0;
+        }
+        taps |= ((ballot(m) >> glo) & gmask) << j;
+    }
+    const bool active = valid && taps != 0;
+    if (valid && gl == 0) out_mask[po] = active ? 1 : 0;
+    if (ballot(active) == 0) return;
+
+    const int c = gl * N;
+    const bool lane_on = active && c < C;
+    Vec<T, N> q[1], tr[1];
+    if (ACT >= 0)
+        load_state<T, 1>(q, tr, active, (size_t)po, gl, G, C, (const T *)epi.prev, (const T *)epi.trunc);
+    float acc[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) acc[j] = 0.f;
+    if (lane_on) {
+        const T *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+        for (int t = 0; t < K2; ++t) {
+            if (!((taps >> t) & 1ull)) continue;
+            const int ky = t / p.Kw, kx = t - ky * p.Kw;
+            const int iy = oy * p.sh - p.pt + ky * p.dh, ix = ox * p.sw - p.pl + kx * p.dw;
+            const T *xr = inb + (size_t)(iy * p.Wi + ix) * p.Ci;
+#pragma unroll
+            for (int ci = 0; ci < MAXCI; ++ci) {
+                if (ci >= p.Ci) break;
+                const float xv = float(xr[ci]);
+                Vec<T, N> w = vload<T, N>(filter + ((size_t)ci * K2 + t) * p.w_co + c);
+                if (p.swz) {
+                    const Vec<T, N> w1 = vload<T, N>(filter + ((size_t)(ci ^ 1) * K2 + t) * p.w_co + c);
+#pragma unroll
+                    for (int j = 1; j < N; j += 2) w.v[j] = w1.v[j];
+                }
+#pragma unroll
+                for (int j = 0; j < N; ++j) acc[j] = __builtin_fmaf(xv, float(w.v[j]), acc[j]);
+            }
+        }
+    }
+    Vec<T, N> dl[1];
+    if (lane_on) {
+        if (bias != nullptr) {
+            const Vec<T, N> bv = vload<T, N>(bias + c);
+#pragma unroll
+            for (int j = 0; j < N; ++j) acc[j] += float(bv.v[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < N; ++j) dl[0].v[j] = T(acc[j]);
+    }
+    if (ACT < 0) {
+        if (lane_on) vstore<T, N>(out + (size_t)po * C + c, dl[0]);
+    } else {
+        act_trunc_pixel<T, 1, (ACT < 0 ? 0 : ACT)>(dl, q, tr, active, (size_t)po, gl, G, C, out,
+                                                     (T *)epi.prev, (T *)epi.trunc, out_mask,
+                                                     T(epi.thr), epi.mode);
     }
 }
 
@@ -244,47 +371,68 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
     const int ksteps = ci_p >> 5;
     const int total = K2 * ksteps;
     const int kvalid = kq * 8;  // this lane's channel offset inside a 32-wide step
+    const int first = KSPLIT ? wave : 0, stride = KSPLIT ? 4 : 1;
+    // Reduction steps are taken S at a time: all fragment loads of a chunk are issued before
+    // its first MFMA, so a chunk costs one memory round trip instead of S.
+    constexpr int S = 4;
     int cur_tap = -1;
     const half_t *xrow[NT];
     bool xok[NT];
     bool tap_used = false;
-    for (int s = KSPLIT ? wave : 0; s < total; s += KSPLIT ? 4 : 1) {
-        const int tap = s / ksteps;
-        const int k0 = (s - tap * ksteps) << 5;
-        if (tap != cur_tap) {
-            cur_tap = tap;
-            const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
-            bool any = false;
+    for (int s0 = first; s0 < total; s0 += S * stride) {
+        half8_t a[S], x[S][NT];
+        bool use[S];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                int ipix = -1;
-                if (oy[nt] >= 0) {
-                    if (pointwise) {
-                        ipix = oy[nt] * p.Wi + ox[nt];
-                    } else {
-                        int iy, ix;
-                        if (tap_src<TR>(oy[nt], ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
-                            tap_src<TR>(ox[nt], kx, p.sw, p.dw, p.pl, p.Wi, ix) &&
-                            mb[iy * p.Wi + ix] != 0)
-                            ipix = iy * p.Wi + ix;
+        for (int i = 0; i < S; ++i) {
+            const int s = s0 + i * stride;
+            use[i] = false;
+            if (s < total) {
+                const int tap = s / ksteps;
+                const int k0 = (s - tap * ksteps) << 5;
+                if (tap != cur_tap) {
+                    cur_tap = tap;
+                    const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
+                    bool any = false;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        int ipix = -1;
+                        if (oy[nt] >= 0) {
+                            if (pointwise) {
+                                ipix = oy[nt] * p.Wi + ox[nt];
+                            } else {
+                                int iy, ix;
+                                if (tap_src<TR>(oy[nt], ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
+                                    tap_src<TR>(ox[nt], kx, p.sw, p.dw, p.pl, p.Wi, ix) &&
+                                    mb[iy * p.Wi + ix] != 0)
+                                    ipix = iy * p.Wi + ix;
+                            }
+                        }
+                        xok[nt] = ipix >= 0;
+                        any |= xok[nt];
+                        xrow[nt] = inb + (size_t)(ipix < 0 ? 0 : ipix) * p.Ci + kvalid;
+                    }
+                    tap_used = ballot(any) != 0;  // does any pixel of this tile use the tap?
+                }
+                use[i] = tap_used;
+                if (tap_used) {
+                    a[i] = *reinterpret_cast<const half8_t *>(wrow + (size_t)tap * ci_p + k0);
+                    const bool kin = k0 + kvalid < p.Ci;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        x[i][nt] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                        if (nt < n_tiles && xok[nt] && kin)
+                            x[i][nt] = *reinterpret_cast<const half8_t *>(xrow[nt] + k0);
                     }
                 }
-                xok[nt] = ipix >= 0;
-                any |= xok[nt];
-                xrow[nt] = inb + (size_t)(ipix < 0 ? 0 : ipix) * p.Ci + kvalid;
             }
-            tap_used = ballot(any) != 0;  // does any pixel of this tile use the tap at all?
         }
-        if (!tap_used) continue;
-        const half8_t a = *reinterpret_cast<const half8_t *>(wrow + (size_t)tap * ci_p + k0);
-        const bool kin = k0 + kvalid < p.Ci;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            if (nt < n_tiles) {
-                half8_t x = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (xok[nt] && kin) x = *reinterpret_cast<const half8_t *>(xrow[nt] + k0);
-                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, x, acc[nt], 0, 0, 0);
-            }
+        for (int i = 0; i < S; ++i) {
+            if (!use[i]) continue;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                if (nt < n_tiles)
+                    acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], x[i][nt], acc[nt], 0, 0, 0);
         }
     }
 
@@ -394,7 +542,11 @@ namespace {
 template <typename T, int ITERS>
 void dw_launch(dim3 grid, hipStream_t s, int act, const ConvP &p, const T *in, const T *filter,
                const T *bias, T *out, const int32_t *mask, int32_t *out_mask, EpiP e, int lg) {
-#define DC_DW(A) conv_dw_kernel<T, ITERS, A><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg)
+#define DC_DW(A) \
+    do { \
+        if (p.Kh == 3 && p.Kw == 3) conv_dw_kernel<T, ITERS, A, true><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg); \
+        else conv_dw_kernel<T, ITERS, A, false><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg); \
+    } while (0)
     switch (act) {
         case DC_ACT_LINEAR: DC_DW(DC_ACT_LINEAR); break;
         case DC_ACT_RELU: DC_DW(DC_ACT_RELU); break;
@@ -435,6 +587,37 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
     return true;
 }
 
+template <typename T>
+bool try_fewcin(const dc_geometry &g, const ConvP &p, const T *in, const T *filter, const T *bias,
+                T *out, const int32_t *mask, int32_t *out_mask, const ActEpilogue *epi,
+                hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    const auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (g.groups != 1 || g.in_c > 4 || g.out_c % N != 0 || g.out_c / N > WAVE) return false;
+    if (g.kernel_h * g.kernel_w > 64) return false;
+    if (!al(filter) || !al(out) || (bias && !al(bias))) return false;
+    if (epi && (!al(epi->prev) || (epi->trunc && !al(epi->trunc)) || epi->mode < 0)) return false;
+    const int64_t P_out = (int64_t)g.batch * g.out_h * g.out_w;
+    const int G = group_lanes(g.out_c / N, 1);
+    dim3 grid((unsigned)ceil_div64(P_out * G, 256));
+    EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f,
+           epi ? epi->mode : 0};
+    const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
+    const int lg = log2i(G);
+#define DC_FC(A) conv_fewcin_kernel<T, A><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg)
+    switch (act) {
+        case DC_ACT_LINEAR: DC_FC(DC_ACT_LINEAR); break;
+        case DC_ACT_RELU: DC_FC(DC_ACT_RELU); break;
+        case DC_ACT_RELU6: DC_FC(DC_ACT_RELU6); break;
+        case DC_ACT_LEAKY: DC_FC(DC_ACT_LEAKY); break;
+        case DC_ACT_SIGMOID: DC_FC(DC_ACT_SIGMOID); break;
+        case DC_ACT_SWISH: DC_FC(DC_ACT_SWISH); break;
+        default: DC_FC(-1); break;
+    }
+#undef DC_FC
+    return true;
+}
+
 }  // namespace
 
 hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
@@ -448,6 +631,10 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
             ? try_depthwise<float>(g, p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, epi, s)
             : try_depthwise<half_t>(g, p, (const half_t *)in, (const half_t *)filter, (const half_t *)bias, (half_t *)out, mask, out_mask, epi, s);
         if (done) return hipGetLastError();
+        const bool few = dtype == DC_F32
+            ? try_fewcin<float>(g, p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, epi, s)
+            : try_fewcin<half_t>(g, p, (const half_t *)in, (const half_t *)filter, (const half_t *)bias, (half_t *)out, mask, out_mask, epi, s);
+        if (few) return hipGetLastError();
     }
     if (packed != nullptr && mfma_eligible(g, dtype)) {
         const int co_tiles = ceil_div(g.out_c, 16);

@@ -109,13 +109,14 @@ act_trunc_vec_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict_
     group_coords(lg, p, gl);
     const bool valid = p < P && mask[p] != 0;
     if (ballot(valid) == 0) return;
-    Vec<T, N> dl[ITERS];
+    Vec<T, N> dl[ITERS], q[ITERS], tr[ITERS];
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int c = (it * G + gl) * N;
         if (valid && c < C) dl[it] = vload<T, N>(delta + (size_t)p * C + c);
     }
-    act_trunc_pixel<T, ITERS, ACT>(dl, valid, (size_t)p, gl, G, C, delta, prev, trunc, mask,
+    load_state<T, ITERS>(q, tr, valid, (size_t)p, gl, G, C, prev, trunc);
+    act_trunc_pixel<T, ITERS, ACT>(dl, q, tr, valid, (size_t)p, gl, G, C, delta, prev, trunc, mask,
                                    T(thr_f), mode);
 }
 

@@ -19,11 +19,31 @@ __device__ __forceinline__ float group_sum(float v, int G) {
     return v;
 }
 
-// `dl[it]` holds channels (it*G + gl)*N .. +N of the incoming delta for pixel `p` (only
-// meaningful where `valid` and the channel offset is < C).  All lanes of the wavefront must
-// call this (it contains wave-wide ballots).  Returns whether the pixel was kept.
+// `dl[it]` holds channels (it*G + gl)*N .. +N of the incoming delta for pixel `p`, `q` / `tr`
+// the same channels of the cached pre-activation and of the truncated remainder (loaded by the
+// caller as early as it can, see load_state; only meaningful where `valid` and the channel
+// offset is < C).  All lanes of the wavefront must call this (it contains wave-wide ballots).
+// Returns whether the pixel was kept.
+template <typename T, int ITERS>
+__device__ __forceinline__ void load_state(Vec<T, Vec16<T>::N> (&q)[ITERS],
+                                           Vec<T, Vec16<T>::N> (&tr)[ITERS], bool valid, size_t p,
+                                           int gl, int G, int C, const T *__restrict__ prev,
+                                           const T *__restrict__ trunc) {
+    constexpr int N = Vec16<T>::N;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int c = (it * G + gl) * N;
+        if (valid && c < C) {
+            q[it] = vload<T, N>(prev + p * C + c);
+            tr[it] = vload<T, N>(trunc + p * C + c);
+        }
+    }
+}
+
 template <typename T, int ITERS, int ACT>
-__device__ __forceinline__ bool act_trunc_pixel(Vec<T, Vec16<T>::N> (&dl)[ITERS], bool valid,
+__device__ __forceinline__ bool act_trunc_pixel(Vec<T, Vec16<T>::N> (&dl)[ITERS],
+                                                const Vec<T, Vec16<T>::N> (&q)[ITERS],
+                                                const Vec<T, Vec16<T>::N> (&tr)[ITERS], bool valid,
                                                 size_t p, int gl, int G, int C,
                                                 T *__restrict__ delta, T *__restrict__ prev,
                                                 T *__restrict__ trunc, int32_t *__restrict__ mask,
@@ -36,14 +56,11 @@ __device__ __forceinline__ bool act_trunc_pixel(Vec<T, Vec16<T>::N> (&dl)[ITERS]
     for (int it = 0; it < ITERS; ++it) {
         const int c = (it * G + gl) * N;
         if (valid && c < C) {
-            const size_t off = p * C + c;
-            const Vec<T, N> q = vload<T, N>(prev + off);
-            const Vec<T, N> tr = vload<T, N>(trunc + off);
 #pragma unroll
             for (int j = 0; j < N; ++j) {
-                t[it].v[j] = tr.v[j] + dl[it].v[j];
-                s[it].v[j] = t[it].v[j] + q.v[j];
-                const T d = act_apply<T>(s[it].v[j], ACT) - act_apply<T>(q.v[j], ACT);
+                t[it].v[j] = tr[it].v[j] + dl[it].v[j];
+                s[it].v[j] = t[it].v[j] + q[it].v[j];
+                const T d = act_apply<T>(s[it].v[j], ACT) - act_apply<T>(q[it].v[j], ACT);
                 dl[it].v[j] = d;
                 hit |= tabs(d) > thr;
                 sq += float(d) * float(d);

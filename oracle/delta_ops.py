@@ -72,7 +72,7 @@ def activation(x: torch.Tensor, act: int) -> torch.Tensor:
     if act == ACT_SIGMOID:
         return (1.0 / (1.0 + torch.exp(-x.float()))).to(x.dtype)
     if act == ACT_SWISH:
-        return (x.float() / (1.0 + torch.exp(-x.float()))).to(x.dtype)
+        return (x.float() * (1.0 / (1.0 + torch.exp(-x.float())))).to(x.dtype)
     raise ValueError(f"activation id {act}")
 
 

@@ -53,6 +53,45 @@ def test_sparsify(lib, dtype, C):
     assert bool(d_delta.cpu()[(want_mask == 0).expand_as(want_delta)].isnan().all())
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C,H,W", [(24, 192, 192), (96, 96, 96), (3, 224, 224)])
+def test_sparsify_large_map(lib, dtype, C, H, W):
+    """Big enough that a lane holds several vectors of its pixel."""
+    g = _gen(150 + C)
+    B = 2
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+    upd = rand_mask(g, B, H, W, 0.2) != 0
+    x = torch.where(upd, (prev.float() + torch.randn(B, C, H, W, generator=g) * 0.5).to(dtype), prev)
+    want_prev = prev.clone()
+    want_delta, want_mask = ops.sparsify(x, want_prev, 0.25)
+    d_prev, d_x = cl(prev), cl(x)
+    d_delta = torch.full_like(d_x, float("nan"))
+    d_mask = torch.full((B, 1, H, W), -7, dtype=torch.int32, device=DEV)
+    hk().sparsify(d_x, d_prev, d_delta, d_mask, 0.25)
+    assert torch.equal(d_mask.cpu(), want_mask)
+    assert_masked_equal(d_delta, want_delta, want_mask, "delta")
+    assert torch.equal(d_prev.cpu(), want_prev)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C,H,W", [(24, 192, 192), (96, 96, 96)])
+def test_activate_truncate_large_map(lib, dtype, C, H, W):
+    g = _gen(250 + C)
+    B = 2
+    mask = rand_mask(g, B, H, W, 0.3)
+    prev = (torch.randn(B, C, H, W, generator=g) * 3).to(dtype)
+    trunc = (torch.randn(B, C, H, W, generator=g) * 0.005).to(dtype)
+    big = rand_mask(g, B, H, W, 0.5).float()
+    delta = (torch.randn(B, C, H, W, generator=g) * (0.005 + 0.5 * big)).to(dtype)
+    w = [delta.clone(), prev.clone(), trunc.clone(), mask.clone()]
+    ops.activate_truncate(*w, 0.1, 2, 0)
+    d = [cl(poison(delta, mask)), cl(prev), cl(trunc), cl(mask)]
+    hk().sparse_activation(*d, 0.1, 2, 0)
+    assert torch.equal(d[3].cpu(), w[3])
+    assert_masked_equal(d[0], w[0], w[3], "delta")
+    assert torch.equal(d[1].cpu(), w[1]) and torch.equal(d[2].cpu(), w[2])
+
+
 # ------------------------------------------------------------------ activation + truncation
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("C", CHANNELS)
@@ -302,27 +341,42 @@ def test_deconv(lib, dtype, cfg, density, packed):
     _check_conv(dtype, out, want, want_mask)
 
 
+FUSED = [
+    (32, 64, 1, 1, 0, 1, 1, 12, 12),        # pointwise (separate epilogue launch)
+    (32, 32, 3, 1, 1, 1, 32, 12, 12),       # depthwise 3x3, epilogue in the kernel
+    (64, 64, 3, 2, 1, 1, 64, 13, 13),       # depthwise stride 2
+    (24, 24, 5, 1, 2, 1, 24, 12, 12),       # depthwise 5x5 (generic tap loop)
+    (3, 32, 3, 2, 1, 1, 1, 24, 24),         # RGB stem
+    (96, 96, 3, 1, 1, 1, 96, 96, 96),       # large map: two vectors per lane
+    (24, 24, 3, 1, 1, 1, 24, 192, 192),     # large map: three vectors per lane
+]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_conv_activation_fused(lib, dtype):
-    """dc_conv_act == dc_conv followed by dc_activate_truncate."""
-    cfg = (32, 64, 1, 1, 0, 1, 1, 12, 12)
+@pytest.mark.parametrize("cfg", FUSED, ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("act,mode", [(2, 0), (1, 0), (3, 1), (5, 0)])
+def test_conv_activation_fused(lib, dtype, cfg, act, mode):
+    """dc_conv_act == dc_conv followed by dc_activate_truncate, also against the oracle."""
+    Cin, Cout, H, W = cfg[0], cfg[1], cfg[7], cfg[8]
     x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 77, 0.4)
     g = _gen(78)
-    x = (x.float() * (0.01 + rand_mask(g, 2, 12, 12, 0.5).float())).to(dtype)  # small and large updates
-    prev = torch.randn(2, 64, 12, 12, generator=g).to(dtype)
-    trunc = (torch.randn(2, 64, 12, 12, generator=g) * 0.01).to(dtype)
+    x = (x.float() * (0.01 + rand_mask(g, 2, H, W, 0.5).float())).to(dtype)  # small and large updates
+    want_conv, want_mask = ops.conv(x, mask, wt, None, s, p, d, groups)
+    prev = torch.randn_like(want_conv.float(), ).to(dtype)
+    trunc = (torch.randn_like(prev.float()) * 0.01).to(dtype)
     d_filt = filt.to(DEV)
-    pk = hk().pack_filter(d_filt, 32, 64, 1)
+    pk = hk().pack_filter(d_filt, Cin, Cout, groups)
     dx, dm = cl(poison(x, mask)), cl(mask)
-    out1, om1 = hk().sparse_conv(dx, d_filt, dm, None, s, p, d, groups, c_out=64, create_out_mask=True,
+    out1, om1 = hk().sparse_conv(dx, d_filt, dm, None, s, p, d, groups, c_out=Cout, create_out_mask=True,
                                  packed_filter=pk)
+    assert torch.equal(om1.cpu(), want_mask)
     p1, t1 = cl(prev), cl(trunc)
-    hk().sparse_activation(out1, p1, t1, om1, 0.3, 2, 0)
+    hk().sparse_activation(out1, p1, t1, om1, 0.3, act, mode)
     p2, t2 = cl(prev), cl(trunc)
-    out2, om2 = hk().sparse_conv_activation(dx, d_filt, dm, None, p2, t2, 0.3, 2, 0, s, p, d, groups, 64,
+    out2, om2 = hk().sparse_conv_activation(dx, d_filt, dm, None, p2, t2, 0.3, act, mode, s, p, d, groups, Cout,
                                             packed_filter=pk)
     assert torch.equal(om1, om2)
-    assert 0 < int(om1.sum()) < int(mask.sum())
+    assert 0 < int(om1.sum()) < int(want_mask.sum())
     assert torch.equal(p1, p2) and torch.equal(t1, t2)
     assert_masked_equal(out2, out1.cpu(), om1.cpu(), "out")
 
