@@ -182,6 +182,8 @@ def main():
     ap.add_argument("--mode", choices=["graph", "eager"], default="graph")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--only-delta", action="store_true",
+                    help="time the delta path only and print a short JSON line (for profiling runs)")
     ap.add_argument("--cpu-frames", type=int, default=12)
     ap.add_argument("--trace-frames", type=int, default=8)
     args = ap.parse_args()
@@ -209,6 +211,10 @@ def main():
     sec = run_delta(delta, frames, args.warmup, args.steps, args.mode)
     fps = 1.0 / sec
     log(f"delta path: {fps:.1f} frames/s ({sec * 1e3:.3f} ms/frame, mode={args.mode})")
+    if args.only_delta:
+        print(json.dumps({"value": round(fps, 2), "unit": "frames/s", "ms_per_step": round(sec * 1e3, 4),
+                          "steps": args.steps, "update_density": args.density}), flush=True)
+        return
     with torch.no_grad():
         ref_logits = dense(frames[-1:]).float()
     dense_eager, dense_graph = run_dense(dense, frames, args.warmup, args.steps)

@@ -38,6 +38,11 @@ struct Vec16 {
     static constexpr int N = 16 / sizeof(T);
 };
 
+// Pin a loaded value at this program point: the compiler may neither sink the load that
+// produced it below this point nor start consuming it earlier, so a run of loads followed by
+// a run of pins is issued back to back and waited for once.
+#define DC_PIN(x) asm volatile("" : "+v"(x))
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
 
 __device__ __forceinline__ uint64_t ballot(bool p) { return __ballot(p); }
@@ -133,6 +138,10 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                        const void *packed, const void *bias, void *out, const int32_t *mask,
                        int32_t *out_mask, int dtype, bool transposed, const ActEpilogue *epi,
                        hipStream_t s);
+bool pointwise_eligible(const dc_geometry &g, int dtype);
+hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *packed,
+                            const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
+                            const ActEpilogue *epi, bool *epilogue_done, hipStream_t s);
 hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *packed, int dtype,
                               bool transposed, hipStream_t s);
 int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed);

@@ -150,33 +150,34 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
     if (active) {
         const T *inb = in + (size_t)b * p.Hi * p.Wi * C;
         if (K3 && ITERS <= 2) {
-            // 3x3: all tap loads are issued before the first multiply (one memory round trip)
+            // 3x3: every tap is loaded unconditionally from a clamped (always valid) address
+            // and zeroed afterwards if the tap is inactive, so all loads are in flight
+            // together: one memory round trip instead of one per tap
             Vec<T, N> x[9][ITERS], w[9][ITERS];
 #pragma unroll
             for (int t = 0; t < 9; ++t) {
-                const bool on = (taps >> t) & 1ull;
                 const int ky = t / 3, kx = t - ky * 3;
-                const int iy = oy * p.sh - p.pt + ky * p.dh, ix = ox * p.sw - p.pl + kx * p.dw;
+                const int iy = min(max(oy * p.sh - p.pt + ky * p.dh, 0), p.Hi - 1);
+                const int ix = min(max(ox * p.sw - p.pl + kx * p.dw, 0), p.Wi - 1);
                 const T *xr = inb + (size_t)(iy * p.Wi + ix) * C;
 #pragma unroll
                 for (int it = 0; it < ITERS; ++it) {
-                    const int c = (it * G + gl) * N;
-                    if (on && c < C) {
-                        x[t][it] = vload<T, N>(xr + c);
-                        w[t][it] = vload<T, N>(filter + (size_t)t * C + c);
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < N; ++j) x[t][it].v[j] = w[t][it].v[j] = T(0);
-                    }
+                    const int c = min((it * G + gl) * N, C - N);
+                    x[t][it] = vload<T, N>(xr + c);
+                    w[t][it] = vload<T, N>(filter + (size_t)t * C + c);
                 }
             }
 #pragma unroll
-            for (int t = 0; t < 9; ++t)
+            for (int t = 0; t < 9; ++t) {
+                const bool on = (taps >> t) & 1ull;
 #pragma unroll
                 for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-                    for (int j = 0; j < N; ++j)
-                        acc[it][j] = __builtin_fmaf(float(x[t][it].v[j]), float(w[t][it].v[j]), acc[it][j]);
+                    for (int j = 0; j < N; ++j) {
+                        const float xv = on ? float(x[t][it].v[j]) : 0.f;
+                        acc[it][j] = __builtin_fmaf(xv, float(w[t][it].v[j]), acc[it][j]);
+                    }
+            }
         } else {
             for (int t = 0; t < K2; ++t) {
                 if (!((taps >> t) & 1ull)) continue;
@@ -635,6 +636,13 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
             ? try_fewcin<float>(g, p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, epi, s)
             : try_fewcin<half_t>(g, p, (const half_t *)in, (const half_t *)filter, (const half_t *)bias, (half_t *)out, mask, out_mask, epi, s);
         if (few) return hipGetLastError();
+    }
+    if (packed != nullptr && !transposed && pointwise_eligible(g, dtype)) {
+        bool epilogue_done = false;
+        hipError_t e = launch_pointwise(g, in, packed, bias, out, mask, out_mask, epi, &epilogue_done, s);
+        if (e != hipSuccess || epi == nullptr || epilogue_done) return e;
+        return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
+                                        epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
     }
     if (packed != nullptr && mfma_eligible(g, dtype)) {
         const int co_tiles = ceil_div(g.out_c, 16);

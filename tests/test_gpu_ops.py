@@ -342,7 +342,12 @@ def test_deconv(lib, dtype, cfg, density, packed):
 
 
 FUSED = [
-    (32, 64, 1, 1, 0, 1, 1, 12, 12),        # pointwise (separate epilogue launch)
+    (32, 64, 1, 1, 0, 1, 1, 12, 12),        # pointwise, few pixels (separate epilogue launch)
+    (16, 96, 1, 1, 0, 1, 1, 40, 40),        # pointwise, epilogue in the kernel: 2 tiles/wave, 1 step
+    (64, 192, 1, 1, 0, 1, 1, 40, 40),       # 3 tiles/wave, 2 steps
+    (32, 384, 1, 1, 0, 1, 1, 40, 40),       # 6 tiles/wave, 1 step
+    (64, 512, 1, 1, 0, 1, 1, 40, 40),       # 8 tiles/wave, 2 steps
+    (24, 40, 1, 1, 0, 1, 1, 40, 40),        # partial channel tile and partial reduction step
     (32, 32, 3, 1, 1, 1, 32, 12, 12),       # depthwise 3x3, epilogue in the kernel
     (64, 64, 3, 2, 1, 1, 64, 13, 13),       # depthwise stride 2
     (24, 24, 5, 1, 2, 1, 24, 12, 12),       # depthwise 5x5 (generic tap loop)
