@@ -19,9 +19,9 @@
 // pw_act_mfma_kernel  convolution + activation/truncation in one launch: a workgroup owns ALL
 //                     output channels of its 16 pixels, so it can take the per-pixel keep/drop
 //                     decision itself; the convolution output never travels through memory.
-//                     Used for layers with many pixels and few channels (the high-resolution
-//                     half of a network); deep layers keep the two-launch form, whose channel
-//                     split over many workgroups is what streams their large filters fast
+//                     Used while the filter fragments of a wavefront fit in registers (up to
+//                     8 channel tiles x 5 reduction steps); larger layers keep the two-launch
+//                     form, whose channel split over many workgroups streams big filters fast
 #include "epilogue.hpp"
 
 namespace dc {
@@ -33,12 +33,15 @@ struct PwP {
     int P, Ci, Co, ci_p, co_tiles;
 };
 
-template <bool KSPLIT>
+// S = reduction steps per memory round trip (chunk): all fragment loads of S steps are in
+// flight together; the host picks the smallest S in {1, 2, 4, 8} that covers a wavefront's
+// share of the reduction, so most layers finish in a single chunk.
+template <bool KSPLIT, int S>
 __global__ void __launch_bounds__(256)
 pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                const half_t *__restrict__ bias, half_t *__restrict__ out,
                const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask) {
-    constexpr int NT = 4, S = 4;
+    constexpr int NT = 4;
     __shared__ float4_t s_red[KSPLIT ? 4 * NT * WAVE : 1];
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;
@@ -105,16 +108,16 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
             for (int nt = 0; nt < NT; ++nt)
                 x[i][nt] = *reinterpret_cast<const half8_t *>(xrow[nt] + k);
         }
+        // No zero-fill is needed: columns of inactive pixels are never stored, and where a step
+        // reaches past Cin the packed filter holds zeros while the clamped address re-reads
+        // finite values of the same pixel.
 #pragma unroll
         for (int i = 0; i < S; ++i) {
-            const int s = s0 + i * stride;
-            const bool kin = s < ksteps && (s << 5) + kvalid < p.Ci;
-            if (s < ksteps) {  // wave-uniform
+            if (s0 + i * stride < ksteps) {  // wave-uniform
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
                     if (nt_on[nt])  // wave-uniform
-                        acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            a[i], (on[nt] && kin) ? x[i][nt] : zero8(), acc[nt], 0, 0, 0);
+                        acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], x[i][nt], acc[nt], 0, 0, 0);
             }
         }
     }
@@ -132,27 +135,19 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
             if (nt == wave) acc[nt] = sum;
     }
     if (ct_raw >= p.co_tiles) return;
-    const int co = ct * 16 + kq * 4;
-    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    const int co = ct * 16 + kq * 4;  // Cout % 4 == 0: a lane's 4 channels are all in or all out
+    if (co >= p.Co) return;
+    float4_t bv = {0.f, 0.f, 0.f, 0.f};
     if (bias != nullptr) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (co + i < p.Co) bv[i] = float(bias[co + i]);
+        const half4_t b = *reinterpret_cast<const half4_t *>(bias + co);
+        bv = float4_t{float(b[0]), float(b[1]), float(b[2]), float(b[3])};
     }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         if (!on[nt] || (KSPLIT && nt != wave)) continue;
-        half_t *o = out + (size_t)px[nt] * p.Co + co;
-        if (co + 3 < p.Co && (p.Co & 3) == 0) {
-            half4_t r;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) r[i] = half_t(acc[nt][i] + bv[i]);
-            *reinterpret_cast<half4_t *>(o) = r;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (co + i < p.Co) o[i] = half_t(acc[nt][i] + bv[i]);
-        }
+        const float4_t r = acc[nt] + bv;
+        *reinterpret_cast<half4_t *>(out + (size_t)px[nt] * p.Co + co) =
+            half4_t{half_t(r[0]), half_t(r[1]), half_t(r[2]), half_t(r[3])};
     }
 }
 
@@ -162,40 +157,97 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
 // the 16 pixels stay in registers for the whole kernel and every loop is fully unrolled without
 // branches (surplus steps multiply zero fragments, surplus tiles are computed and dropped), so
 // the filter stream of a wavefront is one uninterrupted run of loads.  Requires Cout % 4 == 0.
+// Pass 1 of the epilogue: conv output v (rounded to fp16), T = trunc + v, S = T + prev,
+// D = act(S) - act(prev), one rounding each; collects the keep statistics of this lane.
 template <int CTW, int ACT>
-__device__ __forceinline__ void pw_epilogue(const float4_t (&acc)[CTW], const half4_t (&q)[CTW],
-                                            const half4_t (&tr)[CTW], half4_t (&t)[CTW],
-                                            half4_t (&sacc)[CTW], half4_t (&d)[CTW],
-                                            const half_t *__restrict__ bias, bool on, int wave,
-                                            int NW, int kq, const PwP &p, half_t thr, bool &hit,
-                                            float &sq) {
+__device__ __forceinline__ void pw_epilogue_stats(const float4_t (&acc)[CTW], const half4_t (&q)[CTW],
+                                                  const half4_t (&tr)[CTW], half4_t (&v)[CTW],
+                                                  const half_t *__restrict__ bias, bool on, int wave,
+                                                  int NW, int kq, const PwP &p, half_t thr, bool &hit,
+                                                  float &sq) {
 #pragma unroll
     for (int j = 0; j < CTW; ++j) {
         const int ct = wave + j * NW;
+        if (ct >= p.co_tiles) break;  // wave-uniform: surplus tiles of the last wavefronts
         const int co = ct * 16 + kq * 4;
-        const bool live = ct < p.co_tiles && co < p.Co;
+        const bool live = co < p.Co;
+        float4_t r = acc[j];
+        if (bias != nullptr && live) {
+            const half4_t b = *reinterpret_cast<const half4_t *>(bias + co);
+            r += float4_t{float(b[0]), float(b[1]), float(b[2]), float(b[3])};
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float b = (bias != nullptr && live) ? float(bias[co + i]) : 0.f;
-            const half_t v = half_t(acc[j][i] + b);
-            t[j][i] = tr[j][i] + v;
-            sacc[j][i] = t[j][i] + q[j][i];
-            d[j][i] = act_apply<half_t>(sacc[j][i], ACT) - act_apply<half_t>(q[j][i], ACT);
+            v[j][i] = half_t(r[i]);
+            const half_t t = tr[j][i] + v[j][i];
+            const half_t s = t + q[j][i];
+            const half_t d = act_apply<half_t>(s, ACT) - act_apply<half_t>(q[j][i], ACT);
             if (live && on) {
-                hit |= tabs(d[j][i]) > thr;
-                sq += float(d[j][i]) * float(d[j][i]);
+                hit |= tabs(d) > thr;
+                sq += float(d) * float(d);
             }
         }
     }
 }
 
-template <int NW, int CTW, int KS>
+// Pass 2: recompute T, S, D (a handful of ALU operations, cheaper than keeping them in
+// registers across the workgroup barrier) and write the kept / dropped state.
+template <int CTW, int ACT>
+__device__ __forceinline__ void pw_epilogue_store(const half4_t (&q)[CTW], const half4_t (&tr)[CTW],
+                                                  const half4_t (&v)[CTW], bool keep, int wave, int NW,
+                                                  int kq, int px, const PwP &p,
+                                                  half_t *__restrict__ out, half_t *__restrict__ prev,
+                                                  half_t *__restrict__ trunc) {
+#pragma unroll
+    for (int j = 0; j < CTW; ++j) {
+        const int ct = wave + j * NW;
+        if (ct >= p.co_tiles) break;  // wave-uniform
+        const int co = ct * 16 + kq * 4;
+        if (co >= p.Co) continue;
+        const size_t off = (size_t)px * p.Co + co;
+        half4_t t, s, d;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            t[i] = tr[j][i] + v[j][i];
+            s[i] = t[i] + q[j][i];
+            d[i] = act_apply<half_t>(s[i], ACT) - act_apply<half_t>(q[j][i], ACT);
+        }
+        if (keep) {
+            *reinterpret_cast<half4_t *>(prev + off) = s;
+            *reinterpret_cast<half4_t *>(out + off) = d;
+            *reinterpret_cast<half4_t *>(trunc + off) = half4_t{0, 0, 0, 0};
+        } else {
+            *reinterpret_cast<half4_t *>(trunc + off) = t;
+        }
+    }
+}
+
+#define DC_ACT_SWITCH(act, CALL)                                                \
+    switch (act) {                                                              \
+        case DC_ACT_RELU: { constexpr int A = DC_ACT_RELU; CALL; } break;       \
+        case DC_ACT_RELU6: { constexpr int A = DC_ACT_RELU6; CALL; } break;     \
+        case DC_ACT_LEAKY: { constexpr int A = DC_ACT_LEAKY; CALL; } break;     \
+        case DC_ACT_SIGMOID: { constexpr int A = DC_ACT_SIGMOID; CALL; } break; \
+        case DC_ACT_SWISH: { constexpr int A = DC_ACT_SWISH; CALL; } break;     \
+        default: { constexpr int A = DC_ACT_LINEAR; CALL; } break;              \
+    }
+
+// Workgroup = NW wavefronts x 16 pixels x all output channels; wavefront w owns channel tiles
+// w, w + NW, ... (at most CTW of them).  KS bounds the reduction steps.  Every loop is fully
+// unrolled without branches (surplus steps multiply zero fragments, surplus tiles are computed
+// and dropped).  The filter fragments of a wavefront are requested in AB batches: the first
+// together with the mask words, the second together with the input fragments and the cached
+// state, so the kernel is two memory round trips, the MFMAs, one barrier and the stores.
+// Requires Cout % 4 == 0.
+template <int NW, int CTW, int KS, int AB>
 __global__ void __launch_bounds__(NW * WAVE)
 pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                    const half_t *__restrict__ bias, half_t *__restrict__ out,
                    const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
                    half_t *__restrict__ prev, half_t *__restrict__ trunc, float thr_f, int act,
                    int mode) {
+    static_assert(CTW % AB == 0, "filter batches must divide the tiles of a wavefront");
+    constexpr int JB = CTW / AB;
     __shared__ float s_stat[NW][16];
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;
@@ -203,11 +255,11 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
     const int ksteps = p.ci_p >> 5;
     const int px = blockIdx.x * 16 + l16;
     const int m = mask[min(px, p.P - 1)];
-    // round trip 1: the mask word and every filter fragment of this wavefront (they do not
-    // depend on the mask; a workgroup without active pixels wastes a few cached KB)
     half8_t a[CTW][KS];
+    // round trip 1: mask word + first batch of filter fragments (they do not depend on the
+    // mask; a workgroup without active pixels wastes a few cached KB)
 #pragma unroll
-    for (int j = 0; j < CTW; ++j) {
+    for (int j = 0; j < JB; ++j) {
         const int ct = min(wave + j * NW, p.co_tiles - 1);
         const half_t *wrow = wp + (size_t)(ct * 16 + l16) * p.ci_p + kvalid;
 #pragma unroll
@@ -215,7 +267,7 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
             a[j][s] = *reinterpret_cast<const half8_t *>(wrow + (min(s, ksteps - 1) << 5));
     }
 #pragma unroll
-    for (int j = 0; j < CTW; ++j)
+    for (int j = 0; j < JB; ++j)
 #pragma unroll
         for (int s = 0; s < KS; ++s) DC_PIN(a[j][s]);
     const bool on = px < p.P && m != 0;
@@ -223,8 +275,17 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
         if (wave == 0 && kq == 0 && px < p.P) out_mask[px] = 0;
         return;
     }
-    // round trip 2: input fragments and cached state of this lane's (pixel, 4 channel) cells;
-    // inactive pixels all point at pixel 0, their loads share one cache line and are dropped
+    // round trip 2: remaining filter fragments, input fragments and cached state of this
+    // lane's (pixel, 4 channel) cells; inactive pixels all point at pixel 0, their loads share
+    // one cache line and are dropped
+#pragma unroll
+    for (int j = JB; j < CTW; ++j) {
+        const int ct = min(wave + j * NW, p.co_tiles - 1);
+        const half_t *wrow = wp + (size_t)(ct * 16 + l16) * p.ci_p + kvalid;
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            a[j][s] = *reinterpret_cast<const half8_t *>(wrow + (min(s, ksteps - 1) << 5));
+    }
     const half_t *xrow = in + (size_t)(on ? px : 0) * p.Ci;
     half8_t x[KS];
 #pragma unroll
@@ -242,38 +303,31 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
         tr[j] = *reinterpret_cast<const half4_t *>(trunc + off);
     }
 #pragma unroll
+    for (int j = JB; j < CTW; ++j)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) DC_PIN(a[j][s]);
+#pragma unroll
     for (int s = 0; s < KS; ++s) DC_PIN(x[s]);
 #pragma unroll
     for (int j = 0; j < CTW; ++j) {
         DC_PIN(q[j]);
         DC_PIN(tr[j]);
     }
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        const bool kin = s < ksteps && (s << 5) + kvalid < p.Ci;
-        x[s] = (on && kin) ? x[s] : zero8();
-    }
+    // no zero-fill: see pw_mfma_kernel (inactive columns are dropped, padded filter is zero)
     float4_t acc[CTW];
 #pragma unroll
     for (int j = 0; j < CTW; ++j) {
         acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KS; ++s)
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j][s], x[s], acc[j], 0, 0, 0);
+            if (s < ksteps)  // uniform
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j][s], x[s], acc[j], 0, 0, 0);
     }
-    // epilogue: T = trunc + delta; S = T + prev; D = act(S) - act(prev), one rounding each
     const half_t thr = half_t(thr_f);
-    half4_t t[CTW], sacc[CTW], d[CTW];
+    half4_t v[CTW];
     bool hit = false;
     float sq = 0.f;
-    switch (act) {
-        case DC_ACT_RELU: pw_epilogue<CTW, DC_ACT_RELU>(acc, q, tr, t, sacc, d, bias, on, wave, NW, kq, p, thr, hit, sq); break;
-        case DC_ACT_RELU6: pw_epilogue<CTW, DC_ACT_RELU6>(acc, q, tr, t, sacc, d, bias, on, wave, NW, kq, p, thr, hit, sq); break;
-        case DC_ACT_LEAKY: pw_epilogue<CTW, DC_ACT_LEAKY>(acc, q, tr, t, sacc, d, bias, on, wave, NW, kq, p, thr, hit, sq); break;
-        case DC_ACT_SIGMOID: pw_epilogue<CTW, DC_ACT_SIGMOID>(acc, q, tr, t, sacc, d, bias, on, wave, NW, kq, p, thr, hit, sq); break;
-        case DC_ACT_SWISH: pw_epilogue<CTW, DC_ACT_SWISH>(acc, q, tr, t, sacc, d, bias, on, wave, NW, kq, p, thr, hit, sq); break;
-        default: pw_epilogue<CTW, DC_ACT_LINEAR>(acc, q, tr, t, sacc, d, bias, on, wave, NW, kq, p, thr, hit, sq); break;
-    }
+    DC_ACT_SWITCH(act, (pw_epilogue_stats<CTW, A>(acc, q, tr, v, bias, on, wave, NW, kq, p, thr, hit, sq)));
     // per pixel: combine the four k-quarter lanes, then the wavefronts
     float stat;
     if (mode == DC_TRUNC_MAX) {
@@ -294,34 +348,14 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
     else keep = sqrtf(mode == DC_TRUNC_RMS ? tot / float(p.Co) : tot) > float(thr);
     if (wave == 0 && kq == 0 && px < p.P) out_mask[px] = (on && keep) ? 1 : 0;
     if (!on) return;
-#pragma unroll
-    for (int j = 0; j < CTW; ++j) {
-        const int ct = wave + j * NW;
-        const int co = ct * 16 + kq * 4;
-        if (ct >= p.co_tiles || co >= p.Co) continue;
-        const size_t off = (size_t)px * p.Co + co;
-        if (keep) {
-            *reinterpret_cast<half4_t *>(prev + off) = sacc[j];
-            *reinterpret_cast<half4_t *>(out + off) = d[j];
-            *reinterpret_cast<half4_t *>(trunc + off) = half4_t{0, 0, 0, 0};
-        } else {
-            *reinterpret_cast<half4_t *>(trunc + off) = t[j];
-        }
-    }
-}
-
-template <int CTW, int KS>
-void pw_act_launch(dim3 grid, hipStream_t s, const PwP &p, const half_t *in, const half_t *wp,
-                   const half_t *bias, half_t *out, const int32_t *mask, int32_t *out_mask,
-                   half_t *prev, half_t *trunc, float thr, int act, int mode) {
-    pw_act_mfma_kernel<4, CTW, KS><<<grid, 4 * WAVE, 0, s>>>(p, in, wp, bias, out, mask, out_mask,
-                                                            prev, trunc, thr, act, mode);
+    DC_ACT_SWITCH(act, (pw_epilogue_store<CTW, A>(q, tr, v, keep, wave, NW, kq, px, p, out, prev, trunc)));
 }
 
 }  // namespace
 
 bool pointwise_eligible(const dc_geometry &g, int dtype) {
-    return dtype == DC_F16 && g.groups == 1 && g.in_c % 8 == 0 && g.in_c >= 8 && g.kernel_h == 1 &&
+    return dtype == DC_F16 && g.groups == 1 && g.in_c % 8 == 0 && g.in_c >= 8 && g.out_c % 4 == 0 &&
+           g.kernel_h == 1 &&
            g.kernel_w == 1 && g.stride_h == 1 && g.stride_w == 1 && g.pad_top == 0 &&
            g.pad_left == 0 && g.pad_bottom == 0 && g.pad_right == 0;
 }
@@ -343,28 +377,50 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     const int ksteps = p.ci_p / 32;
     *epilogue_done = false;
     const auto al8 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 7u) == 0; };
-    // Fused epilogue where a workgroup can own all output channels of 16 pixels cheaply:
-    // enough pixels to fill the GPU with 16-pixel workgroups, few channel tiles per wavefront
-    // and a short reduction (all filter fragments of a wavefront live in registers).
-    const int ctw = ceil_div(p.co_tiles, 4);
-    const bool shape_ok = (ctw <= 4 && ksteps <= 3) || (ctw <= 8 && ksteps <= 2);
-    if (epi != nullptr && epi->mode >= 0 && shape_ok && p.P > 1024 && g.out_c % 4 == 0 &&
-        al8(epi->prev) && al8(epi->trunc) && al8(out)) {
+    // Fused epilogue where a workgroup can own all output channels of 16 pixels cheaply: few
+    // channel tiles per wavefront and a short reduction, so that all filter fragments of a
+    // wavefront live in registers.
+    const bool fusable = epi != nullptr && epi->mode >= 0 && g.out_c % 4 == 0 && al8(epi->prev) &&
+                         al8(epi->trunc) && al8(out);
+    if (fusable) {
         dim3 grid(ceil_div(p.P, 16));
         const int act = epi->act < 0 ? 0 : epi->act;
-#define DC_GO(CTW, KS) pw_act_launch<CTW, KS>(grid, s, p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, (half_t *)epi->prev, (half_t *)epi->trunc, epi->thr, act, epi->mode)
-        if (ctw <= 4) { if (ksteps <= 1) DC_GO(4, 1); else DC_GO(4, 3); }
-        else { if (ksteps <= 1) DC_GO(8, 1); else DC_GO(8, 2); }
+#define DC_GO(NW, CTW, KS, AB)                                                                       \
+    do {                                                                                             \
+        pw_act_mfma_kernel<NW, CTW, KS, AB><<<grid, NW * WAVE, 0, s>>>(                              \
+            p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, \
+            out_mask, (half_t *)epi->prev, (half_t *)epi->trunc, epi->thr, act, epi->mode);          \
+        *epilogue_done = true;                                                                       \
+        return hipGetLastError();                                                                    \
+    } while (0)
+        // Only maps with enough pixels to occupy the GPU with 16-pixel workgroups: a wavefront
+        // issues one instruction per 4 cycles, so a small map handled by a few fat workgroups is
+        // slower than the two-launch form whose channel split spreads over many wavefronts.
+        if (p.P > 1024) {
+            const int ctw = ceil_div(p.co_tiles, 4);
+            if (ctw <= 2 && ksteps <= 1) DC_GO(4, 2, 1, 1);
+            if (ctw <= 3 && ksteps <= 1) DC_GO(4, 3, 1, 1);
+            if (ctw <= 4 && ksteps <= 1) DC_GO(4, 4, 1, 1);
+            if (ctw <= 2 && ksteps <= 3) DC_GO(4, 2, 3, 1);
+            if (ctw <= 4 && ksteps <= 3) DC_GO(4, 4, 3, 1);
+            if (ctw <= 8 && ksteps <= 1) DC_GO(4, 8, 1, 1);
+            if (ctw <= 8 && ksteps <= 2) DC_GO(4, 8, 2, 1);
+        }
 #undef DC_GO
-        *epilogue_done = true;
-        return hipGetLastError();
     }
     const bool ksplit = ksteps > PW_KSPLIT_STEPS;
     dim3 grid(ceil_div(p.P, 64), ksplit ? p.co_tiles : ceil_div(p.co_tiles, 4));
-    if (ksplit)
-        pw_mfma_kernel<true><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask);
-    else
-        pw_mfma_kernel<false><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask);
+    const int per_wave = ksplit ? ceil_div(ksteps, 4) : ksteps;
+#define DC_PW(KS, SS) pw_mfma_kernel<KS, SS><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask)
+    if (ksplit) {
+        if (per_wave <= 4) DC_PW(true, 4); else DC_PW(true, 8);
+    } else {
+        if (per_wave <= 1) DC_PW(false, 1);
+        else if (per_wave <= 2) DC_PW(false, 2);
+        else if (per_wave <= 4) DC_PW(false, 4);
+        else DC_PW(false, 8);
+    }
+#undef DC_PW
     return hipGetLastError();
 }
 
