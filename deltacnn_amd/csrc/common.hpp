@@ -138,10 +138,17 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                        const void *packed, const void *bias, void *out, const int32_t *mask,
                        int32_t *out_mask, int dtype, bool transposed, const ActEpilogue *epi,
                        hipStream_t s);
+struct Residual {  // optional DCAdd fused behind a pointwise convolution
+    const void *values;
+    const int32_t *mask;
+    float wa, wb;
+};
+
 bool pointwise_eligible(const dc_geometry &g, int dtype);
 hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *packed,
                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
-                            const ActEpilogue *epi, bool *epilogue_done, hipStream_t s);
+                            const ActEpilogue *epi, bool *epilogue_done, const Residual *res,
+                            hipStream_t s);
 hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *packed, int dtype,
                               bool transposed, hipStream_t s);
 int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed);

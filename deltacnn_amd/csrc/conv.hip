@@ -639,7 +639,7 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
     }
     if (packed != nullptr && !transposed && pointwise_eligible(g, dtype)) {
         bool epilogue_done = false;
-        hipError_t e = launch_pointwise(g, in, packed, bias, out, mask, out_mask, epi, &epilogue_done, s);
+        hipError_t e = launch_pointwise(g, in, packed, bias, out, mask, out_mask, epi, &epilogue_done, nullptr, s);
         if (e != hipSuccess || epi == nullptr || epilogue_done) return e;
         return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
                                         epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);

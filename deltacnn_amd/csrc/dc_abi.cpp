@@ -182,6 +182,34 @@ int dc_conv_act(const dc_geometry *g, const void *input, const void *filter,
                                   dtype, false, &epi, (hipStream_t)stream), "dc_conv_act");
 }
 
+int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filter,
+                const void *bias, const int32_t *mask, const void *residual,
+                const int32_t *mask_residual, void *out, int32_t *out_mask, float weight_residual,
+                float weight_conv, int dtype, void *stream) {
+    DC_REQUIRE_DTYPE("dc_conv_add");
+    int rc = check_geometry("dc_conv_add", g, false, false);
+    if (rc != DC_OK) return rc;
+    if (!dc::pointwise_eligible(*g, dtype))
+        return fail(DC_ERR_UNSUPPORTED, "dc_conv_add: only fp16 1x1 stride-1 convolutions with "
+                                        "Cin %% 8 == 0 and Cout %% 4 == 0 have the fused form");
+    DC_REQUIRE_PTR("dc_conv_add", input);
+    DC_REQUIRE_PTR("dc_conv_add", packed_filter);
+    DC_REQUIRE_PTR("dc_conv_add", mask);
+    DC_REQUIRE_PTR("dc_conv_add", residual);
+    DC_REQUIRE_PTR("dc_conv_add", mask_residual);
+    DC_REQUIRE_PTR("dc_conv_add", out);
+    DC_REQUIRE_PTR("dc_conv_add", out_mask);
+    DC_REQUIRE_ALIGNED("dc_conv_add", input, 16);
+    DC_REQUIRE_ALIGNED("dc_conv_add", packed_filter, 16);
+    DC_REQUIRE_ALIGNED("dc_conv_add", residual, 8);
+    DC_REQUIRE_ALIGNED("dc_conv_add", out, 8);
+    DC_REQUIRE_ALIGNED("dc_conv_add", bias, 8);
+    dc::Residual res{residual, mask_residual, weight_residual, weight_conv};
+    bool unused = false;
+    return finish(dc::launch_pointwise(*g, input, packed_filter, bias, out, mask, out_mask, nullptr,
+                                       &unused, &res, (hipStream_t)stream), "dc_conv_add");
+}
+
 int64_t dc_packed_filter_bytes(const dc_geometry *g, int dtype, int transposed) {
     if (g == nullptr || g->in_c <= 0 || g->out_c <= 0 || g->kernel_h <= 0 || g->kernel_w <= 0 ||
         g->groups <= 0)

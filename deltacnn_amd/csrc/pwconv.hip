@@ -36,11 +36,22 @@ struct PwP {
 // S = reduction steps per memory round trip (chunk): all fragment loads of S steps are in
 // flight together; the host picks the smallest S in {1, 2, 4, 8} that covers a wavefront's
 // share of the reduction, so most layers finish in a single chunk.
-template <bool KSPLIT, int S>
+//
+// ADD fuses the residual sum of a DCAdd layer behind the convolution: with a = residual delta
+// (mask Ma) and b = convolution output rounded to fp16 (mask Mb = input mask),
+// out = fma(b, wb, a * wa) on pixels of Ma | Mb, each term present only where its mask is set --
+// the same operations, in the same order and precision, as the stand-alone add kernel.
+struct ResP {
+    const half_t *res;
+    const int32_t *mask;
+    float wa, wb;
+};
+
+template <bool KSPLIT, int S, bool ADD>
 __global__ void __launch_bounds__(256)
 pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                const half_t *__restrict__ bias, half_t *__restrict__ out,
-               const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask) {
+               const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, ResP rp) {
     constexpr int NT = 4;
     __shared__ float4_t s_red[KSPLIT ? 4 * NT * WAVE : 1];
     const int wave = threadIdx.x / WAVE, lane = lane_id();
@@ -54,12 +65,14 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
     const half_t *wrow = wp + (size_t)(ct * 16 + l16) * p.ci_p + kvalid;
 
     int px[NT];
-    bool on[NT];
+    bool on[NT], on_r[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         px[nt] = blockIdx.x * 64 + nt * 16 + l16;
         const int m = mask[min(px[nt], p.P - 1)];
         on[nt] = px[nt] < p.P && m != 0;
+        on_r[nt] = false;
+        if (ADD) on_r[nt] = px[nt] < p.P && rp.mask[min(px[nt], p.P - 1)] != 0;
     }
     // first chunk of filter fragments travels together with the mask words
     half8_t a[S];
@@ -73,14 +86,22 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         nt_on[nt] = ballot(on[nt]) != 0;
-        any |= nt_on[nt];
+        any |= ballot(on[nt] || on_r[nt]) != 0;
     }
     if (cb == 0 && wave == 0 && kq == 0) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-            if (px[nt] < p.P) out_mask[px[nt]] = on[nt] ? 1 : 0;
+            if (px[nt] < p.P) out_mask[px[nt]] = (on[nt] || on_r[nt]) ? 1 : 0;
     }
     if (!any) return;
+    const int co = ct * 16 + kq * 4;  // Cout % 4 == 0: a lane's 4 channels are all in or all out
+    half4_t res[NT];
+    if (ADD) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            res[nt] = *reinterpret_cast<const half4_t *>(
+                rp.res + (size_t)(on_r[nt] ? px[nt] : 0) * p.Co + min(co, p.Co - 4));
+    }
 
     float4_t acc[NT];
 #pragma unroll
@@ -135,19 +156,27 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
             if (nt == wave) acc[nt] = sum;
     }
     if (ct_raw >= p.co_tiles) return;
-    const int co = ct * 16 + kq * 4;  // Cout % 4 == 0: a lane's 4 channels are all in or all out
     if (co >= p.Co) return;
     float4_t bv = {0.f, 0.f, 0.f, 0.f};
     if (bias != nullptr) {
         const half4_t b = *reinterpret_cast<const half4_t *>(bias + co);
         bv = float4_t{float(b[0]), float(b[1]), float(b[2]), float(b[3])};
     }
+    const half_t wa = half_t(rp.wa), wb = half_t(rp.wb);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        if (!on[nt] || (KSPLIT && nt != wave)) continue;
+        if (!(on[nt] || on_r[nt]) || (KSPLIT && nt != wave)) continue;
         const float4_t r = acc[nt] + bv;
-        *reinterpret_cast<half4_t *>(out + (size_t)px[nt] * p.Co + co) =
-            half4_t{half_t(r[0]), half_t(r[1]), half_t(r[2]), half_t(r[3])};
+        half4_t o = half4_t{half_t(r[0]), half_t(r[1]), half_t(r[2]), half_t(r[3])};
+        if (ADD) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                half_t sum = on_r[nt] ? half_t(res[nt][i] * wa) : half_t(0);
+                if (on[nt]) sum = fma_t(o[i], wb, sum);
+                o[i] = sum;
+            }
+        }
+        *reinterpret_cast<half4_t *>(out + (size_t)px[nt] * p.Co + co) = o;
     }
 }
 
@@ -367,7 +396,8 @@ constexpr int PW_KSPLIT_STEPS = 10;
 
 hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *packed,
                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
-                            const ActEpilogue *epi, bool *epilogue_done, hipStream_t s) {
+                            const ActEpilogue *epi, bool *epilogue_done, const Residual *res,
+                            hipStream_t s) {
     PwP p;
     p.P = g.batch * g.in_h * g.in_w;
     p.Ci = g.in_c;
@@ -380,7 +410,7 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     // Fused epilogue where a workgroup can own all output channels of 16 pixels cheaply: few
     // channel tiles per wavefront and a short reduction, so that all filter fragments of a
     // wavefront live in registers.
-    const bool fusable = epi != nullptr && epi->mode >= 0 && g.out_c % 4 == 0 && al8(epi->prev) &&
+    const bool fusable = res == nullptr && epi != nullptr && epi->mode >= 0 && g.out_c % 4 == 0 && al8(epi->prev) &&
                          al8(epi->trunc) && al8(out);
     if (fusable) {
         dim3 grid(ceil_div(p.P, 16));
@@ -411,7 +441,15 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     const bool ksplit = ksteps > PW_KSPLIT_STEPS;
     dim3 grid(ceil_div(p.P, 64), ksplit ? p.co_tiles : ceil_div(p.co_tiles, 4));
     const int per_wave = ksplit ? ceil_div(ksteps, 4) : ksteps;
-#define DC_PW(KS, SS) pw_mfma_kernel<KS, SS><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask)
+    ResP rp{nullptr, nullptr, 1.f, 1.f};
+    if (res != nullptr) rp = ResP{(const half_t *)res->values, res->mask, res->wa, res->wb};
+#define DC_PW(KS, SS)                                                                                \
+    do {                                                                                             \
+        if (res != nullptr)                                                                          \
+            pw_mfma_kernel<KS, SS, true><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
+        else                                                                                         \
+            pw_mfma_kernel<KS, SS, false><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
+    } while (0)
     if (ksplit) {
         if (per_wave <= 4) DC_PW(true, 4); else DC_PW(true, 8);
     } else {

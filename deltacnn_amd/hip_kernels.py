@@ -163,6 +163,29 @@ def sparse_conv_activation(x, filter, mask, bias, prev_out, truncated, threshold
                       (prev_out, truncated, float(threshold), int(activation), int(truncation_mode)))
 
 
+def sparse_conv_add(x, packed_filter, mask, bias, residual, mask_residual, geometry, out, out_mask,
+                    weight_residual=1.0, weight_conv=1.0):
+    """``sparse_add_tensors(residual, sparse_conv(x))`` in the convolution's launch, for
+    pointwise fp16 convolutions with a packed filter.  Returns ``None`` (nothing launched) when
+    the shape has no fused form, so the caller can issue the two separate calls."""
+    lib = _lib.load()
+    _nhwc(x, "x")
+    _nhwc(residual, "residual")
+    if packed_filter is None or x.dtype != torch.float16:
+        return None
+    args = (geometry, x.data_ptr(), packed_filter.data_ptr(), _ptr(bias), _mask(mask, "mask").data_ptr(),
+            residual.data_ptr(), _mask(mask_residual, "mask_residual").data_ptr(), out.data_ptr(),
+            out_mask.data_ptr(), float(weight_residual), float(weight_conv), DC_F16, _stream())
+    meta = dict(g=geometry, esize=2, in_mask=mask, in_mask_b=mask_residual, out_mask=out_mask, mfma=True)
+    try:
+        _call("conv_add", lib.dc_conv_add, args, **meta)
+    except _lib.DeltaCNNError as e:
+        if e.code == -3:
+            return None
+        raise
+    return out, out_mask
+
+
 def sparse_deconv(x, filter, mask=None, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
                   groups=1, c_out: int = None, create_out_mask=False, sub_tile_sparsity=True,
                   out_mask=None, out_shape=None, *, packed_filter=None, out=None, geometry=None):

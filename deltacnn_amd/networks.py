@@ -184,9 +184,13 @@ class _InvertedResidual(nn.Module):
         self.conv = nn.Sequential(*layers)
 
     def forward(self, x):
-        if self.use_res_connect:
+        if not self.use_res_connect:
+            return self.conv(x)
+        fused = getattr(self.sparse_add, "after_conv", None)
+        if fused is None or len(self.conv[-1]) != 1:
             return self.sparse_add(x, self.conv(x))
-        return self.conv(x)
+        # the layer namespace can add the residual inside the last convolution's kernel
+        return fused(x, self.conv[-1][0], self.conv[:-1](x))
 
 
 MOBILENET_V2_SETTING = [  # t, c, n, s  (example/mobilenet_deltacnn.py:160-170)

@@ -367,6 +367,7 @@ class DCConvTranspose2d(_DeltaConvBase, nn.ConvTranspose2d, DCModule):
 class DCAdd(DCModule):
     """Sum of two delta tensors with union mask (sparse_layers.py:1086-1182)."""
     idx = -1
+    fuse_into_conv = True
 
     def __init__(self, activation: str = None, dense_out=False, weight_a=None, weight_b=None, name=""):
         super().__init__()
@@ -410,6 +411,32 @@ class DCAdd(DCModule):
         if self.dense_out:
             return out
         return out, mask_out
+
+    def after_conv(self, a, conv, conv_input):
+        """``self(a, conv(conv_input))`` with the addition fused into the convolution's kernel
+        when that is possible (pointwise fp16 convolution without activation, this layer without
+        activation / dense_out); otherwise exactly the two separate layer calls."""
+        fusable = (DCAdd.fuse_into_conv and type(a) != Tensor and self.activation is None
+                   and not self.dense_out and isinstance(conv, DCConv2d) and conv.activation is None
+                   and not conv.dense_out and conv.backend == DCBackend.deltacnn
+                   and conv.frame_idx >= 0 and type(conv_input) != Tensor)
+        if fusable:
+            # conv.frame_idx >= 0: the convolution has seen its first frame, no bias from here on
+            val_a, mask_a = a
+            x, mask, plan, packed, _, _ = conv._prepare(conv_input)
+            g = plan["g"]
+            if packed is not None and tuple(val_a.shape) == (g.batch, g.out_c, g.out_h, g.out_w):
+                if self.out is None or self.out.shape != val_a.shape or self.out.dtype != val_a.dtype:
+                    self.out = torch.empty_like(val_a)
+                if self.mask_out is None or self.mask_out.shape != mask_a.shape:
+                    self.mask_out = torch.empty_like(mask_a)
+                res = hk.sparse_conv_add(x, packed, mask, None, val_a, mask_a, plan["g"], self.out,
+                                         self.mask_out, self.weight_a, self.weight_b)
+                if res is not None:
+                    DCConv2d.conv_idx += 1
+                    conv.frame_idx += 1
+                    return res
+        return self(a, conv(conv_input))
 
     def reset(self):
         super().reset()

@@ -9,6 +9,7 @@ m = 4-byte mask word, P pixels, n_x = number of active pixels of mask x):
   densify            R = P*m + n*2*C*s                    W = n*C*s
   add                R = 2*P*m + (n_a+n_b)*C*s [+n_out*C*s]  W = n_out*C*s [+n_out*C*s] + P*m
   conv / deconv      R = P_in*m + n_in*Cin*s + K*K*(Cin/g)*Cout*s   W = n_out*Cout*s + P_out*m
+                     (conv_act: the same; conv_add: + P_out*m + n_res*Cout*s for the residual)
                      flops = 2*(Cin/g)*Cout*N_pairs, N_pairs = sum over updated outputs of the
                      active inputs in their window (computed exactly from the masks)
   pool               R = P_in*m + n_in*C*s (x2 for max)   W = n_out*C*s + P_out*m
@@ -40,7 +41,7 @@ class Tracer:
         rec = {"op": op, "meta": meta}
         rec["n_in"] = self._count(meta.get("in_mask"))
         rec["n_in_b"] = self._count(meta.get("in_mask_b"))
-        if self.count_pairs and op in ("conv", "deconv", "conv_act"):
+        if self.count_pairs and op in ("conv", "deconv", "conv_act", "conv_add"):
             rec["pairs"] = self._pairs(meta["g"], meta["in_mask"], op == "deconv")
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
@@ -77,12 +78,14 @@ class Tracer:
             n_out = None if r["n_out"] is None else int(r["n_out"])
             s, m = meta["esize"], 4
             flops = 0
-            if op in ("conv", "deconv", "conv_act"):
+            if op in ("conv", "deconv", "conv_act", "conv_add"):
                 g = meta["g"]
                 p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
                 wbytes = g.kernel_h * g.kernel_w * (g.in_c // g.groups) * g.out_c * s
                 rd = p_in * m + n_in * g.in_c * s + wbytes
                 wr = n_out * g.out_c * s + p_out * m
+                if op == "conv_add":  # + the residual operand of the fused add
+                    rd += p_out * m + n_in_b * g.out_c * s
                 if "pairs" in r:
                     flops = 2 * (g.in_c // g.groups) * g.out_c * int(r["pairs"])
                 dw = g.groups > 1

@@ -99,6 +99,18 @@ int dc_conv_act(const dc_geometry *g, const void *input, const void *filter,
                 int32_t *out_mask, void *prev_out, void *truncated, float threshold,
                 int activation, int truncation_mode, int dtype, void *stream);
 
+/* Fused pointwise conv + residual add: the DCAdd (sparse_layers.py:1086-1182, no activation, not
+ * dense_out) that follows a bottleneck's last 1x1 convolution, in the convolution's launch:
+ * out = weight_residual * residual [mask_residual] + weight_conv * conv(input) [mask], out_mask =
+ * mask | mask_residual.  Results are identical to dc_conv followed by dc_add(residual, conv).  No
+ * counterpart in the reference.  fp16, 1x1, stride 1, no padding, groups 1, Cin % 8 == 0,
+ * Cout % 4 == 0 and a packed filter are required; anything else returns DC_ERR_UNSUPPORTED
+ * before any launch so that the caller can issue the two separate calls. */
+int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filter,
+                const void *bias, const int32_t *mask, const void *residual,
+                const int32_t *mask_residual, void *out, int32_t *out_mask, float weight_residual,
+                float weight_conv, int dtype, void *stream);
+
 /* Number of bytes dc_pack_filter writes for this geometry (0 if the shape has no packed
  * form).  One-time weight relayout for the MFMA kernels: [Cout pad 16][Kh][Kw][Cin pad 32]
  * fp16, un-swizzled. */

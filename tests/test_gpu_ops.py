@@ -391,6 +391,39 @@ def test_conv_activation_fused(lib, dtype, cfg, act, mode):
     assert_masked_equal(out2, out1.cpu(), om1.cpu(), "out")
 
 
+@pytest.mark.parametrize("cfg", [(96, 24, 56, 56), (144, 32, 28, 28), (384, 64, 14, 14), (960, 160, 7, 7),
+                                 (32, 20, 9, 9)], ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("weights", [(1.0, 1.0), (0.5, -1.5)])
+def test_conv_add_fused(lib, cfg, weights):
+    """dc_conv_add == DCAdd(residual, conv(x)) of the oracle, and bit-identical to the two
+    separate library calls."""
+    from deltacnn_amd.hip_kernels import conv_geometry
+    Cin, Cout, H, W = cfg
+    dtype = torch.float16
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, (Cin, Cout, 1, 1, 0, 1, 1, H, W), 91, 0.3)
+    g = _gen(92)
+    mres = rand_mask(g, 2, H, W, 0.3)
+    res = torch.randn(2, Cout, H, W, generator=g).to(dtype)
+    want_conv, want_cm = ops.conv(x, mask, wt, None, s, p, d, groups)
+    want, want_mask = ops.add(res, mres, want_conv, want_cm, None, weights[0], weights[1], 0, False)
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, Cin, Cout, 1)
+    dx, dm, dres, dmres = cl(poison(x, mask)), cl(mask), cl(poison(res, mres)), cl(mres)
+    geo = conv_geometry(x.shape, K, Cout, s, p, d, 1)
+    out = torch.full((2, Cout, H, W), float("nan"), dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+    om = torch.full((2, 1, H, W), -5, dtype=torch.int32, device=DEV)
+    got = hk().sparse_conv_add(dx, pk, dm, None, dres, dmres, geo, out, om, weights[0], weights[1])
+    assert got is not None
+    assert torch.equal(om.cpu(), want_mask)
+    assert_masked_close(out, want, want_mask, 0, 2e-2, "out")
+    c_out, c_mask = hk().sparse_conv(dx, d_filt, dm, None, s, p, d, 1, c_out=Cout, create_out_mask=True, packed_filter=pk)
+    two = torch.empty_like(out)
+    two_mask = torch.empty_like(om)
+    hk().sparse_add_tensors(dres, c_out, None, two, dmres, c_mask, two_mask, weights[0], weights[1], 0, False)
+    assert torch.equal(two_mask, om)
+    assert_masked_equal(out, two.cpu(), want_mask, "fused vs two calls")
+
+
 # --------------------------------------------------------------------------------- pooling
 POOLS = [
     # C, K, stride, padding, dilation, H, W
