@@ -1,8 +1,15 @@
 """Whole-frame HIP graph capture for the delta path.
 
-At batch 1 a frame is ~100 kernels of a few microseconds each, so host launch cost dominates.
-All shapes of a DeltaCNN frame are static (sparsity only changes what kernels do inside), so
-the launches of one frame can be recorded once and replayed with a single graph launch.
+At batch 1 a frame is ~70 kernels of about two microseconds each, so host launch cost
+dominates eager execution.  All shapes of a DeltaCNN frame are static (sparsity only changes
+what kernels do inside), so the launches of one frame are recorded once and replayed with a
+single graph launch.
+
+An ordinary stream operation between two graph launches (for example copying the next frame
+into the graph's input buffer) stalls the replay pipeline for far longer than the copy itself
+takes.  :class:`VideoGraph` therefore keeps the frame fetch inside the graph: the clip lives
+in device memory and a device-side counter selects the frame, so a replay needs no other
+stream work at all.  :class:`FrameGraph` is the general form (one frame handed over per call).
 """
 from __future__ import annotations
 
@@ -31,5 +38,38 @@ class FrameGraph:
     @torch.no_grad()
     def __call__(self, frame: torch.Tensor):
         self.static_in.copy_(frame)
+        self.graph.replay()
+        return self.static_out
+
+
+class VideoGraph:
+    """Replay ``model(frames[t])`` for t = start, start + 1, ... with the frame fetch inside
+    the graph.
+
+    ``frames`` is a device tensor ``[T, C, H, W]`` whose frames are NHWC in memory
+    (``torch.channels_last``).  Every :meth:`step` processes the next frame; the caller must
+    not step past the end of the clip.  ``model`` may be any callable on a ``[1, C, H, W]``
+    tensor (the delta model after its first frame, or a dense model).
+    """
+
+    def __init__(self, model, frames: torch.Tensor, start: int = 0):
+        if not frames.is_contiguous(memory_format=torch.channels_last):
+            raise ValueError("frames must be channels_last")
+        t, c, h, w = frames.shape
+        self.length = t
+        self._rows = frames.permute(0, 2, 3, 1).reshape(t, h * w * c)  # a view: NHWC rows
+        self.index = torch.full((1,), start, dtype=torch.int64, device=frames.device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(self.graph):
+            row = self._rows.index_select(0, self.index)
+            frame = row.view(1, h, w, c).permute(0, 3, 1, 2)
+            self.static_out = model(frame)
+            self.index.add_(1)
+
+    def seek(self, t: int) -> None:
+        self.index.fill_(t)
+
+    @torch.no_grad()
+    def step(self):
         self.graph.replay()
         return self.static_out

@@ -49,8 +49,58 @@ class Tracer:
         end.record()
         rec["events"] = (start, end)
         rec["n_out"] = self._count(meta.get("out_mask"))
+        rec["call"] = (fn, args)
         self.records.append(rec)
         return rc
+
+    IN_PLACE = ("activate_truncate", "mul_add")
+
+    def replay_times(self, repeats: int = 20, rounds: int = 5, alt_inputs=None):
+        """Device time per call of every recorded call, free of host and event overhead: the
+        call is captured `repeats` times back to back into a HIP graph (each launch depends on
+        the previous one, as inside a frame) and the graph is replayed `rounds` times between
+        two events.  Returns microseconds per call, one per record.
+
+        Every call has to see the masks of the traced frame, so
+          * records are replayed last to first: a replay only disturbs its own outputs, whose
+            consumers have been timed already;
+          * an operator that works in place is replayed behind its producer (which restores the
+            incoming delta and mask each time) and the producer's own time is subtracted;
+          * sparsify alternates between the frames in `alt_inputs` (device pointers), else
+            its second replay would find an unchanged frame and an empty mask."""
+        stream = torch.cuda.Stream()
+
+        def timed(calls):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                cs = torch.cuda.current_stream().cuda_stream
+                for r in range(repeats):
+                    for op, fn, args in calls:
+                        a = list(args[:-1]) + [cs]
+                        if op == "sparsify" and alt_inputs:
+                            a[0] = alt_inputs[r % len(alt_inputs)]
+                        fn(*a)
+            g.replay()
+            torch.cuda.synchronize()
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(rounds):
+                g.replay()
+            end.record()
+            end.synchronize()
+            return 1e3 * start.elapsed_time(end) / (rounds * repeats)
+
+        times = [0.0] * len(self.records)
+        for i in range(len(self.records) - 1, -1, -1):
+            rec = self.records[i]
+            call = (rec["op"],) + rec["call"]
+            if rec["op"] in self.IN_PLACE and i > 0:
+                prev = self.records[i - 1]
+                pcall = (prev["op"],) + prev["call"]
+                times[i] = max(timed([pcall, call]) - timed([pcall]), 0.0)
+            else:
+                times[i] = timed([call])
+        return times
 
     @staticmethod
     def _pairs(g, mask, transposed):
@@ -134,7 +184,7 @@ class Tracer:
                 else:  # mul_add
                     rd, wr = P * m + n_in * C * s + C * s, n_in * C * s
                     dens = (n_in / P, n_in / P)
-            out.append({"kernel": name, "shape": shape, "ms": r["events"][0].elapsed_time(r["events"][1]),
+            out.append({"kernel": name, "shape": shape, "ms": r.get("ms", r["events"][0].elapsed_time(r["events"][1])),
                         "bytes": rd + wr, "flops": flops, "density_in": dens[0], "density_out": dens[1]})
         self.records = []
         return out

@@ -143,3 +143,26 @@ def test_frame_graph_replay_matches_eager(lib):
             got = fg(frames[t:t + 1]).clone()
             torch.cuda.synchronize()
             assert torch.equal(got, want), f"frame {t}: max diff {float((got - want).abs().max())}"
+
+
+def test_video_graph_matches_eager(lib):
+    """The graph that fetches its frame from a device-resident clip (no stream work between
+    replays) gives the eager model's result on every frame."""
+    from deltacnn_amd.graph import VideoGraph
+    from deltacnn_amd.video import moving_rectangles_video
+    video = moving_rectangles_video(frames=12, height=64, width=64, n_rect=2, min_size=8, max_size=20)
+    state = _calibrated_state(video[:4])
+    _, _, eager = _models(_mobilenet, torch.float16, 0.05, state)
+    _, _, graphed = _models(_mobilenet, torch.float16, 0.05, state)
+    frames = cl(video.half())
+    with torch.no_grad():
+        for m in (eager, graphed):
+            m(frames[0:1])
+            m(frames[1:2])
+        vg = VideoGraph(graphed, frames, start=2)
+        for t in range(2, video.shape[0]):
+            want = eager(frames[t:t + 1]).clone()
+            torch.cuda.synchronize()
+            got = vg.step().clone()
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), f"frame {t}: max diff {float((got - want).abs().max())}"
