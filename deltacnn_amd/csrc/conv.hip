@@ -5,7 +5,7 @@
 //      output mask), writes it, and the active output pixels of the tile are compacted with
 //      ballot + popcount rank; a tile without active pixels ends here;
 //   2. only the compacted pixels are computed.  Inactive or out-of-bounds inputs contribute
-//      zero by selection (their memory is never read).
+//      zero by selection (what a speculative load returns for them is discarded).
 //
 // conv_direct_kernel  any dtype / kernel / stride / dilation / groups, VALU, fp32 accumulate
 // conv_mfma_kernel    fp16, groups == 1, Cin % 8 == 0: implicit GEMM on

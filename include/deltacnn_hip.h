@@ -11,9 +11,11 @@
  *   - the library never allocates, frees or retains memory; pointers are borrowed
  *     for the duration of the asynchronous launch on `stream` (a hipStream_t, NULL =
  *     default stream); no entry point synchronises
- *   - values of inactive pixels are never read; outputs are written only for pixels
- *     whose output mask is 1 (the reference additionally writes the inactive pixels
- *     of partially active tiles, conv_kernel.cu:348-356; nothing downstream reads them)
+ *   - values of inactive pixels never influence any output (they may hold anything,
+ *     NaN included; a kernel may load them speculatively, always inside the tensor,
+ *     and discards them); outputs are written only for pixels whose output mask is 1
+ *     (the reference additionally writes the inactive pixels of partially active
+ *     tiles, conv_kernel.cu:348-356; nothing downstream reads them)
  *   - return value: DC_OK or a negative dc_status; dc_last_error() gives the message
  *     of the calling thread's last failure.  All argument checks run before the first
  *     HIP call, so they can be exercised without a GPU.
@@ -90,10 +92,12 @@ int dc_conv(const dc_geometry *g, const void *input, const void *filter,
             const void *packed_filter, const void *bias, void *out, const int32_t *mask,
             int32_t *out_mask, int dtype, void *stream);
 
-/* Fused conv + activation/truncation epilogue: dc_conv followed by dc_activate_truncate on
- * the conv output, in one launch where one workgroup owns all output channels of its
- * pixels.  No counterpart in the reference (it launches the two kernels separately,
- * sparse_layers.py:636-638); results are identical to the two-call sequence. */
+/* Conv + activation/truncation in one call: dc_conv followed by dc_activate_truncate on the
+ * conv output.  Depthwise, few-input-channel and large-map pointwise shapes run as ONE launch
+ * (the epilogue works on the accumulators, the conv output never travels through memory);
+ * every other shape runs the two kernels back to back inside the call.  No counterpart in
+ * the reference (it launches the two kernels separately, sparse_layers.py:636-638); results
+ * are identical to the two-call sequence bit for bit. */
 int dc_conv_act(const dc_geometry *g, const void *input, const void *filter,
                 const void *packed_filter, const void *bias, void *out, const int32_t *mask,
                 int32_t *out_mask, void *prev_out, void *truncated, float threshold,

@@ -1,0 +1,149 @@
+"""Host-side checks of the C-ABI library that need no GPU: it loads, exports every entry point
+the public header declares, rejects bad arguments with the documented codes before touching
+the device, and the Python shim refuses to run without it (there is no CPU fallback)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "deltacnn_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    return sorted(set(re.findall(r"\b(dc_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_declares_the_operator_set():
+    names = declared_symbols()
+    for op in ("sparsify", "activate_truncate", "conv", "deconv", "pool", "add", "add_to_dense",
+               "upsample", "concat", "mul_add", "version", "last_error"):
+        assert f"dc_{op}" in names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    raw = ctypes.CDLL(lib._name)
+    for name in declared_symbols():
+        assert hasattr(raw, name), f"{name} is declared in the header but not exported"
+
+
+def test_python_bindings_cover_the_header(lib):
+    from deltacnn_amd import _lib
+    assert sorted(_lib._SIGNATURES) == declared_symbols()
+
+
+def test_version_and_error_string(lib):
+    assert b"gfx950" in lib.dc_version()
+    assert isinstance(lib.dc_last_error(), bytes)
+
+
+def _geom(**kw):
+    from deltacnn_amd._lib import Geometry
+    base = dict(batch=1, in_h=8, in_w=8, in_c=16, out_h=8, out_w=8, out_c=16, kernel_h=3, kernel_w=3,
+                stride_h=1, stride_w=1, dilation_h=1, dilation_w=1, pad_top=1, pad_left=1, pad_bottom=1,
+                pad_right=1, groups=1)
+    base.update(kw)
+    return Geometry(**base)
+
+
+def test_bad_arguments_are_rejected_before_any_launch(lib):
+    """Error codes: -1 dtype, -2 shape, -3 unsupported, -4 null, -5 alignment."""
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    assert lib.dc_sparsify(p, p, p, p, 0.1, 16, 4, 7, None) == -1
+    assert b"dtype" in lib.dc_last_error()
+    assert lib.dc_sparsify(None, p, p, p, 0.1, 16, 4, 0, None) == -4
+    assert lib.dc_sparsify(p, p, p, p, 0.1, 0, 4, 0, None) == -2
+    assert lib.dc_sparsify(p, p, p, p, 0.1, 16, -1, 0, None) == -2
+    assert lib.dc_activate_truncate(p, p, None, p, 0.1, 1, 0, 16, 4, 0, None) == -4   # truncation needs its cache
+    assert lib.dc_activate_truncate(p, p, p, p, 0.1, 9, 0, 16, 4, 0, None) == -3      # unknown activation
+    # geometry: output size that does not follow from the input size
+    g = _geom(out_h=7)
+    assert lib.dc_conv(ctypes.byref(g), p, p, None, None, p, p, p, 0, None) == -2
+    assert b"expected 8x8" in lib.dc_last_error()
+    g = _geom(groups=3)
+    assert lib.dc_conv(ctypes.byref(g), p, p, None, None, p, p, p, 0, None) == -2
+    g = _geom()
+    assert lib.dc_conv(ctypes.byref(g), None, p, None, None, p, p, p, 0, None) == -4
+    assert lib.dc_conv(None, p, p, None, None, p, p, p, 0, None) == -4
+    # transposed convolution with asymmetric padding is not defined
+    g = _geom(kernel_h=4, kernel_w=4, stride_h=2, stride_w=2, pad_bottom=2, out_h=15, out_w=16)
+    assert lib.dc_deconv(ctypes.byref(g), p, p, None, None, p, p, p, 0, None) == -3
+    # pooling keeps the channel count
+    g = _geom(out_c=8)
+    assert lib.dc_pool(ctypes.byref(g), p, p, p, p, p, 0, 0, None) == -2
+
+
+def test_packed_filter_size_is_host_arithmetic(lib):
+    """fp16, groups 1: [Cout padded to 16][taps][Cin padded to 32] halves; no packed form for
+    fp32 or grouped convolutions (0)."""
+    g = _geom(in_c=24, out_c=40)
+    assert lib.dc_packed_filter_bytes(ctypes.byref(g), 1, 0) == 48 * 9 * 32 * 2
+    assert lib.dc_packed_filter_bytes(ctypes.byref(g), 0, 0) == 0
+    g = _geom(groups=16)
+    assert lib.dc_packed_filter_bytes(ctypes.byref(g), 1, 0) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from deltacnn_amd import _lib
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libdeltacnn_hip.so"))
+    monkeypatch.setattr(_lib, "_lib", None)
+    with pytest.raises(ImportError):
+        _lib.load()
+
+
+def test_package_does_not_import_the_oracle():
+    """The oracle is test infrastructure: nothing under deltacnn_amd/ may import it."""
+    pkg = os.path.join(ROOT, "deltacnn_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith(".py"):
+                src = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", src, flags=re.M), f
+
+
+@pytest.mark.parametrize("k,s,p,d", [(3, 1, 1, 1), (3, 2, 1, 1), (1, 1, 0, 1), (5, 2, 2, 1), (3, 1, 2, 2), (7, 2, 3, 1)])
+def test_conv_geometry_matches_torch(k, s, p, d):
+    from deltacnn_amd.hip_kernels import conv_geometry
+    x = torch.zeros(2, 4, 23, 17)
+    want = torch.nn.functional.conv2d(x, torch.zeros(6, 4, k, k), stride=s, padding=p, dilation=d).shape
+    g = conv_geometry(x.shape, (k, k), 6, (s, s), (p, p), (d, d), 1)
+    assert (g.batch, g.out_c, g.out_h, g.out_w) == tuple(want)
+    # transposed: the reference formula has no output_padding term
+    gt = conv_geometry(x.shape, (4, 4), 6, (2, 2), (1, 1), (1, 1), 1, True)
+    want = torch.nn.functional.conv_transpose2d(x, torch.zeros(4, 6, 4, 4), stride=2, padding=1).shape
+    assert (gt.out_h, gt.out_w) == tuple(want[2:])
+
+
+def test_filter_layouts():
+    """fp32: W_dc[ci,ky,kx,co] = W[co,ci,ky,kx] (transposed: W[ci,co,ky,kx]).  fp16: channels
+    padded to even, W[ci,co] stored at row ci ^ (co & 1) -- written out as the four cases of the
+    2x2 pair swizzle of filter_conversion.py:34-37."""
+    from deltacnn_amd.filter_conversion import (convert_filter_out_channels_last, convert_half_filter,
+                                                 restore_half_filter)
+    g = torch.Generator().manual_seed(1)
+    w = torch.randn(5, 7, 3, 3, generator=g)   # Cout=5, Cin=7
+    f = convert_filter_out_channels_last(w)
+    assert f.shape == (7, 3, 3, 5) and f.is_contiguous()
+    assert float(f[2, 1, 0, 4]) == float(w[4, 2, 1, 0])
+    ft = convert_filter_out_channels_last(w, transposed=True)
+    assert ft.shape == (5, 3, 3, 7) and float(ft[4, 1, 0, 2]) == float(w[4, 2, 1, 0])
+    h = convert_half_filter(w)
+    assert h.shape == (8, 3, 3, 6) and h.dtype == torch.float16
+    wh = w.half()
+    W = torch.zeros(8, 3, 3, 6, dtype=torch.float16)
+    W[:7, :, :, :5] = wh.permute(1, 2, 3, 0)
+    for i in range(4):
+        for j in range(3):
+            assert torch.equal(h[2 * i, :, :, 2 * j], W[2 * i, :, :, 2 * j])
+            assert torch.equal(h[2 * i, :, :, 2 * j + 1], W[2 * i + 1, :, :, 2 * j + 1])
+            assert torch.equal(h[2 * i + 1, :, :, 2 * j], W[2 * i + 1, :, :, 2 * j])
+            assert torch.equal(h[2 * i + 1, :, :, 2 * j + 1], W[2 * i, :, :, 2 * j + 1])
+    assert torch.equal(restore_half_filter(h, 7, 5), wh.permute(1, 2, 3, 0))
+    dw = torch.randn(6, 1, 3, 3, generator=g)
+    assert convert_half_filter(dw, pixel_wise=True).shape == (1, 3, 3, 6)
