@@ -13,9 +13,9 @@
 // kernel accumulate a given output element with the same instruction sequence, so they agree
 // bit for bit).
 //
-// pw_mfma_kernel      convolution only; a workgroup takes 64 pixels x 64 channels, or with
-//                     KSPLIT 64 pixels x 16 channels with the reduction split over its four
-//                     wavefronts (deep layers: long reduction, few pixels)
+// pw_mfma_kernel      convolution only (optionally + residual add); the arrangement of a
+//                     workgroup's wavefronts over reduction slices, channel tiles and pixel
+//                     tiles is a template parameter set chosen per layer by the host
 // pw_act_mfma_kernel  convolution + activation/truncation in one launch: a workgroup owns ALL
 //                     output channels of its 16 pixels, so it can take the per-pixel keep/drop
 //                     decision itself; the convolution output never travels through memory.
@@ -27,16 +27,10 @@
 namespace dc {
 namespace {
 
-__device__ __forceinline__ half8_t zero8() { return half8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
-
 struct PwP {
     int P, Ci, Co, ci_p, co_tiles;
 };
 
-// S = reduction steps per memory round trip (chunk): all fragment loads of S steps are in
-// flight together; the host picks the smallest S in {1, 2, 4, 8} that covers a wavefront's
-// share of the reduction, so most layers finish in a single chunk.
-//
 // ADD fuses the residual sum of a DCAdd layer behind the convolution: with a = residual delta
 // (mask Ma) and b = convolution output rounded to fp16 (mask Mb = input mask),
 // out = fma(b, wb, a * wa) on pixels of Ma | Mb, each term present only where its mask is set --
@@ -47,136 +41,188 @@ struct ResP {
     float wa, wb;
 };
 
-template <bool KSPLIT, int S, bool ADD>
-__global__ void __launch_bounds__(256)
+// A workgroup takes 64 consecutive pixels (4 pixel tiles of 16) x CBW * R channel tiles of 16.
+// Its KW * CBW * NBW wavefronts are arranged as
+//   KW  slices of the reduction (wavefront kw takes steps kw, kw + KW, ...; the partial sums
+//       meet in LDS and are added in ascending kw, so the result does not depend on timing),
+//   CBW groups of R channel tiles,
+//   NBW groups of NTW pixel tiles (NBW * NTW == 4),
+// so a wavefront accumulates R x NTW tiles and needs R filter + NTW input fragments per
+// reduction step.  The host picks the arrangement per layer: many pixels and few channels
+// favour NBW > 1, few pixels and a long reduction favour KW > 1 with R > 1 (the input
+// fragments are then shared by R channel tiles instead of being fetched again by other
+// workgroups).  S = reduction steps per memory round trip: all fragment loads of S steps are in
+// flight together.
+template <int KW, int CBW, int NBW, int R, int NTW, int S, bool ADD, bool EAGER>
+__global__ void __launch_bounds__(KW * CBW * NBW * WAVE)
 pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                const half_t *__restrict__ bias, half_t *__restrict__ out,
                const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, ResP rp) {
-    constexpr int NT = 4;
-    __shared__ float4_t s_red[KSPLIT ? 4 * NT * WAVE : 1];
+    static_assert(NBW * NTW <= 4, "a workgroup covers at most 64 pixels");
+    constexpr int NW = KW * CBW * NBW, TILES = R * NTW, FT = (TILES + KW - 1) / KW;
+    constexpr int PXW = NBW * NTW * 16;  // pixels per workgroup
+    __shared__ float4_t s_red[KW > 1 ? NW * TILES * WAVE : 1];
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;
-    const int cb = blockIdx.y;
-    const int ct_raw = KSPLIT ? cb : cb * 4 + wave;
-    const int ct = min(ct_raw, p.co_tiles - 1);  // surplus wavefronts compute a tile nobody stores
-    const int kvalid = kq * 8;
+    const int kw = wave % KW, tw = wave / KW, cw = tw % CBW, nw = tw / CBW;
     const int ksteps = p.ci_p >> 5;
-    const int first = KSPLIT ? wave : 0, stride = KSPLIT ? 4 : 1;
-    const half_t *wrow = wp + (size_t)(ct * 16 + l16) * p.ci_p + kvalid;
+    const int pbase = blockIdx.x * PXW;
 
-    int px[NT];
-    bool on[NT], on_r[NT];
+    // the mask words of the workgroup's pixels, one per lane, together with the first chunk
+    // of filter fragments (which do not depend on the masks)
+    const int mp = pbase + lane;
+    const bool mine = lane < PXW && mp < p.P;
+    const int mword = mask[min(mp, p.P - 1)];
+    int rword = 0;
+    if (ADD) rword = rp.mask[min(mp, p.P - 1)];
+    const int ct0 = (blockIdx.y * CBW + cw) * R;
+    const half_t *wrow[R];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        px[nt] = blockIdx.x * 64 + nt * 16 + l16;
-        const int m = mask[min(px[nt], p.P - 1)];
-        on[nt] = px[nt] < p.P && m != 0;
-        on_r[nt] = false;
-        if (ADD) on_r[nt] = px[nt] < p.P && rp.mask[min(px[nt], p.P - 1)] != 0;
-    }
-    // first chunk of filter fragments travels together with the mask words
-    half8_t a[S];
+    for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
+        wrow[r] = wp + (size_t)(min(ct0 + r, p.co_tiles - 1) * 16 + l16) * p.ci_p + kq * 8;
+    half8_t a[S][R];
 #pragma unroll
     for (int i = 0; i < S; ++i) {
-        const int s = min(first + i * stride, ksteps - 1);
-        a[i] = *reinterpret_cast<const half8_t *>(wrow + (s << 5));
-    }
-    bool nt_on[NT];
-    bool any = false;
+        const int s = min(kw + i * KW, ksteps - 1);
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        nt_on[nt] = ballot(on[nt]) != 0;
-        any |= ballot(on[nt] || on_r[nt]) != 0;
+        for (int r = 0; r < R; ++r) a[i][r] = *reinterpret_cast<const half8_t *>(wrow[r] + (s << 5));
     }
-    if (cb == 0 && wave == 0 && kq == 0) {
+    // EAGER: the input fragments of the first chunk are requested before the masks are known
+    // (one memory round trip less in the dependency chain; what inactive pixels return is
+    // never stored)
+    const half_t *xrow[NTW];
+    half8_t x[S][NTW];
+    if (EAGER) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-            if (px[nt] < p.P) out_mask[px[nt]] = (on[nt] || on_r[nt]) ? 1 : 0;
+        for (int j = 0; j < NTW; ++j)
+            xrow[j] = in + (size_t)min(pbase + (nw * NTW + j) * 16 + l16, p.P - 1) * p.Ci;
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            const int s = min(kw + i * KW, ksteps - 1);
+            const int k = min((s << 5) + kq * 8, p.Ci - 8);
+#pragma unroll
+            for (int j = 0; j < NTW; ++j) x[i][j] = *reinterpret_cast<const half8_t *>(xrow[j] + k);
+        }
     }
-    if (!any) return;
-    const int co = ct * 16 + kq * 4;  // Cout % 4 == 0: a lane's 4 channels are all in or all out
-    half4_t res[NT];
-    if (ADD) {
+    const uint64_t bm = ballot(mine && mword != 0);
+    const uint64_t br = ADD ? ballot(mine && rword != 0) : 0;
+    const uint64_t bo = bm | br;
+    if (blockIdx.y == 0 && wave == 0 && mine) out_mask[mp] = int((bo >> lane) & 1);
+    if (bo == 0) return;  // the same for every wavefront of the workgroup
+
+    // tiles this wavefront finishes: all of its own (KW == 1) or tiles kw, kw + KW, ... of
+    // its group after the reduction
+    half4_t res[FT], bh[FT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-            res[nt] = *reinterpret_cast<const half4_t *>(
-                rp.res + (size_t)(on_r[nt] ? px[nt] : 0) * p.Co + min(co, p.Co - 4));
+    for (int m = 0; m < FT; ++m) {
+        const int t = KW > 1 ? kw + m * KW : m;
+        const int r = t / NTW, j = t % NTW;
+        const int co = min((ct0 + r) * 16 + kq * 4, p.Co - 4);
+        bh[m] = half4_t{0, 0, 0, 0};
+        if (bias != nullptr) bh[m] = *reinterpret_cast<const half4_t *>(bias + co);
+        if (ADD) {
+            const int bit = (nw * NTW + j) * 16 + l16;
+            const bool on_r = t < TILES && ((br >> bit) & 1);
+            res[m] = *reinterpret_cast<const half4_t *>(rp.res + (size_t)(on_r ? pbase + bit : 0) * p.Co + co);
+        }
     }
 
-    float4_t acc[NT];
+    float4_t acc[R][NTW];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) acc[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
-    const half_t *xrow[NT];
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-        xrow[nt] = in + (size_t)(on[nt] ? px[nt] : 0) * p.Ci;
+        for (int j = 0; j < NTW; ++j) acc[r][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    bool nt_on[NTW];
+    bool wave_on = false;
+#pragma unroll
+    for (int j = 0; j < NTW; ++j) {
+        const int bit = (nw * NTW + j) * 16;
+        nt_on[j] = ((bm >> bit) & 0xffffu) != 0;
+        wave_on |= nt_on[j];
+        // inactive pixels all point at pixel 0, so their (discarded) loads share one cache line
+        if (!EAGER) xrow[j] = in + (size_t)(((bm >> (bit + l16)) & 1) ? pbase + bit + l16 : 0) * p.Ci;
+    }
 
-    for (int s0 = first; s0 < ksteps; s0 += S * stride) {
-        if (s0 != first) {
+    if (wave_on) {
+        for (int s0 = kw; s0 < ksteps; s0 += S * KW) {
+            if (s0 != kw) {
+#pragma unroll
+                for (int i = 0; i < S; ++i) {
+                    const int s = min(s0 + i * KW, ksteps - 1);
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        a[i][r] = *reinterpret_cast<const half8_t *>(wrow[r] + (s << 5));
+                }
+            }
+            if (!EAGER || s0 != kw) {
+#pragma unroll
+                for (int i = 0; i < S; ++i) {
+                    const int s = min(s0 + i * KW, ksteps - 1);
+                    const int k = min((s << 5) + kq * 8, p.Ci - 8);
+#pragma unroll
+                    for (int j = 0; j < NTW; ++j) x[i][j] = *reinterpret_cast<const half8_t *>(xrow[j] + k);
+                }
+            }
+            // No zero-fill is needed: columns of inactive pixels are never stored, and where a
+            // step reaches past Cin the packed filter holds zeros while the clamped address
+            // re-reads finite values of the same pixel.
 #pragma unroll
             for (int i = 0; i < S; ++i) {
-                const int s = min(s0 + i * stride, ksteps - 1);
-                a[i] = *reinterpret_cast<const half8_t *>(wrow + (s << 5));
-            }
-        }
-        // inactive pixels all point at pixel 0, so their (discarded) loads share one cache line
-        half8_t x[S][NT];
+                if (s0 + i * KW < ksteps) {  // wave-uniform
 #pragma unroll
-        for (int i = 0; i < S; ++i) {
-            const int s = min(s0 + i * stride, ksteps - 1);
-            const int k = min((s << 5) + kvalid, p.Ci - 8);
+                    for (int j = 0; j < NTW; ++j)
+                        if (nt_on[j]) {  // wave-uniform
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-                x[i][nt] = *reinterpret_cast<const half8_t *>(xrow[nt] + k);
-        }
-        // No zero-fill is needed: columns of inactive pixels are never stored, and where a step
-        // reaches past Cin the packed filter holds zeros while the clamped address re-reads
-        // finite values of the same pixel.
-#pragma unroll
-        for (int i = 0; i < S; ++i) {
-            if (s0 + i * stride < ksteps) {  // wave-uniform
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    if (nt_on[nt])  // wave-uniform
-                        acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], x[i][nt], acc[nt], 0, 0, 0);
+                            for (int r = 0; r < R; ++r)
+                                acc[r][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][r], x[i][j], acc[r][j], 0, 0, 0);
+                        }
+                }
             }
         }
     }
 
-    if (KSPLIT) {
+    float4_t fin[FT];
+    if (KW > 1) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) s_red[(wave * NT + nt) * WAVE + lane] = acc[nt];
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < NTW; ++j) s_red[(wave * TILES + r * NTW + j) * WAVE + lane] = acc[r][j];
         __syncthreads();
-        // wavefront w finishes pixel sub-tile w
-        float4_t sum = s_red[(0 * NT + wave) * WAVE + lane];
 #pragma unroll
-        for (int w = 1; w < 4; ++w) sum += s_red[(w * NT + wave) * WAVE + lane];
+        for (int m = 0; m < FT; ++m) {
+            const int t = min(kw + m * KW, TILES - 1);
+            float4_t sum = s_red[((tw * KW) * TILES + t) * WAVE + lane];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-            if (nt == wave) acc[nt] = sum;
+            for (int q = 1; q < KW; ++q) sum += s_red[((tw * KW + q) * TILES + t) * WAVE + lane];
+            fin[m] = sum;
+        }
+    } else {
+#pragma unroll
+        for (int m = 0; m < FT; ++m) fin[m] = acc[m / NTW][m % NTW];
     }
-    if (ct_raw >= p.co_tiles) return;
-    if (co >= p.Co) return;
-    float4_t bv = {0.f, 0.f, 0.f, 0.f};
-    if (bias != nullptr) {
-        const half4_t b = *reinterpret_cast<const half4_t *>(bias + co);
-        bv = float4_t{float(b[0]), float(b[1]), float(b[2]), float(b[3])};
-    }
+
     const half_t wa = half_t(rp.wa), wb = half_t(rp.wb);
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        if (!(on[nt] || on_r[nt]) || (KSPLIT && nt != wave)) continue;
-        const float4_t r = acc[nt] + bv;
-        half4_t o = half4_t{half_t(r[0]), half_t(r[1]), half_t(r[2]), half_t(r[3])};
+    for (int m = 0; m < FT; ++m) {
+        const int t = KW > 1 ? kw + m * KW : m;
+        if (t >= TILES) continue;
+        const int r = t / NTW, j = t % NTW;
+        const int ct = ct0 + r, co = ct * 16 + kq * 4;  // Cout % 4 == 0: a lane's 4 channels are all in or all out
+        if (ct >= p.co_tiles || co >= p.Co) continue;
+        const int bit = (nw * NTW + j) * 16 + l16;
+        const bool on = (bm >> bit) & 1, on_r = (br >> bit) & 1;
+        if (!(on || on_r)) continue;
+        const float4_t v = fin[m] + float4_t{float(bh[m][0]), float(bh[m][1]), float(bh[m][2]), float(bh[m][3])};
+        half4_t o = half4_t{half_t(v[0]), half_t(v[1]), half_t(v[2]), half_t(v[3])};
         if (ADD) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                half_t sum = on_r[nt] ? half_t(res[nt][i] * wa) : half_t(0);
-                if (on[nt]) sum = fma_t(o[i], wb, sum);
+                half_t sum = on_r ? half_t(res[m][i] * wa) : half_t(0);
+                if (on) sum = fma_t(o[i], wb, sum);
                 o[i] = sum;
             }
         }
-        *reinterpret_cast<half4_t *>(out + (size_t)px[nt] * p.Co + co) = o;
+        *reinterpret_cast<half4_t *>(out + (size_t)(pbase + bit) * p.Co + co) = o;
     }
 }
 
@@ -389,10 +435,25 @@ bool pointwise_eligible(const dc_geometry &g, int dtype) {
            g.pad_left == 0 && g.pad_bottom == 0 && g.pad_right == 0;
 }
 
-// Reduction steps above which the convolution-only kernel splits the reduction over the
-// wavefronts of a workgroup.  The fused kernel only takes much shorter reductions, so a layer
-// gets the same summation order with and without the fused epilogue.
-constexpr int PW_KSPLIT_STEPS = 10;
+// Wavefront arrangements of pw_mfma_kernel in use: id, KW, CBW, NBW, R, NTW, EAGER.
+// Measured on MI355X over MobileNetV2's layers and 64x64x256 maps: small problems are bound by
+// the dependent-latency chain and by how many compute units take part, so they run one
+// 16x16 output tile per workgroup (ids 0, 2, 3: reduction over 1, 4 or 8 wavefronts) with eager
+// input loads; large problems are bound by fragment traffic and reuse fragments in registers
+// (ids 4, 5).
+#define DC_PW_CONFIGS(X)                                                                     \
+    X(0, 1, 1, 1, 1, 1, true) X(1, 1, 2, 2, 1, 1, true) X(2, 4, 1, 1, 1, 1, true)             \
+    X(3, 8, 1, 1, 1, 1, true) X(4, 1, 2, 1, 2, 4, false) X(5, 4, 1, 1, 4, 4, false)
+
+// The fused kernel only takes reductions of at most 3 steps, and every arrangement chosen
+// for a reduction of up to 4 steps has KW == 1, so a layer gets the same summation order with
+// and without the fused epilogue.
+int pick_config(const PwP &p, int ksteps) {
+    const int64_t tiles = (int64_t)ceil_div(p.P, 16) * p.co_tiles;
+    if (tiles >= 4096 && ksteps >= 2 && p.co_tiles >= 4) return ksteps >= 5 ? 5 : 4;
+    if (ksteps <= 4) return (ksteps <= 2 && p.P >= 4096 && p.co_tiles >= 2) ? 1 : 0;
+    return ksteps <= 24 ? 2 : 3;
+}
 
 hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *packed,
                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
@@ -438,28 +499,35 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
         }
 #undef DC_GO
     }
-    const bool ksplit = ksteps > PW_KSPLIT_STEPS;
-    dim3 grid(ceil_div(p.P, 64), ksplit ? p.co_tiles : ceil_div(p.co_tiles, 4));
-    const int per_wave = ksplit ? ceil_div(ksteps, 4) : ksteps;
     ResP rp{nullptr, nullptr, 1.f, 1.f};
     if (res != nullptr) rp = ResP{(const half_t *)res->values, res->mask, res->wa, res->wb};
-#define DC_PW(KS, SS)                                                                                \
+    const int cfg = pick_config(p, ksteps);
+#define DC_PW_S(KW, CBW, NBW, R, NTW, EA, SS)                                                        \
     do {                                                                                             \
+        dim3 grid(ceil_div(p.P, NBW * NTW * 16), ceil_div(p.co_tiles, CBW * R));                     \
         if (res != nullptr)                                                                          \
-            pw_mfma_kernel<KS, SS, true><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
+            pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, true, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(  \
+                p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
         else                                                                                         \
-            pw_mfma_kernel<KS, SS, false><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
+            pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, false, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>( \
+                p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
     } while (0)
-    if (ksplit) {
-        if (per_wave <= 4) DC_PW(true, 4); else DC_PW(true, 8);
-    } else {
-        if (per_wave <= 1) DC_PW(false, 1);
-        else if (per_wave <= 2) DC_PW(false, 2);
-        else if (per_wave <= 4) DC_PW(false, 4);
-        else DC_PW(false, 8);
+#define DC_PW(ID, KW, CBW, NBW, R, NTW, EA)                                                          \
+    case ID: {                                                                                       \
+        const int need = ceil_div(ksteps, KW);                                                       \
+        if (need <= 1) DC_PW_S(KW, CBW, NBW, R, NTW, EA, 1);                                         \
+        else if (need <= 2) DC_PW_S(KW, CBW, NBW, R, NTW, EA, 2);                                    \
+        else DC_PW_S(KW, CBW, NBW, R, NTW, EA, 4);                                                   \
+        break;                                                                                       \
+    }
+    switch (cfg) {
+        DC_PW_CONFIGS(DC_PW)
+        default: return hipErrorInvalidValue;
     }
 #undef DC_PW
+#undef DC_PW_S
     return hipGetLastError();
 }
 
 }  // namespace dc
+
