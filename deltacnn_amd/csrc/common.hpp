@@ -99,6 +99,12 @@ __device__ __forceinline__ half_t tabs(half_t x) { return __builtin_fabsf16(x); 
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Workgroup size of the one-group-per-pixel kernels.  A launch of up to 2048 wavefronts runs
+// one wavefront per workgroup so that it spreads over as many compute units as possible (these
+// launches are bound by latency and by the load issue rate of a compute unit, not by
+// occupancy); larger launches use 256 threads.
+inline int group_block(int64_t threads) { return threads <= 2048 * WAVE ? WAVE : 256; }
 inline int pow2_ceil(int v) {
     int p = 1;
     while (p < v) p <<= 1;

@@ -101,7 +101,10 @@ struct EpiP {
     int mode;
 };
 
-template <typename T, int ITERS, int ACT, bool K3>
+// EAGER (3x3 only, small maps): the nine input rows, the filter and the cached state are
+// requested before the mask words have arrived -- their addresses depend on coordinates only --
+// so the whole kernel is one memory round trip; what is loaded for inactive pixels is dropped.
+template <typename T, int ITERS, int ACT, bool K3, bool EAGER>
 __global__ void __launch_bounds__(256)
 conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
                const T *__restrict__ bias, T *__restrict__ out, const int32_t *__restrict__ mask,
@@ -121,6 +124,35 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
     const int glo = lane_id() & ~(G - 1);
     const uint64_t gmask = G >= WAVE ? ~0ull : ((1ull << G) - 1ull);
 
+    Vec<T, N> ex[K3 && EAGER ? 9 : 1][ITERS], ew[K3 && EAGER ? 9 : 1][ITERS], q[ITERS], tr[ITERS];
+    if (K3 && EAGER) {
+        const int pc = valid ? po : 0;
+        const int cb = pc / (p.Ho * p.Wo), cr = pc - cb * p.Ho * p.Wo;
+        const int cy = cr / p.Wo, cx = cr - cy * p.Wo;
+        const T *inb = in + (size_t)cb * p.Hi * p.Wi * C;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const int ky = t / 3, kx = t - ky * 3;
+            const int iy = min(max(cy * p.sh - p.pt + ky * p.dh, 0), p.Hi - 1);
+            const int ix = min(max(cx * p.sw - p.pl + kx * p.dw, 0), p.Wi - 1);
+            const T *xr = inb + (size_t)(iy * p.Wi + ix) * C;
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int c = min((it * G + gl) * N, C - N);
+                ex[t][it] = vload<T, N>(xr + c);
+                ew[t][it] = vload<T, N>(filter + (size_t)t * C + c);
+            }
+        }
+        if (ACT >= 0) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int c = min((it * G + gl) * N, C - N);
+                q[it] = vload<T, N>((const T *)epi.prev + (size_t)pc * C + c);
+                tr[it] = vload<T, N>((const T *)epi.trunc + (size_t)pc * C + c);
+            }
+        }
+    }
+
     uint64_t taps = 0;
     for (int j = 0; j < K2; j += G) {
         const int t = j + gl;
@@ -137,8 +169,7 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
     if (ballot(active) == 0) return;
 
     // cached state of the epilogue: requested now so that it arrives while the taps are summed
-    Vec<T, N> q[ITERS], tr[ITERS];
-    if (ACT >= 0)
+    if (ACT >= 0 && !(K3 && EAGER))
         load_state<T, ITERS>(q, tr, active, (size_t)po, gl, G, C, (const T *)epi.prev,
                              (const T *)epi.trunc);
 
@@ -149,7 +180,19 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
         for (int j = 0; j < N; ++j) acc[it][j] = 0.f;
     if (active) {
         const T *inb = in + (size_t)b * p.Hi * p.Wi * C;
-        if (K3 && ITERS <= 2) {
+        if (K3 && EAGER) {
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                const bool on = (taps >> t) & 1ull;
+#pragma unroll
+                for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+                    for (int j = 0; j < N; ++j) {
+                        const float xv = on ? float(ex[t][it].v[j]) : 0.f;
+                        acc[it][j] = __builtin_fmaf(xv, float(ew[t][it].v[j]), acc[it][j]);
+                    }
+            }
+        } else if (K3 && ITERS <= 2) {
             // 3x3: every tap is loaded unconditionally from a clamped (always valid) address
             // and zeroed afterwards if the tap is inactive, so all loads are in flight
             // together: one memory round trip instead of one per tap
@@ -368,8 +411,8 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    const half_t *wrow = wp + (size_t)(ct * 16 + l16) * K2 * ci_p + kq * 8;
     const int ksteps = ci_p >> 5;
+    const half_t *wfrag = wp + (size_t)ct * K2 * ksteps * 512 + lane * 8;  // fragment order, see pack_filter_kernel
     const int total = K2 * ksteps;
     const int kvalid = kq * 8;  // this lane's channel offset inside a 32-wide step
     const int first = KSPLIT ? wave : 0, stride = KSPLIT ? 4 : 1;
@@ -416,7 +459,7 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
                 }
                 use[i] = tap_used;
                 if (tap_used) {
-                    a[i] = *reinterpret_cast<const half8_t *>(wrow + (size_t)tap * ci_p + k0);
+                    a[i] = *reinterpret_cast<const half8_t *>(wfrag + ((size_t)tap * ksteps + (k0 >> 5)) * 512);
                     const bool kin = k0 + kvalid < p.Ci;
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) {
@@ -481,15 +524,24 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 }
 
 // One-time relayout of a reference-layout fp16 filter [Cin pad 2][K][K][Cout pad 2] (channel
-// pairs swizzled: W[ci][co] is stored at row ci ^ (co & 1)) into [Cout pad 16][K][K][Cin pad 32].
+// pairs swizzled: W[ci][co] is stored at row ci ^ (co & 1)) into MFMA fragment order
+// [Cout tile of 16][tap][Cin step of 32][lane 0..63][8]: lane (kq * 16 + r) of a fragment holds
+// input channels kq * 8 .. + 8 of output channel r, so one A operand of
+// v_mfma_f32_16x16x32_f16 is a single contiguous 1 KB read (16 bytes per lane, consecutive
+// lanes at consecutive addresses).  Channels past Cin / Cout are zero.
 __global__ void pack_filter_kernel(const half_t *__restrict__ f, half_t *__restrict__ wp, int Ci,
                                    int Co, int K2, int w_co, int ci_p, int co_p) {
     const size_t total = (size_t)co_p * K2 * ci_p;
+    const int ksteps = ci_p >> 5;
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total;
          i += (size_t)gridDim.x * blockDim.x) {
-        int ci = int(i % ci_p);
-        int tap = int((i / ci_p) % K2);
-        int co = int(i / ((size_t)ci_p * K2));
+        const int e = int(i & 7), lane = int((i >> 3) & 63);
+        const size_t frag = i >> 9;
+        const int step = int(frag % ksteps);
+        const int tap = int((frag / ksteps) % K2);
+        const int ct = int(frag / ((size_t)ksteps * K2));
+        const int co = ct * 16 + (lane & 15);
+        const int ci = step * 32 + (lane >> 4) * 8 + e;
         half_t v = half_t(0);
         if (ci < Ci && co < Co) v = f[((size_t)(ci ^ (co & 1)) * K2 + tap) * w_co + co];
         wp[i] = v;
@@ -541,12 +593,13 @@ hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *pa
 namespace {
 
 template <typename T, int ITERS>
-void dw_launch(dim3 grid, hipStream_t s, int act, const ConvP &p, const T *in, const T *filter,
+void dw_launch(dim3 grid, int block, bool eager, hipStream_t s, int act, const ConvP &p, const T *in, const T *filter,
                const T *bias, T *out, const int32_t *mask, int32_t *out_mask, EpiP e, int lg) {
 #define DC_DW(A) \
     do { \
-        if (p.Kh == 3 && p.Kw == 3) conv_dw_kernel<T, ITERS, A, true><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg); \
-        else conv_dw_kernel<T, ITERS, A, false><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg); \
+        if (p.Kh == 3 && p.Kw == 3 && eager) conv_dw_kernel<T, (ITERS > 2 ? 2 : ITERS), A, true, true><<<grid, block, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg); \
+        else if (p.Kh == 3 && p.Kw == 3) conv_dw_kernel<T, ITERS, A, true, false><<<grid, block, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg); \
+        else conv_dw_kernel<T, ITERS, A, false, false><<<grid, block, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg); \
     } while (0)
     switch (act) {
         case DC_ACT_LINEAR: DC_DW(DC_ACT_LINEAR); break;
@@ -575,15 +628,19 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
     const int nvec = g.in_c / N;
     const int G = pick_group(nvec, P_out, 4);
     const int iters = ceil_div(nvec, G);
-    dim3 grid((unsigned)ceil_div64(P_out * G, 256));
+    const int block = group_block(P_out * G);
+    dim3 grid((unsigned)ceil_div64(P_out * G, block));
     EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f,
            epi ? epi->mode : 0};
     const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
     const int lg = log2i(G);
+    // eager loads where reading nine rows for every pixel, active or not, costs little: maps
+    // of up to 2 MB of input, and at most two vectors per lane (register budget)
+    const bool eager = iters <= 2 && (int64_t)g.batch * g.in_h * g.in_w * g.in_c * (int64_t)sizeof(T) <= (2 << 20);
     switch (iters) {
-        case 1: dw_launch<T, 1>(grid, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
-        case 2: dw_launch<T, 2>(grid, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
-        default: dw_launch<T, 4>(grid, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
+        case 1: dw_launch<T, 1>(grid, block, eager, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
+        case 2: dw_launch<T, 2>(grid, block, eager, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
+        default: dw_launch<T, 4>(grid, block, false, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
     }
     return true;
 }
@@ -600,12 +657,13 @@ bool try_fewcin(const dc_geometry &g, const ConvP &p, const T *in, const T *filt
     if (epi && (!al(epi->prev) || (epi->trunc && !al(epi->trunc)) || epi->mode < 0)) return false;
     const int64_t P_out = (int64_t)g.batch * g.out_h * g.out_w;
     const int G = group_lanes(g.out_c / N, 1);
-    dim3 grid((unsigned)ceil_div64(P_out * G, 256));
+    const int block = group_block(P_out * G);
+    dim3 grid((unsigned)ceil_div64(P_out * G, block));
     EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f,
            epi ? epi->mode : 0};
     const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
     const int lg = log2i(G);
-#define DC_FC(A) conv_fewcin_kernel<T, A><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg)
+#define DC_FC(A) conv_fewcin_kernel<T, A><<<grid, block, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg)
     switch (act) {
         case DC_ACT_LINEAR: DC_FC(DC_ACT_LINEAR); break;
         case DC_ACT_RELU: DC_FC(DC_ACT_RELU); break;

@@ -99,7 +99,10 @@ sparsify_gen_kernel(const T *__restrict__ in, T *__restrict__ prev, T *__restric
 }
 
 // ----------------------------------------------------------------- activation + truncation
-template <typename T, int ITERS, int ACT>
+// EAGER (small maps): delta, cached state and mask word are requested together -- their
+// addresses depend on coordinates only -- so the kernel is one memory round trip; what is
+// loaded for inactive pixels is dropped.
+template <typename T, int ITERS, int ACT, bool EAGER>
 __global__ void __launch_bounds__(256)
 act_trunc_vec_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict__ trunc,
                      int32_t *__restrict__ mask, float thr_f, int mode, int P, int C, int lg) {
@@ -107,15 +110,27 @@ act_trunc_vec_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict_
     const int G = 1 << lg;
     int p, gl;
     group_coords(lg, p, gl);
-    const bool valid = p < P && mask[p] != 0;
-    if (ballot(valid) == 0) return;
     Vec<T, N> dl[ITERS], q[ITERS], tr[ITERS];
+    if (EAGER) {
+        const size_t row = (size_t)min(p, P - 1) * C;
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-        const int c = (it * G + gl) * N;
-        if (valid && c < C) dl[it] = vload<T, N>(delta + (size_t)p * C + c);
+        for (int it = 0; it < ITERS; ++it) {
+            const int c = min((it * G + gl) * N, C - N);
+            dl[it] = vload<T, N>(delta + row + c);
+            q[it] = vload<T, N>(prev + row + c);
+            tr[it] = vload<T, N>(trunc + row + c);
+        }
     }
-    load_state<T, ITERS>(q, tr, valid, (size_t)p, gl, G, C, prev, trunc);
+    const bool valid = p < P && mask[min(p, P - 1)] != 0;
+    if (ballot(valid) == 0) return;
+    if (!EAGER) {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int c = (it * G + gl) * N;
+            if (valid && c < C) dl[it] = vload<T, N>(delta + (size_t)p * C + c);
+        }
+        load_state<T, ITERS>(q, tr, valid, (size_t)p, gl, G, C, prev, trunc);
+    }
     act_trunc_pixel<T, ITERS, ACT>(dl, q, tr, valid, (size_t)p, gl, G, C, delta, prev, trunc, mask,
                                    T(thr_f), mode);
 }
@@ -420,9 +435,10 @@ bool can_vec(int C, std::initializer_list<const void *> ptrs) {
 
 // Launch shape for one group of G lanes per pixel.
 struct GroupLaunch {
-    int lg;
+    int lg, block;
     dim3 grid;
-    GroupLaunch(int64_t pixels, int G) : lg(log2i(G)), grid((unsigned)ceil_div64(pixels * G, 256)) {}
+    GroupLaunch(int64_t pixels, int G)
+        : lg(log2i(G)), block(group_block(pixels * G)), grid((unsigned)ceil_div64(pixels * G, block)) {}
 };
 
 template <typename T>
@@ -435,22 +451,28 @@ hipError_t sparsify_t(const T *in, T *prev, T *delta, int32_t *mask, float thr, 
         int iters = ceil_div(nvec, G);
         GroupLaunch L(P, G);
         switch (iters) {
-            case 1: sparsify_vec_kernel<T, 1><<<L.grid, 256, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
-            case 2: sparsify_vec_kernel<T, 2><<<L.grid, 256, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
-            default: sparsify_vec_kernel<T, 4><<<L.grid, 256, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
+            case 1: sparsify_vec_kernel<T, 1><<<L.grid, L.block, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
+            case 2: sparsify_vec_kernel<T, 2><<<L.grid, L.block, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
+            default: sparsify_vec_kernel<T, 4><<<L.grid, L.block, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
         }
     } else {
         int G = group_lanes(C, 4);
         GroupLaunch L(P, G);
-        sparsify_gen_kernel<T><<<L.grid, 256, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge);
+        sparsify_gen_kernel<T><<<L.grid, L.block, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge);
     }
     return hipGetLastError();
 }
 
 template <typename T, int ITERS>
-void act_trunc_launch(dim3 grid, hipStream_t s, T *delta, T *prev, T *trunc, int32_t *mask,
+void act_trunc_launch(dim3 grid, int block, hipStream_t s, T *delta, T *prev, T *trunc, int32_t *mask,
                       float thr, int act, int mode, int P, int C, int lg) {
-#define DC_AT(A) act_trunc_vec_kernel<T, ITERS, A><<<grid, 256, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, lg)
+    // eager loads where reading the whole map, active or not, costs little
+    const bool eager = (int64_t)P * C * (int64_t)sizeof(T) <= (1 << 20);
+#define DC_AT(A)                                                                                                    \
+    do {                                                                                                            \
+        if (eager) act_trunc_vec_kernel<T, ITERS, A, true><<<grid, block, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, lg); \
+        else act_trunc_vec_kernel<T, ITERS, A, false><<<grid, block, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, lg);      \
+    } while (0)
     switch (act) {
         case DC_ACT_RELU: DC_AT(DC_ACT_RELU); break;
         case DC_ACT_RELU6: DC_AT(DC_ACT_RELU6); break;
@@ -470,10 +492,10 @@ hipError_t act_trunc_t(T *delta, T *prev, T *trunc, int32_t *mask, float thr, in
     if (mode < 0) {
         if (can_vec<T>(C, {delta, prev})) {
             GroupLaunch L(P, pick_group(C / N, P, 4));
-            accumulate_kernel<T, N><<<L.grid, 256, 0, s>>>(delta, prev, mask, act, P, C, L.lg);
+            accumulate_kernel<T, N><<<L.grid, L.block, 0, s>>>(delta, prev, mask, act, P, C, L.lg);
         } else {
             GroupLaunch L(P, group_lanes(C, 1));
-            accumulate_kernel<T, 1><<<L.grid, 256, 0, s>>>(delta, prev, mask, act, P, C, L.lg);
+            accumulate_kernel<T, 1><<<L.grid, L.block, 0, s>>>(delta, prev, mask, act, P, C, L.lg);
         }
         return hipGetLastError();
     }
@@ -483,13 +505,13 @@ hipError_t act_trunc_t(T *delta, T *prev, T *trunc, int32_t *mask, float thr, in
         int iters = ceil_div(nvec, G);
         GroupLaunch L(P, G);
         switch (iters) {
-            case 1: act_trunc_launch<T, 1>(L.grid, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;
-            case 2: act_trunc_launch<T, 2>(L.grid, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;
-            default: act_trunc_launch<T, 4>(L.grid, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;
+            case 1: act_trunc_launch<T, 1>(L.grid, L.block, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;
+            case 2: act_trunc_launch<T, 2>(L.grid, L.block, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;
+            default: act_trunc_launch<T, 4>(L.grid, L.block, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;
         }
     } else {
         GroupLaunch L(P, group_lanes(C, 1));
-        act_trunc_gen_kernel<T><<<L.grid, 256, 0, s>>>(delta, prev, trunc, mask, thr, act, mode, P, C, L.lg);
+        act_trunc_gen_kernel<T><<<L.grid, L.block, 0, s>>>(delta, prev, trunc, mask, thr, act, mode, P, C, L.lg);
     }
     return hipGetLastError();
 }
@@ -503,11 +525,11 @@ hipError_t add_t(const T *a, const T *b, T *prev, T *out, const int32_t *ma, con
     const bool vec = can_vec<T>(C, {a, b, prev, out});
     GroupLaunch L(P, vec ? pick_group(C / N, P, 4) : group_lanes(C, 1));
     if (dense_out) {
-        if (vec) add_dense_kernel<T, N><<<L.grid, 256, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, L.lg);
-        else add_dense_kernel<T, 1><<<L.grid, 256, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, L.lg);
+        if (vec) add_dense_kernel<T, N><<<L.grid, L.block, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, L.lg);
+        else add_dense_kernel<T, 1><<<L.grid, L.block, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, L.lg);
     } else {
-        if (vec) add_kernel<T, N><<<L.grid, 256, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, L.lg);
-        else add_kernel<T, 1><<<L.grid, 256, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, L.lg);
+        if (vec) add_kernel<T, N><<<L.grid, L.block, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, L.lg);
+        else add_kernel<T, 1><<<L.grid, L.block, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, L.lg);
     }
     return hipGetLastError();
 }
@@ -545,11 +567,11 @@ hipError_t add_to_dense_t(T *a, T *b, const int32_t *ma, int act, int P, int C, 
     const bool vec = can_vec<T>(C, {a, b});
     GroupLaunch L(P, vec ? pick_group(C / N, P, 4) : group_lanes(C, 1));
     if (act > 0) {
-        if (vec) add_to_dense_act_kernel<T, N><<<L.grid, 256, 0, s>>>(a, b, ma, act, P, C, L.lg);
-        else add_to_dense_act_kernel<T, 1><<<L.grid, 256, 0, s>>>(a, b, ma, act, P, C, L.lg);
+        if (vec) add_to_dense_act_kernel<T, N><<<L.grid, L.block, 0, s>>>(a, b, ma, act, P, C, L.lg);
+        else add_to_dense_act_kernel<T, 1><<<L.grid, L.block, 0, s>>>(a, b, ma, act, P, C, L.lg);
     } else {
-        if (vec) add_to_dense_kernel<T, N><<<L.grid, 256, 0, s>>>(a, b, ma, P, C, L.lg);
-        else add_to_dense_kernel<T, 1><<<L.grid, 256, 0, s>>>(a, b, ma, P, C, L.lg);
+        if (vec) add_to_dense_kernel<T, N><<<L.grid, L.block, 0, s>>>(a, b, ma, P, C, L.lg);
+        else add_to_dense_kernel<T, 1><<<L.grid, L.block, 0, s>>>(a, b, ma, P, C, L.lg);
     }
     return hipGetLastError();
 }
@@ -560,10 +582,10 @@ hipError_t upsample_t(const T *in, T *out, const int32_t *mi, int32_t *mo, int B
     int P = B * H * W;
     if (can_vec<T>(C, {in, out})) {
         GroupLaunch L(P, pick_group(C / N, P, 4));
-        upsample_kernel<T, N><<<L.grid, 256, 0, s>>>(in, out, mi, mo, B, H, W, C, S, L.lg);
+        upsample_kernel<T, N><<<L.grid, L.block, 0, s>>>(in, out, mi, mo, B, H, W, C, S, L.lg);
     } else {
         GroupLaunch L(P, group_lanes(C, 1));
-        upsample_kernel<T, 1><<<L.grid, 256, 0, s>>>(in, out, mi, mo, B, H, W, C, S, L.lg);
+        upsample_kernel<T, 1><<<L.grid, L.block, 0, s>>>(in, out, mi, mo, B, H, W, C, S, L.lg);
     }
     return hipGetLastError();
 }
@@ -574,10 +596,10 @@ hipError_t concat_t(const T *a, const T *b, T *out, const int32_t *ma, const int
     int Cm = Ca > Cb ? Ca : Cb;
     if (Ca % N == 0 && Cb % N == 0 && can_vec<T>(Ca, {a, b, out})) {
         GroupLaunch L(P, pick_group(Cm / N, P, 4));
-        concat_kernel<T, N><<<L.grid, 256, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, L.lg);
+        concat_kernel<T, N><<<L.grid, L.block, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, L.lg);
     } else {
         GroupLaunch L(P, group_lanes(Cm, 1));
-        concat_kernel<T, 1><<<L.grid, 256, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, L.lg);
+        concat_kernel<T, 1><<<L.grid, L.block, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, L.lg);
     }
     return hipGetLastError();
 }
@@ -587,10 +609,10 @@ hipError_t mul_add_t(const T *in, const int32_t *mask, T *out, int32_t *mo, cons
     constexpr int N = Vec16<T>::N;
     if (can_vec<T>(C, {in, out, scale, bias})) {
         GroupLaunch L(P, pick_group(C / N, P, 4));
-        mul_add_kernel<T, N><<<L.grid, 256, 0, s>>>(in, mask, out, mo, scale, bias, P, C, L.lg);
+        mul_add_kernel<T, N><<<L.grid, L.block, 0, s>>>(in, mask, out, mo, scale, bias, P, C, L.lg);
     } else {
         GroupLaunch L(P, group_lanes(C, 1));
-        mul_add_kernel<T, 1><<<L.grid, 256, 0, s>>>(in, mask, out, mo, scale, bias, P, C, L.lg);
+        mul_add_kernel<T, 1><<<L.grid, L.block, 0, s>>>(in, mask, out, mo, scale, bias, P, C, L.lg);
     }
     return hipGetLastError();
 }

@@ -8,7 +8,7 @@
 // not depend on the masks -- are requested together with the mask words.
 //
 // Operand roles as in the generic kernel: rows = 16 output channels from the packed filter
-// [Cout pad 16][Cin pad 32], columns = 16 pixels (NHWC rows), fp32 accumulate, reduction in
+// (fragment order, one contiguous KB per channel tile and step), columns = 16 pixels (NHWC rows), fp32 accumulate, reduction in
 // steps of 32 input channels taken in ascending order (both kernels below and the generic
 // kernel accumulate a given output element with the same instruction sequence, so they agree
 // bit for bit).
@@ -76,16 +76,16 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
     int rword = 0;
     if (ADD) rword = rp.mask[min(mp, p.P - 1)];
     const int ct0 = (blockIdx.y * CBW + cw) * R;
-    const half_t *wrow[R];
+    const half_t *wrow[R];  // fragment order: one contiguous KB per (channel tile, step)
 #pragma unroll
     for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
-        wrow[r] = wp + (size_t)(min(ct0 + r, p.co_tiles - 1) * 16 + l16) * p.ci_p + kq * 8;
+        wrow[r] = wp + (size_t)min(ct0 + r, p.co_tiles - 1) * ksteps * 512 + lane * 8;
     half8_t a[S][R];
 #pragma unroll
     for (int i = 0; i < S; ++i) {
         const int s = min(kw + i * KW, ksteps - 1);
 #pragma unroll
-        for (int r = 0; r < R; ++r) a[i][r] = *reinterpret_cast<const half8_t *>(wrow[r] + (s << 5));
+        for (int r = 0; r < R; ++r) a[i][r] = *reinterpret_cast<const half8_t *>(wrow[r] + (s << 9));
     }
     // EAGER: the input fragments of the first chunk are requested before the masks are known
     // (one memory round trip less in the dependency chain; what inactive pixels return is
@@ -151,7 +151,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
                     const int s = min(s0 + i * KW, ksteps - 1);
 #pragma unroll
                     for (int r = 0; r < R; ++r)
-                        a[i][r] = *reinterpret_cast<const half8_t *>(wrow[r] + (s << 5));
+                        a[i][r] = *reinterpret_cast<const half8_t *>(wrow[r] + (s << 9));
                 }
             }
             if (!EAGER || s0 != kw) {
@@ -237,7 +237,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
 template <int CTW, int ACT>
 __device__ __forceinline__ void pw_epilogue_stats(const float4_t (&acc)[CTW], const half4_t (&q)[CTW],
                                                   const half4_t (&tr)[CTW], half4_t (&v)[CTW],
-                                                  const half_t *__restrict__ bias, bool on, int wave,
+                                                  const half4_t (&bh)[CTW], bool on, int wave,
                                                   int NW, int kq, const PwP &p, half_t thr, bool &hit,
                                                   float &sq) {
 #pragma unroll
@@ -246,11 +246,7 @@ __device__ __forceinline__ void pw_epilogue_stats(const float4_t (&acc)[CTW], co
         if (ct >= p.co_tiles) break;  // wave-uniform: surplus tiles of the last wavefronts
         const int co = ct * 16 + kq * 4;
         const bool live = co < p.Co;
-        float4_t r = acc[j];
-        if (bias != nullptr && live) {
-            const half4_t b = *reinterpret_cast<const half4_t *>(bias + co);
-            r += float4_t{float(b[0]), float(b[1]), float(b[2]), float(b[3])};
-        }
+        const float4_t r = acc[j] + float4_t{float(bh[j][0]), float(bh[j][1]), float(bh[j][2]), float(bh[j][3])};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             v[j][i] = half_t(r[i]);
@@ -308,101 +304,103 @@ __device__ __forceinline__ void pw_epilogue_store(const half4_t (&q)[CTW], const
     }
 
 // Workgroup = NW wavefronts x 16 pixels x all output channels; wavefront w owns channel tiles
-// w, w + NW, ... (at most CTW of them).  KS bounds the reduction steps.  Every loop is fully
-// unrolled without branches (surplus steps multiply zero fragments, surplus tiles are computed
-// and dropped).  The filter fragments of a wavefront are requested in AB batches: the first
-// together with the mask words, the second together with the input fragments and the cached
-// state, so the kernel is two memory round trips, the MFMAs, one barrier and the stores.
-// Requires Cout % 4 == 0.
-template <int NW, int CTW, int KS, int AB>
+// w, w + NW, ... (at most CTW of them).  Everything whose address depends on coordinates only
+// -- mask words, the first two reduction steps of filter and input fragments, the cached state
+// and the bias of this lane's (pixel, 4 channel) cells -- is requested at once, so a layer with
+// a reduction of up to 64 input channels is one memory round trip, the MFMAs, one barrier and
+// the stores.  Longer reductions stream two steps per round trip in ascending order (the same
+// summation order as the convolution-only kernel without reduction split).  What is loaded
+// for inactive pixels is dropped.  Requires Cout % 4 == 0.
+template <int NW, int CTW, int ACT>
 __global__ void __launch_bounds__(NW * WAVE)
 pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                    const half_t *__restrict__ bias, half_t *__restrict__ out,
                    const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
-                   half_t *__restrict__ prev, half_t *__restrict__ trunc, float thr_f, int act,
-                   int mode) {
-    static_assert(CTW % AB == 0, "filter batches must divide the tiles of a wavefront");
-    constexpr int JB = CTW / AB;
+                   half_t *__restrict__ prev, half_t *__restrict__ trunc, float thr_f, int mode) {
+    constexpr int S = 2;
     __shared__ float s_stat[NW][16];
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;
-    const int kvalid = kq * 8;
     const int ksteps = p.ci_p >> 5;
     const int px = blockIdx.x * 16 + l16;
-    const int m = mask[min(px, p.P - 1)];
-    half8_t a[CTW][KS];
-    // round trip 1: mask word + first batch of filter fragments (they do not depend on the
-    // mask; a workgroup without active pixels wastes a few cached KB)
+    const int pxc = min(px, p.P - 1);
+    const int m = mask[pxc];
+    const half_t *wrow[CTW];
 #pragma unroll
-    for (int j = 0; j < JB; ++j) {
-        const int ct = min(wave + j * NW, p.co_tiles - 1);
-        const half_t *wrow = wp + (size_t)(ct * 16 + l16) * p.ci_p + kvalid;
+    for (int j = 0; j < CTW; ++j)
+        wrow[j] = wp + (size_t)min(wave + j * NW, p.co_tiles - 1) * ksteps * 512 + lane * 8;
+    const half_t *xrow = in + (size_t)pxc * p.Ci;
+    half8_t a[S][CTW], x[S];
 #pragma unroll
-        for (int s = 0; s < KS; ++s)
-            a[j][s] = *reinterpret_cast<const half8_t *>(wrow + (min(s, ksteps - 1) << 5));
+    for (int i = 0; i < S; ++i) {
+        const int s = min(i, ksteps - 1);
+        x[i] = *reinterpret_cast<const half8_t *>(xrow + min((s << 5) + kq * 8, p.Ci - 8));
+#pragma unroll
+        for (int j = 0; j < CTW; ++j) a[i][j] = *reinterpret_cast<const half8_t *>(wrow[j] + (s << 9));
+    }
+    half4_t q[CTW], tr[CTW], bh[CTW];
+#pragma unroll
+    for (int j = 0; j < CTW; ++j) {
+        const int co = min(min(wave + j * NW, p.co_tiles - 1) * 16 + kq * 4, p.Co - 4);
+        const size_t off = (size_t)pxc * p.Co + co;
+        q[j] = *reinterpret_cast<const half4_t *>(prev + off);
+        tr[j] = *reinterpret_cast<const half4_t *>(trunc + off);
+        bh[j] = half4_t{0, 0, 0, 0};
+        if (bias != nullptr) bh[j] = *reinterpret_cast<const half4_t *>(bias + co);
+    }
+    // all of the above is in flight before anything is waited for
+#pragma unroll
+    for (int i = 0; i < S; ++i) {
+        DC_PIN(x[i]);
+#pragma unroll
+        for (int j = 0; j < CTW; ++j) DC_PIN(a[i][j]);
     }
 #pragma unroll
-    for (int j = 0; j < JB; ++j)
-#pragma unroll
-        for (int s = 0; s < KS; ++s) DC_PIN(a[j][s]);
+    for (int j = 0; j < CTW; ++j) {
+        DC_PIN(q[j]);
+        DC_PIN(tr[j]);
+        DC_PIN(bh[j]);
+    }
     const bool on = px < p.P && m != 0;
     if (ballot(on) == 0) {  // same 16 pixels in every wavefront: the whole workgroup leaves
         if (wave == 0 && kq == 0 && px < p.P) out_mask[px] = 0;
         return;
     }
-    // round trip 2: remaining filter fragments, input fragments and cached state of this
-    // lane's (pixel, 4 channel) cells; inactive pixels all point at pixel 0, their loads share
-    // one cache line and are dropped
-#pragma unroll
-    for (int j = JB; j < CTW; ++j) {
-        const int ct = min(wave + j * NW, p.co_tiles - 1);
-        const half_t *wrow = wp + (size_t)(ct * 16 + l16) * p.ci_p + kvalid;
-#pragma unroll
-        for (int s = 0; s < KS; ++s)
-            a[j][s] = *reinterpret_cast<const half8_t *>(wrow + (min(s, ksteps - 1) << 5));
-    }
-    const half_t *xrow = in + (size_t)(on ? px : 0) * p.Ci;
-    half8_t x[KS];
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        const int k = (min(s, ksteps - 1) << 5) + kvalid;
-        x[s] = *reinterpret_cast<const half8_t *>(xrow + min(k, p.Ci - 8));
-    }
-    half4_t q[CTW], tr[CTW];
-#pragma unroll
-    for (int j = 0; j < CTW; ++j) {
-        const int ct = min(wave + j * NW, p.co_tiles - 1);
-        const int co = min(ct * 16 + kq * 4, p.Co - 4);
-        const size_t off = (size_t)(on ? px : 0) * p.Co + co;
-        q[j] = *reinterpret_cast<const half4_t *>(prev + off);
-        tr[j] = *reinterpret_cast<const half4_t *>(trunc + off);
-    }
-#pragma unroll
-    for (int j = JB; j < CTW; ++j)
-#pragma unroll
-        for (int s = 0; s < KS; ++s) DC_PIN(a[j][s]);
-#pragma unroll
-    for (int s = 0; s < KS; ++s) DC_PIN(x[s]);
-#pragma unroll
-    for (int j = 0; j < CTW; ++j) {
-        DC_PIN(q[j]);
-        DC_PIN(tr[j]);
-    }
     // no zero-fill: see pw_mfma_kernel (inactive columns are dropped, padded filter is zero)
     float4_t acc[CTW];
 #pragma unroll
-    for (int j = 0; j < CTW; ++j) {
-        acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < CTW; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < ksteps; s0 += S) {
+        if (s0 != 0) {
 #pragma unroll
-        for (int s = 0; s < KS; ++s)
-            if (s < ksteps)  // uniform
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j][s], x[s], acc[j], 0, 0, 0);
+            for (int i = 0; i < S; ++i) {
+                const int s = min(s0 + i, ksteps - 1);
+                x[i] = *reinterpret_cast<const half8_t *>(xrow + min((s << 5) + kq * 8, p.Ci - 8));
+#pragma unroll
+                for (int j = 0; j < CTW; ++j)
+                    a[i][j] = *reinterpret_cast<const half8_t *>(wrow[j] + (s << 9));
+            }
+#pragma unroll
+            for (int i = 0; i < S; ++i) {
+                DC_PIN(x[i]);
+#pragma unroll
+                for (int j = 0; j < CTW; ++j) DC_PIN(a[i][j]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            if (s0 + i < ksteps) {  // uniform
+#pragma unroll
+                for (int j = 0; j < CTW; ++j)
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][j], x[i], acc[j], 0, 0, 0);
+            }
+        }
     }
     const half_t thr = half_t(thr_f);
     half4_t v[CTW];
     bool hit = false;
     float sq = 0.f;
-    DC_ACT_SWITCH(act, (pw_epilogue_stats<CTW, A>(acc, q, tr, v, bias, on, wave, NW, kq, p, thr, hit, sq)));
+    pw_epilogue_stats<CTW, ACT>(acc, q, tr, v, bh, on, wave, NW, kq, p, thr, hit, sq);
     // per pixel: combine the four k-quarter lanes, then the wavefronts
     float stat;
     if (mode == DC_TRUNC_MAX) {
@@ -423,7 +421,7 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
     else keep = sqrtf(mode == DC_TRUNC_RMS ? tot / float(p.Co) : tot) > float(thr);
     if (wave == 0 && kq == 0 && px < p.P) out_mask[px] = (on && keep) ? 1 : 0;
     if (!on) return;
-    DC_ACT_SWITCH(act, (pw_epilogue_store<CTW, A>(q, tr, v, keep, wave, NW, kq, px, p, out, prev, trunc)));
+    pw_epilogue_store<CTW, ACT>(q, tr, v, keep, wave, NW, kq, px, p, out, prev, trunc);
 }
 
 }  // namespace
@@ -445,13 +443,15 @@ bool pointwise_eligible(const dc_geometry &g, int dtype) {
     X(0, 1, 1, 1, 1, 1, true) X(1, 1, 2, 2, 1, 1, true) X(2, 4, 1, 1, 1, 1, true)             \
     X(3, 8, 1, 1, 1, 1, true) X(4, 1, 2, 1, 2, 4, false) X(5, 4, 1, 1, 4, 4, false)
 
-// The fused kernel only takes reductions of at most 3 steps, and every arrangement chosen
-// for a reduction of up to 4 steps has KW == 1, so a layer gets the same summation order with
-// and without the fused epilogue.
+// The fused kernel takes reductions of at most PW_FUSED_MAX_STEPS steps in ascending order, and
+// every arrangement chosen here for such a reduction has KW == 1, so a layer gets the same
+// summation order with and without the fused epilogue.
+constexpr int PW_FUSED_MAX_STEPS = 10;
+
 int pick_config(const PwP &p, int ksteps) {
     const int64_t tiles = (int64_t)ceil_div(p.P, 16) * p.co_tiles;
-    if (tiles >= 4096 && ksteps >= 2 && p.co_tiles >= 4) return ksteps >= 5 ? 5 : 4;
-    if (ksteps <= 4) return (ksteps <= 2 && p.P >= 4096 && p.co_tiles >= 2) ? 1 : 0;
+    if (tiles >= 4096 && ksteps >= 2 && p.co_tiles >= 4) return ksteps > PW_FUSED_MAX_STEPS ? 5 : 4;
+    if (ksteps <= PW_FUSED_MAX_STEPS) return (ksteps <= 2 && p.P >= 4096 && p.co_tiles >= 2) ? 1 : 0;
     return ksteps <= 24 ? 2 : 3;
 }
 
@@ -468,35 +468,35 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     const int ksteps = p.ci_p / 32;
     *epilogue_done = false;
     const auto al8 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 7u) == 0; };
-    // Fused epilogue where a workgroup can own all output channels of 16 pixels cheaply: few
-    // channel tiles per wavefront and a short reduction, so that all filter fragments of a
-    // wavefront live in registers.
+    // Fused epilogue: a workgroup owns all output channels of its 16 pixels (up to 16
+    // wavefronts x 5 channel tiles), so it takes the keep / drop decision itself.  Only for maps
+    // of at least 512 pixels: a smaller map gives too few workgroups, the whole filter then
+    // streams through a handful of compute units and the two-launch form (channel tiles spread
+    // over many workgroups) is faster.
     const bool fusable = res == nullptr && epi != nullptr && epi->mode >= 0 && g.out_c % 4 == 0 && al8(epi->prev) &&
                          al8(epi->trunc) && al8(out);
-    if (fusable) {
+    if (fusable && ksteps <= PW_FUSED_MAX_STEPS && p.P >= 512) {
         dim3 grid(ceil_div(p.P, 16));
         const int act = epi->act < 0 ? 0 : epi->act;
-#define DC_GO(NW, CTW, KS, AB)                                                                       \
-    do {                                                                                             \
-        pw_act_mfma_kernel<NW, CTW, KS, AB><<<grid, NW * WAVE, 0, s>>>(                              \
-            p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, \
-            out_mask, (half_t *)epi->prev, (half_t *)epi->trunc, epi->thr, act, epi->mode);          \
-        *epilogue_done = true;                                                                       \
-        return hipGetLastError();                                                                    \
+        // as many wavefronts as channel tiles, up to 16; then several tiles per wavefront
+        const int nw = p.co_tiles <= 4 ? 4 : p.co_tiles <= 8 ? 8 : 16;
+        const int ctw = ceil_div(p.co_tiles, nw);
+#define DC_GO(NW, CTW)                                                                                \
+    do {                                                                                              \
+        DC_ACT_SWITCH(act, (pw_act_mfma_kernel<NW, CTW, A><<<grid, NW * WAVE, 0, s>>>(                \
+                               p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias,   \
+                               (half_t *)out, mask, out_mask, (half_t *)epi->prev,                    \
+                               (half_t *)epi->trunc, epi->thr, epi->mode)));                          \
+        *epilogue_done = true;                                                                        \
+        return hipGetLastError();                                                                     \
     } while (0)
-        // Only maps with enough pixels to occupy the GPU with 16-pixel workgroups: a wavefront
-        // issues one instruction per 4 cycles, so a small map handled by a few fat workgroups is
-        // slower than the two-launch form whose channel split spreads over many wavefronts.
-        if (p.P > 1024) {
-            const int ctw = ceil_div(p.co_tiles, 4);
-            if (ctw <= 2 && ksteps <= 1) DC_GO(4, 2, 1, 1);
-            if (ctw <= 3 && ksteps <= 1) DC_GO(4, 3, 1, 1);
-            if (ctw <= 4 && ksteps <= 1) DC_GO(4, 4, 1, 1);
-            if (ctw <= 2 && ksteps <= 3) DC_GO(4, 2, 3, 1);
-            if (ctw <= 4 && ksteps <= 3) DC_GO(4, 4, 3, 1);
-            if (ctw <= 8 && ksteps <= 1) DC_GO(4, 8, 1, 1);
-            if (ctw <= 8 && ksteps <= 2) DC_GO(4, 8, 2, 1);
-        }
+        if (nw == 4) DC_GO(4, 1);
+        if (nw == 8) DC_GO(8, 1);
+        if (ctw == 1) DC_GO(16, 1);
+        if (ctw == 2) DC_GO(16, 2);
+        if (ctw == 3) DC_GO(16, 3);
+        if (ctw == 4) DC_GO(16, 4);
+        if (ctw == 5) DC_GO(16, 5);
 #undef DC_GO
     }
     ResP rp{nullptr, nullptr, 1.f, 1.f};

@@ -80,7 +80,7 @@ def test_bad_arguments_are_rejected_before_any_launch(lib):
 
 
 def test_packed_filter_size_is_host_arithmetic(lib):
-    """fp16, groups 1: [Cout padded to 16][taps][Cin padded to 32] halves; no packed form for
+    """fp16, groups 1: round_up(Cout, 16) * taps * round_up(Cin, 32) halves; no packed form for
     fp32 or grouped convolutions (0)."""
     g = _geom(in_c=24, out_c=40)
     assert lib.dc_packed_filter_bytes(ctypes.byref(g), 1, 0) == 48 * 9 * 32 * 2
