@@ -158,7 +158,12 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
 hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *packed, int dtype,
                               bool transposed, hipStream_t s);
 int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed);
+hipError_t launch_densify(const void *delta, void *prev, void *out, const int32_t *mask, int P, int C,
+                          int dtype, hipStream_t s);
 hipError_t launch_pool(const dc_geometry &g, const void *in, const void *prev, void *out,
-                       const int32_t *mask, int32_t *out_mask, int mode, int dtype, hipStream_t s);
+                       const int32_t *mask, int32_t *out_mask, int mode, int dtype, bool out_f32,
+                       hipStream_t s);
+// Whether a 1x1-output pooling of this shape can write its result in the tensor's own type.
+bool pool_global_casts(const dc_geometry &g, const void *in, const void *prev, int dtype);
 
 }  // namespace dc

@@ -276,7 +276,10 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
 // the depthwise kernel; a lane owns N consecutive output channels, input values are scalar
 // broadcasts.  fp16 filters are read in the reference layout directly: for an even channel
 // offset the even outputs sit in row ci and the odd ones in row ci ^ 1 of the swizzle.
-template <typename T, int ACT>
+// K3 (3x3): the filter is staged once per workgroup into LDS in [tap][ci][co] order (un-swizzled)
+// and the 9 x Cin input values and the cached state are requested before the mask words have
+// arrived, so the kernel is one memory round trip instead of one per active tap.
+template <typename T, int ACT, bool K3>
 __global__ void __launch_bounds__(256)
 conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
                    const T *__restrict__ bias, T *__restrict__ out,
@@ -298,6 +301,45 @@ conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
     const int glo = lane_id() & ~(G - 1);
     const uint64_t gmask = G >= WAVE ? ~0ull : ((1ull << G) - 1ull);
 
+    extern __shared__ __align__(16) unsigned char s_raw[];
+    T *s_w = reinterpret_cast<T *>(s_raw);
+    float xin[K3 ? 9 : 1][MAXCI];
+    Vec<T, N> q[1], tr[1];
+    if (K3) {
+        const int cv = C / N;  // 16-byte vectors per filter row (C % N == 0, so w_co == C)
+        const int total = 9 * p.Ci * cv;
+        for (int i = threadIdx.x; i < total; i += blockDim.x) {
+            const int v = i % cv, r2 = i / cv;
+            const int ci = r2 % p.Ci, t = r2 / p.Ci;
+            Vec<T, N> w = vload<T, N>(filter + ((size_t)ci * 9 + t) * p.w_co + v * N);
+            if (p.swz) {  // odd output channels live in the partner row of the pair swizzle
+                const Vec<T, N> w1 = vload<T, N>(filter + ((size_t)(ci ^ 1) * 9 + t) * p.w_co + v * N);
+#pragma unroll
+                for (int j = 1; j < N; j += 2) w.v[j] = w1.v[j];
+            }
+            vstore<T, N>(s_w + (size_t)i * N, w);
+        }
+        const int pc = valid ? po : 0;
+        const int cb = pc / (p.Ho * p.Wo), cr = pc - cb * p.Ho * p.Wo;
+        const int cy = cr / p.Wo, cx = cr - cy * p.Wo;
+        const T *inb = in + (size_t)cb * p.Hi * p.Wi * p.Ci;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const int ky = t / 3, kx = t - ky * 3;
+            const int iy = min(max(cy * p.sh - p.pt + ky * p.dh, 0), p.Hi - 1);
+            const int ix = min(max(cx * p.sw - p.pl + kx * p.dw, 0), p.Wi - 1);
+            const T *xr = inb + (size_t)(iy * p.Wi + ix) * p.Ci;
+#pragma unroll
+            for (int ci = 0; ci < MAXCI; ++ci) xin[t][ci] = float(xr[min(ci, p.Ci - 1)]);
+        }
+        if (ACT >= 0) {
+            const int cc = min(gl * N, C - N);
+            q[0] = vload<T, N>((const T *)epi.prev + (size_t)pc * C + cc);
+            tr[0] = vload<T, N>((const T *)epi.trunc + (size_t)pc * C + cc);
+        }
+        __syncthreads();
+    }
+
     uint64_t taps = 0;
     for (int j = 0; j < K2; j += G) {
         const int t = j + gl;
@@ -315,13 +357,27 @@ conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
 
     const int c = gl * N;
     const bool lane_on = active && c < C;
-    Vec<T, N> q[1], tr[1];
-    if (ACT >= 0)
+    if (ACT >= 0 && !K3)
         load_state<T, 1>(q, tr, active, (size_t)po, gl, G, C, (const T *)epi.prev, (const T *)epi.trunc);
     float acc[N];
 #pragma unroll
     for (int j = 0; j < N; ++j) acc[j] = 0.f;
-    if (lane_on) {
+    if (K3) {
+        if (lane_on) {
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                const bool on = (taps >> t) & 1ull;
+#pragma unroll
+                for (int ci = 0; ci < MAXCI; ++ci) {
+                    if (ci >= p.Ci) break;
+                    const float xv = on ? xin[t][ci] : 0.f;
+                    const Vec<T, N> w = vload<T, N>(s_w + (size_t)(t * p.Ci + ci) * C + c);
+#pragma unroll
+                    for (int j = 0; j < N; ++j) acc[j] = __builtin_fmaf(xv, float(w.v[j]), acc[j]);
+                }
+            }
+        }
+    } else if (lane_on) {
         const T *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
         for (int t = 0; t < K2; ++t) {
             if (!((taps >> t) & 1ull)) continue;
@@ -663,7 +719,13 @@ bool try_fewcin(const dc_geometry &g, const ConvP &p, const T *in, const T *filt
            epi ? epi->mode : 0};
     const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
     const int lg = log2i(G);
-#define DC_FC(A) conv_fewcin_kernel<T, A><<<grid, block, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg)
+    const bool k3 = g.kernel_h == 3 && g.kernel_w == 3;
+    const size_t lds = k3 ? (size_t)9 * g.in_c * g.out_c * sizeof(T) : 0;
+#define DC_FC(A)                                                                                              \
+    do {                                                                                                      \
+        if (k3) conv_fewcin_kernel<T, A, true><<<grid, block, lds, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg); \
+        else conv_fewcin_kernel<T, A, false><<<grid, block, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg);     \
+    } while (0)
     switch (act) {
         case DC_ACT_LINEAR: DC_FC(DC_ACT_LINEAR); break;
         case DC_ACT_RELU: DC_FC(DC_ACT_RELU); break;

@@ -242,7 +242,8 @@ int dc_deconv(const dc_geometry *g, const void *input, const void *filter,
 }
 
 int dc_pool(const dc_geometry *g, const void *input, const void *prev_input, void *out,
-            const int32_t *mask, int32_t *out_mask, int pooling_mode, int dtype, void *stream) {
+            const int32_t *mask, int32_t *out_mask, int pooling_mode, int dtype,
+            int global_out_dtype, void *stream) {
     DC_REQUIRE_DTYPE("dc_pool");
     int rc = check_geometry("dc_pool", g, false, true);
     if (rc != DC_OK) return rc;
@@ -255,9 +256,19 @@ int dc_pool(const dc_geometry *g, const void *input, const void *prev_input, voi
     if (pooling_mode == DC_POOL_MAX) DC_REQUIRE_PTR("dc_pool", prev_input);
     DC_REQUIRE_ALIGNED("dc_pool", input, esize(dtype));
     DC_REQUIRE_ALIGNED("dc_pool", prev_input, esize(dtype));
-    DC_REQUIRE_ALIGNED("dc_pool", out, (g->out_h == 1 && g->out_w == 1) ? 4 : esize(dtype));
+    const bool global = g->out_h == 1 && g->out_w == 1;
+    bool out_f32 = true;
+    if (global) {
+        if (global_out_dtype != DC_F32 && global_out_dtype != dtype)
+            return fail(DC_ERR_DTYPE, "dc_pool: global_out_dtype %d is neither float32 nor the tensor type",
+                        global_out_dtype);
+        out_f32 = global_out_dtype == DC_F32;
+        if (!out_f32 && !dc::pool_global_casts(*g, input, prev_input, dtype))
+            return fail(DC_ERR_UNSUPPORTED, "dc_pool: this shape needs a float32 output buffer");
+    }
+    DC_REQUIRE_ALIGNED("dc_pool", out, (global && out_f32) ? 4 : esize(dtype));
     return finish(dc::launch_pool(*g, input, prev_input, out, mask, out_mask, pooling_mode, dtype,
-                                  (hipStream_t)stream), "dc_pool");
+                                  out_f32, (hipStream_t)stream), "dc_pool");
 }
 
 int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_t *mask_a,
@@ -281,6 +292,22 @@ int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_
     return finish(dc::launch_add(a, b, prev_out, out, mask_a, mask_b, mask_out, weight_a, weight_b,
                                  activation, dense_out, pixels, channels, dtype,
                                  (hipStream_t)stream), "dc_add");
+}
+
+int dc_densify(const void *delta, void *prev_out, void *out, const int32_t *mask, int32_t pixels,
+               int32_t channels, int dtype, void *stream) {
+    DC_REQUIRE_DTYPE("dc_densify");
+    int rc = check_pc("dc_densify", pixels, channels);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_PTR("dc_densify", delta);
+    DC_REQUIRE_PTR("dc_densify", prev_out);
+    DC_REQUIRE_PTR("dc_densify", out);
+    DC_REQUIRE_PTR("dc_densify", mask);
+    DC_REQUIRE_ALIGNED("dc_densify", delta, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_densify", prev_out, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_densify", out, esize(dtype));
+    return finish(dc::launch_densify(delta, prev_out, out, mask, pixels, channels, dtype,
+                                     (hipStream_t)stream), "dc_densify");
 }
 
 int dc_add_to_dense(void *a, void *b, const int32_t *mask_a, int activation, int32_t pixels,

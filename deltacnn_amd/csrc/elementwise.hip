@@ -214,6 +214,29 @@ accumulate_kernel(T *__restrict__ delta, T *__restrict__ prev, const int32_t *__
     }
 }
 
+// Densify: prev += delta on active pixels, out = prev on every pixel.
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+densify_kernel(const T *__restrict__ delta, T *__restrict__ prev, T *__restrict__ out,
+               const int32_t *__restrict__ mask, int P, int C, int lg) {
+    const int G = 1 << lg;
+    int p, gl;
+    group_coords(lg, p, gl);
+    if (p >= P) return;
+    const bool on = mask[p] != 0;
+    for (int c = gl * N; c < C; c += G * N) {
+        const size_t off = (size_t)p * C + c;
+        Vec<T, N> q = vload<T, N>(prev + off);
+        if (on) {
+            const Vec<T, N> dl = vload<T, N>(delta + off);
+#pragma unroll
+            for (int j = 0; j < N; ++j) q.v[j] = dl.v[j] + q.v[j];
+            vstore<T, N>(prev + off, q);
+        }
+        vstore<T, N>(out + off, q);
+    }
+}
+
 // ------------------------------------------------------------------------------------ add
 // s = wa*a*[Ma]; s = fma(b, wb, s)*[Mb]; mask_out = Ma | Mb (written for every pixel).
 // act > 0: prev += s, out = act(prev_new) - act(prev_old).
@@ -550,6 +573,25 @@ hipError_t launch_activate_truncate(void *delta, void *prev, void *trunc, int32_
     if (dtype == DC_F32)
         return act_trunc_t<float>((float *)delta, (float *)prev, (float *)trunc, mask, thr, act, mode, P, C, s);
     return act_trunc_t<half_t>((half_t *)delta, (half_t *)prev, (half_t *)trunc, mask, thr, act, mode, P, C, s);
+}
+
+template <typename T>
+hipError_t densify_t(const T *delta, T *prev, T *out, const int32_t *mask, int P, int C, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    if (can_vec<T>(C, {delta, prev, out})) {
+        GroupLaunch L(P, pick_group(C / N, P, 4));
+        densify_kernel<T, N><<<L.grid, L.block, 0, s>>>(delta, prev, out, mask, P, C, L.lg);
+    } else {
+        GroupLaunch L(P, group_lanes(C, 1));
+        densify_kernel<T, 1><<<L.grid, L.block, 0, s>>>(delta, prev, out, mask, P, C, L.lg);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_densify(const void *delta, void *prev, void *out, const int32_t *mask, int P, int C,
+                          int dtype, hipStream_t s) {
+    if (dtype == DC_F32) return densify_t<float>((const float *)delta, (float *)prev, (float *)out, mask, P, C, s);
+    return densify_t<half_t>((const half_t *)delta, (half_t *)prev, (half_t *)out, mask, P, C, s);
 }
 
 hipError_t launch_add(const void *a, const void *b, void *prev, void *out, const int32_t *ma,

@@ -167,9 +167,74 @@ pool_global_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restri
     }
 }
 
+// 1x1 output over the whole unpadded map (global pooling), channels in 16-byte vectors:
+// a workgroup owns VPB channel vectors and splits the pixels over 256 / VPB slices; every
+// load is unconditional (the mask word selects afterwards), partial results meet in LDS and
+// are combined slice by slice in ascending order, so the sum has a fixed order and needs no
+// atomics.  OutT is float (the reference's accumulator protocol) or T (cast fused).
+template <typename T, typename OutT, bool MAX>
+__global__ void __launch_bounds__(256)
+pool_global_vec_kernel(int npx, int C, const T *__restrict__ in, const T *__restrict__ prev,
+                       OutT *__restrict__ out, const int32_t *__restrict__ mask,
+                       int32_t *__restrict__ out_mask) {
+    constexpr int N = Vec16<T>::N, VPB = 8, SL = 256 / VPB;
+    __shared__ float s_hi[SL][VPB * N], s_hp[MAX ? SL : 1][VPB * N];
+    const int b = blockIdx.y;
+    const int vl = threadIdx.x % VPB, sl = threadIdx.x / VPB;
+    const int c = (blockIdx.x * VPB + vl) * N;
+    const int cc = min(c, C - N);
+    const T *inb = in + (size_t)b * npx * C;
+    const T *pvb = MAX ? prev + (size_t)b * npx * C : nullptr;
+    const int32_t *mb = mask + (size_t)b * npx;
+    float hi[N], hp[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        hi[j] = MAX ? -INFINITY : 0.f;
+        hp[j] = -INFINITY;
+    }
+    int any = 0;
+    for (int ip = sl; ip < npx; ip += SL) {
+        const int m = mb[ip];
+        const Vec<T, N> d = vload<T, N>(inb + (size_t)ip * C + cc);
+        Vec<T, N> pf;
+        if (MAX) pf = vload<T, N>(pvb + (size_t)ip * C + cc);
+        any |= m;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const float dv = m != 0 ? float(d.v[j]) : 0.f;
+            if (MAX) {
+                hi[j] = fmaxf(hi[j], dv + float(pf.v[j]));
+                hp[j] = fmaxf(hp[j], float(pf.v[j]));
+            } else {
+                hi[j] += dv;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        s_hi[sl][vl * N + j] = hi[j];
+        if (MAX) s_hp[sl][vl * N + j] = hp[j];
+    }
+    const int wg_any = __syncthreads_or(any);
+    if (threadIdx.x < VPB * N) {
+        const int ch = blockIdx.x * VPB * N + threadIdx.x;
+        float r = s_hi[0][threadIdx.x], rp = MAX ? s_hp[0][threadIdx.x] : 0.f;
+        for (int s2 = 1; s2 < SL; ++s2) {
+            if (MAX) {
+                r = fmaxf(r, s_hi[s2][threadIdx.x]);
+                rp = fmaxf(rp, s_hp[s2][threadIdx.x]);
+            } else {
+                r += s_hi[s2][threadIdx.x];
+            }
+        }
+        if (ch < C) out[(size_t)b * C + ch] = OutT(wg_any ? (MAX ? r - rp : r / float(npx)) : 0.f);
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0 && out_mask != nullptr) out_mask[b] = wg_any ? 1 : 0;
+}
+
 template <typename T>
 hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, const int32_t *mask,
-                  int32_t *out_mask, int mode, hipStream_t s) {
+                  int32_t *out_mask, int mode, bool out_f32, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
     ConvP p;
     p.B = g.batch; p.Hi = g.in_h; p.Wi = g.in_w; p.Ci = g.in_c;
@@ -182,6 +247,21 @@ hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, c
     q.zero_bottom = g.pad_top != g.pad_bottom;
     q.zero_right = g.pad_left != g.pad_right;
     if (g.out_h == 1 && g.out_w == 1) {
+        const bool whole = g.kernel_h == g.in_h && g.kernel_w == g.in_w && g.pad_top == 0 && g.pad_left == 0 &&
+                           g.pad_bottom == 0 && g.pad_right == 0 && g.dilation_h == 1 && g.dilation_w == 1;
+        if (whole && g.in_c % N == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)prev & 15) == 0) {
+            dim3 vgrid(ceil_div(g.in_c / N, 8), g.batch);
+            const int npx = g.in_h * g.in_w;
+#define DC_PG(OT, MX) pool_global_vec_kernel<T, OT, MX><<<vgrid, 256, 0, s>>>(npx, g.in_c, in, prev, (OT *)out, mask, out_mask)
+            if (mode == DC_POOL_MAX) {
+                if (out_f32) DC_PG(float, true); else DC_PG(T, true);
+            } else {
+                if (out_f32) DC_PG(float, false); else DC_PG(T, false);
+            }
+#undef DC_PG
+            return hipGetLastError();
+        }
+        if (!out_f32) return hipErrorInvalidValue;  // checked by the caller: cannot happen
         dim3 grid(ceil_div(g.in_c, WAVE), g.batch);
         if (mode == DC_POOL_MAX)
             pool_global_kernel<T, true><<<grid, 256, 0, s>>>(p, q, in, prev, (float *)out, mask, out_mask);
@@ -206,11 +286,19 @@ hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, c
 
 }  // namespace
 
+bool pool_global_casts(const dc_geometry &g, const void *in, const void *prev, int dtype) {
+    const int n = dtype == DC_F32 ? 4 : 8;
+    return g.out_h == 1 && g.out_w == 1 && g.kernel_h == g.in_h && g.kernel_w == g.in_w && g.pad_top == 0 &&
+           g.pad_left == 0 && g.pad_bottom == 0 && g.pad_right == 0 && g.dilation_h == 1 &&
+           g.dilation_w == 1 && g.in_c % n == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)prev & 15) == 0;
+}
+
 hipError_t launch_pool(const dc_geometry &g, const void *in, const void *prev, void *out,
-                       const int32_t *mask, int32_t *out_mask, int mode, int dtype, hipStream_t s) {
+                       const int32_t *mask, int32_t *out_mask, int mode, int dtype, bool out_f32,
+                       hipStream_t s) {
     if (dtype == DC_F32)
-        return pool_t<float>(g, (const float *)in, (const float *)prev, out, mask, out_mask, mode, s);
-    return pool_t<half_t>(g, (const half_t *)in, (const half_t *)prev, out, mask, out_mask, mode, s);
+        return pool_t<float>(g, (const float *)in, (const float *)prev, out, mask, out_mask, mode, true, s);
+    return pool_t<half_t>(g, (const half_t *)in, (const half_t *)prev, out, mask, out_mask, mode, out_f32, s);
 }
 
 }  // namespace dc

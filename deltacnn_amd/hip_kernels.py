@@ -217,8 +217,9 @@ def pack_filter(filter: torch.Tensor, c_in: int, c_out: int, groups: int = 1,
 def sparse_pooling(x, prev_x, kernel_size, mask=None, stride=(1, 1), padding=(0, 0),
                    dilation=(1, 1), create_out_mask=True, sub_tile_sparsity=True, out_mask=None,
                    pooling_mode_int=0, out_shape=None, *, out=None):
-    """cuda_kernels.py:80-129.  A 1x1 output is accumulated in a float32 buffer and cast
-    back to the input dtype afterwards (:101-124)."""
+    """cuda_kernels.py:80-129.  The reference accumulates a 1x1 output in a float32 buffer and
+    casts it back afterwards (:101-124); here the kernel writes the input dtype directly when
+    the window is the whole unpadded map, and falls back to that protocol otherwise."""
     lib = _lib.load()
     _nhwc(x, "x")
     if mask is None:
@@ -228,14 +229,17 @@ def sparse_pooling(x, prev_x, kernel_size, mask=None, stride=(1, 1), padding=(0,
     if isinstance(out_shape, list) and len(out_shape) == 0:
         out_shape.extend([g.out_h, g.out_w])
     is_global = g.out_h == 1 and g.out_w == 1
+    vec = 16 // x.element_size()
+    direct = (is_global and g.kernel_h == g.in_h and g.kernel_w == g.in_w and tuple(_pad4(padding)) == (0, 0, 0, 0)
+              and tuple(dilation) == (1, 1) and x.shape[1] % vec == 0)
     if out is None:
-        odt = torch.float32 if is_global else x.dtype
+        odt = torch.float32 if is_global and not direct else x.dtype
         out = new_features(g.batch, x.shape[1], g.out_h, g.out_w, odt, x.device)
     if out_mask is None:
         out_mask = new_mask(g.batch, g.out_h, g.out_w, x.device)
     _call("pool", lib.dc_pool,
           (g, x.data_ptr(), _ptr(prev_x), out.data_ptr(), _mask(mask, "mask").data_ptr(),
-           out_mask.data_ptr(), int(pooling_mode_int), _dtype(x), _stream()),
+           out_mask.data_ptr(), int(pooling_mode_int), _dtype(x), _dtype(out), _stream()),
           g=g, esize=x.element_size(), in_mask=mask, out_mask=out_mask, mode=int(pooling_mode_int))
     if out.dtype != x.dtype:
         out = out.to(dtype=x.dtype)
@@ -253,6 +257,17 @@ def sparse_activation(x, prev_x, truncated, mask, threshold, activation, truncat
            float(threshold), int(activation), int(truncation_mode), _pixels(x), x.shape[1],
            _dtype(x), _stream()),
           P=_pixels(x), C=x.shape[1], esize=x.element_size(), in_mask=mask, out_mask=mask)
+
+
+def densify(delta, prev_out, out, mask):
+    """DCDensify in one launch: ``prev_out += delta`` on active pixels, ``out = prev_out``
+    everywhere (sparse_layers.py:1311-1325)."""
+    lib = _lib.load()
+    _nhwc(delta, "delta")
+    _call("densify", lib.dc_densify,
+          (delta.data_ptr(), prev_out.data_ptr(), out.data_ptr(), _mask(mask, "mask").data_ptr(), _pixels(delta),
+           delta.shape[1], _dtype(delta), _stream()),
+          P=_pixels(delta), C=delta.shape[1], esize=delta.element_size(), in_mask=mask, dense_copy=True)
 
 
 def sparsify(input, prev_in, delta, mask, threshold):

@@ -540,6 +540,7 @@ class DCDensify(DCModule):
         self.name = name
         self.activation, self.activation_int = convert_activation_string(activation)
         self.prev_out = None
+        self.out = None
         self.idx = -1
         self.clone_out = clone_out
 
@@ -552,10 +553,14 @@ class DCDensify(DCModule):
             self.idx = DCDensify.idx
             self.prev_out = torch.zeros_like(input)
             DCModule.temp_buffers.append(self.prev_out)
-        hk.sparse_activation(input, self.prev_out, None, mask, -1, -1, DCTruncation.none.value)
-        out = self.prev_out
-        if self.clone_out:
-            out = out.clone()
+        if self.clone_out:  # accumulate and copy in one launch
+            out = self.out if DCModule.reuse_buffers and self.out is not None else torch.empty_like(self.prev_out)
+            if DCModule.reuse_buffers:
+                self.out = out
+            hk.densify(input, self.prev_out, out, mask)
+        else:
+            hk.sparse_activation(input, self.prev_out, None, mask, -1, -1, DCTruncation.none.value)
+            out = self.prev_out
         if self.activation is not None:
             return self.activation(out)
         return out
@@ -563,6 +568,7 @@ class DCDensify(DCModule):
     def reset(self):
         super().reset()
         self.prev_out = None
+        self.out = None
 
 
 class DCUpsamplingNearest2d(DCModule):

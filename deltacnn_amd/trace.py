@@ -6,7 +6,7 @@ m = 4-byte mask word, P pixels, n_x = number of active pixels of mask x):
 
   sparsify           R = 2*P*C*s                          W = 2*n_out*C*s + P*m
   activate_truncate  R = P*m + n_in*3*C*s                 W = n_out*3*C*s + (n_in-n_out)*(C*s + m)
-  densify            R = P*m + n*2*C*s                    W = n*C*s
+  densify            R = P*m + n*2*C*s                    W = n*C*s   (+ dense copy: R += (P-n)*C*s, W += P*C*s)
   add                R = 2*P*m + (n_a+n_b)*C*s [+n_out*C*s]  W = n_out*C*s [+n_out*C*s] + P*m
   conv / deconv      R = P_in*m + n_in*Cin*s + K*K*(Cin/g)*Cout*s   W = n_out*Cout*s + P_out*m
                      (conv_act: the same; conv_add: + P_out*m + n_res*Cout*s for the residual)
@@ -162,6 +162,8 @@ class Tracer:
                     dens = (n_in / P, n_out / P)
                 elif op == "densify":
                     rd, wr = P * m + n_in * 2 * C * s, n_in * C * s
+                    if meta.get("dense_copy"):  # + the dense copy of every pixel
+                        rd, wr = rd + (P - n_in) * C * s, wr + P * C * s
                     dens = (n_in / P, n_in / P)
                 elif op == "add":
                     n_o = n_out if n_out is not None else P

@@ -133,16 +133,27 @@ int dc_deconv(const dc_geometry *g, const void *input, const void *filter,
               int32_t *out_mask, int dtype, void *stream);
 
 /* Replaces sparse_pooling_wrapper_masked (conv_torch_wrapper.cpp:213-293).  `prev_input` is
- * required for DC_POOL_MAX.  When out_h == out_w == 1, `out` is float32 [B][C]
- * irrespective of dtype (cuda_kernels.py:101-109) and is fully overwritten. */
+ * required for DC_POOL_MAX.  When out_h == out_w == 1, `out` is [B][C], fully overwritten, of
+ * type `global_out_dtype`: DC_F32 is the reference's protocol (a float32 accumulator,
+ * cuda_kernels.py:101-109, cast back by the caller, :123-124); passing `dtype` fuses that
+ * cast (window == whole unpadded map, channels a multiple of the 16-byte vector, else
+ * DC_ERR_UNSUPPORTED before any launch).  Ignored for other output sizes. */
 int dc_pool(const dc_geometry *g, const void *input, const void *prev_input, void *out,
-            const int32_t *mask, int32_t *out_mask, int pooling_mode, int dtype, void *stream);
+            const int32_t *mask, int32_t *out_mask, int pooling_mode, int dtype,
+            int global_out_dtype, void *stream);
 
 /* Replaces sparse_add_tensors_wrapper (conv_torch_wrapper.cpp:387-444). */
 int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_t *mask_a,
            const int32_t *mask_b, int32_t *mask_out, float weight_a, float weight_b,
            int activation, int dense_out, int32_t pixels, int32_t channels, int dtype,
            void *stream);
+
+/* DCDensify in one launch (sparse_layers.py:1287-1329): prev_out += delta on active pixels,
+ * then out = prev_out for EVERY pixel (the dense clone of :1324-1325).  No counterpart in the
+ * reference, which runs deltacnn_activate_truncate(..., truncation_mode -1) and a torch clone;
+ * results are identical. */
+int dc_densify(const void *delta, void *prev_out, void *out, const int32_t *mask, int32_t pixels,
+               int32_t channels, int dtype, void *stream);
 
 /* Replaces sparse_add_to_dense_tensor_wrapper (conv_torch_wrapper.cpp:447-482):
  * b[px] += a[px] on active pixels.  With activation > 0 it also writes a = act(b) on every

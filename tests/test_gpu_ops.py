@@ -180,6 +180,24 @@ def test_densify_accumulate(lib, dtype, C, act):
     assert torch.equal(d_mask.cpu(), mask)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C,H,W", [(3, 8, 12), (17, 8, 12), (64, 16, 9), (1280, 1, 1), (2100, 3, 3)])
+def test_densify_fused(lib, dtype, C, H, W):
+    """Accumulate + dense copy in one launch == accumulate, then clone."""
+    g = _gen(550 + C)
+    B = 2
+    mask = rand_mask(g, B, H, W, 0.4)
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+    delta = torch.randn(B, C, H, W, generator=g).to(dtype)
+    w_delta, w_prev = delta.clone(), prev.clone()
+    ops.activate_truncate(w_delta, w_prev, None, mask, -1, -1, -1)
+    d_prev = cl(prev)
+    out = torch.full_like(d_prev, float("nan"))
+    hk().densify(cl(poison(delta, mask)), d_prev, out, cl(mask))
+    assert torch.equal(d_prev.cpu(), w_prev)
+    assert torch.equal(out.cpu(), w_prev)
+
+
 # ------------------------------------------------------------------------------------ add
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("C", [3, 16, 24, 33, 160, 2100])
@@ -472,6 +490,13 @@ def test_pool_global(lib, dtype, mode, C, H, W, density):
     # the average is a float sum over up to H*W values in a different order than the oracle's
     tol = 1e-5 if dtype == torch.float32 else 2e-3
     assert_masked_close(out, want, want_mask, tol, tol, "out")
+    # the reference's protocol: float32 accumulator handed in by the caller, cast afterwards
+    acc = torch.full((B, C, 1, 1), float("nan"), dtype=torch.float32, device=DEV).contiguous(
+        memory_format=torch.channels_last)
+    out2, om2 = hk().sparse_pooling(cl(poison(x, mask)), cl(prev) if mode == 0 else None, (H, W), cl(mask),
+                                    pooling_mode_int=mode, out=acc)
+    assert out2.dtype == dtype and torch.equal(om2.cpu(), want_mask)
+    assert_masked_close(out2, want, want_mask, tol, tol, "out (float32 accumulator)")
 
 
 # ------------------------------------------------------------- upsample / concat / mul_add

@@ -21,7 +21,7 @@ def declared_symbols():
 
 def test_header_declares_the_operator_set():
     names = declared_symbols()
-    for op in ("sparsify", "activate_truncate", "conv", "deconv", "pool", "add", "add_to_dense",
+    for op in ("sparsify", "activate_truncate", "conv", "deconv", "pool", "add", "add_to_dense", "densify",
                "upsample", "concat", "mul_add", "version", "last_error"):
         assert f"dc_{op}" in names
 
@@ -76,7 +76,13 @@ def test_bad_arguments_are_rejected_before_any_launch(lib):
     assert lib.dc_deconv(ctypes.byref(g), p, p, None, None, p, p, p, 0, None) == -3
     # pooling keeps the channel count
     g = _geom(out_c=8)
-    assert lib.dc_pool(ctypes.byref(g), p, p, p, p, p, 0, 0, None) == -2
+    assert lib.dc_pool(ctypes.byref(g), p, p, p, p, p, 0, 0, 0, None) == -2
+    # a 1x1 output in the tensor's own type needs window == whole unpadded map
+    g = _geom(in_h=8, in_w=8, out_h=1, out_w=1, kernel_h=8, kernel_w=8, pad_top=0, pad_left=0, pad_bottom=0, pad_right=0)
+    assert lib.dc_pool(ctypes.byref(g), p, p, p, p, p, 1, 1, 2, None) == -1
+    g = _geom(in_h=6, in_w=6, out_h=1, out_w=1, kernel_h=8, kernel_w=8)
+    assert lib.dc_pool(ctypes.byref(g), p, p, p, p, p, 1, 1, 1, None) == -3
+    assert lib.dc_densify(p, p, None, p, 16, 4, 0, None) == -4
 
 
 def test_packed_filter_size_is_host_arithmetic(lib):
