@@ -11,8 +11,12 @@ All frames are resident in HBM before the timed region.  One JSON line is printe
   dense_gpu        the same model dense (plain PyTorch / MIOpen) on the same GPU, eager and
                    graph-replayed, and the speed-up over the faster of the two
   sweep            frames/sec at 1/5/10/25/50/100 % input update density
-  kernels          per-kernel-class time, algorithmic GB/s and TFLOP/s of one traced pass
-  roofline         the kernel class with the largest share of the frame time
+  kernels          per HIP kernel: launches per frame, device time per launch, algorithmic
+                   bytes per launch, GB/s and TFLOP/s of one traced frame
+  roofline         the kernel with the largest share of the frame time
+  micro            single-layer sweeps on a 64x64 map (3x3 256->256, 1x1 256->1024, depthwise
+                   C=512, each + ReLU/truncation) over the update densities
+  scaled           the memory-bound operators at 512x512, batch 8 (working set beyond the caches)
   cpu_baseline     the CPU oracle of the delta path timed on this host's cores (bounded sample)
 """
 from __future__ import annotations
@@ -141,6 +145,106 @@ def trace_kernels(delta, frames):
     return agg, rows
 
 
+def _trace_calls(fn, alt_inputs=None):
+    """Run fn() once under the tracer, time its library calls by graph replay, return rows."""
+    import torch
+    from deltacnn_amd import hip_kernels as hk
+    from deltacnn_amd.trace import Tracer
+    tr = Tracer()
+    hk.set_tracer(tr)
+    try:
+        with torch.no_grad():
+            fn()
+    finally:
+        hk.set_tracer(None)
+    times = tr.replay_times(alt_inputs=alt_inputs)
+    for rec, us in zip(tr.records, times):
+        rec["ms"] = us * 1e-3
+    return tr.finish()
+
+
+def _row_report(rows):
+    return [{"kernel": r["kernel"], "us": round(r["ms"] * 1e3, 3),
+             "alg_GBps": round(r["bytes"] / (r["ms"] * 1e-3) / 1e9, 1),
+             "hbm_frac": round(r["bytes"] / (r["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+             "alg_TFLOPs": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2),
+             "mfma_frac": round(r["flops"] / (r["ms"] * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 5)} for r in rows]
+
+
+def micro_bench():
+    """Single-layer sweeps on a 64x64 fp16 map: 3x3 256->256, 1x1 256->1024 and depthwise 3x3
+    C=512, each followed by ReLU with truncation (threshold 0.05), update density 1..100 %.
+    Weights N(0,1)/sqrt(fan_in), cached pre-activation N(0,1), deltas N(0,0.5) on a random
+    subset of pixels, N(0,1) garbage elsewhere."""
+    import torch
+    from deltacnn_amd import hip_kernels as hk
+    from deltacnn_amd.filter_conversion import convert_half_filter
+    H = W = 64
+    out = []
+    gen = torch.Generator().manual_seed(1235)
+    for name, cin, cout, k, groups in (("conv3x3_256_256", 256, 256, 3, 1), ("conv1x1_256_1024", 256, 1024, 1, 1),
+                                       ("dw3x3_512", 512, 512, 3, 512)):
+        wt = (torch.randn(cout, cin // groups, k, k, generator=gen) / (cin // groups * k * k) ** 0.5).half()
+        filt = convert_half_filter(wt, pixel_wise=groups > 1).cuda()
+        packed = hk.pack_filter(filt, cin, cout, groups)
+        prev = torch.randn(1, cout, H, W, generator=gen).half().cuda().contiguous(memory_format=torch.channels_last)
+        trunc = torch.zeros_like(prev)
+        obuf, omask = torch.zeros_like(prev), torch.zeros(1, 1, H, W, dtype=torch.int32, device="cuda")
+        for rho in SWEEP:
+            n = max(1, round(rho * H * W))
+            mask = torch.zeros(H * W, dtype=torch.int32)
+            mask[torch.randperm(H * W, generator=gen)[:n]] = 1
+            mask = mask.view(1, 1, H, W).cuda()
+            x = torch.randn(1, cin, H, W, generator=gen)
+            x = torch.where(mask.cpu() != 0, x * 0.5, x).half().cuda().contiguous(memory_format=torch.channels_last)
+            rows = _trace_calls(lambda: hk.sparse_conv_activation(
+                x, filt, mask, None, prev, trunc, THRESHOLD, 1, 0, (1, 1), (k // 2, k // 2), (1, 1), groups, cout,
+                packed_filter=packed, out=obuf, out_mask=omask))
+            out.append({"op": name, "density": rho, "us": round(sum(r["ms"] for r in rows) * 1e3, 3),
+                        "kernels": _row_report(rows)})
+            log(f"  micro {name:18s} density {rho:4.2f}: " +
+                "  ".join(f"{r['kernel']} {r['us']:.2f} us {r['alg_GBps']:.0f} GB/s {r['alg_TFLOPs']:.1f} TF/s"
+                          for r in out[-1]["kernels"]))
+    return out
+
+
+def scaled_bench():
+    """The memory-bound operators on a working set far beyond the caches (512x512, batch 8,
+    64 channels fp16: 268 MB per tensor), where the bandwidth roofline applies."""
+    import torch
+    from deltacnn_amd import hip_kernels as hk
+    B, C, H, W = 8, 64, 512, 512
+    gen = torch.Generator(device="cuda").manual_seed(7)
+
+    def feat():
+        return torch.randn(B, C, H, W, device="cuda", dtype=torch.half, generator=gen).contiguous(
+            memory_format=torch.channels_last)
+    out = []
+    a, b, c, d = feat(), feat(), feat(), feat()
+    wdw = torch.randn(1, 3, 3, C, device="cuda", dtype=torch.half, generator=gen) / 3
+    for rho in (0.1, 1.0):
+        mask = (torch.rand(B, 1, H, W, device="cuda", generator=gen) < rho).to(torch.int32)
+        mask2 = mask.clone()
+        ops = {
+            "sparsify": (lambda: hk.sparsify(a, b, c, mask2, 1e9 if rho < 1 else -1.0), None),
+            "activate_truncate": (lambda: hk.sparse_activation(a, b, c, mask2.copy_(mask), 0.0, 1, 0), None),
+            "densify": (lambda: hk.densify(a, b, c, mask), None),
+            "add": (lambda: hk.sparse_add_tensors(a, b, None, c, mask, mask, mask2, 1.0, 1.0, 0, False), None),
+            "depthwise3x3+relu": (lambda: hk.sparse_conv_activation(a, wdw, mask, None, b, c, 0.0, 1, 0, (1, 1), (1, 1),
+                                                                    (1, 1), C, C, out=d, out_mask=mask2), None),
+        }
+        if rho < 1:
+            ops.pop("sparsify")  # its density is set by the data, measured at 100 % only
+        for name, (fn, _) in ops.items():
+            rows = _trace_calls(fn, alt_inputs=[a.data_ptr(), d.data_ptr()])
+            rep = _row_report(rows)
+            out.append({"op": name, "density": rho, "kernels": rep})
+            log(f"  scaled {name:20s} density {rho:4.2f}: " +
+                "  ".join(f"{r['kernel']} {r['us']:.1f} us {r['alg_GBps']:.0f} GB/s ({100 * r['hbm_frac']:.1f} % of HBM peak)"
+                          for r in rep))
+    return out
+
+
 def cpu_baseline(state, video, n_frames, threads):
     """The CPU oracle of the delta path (pure PyTorch, fp32) on this host, bounded sample."""
     import torch
@@ -177,8 +281,12 @@ def main():
     ap.add_argument("--mode", choices=["graph", "eager"], default="graph")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-micro", action="store_true", help="skip the single-layer and scaled-shape sections")
     ap.add_argument("--only-delta", action="store_true",
                     help="time the delta path only and print a short JSON line (for profiling runs)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="with --only-delta: end with one 256 MiB device-to-device copy kernel, the known-size "
+                         "reference that hardware traffic counters of a profiling run are scaled by")
     ap.add_argument("--cpu-frames", type=int, default=12)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -206,6 +314,12 @@ def main():
     fps = 1.0 / sec
     log(f"delta path: {fps:.1f} frames/s ({sec * 1e3:.3f} ms/frame, mode={args.mode})")
     if args.only_delta:
+        if args.calibrate_copy:
+            src = torch.ones(64 << 20, dtype=torch.float32, device="cuda")
+            dst = torch.empty_like(src)
+            torch.cuda.synchronize()
+            dst.copy_(src)  # 256 MiB read + 256 MiB written by one copy kernel
+            torch.cuda.synchronize()
         print(json.dumps({"value": round(fps, 2), "unit": "frames/s", "ms_per_step": round(sec * 1e3, 4),
                           "steps": args.steps, "update_density": args.density}), flush=True)
         return
@@ -231,9 +345,21 @@ def main():
     kernels = {k: {"launches_per_frame": round(a["launches_per_frame"], 2),
                    "us_per_launch": round(a["us_per_launch"], 3),
                    "ms_per_frame": round(a["ms_per_frame"], 4),
+                   "alg_bytes_per_launch": round(a["bytes_per_launch"], 1),
                    "alg_GBps": round(a["GBps"], 2), "alg_TFLOPs": round(a["TFLOPs"], 3)}
                for k, a in sorted(agg.items(), key=lambda kv: -kv[1]["ms"])}
     alg_frame_bytes = sum(a["bytes"] for a in agg.values())
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
+    if os.path.exists(tpath):  # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+        with open(tpath) as f:
+            traffic = json.load(f).get(dom_name, {}).get("bytes_per_launch")
+    micro = scaled = None
+    if not args.no_micro:
+        log("single-layer sweeps (64x64 fp16):")
+        micro = micro_bench()
+        log("scaled shapes (512x512, batch 8, C=64 fp16):")
+        scaled = scaled_bench()
 
     cpu = None
     if not args.no_cpu:
@@ -261,12 +387,14 @@ def main():
         "kernels": kernels,
         "roofline": {"bound": "hbm", "kernel": dom_name,
                      "achieved": round(dom["GBps"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom["GBps"] / HBM_PEAK_GBS, 5), "traffic": None,
+                     "frac": round(dom["GBps"] / HBM_PEAK_GBS, 5), "traffic": traffic,
                      "bytes_per_launch": round(dom["bytes_per_launch"], 1),
                      "us_per_launch": round(dom["us_per_launch"], 3),
                      "note": "latency-bound regime: the feature maps of this workload are <= 2.4 MB and "
                              "an empty dependent kernel in a HIP graph already costs ~1.6 us"},
         "cpu_baseline": cpu,
+        "micro": micro,
+        "scaled": scaled,
     }
     with torch.no_grad():
         delta.reset_layers()

@@ -30,6 +30,7 @@ _G = POINTER(Geometry)
 _SIGNATURES = {
     "dc_version": (c_char_p, []),
     "dc_last_error": (c_char_p, []),
+    "dc_last_kernels": (ctypes.c_char_p, []),
     "dc_sparsify": (c_int, [_P, _P, _P, _P, c_float, c_int32, c_int32, c_int, _P]),
     "dc_activate_truncate": (c_int, [_P, _P, _P, _P, c_float, c_int, c_int, c_int32, c_int32, c_int, _P]),
     "dc_conv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),

@@ -100,6 +100,13 @@ __device__ __forceinline__ half_t tabs(half_t x) { return __builtin_fabsf16(x); 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Names of the kernels launched by the calling thread's current entry point ('+'-separated),
+// for tracing tools: kernel_log_reset() at the start of an entry point, note_kernel() at every
+// launch site.
+void kernel_log_reset();
+void note_kernel(const char *name);
+const char *kernel_log();
+
 // Workgroup size of the one-group-per-pixel kernels.  A launch of up to 2048 wavefronts runs
 // one wavefront per workgroup so that it spreads over as many compute units as possible (these
 // launches are bound by latency and by the load issue rate of a compute unit, not by

@@ -641,6 +641,7 @@ hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *pa
     const size_t total = (size_t)co_p * K2 * ci_p;
     int blocks = (int)((total + 255) / 256);
     if (blocks > 4096) blocks = 4096;
+    note_kernel("pack_filter_kernel");
     pack_filter_kernel<<<blocks, 256, 0, s>>>((const half_t *)filter, (half_t *)packed, g.in_c,
                                               g.out_c, K2, g.out_c + (g.out_c & 1), ci_p, co_p);
     return hipGetLastError();
@@ -685,6 +686,7 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
     const int G = pick_group(nvec, P_out, 4);
     const int iters = ceil_div(nvec, G);
     const int block = group_block(P_out * G);
+    note_kernel("conv_dw_kernel");
     dim3 grid((unsigned)ceil_div64(P_out * G, block));
     EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f,
            epi ? epi->mode : 0};
@@ -719,6 +721,7 @@ bool try_fewcin(const dc_geometry &g, const ConvP &p, const T *in, const T *filt
            epi ? epi->mode : 0};
     const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
     const int lg = log2i(G);
+    note_kernel("conv_fewcin_kernel");
     const bool k3 = g.kernel_h == 3 && g.kernel_w == 3;
     const size_t lds = k3 ? (size_t)9 * g.in_c * g.out_c * sizeof(T) : 0;
 #define DC_FC(A)                                                                                              \
@@ -771,12 +774,14 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
         const bool ksplit = steps >= 8;
         const int co_blocks = ksplit ? co_tiles : ceil_div(co_tiles, 4);
         dim3 grid(tx, ty, g.batch * co_blocks);
+        note_kernel("conv_mfma_kernel");
 #define DC_MFMA(TRF, KS) conv_mfma_kernel<TRF, KS><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, co_blocks, ci_p)
         if (transposed) { if (ksplit) DC_MFMA(true, true); else DC_MFMA(true, false); }
         else { if (ksplit) DC_MFMA(false, true); else DC_MFMA(false, false); }
 #undef DC_MFMA
     } else {
         dim3 grid(tx, ty, g.batch);
+        note_kernel("conv_direct_kernel");
         int COT = pow2_ceil(g.out_c);
         if (COT > 256) COT = 256;
         if (dtype == DC_F32) {

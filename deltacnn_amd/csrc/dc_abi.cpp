@@ -2,12 +2,14 @@
 // Every check runs before the first HIP call, so bad arguments are reported without a GPU.
 #include <cstdarg>
 #include <cstdio>
+#include <cstring>
 
 #include "common.hpp"
 
 namespace {
 
 thread_local char g_error[512] = "";
+thread_local char g_kernels[256] = "";
 
 int fail(int code, const char *fmt, ...) {
     va_list ap;
@@ -109,14 +111,26 @@ int check_conv(const char *fn, const dc_geometry *g, const void *input, const vo
 
 }  // namespace
 
+namespace dc {
+void kernel_log_reset() { g_kernels[0] = 0; }
+void note_kernel(const char *name) {
+    const size_t used = strlen(g_kernels);
+    snprintf(g_kernels + used, sizeof(g_kernels) - used, "%s%s", used ? "+" : "", name);
+}
+const char *kernel_log() { return g_kernels; }
+}  // namespace dc
+
 extern "C" {
 
 const char *dc_version(void) { return "deltacnn-hip 0.1 (gfx950)"; }
 
 const char *dc_last_error(void) { return g_error; }
 
+const char *dc_last_kernels(void) { return g_kernels; }
+
 int dc_sparsify(const void *input, void *prev_input, void *delta, int32_t *mask, float threshold,
                 int32_t pixels, int32_t channels, int dtype, void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_sparsify");
     int rc = check_pc("dc_sparsify", pixels, channels);
     if (rc != DC_OK) return rc;
@@ -135,6 +149,7 @@ int dc_sparsify(const void *input, void *prev_input, void *delta, int32_t *mask,
 int dc_activate_truncate(void *delta, void *prev_input, void *truncated, int32_t *mask,
                          float threshold, int activation, int truncation_mode, int32_t pixels,
                          int32_t channels, int dtype, void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_activate_truncate");
     int rc = check_pc("dc_activate_truncate", pixels, channels);
     if (rc != DC_OK) return rc;
@@ -158,6 +173,7 @@ int dc_activate_truncate(void *delta, void *prev_input, void *truncated, int32_t
 int dc_conv(const dc_geometry *g, const void *input, const void *filter, const void *packed_filter,
             const void *bias, void *out, const int32_t *mask, int32_t *out_mask, int dtype,
             void *stream) {
+    dc::kernel_log_reset();
     int rc = check_conv("dc_conv", g, input, filter, out, mask, out_mask, dtype, false);
     if (rc != DC_OK) return rc;
     DC_REQUIRE_ALIGNED("dc_conv", packed_filter, 16);
@@ -169,6 +185,7 @@ int dc_conv_act(const dc_geometry *g, const void *input, const void *filter,
                 const void *packed_filter, const void *bias, void *out, const int32_t *mask,
                 int32_t *out_mask, void *prev_out, void *truncated, float threshold, int activation,
                 int truncation_mode, int dtype, void *stream) {
+    dc::kernel_log_reset();
     int rc = check_conv("dc_conv_act", g, input, filter, out, mask, out_mask, dtype, false);
     if (rc != DC_OK) return rc;
     DC_REQUIRE_ALIGNED("dc_conv_act", packed_filter, 16);
@@ -186,6 +203,7 @@ int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filt
                 const void *bias, const int32_t *mask, const void *residual,
                 const int32_t *mask_residual, void *out, int32_t *out_mask, float weight_residual,
                 float weight_conv, int dtype, void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_conv_add");
     int rc = check_geometry("dc_conv_add", g, false, false);
     if (rc != DC_OK) return rc;
@@ -219,6 +237,7 @@ int64_t dc_packed_filter_bytes(const dc_geometry *g, int dtype, int transposed) 
 
 int dc_pack_filter(const dc_geometry *g, const void *filter, void *packed_filter, int dtype,
                    int transposed, void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_pack_filter");
     if (g == nullptr) return fail(DC_ERR_NULL, "dc_pack_filter: geometry is NULL");
     if (dc_packed_filter_bytes(g, dtype, transposed) == 0)
@@ -234,6 +253,7 @@ int dc_pack_filter(const dc_geometry *g, const void *filter, void *packed_filter
 int dc_deconv(const dc_geometry *g, const void *input, const void *filter,
               const void *packed_filter, const void *bias, void *out, const int32_t *mask,
               int32_t *out_mask, int dtype, void *stream) {
+    dc::kernel_log_reset();
     int rc = check_conv("dc_deconv", g, input, filter, out, mask, out_mask, dtype, true);
     if (rc != DC_OK) return rc;
     DC_REQUIRE_ALIGNED("dc_deconv", packed_filter, 16);
@@ -244,6 +264,7 @@ int dc_deconv(const dc_geometry *g, const void *input, const void *filter,
 int dc_pool(const dc_geometry *g, const void *input, const void *prev_input, void *out,
             const int32_t *mask, int32_t *out_mask, int pooling_mode, int dtype,
             int global_out_dtype, void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_pool");
     int rc = check_geometry("dc_pool", g, false, true);
     if (rc != DC_OK) return rc;
@@ -274,6 +295,7 @@ int dc_pool(const dc_geometry *g, const void *input, const void *prev_input, voi
 int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_t *mask_a,
            const int32_t *mask_b, int32_t *mask_out, float weight_a, float weight_b, int activation,
            int dense_out, int32_t pixels, int32_t channels, int dtype, void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_add");
     int rc = check_pc("dc_add", pixels, channels);
     if (rc != DC_OK) return rc;
@@ -296,6 +318,7 @@ int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_
 
 int dc_densify(const void *delta, void *prev_out, void *out, const int32_t *mask, int32_t pixels,
                int32_t channels, int dtype, void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_densify");
     int rc = check_pc("dc_densify", pixels, channels);
     if (rc != DC_OK) return rc;
@@ -312,6 +335,7 @@ int dc_densify(const void *delta, void *prev_out, void *out, const int32_t *mask
 
 int dc_add_to_dense(void *a, void *b, const int32_t *mask_a, int activation, int32_t pixels,
                     int32_t channels, int dtype, void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_add_to_dense");
     int rc = check_pc("dc_add_to_dense", pixels, channels);
     if (rc != DC_OK) return rc;
@@ -329,6 +353,7 @@ int dc_add_to_dense(void *a, void *b, const int32_t *mask_a, int activation, int
 int dc_upsample(const void *input, void *out, const int32_t *mask_in, int32_t *mask_out,
                 int32_t batch, int32_t in_h, int32_t in_w, int32_t channels, int32_t scale,
                 int dtype, void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_upsample");
     if (batch <= 0 || in_h <= 0 || in_w <= 0 || channels <= 0 || scale <= 0)
         return fail(DC_ERR_SHAPE, "dc_upsample: non-positive dimension");
@@ -347,6 +372,7 @@ int dc_upsample(const void *input, void *out, const int32_t *mask_in, int32_t *m
 int dc_concat(const void *a, const void *b, void *out, const int32_t *mask_a, const int32_t *mask_b,
               int32_t *mask_out, int32_t pixels, int32_t channels_a, int32_t channels_b, int dtype,
               void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_concat");
     int rc = check_pc("dc_concat", pixels, channels_a);
     if (rc != DC_OK) return rc;
@@ -368,6 +394,7 @@ int dc_concat(const void *a, const void *b, void *out, const int32_t *mask_a, co
 int dc_mul_add(const void *input, const int32_t *mask, void *out, int32_t *mask_out,
                const void *scale, const void *bias, int32_t pixels, int32_t channels, int dtype,
                void *stream) {
+    dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_mul_add");
     int rc = check_pc("dc_mul_add", pixels, channels);
     if (rc != DC_OK) return rc;

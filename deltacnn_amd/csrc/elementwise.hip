@@ -473,6 +473,7 @@ hipError_t sparsify_t(const T *in, T *prev, T *delta, int32_t *mask, float thr, 
         int G = pick_group(nvec, P, 4);
         int iters = ceil_div(nvec, G);
         GroupLaunch L(P, G);
+        note_kernel("sparsify_vec_kernel");
         switch (iters) {
             case 1: sparsify_vec_kernel<T, 1><<<L.grid, L.block, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
             case 2: sparsify_vec_kernel<T, 2><<<L.grid, L.block, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge); break;
@@ -481,6 +482,7 @@ hipError_t sparsify_t(const T *in, T *prev, T *delta, int32_t *mask, float thr, 
     } else {
         int G = group_lanes(C, 4);
         GroupLaunch L(P, G);
+        note_kernel("sparsify_gen_kernel");
         sparsify_gen_kernel<T><<<L.grid, L.block, 0, s>>>(in, prev, delta, mask, thr, P, C, G, ge);
     }
     return hipGetLastError();
@@ -489,6 +491,7 @@ hipError_t sparsify_t(const T *in, T *prev, T *delta, int32_t *mask, float thr, 
 template <typename T, int ITERS>
 void act_trunc_launch(dim3 grid, int block, hipStream_t s, T *delta, T *prev, T *trunc, int32_t *mask,
                       float thr, int act, int mode, int P, int C, int lg) {
+    note_kernel("act_trunc_vec_kernel");
     // eager loads where reading the whole map, active or not, costs little
     const bool eager = (int64_t)P * C * (int64_t)sizeof(T) <= (1 << 20);
 #define DC_AT(A)                                                                                                    \
@@ -515,9 +518,11 @@ hipError_t act_trunc_t(T *delta, T *prev, T *trunc, int32_t *mask, float thr, in
     if (mode < 0) {
         if (can_vec<T>(C, {delta, prev})) {
             GroupLaunch L(P, pick_group(C / N, P, 4));
+            note_kernel("accumulate_kernel");
             accumulate_kernel<T, N><<<L.grid, L.block, 0, s>>>(delta, prev, mask, act, P, C, L.lg);
         } else {
             GroupLaunch L(P, group_lanes(C, 1));
+            note_kernel("accumulate_kernel");
             accumulate_kernel<T, 1><<<L.grid, L.block, 0, s>>>(delta, prev, mask, act, P, C, L.lg);
         }
         return hipGetLastError();
@@ -534,6 +539,7 @@ hipError_t act_trunc_t(T *delta, T *prev, T *trunc, int32_t *mask, float thr, in
         }
     } else {
         GroupLaunch L(P, group_lanes(C, 1));
+        note_kernel("act_trunc_gen_kernel");
         act_trunc_gen_kernel<T><<<L.grid, L.block, 0, s>>>(delta, prev, trunc, mask, thr, act, mode, P, C, L.lg);
     }
     return hipGetLastError();
@@ -547,6 +553,7 @@ hipError_t add_t(const T *a, const T *b, T *prev, T *out, const int32_t *ma, con
     if (act < 0) act = 0;
     const bool vec = can_vec<T>(C, {a, b, prev, out});
     GroupLaunch L(P, vec ? pick_group(C / N, P, 4) : group_lanes(C, 1));
+    note_kernel(dense_out ? "add_dense_kernel" : "add_kernel");
     if (dense_out) {
         if (vec) add_dense_kernel<T, N><<<L.grid, L.block, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, L.lg);
         else add_dense_kernel<T, 1><<<L.grid, L.block, 0, s>>>(a, b, prev, out, ma, mb, wa, wb, act, P, C, L.lg);
@@ -580,9 +587,11 @@ hipError_t densify_t(const T *delta, T *prev, T *out, const int32_t *mask, int P
     constexpr int N = Vec16<T>::N;
     if (can_vec<T>(C, {delta, prev, out})) {
         GroupLaunch L(P, pick_group(C / N, P, 4));
+        note_kernel("densify_kernel");
         densify_kernel<T, N><<<L.grid, L.block, 0, s>>>(delta, prev, out, mask, P, C, L.lg);
     } else {
         GroupLaunch L(P, group_lanes(C, 1));
+        note_kernel("densify_kernel");
         densify_kernel<T, 1><<<L.grid, L.block, 0, s>>>(delta, prev, out, mask, P, C, L.lg);
     }
     return hipGetLastError();
@@ -608,6 +617,7 @@ hipError_t add_to_dense_t(T *a, T *b, const int32_t *ma, int act, int P, int C, 
     constexpr int N = Vec16<T>::N;
     const bool vec = can_vec<T>(C, {a, b});
     GroupLaunch L(P, vec ? pick_group(C / N, P, 4) : group_lanes(C, 1));
+    note_kernel(act > 0 ? "add_to_dense_act_kernel" : "add_to_dense_kernel");
     if (act > 0) {
         if (vec) add_to_dense_act_kernel<T, N><<<L.grid, L.block, 0, s>>>(a, b, ma, act, P, C, L.lg);
         else add_to_dense_act_kernel<T, 1><<<L.grid, L.block, 0, s>>>(a, b, ma, act, P, C, L.lg);
@@ -624,9 +634,11 @@ hipError_t upsample_t(const T *in, T *out, const int32_t *mi, int32_t *mo, int B
     int P = B * H * W;
     if (can_vec<T>(C, {in, out})) {
         GroupLaunch L(P, pick_group(C / N, P, 4));
+        note_kernel("upsample_kernel");
         upsample_kernel<T, N><<<L.grid, L.block, 0, s>>>(in, out, mi, mo, B, H, W, C, S, L.lg);
     } else {
         GroupLaunch L(P, group_lanes(C, 1));
+        note_kernel("upsample_kernel");
         upsample_kernel<T, 1><<<L.grid, L.block, 0, s>>>(in, out, mi, mo, B, H, W, C, S, L.lg);
     }
     return hipGetLastError();
@@ -638,9 +650,11 @@ hipError_t concat_t(const T *a, const T *b, T *out, const int32_t *ma, const int
     int Cm = Ca > Cb ? Ca : Cb;
     if (Ca % N == 0 && Cb % N == 0 && can_vec<T>(Ca, {a, b, out})) {
         GroupLaunch L(P, pick_group(Cm / N, P, 4));
+        note_kernel("concat_kernel");
         concat_kernel<T, N><<<L.grid, L.block, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, L.lg);
     } else {
         GroupLaunch L(P, group_lanes(Cm, 1));
+        note_kernel("concat_kernel");
         concat_kernel<T, 1><<<L.grid, L.block, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, L.lg);
     }
     return hipGetLastError();
@@ -651,9 +665,11 @@ hipError_t mul_add_t(const T *in, const int32_t *mask, T *out, int32_t *mo, cons
     constexpr int N = Vec16<T>::N;
     if (can_vec<T>(C, {in, out, scale, bias})) {
         GroupLaunch L(P, pick_group(C / N, P, 4));
+        note_kernel("mul_add_kernel");
         mul_add_kernel<T, N><<<L.grid, L.block, 0, s>>>(in, mask, out, mo, scale, bias, P, C, L.lg);
     } else {
         GroupLaunch L(P, group_lanes(C, 1));
+        note_kernel("mul_add_kernel");
         mul_add_kernel<T, 1><<<L.grid, L.block, 0, s>>>(in, mask, out, mo, scale, bias, P, C, L.lg);
     }
     return hipGetLastError();

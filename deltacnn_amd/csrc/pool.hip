@@ -250,6 +250,7 @@ hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, c
         const bool whole = g.kernel_h == g.in_h && g.kernel_w == g.in_w && g.pad_top == 0 && g.pad_left == 0 &&
                            g.pad_bottom == 0 && g.pad_right == 0 && g.dilation_h == 1 && g.dilation_w == 1;
         if (whole && g.in_c % N == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)prev & 15) == 0) {
+            note_kernel("pool_global_vec_kernel");
             dim3 vgrid(ceil_div(g.in_c / N, 8), g.batch);
             const int npx = g.in_h * g.in_w;
 #define DC_PG(OT, MX) pool_global_vec_kernel<T, OT, MX><<<vgrid, 256, 0, s>>>(npx, g.in_c, in, prev, (OT *)out, mask, out_mask)
@@ -262,6 +263,7 @@ hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, c
             return hipGetLastError();
         }
         if (!out_f32) return hipErrorInvalidValue;  // checked by the caller: cannot happen
+        note_kernel("pool_global_kernel");
         dim3 grid(ceil_div(g.in_c, WAVE), g.batch);
         if (mode == DC_POOL_MAX)
             pool_global_kernel<T, true><<<grid, 256, 0, s>>>(p, q, in, prev, (float *)out, mask, out_mask);
@@ -269,6 +271,7 @@ hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, c
             pool_global_kernel<T, false><<<grid, 256, 0, s>>>(p, q, in, prev, (float *)out, mask, out_mask);
         return hipGetLastError();
     }
+    note_kernel("pool_window_kernel");
     dim3 grid(ceil_div(g.out_w, TILE), ceil_div(g.out_h, TILE), g.batch);
     const bool vec = g.in_c % N == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
                      ((uintptr_t)prev & 15) == 0;

@@ -29,6 +29,12 @@ namespace {
 
 struct PwP {
     int P, Ci, Co, ci_p, co_tiles;
+    // XCD-aware launch (xcd != 0): the grid is one-dimensional, nx * round_up(ny, 8) workgroups.
+    // The hardware deals workgroups to the 8 XCDs round-robin by linear id, each XCD has its own
+    // L2; workgroup L takes channel group (L % 8) + 8 * ((L / 8) / nx) and pixel tile
+    // (L / 8) % nx, so all pixel tiles of a channel group run on ONE XCD and its filter
+    // fragments are fetched into one L2 instead of up to eight.
+    int xcd, nx, ny;
 };
 
 // ADD fuses the residual sum of a DCAdd layer behind the convolution: with a = residual delta
@@ -66,7 +72,14 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
     const int l16 = lane & 15, kq = lane >> 4;
     const int kw = wave % KW, tw = wave / KW, cw = tw % CBW, nw = tw / CBW;
     const int ksteps = p.ci_p >> 5;
-    const int pbase = blockIdx.x * PXW;
+    int bx = blockIdx.x, by = blockIdx.y;
+    if (p.xcd) {
+        const int slot = blockIdx.x >> 3;
+        by = (blockIdx.x & 7) + 8 * (slot / p.nx);
+        bx = slot % p.nx;
+        if (by >= p.ny) return;  // padding of the channel groups to a multiple of 8
+    }
+    const int pbase = bx * PXW;
 
     // the mask words of the workgroup's pixels, one per lane, together with the first chunk
     // of filter fragments (which do not depend on the masks)
@@ -75,7 +88,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
     const int mword = mask[min(mp, p.P - 1)];
     int rword = 0;
     if (ADD) rword = rp.mask[min(mp, p.P - 1)];
-    const int ct0 = (blockIdx.y * CBW + cw) * R;
+    const int ct0 = (by * CBW + cw) * R;
     const half_t *wrow[R];  // fragment order: one contiguous KB per (channel tile, step)
 #pragma unroll
     for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
@@ -107,7 +120,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
     const uint64_t bm = ballot(mine && mword != 0);
     const uint64_t br = ADD ? ballot(mine && rword != 0) : 0;
     const uint64_t bo = bm | br;
-    if (blockIdx.y == 0 && wave == 0 && mine) out_mask[mp] = int((bo >> lane) & 1);
+    if (by == 0 && wave == 0 && mine) out_mask[mp] = int((bo >> lane) & 1);
     if (bo == 0) return;  // the same for every wavefront of the workgroup
 
     // tiles this wavefront finishes: all of its own (KW == 1) or tiles kw, kw + KW, ... of
@@ -465,6 +478,8 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     p.Co = g.out_c;
     p.ci_p = (g.in_c + 31) / 32 * 32;
     p.co_tiles = ceil_div(g.out_c, 16);
+    p.xcd = 0;
+    p.nx = p.ny = 0;
     const int ksteps = p.ci_p / 32;
     *epilogue_done = false;
     const auto al8 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 7u) == 0; };
@@ -478,6 +493,7 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     if (fusable && ksteps <= PW_FUSED_MAX_STEPS && p.P >= 512) {
         dim3 grid(ceil_div(p.P, 16));
         const int act = epi->act < 0 ? 0 : epi->act;
+        note_kernel("pw_act_mfma_kernel");
         // as many wavefronts as channel tiles, up to 16; then several tiles per wavefront
         const int nw = p.co_tiles <= 4 ? 4 : p.co_tiles <= 8 ? 8 : 16;
         const int ctw = ceil_div(p.co_tiles, nw);
@@ -502,9 +518,14 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     ResP rp{nullptr, nullptr, 1.f, 1.f};
     if (res != nullptr) rp = ResP{(const half_t *)res->values, res->mask, res->wa, res->wb};
     const int cfg = pick_config(p, ksteps);
+    note_kernel("pw_mfma_kernel");
 #define DC_PW_S(KW, CBW, NBW, R, NTW, EA, SS)                                                        \
     do {                                                                                             \
-        dim3 grid(ceil_div(p.P, NBW * NTW * 16), ceil_div(p.co_tiles, CBW * R));                     \
+        p.nx = ceil_div(p.P, NBW * NTW * 16);                                                        \
+        p.ny = ceil_div(p.co_tiles, CBW * R);                                                        \
+        /* filter bytes dominate and the plain order would spread a channel group over XCDs */      \
+        p.xcd = (p.nx % 8 != 0 && p.ny > 1 && (int64_t)p.ci_p * p.Co > (int64_t)p.P * p.Ci) ? 1 : 0; \
+        dim3 grid(p.xcd ? p.nx * ((p.ny + 7) / 8 * 8) : p.nx, p.xcd ? 1 : p.ny);                     \
         if (res != nullptr)                                                                          \
             pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, true, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(  \
                 p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \

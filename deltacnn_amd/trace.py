@@ -9,7 +9,10 @@ m = 4-byte mask word, P pixels, n_x = number of active pixels of mask x):
   densify            R = P*m + n*2*C*s                    W = n*C*s   (+ dense copy: R += (P-n)*C*s, W += P*C*s)
   add                R = 2*P*m + (n_a+n_b)*C*s [+n_out*C*s]  W = n_out*C*s [+n_out*C*s] + P*m
   conv / deconv      R = P_in*m + n_in*Cin*s + K*K*(Cin/g)*Cout*s   W = n_out*Cout*s + P_out*m
-                     (conv_act: the same; conv_add: + P_out*m + n_res*Cout*s for the residual)
+                     (conv_add: + P_out*m + n_res*Cout*s for the residual; conv_act in one launch:
+                     + the activate_truncate state traffic R += n_mid*2*Cout*s,
+                     W += n_out*2*Cout*s + (n_mid-n_out)*Cout*s, n_mid = updated outputs before
+                     truncation; conv_act in two launches: a conv row and an activate_truncate row)
                      flops = 2*(Cin/g)*Cout*N_pairs, N_pairs = sum over updated outputs of the
                      active inputs in their window (computed exactly from the masks)
   pool               R = P_in*m + n_in*C*s (x2 for max)   W = n_out*C*s + P_out*m
@@ -24,6 +27,8 @@ from collections import defaultdict
 
 import torch
 import torch.nn.functional as F
+
+from . import _lib
 
 
 class Tracer:
@@ -42,12 +47,13 @@ class Tracer:
         rec["n_in"] = self._count(meta.get("in_mask"))
         rec["n_in_b"] = self._count(meta.get("in_mask_b"))
         if self.count_pairs and op in ("conv", "deconv", "conv_act", "conv_add"):
-            rec["pairs"] = self._pairs(meta["g"], meta["in_mask"], op == "deconv")
+            rec["pairs"], rec["n_mid"] = self._pairs(meta["g"], meta["in_mask"], op == "deconv")
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
         rc = fn(*args)
         end.record()
         rec["events"] = (start, end)
+        rec["kernels"] = _lib.load().dc_last_kernels().decode().split("+")
         rec["n_out"] = self._count(meta.get("out_mask"))
         rec["call"] = (fn, args)
         self.records.append(rec)
@@ -59,7 +65,8 @@ class Tracer:
         """Device time per call of every recorded call, free of host and event overhead: the
         call is captured `repeats` times back to back into a HIP graph (each launch depends on
         the previous one, as inside a frame) and the graph is replayed `rounds` times between
-        two events.  Returns microseconds per call, one per record.
+        two events.  Returns microseconds per call, one per record; a call that launches two
+        kernels (convolution, then activation/truncation) also gets ``split_us`` per kernel.
 
         Every call has to see the masks of the traced frame, so
           * records are replayed last to first: a replay only disturbs its own outputs, whose
@@ -100,13 +107,21 @@ class Tracer:
                 times[i] = max(timed([pcall, call]) - timed([pcall]), 0.0)
             else:
                 times[i] = timed([call])
+            if rec["op"] == "conv_act" and len(rec["kernels"]) == 2:
+                # the convolution launch of a two-launch call on its own: dc_conv with the same
+                # operands runs the same kernel; the activation kernel gets the remainder
+                a = rec["call"][1]
+                conv_only = ("conv", _lib.load().dc_conv, a[:8] + a[13:])
+                t_conv = min(timed([conv_only]), times[i])
+                rec["split_us"] = [t_conv, times[i] - t_conv]
         return times
 
     @staticmethod
     def _pairs(g, mask, transposed):
         """N_pairs: number of (updated output pixel, active input pixel in its window) pairs.
         Every active input pixel reaches each output pixel of its footprint, and each of
-        those outputs is updated, so N_pairs = sum over taps of the shifted mask."""
+        those outputs is updated, so N_pairs = sum over taps of the shifted mask.  Also returns
+        the number of updated output pixels (the population of the dilated mask)."""
         m = (mask != 0).float()
         ones = torch.ones(1, 1, g.kernel_h, g.kernel_w, device=m.device)
         if transposed:
@@ -115,10 +130,12 @@ class Tracer:
         else:
             mp = F.pad(m, (g.pad_left, g.pad_right, g.pad_top, g.pad_bottom))
             cnt = F.conv2d(mp, ones, stride=(g.stride_h, g.stride_w), dilation=(g.dilation_h, g.dilation_w))
-        return cnt.sum()
+        return cnt.sum(), (cnt > 0).sum()
 
     def finish(self):
-        """Synchronise and turn the records into dicts with ``ms``, ``bytes``, ``flops``."""
+        """Synchronise and turn the records into one dict per KERNEL LAUNCH with ``kernel`` (the
+        HIP kernel's name as reported by the library), ``call`` (the library operator),
+        ``ms``, ``bytes``, ``flops``."""
         torch.cuda.synchronize()
         out = []
         for r in self.records:
@@ -128,31 +145,42 @@ class Tracer:
             n_out = None if r["n_out"] is None else int(r["n_out"])
             s, m = meta["esize"], 4
             flops = 0
+            extra = None  # second kernel of a two-launch call
+            ms = r.get("ms", r["events"][0].elapsed_time(r["events"][1]))
             if op in ("conv", "deconv", "conv_act", "conv_add"):
                 g = meta["g"]
                 p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
                 wbytes = g.kernel_h * g.kernel_w * (g.in_c // g.groups) * g.out_c * s
+                n_mid = int(r["n_mid"]) if "n_mid" in r else n_out  # updated outputs before truncation
+                two = op == "conv_act" and len(r["kernels"]) == 2
                 rd = p_in * m + n_in * g.in_c * s + wbytes
-                wr = n_out * g.out_c * s + p_out * m
+                wr = (n_mid if two else n_out) * g.out_c * s + p_out * m
                 if op == "conv_add":  # + the residual operand of the fused add
                     rd += p_out * m + n_in_b * g.out_c * s
+                if op == "conv_act" and not two:  # fused epilogue: cached state of every updated output
+                    rd += n_mid * 2 * g.out_c * s
+                    wr += n_out * 2 * g.out_c * s + (n_mid - n_out) * g.out_c * s
                 if "pairs" in r:
                     flops = 2 * (g.in_c // g.groups) * g.out_c * int(r["pairs"])
-                dw = g.groups > 1
-                kind = ("dw" if dw else "pw" if g.kernel_h == 1 and g.kernel_w == 1 else "kxk")
-                name = f"{op}_{kind}{'_mfma' if meta.get('mfma') and not dw else ''}"
                 shape = f"{g.in_c}->{g.out_c} k{g.kernel_h} s{g.stride_h} @{g.in_h}x{g.in_w}"
                 dens = (n_in / p_in, n_out / p_out)
+                if two:
+                    t_conv, t_act = r.get("split_us", [ms * 1e3 / 2, ms * 1e3 / 2])
+                    ms = t_conv * 1e-3
+                    C = g.out_c
+                    extra = {"kernel": r["kernels"][1], "call": op, "shape": f"C{C} P{p_out}", "ms": t_act * 1e-3,
+                             "bytes": p_out * m + n_mid * 3 * C * s + n_out * 3 * C * s + (n_mid - n_out) * (C * s + m),
+                             "flops": 0, "density_in": n_mid / p_out, "density_out": n_out / p_out}
             elif op == "pool":
                 g = meta["g"]
                 p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
                 rd = p_in * m + n_in * g.in_c * s * (2 if meta["mode"] == 0 else 1)
                 wr = n_out * g.in_c * s + p_out * m
-                name, shape = "pool", f"C{g.in_c} k{g.kernel_h} @{g.in_h}x{g.in_w}"
+                shape = f"C{g.in_c} k{g.kernel_h} @{g.in_h}x{g.in_w}"
                 dens = (n_in / p_in, n_out / p_out)
             else:
                 P, C = meta["P"], meta["C"]
-                name, shape = op, f"C{C} P{P}"
+                shape = f"C{C} P{P}"
                 if op == "sparsify":
                     rd, wr = 2 * P * C * s, 2 * n_out * C * s + P * m
                     dens = (1.0, n_out / P)
@@ -167,9 +195,9 @@ class Tracer:
                     dens = (n_in / P, n_in / P)
                 elif op == "add":
                     n_o = n_out if n_out is not None else P
-                    extra = n_o * C * s if meta["with_prev"] else 0
-                    rd = 2 * P * m + (n_in + n_in_b) * C * s + extra
-                    wr = n_o * C * s + extra + P * m
+                    ext = n_o * C * s if meta["with_prev"] else 0
+                    rd = 2 * P * m + (n_in + n_in_b) * C * s + ext
+                    wr = n_o * C * s + ext + P * m
                     dens = ((n_in + n_in_b) / (2 * P), n_o / P)
                 elif op == "add_to_dense":
                     rd, wr = P * m + 2 * n_in * C * s, n_in * C * s
@@ -186,8 +214,10 @@ class Tracer:
                 else:  # mul_add
                     rd, wr = P * m + n_in * C * s + C * s, n_in * C * s
                     dens = (n_in / P, n_in / P)
-            out.append({"kernel": name, "shape": shape, "ms": r.get("ms", r["events"][0].elapsed_time(r["events"][1])),
+            out.append({"kernel": r["kernels"][0] or op, "call": op, "shape": shape, "ms": ms,
                         "bytes": rd + wr, "flops": flops, "density_in": dens[0], "density_out": dens[1]})
+            if extra is not None:
+                out.append(extra)
         self.records = []
         return out
 

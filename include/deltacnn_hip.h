@@ -68,6 +68,11 @@ typedef struct dc_geometry {
 const char *dc_version(void);
 const char *dc_last_error(void);
 
+/* Names of the kernels that the calling thread's last entry point launched, '+'-separated
+ * (e.g. "pw_mfma_kernel+act_trunc_vec_kernel"); empty if it launched nothing.  For tracing
+ * tools; no counterpart in the reference. */
+const char *dc_last_kernels(void);
+
 /* Replaces deltacnn_prepare_diff_mask_wrapper (conv_torch_wrapper.cpp:347-384).
  * delta = input - prev_input; active pixels get delta and prev_input := input on all
  * channels; mask is written for every pixel. */
