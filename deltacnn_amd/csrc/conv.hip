@@ -419,17 +419,24 @@ conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
 }
 
 // ------------------------------------------------------------------------------------ MFMA
-// Implicit GEMM on v_mfma_f32_16x16x32_f16: rows = 16 output channels (packed filter rows),
-// columns = 16 compacted pixels (NHWC input rows), reduction over (tap, input channel) in
-// steps of 32.  A wavefront keeps up to four pixel sub-tiles (64 pixels) in accumulators, so a
-// filter fragment is loaded once per step and reused four times.
-//   KSPLIT = false: the four wavefronts of a workgroup take four different channel tiles.
-//   KSPLIT = true : the workgroup owns one channel tile and its wavefronts split the reduction
-//                   steps round-robin; partial accumulators meet in LDS.  This is what keeps
-//                   deep layers with tiny maps (7x7 x 960 channels) from being one long serial
-//                   chain in a handful of wavefronts.
-template <bool TR, bool KSPLIT>
-__global__ void __launch_bounds__(256)
+// Implicit GEMM on v_mfma_f32_16x16x32_f16 for any kernel size / stride / dilation and for the
+// transposed convolution: rows = 16 output channels (packed filter, fragment order), columns =
+// 16 compacted output pixels of the 8x8 tile, reduction over (tap, input channel) in steps of
+// 32, step index s = tap * ksteps + channel step (the packed filter is linear in s).
+//
+//   * after the mask phase the workgroup builds a table in LDS: for every (tap, compacted
+//     pixel) the index of the input pixel it reads, or -1 if that input is out of bounds or
+//     inactive; taps that no pixel of the tile uses are skipped altogether;
+//   * a wavefront accumulates R channel tiles x 4 pixel tiles, so a reduction step costs
+//     R + 4 fragment loads for 4 * R MFMAs; the KW wavefronts of a workgroup split the steps
+//     round-robin and their partial sums meet in LDS (added in ascending wavefront order);
+//   * all fragment loads of S steps are issued unconditionally (clamped addresses) before the
+//     first MFMA of the chunk; input fragments of invalid (tap, pixel) pairs are zeroed by
+//     selection afterwards -- unlike the pointwise case they would reach valid outputs.
+constexpr int MFMA_MAX_TAPS = 49;
+
+template <bool TR, int KW, int R, int S>
+__global__ void __launch_bounds__(KW * WAVE)
 conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                  const half_t *__restrict__ bias, half_t *__restrict__ out,
                  const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, int co_blocks,
@@ -437,144 +444,136 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
     constexpr int NT = 4;
     __shared__ int s_list[TILE_PX];
     __shared__ int s_n;
-    __shared__ float4_t s_red[KSPLIT ? 4 * NT * WAVE : 1];
+    __shared__ int s_src[MFMA_MAX_TAPS * TILE_PX];
+    __shared__ unsigned long long s_taps;
+    __shared__ float4_t s_red[KW > 1 ? KW * NT * WAVE : 1];
     const int b = blockIdx.z / co_blocks;
     const int cb = blockIdx.z % co_blocks;
+    if (threadIdx.x == 0) s_taps = 0;
     const int n = tile_mask_phase<TR>(p, mask, out_mask, b, blockIdx.y * TILE, blockIdx.x * TILE,
                                       cb == 0, s_list, &s_n);
     if (n == 0) return;
 
-    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int kw = threadIdx.x / WAVE, lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;  // row / column inside a tile, k-quarter
     const int K2 = p.Kh * p.Kw;
     const int n_tiles = (n + 15) >> 4;
     const int co_tiles = (p.Co + 15) >> 4;
-    const int ct = KSPLIT ? cb : cb * 4 + wave;
-    if (!KSPLIT && ct >= co_tiles) return;
     const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
     const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
-    const bool pointwise = !TR && K2 == 1 && p.sh == 1 && p.sw == 1 && p.pt == 0 && p.pl == 0;
 
-    int oy[NT], ox[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        const int pix = nt * 16 + l16;
-        const int code = pix < n ? s_list[pix] : -1;
-        oy[nt] = code < 0 ? -1 : code >> 16;
-        ox[nt] = code & 0xffff;
+    // source table: entry (tap, pixel) for all taps and the 64 pixel slots of the tile
+    unsigned long long used = 0;
+    for (int e = threadIdx.x; e < K2 * TILE_PX; e += KW * WAVE) {
+        const int tap = e >> 6, pix = e & 63;
+        int src = -1;
+        if (pix < n) {
+            const int code = s_list[pix];
+            const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
+            int iy, ix;
+            if (tap_src<TR>(code >> 16, ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
+                tap_src<TR>(code & 0xffff, kx, p.sw, p.dw, p.pl, p.Wi, ix) && mb[iy * p.Wi + ix] != 0)
+                src = iy * p.Wi + ix;
+        }
+        s_src[e] = src;
+        if (src >= 0) used |= 1ull << tap;
     }
-    float4_t acc[NT];
+    // one LDS atomic per wavefront: OR of the lanes' tap sets
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) acc[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int o = 1; o < WAVE; o <<= 1) used |= __shfl_xor(used, o, WAVE);
+    if (lane == 0 && used != 0) atomicOr(&s_taps, used);
+    __syncthreads();
+    const unsigned long long taps = s_taps;
 
+    float4_t acc[R][NT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[r][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
     const int ksteps = ci_p >> 5;
-    const half_t *wfrag = wp + (size_t)ct * K2 * ksteps * 512 + lane * 8;  // fragment order, see pack_filter_kernel
     const int total = K2 * ksteps;
-    const int kvalid = kq * 8;  // this lane's channel offset inside a 32-wide step
-    const int first = KSPLIT ? wave : 0, stride = KSPLIT ? 4 : 1;
-    // Reduction steps are taken S at a time: all fragment loads of a chunk are issued before
-    // its first MFMA, so a chunk costs one memory round trip instead of S.
-    constexpr int S = 4;
-    int cur_tap = -1;
-    const half_t *xrow[NT];
-    bool xok[NT];
-    bool tap_used = false;
-    for (int s0 = first; s0 < total; s0 += S * stride) {
-        half8_t a[S], x[S][NT];
+    const half_t *wfrag[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
+        wfrag[r] = wp + (size_t)min(cb * R + r, co_tiles - 1) * total * 512 + lane * 8;
+
+    for (int s0 = kw; s0 < total; s0 += S * KW) {
+        half8_t a[S][R], x[S][NT];
+        int src[S][NT];
         bool use[S];
 #pragma unroll
         for (int i = 0; i < S; ++i) {
-            const int s = s0 + i * stride;
-            use[i] = false;
-            if (s < total) {
-                const int tap = s / ksteps;
-                const int k0 = (s - tap * ksteps) << 5;
-                if (tap != cur_tap) {
-                    cur_tap = tap;
-                    const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
-                    bool any = false;
+            const int s = min(s0 + i * KW, total - 1);
+            const int tap = s / ksteps;
+            const int k = min(((s - tap * ksteps) << 5) + kq * 8, p.Ci - 8);
+            use[i] = s0 + i * KW < total && ((taps >> tap) & 1ull);  // wave-uniform
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        int ipix = -1;
-                        if (oy[nt] >= 0) {
-                            if (pointwise) {
-                                ipix = oy[nt] * p.Wi + ox[nt];
-                            } else {
-                                int iy, ix;
-                                if (tap_src<TR>(oy[nt], ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
-                                    tap_src<TR>(ox[nt], kx, p.sw, p.dw, p.pl, p.Wi, ix) &&
-                                    mb[iy * p.Wi + ix] != 0)
-                                    ipix = iy * p.Wi + ix;
-                            }
-                        }
-                        xok[nt] = ipix >= 0;
-                        any |= xok[nt];
-                        xrow[nt] = inb + (size_t)(ipix < 0 ? 0 : ipix) * p.Ci + kvalid;
-                    }
-                    tap_used = ballot(any) != 0;  // does any pixel of this tile use the tap?
-                }
-                use[i] = tap_used;
-                if (tap_used) {
-                    a[i] = *reinterpret_cast<const half8_t *>(wfrag + ((size_t)tap * ksteps + (k0 >> 5)) * 512);
-                    const bool kin = k0 + kvalid < p.Ci;
+            for (int r = 0; r < R; ++r)
+                a[i][r] = *reinterpret_cast<const half8_t *>(wfrag[r] + (size_t)s * 512);
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        x[i][nt] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-                        if (nt < n_tiles && xok[nt] && kin)
-                            x[i][nt] = *reinterpret_cast<const half8_t *>(xrow[nt] + k0);
-                    }
-                }
+            for (int nt = 0; nt < NT; ++nt) {
+                src[i][nt] = s_src[(tap << 6) + nt * 16 + l16];
+                x[i][nt] = *reinterpret_cast<const half8_t *>(inb + (size_t)max(src[i][nt], 0) * p.Ci + k);
             }
         }
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             if (!use[i]) continue;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-                if (nt < n_tiles)
-                    acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i], x[i][nt], acc[nt], 0, 0, 0);
+            for (int nt = 0; nt < NT; ++nt) {
+                if (nt >= n_tiles) continue;  // wave-uniform
+                const half8_t xz = src[i][nt] >= 0 ? x[i][nt] : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    acc[r][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][r], xz, acc[r][nt], 0, 0, 0);
+            }
         }
     }
 
-    if (KSPLIT) {
+    // wavefront kw finishes pixel tiles kw, kw + KW, ... of every channel tile
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-            if (nt < n_tiles) s_red[(wave * NT + nt) * WAVE + lane] = acc[nt];
-        __syncthreads();
-        // wavefront w finishes pixel sub-tile w
-        if (wave >= n_tiles) return;
-        float4_t sum = s_red[(0 * NT + wave) * WAVE + lane];
+    for (int r = 0; r < R; ++r) {
+        if (KW > 1) {
+            if (r > 0) __syncthreads();
 #pragma unroll
-        for (int w = 1; w < 4; ++w) {
-            const float4_t v = s_red[(w * NT + wave) * WAVE + lane];
-            sum += v;
+            for (int nt = 0; nt < NT; ++nt) s_red[(kw * NT + nt) * WAVE + lane] = acc[r][nt];
+            __syncthreads();
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                if ((nt % KW) != kw) continue;
+                float4_t sum = s_red[nt * WAVE + lane];
+#pragma unroll
+                for (int q = 1; q < KW; ++q) sum += s_red[(q * NT + nt) * WAVE + lane];
+                acc[r][nt] = sum;
+            }
         }
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-            if (nt == wave) acc[nt] = sum;
-    }
-    // lane holds channels ct*16 + kq*4 + {0..3} of pixel (nt, l16)
-    const int co = ct * 16 + kq * 4;
-    float bv[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bias != nullptr) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (co + i < p.Co) bv[i] = float(bias[co + i]);
-    }
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        if (nt >= n_tiles || oy[nt] < 0) continue;
-        if (KSPLIT && nt != wave) continue;
-        half_t *o = out + (((size_t)b * p.Ho + oy[nt]) * p.Wo + ox[nt]) * p.Co + co;
-        if (co + 3 < p.Co && (p.Co & 3) == 0) {
-            half4_t r;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) r[i] = half_t(acc[nt][i] + bv[i]);
-            *reinterpret_cast<half4_t *>(o) = r;
-        } else {
+        const int ct = cb * R + r;
+        if (ct >= co_tiles) continue;
+        // lane holds channels ct*16 + kq*4 + {0..3} of pixel (nt, l16)
+        const int co = ct * 16 + kq * 4;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias != nullptr) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (co + i < p.Co) o[i] = half_t(acc[nt][i] + bv[i]);
+                if (co + i < p.Co) bv[i] = float(bias[co + i]);
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            if ((nt % KW) != kw && KW > 1) continue;
+            const int pix = nt * 16 + l16;
+            if (pix >= n) continue;
+            const int code = s_list[pix];
+            half_t *o = out + (((size_t)b * p.Ho + (code >> 16)) * p.Wo + (code & 0xffff)) * p.Co + co;
+            if (co + 3 < p.Co && (p.Co & 3) == 0) {
+                half4_t v;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] = half_t(acc[r][nt][i] + bv[i]);
+                *reinterpret_cast<half4_t *>(o) = v;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (co + i < p.Co) o[i] = half_t(acc[r][nt][i] + bv[i]);
+            }
         }
     }
 }
@@ -767,18 +766,33 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
         return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
                                         epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
     }
-    if (packed != nullptr && mfma_eligible(g, dtype)) {
+    if (packed != nullptr && mfma_eligible(g, dtype) && g.kernel_h * g.kernel_w <= MFMA_MAX_TAPS) {
         const int co_tiles = ceil_div(g.out_c, 16);
         const int ci_p = round_up(g.in_c, 32);
         const int steps = g.kernel_h * g.kernel_w * (ci_p / 32);
+        // channel tiles per wavefront: as many as keep at least ~2 workgroups per compute unit
+        int R = co_tiles >= 4 ? 4 : co_tiles >= 2 ? 2 : 1;
+        while (R > 1 && (int64_t)tx * ty * g.batch * ceil_div(co_tiles, R) < 512) R >>= 1;
         const bool ksplit = steps >= 8;
-        const int co_blocks = ksplit ? co_tiles : ceil_div(co_tiles, 4);
+        const int co_blocks = ceil_div(co_tiles, R);
         dim3 grid(tx, ty, g.batch * co_blocks);
         note_kernel("conv_mfma_kernel");
-#define DC_MFMA(TRF, KS) conv_mfma_kernel<TRF, KS><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, co_blocks, ci_p)
-        if (transposed) { if (ksplit) DC_MFMA(true, true); else DC_MFMA(true, false); }
-        else { if (ksplit) DC_MFMA(false, true); else DC_MFMA(false, false); }
+#define DC_MFMA_L(TRF, KWV, RV, SV) conv_mfma_kernel<TRF, KWV, RV, SV><<<grid, KWV * WAVE, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, co_blocks, ci_p)
+#define DC_MFMA(TRF)                                                                   \
+    do {                                                                               \
+        if (ksplit) {                                                                  \
+            if (R == 4) DC_MFMA_L(TRF, 4, 4, 2);                                       \
+            else if (R == 2) DC_MFMA_L(TRF, 4, 2, 2);                                  \
+            else DC_MFMA_L(TRF, 4, 1, 4);                                              \
+        } else {                                                                       \
+            if (R == 4) DC_MFMA_L(TRF, 1, 4, 2);                                       \
+            else if (R == 2) DC_MFMA_L(TRF, 1, 2, 2);                                  \
+            else DC_MFMA_L(TRF, 1, 1, 4);                                              \
+        }                                                                              \
+    } while (0)
+        if (transposed) DC_MFMA(true); else DC_MFMA(false);
 #undef DC_MFMA
+#undef DC_MFMA_L
     } else {
         dim3 grid(tx, ty, g.batch);
         note_kernel("conv_direct_kernel");
