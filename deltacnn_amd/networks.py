@@ -269,3 +269,257 @@ def fold_data_statistics(dense_model: nn.Module, frames: torch.Tensor) -> None:
         conv.weight.mul_((1.0 / std).to(conv.weight.dtype)[:, None, None, None])
         if conv.bias is not None:
             conv.bias.copy_((-mean / std).to(conv.bias.dtype))
+
+
+# ---------------------------------------------------------------------------- HRNet-W32
+def _conv_act(L, inp, oup, k=3, stride=1, act="relu"):
+    """conv + folded batch norm (+ activation): one biased convolution."""
+    return L.DCConv2d(inp, oup, k, stride, (k - 1) // 2, bias=True, activation=act)
+
+
+class _BasicBlock(nn.Module):
+    """Two 3x3 convolutions and a residual sum followed by ReLU."""
+    expansion = 1
+
+    def __init__(self, L, inp, planes, stride=1, project=False):
+        super().__init__()
+        self.conv1 = _conv_act(L, inp, planes, 3, stride)
+        self.conv2 = _conv_act(L, planes, planes, 3, 1, act=None)
+        self.project = _conv_act(L, inp, planes, 1, stride, act=None) if project else None
+        self.add = L.DCAdd(activation="relu")
+
+    def forward(self, x):
+        res = x if self.project is None else self.project(x)
+        return self.add(self.conv2(self.conv1(x)), res)
+
+
+class _Bottleneck(nn.Module):
+    """1x1 -> 3x3 -> 1x1 (x4 channels) and a residual sum followed by ReLU."""
+    expansion = 4
+
+    def __init__(self, L, inp, planes, stride=1, project=False):
+        super().__init__()
+        self.conv1 = _conv_act(L, inp, planes, 1)
+        self.conv2 = _conv_act(L, planes, planes, 3, stride)
+        self.conv3 = _conv_act(L, planes, planes * 4, 1, act=None)
+        self.project = _conv_act(L, inp, planes * 4, 1, stride, act=None) if project else None
+        self.add = L.DCAdd(activation="relu")
+
+    def forward(self, x):
+        res = x if self.project is None else self.project(x)
+        return self.add(self.conv3(self.conv2(self.conv1(x))), res)
+
+
+class _HRModule(nn.Module):
+    """Parallel branches of basic blocks followed by the multi-resolution exchange: every output
+    branch i sums all input branches j, brought to its resolution by strided 3x3 convolutions
+    (j < i) or a 1x1 convolution + nearest upsampling (j > i), then ReLU."""
+
+    def __init__(self, L, channels, blocks=4, multi_scale_output=True):
+        super().__init__()
+        n = len(channels)
+        self.branches = nn.ModuleList(
+            nn.Sequential(*[_BasicBlock(L, c, c) for _ in range(blocks)]) for c in channels)
+        n_out = n if multi_scale_output else 1
+        self.fuse = nn.ModuleList()
+        self.adds = nn.ModuleList()
+        for i in range(n_out):
+            row = nn.ModuleList()
+            for j in range(n):
+                if j == i:
+                    row.append(nn.Identity())
+                elif j > i:
+                    row.append(nn.Sequential(_conv_act(L, channels[j], channels[i], 1, act=None),
+                                             L.DCUpsamplingNearest2d(scale_factor=2 ** (j - i))))
+                else:
+                    steps = [_conv_act(L, channels[j], channels[j], 3, 2) for _ in range(i - j - 1)]
+                    steps.append(_conv_act(L, channels[j], channels[i], 3, 2, act=None))
+                    row.append(nn.Sequential(*steps))
+            self.fuse.append(row)
+            # n - 1 sums per output; the last one carries the ReLU
+            self.adds.append(nn.ModuleList(L.DCAdd(activation="relu" if k == n - 2 else None)
+                                           for k in range(n - 1)))
+
+    def forward(self, xs):
+        xs = [b(x) for b, x in zip(self.branches, xs)]
+        outs = []
+        for row, adds in zip(self.fuse, self.adds):
+            y = row[0](xs[0])
+            for j in range(1, len(xs)):
+                y = adds[j - 1](y, row[j](xs[j]))
+            outs.append(y)
+        return outs
+
+
+class HRNet(_Net):
+    """HRNet pose network (width 32 by default): stem of two strided 3x3 convolutions, a
+    bottleneck stage, then 1 / 4 / 3 exchange modules on 2 / 3 / 4 resolutions, and a 1x1 head
+    producing ``num_joints`` heat maps at 1/4 resolution.  Batch norm is folded."""
+
+    def __init__(self, L=_hip_layers, width=32, num_joints=17, modules=(1, 4, 3), blocks=4):
+        super().__init__()
+        c = [width, width * 2, width * 4, width * 8]
+        self.sparsify = L.DCSparsify()
+        self.stem = nn.Sequential(_conv_act(L, 3, 64, 3, 2), _conv_act(L, 64, 64, 3, 2))
+        self.layer1 = nn.Sequential(_Bottleneck(L, 64, 64, project=True),
+                                    *[_Bottleneck(L, 256, 64) for _ in range(3)])
+        self.transition1 = nn.ModuleList([_conv_act(L, 256, c[0], 3, 1), _conv_act(L, 256, c[1], 3, 2)])
+        self.stage2 = nn.ModuleList(_HRModule(L, c[:2], blocks) for _ in range(modules[0]))
+        self.transition2 = _conv_act(L, c[1], c[2], 3, 2)
+        self.stage3 = nn.ModuleList(_HRModule(L, c[:3], blocks) for _ in range(modules[1]))
+        self.transition3 = _conv_act(L, c[2], c[3], 3, 2)
+        self.stage4 = nn.ModuleList(_HRModule(L, c[:4], blocks, multi_scale_output=(k < modules[2] - 1))
+                                    for k in range(modules[2]))
+        self.final = L.DCConv2d(c[0], num_joints, 1, bias=True, dense_out=True)
+
+    def forward(self, x):
+        x = self.layer1(self.stem(self.sparsify(x)))
+        xs = [t(x) for t in self.transition1]
+        for m in self.stage2:
+            xs = m(xs)
+        xs.append(self.transition2(xs[-1]))
+        for m in self.stage3:
+            xs = m(xs)
+        xs.append(self.transition3(xs[-1]))
+        for m in self.stage4:
+            xs = m(xs)
+        return self.final(xs[0])
+
+
+# ------------------------------------------------------------------- DLA-34 + CenterNet head
+class _Root(nn.Module):
+    """1x1 convolution over the concatenated children of a tree node, + ReLU."""
+
+    def __init__(self, L, in_channels, out_channels, n_inputs):
+        super().__init__()
+        self.cats = nn.ModuleList(L.DCConcatenate() for _ in range(n_inputs - 1))
+        self.conv = _conv_act(L, in_channels, out_channels, 1)
+
+    def forward(self, xs):
+        y = xs[0]
+        for cat, x in zip(self.cats, xs[1:]):
+            y = cat(y, x)
+        return self.conv(y)
+
+
+class _Tree(nn.Module):
+    """Deep layer aggregation tree: two sub-trees (basic blocks at the leaves) whose outputs,
+    with the down-sampled input when ``level_root``, are aggregated by a root node."""
+
+    def __init__(self, L, levels, inp, oup, stride=1, level_root=False, root_dim=0, n_children=0):
+        super().__init__()
+        if root_dim == 0:
+            root_dim = 2 * oup
+        if level_root:
+            root_dim += inp
+        self.levels, self.level_root = levels, level_root
+        self.downsample = L.DCMaxPooling(stride, stride=stride) if stride > 1 else None
+        self.project = _conv_act(L, inp, oup, 1, act=None) if inp != oup else None
+        if levels == 1:
+            self.tree1 = _BasicBlockExt(L, inp, oup, stride)
+            self.tree2 = _BasicBlockExt(L, oup, oup, 1)
+            self.root = _Root(L, root_dim, oup, 2 + n_children + (1 if level_root else 0))
+        else:
+            self.tree1 = _Tree(L, levels - 1, inp, oup, stride, root_dim=0)
+            self.tree2 = _Tree(L, levels - 1, oup, oup, root_dim=root_dim + oup,
+                               n_children=n_children + (1 if level_root else 0) + 1)
+            self.root = None
+
+    def forward(self, x, residual=None, children=None):
+        children = [] if children is None else children
+        bottom = self.downsample(x) if self.downsample is not None else x
+        residual = self.project(bottom) if self.project is not None else bottom
+        if self.level_root:
+            children.append(bottom)
+        x1 = self.tree1(x, residual)
+        if self.levels == 1:
+            x2 = self.tree2(x1)
+            return self.root([x2, x1] + children)
+        children.append(x1)
+        return self.tree2(x1, children=children)
+
+
+class _BasicBlockExt(nn.Module):
+    """Basic block whose residual operand is handed in (the tree computes it once)."""
+
+    def __init__(self, L, inp, planes, stride=1):
+        super().__init__()
+        self.conv1 = _conv_act(L, inp, planes, 3, stride)
+        self.conv2 = _conv_act(L, planes, planes, 3, 1, act=None)
+        self.add = L.DCAdd(activation="relu")
+
+    def forward(self, x, residual=None, children=None):
+        residual = x if residual is None else residual
+        return self.add(self.conv2(self.conv1(x)), residual)
+
+
+class _IDAUp(nn.Module):
+    """Iterative aggregation: every deeper level is projected (3x3), up-sampled by a transposed
+    convolution (kernel 2f, stride f, padding f/2, dense groups) and merged (sum + 3x3 node)."""
+
+    def __init__(self, L, out_dim, channels, factors):
+        super().__init__()
+        self.proj, self.up, self.add, self.node = (nn.ModuleList() for _ in range(4))
+        for c, f in zip(channels[1:], factors[1:]):
+            self.proj.append(_conv_act(L, c, out_dim, 3))
+            self.up.append(L.DCConvTranspose2d(out_dim, out_dim, f * 2, stride=f, padding=f // 2, bias=False))
+            self.add.append(L.DCAdd())
+            self.node.append(_conv_act(L, out_dim, out_dim, 3))
+
+    def forward(self, layers, start, end):
+        for i in range(start + 1, end):
+            k = i - start - 1
+            up = self.up[k](self.proj[k](layers[i]))
+            layers[i] = self.node[k](self.add[k](up, layers[i - 1]))
+
+
+class DLA34CenterNet(_Net):
+    """DLA-34 backbone, DLA-up / IDA-up decoder at output stride 4 and three CenterNet heads
+    (heat map, size, offset).  The 7x7 stem has stride 1, tree nodes down-sample with 2x2
+    max-pooling, roots concatenate, the decoder up-samples with transposed convolutions
+    (kernel 4, stride 2, padding 1, groups 1).  Batch norm is folded."""
+
+    def __init__(self, L=_hip_layers, num_classes=80, head_conv=256,
+                 channels=(16, 32, 64, 128, 256, 512)):
+        super().__init__()
+        c = list(channels)
+        self.sparsify = L.DCSparsify()
+        self.base_layer = _conv_act(L, 3, c[0], 7)
+        self.level0 = _conv_act(L, c[0], c[0], 3)
+        self.level1 = _conv_act(L, c[0], c[1], 3, 2)
+        self.level2 = _Tree(L, 1, c[1], c[2], 2)
+        self.level3 = _Tree(L, 2, c[2], c[3], 2, level_root=True)
+        self.level4 = _Tree(L, 2, c[3], c[4], 2, level_root=True)
+        self.level5 = _Tree(L, 1, c[4], c[5], 2, level_root=True)
+        # DLA-up over levels 2..5 (strides 4..32)
+        up_c = c[2:]
+        scales = [1, 2, 4, 8]
+        self.dla_up = nn.ModuleList()
+        in_c = list(up_c)
+        sc = list(scales)
+        for i in range(len(up_c) - 1):
+            j = -i - 2
+            self.dla_up.append(_IDAUp(L, up_c[j], in_c[j:], [s // sc[j] for s in sc[j:]]))
+            sc[j + 1:] = [sc[j]] * len(sc[j + 1:])
+            in_c[j + 1:] = [up_c[j]] * len(in_c[j + 1:])
+        self.ida_up = _IDAUp(L, up_c[0], up_c[:3], [1, 2, 4])
+        self.heads = nn.ModuleDict({
+            name: nn.Sequential(_conv_act(L, up_c[0], head_conv, 3),
+                                L.DCConv2d(head_conv, n, 1, bias=True, dense_out=True))
+            for name, n in (("hm", num_classes), ("wh", 2), ("reg", 2))})
+
+    def forward(self, x):
+        x = self.level0(self.base_layer(self.sparsify(x)))
+        x = self.level1(x)
+        feats = []
+        for lvl in (self.level2, self.level3, self.level4, self.level5):
+            x = lvl(x)
+            feats.append(x)
+        layers = list(feats)
+        outs = [layers[-1]]
+        for i, ida in enumerate(self.dla_up):
+            ida(layers, len(layers) - i - 2, len(layers))
+            outs.insert(0, layers[-1])
+        y = outs[:3]
+        self.ida_up(y, 0, len(y))
+        return {name: head(y[-1]) for name, head in self.heads.items()}

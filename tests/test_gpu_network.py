@@ -166,3 +166,61 @@ def test_video_graph_matches_eager(lib):
             got = vg.step().clone()
             torch.cuda.synchronize()
             assert torch.equal(got, want), f"frame {t}: max diff {float((got - want).abs().max())}"
+
+
+def _out_err(got, want):
+    if isinstance(want, dict):
+        return max(_out_err(got[k], want[k]) for k in want)
+    return float((got.float().cpu() - want.float()).abs().max())
+
+
+def _out_scale(want):
+    if isinstance(want, dict):
+        return max(_out_scale(v) for v in want.values())
+    return max(1.0, float(want.abs().max()))
+
+
+def _hrnet(L):
+    from deltacnn_amd.networks import HRNet
+    return HRNet(L, modules=(1, 2, 1))
+
+
+def _dla(L):
+    from deltacnn_amd.networks import DLA34CenterNet
+    return DLA34CenterNet(L, num_classes=8, head_conv=64)
+
+
+def _calibrated(builder, frames):
+    from deltacnn_amd.networks import DenseLayers, fold_data_statistics
+    torch.manual_seed(0)
+    dense = builder(DenseLayers).eval()
+    with torch.no_grad():
+        fold_data_statistics(dense, frames)
+    return dense.state_dict()
+
+
+@pytest.mark.parametrize("builder,size", [(_hrnet, (64, 64)), (_dla, (64, 96))], ids=["hrnet", "dla34"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_multibranch_networks(lib, builder, size, dtype):
+    """HRNet (multi-resolution exchange: strided 3x3, 1x1 + nearest upsampling, chained adds
+    with ReLU) and DLA-34 + CenterNet heads (7x7 stride-1 stem, 2x2 max-pooling, concatenating
+    roots, transposed convolutions, three dense heads), reduced in depth / head width, 8 frames,
+    threshold 0.05.  fp32: HIP equals the oracle to 1e-4 relative on every frame; fp16: HIP
+    tracks the dense model as closely as the oracle does (see test_mobilenet_32_frames)."""
+    from deltacnn_amd.video import moving_rectangles_video
+    video = moving_rectangles_video(frames=8, height=size[0], width=size[1], n_rect=2, min_size=8, max_size=24)
+    state = _calibrated(builder, video[:3])
+    dense, ref, dut = _models(builder, dtype, 0.05, state)
+    e_ref = e_dut = 0.0
+    with torch.no_grad():
+        for t in range(video.shape[0]):
+            frame = video[t:t + 1].to(dtype)
+            full = dense(frame.float())
+            want = ref(frame)
+            got = dut(cl(frame))
+            e_ref = max(e_ref, _out_err(want, full))
+            e_dut = max(e_dut, _out_err(got, full))
+            if dtype == torch.float32:
+                assert _out_err(got, want) <= 1e-4 * _out_scale(want), f"frame {t}"
+    print(f"{dtype}: |oracle-dense| {e_ref:.4f}  |hip-dense| {e_dut:.4f}")
+    assert e_dut <= 1.5 * e_ref + 2e-2

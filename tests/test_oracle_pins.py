@@ -341,3 +341,29 @@ def test_truncation_error_stays_bounded():
         for t in range(video.shape[0]):
             errs.append(float((model(video[t:t + 1]) - dense(video[t:t + 1])).abs().max()))
     assert max(errs[12:]) <= 2.0 * max(errs[:12]) + 1e-3 and max(errs) < 0.5
+
+
+@pytest.mark.parametrize("which", ["hrnet", "dla34"])
+def test_multibranch_networks_threshold_zero_equal_dense(which):
+    """HRNet (strided 3x3 exchange convolutions, 1x1 + nearest upsampling, chained adds with
+    ReLU) and DLA-34 + CenterNet heads (7x7 stem, 2x2 max-pooling, concatenating roots,
+    transposed convolutions): with threshold 0 the delta model reproduces the dense model."""
+    from deltacnn_amd.networks import HRNet, DLA34CenterNet
+    from deltacnn_amd.video import moving_rectangles_video
+    if which == "hrnet":
+        def builder(L):
+            return HRNet(L, modules=(1, 1, 1), blocks=2)
+        size = (64, 64)
+    else:
+        def builder(L):
+            return DLA34CenterNet(L, num_classes=4, head_conv=32)
+        size = (64, 96)
+    dense, model = _pair(builder, 0.0)
+    video = moving_rectangles_video(frames=3, height=size[0], width=size[1], n_rect=2, min_size=8, max_size=20)
+    with torch.no_grad():
+        for t in range(video.shape[0]):
+            want, got = dense(video[t:t + 1]), model(video[t:t + 1])
+            if not isinstance(want, dict):
+                want, got = {"out": want}, {"out": got}
+            for k in want:
+                assert torch.allclose(got[k], want[k], rtol=1e-3, atol=1e-4 * max(1.0, float(want[k].abs().max()))), (t, k)
