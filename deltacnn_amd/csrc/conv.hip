@@ -424,9 +424,9 @@ conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
 // 16 compacted output pixels of the 8x8 tile, reduction over (tap, input channel) in steps of
 // 32, step index s = tap * ksteps + channel step (the packed filter is linear in s).
 //
-//   * after the mask phase the workgroup builds a table in LDS: for every (tap, compacted
-//     pixel) the index of the input pixel it reads, or -1 if that input is out of bounds or
-//     inactive; taps that no pixel of the tile uses are skipped altogether;
+//   * the mask phase also builds a table in LDS: for every (tap, compacted pixel) the index of
+//     the input pixel it reads, or -1 if that input is out of bounds or inactive; taps that no
+//     pixel of the tile uses are skipped altogether;
 //   * a wavefront accumulates R channel tiles x 4 pixel tiles, so a reduction step costs
 //     R + 4 fragment loads for 4 * R MFMAs; the KW wavefronts of a workgroup split the steps
 //     round-robin and their partial sums meet in LDS (added in ascending wavefront order);
@@ -449,9 +449,8 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
     __shared__ float4_t s_red[KW > 1 ? KW * NT * WAVE : 1];
     const int b = blockIdx.z / co_blocks;
     const int cb = blockIdx.z % co_blocks;
-    if (threadIdx.x == 0) s_taps = 0;
-    const int n = tile_mask_phase<TR>(p, mask, out_mask, b, blockIdx.y * TILE, blockIdx.x * TILE,
-                                      cb == 0, s_list, &s_n);
+    const int n = tile_front<TR>(p, mask, out_mask, b, blockIdx.y * TILE, blockIdx.x * TILE, cb == 0,
+                                 s_list, s_src, &s_taps, &s_n);
     if (n == 0) return;
 
     const int kw = threadIdx.x / WAVE, lane = lane_id();
@@ -460,29 +459,6 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
     const int n_tiles = (n + 15) >> 4;
     const int co_tiles = (p.Co + 15) >> 4;
     const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
-    const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
-
-    // source table: entry (tap, pixel) for all taps and the 64 pixel slots of the tile
-    unsigned long long used = 0;
-    for (int e = threadIdx.x; e < K2 * TILE_PX; e += KW * WAVE) {
-        const int tap = e >> 6, pix = e & 63;
-        int src = -1;
-        if (pix < n) {
-            const int code = s_list[pix];
-            const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
-            int iy, ix;
-            if (tap_src<TR>(code >> 16, ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
-                tap_src<TR>(code & 0xffff, kx, p.sw, p.dw, p.pl, p.Wi, ix) && mb[iy * p.Wi + ix] != 0)
-                src = iy * p.Wi + ix;
-        }
-        s_src[e] = src;
-        if (src >= 0) used |= 1ull << tap;
-    }
-    // one LDS atomic per wavefront: OR of the lanes' tap sets
-#pragma unroll
-    for (int o = 1; o < WAVE; o <<= 1) used |= __shfl_xor(used, o, WAVE);
-    if (lane == 0 && used != 0) atomicOr(&s_taps, used);
-    __syncthreads();
     const unsigned long long taps = s_taps;
 
     float4_t acc[R][NT];

@@ -490,7 +490,11 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     // over many workgroups) is faster.
     const bool fusable = res == nullptr && epi != nullptr && epi->mode >= 0 && g.out_c % 4 == 0 && al8(epi->prev) &&
                          al8(epi->trunc) && al8(out);
-    if (fusable && ksteps <= PW_FUSED_MAX_STEPS && p.P >= 512) {
+    // ... and not for large problems either (>= 4096 output tiles of 16x16 with a reduction of
+    // several steps): there fragment traffic dominates, and the convolution-only kernel reuses
+    // every fragment 4 times where a 16-pixel workgroup cannot.
+    const bool large = (int64_t)ceil_div(p.P, 16) * p.co_tiles >= 4096 && ksteps >= 2;
+    if (fusable && ksteps <= PW_FUSED_MAX_STEPS && p.P >= 512 && !large) {
         dim3 grid(ceil_div(p.P, 16));
         const int act = epi->act < 0 ? 0 : epi->act;
         note_kernel("pw_act_mfma_kernel");

@@ -64,4 +64,68 @@ __device__ __forceinline__ int tile_mask_phase(const ConvP &p, const int32_t *__
     return *s_n;
 }
 
+// Phase 1 of the MFMA convolution: the mask phase and the source table in one pass.  Lane i of
+// the first wavefront owns output pixel i of the 8x8 tile; it requests the mask words of all its
+// taps at once (nine at a time, clamped addresses), so the whole phase is one memory round trip.
+// Results in LDS: s_list[0..n) = active output pixels (oy << 16 | ox); s_src[tap * 64 + slot] =
+// input pixel index read by compacted pixel `slot` through `tap`, or -1 (out of bounds, inactive,
+// or slot >= n); *s_taps = set of taps used by at least one pixel.  Returns n.  Must be called
+// by the whole workgroup (K2 <= 64).
+template <bool TR>
+__device__ __forceinline__ int tile_front(const ConvP &p, const int32_t *__restrict__ mask,
+                                          int32_t *__restrict__ out_mask, int b, int ty0, int tx0,
+                                          bool write_mask, int *s_list, int *s_src,
+                                          unsigned long long *s_taps, int *s_n) {
+    if (threadIdx.x < WAVE) {
+        const int K2 = p.Kh * p.Kw;
+        const int oy = ty0 + (threadIdx.x >> 3), ox = tx0 + (threadIdx.x & 7);
+        const bool inb = oy < p.Ho && ox < p.Wo;
+        const int32_t *m = mask + (size_t)b * p.Hi * p.Wi;
+        unsigned long long bits = 0;
+        for (int t0 = 0; t0 < K2; t0 += 9) {
+            int word[9];
+            bool ok[9];
+#pragma unroll
+            for (int j = 0; j < 9; ++j) {
+                const int tap = min(t0 + j, K2 - 1);
+                const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
+                int iy = 0, ix = 0;
+                ok[j] = inb && t0 + j < K2 && tap_src<TR>(oy, ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
+                        tap_src<TR>(ox, kx, p.sw, p.dw, p.pl, p.Wi, ix);
+                word[j] = m[ok[j] ? iy * p.Wi + ix : 0];
+            }
+#pragma unroll
+            for (int j = 0; j < 9; ++j)
+                if (ok[j] && word[j] != 0) bits |= 1ull << (t0 + j);
+        }
+        const bool upd = bits != 0;
+        if (inb && write_mask) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = upd ? 1 : 0;
+        int n;
+        const int rank = wave_rank(upd, n);
+        // active pixels take slots 0..n-1 in lane order, the others fill n..63 with -1 rows
+        const int slot = upd ? rank : n + (int)threadIdx.x - rank;
+        if (upd) s_list[rank] = (oy << 16) | ox;
+        for (int tap = 0; tap < K2; ++tap) {
+            int src = -1;
+            if ((bits >> tap) & 1ull) {
+                const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
+                int iy, ix;
+                tap_src<TR>(oy, ky, p.sh, p.dh, p.pt, p.Hi, iy);
+                tap_src<TR>(ox, kx, p.sw, p.dw, p.pl, p.Wi, ix);
+                src = iy * p.Wi + ix;
+            }
+            s_src[tap * TILE_PX + slot] = src;
+        }
+        unsigned long long used = bits;
+#pragma unroll
+        for (int o = 1; o < WAVE; o <<= 1) used |= __shfl_xor(used, o, WAVE);
+        if (threadIdx.x == 0) {
+            *s_n = n;
+            *s_taps = used;
+        }
+    }
+    __syncthreads();
+    return *s_n;
+}
+
 }  // namespace dc
