@@ -32,6 +32,21 @@ __device__ __forceinline__ void vstore(T *p, const Vec<T, N> &x) {
     *reinterpret_cast<Vec<T, N> *>(p) = x;
 }
 
+// A 16-byte vector kept if `on`, else all-zero bits: four 32-bit selects whatever the element
+// type (a per-element select on halves costs twice as many instructions).
+template <typename T, int N>
+__device__ __forceinline__ Vec<T, N> vkeep(const Vec<T, N> &x, bool on) {
+    static_assert(sizeof(Vec<T, N>) == 16, "16-byte vectors only");
+    union {
+        Vec<T, N> v;
+        uint32_t u[4];
+    } c;
+    c.v = x;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) c.u[k] = on ? c.u[k] : 0u;
+    return c.v;
+}
+
 // Elements per 16-byte vector.
 template <typename T>
 struct Vec16 {
@@ -76,11 +91,20 @@ __device__ __attribute__((noinline)) half_t swish_t(half_t x) {
     return half_t(float(x) * (1.0f / (1.0f + expf(-float(x)))));
 }
 
+// max / min as single instructions (v_max_f16, v_max_f32, ...).  For finite operands they give
+// the values of the compare-and-select form `x < 0 ? 0 : x`; the two differ only for NaN (here
+// replaced by the other operand) and in the sign of a zero result, and NaN never reaches an
+// active pixel.
+__device__ __forceinline__ float tmax(float a, float b) { return __builtin_fmaxf(a, b); }
+__device__ __forceinline__ float tmin(float a, float b) { return __builtin_fminf(a, b); }
+__device__ __forceinline__ half_t tmax(half_t a, half_t b) { return __builtin_fmaxf16(a, b); }
+__device__ __forceinline__ half_t tmin(half_t a, half_t b) { return __builtin_fminf16(a, b); }
+
 template <typename T>
 __device__ __forceinline__ T act_apply(T x, int act) {
     switch (act) {
-        case DC_ACT_RELU: return x < T(0) ? T(0) : x;
-        case DC_ACT_RELU6: return x < T(0) ? T(0) : (x > T(6) ? T(6) : x);
+        case DC_ACT_RELU: return tmax(x, T(0));
+        case DC_ACT_RELU6: return tmin(tmax(x, T(0)), T(6));
         case DC_ACT_LEAKY: return x < T(0) ? x * T(0.1f) : x;
         case DC_ACT_SIGMOID: return sigmoid_t(x);
         case DC_ACT_SWISH: return swish_t(x);

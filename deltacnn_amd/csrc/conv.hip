@@ -185,12 +185,12 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
             for (int t = 0; t < 9; ++t) {
                 const bool on = (taps >> t) & 1ull;
 #pragma unroll
-                for (int it = 0; it < ITERS; ++it)
+                for (int it = 0; it < ITERS; ++it) {
+                    const Vec<T, N> xs = vkeep<T, N>(ex[t][it], on);
 #pragma unroll
-                    for (int j = 0; j < N; ++j) {
-                        const float xv = on ? float(ex[t][it].v[j]) : 0.f;
-                        acc[it][j] = __builtin_fmaf(xv, float(ew[t][it].v[j]), acc[it][j]);
-                    }
+                    for (int j = 0; j < N; ++j)
+                        acc[it][j] = __builtin_fmaf(float(xs.v[j]), float(ew[t][it].v[j]), acc[it][j]);
+                }
             }
         } else if (K3 && ITERS <= 2) {
             // 3x3: every tap is loaded unconditionally from a clamped (always valid) address
@@ -214,12 +214,12 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
             for (int t = 0; t < 9; ++t) {
                 const bool on = (taps >> t) & 1ull;
 #pragma unroll
-                for (int it = 0; it < ITERS; ++it)
+                for (int it = 0; it < ITERS; ++it) {
+                    const Vec<T, N> xs = vkeep<T, N>(x[t][it], on);
 #pragma unroll
-                    for (int j = 0; j < N; ++j) {
-                        const float xv = on ? float(x[t][it].v[j]) : 0.f;
-                        acc[it][j] = __builtin_fmaf(xv, float(w[t][it].v[j]), acc[it][j]);
-                    }
+                    for (int j = 0; j < N; ++j)
+                        acc[it][j] = __builtin_fmaf(float(xs.v[j]), float(w[t][it].v[j]), acc[it][j]);
+                }
             }
         } else {
             for (int t = 0; t < K2; ++t) {
