@@ -79,20 +79,32 @@ def time_steps(step, warmup, steps):
     return (time.perf_counter() - t0) / steps
 
 
+UNROLL = 8  # frames per graph launch (processed one after the other)
+
+
+def time_graph(model, frames, start, warmup, steps):
+    """Seconds per frame of model(frame) replayed from a HIP graph that holds UNROLL consecutive
+    frames per launch (exactly `steps` timed frames after at least `warmup` untimed ones)."""
+    from deltacnn_amd.graph import VideoGraph
+    unroll = UNROLL if steps % UNROLL == 0 else 1
+    vg = VideoGraph(model, frames, start=start, unroll=unroll)
+    warm = -(-warmup // unroll)
+    assert start + (warm + steps // unroll) * unroll <= frames.shape[0]
+    return time_steps(vg.step, warm, steps // unroll) / unroll
+
+
 def run_delta(delta, frames, warmup, steps, mode):
     """frames: [T,3,H,W] on the GPU with T >= warmup + steps + 2.  Frame 0 initialises the
     caches (dense first frame), frame 1 runs eagerly (lazy weight packing, buffers); the timed
     region covers frames 2+warmup .. 2+warmup+steps-1."""
     import torch
     from deltacnn_amd.graph import VideoGraph
-    assert frames.shape[0] >= warmup + steps + 2
     delta.reset_layers()
     with torch.no_grad():
         delta(frames[0:1])
         delta(frames[1:2])
         if mode == "graph":
-            vg = VideoGraph(delta, frames, start=2)
-            return time_steps(vg.step, warmup, steps)
+            return time_graph(delta, frames, 2, warmup, steps)
         it = iter(range(2, frames.shape[0]))
         return time_steps(lambda: delta(frames[next(it):][:1]), warmup, steps)
 
@@ -106,8 +118,7 @@ def run_dense(dense, frames, warmup, steps):
         dense(frames[0:1])
         it = iter(range(1, frames.shape[0]))
         eager = time_steps(lambda: dense(frames[next(it):][:1]), warmup, steps)
-        vg = VideoGraph(dense, frames, start=1)
-        graph = time_steps(vg.step, warmup, steps)
+        graph = time_graph(dense, frames, 1, warmup, steps)
     return eager, graph
 
 
@@ -304,7 +315,7 @@ def main():
     _lib.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
 
-    n_frames = args.warmup + args.steps + 3
+    n_frames = args.warmup + args.steps + 3 + UNROLL
     video = controlled_density_video(frames=n_frames, density=args.density)
     stats_video = moving_rectangles_video(frames=4)
     dense, delta, state = build_models(stats_video.to("cuda").contiguous(memory_format=torch.channels_last))
@@ -332,8 +343,8 @@ def main():
     sweep = []
     if not args.no_sweep:
         for rho in SWEEP:
-            sw_steps = min(args.steps, 100)
-            v = gpu_frames(controlled_density_video(frames=sw_steps + 13, density=rho))
+            sw_steps = min(args.steps, 12 * UNROLL)
+            v = gpu_frames(controlled_density_video(frames=sw_steps + 13 + UNROLL, density=rho))
             s = run_delta(delta, v, 10, sw_steps, args.mode)
             sweep.append({"density": rho, "fps": round(1.0 / s, 1), "ms_per_frame": round(s * 1e3, 4),
                           "speedup_vs_dense_gpu": round(dense_best / s, 3)})
@@ -378,6 +389,7 @@ def main():
         "config": {"workload": "MobileNetV2 w1.0 (BN folded, 1000-way head) 224x224 fp16 channels-last "
                                "batch 1, threshold 0.05 on all layers, controlled-density video",
                    "update_density": args.density, "launch_mode": args.mode,
+                   "frames_per_graph_launch": UNROLL if args.mode == "graph" and args.steps % UNROLL == 0 else 1,
                    "weights": "random init (seed 0) rescaled per conv to unit output variance"},
         "dense_gpu": {"eager_fps": round(1 / dense_eager, 1), "graph_fps": round(1 / dense_graph, 1),
                       "speedup_vs_dense_gpu": round(dense_best / sec, 3)},

@@ -47,27 +47,31 @@ class VideoGraph:
     the graph.
 
     ``frames`` is a device tensor ``[T, C, H, W]`` whose frames are NHWC in memory
-    (``torch.channels_last``).  Every :meth:`step` processes the next frame; the caller must
-    not step past the end of the clip.  ``model`` may be any callable on a ``[1, C, H, W]``
-    tensor (the delta model after its first frame, or a dense model).
+    (``torch.channels_last``).  One :meth:`step` processes the next ``unroll`` frames, one after
+    the other, from a single graph launch (one gather fetches them, one add advances the
+    counter), and returns the output of the last one -- or, with ``unroll > 1``, the list of
+    all ``unroll`` outputs; the caller must not step past the end of the clip.  ``model`` may be
+    any callable on a ``[1, C, H, W]`` tensor (the delta model after its first frame, or a
+    dense model).
     """
 
-    def __init__(self, model, frames: torch.Tensor, start: int = 0):
+    def __init__(self, model, frames: torch.Tensor, start: int = 0, unroll: int = 1):
         if not frames.is_contiguous(memory_format=torch.channels_last):
             raise ValueError("frames must be channels_last")
         t, c, h, w = frames.shape
         self.length = t
+        self.unroll = unroll
         self._rows = frames.permute(0, 2, 3, 1).reshape(t, h * w * c)  # a view: NHWC rows
-        self.index = torch.full((1,), start, dtype=torch.int64, device=frames.device)
+        self.index = torch.arange(start, start + unroll, dtype=torch.int64, device=frames.device)
         self.graph = torch.cuda.CUDAGraph()
         with torch.no_grad(), torch.cuda.graph(self.graph):
-            row = self._rows.index_select(0, self.index)
-            frame = row.view(1, h, w, c).permute(0, 3, 1, 2)
-            self.static_out = model(frame)
-            self.index.add_(1)
+            staged = self._rows.index_select(0, self.index).view(unroll, h, w, c).permute(0, 3, 1, 2)
+            outs = [model(staged[i:i + 1]) for i in range(unroll)]
+            self.index.add_(unroll)
+        self.static_out = outs[0] if unroll == 1 else outs
 
     def seek(self, t: int) -> None:
-        self.index.fill_(t)
+        self.index.copy_(torch.arange(t, t + self.unroll, dtype=torch.int64, device=self.index.device))
 
     @torch.no_grad()
     def step(self):

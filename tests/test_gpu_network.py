@@ -168,6 +168,29 @@ def test_video_graph_matches_eager(lib):
             assert torch.equal(got, want), f"frame {t}: max diff {float((got - want).abs().max())}"
 
 
+def test_video_graph_unrolled_matches_eager(lib):
+    """Four frames per graph launch: every output of every launch equals the eager model's."""
+    from deltacnn_amd.graph import VideoGraph
+    from deltacnn_amd.video import moving_rectangles_video
+    video = moving_rectangles_video(frames=14, height=64, width=64, n_rect=2, min_size=8, max_size=20)
+    state = _calibrated_state(video[:4])
+    _, _, eager = _models(_mobilenet, torch.float16, 0.05, state)
+    _, _, graphed = _models(_mobilenet, torch.float16, 0.05, state)
+    frames = cl(video.half())
+    with torch.no_grad():
+        for m in (eager, graphed):
+            m(frames[0:1])
+            m(frames[1:2])
+        vg = VideoGraph(graphed, frames, start=2, unroll=4)
+        for r in range(3):
+            want = [eager(frames[t:t + 1]).clone() for t in range(2 + 4 * r, 6 + 4 * r)]
+            torch.cuda.synchronize()
+            got = [o.clone() for o in vg.step()]
+            torch.cuda.synchronize()
+            for i in range(4):
+                assert torch.equal(got[i], want[i]), f"launch {r} frame {i}"
+
+
 def _out_err(got, want):
     if isinstance(want, dict):
         return max(_out_err(got[k], want[k]) for k in want)
