@@ -154,8 +154,9 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
     }
 
     uint64_t taps = 0;
-    for (int j = 0; j < K2; j += G) {
-        const int t = j + gl;
+    const int GW = G > WAVE ? WAVE : G;  // a group wider than a wavefront: every wavefront scans
+    for (int j = 0; j < K2; j += GW) {
+        const int t = j + (gl & (GW - 1));
         bool m = false;
         if (valid && t < K2) {
             const int ky = t / p.Kw, kx = t - ky * p.Kw;
@@ -658,9 +659,10 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
     if (epi && (!al(epi->prev) || (epi->trunc && !al(epi->trunc)) || epi->mode < 0)) return false;
     const int64_t P_out = (int64_t)g.batch * g.out_h * g.out_w;
     const int nvec = g.in_c / N;
-    const int G = pick_group(nvec, P_out, 4);
+    const int wide = (epi == nullptr || epi->mode == DC_TRUNC_MAX) ? wide_group(nvec, P_out) : 0;
+    const int G = wide ? wide : pick_group(nvec, P_out, 4);
     const int iters = ceil_div(nvec, G);
-    const int block = group_block(P_out * G);
+    const int block = wide ? wide : group_block(P_out * G);
     note_kernel("conv_dw_kernel");
     dim3 grid((unsigned)ceil_div64(P_out * G, block));
     EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f,

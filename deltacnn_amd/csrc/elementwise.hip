@@ -529,9 +529,14 @@ hipError_t act_trunc_t(T *delta, T *prev, T *trunc, int32_t *mask, float thr, in
     }
     if (can_vec<T>(C, {delta, prev, trunc}) && C / N <= WAVE * 4) {
         int nvec = C / N;
-        int G = pick_group(nvec, P, 4);
+        const int wide = mode == DC_TRUNC_MAX ? wide_group(nvec, P) : 0;
+        int G = wide ? wide : pick_group(nvec, P, 4);
         int iters = ceil_div(nvec, G);
         GroupLaunch L(P, G);
+        if (wide) {  // one pixel per workgroup
+            L.block = wide;
+            L.grid = dim3((unsigned)P);
+        }
         switch (iters) {
             case 1: act_trunc_launch<T, 1>(L.grid, L.block, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;
             case 2: act_trunc_launch<T, 2>(L.grid, L.block, s, delta, prev, trunc, mask, thr, act, mode, P, C, L.lg); break;

@@ -22,7 +22,8 @@ __device__ __forceinline__ float group_sum(float v, int G) {
 // `dl[it]` holds channels (it*G + gl)*N .. +N of the incoming delta for pixel `p`, `q` / `tr`
 // the same channels of the cached pre-activation and of the truncated remainder (loaded by the
 // caller as early as it can, see load_state; only meaningful where `valid` and the channel
-// offset is < C).  All lanes of the wavefront must call this (it contains wave-wide ballots).
+// offset is < C).  All lanes of the wavefront must call this (it contains wave-wide ballots);
+// with G > 64 (one pixel per workgroup, mode max only) all wavefronts of the workgroup must.
 // Returns whether the pixel was kept.
 template <typename T, int ITERS>
 __device__ __forceinline__ void load_state(Vec<T, Vec16<T>::N> (&q)[ITERS],
@@ -70,6 +71,8 @@ __device__ __forceinline__ bool act_trunc_pixel(Vec<T, Vec16<T>::N> (&dl)[ITERS]
     bool keep;
     if (mode == DC_TRUNC_MAX) {
         keep = group_any(hit, G);
+        // a group wider than a wavefront is a whole workgroup working on one pixel
+        if (G > WAVE) keep = __syncthreads_or(keep) != 0;
     } else {
         sq = group_sum(sq, G);
         if (mode == DC_TRUNC_RMS) sq /= float(C);
@@ -96,6 +99,14 @@ __device__ __forceinline__ bool act_trunc_pixel(Vec<T, Vec16<T>::N> (&dl)[ITERS]
         if (!keep && gl == 0) mask[p] = 0;
     }
     return keep;
+}
+
+// One pixel per workgroup of 128 / 256 lanes, one vector per lane: for rows of more than 64
+// vectors on small maps, where a lane holding several vectors makes the wavefront's
+// instruction stream -- which is the kernel time at this size -- several times longer.
+inline int wide_group(int nvec, int64_t pixels) {
+    if (nvec <= WAVE || nvec > 256 || pixels > 1024) return 0;
+    return nvec <= 128 ? 128 : 256;
 }
 
 // Lanes per pixel for `nvec` 16-byte vectors per row when a lane may hold up to `max_iters`.
