@@ -116,20 +116,20 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
     const int po = gid >> lg, gl = gid & (G - 1);
     const int P_out = p.B * p.Ho * p.Wo;
     const bool valid = po < P_out;
-    const int b = po / (p.Ho * p.Wo);
-    const int r = po - b * p.Ho * p.Wo;
+    const int pc = min(po, P_out - 1);  // surplus groups of the last workgroup shadow the last pixel
+    const int b = pc / (p.Ho * p.Wo);
+    const int r = pc - b * p.Ho * p.Wo;
     const int oy = r / p.Wo, ox = r - oy * p.Wo;
-    const int K2 = p.Kh * p.Kw;
+    const int K2 = K3 ? 9 : p.Kh * p.Kw;
+    const int Kw = K3 ? 3 : p.Kw;
     const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
     const int glo = lane_id() & ~(G - 1);
     const uint64_t gmask = G >= WAVE ? ~0ull : ((1ull << G) - 1ull);
 
     Vec<T, N> ex[K3 && EAGER ? 9 : 1][ITERS], ew[K3 && EAGER ? 9 : 1][ITERS], q[ITERS], tr[ITERS];
     if (K3 && EAGER) {
-        const int pc = valid ? po : 0;
-        const int cb = pc / (p.Ho * p.Wo), cr = pc - cb * p.Ho * p.Wo;
-        const int cy = cr / p.Wo, cx = cr - cy * p.Wo;
-        const T *inb = in + (size_t)cb * p.Hi * p.Wi * C;
+        const int cy = oy, cx = ox;
+        const T *inb = in + (size_t)b * p.Hi * p.Wi * C;
 #pragma unroll
         for (int t = 0; t < 9; ++t) {
             const int ky = t / 3, kx = t - ky * 3;
@@ -159,7 +159,7 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
         const int t = j + (gl & (GW - 1));
         bool m = false;
         if (valid && t < K2) {
-            const int ky = t / p.Kw, kx = t - ky * p.Kw;
+            const int ky = t / Kw, kx = t - ky * Kw;
             const int iy = oy * p.sh - p.pt + ky * p.dh, ix = ox * p.sw - p.pl + kx * p.dw;
             if (iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi) m = mb[iy * p.Wi + ix] != 0;
         }

@@ -64,7 +64,16 @@ __device__ __forceinline__ bool act_trunc_pixel(Vec<T, Vec16<T>::N> (&dl)[ITERS]
                 const T d = act_apply<T>(s[it].v[j], ACT) - act_apply<T>(q[it].v[j], ACT);
                 dl[it].v[j] = d;
                 hit |= tabs(d) > thr;
-                sq += float(d) * float(d);
+            }
+        }
+    }
+    if (mode != DC_TRUNC_MAX) {  // uniform: the squares are only needed by the norm modes
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int c = (it * G + gl) * N;
+            if (valid && c < C) {
+#pragma unroll
+                for (int j = 0; j < N; ++j) sq += float(dl[it].v[j]) * float(dl[it].v[j]);
             }
         }
     }

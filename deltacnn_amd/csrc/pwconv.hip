@@ -251,8 +251,8 @@ template <int CTW, int ACT>
 __device__ __forceinline__ void pw_epilogue_stats(const float4_t (&acc)[CTW], const half4_t (&q)[CTW],
                                                   const half4_t (&tr)[CTW], half4_t (&v)[CTW],
                                                   const half4_t (&bh)[CTW], bool on, int wave,
-                                                  int NW, int kq, const PwP &p, half_t thr, bool &hit,
-                                                  float &sq) {
+                                                  int NW, int kq, const PwP &p, half_t thr, bool norm,
+                                                  bool &hit, float &sq) {
 #pragma unroll
     for (int j = 0; j < CTW; ++j) {
         const int ct = wave + j * NW;
@@ -268,7 +268,7 @@ __device__ __forceinline__ void pw_epilogue_stats(const float4_t (&acc)[CTW], co
             const half_t d = act_apply<half_t>(s, ACT) - act_apply<half_t>(q[j][i], ACT);
             if (live && on) {
                 hit |= tabs(d) > thr;
-                sq += float(d) * float(d);
+                if (norm) sq += float(d) * float(d);  // uniform: only the norm modes need it
             }
         }
     }
@@ -413,7 +413,7 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
     half4_t v[CTW];
     bool hit = false;
     float sq = 0.f;
-    pw_epilogue_stats<CTW, ACT>(acc, q, tr, v, bh, on, wave, NW, kq, p, thr, hit, sq);
+    pw_epilogue_stats<CTW, ACT>(acc, q, tr, v, bh, on, wave, NW, kq, p, thr, mode != DC_TRUNC_MAX, hit, sq);
     // per pixel: combine the four k-quarter lanes, then the wavefronts
     float stat;
     if (mode == DC_TRUNC_MAX) {
