@@ -555,6 +555,133 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
     }
 }
 
+// Small layers (few output tiles, as on the low-resolution branches of multi-branch networks):
+// one 4x4 patch of output pixels x R channel tiles per workgroup, no compaction, no source
+// table, no barrier before the reduction.  Lane (l16, kq) owns output pixel l16 of the patch; it
+// requests the mask words of all its taps, and -- before they arrive -- the input and filter
+// fragments of its first chunk of reduction steps, whose addresses depend on coordinates only.
+// Fragments of taps that are out of bounds or inactive are zeroed by selection; outputs are
+// stored for updated pixels only.  KW wavefronts split the reduction steps round-robin.
+template <bool TR, int KW, int R, int S>
+__global__ void __launch_bounds__(KW * WAVE)
+conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
+                       const half_t *__restrict__ bias, half_t *__restrict__ out,
+                       const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
+                       int co_blocks, int ci_p) {
+    __shared__ float4_t s_red[KW > 1 ? KW * R * WAVE : 1];
+    const int b = blockIdx.z / co_blocks, cb = blockIdx.z % co_blocks;
+    const int kw = threadIdx.x / WAVE, lane = lane_id();
+    const int l16 = lane & 15, kq = lane >> 4;
+    const int oy = blockIdx.y * 4 + (l16 >> 2), ox = blockIdx.x * 4 + (l16 & 3);
+    const bool inside = oy < p.Ho && ox < p.Wo;
+    const int K2 = p.Kh * p.Kw;
+    const int co_tiles = (p.Co + 15) >> 4;
+    const int ksteps = ci_p >> 5;
+    const int total = K2 * ksteps;
+    const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+    const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
+    const half_t *wfrag[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
+        wfrag[r] = wp + (size_t)min(cb * R + r, co_tiles - 1) * total * 512 + lane * 8;
+
+    // source pixel of (this lane's output pixel, tap): index or -1 if there is none
+    auto source = [&](int tap) -> int {
+        const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
+        int iy = 0, ix = 0;
+        const bool ok = inside && tap_src<TR>(oy, ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
+                        tap_src<TR>(ox, kx, p.sw, p.dw, p.pl, p.Wi, ix);
+        return ok ? iy * p.Wi + ix : -1;
+    };
+    auto load_chunk = [&](int s0, half8_t (&a)[S][R], half8_t (&x)[S], int (&tp)[S]) {
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            const int s = min(s0 + i * KW, total - 1);
+            const int tap = s / ksteps;
+            tp[i] = tap;
+            const int k = min(((s - tap * ksteps) << 5) + kq * 8, p.Ci - 8);
+#pragma unroll
+            for (int r = 0; r < R; ++r) a[i][r] = *reinterpret_cast<const half8_t *>(wfrag[r] + (size_t)s * 512);
+            x[i] = *reinterpret_cast<const half8_t *>(inb + (size_t)max(source(tap), 0) * p.Ci + k);
+        }
+    };
+
+    // eager: first chunk of fragments, then the mask words of all taps
+    half8_t a[S][R], x[S];
+    int tp[S];
+    load_chunk(kw, a, x, tp);
+    unsigned long long bits = 0;
+    for (int t0 = 0; t0 < K2; t0 += 9) {
+        int word[9], src[9];
+#pragma unroll
+        for (int j = 0; j < 9; ++j) {
+            src[j] = t0 + j < K2 ? source(t0 + j) : -1;
+            word[j] = mb[max(src[j], 0)];
+        }
+#pragma unroll
+        for (int j = 0; j < 9; ++j)
+            if (src[j] >= 0 && word[j] != 0) bits |= 1ull << (t0 + j);
+    }
+    const bool upd = bits != 0;
+    if (cb == 0 && kw == 0 && kq == 0 && inside) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = upd ? 1 : 0;
+    if (ballot(upd) == 0) return;  // the same in every wavefront of the workgroup
+    unsigned long long used = bits;  // taps some pixel of the patch uses
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) used |= __shfl_xor(used, o, WAVE);
+
+    float4_t acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = kw; s0 < total; s0 += S * KW) {
+        if (s0 != kw) load_chunk(s0, a, x, tp);
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            if (s0 + i * KW >= total || !((used >> tp[i]) & 1ull)) continue;  // wave-uniform
+            const half8_t xz = ((bits >> tp[i]) & 1ull) ? x[i] : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][r], xz, acc[r], 0, 0, 0);
+        }
+    }
+    if (KW > 1) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) s_red[(kw * R + r) * WAVE + lane] = acc[r];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if ((r % KW) != kw) continue;  // wavefront kw finishes channel tiles kw, kw + KW, ...
+            float4_t sum = s_red[r * WAVE + lane];
+#pragma unroll
+            for (int q = 1; q < KW; ++q) sum += s_red[(q * R + r) * WAVE + lane];
+            acc[r] = sum;
+        }
+    }
+    if (!upd) return;
+    half_t *o = out + (((size_t)b * p.Ho + oy) * p.Wo + ox) * p.Co;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (KW > 1 && (r % KW) != kw) continue;
+        const int ct = cb * R + r, co = ct * 16 + kq * 4;
+        if (ct >= co_tiles) continue;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias != nullptr) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (co + i < p.Co) bv[i] = float(bias[co + i]);
+        }
+        if (co + 3 < p.Co && (p.Co & 3) == 0) {
+            half4_t v;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = half_t(acc[r][i] + bv[i]);
+            *reinterpret_cast<half4_t *>(o + co) = v;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (co + i < p.Co) o[co + i] = half_t(acc[r][i] + bv[i]);
+        }
+    }
+}
+
 // One-time relayout of a reference-layout fp16 filter [Cin pad 2][K][K][Cout pad 2] (channel
 // pairs swizzled: W[ci][co] is stored at row ci ^ (co & 1)) into MFMA fragment order
 // [Cout tile of 16][tap][Cin step of 32][lane 0..63][8]: lane (kq * 16 + r) of a fragment holds
@@ -748,6 +875,30 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
         const int co_tiles = ceil_div(g.out_c, 16);
         const int ci_p = round_up(g.in_c, 32);
         const int steps = g.kernel_h * g.kernel_w * (ci_p / 32);
+        // Small layers: one 4x4 output patch per workgroup (see conv_patch_mfma_kernel).  The
+        // filter is re-read by every patch, so this only pays while patches x filter stays small.
+        const int64_t patches = (int64_t)ceil_div(g.out_w, 4) * ceil_div(g.out_h, 4) * g.batch;
+        if (patches * co_tiles * steps <= 32768) {
+            const int kwv = steps <= 12 ? 1 : steps <= 48 ? 4 : 8;
+            const int rv = (co_tiles >= 2 && patches * co_tiles >= 512) ? 2 : 1;
+            const int cbk = ceil_div(co_tiles, rv);
+            dim3 pgrid(ceil_div(g.out_w, 4), ceil_div(g.out_h, 4), g.batch * cbk);
+            note_kernel("conv_patch_mfma_kernel");
+#define DC_PATCH_L(TRF, KWV, RV, SV) conv_patch_mfma_kernel<TRF, KWV, RV, SV><<<pgrid, KWV * WAVE, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbk, ci_p)
+#define DC_PATCH(TRF)                                                                  \
+    do {                                                                               \
+        if (kwv == 1) { if (rv == 2) DC_PATCH_L(TRF, 1, 2, 6); else DC_PATCH_L(TRF, 1, 1, 12); } \
+        else if (kwv == 4) { if (rv == 2) DC_PATCH_L(TRF, 4, 2, 6); else DC_PATCH_L(TRF, 4, 1, 12); } \
+        else { if (rv == 2) DC_PATCH_L(TRF, 8, 2, 6); else DC_PATCH_L(TRF, 8, 1, 12); } \
+    } while (0)
+            if (transposed) DC_PATCH(true); else DC_PATCH(false);
+#undef DC_PATCH
+#undef DC_PATCH_L
+            hipError_t pe = hipGetLastError();
+            if (pe != hipSuccess || epi == nullptr) return pe;
+            return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
+                                            epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
+        }
         // channel tiles per wavefront: as many as keep at least ~2 workgroups per compute unit
         int R = co_tiles >= 4 ? 4 : co_tiles >= 2 ? 2 : 1;
         while (R > 1 && (int64_t)tx * ty * g.batch * ceil_div(co_tiles, R) < 512) R >>= 1;
