@@ -569,6 +569,7 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
                        const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
                        int co_blocks, int ci_p) {
     __shared__ float4_t s_red[KW > 1 ? KW * R * WAVE : 1];
+    __shared__ int s_src[KW * MFMA_MAX_TAPS * 16];
     const int b = blockIdx.z / co_blocks, cb = blockIdx.z % co_blocks;
     const int kw = threadIdx.x / WAVE, lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;
@@ -585,43 +586,58 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
         wfrag[r] = wp + (size_t)min(cb * R + r, co_tiles - 1) * total * 512 + lane * 8;
 
-    // source pixel of (this lane's output pixel, tap): index or -1 if there is none
-    auto source = [&](int tap) -> int {
-        const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
-        int iy = 0, ix = 0;
-        const bool ok = inside && tap_src<TR>(oy, ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
-                        tap_src<TR>(ox, kx, p.sw, p.dw, p.pl, p.Wi, ix);
-        return ok ? iy * p.Wi + ix : -1;
-    };
-    auto load_chunk = [&](int s0, half8_t (&a)[S][R], half8_t (&x)[S], int (&tp)[S]) {
-#pragma unroll
-        for (int i = 0; i < S; ++i) {
-            const int s = min(s0 + i * KW, total - 1);
-            const int tap = s / ksteps;
-            tp[i] = tap;
-            const int k = min(((s - tap * ksteps) << 5) + kq * 8, p.Ci - 8);
-#pragma unroll
-            for (int r = 0; r < R; ++r) a[i][r] = *reinterpret_cast<const half8_t *>(wfrag[r] + (size_t)s * 512);
-            x[i] = *reinterpret_cast<const half8_t *>(inb + (size_t)max(source(tap), 0) * p.Ci + k);
-        }
-    };
-
-    // eager: first chunk of fragments, then the mask words of all taps
-    half8_t a[S][R], x[S];
-    int tp[S];
-    load_chunk(kw, a, x, tp);
+    // Source table of this wavefront in LDS: s_src[tap * 16 + pixel] = input pixel index read by
+    // the lane's output pixel through `tap`, or -1 if it is out of bounds.  The four k-quarter
+    // lanes of a pixel share the taps (kq, kq + 4, ...), each also fetches the mask word of its
+    // taps; the activity bits are then combined across the four lanes.
+    int *src_tab = s_src + kw * (MFMA_MAX_TAPS * 16);
     unsigned long long bits = 0;
-    for (int t0 = 0; t0 < K2; t0 += 9) {
-        int word[9], src[9];
+    for (int t0 = 0; t0 < K2; t0 += 12) {
+        int word[3], src[3];
 #pragma unroll
-        for (int j = 0; j < 9; ++j) {
-            src[j] = t0 + j < K2 ? source(t0 + j) : -1;
+        for (int j = 0; j < 3; ++j) {
+            const int tap = t0 + kq + 4 * j;
+            src[j] = -1;
+            if (tap < K2) {
+                const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
+                int iy = 0, ix = 0;
+                if (inside && tap_src<TR>(oy, ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
+                    tap_src<TR>(ox, kx, p.sw, p.dw, p.pl, p.Wi, ix))
+                    src[j] = iy * p.Wi + ix;
+                src_tab[tap * 16 + l16] = src[j];
+            }
             word[j] = mb[max(src[j], 0)];
         }
 #pragma unroll
-        for (int j = 0; j < 9; ++j)
-            if (src[j] >= 0 && word[j] != 0) bits |= 1ull << (t0 + j);
+        for (int j = 0; j < 3; ++j)
+            if (src[j] >= 0 && word[j] != 0) bits |= 1ull << (t0 + kq + 4 * j);
     }
+    // Steps of this wavefront: s = kw, kw + KW, ...; (tap, channel step) advance with it and are
+    // wave-uniform, so they live in scalar registers.
+    int n_tap = 0, n_ks = kw;
+    while (n_ks >= ksteps) { n_ks -= ksteps; ++n_tap; }
+    auto load_chunk = [&](half8_t (&a)[S][R], half8_t (&x)[S], int (&tp)[S]) {
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            const int tap = min(n_tap, K2 - 1), ks = n_tap < K2 ? n_ks : ksteps - 1;  // past the end: last step again
+            tp[i] = tap;
+            const int k = min((ks << 5) + kq * 8, p.Ci - 8);
+            const int sp = src_tab[tap * 16 + l16];
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                a[i][r] = *reinterpret_cast<const half8_t *>(wfrag[r] + (size_t)(tap * ksteps + ks) * 512);
+            x[i] = *reinterpret_cast<const half8_t *>(inb + (size_t)max(sp, 0) * p.Ci + k);
+            n_ks += KW;
+            while (n_ks >= ksteps) { n_ks -= ksteps; ++n_tap; }
+        }
+    };
+
+    // eager: the first chunk of fragments is requested while the mask words are in flight
+    half8_t a[S][R], x[S];
+    int tp[S];
+    load_chunk(a, x, tp);
+    bits |= __shfl_xor(bits, 16, WAVE);
+    bits |= __shfl_xor(bits, 32, WAVE);
     const bool upd = bits != 0;
     if (cb == 0 && kw == 0 && kq == 0 && inside) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = upd ? 1 : 0;
     if (ballot(upd) == 0) return;  // the same in every wavefront of the workgroup
@@ -633,7 +649,7 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = float4_t{0.f, 0.f, 0.f, 0.f};
     for (int s0 = kw; s0 < total; s0 += S * KW) {
-        if (s0 != kw) load_chunk(s0, a, x, tp);
+        if (s0 != kw) load_chunk(a, x, tp);
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             if (s0 + i * KW >= total || !((used >> tp[i]) & 1ull)) continue;  // wave-uniform
