@@ -47,6 +47,18 @@ __device__ __forceinline__ Vec<T, N> vkeep(const Vec<T, N> &x, bool on) {
     return c.v;
 }
 
+// The same for an MFMA operand fragment of 8 halves.
+__device__ __forceinline__ half8_t keep8(half8_t x, bool on) {
+    union {
+        half8_t v;
+        uint32_t u[4];
+    } c;
+    c.v = x;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) c.u[k] = on ? c.u[k] : 0u;
+    return c.v;
+}
+
 // Elements per 16-byte vector.
 template <typename T>
 struct Vec16 {
@@ -59,6 +71,11 @@ struct Vec16 {
 #define DC_PIN(x) asm volatile("" : "+v"(x))
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
+
+// Index of the wavefront inside its workgroup, as a scalar: the compiler cannot see that
+// threadIdx.x / 64 is the same in all lanes, and would keep everything derived from it
+// (step counters, filter addresses, loop conditions) in vector registers and masked branches.
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE); }
 
 __device__ __forceinline__ uint64_t ballot(bool p) { return __ballot(p); }
 

@@ -454,7 +454,7 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
                                  s_list, s_src, &s_taps, &s_n);
     if (n == 0) return;
 
-    const int kw = threadIdx.x / WAVE, lane = lane_id();
+    const int kw = wave_id(), lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;  // row / column inside a tile, k-quarter
     const int K2 = p.Kh * p.Kw;
     const int n_tiles = (n + 15) >> 4;
@@ -499,7 +499,7 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 if (nt >= n_tiles) continue;  // wave-uniform
-                const half8_t xz = src[i][nt] >= 0 ? x[i][nt] : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                const half8_t xz = keep8(x[i][nt], src[i][nt] >= 0);
 #pragma unroll
                 for (int r = 0; r < R; ++r)
                     acc[r][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][r], xz, acc[r][nt], 0, 0, 0);
@@ -560,8 +560,9 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 // table, no barrier before the reduction.  Lane (l16, kq) owns output pixel l16 of the patch; it
 // requests the mask words of all its taps, and -- before they arrive -- the input and filter
 // fragments of its first chunk of reduction steps, whose addresses depend on coordinates only.
-// Fragments of taps that are out of bounds or inactive are zeroed by selection; outputs are
-// stored for updated pixels only.  KW wavefronts split the reduction steps round-robin.
+// Fragments of taps that are out of bounds or inactive are zeroed by selection (every step is
+// computed: at this size the instruction stream, not the MFMA count, is the kernel time);
+// outputs are stored for updated pixels only.  KW wavefronts split the reduction steps round-robin.
 template <bool TR, int KW, int R, int S>
 __global__ void __launch_bounds__(KW * WAVE)
 conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
@@ -571,7 +572,7 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     __shared__ float4_t s_red[KW > 1 ? KW * R * WAVE : 1];
     __shared__ int s_src[KW * MFMA_MAX_TAPS * 16];
     const int b = blockIdx.z / co_blocks, cb = blockIdx.z % co_blocks;
-    const int kw = threadIdx.x / WAVE, lane = lane_id();
+    const int kw = wave_id(), lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;
     const int oy = blockIdx.y * 4 + (l16 >> 2), ox = blockIdx.x * 4 + (l16 & 3);
     const bool inside = oy < p.Ho && ox < p.Wo;
@@ -641,9 +642,6 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     const bool upd = bits != 0;
     if (cb == 0 && kw == 0 && kq == 0 && inside) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = upd ? 1 : 0;
     if (ballot(upd) == 0) return;  // the same in every wavefront of the workgroup
-    unsigned long long used = bits;  // taps some pixel of the patch uses
-#pragma unroll
-    for (int o = 1; o < 16; o <<= 1) used |= __shfl_xor(used, o, WAVE);
 
     float4_t acc[R];
 #pragma unroll
@@ -652,8 +650,8 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
         if (s0 != kw) load_chunk(a, x, tp);
 #pragma unroll
         for (int i = 0; i < S; ++i) {
-            if (s0 + i * KW >= total || !((used >> tp[i]) & 1ull)) continue;  // wave-uniform
-            const half8_t xz = ((bits >> tp[i]) & 1ull) ? x[i] : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            // straight-line: a step past the end or an invalid (tap, pixel) pair multiplies zeros
+            const half8_t xz = keep8(x[i], s0 + i * KW < total && ((bits >> tp[i]) & 1ull));
 #pragma unroll
             for (int r = 0; r < R; ++r)
                 acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][r], xz, acc[r], 0, 0, 0);

@@ -68,7 +68,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
     constexpr int NW = KW * CBW * NBW, TILES = R * NTW, FT = (TILES + KW - 1) / KW;
     constexpr int PXW = NBW * NTW * 16;  // pixels per workgroup
     __shared__ float4_t s_red[KW > 1 ? NW * TILES * WAVE : 1];
-    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int wave = wave_id(), lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;
     const int kw = wave % KW, tw = wave / KW, cw = tw % CBW, nw = tw / CBW;
     const int ksteps = p.ci_p >> 5;
@@ -332,7 +332,7 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
                    half_t *__restrict__ prev, half_t *__restrict__ trunc, float thr_f, int mode) {
     constexpr int S = 2;
     __shared__ float s_stat[NW][16];
-    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int wave = wave_id(), lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;
     const int ksteps = p.ci_p >> 5;
     const int px = blockIdx.x * 16 + l16;
