@@ -555,6 +555,234 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
     }
 }
 
+// Larger layers: the input window ("halo") of an 8x8 output tile is staged in LDS once and the
+// input fragments of every tap are read from there, so global traffic per workgroup is the halo
+// plus the filter fragments.  Inactive and out-of-bounds halo pixels are staged as zeros, which
+// removes every per-fragment validity test from the reduction loop.
+//   * the four wavefronts of a workgroup split the output channels (R tiles of 16 each) and all
+//     accumulate the same (up to four) compacted 16-pixel tiles; no cross-wave reduction;
+//   * the halo is staged in chunks of `kcc` reduction steps (32 channels each) sized to the LDS
+//     budget; a pixel row is padded by 16 bytes so that neighbouring pixels start in different
+//     banks;
+//   * filter fragments (contiguous 1 KB reads) stream through a ring of D register buffers of
+//     S steps each, so D - 1 chunks are in flight while one is consumed: 4 LDS reads and
+//     4 * R MFMAs per step.
+constexpr int LDS_MAX_HALO = 1024;
+constexpr int LDS_MAX_STEPS = 1024;
+
+template <int R, int S, int D>
+__global__ void __launch_bounds__(4 * WAVE)
+conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
+                     const half_t *__restrict__ bias, half_t *__restrict__ out,
+                     const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
+                     int co_blocks, int ci_p, int hal_h, int hal_w, int kcc, int lgv) {
+    constexpr int NT = 4;
+    extern __shared__ __align__(16) unsigned char s_halo[];
+    __shared__ int s_hpix[LDS_MAX_HALO];
+    __shared__ int2 s_step[LDS_MAX_STEPS];
+    __shared__ int s_list[TILE_PX];
+    __shared__ int s_n;
+    const int b = blockIdx.z / co_blocks, cb = blockIdx.z % co_blocks;
+    const int ty0 = blockIdx.y * TILE, tx0 = blockIdx.x * TILE;
+    const int tid = threadIdx.x, nthr = blockDim.x, nw = nthr / WAVE;
+    const int wv = wave_id(), lane = lane_id();
+    const int l16 = lane & 15, kq = lane >> 4;
+    const int hpx = hal_h * hal_w;
+    const int iy0 = ty0 * p.sh - p.pt, ix0 = tx0 * p.sw - p.pl;
+    const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
+    const int co_tiles = (p.Co + 15) >> 4;
+    const int ksteps = ci_p >> 5;
+    const int K2 = p.Kh * p.Kw;
+    const int row = kcc * 64 + 16;  // bytes per staged halo pixel
+
+    // Step table of a channel chunk: for reduction step j = tap * kcur + ks the LDS byte offset of
+    // its input fragment relative to a pixel's halo origin, and its fragment offset in the
+    // packed filter.  Entries past the last step repeat it (their products are zeroed).
+    auto build_steps = [&](int kbase, int kcur) {
+        const int nsteps = K2 * kcur;
+        const int padded = (nsteps + S * D - 1) / (S * D) * (S * D);
+        for (int j = tid; j < padded; j += nthr) {
+            const int jj = min(j, nsteps - 1);
+            const int tap = jj / kcur, ks = jj - tap * kcur;
+            const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
+            s_step[j] = int2{(ky * p.dh * hal_w + kx * p.dw) * row + ks * 64, (tap * ksteps + kbase + ks) * 512};
+        }
+    };
+    build_steps(0, min(kcc, ksteps));
+    // halo table: global pixel index of every active in-bounds halo pixel, -1 otherwise
+    for (int i = tid; i < hpx; i += nthr) {
+        const int hy = i / hal_w, hx = i - hy * hal_w;
+        const int iy = iy0 + hy, ix = ix0 + hx;
+        const bool ok = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
+        const int px = ok ? iy * p.Wi + ix : 0;
+        const int word = mb[px];
+        s_hpix[i] = (ok && word != 0) ? px : -1;
+    }
+    __syncthreads();
+
+    // Filter fragments stream through a ring of D register buffers of S steps each, so D - 1
+    // chunks are in flight while one is consumed.  The first D chunks are requested here, before
+    // the mask phase and the staging, whose latencies they overlap.
+    unsigned wfrag[R];  // element offset of the wavefront's channel tiles in the packed filter
+#pragma unroll
+    for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
+        wfrag[r] = (unsigned)min((cb * nw + wv) * R + r, co_tiles - 1) * K2 * ksteps * 512 + lane * 8;
+    half8_t a[D][S][R];
+    int xo[D][S];
+    int jl = 0;
+    auto load_chunk = [&](half8_t (&ac)[S][R], int (&xc)[S]) {
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            const int2 e = s_step[jl + i];
+            xc[i] = e.x;
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                ac[i][r] = *reinterpret_cast<const half8_t *>(wp + (wfrag[r] + (unsigned)e.y));
+        }
+        jl += S;
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) load_chunk(a[d], xo[d]);
+    half_t bv[R][4];  // bias of the lane's four channels per tile, requested early as well
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int co = ((cb * nw + wv) * R + r) * 16 + kq * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bv[r][i] = bias != nullptr ? bias[min(co + i, p.Co - 1)] : half_t(0);
+    }
+
+    if (tid < WAVE) {  // dilate the mask over the window, compact the updated pixels
+        const int ly = tid >> 3, lx = tid & 7;
+        const bool inb = ty0 + ly < p.Ho && tx0 + lx < p.Wo;
+        bool upd = false;
+        const int base = ly * p.sh * hal_w + lx * p.sw;
+        for (int ky = 0; ky < p.Kh; ++ky)
+            for (int kx = 0; kx < p.Kw; ++kx) upd |= s_hpix[base + ky * p.dh * hal_w + kx * p.dw] >= 0;
+        upd = upd && inb;
+        if (inb && cb == 0) out_mask[((size_t)b * p.Ho + ty0 + ly) * p.Wo + tx0 + lx] = upd ? 1 : 0;
+        int n;
+        const int rank = wave_rank(upd, n);
+        if (upd) s_list[rank] = tid;
+        if (tid == 0) s_n = n;
+    }
+    __syncthreads();
+    const int n = s_n;
+    if (n == 0) return;
+
+    const int n_tiles = (n + 15) >> 4;
+    const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+    int hbase[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int slot = nt * 16 + l16;
+        const int loc = slot < n ? s_list[slot] : 0;
+        hbase[nt] = ((loc >> 3) * p.sh * hal_w + (loc & 7) * p.sw) * row + kq * 16;
+    }
+    float4_t acc[R][NT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[r][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int kbase = 0; kbase < ksteps; kbase += kcc) {
+        const int kcur = min(kcc, ksteps - kbase);
+        if (kbase > 0) {
+            __syncthreads();
+            build_steps(kbase, kcur);
+        }
+        {   // stage channels [kbase * 32, (kbase + kcur) * 32) of the halo: 2^lgv lanes per pixel,
+            // four pixels per lane in flight; inactive pixels read one shared dummy address
+            const int v = tid & ((1 << lgv) - 1);
+            const int c = min((kbase << 5) + v * 8, p.Ci - 8);
+            const bool vok = v < kcur * 4 && (kbase << 5) + v * 8 < p.Ci;
+            const int hstep = nthr >> lgv;
+            for (int h0 = tid >> lgv; h0 < hpx; h0 += 4 * hstep) {
+                half8_t val[4];
+                int px[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    px[u] = s_hpix[min(h0 + u * hstep, hpx - 1)];
+                    val[u] = *reinterpret_cast<const half8_t *>(inb + (size_t)max(px[u], 0) * p.Ci + c);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int hp = h0 + u * hstep;
+                    if (hp < hpx && v < kcur * 4)
+                        *reinterpret_cast<half8_t *>(s_halo + hp * row + v * 16) = keep8(val[u], vok && px[u] >= 0);
+                }
+            }
+        }
+        __syncthreads();
+        const int nsteps = K2 * kcur;
+        const int groups = (nsteps + S * D - 1) / (S * D);
+        if (kbase > 0) {
+            jl = 0;
+#pragma unroll
+            for (int d = 0; d < D; ++d) load_chunk(a[d], xo[d]);
+        }
+        // All groups but the last are complete and run without any test; NTA (number of 16-pixel
+        // tiles in use) is a compile-time constant, so the loop body is one branch-free block.
+        auto reduce = [&](auto nta_tag) {
+            constexpr int NTA = decltype(nta_tag)::value;
+            auto compute_chunk = [&](const half8_t (&ac)[S][R], const int (&xc)[S], auto tail_tag, int j0) {
+#pragma unroll
+                for (int i = 0; i < S; ++i) {
+                    half8_t x[NTA];
+#pragma unroll
+                    for (int nt = 0; nt < NTA; ++nt)
+                        x[nt] = *reinterpret_cast<const half8_t *>(s_halo + hbase[nt] + xc[i]);
+#pragma unroll
+                    for (int nt = 0; nt < NTA; ++nt) {
+                        if (decltype(tail_tag)::value) x[nt] = keep8(x[nt], j0 + i < nsteps);
+#pragma unroll
+                        for (int r = 0; r < R; ++r)
+                            acc[r][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ac[i][r], x[nt], acc[r][nt], 0, 0, 0);
+                    }
+                }
+            };
+            for (int g = 0; g + 1 < groups; ++g) {
+#pragma unroll
+                for (int d = 0; d < D; ++d) {
+                    compute_chunk(a[d], xo[d], std::false_type{}, 0);
+                    load_chunk(a[d], xo[d]);
+                }
+            }
+#pragma unroll
+            for (int d = 0; d < D; ++d) compute_chunk(a[d], xo[d], std::true_type{}, ((groups - 1) * D + d) * S);
+        };
+        switch (n_tiles) {
+            case 1: reduce(std::integral_constant<int, 1>{}); break;
+            case 2: reduce(std::integral_constant<int, 2>{}); break;
+            case 3: reduce(std::integral_constant<int, 3>{}); break;
+            default: reduce(std::integral_constant<int, 4>{}); break;
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int ct = (cb * nw + wv) * R + r;
+        if (ct >= co_tiles) continue;
+        const int co = ct * 16 + kq * 4;  // lane holds channels co .. co + 3 of pixel (nt, l16)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int pix = nt * 16 + l16;
+            if (pix >= n) continue;
+            const int loc = s_list[pix];
+            half_t *o = out + (((size_t)b * p.Ho + ty0 + (loc >> 3)) * p.Wo + tx0 + (loc & 7)) * p.Co + co;
+            if (co + 3 < p.Co && (p.Co & 3) == 0) {
+                half4_t v;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] = half_t(acc[r][nt][i] + float(bv[r][i]));
+                *reinterpret_cast<half4_t *>(o) = v;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (co + i < p.Co) o[i] = half_t(acc[r][nt][i] + float(bv[r][i]));
+            }
+        }
+    }
+}
+
 // Small layers (few output tiles, as on the low-resolution branches of multi-branch networks):
 // one 4x4 patch of output pixels x R channel tiles per workgroup, no compaction, no source
 // table, no barrier before the reduction.  Lane (l16, kq) owns output pixel l16 of the patch; it
@@ -912,6 +1140,35 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
             if (pe != hipSuccess || epi == nullptr) return pe;
             return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
                                             epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
+        }
+        // Larger layers: halo staged in LDS (see conv_lds_mfma_kernel).
+        if (!transposed) {
+            const int hal_h = (TILE - 1) * g.stride_h + (g.kernel_h - 1) * g.dilation_h + 1;
+            const int hal_w = (TILE - 1) * g.stride_w + (g.kernel_w - 1) * g.dilation_w + 1;
+            const int hpx = hal_h * hal_w;
+            const int ksteps_all = ci_p / 32;
+            const int kmax = hpx <= LDS_MAX_HALO ? ((48 << 10) / hpx - 16) / 64 : 0;
+            const int kcc = kmax >= 1 ? ceil_div(ksteps_all, ceil_div(ksteps_all, kmax)) : 0;
+            // the step table holds all steps of a channel chunk plus the ring's run-out
+            if (kmax >= 1 && g.kernel_h * g.kernel_w * kcc + 48 <= LDS_MAX_STEPS) {
+                const int64_t tiles = (int64_t)tx * ty * g.batch;
+                // Two channel tiles per wavefront halve the LDS reads per MFMA but double the
+                // registers; measured, that only pays for wide outputs on many tiles.
+                const int rl = (co_tiles >= 16 && tiles * ceil_div(co_tiles, 8) >= 512) ? 2 : 1;
+                const int nwv = std::min(4, ceil_div(co_tiles, rl));  // wavefronts per workgroup
+                const int cbl = ceil_div(co_tiles, nwv * rl);
+                const size_t lds = (size_t)hpx * (kcc * 64 + 16);
+                const int lgv = log2i(pow2_ceil(kcc * 4));  // lanes per halo pixel while staging
+                dim3 lgrid(tx, ty, g.batch * cbl);
+                note_kernel("conv_lds_mfma_kernel");
+#define DC_LDS_L(RV, SV, DV) conv_lds_mfma_kernel<RV, SV, DV><<<lgrid, nwv * WAVE, lds, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
+                if (rl == 2) DC_LDS_L(2, 2, 2); else DC_LDS_L(1, 4, 2);
+#undef DC_LDS_L
+                hipError_t le = hipGetLastError();
+                if (le != hipSuccess || epi == nullptr) return le;
+                return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
+                                                epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
+            }
         }
         // channel tiles per wavefront: as many as keep at least ~2 workgroups per compute unit
         int R = co_tiles >= 4 ? 4 : co_tiles >= 2 ? 2 : 1;
