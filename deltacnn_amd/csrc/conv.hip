@@ -434,7 +434,7 @@ conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
 //   * all fragment loads of S steps are issued unconditionally (clamped addresses) before the
 //     first MFMA of the chunk; input fragments of invalid (tap, pixel) pairs are zeroed by
 //     selection afterwards -- unlike the pointwise case they would reach valid outputs.
-constexpr int MFMA_MAX_TAPS = 49;
+constexpr int MFMA_MAX_TAPS = 64;
 
 template <bool TR, int KW, int R, int S>
 __global__ void __launch_bounds__(KW * WAVE)
@@ -446,12 +446,17 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
     __shared__ int s_list[TILE_PX];
     __shared__ int s_n;
     __shared__ int s_src[MFMA_MAX_TAPS * TILE_PX];
-    __shared__ unsigned long long s_taps;
+    __shared__ int s_taplist[MFMA_MAX_TAPS];
+    __shared__ int s_ntaps;
     __shared__ float4_t s_red[KW > 1 ? KW * NT * WAVE : 1];
     const int b = blockIdx.z / co_blocks;
     const int cb = blockIdx.z % co_blocks;
-    const int n = tile_front<TR>(p, mask, out_mask, b, blockIdx.y * TILE, blockIdx.x * TILE, cb == 0,
-                                 s_list, s_src, &s_taps, &s_n);
+    // transposed: blockIdx = (tile, stride phase) interleaved, pixels of a tile one stride apart
+    const int ys = TR ? p.sh : 1, xs = TR ? p.sw : 1;
+    const int ty0 = (blockIdx.y / ys) * TILE * ys + blockIdx.y % ys;
+    const int tx0 = (blockIdx.x / xs) * TILE * xs + blockIdx.x % xs;
+    const int n = tile_front<TR>(p, mask, out_mask, b, ty0, tx0, ys, xs, cb == 0, s_list, s_src,
+                                 s_taplist, &s_ntaps, &s_n);
     if (n == 0) return;
 
     const int kw = wave_id(), lane = lane_id();
@@ -460,7 +465,6 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
     const int n_tiles = (n + 15) >> 4;
     const int co_tiles = (p.Co + 15) >> 4;
     const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
-    const unsigned long long taps = s_taps;
 
     float4_t acc[R][NT];
 #pragma unroll
@@ -468,11 +472,11 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[r][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
     const int ksteps = ci_p >> 5;
-    const int total = K2 * ksteps;
+    const int total = s_ntaps * ksteps;  // steps over the taps in use only
     const half_t *wfrag[R];
 #pragma unroll
     for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
-        wfrag[r] = wp + (size_t)min(cb * R + r, co_tiles - 1) * total * 512 + lane * 8;
+        wfrag[r] = wp + (size_t)min(cb * R + r, co_tiles - 1) * K2 * ksteps * 512 + lane * 8;
 
     for (int s0 = kw; s0 < total; s0 += S * KW) {
         half8_t a[S][R], x[S][NT];
@@ -481,12 +485,13 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             const int s = min(s0 + i * KW, total - 1);
-            const int tap = s / ksteps;
-            const int k = min(((s - tap * ksteps) << 5) + kq * 8, p.Ci - 8);
-            use[i] = s0 + i * KW < total && ((taps >> tap) & 1ull);  // wave-uniform
+            const int ti = s / ksteps, ks = s - ti * ksteps;
+            const int tap = s_taplist[ti];
+            const int k = min((ks << 5) + kq * 8, p.Ci - 8);
+            use[i] = s0 + i * KW < total;  // wave-uniform
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                a[i][r] = *reinterpret_cast<const half8_t *>(wfrag[r] + (size_t)s * 512);
+                a[i][r] = *reinterpret_cast<const half8_t *>(wfrag[r] + (size_t)(tap * ksteps + ks) * 512);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 src[i][nt] = s_src[(tap << 6) + nt * 16 + l16];
@@ -1171,11 +1176,16 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
             }
         }
         // channel tiles per wavefront: as many as keep at least ~2 workgroups per compute unit
+        // transposed: one tile per (8x8 block of pixels one stride apart, stride phase)
+        const int gtx = transposed ? ceil_div(ceil_div(g.out_w, g.stride_w), TILE) * g.stride_w : tx;
+        const int gty = transposed ? ceil_div(ceil_div(g.out_h, g.stride_h), TILE) * g.stride_h : ty;
         int R = co_tiles >= 4 ? 4 : co_tiles >= 2 ? 2 : 1;
-        while (R > 1 && (int64_t)tx * ty * g.batch * ceil_div(co_tiles, R) < 512) R >>= 1;
-        const bool ksplit = steps >= 8;
+        while (R > 1 && (int64_t)gtx * gty * g.batch * ceil_div(co_tiles, R) < 512) R >>= 1;
+        // steps a tile actually runs: a transposed convolution uses (K / stride)^2 taps per phase
+        const int tile_steps = transposed ? ceil_div(g.kernel_h, g.stride_h) * ceil_div(g.kernel_w, g.stride_w) * (ci_p / 32) : steps;
+        const bool ksplit = tile_steps >= 8;
         const int co_blocks = ceil_div(co_tiles, R);
-        dim3 grid(tx, ty, g.batch * co_blocks);
+        dim3 grid(gtx, gty, g.batch * co_blocks);
         note_kernel("conv_mfma_kernel");
 #define DC_MFMA_L(TRF, KWV, RV, SV) conv_mfma_kernel<TRF, KWV, RV, SV><<<grid, KWV * WAVE, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, co_blocks, ci_p)
 #define DC_MFMA(TRF)                                                                   \

@@ -69,16 +69,19 @@ __device__ __forceinline__ int tile_mask_phase(const ConvP &p, const int32_t *__
 // taps at once (nine at a time, clamped addresses), so the whole phase is one memory round trip.
 // Results in LDS: s_list[0..n) = active output pixels (oy << 16 | ox); s_src[tap * 64 + slot] =
 // input pixel index read by compacted pixel `slot` through `tap`, or -1 (out of bounds, inactive,
-// or slot >= n); *s_taps = set of taps used by at least one pixel.  Returns n.  Must be called
-// by the whole workgroup (K2 <= 64).
+// or slot >= n); s_taplist[0..*s_ntaps) = the taps used by at least one pixel, ascending.
+// The tile's pixels are (ty0 + i * ystep, tx0 + j * xstep), i, j = 0..7: a transposed
+// convolution takes the stride as step, so that all pixels of a tile share one stride phase
+// and hence one set of (K / stride)^2 taps.  Returns n.  Must be called by the whole workgroup
+// (K2 <= 64).
 template <bool TR>
 __device__ __forceinline__ int tile_front(const ConvP &p, const int32_t *__restrict__ mask,
                                           int32_t *__restrict__ out_mask, int b, int ty0, int tx0,
-                                          bool write_mask, int *s_list, int *s_src,
-                                          unsigned long long *s_taps, int *s_n) {
+                                          int ystep, int xstep, bool write_mask, int *s_list,
+                                          int *s_src, int *s_taplist, int *s_ntaps, int *s_n) {
     if (threadIdx.x < WAVE) {
         const int K2 = p.Kh * p.Kw;
-        const int oy = ty0 + (threadIdx.x >> 3), ox = tx0 + (threadIdx.x & 7);
+        const int oy = ty0 + (threadIdx.x >> 3) * ystep, ox = tx0 + (threadIdx.x & 7) * xstep;
         const bool inb = oy < p.Ho && ox < p.Wo;
         const int32_t *m = mask + (size_t)b * p.Hi * p.Wi;
         unsigned long long bits = 0;
@@ -119,9 +122,11 @@ __device__ __forceinline__ int tile_front(const ConvP &p, const int32_t *__restr
         unsigned long long used = bits;
 #pragma unroll
         for (int o = 1; o < WAVE; o <<= 1) used |= __shfl_xor(used, o, WAVE);
+        if ((int)threadIdx.x < K2 && ((used >> threadIdx.x) & 1ull))
+            s_taplist[__popcll(used & ((1ull << threadIdx.x) - 1ull))] = threadIdx.x;
         if (threadIdx.x == 0) {
             *s_n = n;
-            *s_taps = used;
+            *s_ntaps = __popcll(used);
         }
     }
     __syncthreads();

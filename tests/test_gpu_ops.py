@@ -335,6 +335,9 @@ DECONVS = [
     (24, 16, 2, 2, 0, 1, 1, 7, 7),
     (8, 12, 3, 1, 1, 1, 1, 8, 9),
     (5, 3, 4, 2, 1, 1, 1, 6, 6),
+    (64, 48, 4, 2, 1, 1, 1, 37, 41),   # large enough for the tiled MFMA kernel: stride-phase tiles
+    (32, 32, 8, 4, 2, 1, 1, 20, 23),   # k8 s4: 64 taps, four per phase
+    (40, 24, 3, 2, 1, 1, 1, 33, 30),   # kernel not a multiple of the stride: phases differ in tap count
 ]
 
 
