@@ -698,9 +698,9 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
         {   // stage channels [kbase * 32, (kbase + kcur) * 32) of the halo: 2^lgv lanes per pixel,
             // four pixels per lane in flight; inactive pixels read one shared dummy address
             const int v = tid & ((1 << lgv) - 1);
+            const int hstep = nthr >> lgv;
             const int c = min((kbase << 5) + v * 8, p.Ci - 8);
             const bool vok = v < kcur * 4 && (kbase << 5) + v * 8 < p.Ci;
-            const int hstep = nthr >> lgv;
             for (int h0 = tid >> lgv; h0 < hpx; h0 += 4 * hstep) {
                 half8_t val[4];
                 int px[4];
@@ -729,31 +729,42 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
         // tiles in use) is a compile-time constant, so the loop body is one branch-free block.
         auto reduce = [&](auto nta_tag) {
             constexpr int NTA = decltype(nta_tag)::value;
-            auto compute_chunk = [&](const half8_t (&ac)[S][R], const int (&xc)[S], auto tail_tag, int j0) {
+            // input fragments are read from LDS one step ahead of the MFMAs that consume them
+            half8_t xq[NTA];
+            auto read_x = [&](half8_t (&x)[NTA], int off) {
+#pragma unroll
+                for (int nt = 0; nt < NTA; ++nt)
+                    x[nt] = *reinterpret_cast<const half8_t *>(s_halo + hbase[nt] + off);
+            };
+            auto compute_chunk = [&](const half8_t (&ac)[S][R], const int (&xc)[S], int next_off, auto tail_tag, int j0) {
 #pragma unroll
                 for (int i = 0; i < S; ++i) {
-                    half8_t x[NTA];
-#pragma unroll
-                    for (int nt = 0; nt < NTA; ++nt)
-                        x[nt] = *reinterpret_cast<const half8_t *>(s_halo + hbase[nt] + xc[i]);
+                    half8_t xn[NTA];
+                    read_x(xn, i + 1 < S ? xc[i + 1] : next_off);
 #pragma unroll
                     for (int nt = 0; nt < NTA; ++nt) {
-                        if (decltype(tail_tag)::value) x[nt] = keep8(x[nt], j0 + i < nsteps);
+                        if (decltype(tail_tag)::value) xq[nt] = keep8(xq[nt], j0 + i < nsteps);
 #pragma unroll
                         for (int r = 0; r < R; ++r)
-                            acc[r][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ac[i][r], x[nt], acc[r][nt], 0, 0, 0);
+                            acc[r][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ac[i][r], xq[nt], acc[r][nt], 0, 0, 0);
                     }
+#pragma unroll
+                    for (int nt = 0; nt < NTA; ++nt) xq[nt] = xn[nt];
                 }
             };
+            read_x(xq, xo[0][0]);
             for (int g = 0; g + 1 < groups; ++g) {
 #pragma unroll
                 for (int d = 0; d < D; ++d) {
-                    compute_chunk(a[d], xo[d], std::false_type{}, 0);
+                    // the chunk after the last one of the ring is the first of the next group,
+                    // already reloaded below
+                    compute_chunk(a[d], xo[d], xo[(d + 1) % D][0], std::false_type{}, 0);
                     load_chunk(a[d], xo[d]);
                 }
             }
 #pragma unroll
-            for (int d = 0; d < D; ++d) compute_chunk(a[d], xo[d], std::true_type{}, ((groups - 1) * D + d) * S);
+            for (int d = 0; d < D; ++d)
+                compute_chunk(a[d], xo[d], xo[(d + 1) % D][0], std::true_type{}, ((groups - 1) * D + d) * S);
         };
         switch (n_tiles) {
             case 1: reduce(std::integral_constant<int, 1>{}); break;
@@ -1167,7 +1178,7 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                 dim3 lgrid(tx, ty, g.batch * cbl);
                 note_kernel("conv_lds_mfma_kernel");
 #define DC_LDS_L(RV, SV, DV) conv_lds_mfma_kernel<RV, SV, DV><<<lgrid, nwv * WAVE, lds, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
-                if (rl == 2) DC_LDS_L(2, 2, 2); else DC_LDS_L(1, 4, 2);
+                if (rl == 2) DC_LDS_L(2, 2, 2); else DC_LDS_L(1, 2, 3);
 #undef DC_LDS_L
                 hipError_t le = hipGetLastError();
                 if (le != hipSuccess || epi == nullptr) return le;
