@@ -298,6 +298,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="with --only-delta: end with one 256 MiB device-to-device copy kernel, the known-size "
                          "reference that hardware traffic counters of a profiling run are scaled by")
+    ap.add_argument("--only-micro", action="store_true",
+                    help="run the single-layer and scaled-shape sections only (for profiling runs)")
     ap.add_argument("--cpu-frames", type=int, default=12)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -314,6 +316,9 @@ def main():
         build()
     _lib.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.only_micro:
+        print(json.dumps({"micro": micro_bench(), "scaled": scaled_bench()}), flush=True)
+        return
 
     n_frames = args.warmup + args.steps + 3 + UNROLL
     video = controlled_density_video(frames=n_frames, density=args.density)
