@@ -564,8 +564,11 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 // input fragments of every tap are read from there, so global traffic per workgroup is the halo
 // plus the filter fragments.  Inactive and out-of-bounds halo pixels are staged as zeros, which
 // removes every per-fragment validity test from the reduction loop.
-//   * the four wavefronts of a workgroup split the output channels (R tiles of 16 each) and all
-//     accumulate the same (up to four) compacted 16-pixel tiles; no cross-wave reduction;
+//   * the wavefronts of a workgroup split the output channels (R tiles of 16 each) and, KS-fold,
+//     the reduction steps; all accumulate the same (up to four) compacted 16-pixel tiles.  LDS
+//     read bandwidth (128 bytes per clock per compute unit) bounds the reduction: an input
+//     fragment read feeds R MFMAs, so R = 2 with the steps split over two wavefronts moves half
+//     the LDS bytes of R = 1 with four channel groups, at the same number of wavefronts;
 //   * the halo is staged in chunks of `kcc` reduction steps (32 channels each) sized to the LDS
 //     budget; a pixel row is padded by 16 bytes so that neighbouring pixels start in different
 //     banks;
@@ -575,7 +578,7 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 constexpr int LDS_MAX_HALO = 1024;
 constexpr int LDS_MAX_STEPS = 1024;
 
-template <int R, int S, int D>
+template <int R, int S, int D, int KS>
 __global__ void __launch_bounds__(4 * WAVE)
 conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                      const half_t *__restrict__ bias, half_t *__restrict__ out,
@@ -591,6 +594,8 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
     const int ty0 = blockIdx.y * TILE, tx0 = blockIdx.x * TILE;
     const int tid = threadIdx.x, nthr = blockDim.x, nw = nthr / WAVE;
     const int wv = wave_id(), lane = lane_id();
+    // wavefront = (channel group cw, reduction slice kz): slice kz takes steps kz, kz + KS, ...
+    const int ncw = nw / KS, cw = wv % ncw, kz = wv / ncw;
     const int l16 = lane & 15, kq = lane >> 4;
     const int hpx = hal_h * hal_w;
     const int iy0 = ty0 * p.sh - p.pt, ix0 = tx0 * p.sw - p.pl;
@@ -605,7 +610,7 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
     // packed filter.  Entries past the last step repeat it (their products are zeroed).
     auto build_steps = [&](int kbase, int kcur) {
         const int nsteps = K2 * kcur;
-        const int padded = (nsteps + S * D - 1) / (S * D) * (S * D);
+        const int padded = (nsteps + S * D * KS - 1) / (S * D * KS) * (S * D * KS);
         for (int j = tid; j < padded; j += nthr) {
             const int jj = min(j, nsteps - 1);
             const int tap = jj / kcur, ks = jj - tap * kcur;
@@ -631,14 +636,14 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
     unsigned wfrag[R];  // element offset of the wavefront's channel tiles in the packed filter
 #pragma unroll
     for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
-        wfrag[r] = (unsigned)min((cb * nw + wv) * R + r, co_tiles - 1) * K2 * ksteps * 512 + lane * 8;
+        wfrag[r] = (unsigned)min((cb * ncw + cw) * R + r, co_tiles - 1) * K2 * ksteps * 512 + lane * 8;
     half8_t a[D][S][R];
     int xo[D][S];
     int jl = 0;
     auto load_chunk = [&](half8_t (&ac)[S][R], int (&xc)[S]) {
 #pragma unroll
         for (int i = 0; i < S; ++i) {
-            const int2 e = s_step[jl + i];
+            const int2 e = s_step[(jl + i) * KS + kz];
             xc[i] = e.x;
 #pragma unroll
             for (int r = 0; r < R; ++r)
@@ -651,7 +656,7 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
     half_t bv[R][4];  // bias of the lane's four channels per tile, requested early as well
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int co = ((cb * nw + wv) * R + r) * 16 + kq * 4;
+        const int co = ((cb * ncw + cw) * R + r) * 16 + kq * 4;
 #pragma unroll
         for (int i = 0; i < 4; ++i) bv[r][i] = bias != nullptr ? bias[min(co + i, p.Co - 1)] : half_t(0);
     }
@@ -719,7 +724,7 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
         }
         __syncthreads();
         const int nsteps = K2 * kcur;
-        const int groups = (nsteps + S * D - 1) / (S * D);
+        const int groups = (nsteps + S * D * KS - 1) / (S * D * KS);  // of D chunks of S steps per slice
         if (kbase > 0) {
             jl = 0;
 #pragma unroll
@@ -743,7 +748,7 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
                     read_x(xn, i + 1 < S ? xc[i + 1] : next_off);
 #pragma unroll
                     for (int nt = 0; nt < NTA; ++nt) {
-                        if (decltype(tail_tag)::value) xq[nt] = keep8(xq[nt], j0 + i < nsteps);
+                        if (decltype(tail_tag)::value) xq[nt] = keep8(xq[nt], (j0 + i) * KS + kz < nsteps);
 #pragma unroll
                         for (int r = 0; r < R; ++r)
                             acc[r][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ac[i][r], xq[nt], acc[r][nt], 0, 0, 0);
@@ -774,9 +779,29 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
         }
     }
 
+    if (KS > 1) {  // partial sums of the reduction slices meet in LDS (the halo is no longer needed)
+        float4_t *s_part = reinterpret_cast<float4_t *>(s_halo);
+        __syncthreads();
+        if (kz > 0) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    s_part[((((kz - 1) * ncw + cw) * R + r) * NT + nt) * WAVE + lane] = acc[r][nt];
+        }
+        __syncthreads();
+        if (kz > 0) return;
+#pragma unroll
+        for (int q = 1; q < KS; ++q)  // ascending slice order
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    acc[r][nt] += s_part[((((q - 1) * ncw + cw) * R + r) * NT + nt) * WAVE + lane];
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int ct = (cb * nw + wv) * R + r;
+        const int ct = (cb * ncw + cw) * R + r;
         if (ct >= co_tiles) continue;
         const int co = ct * 16 + kq * 4;  // lane holds channels co .. co + 3 of pixel (nt, l16)
 #pragma unroll
@@ -1168,17 +1193,26 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
             // the step table holds all steps of a channel chunk plus the ring's run-out
             if (kmax >= 1 && g.kernel_h * g.kernel_w * kcc + 48 <= LDS_MAX_STEPS) {
                 const int64_t tiles = (int64_t)tx * ty * g.batch;
-                // Two channel tiles per wavefront halve the LDS reads per MFMA but double the
-                // registers; measured, that only pays for wide outputs on many tiles.
-                const int rl = (co_tiles >= 16 && tiles * ceil_div(co_tiles, 8) >= 512) ? 2 : 1;
-                const int nwv = std::min(4, ceil_div(co_tiles, rl));  // wavefronts per workgroup
-                const int cbl = ceil_div(co_tiles, nwv * rl);
-                const size_t lds = (size_t)hpx * (kcc * 64 + 16);
+                // Arrangements (R channel tiles per wavefront, KS reduction slices, channel groups):
+                // wide outputs on many tiles: R = 2, four channel groups; otherwise, with enough
+                // steps to split, R = 2 and two slices (x two or one channel groups); short
+                // reductions: R = 1, up to four channel groups.
+                const int nsteps_chunk = g.kernel_h * g.kernel_w * kcc;
+                int rl = 1, ksl = 1, ncw = std::min(4, co_tiles);
+                if (co_tiles >= 16 && tiles * ceil_div(co_tiles, 8) >= 512) { rl = 2; ncw = 4; }
+                else if (nsteps_chunk >= 16 && co_tiles >= 4) { rl = 2; ksl = 2; ncw = 2; }
+                else if (nsteps_chunk >= 16 && co_tiles >= 2) { rl = 2; ksl = 4; ncw = 1; }
+                const int nwv = ncw * ksl;  // wavefronts per workgroup
+                const int cbl = ceil_div(co_tiles, ncw * rl);
+                const size_t lds = std::max((size_t)hpx * (kcc * 64 + 16), (size_t)(ksl - 1) * ncw * rl * 4 * 1024);
                 const int lgv = log2i(pow2_ceil(kcc * 4));  // lanes per halo pixel while staging
                 dim3 lgrid(tx, ty, g.batch * cbl);
                 note_kernel("conv_lds_mfma_kernel");
-#define DC_LDS_L(RV, SV, DV) conv_lds_mfma_kernel<RV, SV, DV><<<lgrid, nwv * WAVE, lds, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
-                if (rl == 2) DC_LDS_L(2, 2, 2); else DC_LDS_L(1, 2, 3);
+#define DC_LDS_L(RV, SV, DV, KV) conv_lds_mfma_kernel<RV, SV, DV, KV><<<lgrid, nwv * WAVE, lds, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
+                if (rl == 1) DC_LDS_L(1, 2, 3, 1);
+                else if (ksl == 1) DC_LDS_L(2, 2, 2, 1);
+                else if (ksl == 2) DC_LDS_L(2, 2, 2, 2);
+                else DC_LDS_L(2, 2, 2, 4);
 #undef DC_LDS_L
                 hipError_t le = hipGetLastError();
                 if (le != hipSuccess || epi == nullptr) return le;
