@@ -272,6 +272,115 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
     }
 }
 
+// Depthwise 3x3, stride 1, on large maps (bandwidth regime): one group of lanes computes a strip
+// of PX consecutive output pixels of a row.  The 3 x (PX + 2) input rows of the strip are
+// loaded once (instead of 9 per pixel) and the filter stays in registers for the whole strip,
+// which cuts load instructions and conversions per output pixel by more than half.  Per pixel
+// the arithmetic (tap order, zero-select of inactive taps, bias, epilogue) is that of
+// conv_dw_kernel, so the results are identical.
+template <typename T, int ACT>
+__global__ void __launch_bounds__(256)
+conv_dw_strip_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
+                     const T *__restrict__ bias, T *__restrict__ out,
+                     const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, EpiP epi,
+                     int lg) {
+    constexpr int N = Vec16<T>::N;
+    constexpr int PX = 4, COLS = PX + 2, WORDS = 3 * COLS;
+    const int G = 1 << lg;
+    const int C = p.Ci;
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int sidx = gid >> lg, gl = gid & (G - 1);
+    const int SW = (p.Wo + PX - 1) / PX;  // strips per row
+    const int total = p.B * p.Ho * SW;
+    const bool valid = sidx < total;
+    const int sc = min(sidx, total - 1);  // surplus groups of the last workgroup shadow the last strip
+    const int b = sc / (p.Ho * SW);
+    const int r = sc - b * p.Ho * SW;
+    const int oy = r / SW, ox0 = (r - oy * SW) * PX;
+    const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
+    const int glo = lane_id() & ~(G - 1);
+    const uint64_t gmask = G >= WAVE ? ~0ull : ((1ull << G) - 1ull);
+    const int iy0 = oy - p.pt, ix0 = ox0 - p.pl;
+
+    // activity of the 3 x COLS input pixels of the strip, one mask word per lane and pass
+    uint32_t words = 0;
+    for (int j = 0; j < WORDS; j += G) {
+        const int w = j + gl;
+        bool m = false;
+        if (valid && w < WORDS) {
+            const int wy = w / COLS, wx = w - wy * COLS;
+            const int iy = iy0 + wy, ix = ix0 + wx;
+            if (iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi) m = mb[iy * p.Wi + ix] != 0;
+        }
+        words |= (uint32_t)((ballot(m) >> glo) & gmask) << j;
+    }
+    uint32_t taps[PX];
+    bool active[PX];
+    bool any = false;
+    const size_t po0 = ((size_t)b * p.Ho + oy) * p.Wo + ox0;
+#pragma unroll
+    for (int j = 0; j < PX; ++j) {
+        taps[j] = ((words >> j) & 7u) | (((words >> (COLS + j)) & 7u) << 3) | (((words >> (2 * COLS + j)) & 7u) << 6);
+        active[j] = valid && ox0 + j < p.Wo && taps[j] != 0;
+        any |= active[j];
+        if (valid && ox0 + j < p.Wo && gl == 0) out_mask[po0 + j] = active[j] ? 1 : 0;
+    }
+    if (ballot(any) == 0) return;
+
+    const int c = min(gl * N, C - N);
+    const bool lane_on = gl * N < C;
+    Vec<T, N> q[PX][1], tr[PX][1];
+    if (ACT >= 0) {
+#pragma unroll
+        for (int j = 0; j < PX; ++j)
+            load_state<T, 1>(q[j], tr[j], active[j], po0 + j, gl, G, C, (const T *)epi.prev, (const T *)epi.trunc);
+    }
+    // all rows of the strip and the filter are requested together (clamped, always valid
+    // addresses); inactive taps are zeroed by selection afterwards
+    Vec<T, N> x[3][COLS], w[9];
+    const T *inb = in + (size_t)b * p.Hi * p.Wi * C;
+#pragma unroll
+    for (int wy = 0; wy < 3; ++wy) {
+        const int iy = min(max(iy0 + wy, 0), p.Hi - 1);
+#pragma unroll
+        for (int wx = 0; wx < COLS; ++wx) {
+            const int ix = min(max(ix0 + wx, 0), p.Wi - 1);
+            x[wy][wx] = vload<T, N>(inb + (size_t)(iy * p.Wi + ix) * C + c);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < 9; ++t) w[t] = vload<T, N>(filter + (size_t)t * C + c);
+    Vec<T, N> bv;
+    if (bias != nullptr) bv = vload<T, N>(bias + c);
+
+#pragma unroll
+    for (int j = 0; j < PX; ++j) {
+        float acc[N];
+#pragma unroll
+        for (int e = 0; e < N; ++e) acc[e] = 0.f;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const Vec<T, N> xs = vkeep<T, N>(x[t / 3][j + t % 3], (taps[j] >> t) & 1u);
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc[e] = __builtin_fmaf(float(xs.v[e]), float(w[t].v[e]), acc[e]);
+        }
+        Vec<T, N> dl[1];
+        if (bias != nullptr) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc[e] += float(bv.v[e]);
+        }
+#pragma unroll
+        for (int e = 0; e < N; ++e) dl[0].v[e] = T(acc[e]);
+        if (ACT < 0) {
+            if (active[j] && lane_on) vstore<T, N>(out + (po0 + j) * C + c, dl[0]);
+        } else {
+            act_trunc_pixel<T, 1, (ACT < 0 ? 0 : ACT)>(dl, q[j], tr[j], active[j], po0 + j, gl, G, C, out,
+                                                        (T *)epi.prev, (T *)epi.trunc, out_mask,
+                                                        T(epi.thr), epi.mode);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ few input channels
 // Network stems (RGB input): groups == 1, Cin <= 4.  Same one-group-per-output-pixel shape as
 // the depthwise kernel; a lane owns N consecutive output channels, input values are scalar
@@ -1069,6 +1178,29 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
     if (epi && (!al(epi->prev) || (epi->trunc && !al(epi->trunc)) || epi->mode < 0)) return false;
     const int64_t P_out = (int64_t)g.batch * g.out_h * g.out_w;
     const int nvec = g.in_c / N;
+    // large maps: strips of four output pixels per group of lanes (see conv_dw_strip_kernel)
+    if (g.kernel_h == 3 && g.kernel_w == 3 && g.stride_h == 1 && g.stride_w == 1 && g.dilation_h == 1 &&
+        g.dilation_w == 1 && nvec <= WAVE && P_out * g.in_c * (int64_t)sizeof(T) >= (32 << 20)) {
+        const int G = group_lanes(nvec, 1);
+        const int lg = log2i(G);
+        const int64_t strips = (int64_t)g.batch * g.out_h * ceil_div(g.out_w, 4);
+        dim3 grid((unsigned)ceil_div64(strips * G, 256));
+        EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f, epi ? epi->mode : 0};
+        const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
+        note_kernel("conv_dw_strip_kernel");
+#define DC_DWS(A) conv_dw_strip_kernel<T, A><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg)
+        switch (act) {
+            case DC_ACT_LINEAR: DC_DWS(DC_ACT_LINEAR); break;
+            case DC_ACT_RELU: DC_DWS(DC_ACT_RELU); break;
+            case DC_ACT_RELU6: DC_DWS(DC_ACT_RELU6); break;
+            case DC_ACT_LEAKY: DC_DWS(DC_ACT_LEAKY); break;
+            case DC_ACT_SIGMOID: DC_DWS(DC_ACT_SIGMOID); break;
+            case DC_ACT_SWISH: DC_DWS(DC_ACT_SWISH); break;
+            default: DC_DWS(-1); break;
+        }
+#undef DC_DWS
+        return true;
+    }
     const int wide = (epi == nullptr || epi->mode == DC_TRUNC_MAX) ? wide_group(nvec, P_out) : 0;
     const int G = wide ? wide : pick_group(nvec, P_out, 4);
     const int iters = ceil_div(nvec, G);

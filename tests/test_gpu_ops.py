@@ -268,6 +268,8 @@ CONVS = [
     (40, 24, (1, 3), (1, 2), (0, 1), 1, 1, 8, 16),
     (12, 18, 3, 1, 1, 1, 3, 8, 8),          # general groups (fp32 only)
     (5, 7, 3, 1, 1, 1, 1, 9, 9),            # odd channels: fp16 padding rows/cols of the swizzle
+    (16, 16, 3, 1, 1, 1, 16, 726, 727),     # depthwise on a large map: strips of four pixels per lane group
+    (24, 24, 3, 1, 1, 1, 24, 600, 601),     # ... with idle lanes in the group
 ]
 
 
@@ -380,6 +382,7 @@ FUSED = [
     (3, 32, 3, 2, 1, 1, 1, 24, 24),         # RGB stem
     (96, 96, 3, 1, 1, 1, 96, 96, 96),       # large map: two vectors per lane
     (24, 24, 3, 1, 1, 1, 24, 192, 192),     # large map: three vectors per lane
+    (16, 16, 3, 1, 1, 1, 16, 726, 727),     # very large map: strips of four pixels per lane group
 ]
 
 
