@@ -300,7 +300,8 @@ def main():
                          "reference that hardware traffic counters of a profiling run are scaled by")
     ap.add_argument("--only-micro", action="store_true",
                     help="run the single-layer and scaled-shape sections only (for profiling runs)")
-    ap.add_argument("--cpu-frames", type=int, default=12)
+    ap.add_argument("--cpu-frames", type=int, default=200,
+                    help="delta frames of the clip timed on the host CPU (bounded by the clip length)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path runs on ONE GPU (frames of a stream are strictly serial and a "
@@ -380,9 +381,10 @@ def main():
     cpu = None
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
-        d_fps, dn_fps = cpu_baseline(state, video, args.cpu_frames, threads)
+        cpu_frames = max(1, min(args.cpu_frames, video.shape[0] - 1))
+        d_fps, dn_fps = cpu_baseline(state, video, cpu_frames, threads)
         cpu = {"value": round(d_fps, 3), "unit": "frames/s", "cores": threads, "kind": "port",
-               "sample": f"{args.cpu_frames} delta frames of the same video through the fp32 CPU "
+               "sample": f"{cpu_frames} delta frames of the same video through the fp32 CPU "
                          f"oracle (pure PyTorch layers) after the dense first frame",
                "dense_cpu_fps": round(dn_fps, 3)}
 

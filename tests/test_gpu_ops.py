@@ -268,6 +268,16 @@ CONVS = [
     (40, 24, (1, 3), (1, 2), (0, 1), 1, 1, 8, 16),
     (12, 18, 3, 1, 1, 1, 3, 8, 8),          # general groups (fp32 only)
     (5, 7, 3, 1, 1, 1, 1, 9, 9),            # odd channels: fp16 padding rows/cols of the swizzle
+    # layers large enough for the LDS-halo MFMA kernel (fp16 packed), one per arrangement / corner
+    (64, 64, 3, 1, 1, 1, 1, 72, 70),        # two channel tiles per wave, steps split over two waves
+    (64, 32, 3, 1, 1, 1, 1, 100, 100),      # ... over four waves (one channel group)
+    (16, 64, 3, 1, 1, 1, 1, 120, 120),      # short reduction: one tile per wave, four channel groups
+    (32, 256, 3, 1, 1, 1, 1, 90, 90),       # wide output on many tiles: two tiles per wave, no split
+    (320, 32, 3, 1, 1, 1, 1, 40, 40),       # input channels staged in two chunks
+    (64, 80, 3, 2, 1, 1, 1, 120, 121),      # stride 2
+    (64, 48, 3, 1, 2, 2, 1, 80, 81),        # dilation 2
+    (32, 64, 5, 1, 2, 1, 1, 64, 66),        # 5x5
+    (24, 40, 3, 1, 1, 1, 1, 128, 130),      # partial reduction step and partial channel tile
     (16, 16, 3, 1, 1, 1, 16, 726, 727),     # depthwise on a large map: strips of four pixels per lane group
     (24, 24, 3, 1, 1, 1, 24, 600, 601),     # ... with idle lanes in the group
 ]
@@ -329,6 +339,28 @@ def test_conv(lib, dtype, cfg, density, use_bias, packed):
     assert out.shape == want.shape
     assert torch.equal(om.cpu(), want_mask)
     _check_conv(dtype, out, want, want_mask)
+
+
+@pytest.mark.parametrize("cfg,kernel", [
+    ((32, 32, 3, 1, 1, 1, 1, 16, 16), "conv_patch_mfma_kernel"),
+    ((64, 64, 3, 1, 1, 1, 1, 72, 70), "conv_lds_mfma_kernel"),
+    ((16, 64, 3, 1, 1, 1, 1, 120, 120), "conv_lds_mfma_kernel"),
+    ((320, 32, 3, 1, 1, 1, 1, 40, 40), "conv_lds_mfma_kernel"),
+    ((64, 256, 1, 1, 0, 1, 1, 20, 20), "pw_mfma_kernel"),
+    ((32, 32, 3, 1, 1, 1, 32, 15, 18), "conv_dw_kernel"),
+    ((16, 16, 3, 1, 1, 1, 16, 726, 727), "conv_dw_strip_kernel"),
+    ((3, 32, 3, 2, 1, 1, 1, 33, 31), "conv_fewcin_kernel"),
+], ids=lambda v: v if isinstance(v, str) else "-".join(str(x) for x in v))
+def test_conv_dispatch(lib, cfg, kernel):
+    """The shapes the parity cases above are chosen for reach the kernel they are meant to cover
+    (the library names the kernels of the last call)."""
+    from deltacnn_amd import _lib
+    Cin, Cout, groups = cfg[0], cfg[1], cfg[6]
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(torch.float16, cfg, 5, 0.5)
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, Cin, Cout, groups)
+    hk().sparse_conv(cl(x), d_filt, cl(mask), None, s, p, d, groups, c_out=Cout, create_out_mask=True, packed_filter=pk)
+    assert _lib.load().dc_last_kernels().decode() == kernel
 
 
 DECONVS = [
