@@ -35,7 +35,7 @@ _SIGNATURES = {
     "dc_activate_truncate": (c_int, [_P, _P, _P, _P, c_float, c_int, c_int, c_int32, c_int32, c_int, _P]),
     "dc_conv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),
     "dc_conv_act": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_float, c_int, c_int, c_int, _P]),
-    "dc_conv_add": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, _P, c_float, c_float, c_int, _P]),
+    "dc_conv_add": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, _P, c_float, c_float, _P, c_int, c_int, _P]),
     "dc_packed_filter_bytes": (c_int64, [_G, c_int, c_int]),
     "dc_pack_filter": (c_int, [_G, _P, _P, c_int, c_int, _P]),
     "dc_deconv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),

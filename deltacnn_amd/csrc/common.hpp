@@ -192,13 +192,19 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                        const void *packed, const void *bias, void *out, const int32_t *mask,
                        int32_t *out_mask, int dtype, bool transposed, const ActEpilogue *epi,
                        hipStream_t s);
-struct Residual {  // optional DCAdd fused behind a pointwise convolution
+struct Residual {  // optional DCAdd fused behind a convolution
     const void *values;
     const int32_t *mask;
     float wa, wb;
+    void *prev = nullptr;  // accumulated sum kept by a DCAdd with activation
+    int act = 0;           // its activation (0: none)
 };
 
 bool pointwise_eligible(const dc_geometry &g, int dtype);
+bool patch_eligible(const dc_geometry &g, int dtype);
+hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *packed,
+                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
+                             bool transposed, const Residual *res, hipStream_t s);
 hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *packed,
                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
                             const ActEpilogue *epi, bool *epilogue_done, const Residual *res,

@@ -941,12 +941,24 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
 // Fragments of taps that are out of bounds or inactive are zeroed by selection (every step is
 // computed: at this size the instruction stream, not the MFMA count, is the kernel time);
 // outputs are stored for updated pixels only.  KW wavefronts split the reduction steps round-robin.
-template <bool TR, int KW, int R, int S>
+struct PatchRes {  // DCAdd fused behind the convolution: a = residual, b = convolution
+    const half_t *values;
+    const int32_t *mask;
+    half_t *prev;
+    float wa, wb;
+    int act;
+};
+
+// ADD: out = wa * residual [its mask] + wb * conv [updated pixels], out_mask = the union; with an
+// activation the sum is accumulated in `prev` and its activated difference is emitted -- the
+// arithmetic of add_kernel applied to the convolution result rounded to fp16, so the output
+// equals that of the two separate launches bit for bit.
+template <bool TR, int KW, int R, int S, bool ADD>
 __global__ void __launch_bounds__(KW * WAVE)
 conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                        const half_t *__restrict__ bias, half_t *__restrict__ out,
                        const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
-                       int co_blocks, int ci_p) {
+                       int co_blocks, int ci_p, PatchRes rs) {
     __shared__ float4_t s_red[KW > 1 ? KW * R * WAVE : 1];
     __shared__ int s_src[KW * MFMA_MAX_TAPS * 16];
     const int b = blockIdx.z / co_blocks, cb = blockIdx.z % co_blocks;
@@ -991,6 +1003,9 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
         for (int j = 0; j < 3; ++j)
             if (src[j] >= 0 && word[j] != 0) bits |= 1ull << (t0 + kq + 4 * j);
     }
+    const size_t opix = ((size_t)b * p.Ho + min(oy, p.Ho - 1)) * p.Wo + min(ox, p.Wo - 1);
+    int rword = 0;
+    if (ADD) rword = rs.mask[opix];
     // Steps of this wavefront: s = kw, kw + KW, ...; (tap, channel step) advance with it and are
     // wave-uniform, so they live in scalar registers.
     int n_tap = 0, n_ks = kw;
@@ -1018,13 +1033,34 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     bits |= __shfl_xor(bits, 16, WAVE);
     bits |= __shfl_xor(bits, 32, WAVE);
     const bool upd = bits != 0;
-    if (cb == 0 && kw == 0 && kq == 0 && inside) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = upd ? 1 : 0;
-    if (ballot(upd) == 0) return;  // the same in every wavefront of the workgroup
+    const bool radd = ADD && inside && rword != 0;
+    if (cb == 0 && kw == 0 && kq == 0 && inside) out_mask[opix] = (upd || radd) ? 1 : 0;
+    const bool reduce = ballot(upd) != 0;  // the same in every wavefront of the workgroup
+    if (!reduce && ballot(radd) == 0) return;
+    // operands of the fused sum, requested now so that they arrive during the reduction
+    half4_t rv[R], qv[R];
+    if (ADD) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int co = min((cb * R + r) * 16 + kq * 4, ((p.Co + 3) & ~3) - 4);
+            if ((p.Co & 3) == 0) {
+                rv[r] = *reinterpret_cast<const half4_t *>(rs.values + opix * p.Co + co);
+                if (rs.act > 0) qv[r] = *reinterpret_cast<const half4_t *>(rs.prev + opix * p.Co + co);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int c = min((cb * R + r) * 16 + kq * 4 + i, p.Co - 1);
+                    rv[r][i] = rs.values[opix * p.Co + c];
+                    if (rs.act > 0) qv[r][i] = rs.prev[opix * p.Co + c];
+                }
+            }
+        }
+    }
 
     float4_t acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = float4_t{0.f, 0.f, 0.f, 0.f};
-    for (int s0 = kw; s0 < total; s0 += S * KW) {
+    for (int s0 = kw; s0 < total && reduce; s0 += S * KW) {
         if (s0 != kw) load_chunk(a, x, tp);
 #pragma unroll
         for (int i = 0; i < S; ++i) {
@@ -1035,7 +1071,7 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
                 acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][r], xz, acc[r], 0, 0, 0);
         }
     }
-    if (KW > 1) {
+    if (KW > 1 && reduce) {
 #pragma unroll
         for (int r = 0; r < R; ++r) s_red[(kw * R + r) * WAVE + lane] = acc[r];
         __syncthreads();
@@ -1048,8 +1084,8 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
             acc[r] = sum;
         }
     }
-    if (!upd) return;
-    half_t *o = out + (((size_t)b * p.Ho + oy) * p.Wo + ox) * p.Co;
+    if (!(upd || radd)) return;
+    half_t *o = out + opix * p.Co;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (KW > 1 && (r % KW) != kw) continue;
@@ -1061,15 +1097,35 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
             for (int i = 0; i < 4; ++i)
                 if (co + i < p.Co) bv[i] = float(bias[co + i]);
         }
-        if (co + 3 < p.Co && (p.Co & 3) == 0) {
-            half4_t v;
+        half4_t v;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = half_t(acc[r][i] + bv[i]);
+        for (int i = 0; i < 4; ++i) v[i] = half_t(acc[r][i] + bv[i]);
+        half4_t q;
+        if (ADD) {  // add_kernel's sequence: s = a * wa; s = fma(b, wb, s); n = s + prev; ...
+            const half_t wa = half_t(rs.wa), wb = half_t(rs.wb);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                half_t sum = half_t(0);
+                if (radd) sum = rv[r][i] * wa;
+                if (upd) sum = fma_t(v[i], wb, sum);
+                if (rs.act > 0) {
+                    const half_t n = sum + qv[r][i];
+                    sum = act_apply<half_t>(n, rs.act) - act_apply<half_t>(qv[r][i], rs.act);
+                    q[i] = n;
+                }
+                v[i] = sum;
+            }
+        }
+        if (co + 3 < p.Co && (p.Co & 3) == 0) {
             *reinterpret_cast<half4_t *>(o + co) = v;
+            if (ADD && rs.act > 0) *reinterpret_cast<half4_t *>(rs.prev + opix * p.Co + co) = q;
         } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (co + i < p.Co) o[co + i] = half_t(acc[r][i] + bv[i]);
+                if (co + i < p.Co) {
+                    o[co + i] = v[i];
+                    if (ADD && rs.act > 0) rs.prev[opix * p.Co + co + i] = q[i];
+                }
         }
     }
 }
@@ -1263,6 +1319,46 @@ bool try_fewcin(const dc_geometry &g, const ConvP &p, const T *in, const T *filt
 
 }  // namespace
 
+// The filter is re-read by every patch, so the patch kernel only pays while
+// patches x channel tiles x reduction steps stays small.
+bool patch_eligible(const dc_geometry &g, int dtype) {
+    if (!mfma_eligible(g, dtype) || g.kernel_h * g.kernel_w > MFMA_MAX_TAPS) return false;
+    const int64_t patches = (int64_t)ceil_div(g.out_w, 4) * ceil_div(g.out_h, 4) * g.batch;
+    const int steps = g.kernel_h * g.kernel_w * (round_up(g.in_c, 32) / 32);
+    return patches * ceil_div(g.out_c, 16) * steps <= 32768;
+}
+
+hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *packed,
+                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
+                             bool transposed, const Residual *res, hipStream_t s) {
+    ConvP p = make_params(g, DC_F16);
+    const int co_tiles = ceil_div(g.out_c, 16);
+    const int ci_p = round_up(g.in_c, 32);
+    const int steps = g.kernel_h * g.kernel_w * (ci_p / 32);
+    const int64_t patches = (int64_t)ceil_div(g.out_w, 4) * ceil_div(g.out_h, 4) * g.batch;
+    const int kwv = steps <= 12 ? 1 : steps <= 48 ? 4 : 8;
+    const int rv = (co_tiles >= 2 && patches * co_tiles >= 512) ? 2 : 1;
+    const int cbk = ceil_div(co_tiles, rv);
+    dim3 pgrid(ceil_div(g.out_w, 4), ceil_div(g.out_h, 4), g.batch * cbk);
+    PatchRes rs{nullptr, nullptr, nullptr, 0.f, 0.f, 0};
+    if (res != nullptr)
+        rs = PatchRes{(const half_t *)res->values, res->mask, (half_t *)res->prev, res->wa, res->wb, res->act};
+    note_kernel("conv_patch_mfma_kernel");
+#define DC_PATCH_L(TRF, KWV, RV, SV, AV) conv_patch_mfma_kernel<TRF, KWV, RV, SV, AV><<<pgrid, KWV * WAVE, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbk, ci_p, rs)
+#define DC_PATCH(TRF, AV)                                                                       \
+    do {                                                                                        \
+        if (kwv == 1) { if (rv == 2) DC_PATCH_L(TRF, 1, 2, 6, AV); else DC_PATCH_L(TRF, 1, 1, 12, AV); } \
+        else if (kwv == 4) { if (rv == 2) DC_PATCH_L(TRF, 4, 2, 6, AV); else DC_PATCH_L(TRF, 4, 1, 12, AV); } \
+        else { if (rv == 2) DC_PATCH_L(TRF, 8, 2, 6, AV); else DC_PATCH_L(TRF, 8, 1, 12, AV); } \
+    } while (0)
+    if (res != nullptr) DC_PATCH(false, true);  // the fused sum exists for plain convolutions only
+    else if (transposed) DC_PATCH(true, false);
+    else DC_PATCH(false, false);
+#undef DC_PATCH
+#undef DC_PATCH_L
+    return hipGetLastError();
+}
+
 hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                        const void *packed, const void *bias, void *out, const int32_t *mask,
                        int32_t *out_mask, int dtype, bool transposed, const ActEpilogue *epi,
@@ -1290,26 +1386,9 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
         const int co_tiles = ceil_div(g.out_c, 16);
         const int ci_p = round_up(g.in_c, 32);
         const int steps = g.kernel_h * g.kernel_w * (ci_p / 32);
-        // Small layers: one 4x4 output patch per workgroup (see conv_patch_mfma_kernel).  The
-        // filter is re-read by every patch, so this only pays while patches x filter stays small.
-        const int64_t patches = (int64_t)ceil_div(g.out_w, 4) * ceil_div(g.out_h, 4) * g.batch;
-        if (patches * co_tiles * steps <= 32768) {
-            const int kwv = steps <= 12 ? 1 : steps <= 48 ? 4 : 8;
-            const int rv = (co_tiles >= 2 && patches * co_tiles >= 512) ? 2 : 1;
-            const int cbk = ceil_div(co_tiles, rv);
-            dim3 pgrid(ceil_div(g.out_w, 4), ceil_div(g.out_h, 4), g.batch * cbk);
-            note_kernel("conv_patch_mfma_kernel");
-#define DC_PATCH_L(TRF, KWV, RV, SV) conv_patch_mfma_kernel<TRF, KWV, RV, SV><<<pgrid, KWV * WAVE, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbk, ci_p)
-#define DC_PATCH(TRF)                                                                  \
-    do {                                                                               \
-        if (kwv == 1) { if (rv == 2) DC_PATCH_L(TRF, 1, 2, 6); else DC_PATCH_L(TRF, 1, 1, 12); } \
-        else if (kwv == 4) { if (rv == 2) DC_PATCH_L(TRF, 4, 2, 6); else DC_PATCH_L(TRF, 4, 1, 12); } \
-        else { if (rv == 2) DC_PATCH_L(TRF, 8, 2, 6); else DC_PATCH_L(TRF, 8, 1, 12); } \
-    } while (0)
-            if (transposed) DC_PATCH(true); else DC_PATCH(false);
-#undef DC_PATCH
-#undef DC_PATCH_L
-            hipError_t pe = hipGetLastError();
+        // Small layers: one 4x4 output patch per workgroup (see conv_patch_mfma_kernel).
+        if (patch_eligible(g, dtype)) {
+            hipError_t pe = launch_patch_conv(g, in, packed, bias, out, mask, out_mask, transposed, nullptr, s);
             if (pe != hipSuccess || epi == nullptr) return pe;
             return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
                                             epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);

@@ -202,14 +202,18 @@ int dc_conv_act(const dc_geometry *g, const void *input, const void *filter,
 int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filter,
                 const void *bias, const int32_t *mask, const void *residual,
                 const int32_t *mask_residual, void *out, int32_t *out_mask, float weight_residual,
-                float weight_conv, int dtype, void *stream) {
+                float weight_conv, void *prev_out, int activation, int dtype, void *stream) {
     dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_conv_add");
     int rc = check_geometry("dc_conv_add", g, false, false);
     if (rc != DC_OK) return rc;
-    if (!dc::pointwise_eligible(*g, dtype))
+    if (activation < 0 || activation > DC_ACT_SWISH)
+        return fail(DC_ERR_UNSUPPORTED, "dc_conv_add: activation %d", activation);
+    const bool pointwise = activation == 0 && dc::pointwise_eligible(*g, dtype);
+    if (!pointwise && !dc::patch_eligible(*g, dtype))
         return fail(DC_ERR_UNSUPPORTED, "dc_conv_add: only fp16 1x1 stride-1 convolutions with "
-                                        "Cin %% 8 == 0 and Cout %% 4 == 0 have the fused form");
+                                        "Cin %% 8 == 0 and Cout %% 4 == 0 (no activation) and small "
+                                        "fp16 layers with Cin %% 8 == 0 have the fused form");
     DC_REQUIRE_PTR("dc_conv_add", input);
     DC_REQUIRE_PTR("dc_conv_add", packed_filter);
     DC_REQUIRE_PTR("dc_conv_add", mask);
@@ -217,15 +221,21 @@ int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filt
     DC_REQUIRE_PTR("dc_conv_add", mask_residual);
     DC_REQUIRE_PTR("dc_conv_add", out);
     DC_REQUIRE_PTR("dc_conv_add", out_mask);
+    if (activation > 0) DC_REQUIRE_PTR("dc_conv_add", prev_out);
     DC_REQUIRE_ALIGNED("dc_conv_add", input, 16);
     DC_REQUIRE_ALIGNED("dc_conv_add", packed_filter, 16);
     DC_REQUIRE_ALIGNED("dc_conv_add", residual, 8);
     DC_REQUIRE_ALIGNED("dc_conv_add", out, 8);
+    DC_REQUIRE_ALIGNED("dc_conv_add", prev_out, 8);
     DC_REQUIRE_ALIGNED("dc_conv_add", bias, 8);
-    dc::Residual res{residual, mask_residual, weight_residual, weight_conv};
-    bool unused = false;
-    return finish(dc::launch_pointwise(*g, input, packed_filter, bias, out, mask, out_mask, nullptr,
-                                       &unused, &res, (hipStream_t)stream), "dc_conv_add");
+    dc::Residual res{residual, mask_residual, weight_residual, weight_conv, prev_out, activation};
+    if (pointwise) {
+        bool unused = false;
+        return finish(dc::launch_pointwise(*g, input, packed_filter, bias, out, mask, out_mask, nullptr,
+                                           &unused, &res, (hipStream_t)stream), "dc_conv_add");
+    }
+    return finish(dc::launch_patch_conv(*g, input, packed_filter, bias, out, mask, out_mask, false, &res,
+                                        (hipStream_t)stream), "dc_conv_add");
 }
 
 int64_t dc_packed_filter_bytes(const dc_geometry *g, int dtype, int transposed) {

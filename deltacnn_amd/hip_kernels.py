@@ -164,18 +164,21 @@ def sparse_conv_activation(x, filter, mask, bias, prev_out, truncated, threshold
 
 
 def sparse_conv_add(x, packed_filter, mask, bias, residual, mask_residual, geometry, out, out_mask,
-                    weight_residual=1.0, weight_conv=1.0):
-    """``sparse_add_tensors(residual, sparse_conv(x))`` in the convolution's launch, for
-    pointwise fp16 convolutions with a packed filter.  Returns ``None`` (nothing launched) when
+                    weight_residual=1.0, weight_conv=1.0, prev_out=None, activation=0):
+    """``sparse_add_tensors(residual, sparse_conv(x), prev_out, ..., activation)`` in the
+    convolution's launch, for fp16 convolutions with a packed filter: pointwise ones (without
+    activation) and small layers of any kernel size.  Returns ``None`` (nothing launched) when
     the shape has no fused form, so the caller can issue the two separate calls."""
     lib = _lib.load()
     _nhwc(x, "x")
     _nhwc(residual, "residual")
     if packed_filter is None or x.dtype != torch.float16:
         return None
+    activation = max(int(activation), 0)
     args = (geometry, x.data_ptr(), packed_filter.data_ptr(), _ptr(bias), _mask(mask, "mask").data_ptr(),
             residual.data_ptr(), _mask(mask_residual, "mask_residual").data_ptr(), out.data_ptr(),
-            out_mask.data_ptr(), float(weight_residual), float(weight_conv), DC_F16, _stream())
+            out_mask.data_ptr(), float(weight_residual), float(weight_conv), _ptr(prev_out), activation,
+            DC_F16, _stream())
     meta = dict(g=geometry, esize=2, in_mask=mask, in_mask_b=mask_residual, out_mask=out_mask, mfma=True)
     try:
         _call("conv_add", lib.dc_conv_add, args, **meta)

@@ -277,6 +277,15 @@ def _conv_act(L, inp, oup, k=3, stride=1, act="relu"):
     return L.DCConv2d(inp, oup, k, stride, (k - 1) // 2, bias=True, activation=act)
 
 
+def _residual_sum(add, residual, conv, conv_input):
+    """``add(residual, conv(conv_input))``; a layer namespace whose DCAdd has ``after_conv`` may
+    run the sum inside the convolution's kernel."""
+    fused = getattr(add, "after_conv", None)
+    if fused is None:
+        return add(residual, conv(conv_input))
+    return fused(residual, conv, conv_input)
+
+
 class _BasicBlock(nn.Module):
     """Two 3x3 convolutions and a residual sum followed by ReLU."""
     expansion = 1
@@ -290,7 +299,7 @@ class _BasicBlock(nn.Module):
 
     def forward(self, x):
         res = x if self.project is None else self.project(x)
-        return self.add(self.conv2(self.conv1(x)), res)
+        return _residual_sum(self.add, res, self.conv2, self.conv1(x))
 
 
 class _Bottleneck(nn.Module):
@@ -307,7 +316,7 @@ class _Bottleneck(nn.Module):
 
     def forward(self, x):
         res = x if self.project is None else self.project(x)
-        return self.add(self.conv3(self.conv2(self.conv1(x))), res)
+        return _residual_sum(self.add, res, self.conv3, self.conv2(self.conv1(x)))
 
 
 class _HRModule(nn.Module):
@@ -450,7 +459,7 @@ class _BasicBlockExt(nn.Module):
 
     def forward(self, x, residual=None, children=None):
         residual = x if residual is None else residual
-        return self.add(self.conv2(self.conv1(x)), residual)
+        return _residual_sum(self.add, residual, self.conv2, self.conv1(x))
 
 
 class _IDAUp(nn.Module):

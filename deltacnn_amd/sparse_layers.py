@@ -414,14 +414,16 @@ class DCAdd(DCModule):
 
     def after_conv(self, a, conv, conv_input):
         """``self(a, conv(conv_input))`` with the addition fused into the convolution's kernel
-        when that is possible (pointwise fp16 convolution without activation, this layer without
-        activation / dense_out); otherwise exactly the two separate layer calls."""
-        fusable = (DCAdd.fuse_into_conv and type(a) != Tensor and self.activation is None
+        when that is possible (fp16 convolution without activation of its own -- pointwise, or a
+        small layer of any kernel size, which may also carry this layer's activation -- and no
+        dense_out); otherwise exactly the two separate layer calls."""
+        fusable = (DCAdd.fuse_into_conv and type(a) != Tensor and not self.first_iter
                    and not self.dense_out and isinstance(conv, DCConv2d) and conv.activation is None
                    and not conv.dense_out and conv.backend == DCBackend.deltacnn
                    and conv.frame_idx >= 0 and type(conv_input) != Tensor)
         if fusable:
-            # conv.frame_idx >= 0: the convolution has seen its first frame, no bias from here on
+            # conv.frame_idx >= 0: the convolution has seen its first frame, no bias from here on;
+            # not self.first_iter: this layer's accumulated sum exists if it has an activation
             val_a, mask_a = a
             x, mask, plan, packed, _, _ = conv._prepare(conv_input)
             g = plan["g"]
@@ -431,7 +433,9 @@ class DCAdd(DCModule):
                 if self.mask_out is None or self.mask_out.shape != mask_a.shape:
                     self.mask_out = torch.empty_like(mask_a)
                 res = hk.sparse_conv_add(x, packed, mask, None, val_a, mask_a, plan["g"], self.out,
-                                         self.mask_out, self.weight_a, self.weight_b)
+                                         self.mask_out, self.weight_a, self.weight_b,
+                                         self.prev_out if self.activation is not None else None,
+                                         self.activation_int if self.activation is not None else 0)
                 if res is not None:
                     DCConv2d.conv_idx += 1
                     conv.frame_idx += 1

@@ -108,17 +108,22 @@ int dc_conv_act(const dc_geometry *g, const void *input, const void *filter,
                 int32_t *out_mask, void *prev_out, void *truncated, float threshold,
                 int activation, int truncation_mode, int dtype, void *stream);
 
-/* Fused pointwise conv + residual add: the DCAdd (sparse_layers.py:1086-1182, no activation, not
- * dense_out) that follows a bottleneck's last 1x1 convolution, in the convolution's launch:
- * out = weight_residual * residual [mask_residual] + weight_conv * conv(input) [mask], out_mask =
- * mask | mask_residual.  Results are identical to dc_conv followed by dc_add(residual, conv).  No
- * counterpart in the reference.  fp16, 1x1, stride 1, no padding, groups 1, Cin % 8 == 0,
- * Cout % 4 == 0 and a packed filter are required; anything else returns DC_ERR_UNSUPPORTED
- * before any launch so that the caller can issue the two separate calls. */
+/* Fused conv + residual add: the DCAdd (sparse_layers.py:1086-1182, not dense_out) that follows a
+ * block's last convolution, in the convolution's launch: with a = residual, b = conv(input),
+ * s = weight_residual * a [mask_residual] + weight_conv * b [mask]; activation == 0: out = s;
+ * activation > 0 (other_nn_layers.cu:1379-1559): prev_out += s, out = act(prev_out) - act(old
+ * prev_out).  out_mask = mask | mask_residual.  Results are identical to dc_conv followed by
+ * dc_add(residual, conv).  No counterpart in the reference.  Two forms exist: fp16 1x1 stride-1
+ * convolutions without padding (Cin % 8 == 0, Cout % 4 == 0, activation == 0), and small fp16
+ * layers of any kernel size (Cin % 8 == 0, groups 1, at most 64 taps,
+ * ceil(W/4) * ceil(H/4) * B * ceil(Cout/16) * Kh * Kw * ceil(Cin/32) <= 32768) with or without
+ * activation.  Both need a packed filter; anything else returns DC_ERR_UNSUPPORTED before any
+ * launch so that the caller can issue the two separate calls.  prev_out may be NULL when
+ * activation == 0. */
 int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filter,
                 const void *bias, const int32_t *mask, const void *residual,
                 const int32_t *mask_residual, void *out, int32_t *out_mask, float weight_residual,
-                float weight_conv, int dtype, void *stream);
+                float weight_conv, void *prev_out, int activation, int dtype, void *stream);
 
 /* Number of bytes dc_pack_filter writes for this geometry (0 if the shape has no packed
  * form).  One-time weight relayout for the MFMA kernels, fp16, un-swizzled, in fragment order

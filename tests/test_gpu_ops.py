@@ -480,6 +480,50 @@ def test_conv_add_fused(lib, cfg, weights):
     assert_masked_equal(out, two.cpu(), want_mask, "fused vs two calls")
 
 
+@pytest.mark.parametrize("cfg", [(32, 32, 3, 1, 1, 1, 1, 16, 16), (64, 64, 3, 1, 1, 1, 1, 12, 13),
+                                 (128, 128, 3, 1, 1, 1, 1, 8, 8), (24, 20, 3, 2, 1, 1, 1, 17, 19),
+                                 (16, 18, 5, 1, 2, 1, 1, 9, 9), (48, 32, 1, 1, 0, 1, 1, 10, 10)],
+                         ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("act", [0, 1, 3])
+@pytest.mark.parametrize("weights", [(1.0, 1.0), (0.5, -1.5)])
+def test_conv_add_fused_small_layers(lib, cfg, act, weights):
+    """dc_conv_add on small KxK layers, with the DCAdd's activation and accumulated sum: equal to
+    the oracle's conv + add, bit-identical to dc_conv followed by dc_add (outputs and state)."""
+    from deltacnn_amd.hip_kernels import conv_geometry
+    Cin, Cout = cfg[0], cfg[1]
+    dtype = torch.float16
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 93, 0.05)
+    want_conv, want_cm = ops.conv(x, mask, wt, None, s, p, d, groups)
+    B, _, Ho, Wo = want_conv.shape
+    g = _gen(94)
+    mres = rand_mask(g, B, Ho, Wo, 0.3)
+    res = torch.randn(B, Cout, Ho, Wo, generator=g).to(dtype)
+    prev = torch.randn(B, Cout, Ho, Wo, generator=g).to(dtype)
+    want_prev = prev.clone()
+    want, want_mask = ops.add(res, mres, want_conv, want_cm, want_prev if act else None, weights[0], weights[1], act, False)
+    assert 0 < int((want_cm & (1 - mres)).sum()) and 0 < int(((1 - want_cm) & mres).sum())  # both one-sided cases
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, Cin, Cout, 1)
+    dx, dm, dres, dmres = cl(poison(x, mask)), cl(mask), cl(poison(res, mres)), cl(mres)
+    geo = conv_geometry(x.shape, K, Cout, s, p, d, 1)
+    out = torch.full((B, Cout, Ho, Wo), float("nan"), dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+    om = torch.full((B, 1, Ho, Wo), -5, dtype=torch.int32, device=DEV)
+    p1 = cl(prev)
+    got = hk().sparse_conv_add(dx, pk, dm, None, dres, dmres, geo, out, om, weights[0], weights[1],
+                               p1 if act else None, act)
+    assert got is not None
+    assert torch.equal(om.cpu(), want_mask)
+    assert_masked_close(out, want, want_mask, 0, 2e-2, "out")
+    c_out, c_mask = hk().sparse_conv(dx, d_filt, dm, None, s, p, d, 1, c_out=Cout, create_out_mask=True, packed_filter=pk)
+    two, two_mask, p2 = torch.empty_like(out), torch.empty_like(om), cl(prev)
+    hk().sparse_add_tensors(dres, c_out, p2 if act else None, two, dmres, c_mask, two_mask, weights[0], weights[1], act, False)
+    assert torch.equal(two_mask, om)
+    assert_masked_equal(out, two.cpu(), want_mask, "fused vs two calls")
+    assert torch.equal(p1, p2)
+    if act:
+        assert_masked_close(p1, want_prev, torch.ones_like(want_mask), 0, 2e-2, "prev_out")
+
+
 # --------------------------------------------------------------------------------- pooling
 POOLS = [
     # C, K, stride, padding, dilation, H, W
