@@ -122,6 +122,43 @@ def run_dense(dense, frames, warmup, steps):
     return eager, graph
 
 
+def streams_bench(delta, dense, frames, batch=8, steps=64, warmup=16):
+    """Supplementary: `batch` independent video streams (the same clip at different offsets)
+    through ONE model instance as a batch, i.e. the same kernels on maps `batch` times larger.
+    Every stream keeps its own caches (they are the batch dimension of the layers' state).
+    Returns total frames/s for the delta path and for the dense model, both from HIP graphs."""
+    import torch
+    t, c, h, w = frames.shape
+    rows = frames.permute(0, 2, 3, 1).reshape(t, h * w * c)
+    unroll = 4
+    span = t - (2 + warmup + steps + unroll)
+    offsets = torch.arange(batch, device=frames.device) * max(1, span // batch)
+    assert int(offsets[-1]) + 2 + warmup + steps + unroll <= t
+
+    def fetch(index):
+        return rows.index_select(0, index).view(-1, batch, h, w, c).permute(0, 1, 4, 2, 3)
+
+    def timed(model, start):
+        index = ((start + torch.arange(unroll, device=frames.device))[:, None] + offsets[None, :]).reshape(-1)
+        graph = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(graph):
+            staged = fetch(index)
+            outs = [model(staged[i]) for i in range(unroll)]
+            index.add_(unroll)
+        return time_steps(graph.replay, -(-warmup // unroll), steps // unroll) / unroll
+
+    with torch.no_grad():
+        delta.reset_layers()
+        for i in range(2):  # dense first frame of every stream, one eager delta frame
+            delta(fetch(offsets + i)[0])
+        d = timed(delta, 2)
+        dense(fetch(offsets)[0])
+        dn = timed(dense, 2)
+        delta.reset_layers()
+    return {"streams": batch, "delta_fps_total": round(batch / d, 1), "dense_graph_fps_total": round(batch / dn, 1),
+            "ms_per_step": round(d * 1e3, 4)}
+
+
 def trace_kernels(delta, frames):
     """Device time per call and algorithmic bytes / flops of every library call of one delta
     frame.  The calls are recorded during an eager pass; each is then timed on the device by
@@ -371,6 +408,12 @@ def main():
     if os.path.exists(tpath):  # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
         with open(tpath) as f:
             traffic = json.load(f).get(dom_name, {}).get("bytes_per_launch")
+    streams = None
+    if not args.no_micro:
+        streams = [streams_bench(delta, dense, frames, batch=nb) for nb in (8, 32)]
+        for st in streams:
+            log(f"{st['streams']} streams as a batch: delta {st['delta_fps_total']:.0f} frames/s in total, "
+                f"dense graph {st['dense_graph_fps_total']:.0f}")
     micro = scaled = None
     if not args.no_micro:
         log("single-layer sweeps (64x64 fp16):")
@@ -412,6 +455,7 @@ def main():
                      "note": "latency-bound regime: the feature maps of this workload are <= 2.4 MB and "
                              "an empty dependent kernel in a HIP graph already costs ~1.6 us"},
         "cpu_baseline": cpu,
+        "streams_as_batch": streams,
         "micro": micro,
         "scaled": scaled,
     }

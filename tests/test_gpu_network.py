@@ -110,6 +110,35 @@ def test_mobilenet_32_frames(lib, dtype):
     assert e_dut <= 1.5 * e_ref + 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_mobilenet_batch_of_streams(lib, dtype):
+    """Three independent streams through one model instance as a batch (every stream's caches are
+    a slice of the layers' state) against the same streams processed one by one: the per-stream
+    outputs agree (fp32: 1e-4 relative on every frame; fp16: both track the dense model)."""
+    from deltacnn_amd.video import moving_rectangles_video
+    video = moving_rectangles_video(frames=30, height=64, width=64, n_rect=2, min_size=8, max_size=24)
+    state = _calibrated_state(video[:4])
+    dense, _, batch_model = _models(_mobilenet, dtype, 0.05, state)
+    offsets = (0, 7, 13)
+    frames = 12
+    with torch.no_grad():
+        outs = []
+        for t in range(frames):
+            x = torch.cat([video[o + t:o + t + 1] for o in offsets]).to(dtype)
+            outs.append(batch_model(cl(x)).float().cpu())
+        for b, o in enumerate(offsets):
+            _, _, single = _models(_mobilenet, dtype, 0.05, state)
+            for t in range(frames):
+                frame = video[o + t:o + t + 1].to(dtype)
+                got = single(cl(frame)).float().cpu()
+                want = outs[t][b:b + 1]
+                if dtype == torch.float32:
+                    assert float((got - want).abs().max()) <= 1e-4 * max(1.0, float(want.abs().max())), (b, t)
+                else:
+                    full = dense(frame.float())
+                    assert float((want - full).abs().max()) <= 1.5 * float((got - full).abs().max()) + 2e-2, (b, t)
+
+
 def test_mobilenet_unfolded_batchnorm(lib):
     """The reference topology with DCBatchNorm2d layers (un-folded checkpoint), fp32."""
     from deltacnn_amd.video import noise_block_video
