@@ -272,7 +272,7 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
     }
 }
 
-// Depthwise 3x3, stride 1, on large maps (bandwidth regime): one group of lanes computes a strip
+// Depthwise 3x3, stride 1, on maps of 4 MB and more (bandwidth regime): one group of lanes computes a strip
 // of PX consecutive output pixels of a row.  The 3 x (PX + 2) input rows of the strip are
 // loaded once (instead of 9 per pixel) and the filter stays in registers for the whole strip,
 // which cuts load instructions and conversions per output pixel by more than half.  Per pixel
@@ -1236,7 +1236,7 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
     const int nvec = g.in_c / N;
     // large maps: strips of four output pixels per group of lanes (see conv_dw_strip_kernel)
     if (g.kernel_h == 3 && g.kernel_w == 3 && g.stride_h == 1 && g.stride_w == 1 && g.dilation_h == 1 &&
-        g.dilation_w == 1 && nvec <= WAVE && P_out * g.in_c * (int64_t)sizeof(T) >= (32 << 20)) {
+        g.dilation_w == 1 && nvec <= WAVE && P_out * g.in_c * (int64_t)sizeof(T) >= (4 << 20)) {
         const int G = group_lanes(nvec, 1);
         const int lg = log2i(G);
         const int64_t strips = (int64_t)g.batch * g.out_h * ceil_div(g.out_w, 4);
