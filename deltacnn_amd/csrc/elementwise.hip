@@ -135,6 +135,48 @@ act_trunc_vec_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict_
                                    T(thr_f), mode);
 }
 
+// Large maps: a wavefront scans the mask words of 64 consecutive pixels in one coalesced read,
+// compacts the active ones by ballot and then works through them 64 / G pixels at a time.  With
+// one group per pixel a sparse map costs a wavefront launch per 64 / G pixels, most of which
+// leave at once; here a wavefront exists per 64 pixels and only active pixels occupy lanes.
+constexpr int SCAN_MIN_PIXELS = 1 << 16;
+
+template <typename T, int ACT>
+__global__ void __launch_bounds__(256)
+act_trunc_scan_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict__ trunc,
+                      int32_t *__restrict__ mask, float thr_f, int mode, int P, int C, int lg) {
+    constexpr int N = Vec16<T>::N;
+    __shared__ int s_list[4][WAVE];
+    const int G = 1 << lg;
+    const int wave = wave_id(), lane = lane_id();
+    const int pm = (blockIdx.x * 4 + wave) * WAVE + lane;
+    const bool on = pm < P && mask[min(pm, P - 1)] != 0;
+    const uint64_t bits = ballot(on);
+    if (bits == 0) return;
+    const int n = __popcll((unsigned long long)bits);
+    if (on) s_list[wave][__popcll((unsigned long long)(bits & ((1ull << lane) - 1ull)))] = pm;
+    const int gl = lane & (G - 1), grp = lane >> lg, ppi = WAVE >> lg;
+    constexpr int U = 2;  // pixels per group and pass: their loads are in flight together
+    for (int k = 0; k < n; k += U * ppi) {  // n is wave-uniform
+        Vec<T, N> dl[U][1], q[U][1], tr[U][1];
+        bool valid[U];
+        size_t p[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int idx = k + u * ppi + grp;
+            valid[u] = idx < n;
+            p[u] = (size_t)s_list[wave][min(idx, n - 1)];
+            if (valid[u] && gl * N < C) dl[u][0] = vload<T, N>(delta + p[u] * C + gl * N);
+            load_state<T, 1>(q[u], tr[u], valid[u], p[u], gl, G, C, prev, trunc);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (k + u * ppi < n)  // wave-uniform
+                act_trunc_pixel<T, 1, ACT>(dl[u], q[u], tr[u], valid[u], p[u], gl, G, C, delta, prev, trunc, mask,
+                                           T(thr_f), mode);
+    }
+}
+
 // Any C / alignment: scalar, two passes (decide, then recompute and write).
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -279,6 +321,68 @@ add_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ pre
             vstore<T, N>(prev + off, n);
         }
         vstore<T, N>(out + off, s);
+    }
+}
+
+// add_kernel for large maps: mask scan and compaction per wavefront (see act_trunc_scan_kernel).
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+add_scan_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ prev,
+                T *__restrict__ out, const int32_t *__restrict__ ma, const int32_t *__restrict__ mb,
+                int32_t *__restrict__ mo, float wa_f, float wb_f, int act, int P, int C, int lg) {
+    __shared__ int s_list[4][WAVE];
+    const T wa = T(wa_f), wb = T(wb_f);
+    const int G = 1 << lg;
+    const int wave = wave_id(), lane = lane_id();
+    const int p0 = (blockIdx.x * 4 + wave) * WAVE;
+    const int pm = p0 + lane;
+    const bool la = pm < P && ma[min(pm, P - 1)] != 0, lb = pm < P && mb[min(pm, P - 1)] != 0;
+    if (pm < P) mo[pm] = (la || lb) ? 1 : 0;
+    const uint64_t bits_a = ballot(la), bits_b = ballot(lb), bits = bits_a | bits_b;
+    if (bits == 0) return;
+    const int n = __popcll((unsigned long long)bits);
+    if (la || lb) s_list[wave][__popcll((unsigned long long)(bits & ((1ull << lane) - 1ull)))] = lane;
+    const int gl = lane & (G - 1), grp = lane >> lg, ppi = WAVE >> lg;
+    constexpr int U = 2;  // pixels per group and pass: their loads are in flight together
+    for (int k = 0; k < n; k += U * ppi) {
+        for (int c = gl * N; c < C; c += G * N) {
+            Vec<T, N> va[U], vb[U], q[U];
+            bool aa[U], ab[U], valid[U];
+            size_t off[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {  // operands of inactive sides read the row of the other side
+                const int idx = k + u * ppi + grp;
+                valid[u] = idx < n;
+                const int l = s_list[wave][min(idx, n - 1)];
+                aa[u] = (bits_a >> l) & 1ull;
+                ab[u] = (bits_b >> l) & 1ull;
+                off[u] = ((size_t)p0 + l) * C + c;
+                va[u] = vload<T, N>((aa[u] ? a : b) + off[u]);
+                vb[u] = vload<T, N>((ab[u] ? b : a) + off[u]);
+                if (act > 0) q[u] = vload<T, N>(prev + off[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (!valid[u]) continue;
+                Vec<T, N> s;
+#pragma unroll
+                for (int j = 0; j < N; ++j) s.v[j] = aa[u] ? va[u].v[j] * wa : T(0);
+                if (ab[u]) {
+#pragma unroll
+                    for (int j = 0; j < N; ++j) s.v[j] = fma_t(vb[u].v[j], wb, s.v[j]);
+                }
+                if (act > 0) {
+                    Vec<T, N> nn;
+#pragma unroll
+                    for (int j = 0; j < N; ++j) {
+                        nn.v[j] = s.v[j] + q[u].v[j];
+                        s.v[j] = act_apply<T>(nn.v[j], act) - act_apply<T>(q[u].v[j], act);
+                    }
+                    vstore<T, N>(prev + off[u], nn);
+                }
+                vstore<T, N>(out + off[u], s);
+            }
+        }
     }
 }
 
@@ -532,6 +636,21 @@ hipError_t act_trunc_t(T *delta, T *prev, T *trunc, int32_t *mask, float thr, in
         const int wide = mode == DC_TRUNC_MAX ? wide_group(nvec, P) : 0;
         int G = wide ? wide : pick_group(nvec, P, 4);
         int iters = ceil_div(nvec, G);
+        if (P >= SCAN_MIN_PIXELS && nvec <= WAVE) {
+            G = group_lanes(nvec, 1);
+            const int lg = log2i(G);
+            dim3 grid((unsigned)ceil_div(P, 4 * WAVE));
+            note_kernel("act_trunc_scan_kernel");
+            switch (act) {
+                case DC_ACT_RELU: act_trunc_scan_kernel<T, DC_ACT_RELU><<<grid, 256, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, lg); break;
+                case DC_ACT_RELU6: act_trunc_scan_kernel<T, DC_ACT_RELU6><<<grid, 256, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, lg); break;
+                case DC_ACT_LEAKY: act_trunc_scan_kernel<T, DC_ACT_LEAKY><<<grid, 256, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, lg); break;
+                case DC_ACT_SIGMOID: act_trunc_scan_kernel<T, DC_ACT_SIGMOID><<<grid, 256, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, lg); break;
+                case DC_ACT_SWISH: act_trunc_scan_kernel<T, DC_ACT_SWISH><<<grid, 256, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, lg); break;
+                default: act_trunc_scan_kernel<T, DC_ACT_LINEAR><<<grid, 256, 0, s>>>(delta, prev, trunc, mask, thr, mode, P, C, lg); break;
+            }
+            return hipGetLastError();
+        }
         GroupLaunch L(P, G);
         if (wide) {  // one pixel per workgroup
             L.block = wide;
@@ -557,6 +676,12 @@ hipError_t add_t(const T *a, const T *b, T *prev, T *out, const int32_t *ma, con
     constexpr int N = Vec16<T>::N;
     if (act < 0) act = 0;
     const bool vec = can_vec<T>(C, {a, b, prev, out});
+    if (!dense_out && vec && P >= SCAN_MIN_PIXELS) {
+        const int lg = log2i(group_lanes(C / N, 1));
+        note_kernel("add_scan_kernel");
+        add_scan_kernel<T, N><<<dim3((unsigned)ceil_div(P, 4 * WAVE)), 256, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, P, C, lg);
+        return hipGetLastError();
+    }
     GroupLaunch L(P, vec ? pick_group(C / N, P, 4) : group_lanes(C, 1));
     note_kernel(dense_out ? "add_dense_kernel" : "add_kernel");
     if (dense_out) {

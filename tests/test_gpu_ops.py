@@ -92,6 +92,57 @@ def test_activate_truncate_large_map(lib, dtype, C, H, W):
     assert torch.equal(d[1].cpu(), w[1]) and torch.equal(d[2].cpu(), w[2])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C,act,mode", [(40, 1, 0), (64, 3, 1), (8, 2, 2), (264, 1, 0)])
+@pytest.mark.parametrize("density", [0.02, 0.6])
+def test_activate_truncate_scanned_map(lib, dtype, C, act, mode, density):
+    """Maps of 65536 pixels and more: mask scan and compaction per wavefront (uneven tail)."""
+    g = _gen(260 + C)
+    B, H, W = 2, 190, 181
+    mask = rand_mask(g, B, H, W, density)
+    prev = (torch.randn(B, C, H, W, generator=g) * 3).to(dtype)
+    trunc = (torch.randn(B, C, H, W, generator=g) * 0.005).to(dtype)
+    big = rand_mask(g, B, H, W, 0.5).float()
+    delta = (torch.randn(B, C, H, W, generator=g) * (0.005 + 0.5 * big)).to(dtype)
+    w = [delta.clone(), prev.clone(), trunc.clone(), mask.clone()]
+    ops.activate_truncate(*w, 0.1, act, mode)
+    d = [cl(poison(delta, mask)), cl(prev), cl(trunc), cl(mask)]
+    hk().sparse_activation(*d, 0.1, act, mode)
+    if mode == 0:
+        assert torch.equal(d[3].cpu(), w[3])
+        assert_masked_equal(d[0], w[0], w[3], "delta")
+        assert torch.equal(d[1].cpu(), w[1]) and torch.equal(d[2].cpu(), w[2])
+    else:  # norm / rms: the sum order differs from the oracle's, decisions may differ at ties
+        agree = (d[3].cpu() == w[3])
+        assert float(agree.float().mean()) > 0.999
+        both = (agree & (w[3] != 0)).to(torch.int32)
+        assert_masked_equal(d[0], w[0], both, "delta")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [24, 64, 520])
+@pytest.mark.parametrize("act", [-1, 1])
+def test_add_scanned_map(lib, dtype, C, act):
+    g = _gen(640 + C)
+    B, H, W = 2, 190, 181
+    ma, mb = rand_mask(g, B, H, W, 0.05), rand_mask(g, B, H, W, 0.3)
+    a = torch.randn(B, C, H, W, generator=g).to(dtype)
+    b = torch.randn(B, C, H, W, generator=g).to(dtype)
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype) if act > 0 else None
+    w_prev = prev.clone() if act > 0 else None
+    w_out, w_mask = ops.add(a, ma, b, mb, w_prev, 0.5, -1.25, act, False)
+    d_prev = cl(prev) if act > 0 else None
+    d_out = torch.full((B, C, H, W), float("nan"), dtype=dtype, device=DEV).contiguous(
+        memory_format=torch.channels_last)
+    d_mo = torch.full((B, 1, H, W), -3, dtype=torch.int32, device=DEV)
+    hk().sparse_add_tensors(cl(poison(a, ma)), cl(poison(b, mb)), d_prev, d_out, cl(ma), cl(mb), d_mo,
+                            0.5, -1.25, act, False)
+    assert torch.equal(d_mo.cpu(), w_mask)
+    assert_masked_equal(d_out, w_out, w_mask, "out")
+    if act > 0:
+        assert torch.equal(d_prev.cpu(), w_prev)
+
+
 # ------------------------------------------------------------------ activation + truncation
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("C", CHANNELS)
