@@ -954,7 +954,7 @@ struct PatchRes {  // DCAdd fused behind the convolution: a = residual, b = conv
 // activation the sum is accumulated in `prev` and its activated difference is emitted -- the
 // arithmetic of add_kernel applied to the convolution result rounded to fp16, so the output
 // equals that of the two separate launches bit for bit.
-template <bool TR, int KW, int R, int S, bool ADD>
+template <bool TR, int KW, int R, int S, bool ADD, bool K3>
 __global__ void __launch_bounds__(KW * WAVE)
 conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                        const half_t *__restrict__ bias, half_t *__restrict__ out,
@@ -967,7 +967,8 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     const int l16 = lane & 15, kq = lane >> 4;
     const int oy = blockIdx.y * 4 + (l16 >> 2), ox = blockIdx.x * 4 + (l16 & 3);
     const bool inside = oy < p.Ho && ox < p.Wo;
-    const int K2 = p.Kh * p.Kw;
+    const int K2 = K3 ? 9 : p.Kh * p.Kw;  // K3: a 3x3 kernel, tap arithmetic with constants
+    const int Kw = K3 ? 3 : p.Kw;
     const int co_tiles = (p.Co + 15) >> 4;
     const int ksteps = ci_p >> 5;
     const int total = K2 * ksteps;
@@ -991,7 +992,7 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
             const int tap = t0 + kq + 4 * j;
             src[j] = -1;
             if (tap < K2) {
-                const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
+                const int ky = tap / Kw, kx = tap - ky * Kw;
                 int iy = 0, ix = 0;
                 if (inside && tap_src<TR>(oy, ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
                     tap_src<TR>(ox, kx, p.sw, p.dw, p.pl, p.Wi, ix))
@@ -1344,8 +1345,14 @@ hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *p
     PatchRes rs{nullptr, nullptr, nullptr, 0.f, 0.f, 0};
     if (res != nullptr)
         rs = PatchRes{(const half_t *)res->values, res->mask, (half_t *)res->prev, res->wa, res->wb, res->act};
+    const bool k3 = g.kernel_h == 3 && g.kernel_w == 3;
     note_kernel("conv_patch_mfma_kernel");
-#define DC_PATCH_L(TRF, KWV, RV, SV, AV) conv_patch_mfma_kernel<TRF, KWV, RV, SV, AV><<<pgrid, KWV * WAVE, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbk, ci_p, rs)
+#define DC_PATCH_ARGS (p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbk, ci_p, rs)
+#define DC_PATCH_L(TRF, KWV, RV, SV, AV)                                                                      \
+    do {                                                                                                      \
+        if (k3) conv_patch_mfma_kernel<TRF, KWV, RV, SV, AV, true><<<pgrid, KWV * WAVE, 0, s>>> DC_PATCH_ARGS; \
+        else conv_patch_mfma_kernel<TRF, KWV, RV, SV, AV, false><<<pgrid, KWV * WAVE, 0, s>>> DC_PATCH_ARGS;  \
+    } while (0)
 #define DC_PATCH(TRF, AV)                                                                       \
     do {                                                                                        \
         if (kwv == 1) { if (rv == 2) DC_PATCH_L(TRF, 1, 2, 6, AV); else DC_PATCH_L(TRF, 1, 1, 12, AV); } \
@@ -1357,6 +1364,7 @@ hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *p
     else DC_PATCH(false, false);
 #undef DC_PATCH
 #undef DC_PATCH_L
+#undef DC_PATCH_ARGS
     return hipGetLastError();
 }
 
