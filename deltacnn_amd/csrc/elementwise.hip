@@ -139,7 +139,7 @@ act_trunc_vec_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict_
 // compacts the active ones by ballot and then works through them 64 / G pixels at a time.  With
 // one group per pixel a sparse map costs a wavefront launch per 64 / G pixels, most of which
 // leave at once; here a wavefront exists per 64 pixels and only active pixels occupy lanes.
-constexpr int SCAN_MIN_PIXELS = 1 << 16;
+constexpr int SCAN_MIN_PIXELS = 1 << 18;  // 4096 wavefronts: enough to fill the chip
 
 template <typename T, int ACT>
 __global__ void __launch_bounds__(256)

@@ -93,12 +93,12 @@ def test_activate_truncate_large_map(lib, dtype, C, H, W):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("C,act,mode", [(40, 1, 0), (64, 3, 1), (8, 2, 2), (264, 1, 0)])
+@pytest.mark.parametrize("C,act,mode", [(40, 1, 0), (64, 3, 1), (8, 2, 2), (136, 1, 0)])
 @pytest.mark.parametrize("density", [0.02, 0.6])
 def test_activate_truncate_scanned_map(lib, dtype, C, act, mode, density):
-    """Maps of 65536 pixels and more: mask scan and compaction per wavefront (uneven tail)."""
+    """Maps of 262144 pixels and more: mask scan and compaction per wavefront (uneven tail)."""
     g = _gen(260 + C)
-    B, H, W = 2, 190, 181
+    B, H, W = 2, 401, 331
     mask = rand_mask(g, B, H, W, density)
     prev = (torch.randn(B, C, H, W, generator=g) * 3).to(dtype)
     trunc = (torch.randn(B, C, H, W, generator=g) * 0.005).to(dtype)
@@ -120,11 +120,11 @@ def test_activate_truncate_scanned_map(lib, dtype, C, act, mode, density):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("C", [24, 64, 520])
+@pytest.mark.parametrize("C", [24, 64, 136])
 @pytest.mark.parametrize("act", [-1, 1])
 def test_add_scanned_map(lib, dtype, C, act):
     g = _gen(640 + C)
-    B, H, W = 2, 190, 181
+    B, H, W = 2, 401, 331
     ma, mb = rand_mask(g, B, H, W, 0.05), rand_mask(g, B, H, W, 0.3)
     a = torch.randn(B, C, H, W, generator=g).to(dtype)
     b = torch.randn(B, C, H, W, generator=g).to(dtype)
