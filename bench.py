@@ -293,6 +293,49 @@ def scaled_bench():
     return out
 
 
+def network_bench(which, steps, warmup):
+    """The two larger configurations (parity cases, not the headline): HRNet-W32 pose network at
+    256x256 and the DLA-34 CenterNet detector at 544x960, fp16, batch 1, random-init weights
+    rescaled on two frames, threshold 0.05; synthetic static-camera clips (one large moving blob /
+    twelve pedestrian-sized rectangles, no sensor noise)."""
+    import torch
+    from deltacnn_amd import sparse_layers as SL
+    from deltacnn_amd.networks import DLA34CenterNet, DenseLayers, HRNet, fold_data_statistics
+    from deltacnn_amd.video import moving_rectangles_video
+    builder, size, kw = {
+        "hrnet": (HRNet, (256, 256), dict(n_rect=1, min_size=100, max_size=180, min_speed=2, max_speed=6)),
+        "dla34": (DLA34CenterNet, (544, 960), dict(n_rect=12, min_size=30, max_size=200, min_speed=1, max_speed=5)),
+    }[which]
+    video = moving_rectangles_video(frames=steps + warmup + 3 + UNROLL, height=size[0], width=size[1],
+                                    noise_sigma=0.0, **kw)
+    torch.manual_seed(0)
+    dense = builder(DenseLayers).eval().to("cuda", memory_format=torch.channels_last)
+    with torch.no_grad():
+        fold_data_statistics(dense, video[:2].to("cuda").contiguous(memory_format=torch.channels_last))
+    state = {k: v.clone() for k, v in dense.state_dict().items()}
+    dense = dense.half()
+    SL.DCThreshold.t_default = THRESHOLD
+    delta = builder(SL).eval()
+    delta.load_state_dict(state)
+    delta = delta.to("cuda", memory_format=torch.channels_last).half()
+    delta.process_filters()
+    frames = gpu_frames(video)
+    sec = run_delta(delta, frames, warmup, steps, "graph")
+    dense_eager, dense_graph = run_dense(dense, frames, warmup, steps)
+    agg, rows = trace_kernels(delta, frames)
+    return {
+        "network": which, "input": list(size), "value": round(1 / sec, 1), "unit": "frames/s",
+        "ms_per_step": round(sec * 1e3, 4), "steps": steps, "warmup": warmup,
+        "dense_gpu": {"eager_fps": round(1 / dense_eager, 1), "graph_fps": round(1 / dense_graph, 1),
+                      "speedup_vs_dense_gpu": round(min(dense_eager, dense_graph) / sec, 3)},
+        "mean_input_density_of_library_calls": round(sum(r["density_in"] for r in rows) / len(rows), 3),
+        "kernels": {k: {"launches_per_frame": a["launches"], "us_per_launch": round(a["us_per_launch"], 3),
+                        "ms_per_frame": round(a["ms_per_frame"], 4), "alg_GBps": round(a["GBps"], 1),
+                        "alg_TFLOPs": round(a["TFLOPs"], 2)}
+                    for k, a in sorted(agg.items(), key=lambda kv: -kv[1]["ms"])},
+    }
+
+
 def cpu_baseline(state, video, n_frames, threads):
     """The CPU oracle of the delta path (pure PyTorch, fp32) on this host, bounded sample."""
     import torch
@@ -335,6 +378,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="with --only-delta: end with one 256 MiB device-to-device copy kernel, the known-size "
                          "reference that hardware traffic counters of a profiling run are scaled by")
+    ap.add_argument("--network", choices=["mobilenetv2", "hrnet", "dla34"], default="mobilenetv2",
+                    help="hrnet / dla34: time that configuration instead and print a short JSON line")
     ap.add_argument("--only-micro", action="store_true",
                     help="run the single-layer and scaled-shape sections only (for profiling runs)")
     ap.add_argument("--cpu-frames", type=int, default=200,
@@ -356,6 +401,10 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     if args.only_micro:
         print(json.dumps({"micro": micro_bench(), "scaled": scaled_bench()}), flush=True)
+        return
+    if args.network != "mobilenetv2":
+        steps = args.steps - args.steps % UNROLL if args.steps >= UNROLL else args.steps
+        print(json.dumps(network_bench(args.network, min(steps, 64), min(args.warmup, 16))), flush=True)
         return
 
     n_frames = args.warmup + args.steps + 3 + UNROLL
