@@ -689,7 +689,7 @@ constexpr int LDS_MAX_HALO = 1024;
 constexpr int LDS_MAX_STEPS = 1024;
 
 template <int R, int S, int D, int KS>
-__global__ void __launch_bounds__(4 * WAVE)
+__global__ void __launch_bounds__(8 * WAVE)
 conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                      const half_t *__restrict__ bias, half_t *__restrict__ out,
                      const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
@@ -1415,12 +1415,16 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                 const int64_t tiles = (int64_t)tx * ty * g.batch;
                 // Arrangements (R channel tiles per wavefront, KS reduction slices, channel groups):
                 // wide outputs on many tiles: R = 2, four channel groups; otherwise, with enough
-                // steps to split, R = 2 and two slices (x two or one channel groups); short
+                // steps to split, R = 2 and two or four slices (x two or one channel groups); short
                 // reductions: R = 1, up to four channel groups.
                 const int nsteps_chunk = g.kernel_h * g.kernel_w * kcc;
                 int rl = 1, ksl = 1, ncw = std::min(4, co_tiles);
                 if (co_tiles >= 16 && tiles * ceil_div(co_tiles, 8) >= 512) { rl = 2; ncw = 4; }
-                else if (nsteps_chunk >= 16 && co_tiles >= 4) { rl = 2; ksl = 2; ncw = 2; }
+                else if (nsteps_chunk >= 16 && co_tiles >= 4) {
+                    // fewer workgroups than compute units and a long reduction: eight wavefronts
+                    rl = 2; ncw = 2;
+                    ksl = (nsteps_chunk >= 36 && tiles * ceil_div(co_tiles, 4) < 256) ? 4 : 2;
+                }
                 else if (nsteps_chunk >= 16 && co_tiles >= 2) { rl = 2; ksl = 4; ncw = 1; }
                 const int nwv = ncw * ksl;  // wavefronts per workgroup
                 const int cbl = ceil_div(co_tiles, ncw * rl);

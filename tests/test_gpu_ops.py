@@ -325,6 +325,7 @@ CONVS = [
     (16, 64, 3, 1, 1, 1, 1, 120, 120),      # short reduction: one tile per wave, four channel groups
     (32, 256, 3, 1, 1, 1, 1, 90, 90),       # wide output on many tiles: two tiles per wave, no split
     (320, 32, 3, 1, 1, 1, 1, 40, 40),       # input channels staged in two chunks
+    (128, 128, 3, 1, 1, 1, 1, 40, 40),      # few tiles, long reduction: eight waves, steps split four ways
     (64, 80, 3, 2, 1, 1, 1, 120, 121),      # stride 2
     (64, 48, 3, 1, 2, 2, 1, 80, 81),        # dilation 2
     (32, 64, 5, 1, 2, 1, 1, 64, 66),        # 5x5
