@@ -1421,9 +1421,9 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                 int rl = 1, ksl = 1, ncw = std::min(4, co_tiles);
                 if (co_tiles >= 16 && tiles * ceil_div(co_tiles, 8) >= 512) { rl = 2; ncw = 4; }
                 else if (nsteps_chunk >= 16 && co_tiles >= 4) {
-                    // fewer workgroups than compute units and a long reduction: eight wavefronts
+                    // no more workgroups than compute units and a long reduction: eight wavefronts
                     rl = 2; ncw = 2;
-                    ksl = (nsteps_chunk >= 36 && tiles * ceil_div(co_tiles, 4) < 256) ? 4 : 2;
+                    ksl = (nsteps_chunk >= 36 && tiles * ceil_div(co_tiles, 4) <= 256) ? 4 : 2;
                 }
                 else if (nsteps_chunk >= 16 && co_tiles >= 2) { rl = 2; ksl = 4; ncw = 1; }
                 const int nwv = ncw * ksl;  // wavefronts per workgroup
