@@ -394,7 +394,7 @@ __global__ void __launch_bounds__(256)
 conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
                    const T *__restrict__ bias, T *__restrict__ out,
                    const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, EpiP epi,
-                   int lg) {
+                   int lg, int staged) {
     constexpr int N = Vec16<T>::N;
     constexpr int MAXCI = 4;
     const int G = 1 << lg;
@@ -415,20 +415,22 @@ conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
     T *s_w = reinterpret_cast<T *>(s_raw);
     float xin[K3 ? 9 : 1][MAXCI];
     Vec<T, N> q[1], tr[1];
-    if (K3) {
+    if (K3 || staged) {  // the filter, un-swizzled, in [tap][ci][co] order
         const int cv = C / N;  // 16-byte vectors per filter row (C % N == 0, so w_co == C)
-        const int total = 9 * p.Ci * cv;
+        const int total = K2 * p.Ci * cv;
         for (int i = threadIdx.x; i < total; i += blockDim.x) {
             const int v = i % cv, r2 = i / cv;
             const int ci = r2 % p.Ci, t = r2 / p.Ci;
-            Vec<T, N> w = vload<T, N>(filter + ((size_t)ci * 9 + t) * p.w_co + v * N);
+            Vec<T, N> w = vload<T, N>(filter + ((size_t)ci * K2 + t) * p.w_co + v * N);
             if (p.swz) {  // odd output channels live in the partner row of the pair swizzle
-                const Vec<T, N> w1 = vload<T, N>(filter + ((size_t)(ci ^ 1) * 9 + t) * p.w_co + v * N);
+                const Vec<T, N> w1 = vload<T, N>(filter + ((size_t)(ci ^ 1) * K2 + t) * p.w_co + v * N);
 #pragma unroll
                 for (int j = 1; j < N; j += 2) w.v[j] = w1.v[j];
             }
             vstore<T, N>(s_w + (size_t)i * N, w);
         }
+    }
+    if (K3) {
         const int pc = valid ? po : 0;
         const int cb = pc / (p.Ho * p.Wo), cr = pc - cb * p.Ho * p.Wo;
         const int cy = cr / p.Wo, cx = cr - cy * p.Wo;
@@ -447,8 +449,8 @@ conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
             q[0] = vload<T, N>((const T *)epi.prev + (size_t)pc * C + cc);
             tr[0] = vload<T, N>((const T *)epi.trunc + (size_t)pc * C + cc);
         }
-        __syncthreads();
     }
+    if (K3 || staged) __syncthreads();
 
     uint64_t taps = 0;
     for (int j = 0; j < K2; j += G) {
@@ -484,6 +486,40 @@ conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
                     const Vec<T, N> w = vload<T, N>(s_w + (size_t)(t * p.Ci + ci) * C + c);
 #pragma unroll
                     for (int j = 0; j < N; ++j) acc[j] = __builtin_fmaf(xv, float(w.v[j]), acc[j]);
+                }
+            }
+        }
+    } else if (staged) {
+        // any kernel size with the filter in LDS: the inputs of up to seven taps of a filter row
+        // are requested together from clamped addresses and zero-selected afterwards
+        if (lane_on) {
+            constexpr int RW = 7;
+            const T *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+            for (int ky = 0; ky < p.Kh; ++ky) {
+                const int iy = min(max(oy * p.sh - p.pt + ky * p.dh, 0), p.Hi - 1);
+                for (int kx0 = 0; kx0 < p.Kw; kx0 += RW) {
+                    float xr[RW][MAXCI];
+#pragma unroll
+                    for (int u = 0; u < RW; ++u) {
+                        const int ix = min(max(ox * p.sw - p.pl + min(kx0 + u, p.Kw - 1) * p.dw, 0), p.Wi - 1);
+                        const T *xp = inb + (size_t)(iy * p.Wi + ix) * p.Ci;
+#pragma unroll
+                        for (int ci = 0; ci < MAXCI; ++ci) xr[u][ci] = float(xp[min(ci, p.Ci - 1)]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < RW; ++u) {
+                        if (kx0 + u >= p.Kw) break;  // uniform
+                        const int t = ky * p.Kw + kx0 + u;
+                        const bool on = (taps >> t) & 1ull;
+#pragma unroll
+                        for (int ci = 0; ci < MAXCI; ++ci) {
+                            if (ci >= p.Ci) break;
+                            const float xv = on ? xr[u][ci] : 0.f;
+                            const Vec<T, N> w = vload<T, N>(s_w + (size_t)(t * p.Ci + ci) * C + c);
+#pragma unroll
+                            for (int j = 0; j < N; ++j) acc[j] = __builtin_fmaf(xv, float(w.v[j]), acc[j]);
+                        }
+                    }
                 }
             }
         }
@@ -1300,11 +1336,14 @@ bool try_fewcin(const dc_geometry &g, const ConvP &p, const T *in, const T *filt
     const int lg = log2i(G);
     note_kernel("conv_fewcin_kernel");
     const bool k3 = g.kernel_h == 3 && g.kernel_w == 3;
-    const size_t lds = k3 ? (size_t)9 * g.in_c * g.out_c * sizeof(T) : 0;
+    // the un-swizzled filter goes to LDS when it fits (always for 3x3)
+    const size_t fbytes = (size_t)g.kernel_h * g.kernel_w * g.in_c * g.out_c * sizeof(T);
+    const int staged = !k3 && fbytes <= (32 << 10) ? 1 : 0;
+    const size_t lds = (k3 || staged) ? fbytes : 0;
 #define DC_FC(A)                                                                                              \
     do {                                                                                                      \
-        if (k3) conv_fewcin_kernel<T, A, true><<<grid, block, lds, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg); \
-        else conv_fewcin_kernel<T, A, false><<<grid, block, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg);     \
+        if (k3) conv_fewcin_kernel<T, A, true><<<grid, block, lds, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg, 0); \
+        else conv_fewcin_kernel<T, A, false><<<grid, block, lds, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg, staged); \
     } while (0)
     switch (act) {
         case DC_ACT_LINEAR: DC_FC(DC_ACT_LINEAR); break;
