@@ -20,7 +20,10 @@ struct PoolQ {          // the literal zero that joins the maximum for bottom / 
     int pb, pr;
 };
 
-template <typename T, int N, bool MAX>
+// K = 2, 3: square window of that size -- mask words, deltas and cached inputs of all taps are
+// requested together from clamped addresses and selected afterwards (one memory round trip per
+// output instead of one per tap); K = 0: any window, tap by tap.  Same order of operations.
+template <typename T, int N, bool MAX, int K>
 __global__ void __launch_bounds__(256)
 pool_window_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restrict__ prev,
                    T *__restrict__ out, const int32_t *__restrict__ mask,
@@ -46,7 +49,21 @@ pool_window_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restri
                 hi[j] = MAX ? -INFINITY : 0.f;
                 hp[j] = -INFINITY;
             }
-            for (int ky = 0; ky < p.Kh; ++ky) {
+            constexpr int KK = K > 0 ? K * K : 1;
+            Vec<T, N> pd[KK], pp[KK];
+            int pm[KK];
+            if (K > 0) {
+#pragma unroll
+                for (int t = 0; t < KK; ++t) {
+                    const int iy = min(max(oy * p.sh - p.pt + (t / K) * p.dh, 0), p.Hi - 1);
+                    const int ix = min(max(ox * p.sw - p.pl + (t % K) * p.dw, 0), p.Wi - 1);
+                    const int ip = iy * p.Wi + ix;
+                    pm[t] = mb[ip];
+                    pd[t] = vload<T, N>(inb + (size_t)ip * C + c);
+                    if (MAX) pp[t] = vload<T, N>(pvb + (size_t)ip * C + c);
+                }
+            }
+            for (int ky = 0; ky < (K > 0 ? K : p.Kh); ++ky) {  // constant trip counts unroll fully
                 const int iy = oy * p.sh - p.pt + ky * p.dh;
                 if (iy < 0) continue;
                 if (iy >= p.Hi) {
@@ -59,7 +76,7 @@ pool_window_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restri
                     }
                     continue;
                 }
-                for (int kx = 0; kx < p.Kw; ++kx) {
+                for (int kx = 0; kx < (K > 0 ? K : p.Kw); ++kx) {
                     const int ix = ox * p.sw - p.pl + kx * p.dw;
                     if (ix < 0) continue;
                     if (ix >= p.Wi) {
@@ -73,14 +90,15 @@ pool_window_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restri
                         continue;
                     }
                     const int ip = iy * p.Wi + ix;
-                    const bool act = mb[ip] != 0;
+                    const int t = K > 0 ? ky * K + kx : 0;
+                    const bool act = (K > 0 ? pm[t] : mb[ip]) != 0;
                     if (!MAX && !act) continue;
                     Vec<T, N> d;
 #pragma unroll
                     for (int j = 0; j < N; ++j) d.v[j] = T(0);
-                    if (act) d = vload<T, N>(inb + (size_t)ip * C + c);
+                    if (act) d = K > 0 ? pd[t] : vload<T, N>(inb + (size_t)ip * C + c);
                     if (MAX) {
-                        Vec<T, N> pv = vload<T, N>(pvb + (size_t)ip * C + c);
+                        Vec<T, N> pv = K > 0 ? pp[t] : vload<T, N>(pvb + (size_t)ip * C + c);
 #pragma unroll
                         for (int j = 0; j < N; ++j) {
                             float pf = float(pv.v[j]);
@@ -277,7 +295,13 @@ hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, c
                      ((uintptr_t)prev & 15) == 0;
     int G = pow2_ceil(vec ? g.in_c / N : g.in_c);
     if (G > WAVE) G = WAVE;
-#define DC_POOL(NN, MX) pool_window_kernel<T, NN, MX><<<grid, 256, 0, s>>>(p, q, in, prev, (T *)out, mask, out_mask, G)
+    const int ksq = (g.kernel_h == g.kernel_w && (g.kernel_h == 2 || g.kernel_h == 3)) ? g.kernel_h : 0;
+#define DC_POOL(NN, MX)                                                                                           \
+    do {                                                                                                          \
+        if (ksq == 2) pool_window_kernel<T, NN, MX, 2><<<grid, 256, 0, s>>>(p, q, in, prev, (T *)out, mask, out_mask, G); \
+        else if (ksq == 3) pool_window_kernel<T, NN, MX, 3><<<grid, 256, 0, s>>>(p, q, in, prev, (T *)out, mask, out_mask, G); \
+        else pool_window_kernel<T, NN, MX, 0><<<grid, 256, 0, s>>>(p, q, in, prev, (T *)out, mask, out_mask, G);   \
+    } while (0)
     if (mode == DC_POOL_MAX) {
         if (vec) DC_POOL(N, true); else DC_POOL(1, true);
     } else {
