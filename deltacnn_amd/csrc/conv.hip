@@ -724,7 +724,7 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 constexpr int LDS_MAX_HALO = 1024;
 constexpr int LDS_MAX_STEPS = 1024;
 
-template <int R, int S, int D, int KS>
+template <int R, int S, int D, int KS, bool TR>
 __global__ void __launch_bounds__(8 * WAVE)
 conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                      const half_t *__restrict__ bias, half_t *__restrict__ out,
@@ -737,14 +737,34 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
     __shared__ int s_list[TILE_PX];
     __shared__ int s_n;
     const int b = blockIdx.z / co_blocks, cb = blockIdx.z % co_blocks;
-    const int ty0 = blockIdx.y * TILE, tx0 = blockIdx.x * TILE;
+    // TR (transposed, dilation 1): the outputs of one stride phase (py, px) form an ordinary
+    // convolution of the input with the A x Bt filter taps ky = ry + a * stride, kx = rx + b * stride:
+    // out[(J * sh + py), (I * sw + px)] = sum_ab W[ky][kx] * in[J + qy - a][I + qx - b].  A tile is
+    // 8 x 8 such outputs (J, I); blockIdx = (tile, phase) interleaved.
+    const int ys = TR ? p.sh : 1, xs = TR ? p.sw : 1;
+    const int phy = blockIdx.y % ys, phx = blockIdx.x % xs;
+    const int ty0 = (blockIdx.y / ys) * TILE, tx0 = (blockIdx.x / xs) * TILE;
+    const int ry = TR ? (phy + p.pt) % p.sh : 0, rx = TR ? (phx + p.pl) % p.sw : 0;
+    const int A = TR ? (p.Kh - ry + p.sh - 1) / p.sh : p.Kh;   // taps of this tile per dimension
+    const int Bt = TR ? (p.Kw - rx + p.sw - 1) / p.sw : p.Kw;
+    const int Amax = (p.Kh + p.sh - 1) / p.sh, Bmax = (p.Kw + p.sw - 1) / p.sw;
+    const int VK2 = A * Bt;
+    // output coordinate of tile pixel (ly, lx); halo step per output step
+    auto out_y = [&](int ly) { return TR ? (ty0 + ly) * ys + phy : ty0 + ly; };
+    auto out_x = [&](int lx) { return TR ? (tx0 + lx) * xs + phx : tx0 + lx; };
+    const int vsy = TR ? 1 : p.sh, vsx = TR ? 1 : p.sw;
+    // halo element offset of tap (a, b2) relative to an output's halo origin
+    auto tap_off = [&](int a, int b2) {
+        return TR ? (Amax - 1 - a) * hal_w + (Bmax - 1 - b2) : a * p.dh * hal_w + b2 * p.dw;
+    };
     const int tid = threadIdx.x, nthr = blockDim.x, nw = nthr / WAVE;
     const int wv = wave_id(), lane = lane_id();
     // wavefront = (channel group cw, reduction slice kz): slice kz takes steps kz, kz + KS, ...
     const int ncw = nw / KS, cw = wv % ncw, kz = wv / ncw;
     const int l16 = lane & 15, kq = lane >> 4;
     const int hpx = hal_h * hal_w;
-    const int iy0 = ty0 * p.sh - p.pt, ix0 = tx0 * p.sw - p.pl;
+    const int iy0 = TR ? ty0 + (phy + p.pt - ry) / p.sh - (Amax - 1) : ty0 * p.sh - p.pt;
+    const int ix0 = TR ? tx0 + (phx + p.pl - rx) / p.sw - (Bmax - 1) : tx0 * p.sw - p.pl;
     const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
     const int co_tiles = (p.Co + 15) >> 4;
     const int ksteps = ci_p >> 5;
@@ -755,15 +775,23 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
     // its input fragment relative to a pixel's halo origin, and its fragment offset in the
     // packed filter.  Entries past the last step repeat it (their products are zeroed).
     auto build_steps = [&](int kbase, int kcur) {
-        const int nsteps = K2 * kcur;
+        const int nsteps = VK2 * kcur;
         const int padded = (nsteps + S * D * KS - 1) / (S * D * KS) * (S * D * KS);
         for (int j = tid; j < padded; j += nthr) {
             const int jj = min(j, nsteps - 1);
             const int tap = jj / kcur, ks = jj - tap * kcur;
-            const int ky = tap / p.Kw, kx = tap - ky * p.Kw;
-            s_step[j] = int2{(ky * p.dh * hal_w + kx * p.dw) * row + ks * 64, (tap * ksteps + kbase + ks) * 512};
+            const int ta = tap / Bt, tb = tap - ta * Bt;
+            const int real = TR ? (ry + ta * p.sh) * p.Kw + rx + tb * p.sw : tap;  // tap of the filter
+            s_step[j] = int2{tap_off(ta, tb) * row + ks * 64, (real * ksteps + kbase + ks) * 512};
         }
     };
+    if (TR && VK2 == 0) {  // a phase without taps (kernel smaller than the stride): nothing updated
+        if (cb == 0 && tid < WAVE) {
+            const int oy = out_y(tid >> 3), ox = out_x(tid & 7);
+            if (oy < p.Ho && ox < p.Wo) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = 0;
+        }
+        return;
+    }
     build_steps(0, min(kcc, ksteps));
     // halo table: global pixel index of every active in-bounds halo pixel, -1 otherwise
     for (int i = tid; i < hpx; i += nthr) {
@@ -809,13 +837,14 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
 
     if (tid < WAVE) {  // dilate the mask over the window, compact the updated pixels
         const int ly = tid >> 3, lx = tid & 7;
-        const bool inb = ty0 + ly < p.Ho && tx0 + lx < p.Wo;
+        const int oy = out_y(ly), ox = out_x(lx);
+        const bool inb = oy < p.Ho && ox < p.Wo;
         bool upd = false;
-        const int base = ly * p.sh * hal_w + lx * p.sw;
-        for (int ky = 0; ky < p.Kh; ++ky)
-            for (int kx = 0; kx < p.Kw; ++kx) upd |= s_hpix[base + ky * p.dh * hal_w + kx * p.dw] >= 0;
+        const int base = ly * vsy * hal_w + lx * vsx;
+        for (int ta = 0; ta < A; ++ta)
+            for (int tb = 0; tb < Bt; ++tb) upd |= s_hpix[base + tap_off(ta, tb)] >= 0;
         upd = upd && inb;
-        if (inb && cb == 0) out_mask[((size_t)b * p.Ho + ty0 + ly) * p.Wo + tx0 + lx] = upd ? 1 : 0;
+        if (inb && cb == 0) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = upd ? 1 : 0;
         int n;
         const int rank = wave_rank(upd, n);
         if (upd) s_list[rank] = tid;
@@ -832,7 +861,7 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
     for (int nt = 0; nt < NT; ++nt) {
         const int slot = nt * 16 + l16;
         const int loc = slot < n ? s_list[slot] : 0;
-        hbase[nt] = ((loc >> 3) * p.sh * hal_w + (loc & 7) * p.sw) * row + kq * 16;
+        hbase[nt] = ((loc >> 3) * vsy * hal_w + (loc & 7) * vsx) * row + kq * 16;
     }
     float4_t acc[R][NT];
 #pragma unroll
@@ -869,7 +898,7 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
             }
         }
         __syncthreads();
-        const int nsteps = K2 * kcur;
+        const int nsteps = VK2 * kcur;
         const int groups = (nsteps + S * D * KS - 1) / (S * D * KS);  // of D chunks of S steps per slice
         if (kbase > 0) {
             jl = 0;
@@ -955,7 +984,7 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
             const int pix = nt * 16 + l16;
             if (pix >= n) continue;
             const int loc = s_list[pix];
-            half_t *o = out + (((size_t)b * p.Ho + ty0 + (loc >> 3)) * p.Wo + tx0 + (loc & 7)) * p.Co + co;
+            half_t *o = out + (((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7)) * p.Co + co;
             if (co + 3 < p.Co && (p.Co & 3) == 0) {
                 half4_t v;
 #pragma unroll
@@ -1442,21 +1471,27 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                                             epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
         }
         // Larger layers: halo staged in LDS (see conv_lds_mfma_kernel).
-        if (!transposed) {
-            const int hal_h = (TILE - 1) * g.stride_h + (g.kernel_h - 1) * g.dilation_h + 1;
-            const int hal_w = (TILE - 1) * g.stride_w + (g.kernel_w - 1) * g.dilation_w + 1;
+        if (!transposed || (g.dilation_h == 1 && g.dilation_w == 1)) {
+            // taps per dimension seen by a tile: all of them, or those of one stride phase
+            const int vkh = transposed ? ceil_div(g.kernel_h, g.stride_h) : g.kernel_h;
+            const int vkw = transposed ? ceil_div(g.kernel_w, g.stride_w) : g.kernel_w;
+            const int hal_h = transposed ? TILE + vkh - 1 : (TILE - 1) * g.stride_h + (g.kernel_h - 1) * g.dilation_h + 1;
+            const int hal_w = transposed ? TILE + vkw - 1 : (TILE - 1) * g.stride_w + (g.kernel_w - 1) * g.dilation_w + 1;
+            // transposed: one tile per (8x8 block of pixels one stride apart, stride phase)
+            const int ltx = transposed ? ceil_div(ceil_div(g.out_w, g.stride_w), TILE) * g.stride_w : tx;
+            const int lty = transposed ? ceil_div(ceil_div(g.out_h, g.stride_h), TILE) * g.stride_h : ty;
             const int hpx = hal_h * hal_w;
             const int ksteps_all = ci_p / 32;
             const int kmax = hpx <= LDS_MAX_HALO ? ((48 << 10) / hpx - 16) / 64 : 0;
             const int kcc = kmax >= 1 ? ceil_div(ksteps_all, ceil_div(ksteps_all, kmax)) : 0;
             // the step table holds all steps of a channel chunk plus the ring's run-out
-            if (kmax >= 1 && g.kernel_h * g.kernel_w * kcc + 48 <= LDS_MAX_STEPS) {
-                const int64_t tiles = (int64_t)tx * ty * g.batch;
+            if (kmax >= 1 && vkh * vkw * kcc + 48 <= LDS_MAX_STEPS) {
+                const int64_t tiles = (int64_t)ltx * lty * g.batch;
                 // Arrangements (R channel tiles per wavefront, KS reduction slices, channel groups):
                 // wide outputs on many tiles: R = 2, four channel groups; otherwise, with enough
                 // steps to split, R = 2 and two or four slices (x two or one channel groups); short
                 // reductions: R = 1, up to four channel groups.
-                const int nsteps_chunk = g.kernel_h * g.kernel_w * kcc;
+                const int nsteps_chunk = vkh * vkw * kcc;
                 int rl = 1, ksl = 1, ncw = std::min(4, co_tiles);
                 if (co_tiles >= 16 && tiles * ceil_div(co_tiles, 8) >= 512) { rl = 2; ncw = 4; }
                 else if (nsteps_chunk >= 16 && co_tiles >= 4) {
@@ -1469,14 +1504,20 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                 const int cbl = ceil_div(co_tiles, ncw * rl);
                 const size_t lds = std::max((size_t)hpx * (kcc * 64 + 16), (size_t)(ksl - 1) * ncw * rl * 4 * 1024);
                 const int lgv = log2i(pow2_ceil(kcc * 4));  // lanes per halo pixel while staging
-                dim3 lgrid(tx, ty, g.batch * cbl);
+                dim3 lgrid(ltx, lty, g.batch * cbl);
                 note_kernel("conv_lds_mfma_kernel");
-#define DC_LDS_L(RV, SV, DV, KV) conv_lds_mfma_kernel<RV, SV, DV, KV><<<lgrid, nwv * WAVE, lds, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
+#define DC_LDS_ARGS (p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
+#define DC_LDS_L(RV, SV, DV, KV)                                                                            \
+    do {                                                                                                    \
+        if (transposed) conv_lds_mfma_kernel<RV, SV, DV, KV, true><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS; \
+        else conv_lds_mfma_kernel<RV, SV, DV, KV, false><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS;         \
+    } while (0)
                 if (rl == 1) DC_LDS_L(1, 2, 3, 1);
                 else if (ksl == 1) DC_LDS_L(2, 2, 2, 1);
                 else if (ksl == 2) DC_LDS_L(2, 2, 2, 2);
                 else DC_LDS_L(2, 2, 2, 4);
 #undef DC_LDS_L
+#undef DC_LDS_ARGS
                 hipError_t le = hipGetLastError();
                 if (le != hipSuccess || epi == nullptr) return le;
                 return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,

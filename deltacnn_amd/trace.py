@@ -52,6 +52,8 @@ class Tracer:
         start.record()
         rc = fn(*args)
         end.record()
+        if rc != 0:  # nothing was launched (e.g. a fused form that does not exist for this shape)
+            return rc
         rec["events"] = (start, end)
         rec["kernels"] = _lib.load().dc_last_kernels().decode().split("+")
         rec["n_out"] = self._count(meta.get("out_mask"))

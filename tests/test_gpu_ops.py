@@ -415,6 +415,21 @@ def test_conv_dispatch(lib, cfg, kernel):
     assert _lib.load().dc_last_kernels().decode() == kernel
 
 
+@pytest.mark.parametrize("cfg,kernel", [
+    ((16, 8, 4, 2, 1, 1, 1, 9, 11), "conv_patch_mfma_kernel"),
+    ((64, 48, 4, 2, 1, 1, 1, 37, 41), "conv_lds_mfma_kernel"),
+    ((64, 64, 3, 2, 1, 2, 1, 40, 41), "conv_mfma_kernel"),
+], ids=lambda v: v if isinstance(v, str) else "-".join(str(x) for x in v))
+def test_deconv_dispatch(lib, cfg, kernel):
+    from deltacnn_amd import _lib
+    Cin, Cout = cfg[0], cfg[1]
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(torch.float16, cfg, 6, 0.5, True)
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, Cin, Cout, groups, transposed=True)
+    hk().sparse_deconv(cl(x), d_filt, cl(mask), None, s, p, d, groups, c_out=Cout, create_out_mask=True, packed_filter=pk)
+    assert _lib.load().dc_last_kernels().decode() == kernel
+
+
 DECONVS = [
     (16, 8, 4, 2, 1, 1, 1, 9, 11),     # k4 s2 p1 (reference config)
     (8, 8, 6, 4, 1, 1, 1, 6, 7),       # k6 s4 p1 (reference config)
@@ -424,6 +439,8 @@ DECONVS = [
     (64, 48, 4, 2, 1, 1, 1, 37, 41),   # large enough for the tiled MFMA kernel: stride-phase tiles
     (32, 32, 8, 4, 2, 1, 1, 20, 23),   # k8 s4: 64 taps, four per phase
     (40, 24, 3, 2, 1, 1, 1, 33, 30),   # kernel not a multiple of the stride: phases differ in tap count
+    (64, 64, 3, 2, 1, 2, 1, 40, 41),   # dilation 2: compacted-tile kernel on stride-phase tiles
+    (16, 16, 2, 3, 0, 1, 1, 30, 31),   # kernel smaller than the stride: phases without any tap
 ]
 
 
