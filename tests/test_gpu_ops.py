@@ -594,6 +594,66 @@ def test_conv_add_fused_small_layers(lib, cfg, act, weights):
         assert_masked_close(p1, want_prev, torch.ones_like(want_mask), 0, 2e-2, "prev_out")
 
 
+# ------------------------------------------------------------------ nothing active / all active
+@pytest.mark.parametrize("fill", [0, 1], ids=["all-inactive", "all-active"])
+@pytest.mark.parametrize("cfg", [
+    (32, 32, 3, 1, 1, 1, 1, 16, 16),        # patch kernel
+    (64, 64, 3, 1, 1, 1, 1, 72, 70),        # LDS-halo kernel
+    (64, 256, 1, 1, 0, 1, 1, 20, 20),       # pointwise
+    (32, 32, 3, 1, 1, 1, 32, 15, 18),       # depthwise
+    (16, 16, 3, 1, 1, 1, 16, 726, 727),     # depthwise strips
+    (3, 32, 3, 2, 1, 1, 1, 33, 31),         # stem
+], ids=lambda c: "-".join(str(v) for v in c))
+def test_conv_uniform_masks(lib, cfg, fill):
+    """A map without a single active pixel writes an all-zero output mask and touches no output
+    value (the output buffer keeps its NaN fill); a fully active map is the dense convolution."""
+    Cin, Cout = cfg[0], cfg[1]
+    dtype = torch.float16
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 31, 0.5)
+    mask = torch.full_like(mask, fill)
+    want, want_mask = ops.conv(x, mask, wt, None, s, p, d, groups)
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, Cin, Cout, groups)
+    out = torch.full(tuple(want.shape), float("nan"), dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+    om = torch.full(tuple(want_mask.shape), -7, dtype=torch.int32, device=DEV)
+    hk().sparse_conv(cl(poison(x, mask)), d_filt, cl(mask), None, s, p, d, groups, c_out=Cout,
+                     create_out_mask=True, packed_filter=pk, out=out, out_mask=om)
+    assert torch.equal(om.cpu(), want_mask)
+    if fill == 0:
+        assert int(om.abs().sum()) == 0 and bool(out.isnan().all())
+    else:
+        _check_conv(dtype, out, want, want_mask)
+
+
+@pytest.mark.parametrize("fill", [0, 1], ids=["all-inactive", "all-active"])
+def test_scanned_kernels_uniform_masks(lib, fill):
+    """The mask-scanning activation and add kernels on a map with no / only active pixels."""
+    g = _gen(77)
+    B, C, H, W = 1, 16, 520, 511
+    dtype = torch.float16
+    mask = torch.full((B, 1, H, W), fill, dtype=torch.int32)
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+    trunc = (torch.randn(B, C, H, W, generator=g) * 0.01).to(dtype)
+    delta = torch.randn(B, C, H, W, generator=g).to(dtype)
+    w = [delta.clone(), prev.clone(), trunc.clone(), mask.clone()]
+    ops.activate_truncate(*w, 0.1, 1, 0)
+    d = [cl(poison(delta, mask)), cl(prev), cl(trunc), cl(mask)]
+    hk().sparse_activation(*d, 0.1, 1, 0)
+    assert torch.equal(d[3].cpu(), w[3])
+    assert_masked_equal(d[0], w[0], w[3], "delta")
+    assert torch.equal(d[1].cpu(), w[1]) and torch.equal(d[2].cpu(), w[2])
+    b = torch.randn(B, C, H, W, generator=g).to(dtype)
+    w_out, w_mask = ops.add(delta, mask, b, mask, None, 1.0, 1.0, 0, False)
+    d_out = torch.full((B, C, H, W), float("nan"), dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+    d_mo = torch.full((B, 1, H, W), -3, dtype=torch.int32, device=DEV)
+    hk().sparse_add_tensors(cl(poison(delta, mask)), cl(poison(b, mask)), None, d_out, cl(mask), cl(mask), d_mo,
+                            1.0, 1.0, 0, False)
+    assert torch.equal(d_mo.cpu(), w_mask)
+    assert_masked_equal(d_out, w_out, w_mask, "out")
+    if fill == 0:
+        assert bool(d_out.isnan().all())
+
+
 # --------------------------------------------------------------------------------- pooling
 POOLS = [
     # C, K, stride, padding, dilation, H, W
