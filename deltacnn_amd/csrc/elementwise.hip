@@ -473,28 +473,26 @@ add_to_dense_act_kernel(T *__restrict__ a, T *__restrict__ b, const int32_t *__r
 }
 
 // ------------------------------------------------------------------------------- upsample
+// One group of lanes per OUTPUT pixel (oy, ox), which copies input pixel (oy / S, ox / S) and its
+// mask word: S * S times the parallelism of a group per input pixel, coalesced stores, no loop
+// over the S x S block; the repeated reads of an input row come from the caches.
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
 upsample_kernel(const T *__restrict__ in, T *__restrict__ out, const int32_t *__restrict__ mi,
                 int32_t *__restrict__ mo, int B, int H, int W, int C, int S, int lg) {
-    const int P = B * H * W;
+    const int Ho = H * S, Wo = W * S;
+    const int P = B * Ho * Wo;
     const int G = 1 << lg;
-    int p, gl;
-    group_coords(lg, p, gl);
-    if (p >= P) return;
-    const int Wo = W * S;
-    const bool active = mi[p] != 0;
-    const int row = p / W, x = p - row * W;  // row = b*H + y
-    for (int i = gl; i < S * S; i += G)
-        mo[(size_t)(row * S + i / S) * Wo + x * S + i % S] = active ? 1 : 0;
+    int po, gl;
+    group_coords(lg, po, gl);
+    if (po >= P) return;
+    const int row = po / Wo, ox = po - row * Wo;  // row = b * Ho + oy
+    const int bb = row / Ho, oy = row - bb * Ho;
+    const size_t pi = ((size_t)bb * H + oy / S) * W + ox / S;
+    const bool active = mi[pi] != 0;
+    if (gl == 0) mo[po] = active ? 1 : 0;
     if (!active) return;
-    for (int c = gl * N; c < C; c += G * N) {
-        Vec<T, N> v = vload<T, N>(in + (size_t)p * C + c);
-        for (int i = 0; i < S * S; ++i) {
-            size_t op = (size_t)(row * S + i / S) * Wo + x * S + i % S;
-            vstore<T, N>(out + op * C + c, v);
-        }
-    }
+    for (int c = gl * N; c < C; c += G * N) vstore<T, N>(out + (size_t)po * C + c, vload<T, N>(in + pi * C + c));
 }
 
 // ---------------------------------------------------------------------------- concatenate
@@ -761,7 +759,7 @@ template <typename T>
 hipError_t upsample_t(const T *in, T *out, const int32_t *mi, int32_t *mo, int B, int H, int W,
                       int C, int S, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
-    int P = B * H * W;
+    int P = B * H * W * S * S;  // output pixels
     if (can_vec<T>(C, {in, out})) {
         GroupLaunch L(P, pick_group(C / N, P, 4));
         note_kernel("upsample_kernel");
