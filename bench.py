@@ -270,6 +270,12 @@ def scaled_bench():
     out = []
     a, b, c, d = feat(), feat(), feat(), feat()
     wdw = torch.randn(1, 3, 3, C, device="cuda", dtype=torch.half, generator=gen) / 3
+    q = torch.randn(B, C, H // 2, W // 2, device="cuda", dtype=torch.half, generator=gen).contiguous(
+        memory_format=torch.channels_last)
+    qmask = torch.zeros(B, 1, H // 2, W // 2, dtype=torch.int32, device="cuda")
+    h1, h2 = (torch.randn(B, C // 2, H, W, device="cuda", dtype=torch.half, generator=gen).contiguous(
+        memory_format=torch.channels_last) for _ in range(2))
+    scale, shift = (torch.randn(C, device="cuda", dtype=torch.half, generator=gen) for _ in range(2))
     for rho in (0.1, 1.0):
         mask = (torch.rand(B, 1, H, W, device="cuda", generator=gen) < rho).to(torch.int32)
         mask2 = mask.clone()
@@ -281,6 +287,15 @@ def scaled_bench():
             "depthwise3x3+relu": (lambda: hk.sparse_conv_activation(a, wdw, mask, None, b, c, 0.0, 1, 0, (1, 1), (1, 1),
                                                                     (1, 1), C, C, out=d, out_mask=mask2), None),
         }
+        ops.update({
+            "maxpool2x2": (lambda: hk.sparse_pooling(a, b, (2, 2), mask, (2, 2), pooling_mode_int=0, out=q, out_mask=qmask), None),
+            "avgpool2x2": (lambda: hk.sparse_pooling(a, None, (2, 2), mask, (2, 2), pooling_mode_int=1, out=q, out_mask=qmask), None),
+            "upsample_x2": (lambda: hk.sparse_upsample(q, qmask_in, 2, out=(d, mask2)), None),
+            "concat": (lambda: hk.sparse_concatenate((h1, mask), (h2, mask), out=(d, mask2)), None),
+            "mul_add": (lambda: hk.sparse_mul_add(a, mask, d, mask2, scale, shift), None),
+            "add_to_dense": (lambda: hk.sparse_add_to_dense_tensor(a, d, mask), None),
+        })
+        qmask_in = (torch.rand(B, 1, H // 2, W // 2, device="cuda", generator=gen) < rho).to(torch.int32)
         if rho < 1:
             ops.pop("sparsify")  # its density is set by the data, measured at 100 % only
         for name, (fn, _) in ops.items():

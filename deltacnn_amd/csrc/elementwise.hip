@@ -547,6 +547,197 @@ mul_add_kernel(const T *__restrict__ in, const int32_t *__restrict__ mask, T *__
     }
 }
 
+// ------------------------------------------------------------- large maps: scanning forms
+// The four operators above for maps of at least SCAN_MIN_PIXELS pixels (see
+// act_trunc_scan_kernel): a wavefront reads 64 mask words, writes the 64 output mask words,
+// lists its updated pixels in LDS and then serves them U at a time per lane group, so a sparse
+// map costs no wavefront launches for pixels that have nothing to do.  One 16-byte vector per
+// lane and pixel: G >= C / N.
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+mul_add_scan_kernel(const T *in, const int32_t *mask, T *out, int32_t *mo, const T *__restrict__ scale,
+                    const T *__restrict__ bias, int P, int C, int lg) {
+    __shared__ int s_list[4][WAVE];
+    const int wave = wave_id(), lane = lane_id();
+    const int pm = (blockIdx.x * 4 + wave) * WAVE + lane;
+    const bool on = pm < P && mask[min(pm, P - 1)] != 0;
+    if (mo != mask && pm < P) mo[pm] = on ? 1 : 0;
+    int n;
+    const int rank = wave_rank(on, n);
+    if (n == 0) return;
+    if (on) s_list[wave][rank] = pm;
+    const int G = 1 << lg, gl = lane & (G - 1), grp = lane >> lg, ppi = WAVE >> lg;
+    const bool mine = gl * N < C;
+    const int c = min(gl * N, C - N);
+    const Vec<T, N> sc = vload<T, N>(scale + c);
+    Vec<T, N> bi;
+    if (bias != nullptr) bi = vload<T, N>(bias + c);
+    constexpr int U = 4;
+    for (int k = 0; k < n; k += U * ppi) {
+        Vec<T, N> v[U];
+        bool valid[U];
+        size_t off[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int idx = k + u * ppi + grp;
+            valid[u] = idx < n && mine;
+            off[u] = (size_t)s_list[wave][min(idx, n - 1)] * C + c;
+            v[u] = vload<T, N>(in + off[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!valid[u]) continue;
+            if (bias != nullptr) {
+#pragma unroll
+                for (int j = 0; j < N; ++j) v[u].v[j] = fma_t(v[u].v[j], sc.v[j], bi.v[j]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < N; ++j) v[u].v[j] = v[u].v[j] * sc.v[j];
+            }
+            vstore<T, N>(out + off[u], v[u]);
+        }
+    }
+}
+
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+add_to_dense_scan_kernel(const T *__restrict__ a, T *__restrict__ b, const int32_t *__restrict__ ma,
+                         int P, int C, int lg) {
+    __shared__ int s_list[4][WAVE];
+    const int wave = wave_id(), lane = lane_id();
+    const int pm = (blockIdx.x * 4 + wave) * WAVE + lane;
+    const bool on = pm < P && ma[min(pm, P - 1)] != 0;
+    int n;
+    const int rank = wave_rank(on, n);
+    if (n == 0) return;
+    if (on) s_list[wave][rank] = pm;
+    const int G = 1 << lg, gl = lane & (G - 1), grp = lane >> lg, ppi = WAVE >> lg;
+    const bool mine = gl * N < C;
+    const int c = min(gl * N, C - N);
+    constexpr int U = 2;
+    for (int k = 0; k < n; k += U * ppi) {
+        Vec<T, N> va[U], vb[U];
+        bool valid[U];
+        size_t off[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int idx = k + u * ppi + grp;
+            valid[u] = idx < n && mine;
+            off[u] = (size_t)s_list[wave][min(idx, n - 1)] * C + c;
+            va[u] = vload<T, N>(a + off[u]);
+            vb[u] = vload<T, N>(b + off[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!valid[u]) continue;
+#pragma unroll
+            for (int j = 0; j < N; ++j) vb[u].v[j] = vb[u].v[j] + va[u].v[j];
+            vstore<T, N>(b + off[u], vb[u]);
+        }
+    }
+}
+
+// Lane gl of a group copies output vector gl of the Ca + Cb channels: from a, or from b behind it
+// (zeros where that side was not updated).
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+concat_scan_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ out,
+                   const int32_t *__restrict__ ma, const int32_t *__restrict__ mb,
+                   int32_t *__restrict__ mo, int P, int Ca, int Cb, int lg) {
+    __shared__ int s_list[4][WAVE];
+    const int wave = wave_id(), lane = lane_id();
+    const int p0 = (blockIdx.x * 4 + wave) * WAVE;
+    const int pm = p0 + lane;
+    const bool la = pm < P && ma[min(pm, P - 1)] != 0, lb = pm < P && mb[min(pm, P - 1)] != 0;
+    if (pm < P) mo[pm] = (la || lb) ? 1 : 0;
+    const uint64_t bits_a = ballot(la), bits_b = ballot(lb);
+    int n;
+    const int rank = wave_rank(la || lb, n);
+    if (n == 0) return;
+    if (la || lb) s_list[wave][rank] = lane;
+    const int G = 1 << lg, gl = lane & (G - 1), grp = lane >> lg, ppi = WAVE >> lg;
+    const bool side_a = gl * N < Ca;
+    const bool mine = gl * N < Ca + Cb;
+    const int cs = side_a ? gl * N : min(gl * N - Ca, Cb - N);  // channel within the lane's side
+    constexpr int U = 4;
+    for (int k = 0; k < n; k += U * ppi) {
+        Vec<T, N> v[U];
+        bool valid[U], have[U];
+        size_t po[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int idx = k + u * ppi + grp;
+            valid[u] = idx < n && mine;
+            const int l = s_list[wave][min(idx, n - 1)];
+            const bool aa = (bits_a >> l) & 1ull, ab = (bits_b >> l) & 1ull;
+            po[u] = (size_t)p0 + l;
+            have[u] = side_a ? aa : ab;
+            // a side that was not updated is not read: the request goes to the other side's row
+            const T *mine_p = side_a ? a + po[u] * Ca + cs : b + po[u] * Cb + cs;
+            const T *other_p = side_a ? b + po[u] * Cb : a + po[u] * Ca;
+            v[u] = vload<T, N>(have[u] ? mine_p : other_p);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!valid[u]) continue;
+            if (!have[u]) {
+#pragma unroll
+                for (int j = 0; j < N; ++j) v[u].v[j] = T(0);
+            }
+            vstore<T, N>(out + po[u] * (Ca + Cb) + (side_a ? cs : Ca + cs), v[u]);
+        }
+    }
+}
+
+// Scans INPUT pixels; an updated pixel is read once and stored S x S times.
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+upsample_scan_kernel(const T *__restrict__ in, T *__restrict__ out, const int32_t *__restrict__ mi,
+                     int32_t *__restrict__ mo, int B, int H, int W, int C, int S, int lg) {
+    __shared__ int s_in[4][WAVE], s_out[4][WAVE];
+    const int P = B * H * W, Wo = W * S;
+    const int wave = wave_id(), lane = lane_id();
+    const int pm = (blockIdx.x * 4 + wave) * WAVE + lane;
+    const int pc = min(pm, P - 1);
+    const bool on = pm < P && mi[pc] != 0;
+    const int row = pc / W, x = pc - row * W;         // row = b * H + y
+    const int obase = row * S * Wo + x * S;            // top left output pixel of the block
+    if (pm < P) {
+        for (int dy = 0; dy < S; ++dy)
+            for (int dx = 0; dx < S; ++dx) mo[(size_t)obase + dy * Wo + dx] = on ? 1 : 0;
+    }
+    int n;
+    const int rank = wave_rank(on, n);
+    if (n == 0) return;
+    if (on) {
+        s_in[wave][rank] = pm;
+        s_out[wave][rank] = obase;
+    }
+    const int G = 1 << lg, gl = lane & (G - 1), grp = lane >> lg, ppi = WAVE >> lg;
+    const bool mine = gl * N < C;
+    const int c = min(gl * N, C - N);
+    constexpr int U = 4;
+    for (int k = 0; k < n; k += U * ppi) {
+        Vec<T, N> v[U];
+        bool valid[U];
+        size_t ob[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int idx = k + u * ppi + grp;
+            valid[u] = idx < n && mine;
+            const int e = min(idx, n - 1);
+            ob[u] = (size_t)s_out[wave][e];
+            v[u] = vload<T, N>(in + (size_t)s_in[wave][e] * C + c);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!valid[u]) continue;
+            for (int dy = 0; dy < S; ++dy)
+                for (int dx = 0; dx < S; ++dx) vstore<T, N>(out + (ob[u] + (size_t)dy * Wo + dx) * C + c, v[u]);
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------- host helpers
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -565,6 +756,11 @@ struct GroupLaunch {
     GroupLaunch(int64_t pixels, int G)
         : lg(log2i(G)), block(group_block(pixels * G)), grid((unsigned)ceil_div64(pixels * G, block)) {}
 };
+
+// the scanning kernels: 16-byte vectors, at most one per lane of a wavefront, a large map
+inline bool scan_eligible(bool vec, int64_t pixels, int nvec) {
+    return vec && nvec >= 1 && nvec <= WAVE && pixels >= SCAN_MIN_PIXELS;
+}
 
 template <typename T>
 hipError_t sparsify_t(const T *in, T *prev, T *delta, int32_t *mask, float thr, int P, int C,
@@ -744,6 +940,11 @@ template <typename T>
 hipError_t add_to_dense_t(T *a, T *b, const int32_t *ma, int act, int P, int C, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
     const bool vec = can_vec<T>(C, {a, b});
+    if (act <= 0 && scan_eligible(vec, P, C / N)) {
+        note_kernel("add_to_dense_scan_kernel");
+        add_to_dense_scan_kernel<T, N><<<dim3((unsigned)ceil_div(P, 4 * WAVE)), 256, 0, s>>>(a, b, ma, P, C, log2i(group_lanes(C / N, 1)));
+        return hipGetLastError();
+    }
     GroupLaunch L(P, vec ? pick_group(C / N, P, 4) : group_lanes(C, 1));
     note_kernel(act > 0 ? "add_to_dense_act_kernel" : "add_to_dense_kernel");
     if (act > 0) {
@@ -760,6 +961,11 @@ hipError_t upsample_t(const T *in, T *out, const int32_t *mi, int32_t *mo, int B
                       int C, int S, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
     int P = B * H * W * S * S;  // output pixels
+    if (scan_eligible(can_vec<T>(C, {in, out}), B * H * W, C / N)) {
+        note_kernel("upsample_scan_kernel");
+        upsample_scan_kernel<T, N><<<dim3((unsigned)ceil_div(B * H * W, 4 * WAVE)), 256, 0, s>>>(in, out, mi, mo, B, H, W, C, S, log2i(group_lanes(C / N, 1)));
+        return hipGetLastError();
+    }
     if (can_vec<T>(C, {in, out})) {
         GroupLaunch L(P, pick_group(C / N, P, 4));
         note_kernel("upsample_kernel");
@@ -776,6 +982,11 @@ hipError_t concat_t(const T *a, const T *b, T *out, const int32_t *ma, const int
                     int32_t *mo, int P, int Ca, int Cb, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
     int Cm = Ca > Cb ? Ca : Cb;
+    if (Ca % N == 0 && Cb % N == 0 && scan_eligible(can_vec<T>(Ca, {a, b, out}), P, (Ca + Cb) / N)) {
+        note_kernel("concat_scan_kernel");
+        concat_scan_kernel<T, N><<<dim3((unsigned)ceil_div(P, 4 * WAVE)), 256, 0, s>>>(a, b, out, ma, mb, mo, P, Ca, Cb, log2i(group_lanes((Ca + Cb) / N, 1)));
+        return hipGetLastError();
+    }
     if (Ca % N == 0 && Cb % N == 0 && can_vec<T>(Ca, {a, b, out})) {
         GroupLaunch L(P, pick_group(Cm / N, P, 4));
         note_kernel("concat_kernel");
@@ -791,6 +1002,11 @@ template <typename T>
 hipError_t mul_add_t(const T *in, const int32_t *mask, T *out, int32_t *mo, const T *scale,
                      const T *bias, int P, int C, hipStream_t s) {
     constexpr int N = Vec16<T>::N;
+    if (scan_eligible(can_vec<T>(C, {in, out, scale, bias}), P, C / N)) {
+        note_kernel("mul_add_scan_kernel");
+        mul_add_scan_kernel<T, N><<<dim3((unsigned)ceil_div(P, 4 * WAVE)), 256, 0, s>>>(in, mask, out, mo, scale, bias, P, C, log2i(group_lanes(C / N, 1)));
+        return hipGetLastError();
+    }
     if (can_vec<T>(C, {in, out, scale, bias})) {
         GroupLaunch L(P, pick_group(C / N, P, 4));
         note_kernel("mul_add_kernel");

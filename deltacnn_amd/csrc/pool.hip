@@ -49,14 +49,14 @@ pool_window_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restri
                 hi[j] = MAX ? -INFINITY : 0.f;
                 hp[j] = -INFINITY;
             }
-            constexpr int KK = K > 0 ? K * K : 1;
+            constexpr int KK = K > 0 ? K * K : 1, KD = K > 0 ? K : 1;
             Vec<T, N> pd[KK], pp[KK];
             int pm[KK];
             if (K > 0) {
 #pragma unroll
                 for (int t = 0; t < KK; ++t) {
-                    const int iy = min(max(oy * p.sh - p.pt + (t / K) * p.dh, 0), p.Hi - 1);
-                    const int ix = min(max(ox * p.sw - p.pl + (t % K) * p.dw, 0), p.Wi - 1);
+                    const int iy = min(max(oy * p.sh - p.pt + (t / KD) * p.dh, 0), p.Hi - 1);
+                    const int ix = min(max(ox * p.sw - p.pl + (t % KD) * p.dw, 0), p.Wi - 1);
                     const int ip = iy * p.Wi + ix;
                     pm[t] = mb[ip];
                     pd[t] = vload<T, N>(inb + (size_t)ip * C + c);
@@ -116,6 +116,149 @@ pool_window_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restri
 #pragma unroll
             for (int j = 0; j < N; ++j) r.v[j] = MAX ? T(hi[j] - hp[j]) : T(hi[j] / area);
             vstore<T, N>(out + (((size_t)b * p.Ho + oy) * p.Wo + ox) * C + c, r);
+        }
+    }
+}
+
+// The K x K window kernel for maps of at least 2^18 outputs: a wavefront owns 64 consecutive
+// output pixels, one per lane while the window's mask words are read and the output mask is
+// written; the updated outputs are listed in LDS -- pixel, coordinates and the set of updated
+// taps -- and served U at a time per lane group (one 16-byte vector per lane).  No workgroup
+// barrier, a sparse map costs no idle groups, and the delta of a tap that was not updated is
+// not fetched (its request goes to an updated tap's row, which is being read anyway).  Same
+// operations in the same order as pool_window_kernel.
+template <typename T, int N, bool MAX, int K>
+__global__ void __launch_bounds__(256)
+pool_scan_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restrict__ prev,
+                 T *__restrict__ out, const int32_t *__restrict__ mask,
+                 int32_t *__restrict__ out_mask, int lg) {
+    constexpr int KK = K * K;
+    __shared__ int s_pix[4][WAVE], s_yx[4][WAVE], s_img[4][WAVE], s_taps[4][WAVE];
+    const int Po = p.B * p.Ho * p.Wo, C = p.Ci;
+    const int wave = wave_id(), lane = lane_id();
+    const int po = (blockIdx.x * 4 + wave) * WAVE + lane;
+    int taps = 0;  // bit t: tap t is inside the map and updated
+    int yx, img;
+    {
+        const int pc = min(po, Po - 1);
+        const int row = pc / p.Wo, ox = pc - row * p.Wo;
+        const int b = row / p.Ho, oy = row - b * p.Ho;
+        yx = (oy << 16) | ox;
+        img = b * p.Hi * p.Wi;
+        int mw[KK];
+        bool inside[KK];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) {
+            const int iy = oy * p.sh - p.pt + (t / K) * p.dh, ix = ox * p.sw - p.pl + (t % K) * p.dw;
+            inside[t] = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
+            mw[t] = mask[(size_t)img + min(max(iy, 0), p.Hi - 1) * p.Wi + min(max(ix, 0), p.Wi - 1)];
+        }
+#pragma unroll
+        for (int t = 0; t < KK; ++t) taps |= (inside[t] && mw[t] != 0) ? 1 << t : 0;
+    }
+    if (po >= Po) taps = 0;
+    if (po < Po) out_mask[po] = taps != 0 ? 1 : 0;
+    int n;
+    const int rank = wave_rank(taps != 0, n);
+    if (n == 0) return;
+    if (taps != 0) {
+        s_pix[wave][rank] = po;
+        s_yx[wave][rank] = yx;
+        s_img[wave][rank] = img;
+        s_taps[wave][rank] = taps;
+    }
+    const int G = 1 << lg, gl = lane & (G - 1), grp = lane >> lg, ppi = WAVE >> lg;
+    const bool mine = gl * N < C;
+    const int c = min(gl * N, C - N);
+    constexpr int U = K == 2 ? 2 : 1;
+    for (int k = 0; k < n; k += U * ppi) {
+        Vec<T, N> pd[U][KK], pp[U][KK];
+        bool valid[U];
+        int pix[U], oy[U], ox[U], tp[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int idx = k + u * ppi + grp, e = min(idx, n - 1);
+            valid[u] = idx < n && mine;
+            pix[u] = s_pix[wave][e];
+            oy[u] = s_yx[wave][e] >> 16;
+            ox[u] = s_yx[wave][e] & 0xffff;
+            tp[u] = s_taps[wave][e];
+            const size_t base = (size_t)s_img[wave][e];
+            const int first = __builtin_ctz(tp[u]);  // an updated tap: the list holds no other pixels
+            size_t ip[KK];
+#pragma unroll
+            for (int t = 0; t < KK; ++t) {
+                const int iy = min(max(oy[u] * p.sh - p.pt + (t / K) * p.dh, 0), p.Hi - 1);
+                const int ix = min(max(ox[u] * p.sw - p.pl + (t % K) * p.dw, 0), p.Wi - 1);
+                ip[t] = base + (size_t)iy * p.Wi + ix;
+            }
+            size_t ifirst = ip[0];
+#pragma unroll
+            for (int t = 1; t < KK; ++t) ifirst = first == t ? ip[t] : ifirst;
+#pragma unroll
+            for (int t = 0; t < KK; ++t) {
+                pd[u][t] = vload<T, N>(in + (((tp[u] >> t) & 1) ? ip[t] : ifirst) * C + c);
+                if (MAX) pp[u][t] = vload<T, N>(prev + ip[t] * C + c);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!valid[u]) continue;
+            float hi[N], hp[N];
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                hi[j] = MAX ? -INFINITY : 0.f;
+                hp[j] = -INFINITY;
+            }
+#pragma unroll
+            for (int ky = 0; ky < K; ++ky) {
+                const int iy = oy[u] * p.sh - p.pt + ky * p.dh;
+                if (iy < 0) continue;
+                if (iy >= p.Hi) {
+                    if (MAX && q.zero_bottom && iy < p.Hi + q.pb) {
+#pragma unroll
+                        for (int j = 0; j < N; ++j) {
+                            hi[j] = fmaxf(hi[j], 0.f);
+                            hp[j] = fmaxf(hp[j], 0.f);
+                        }
+                    }
+                    continue;
+                }
+#pragma unroll
+                for (int kx = 0; kx < K; ++kx) {
+                    const int ix = ox[u] * p.sw - p.pl + kx * p.dw;
+                    if (ix < 0) continue;
+                    if (ix >= p.Wi) {
+                        if (MAX && q.zero_right && ix < p.Wi + q.pr) {
+#pragma unroll
+                            for (int j = 0; j < N; ++j) {
+                                hi[j] = fmaxf(hi[j], 0.f);
+                                hp[j] = fmaxf(hp[j], 0.f);
+                            }
+                        }
+                        continue;
+                    }
+                    const int t = ky * K + kx;
+                    const bool act = (tp[u] >> t) & 1;
+                    if (!MAX && !act) continue;
+#pragma unroll
+                    for (int j = 0; j < N; ++j) {
+                        const float d = act ? float(pd[u][t].v[j]) : 0.f;
+                        if (MAX) {
+                            const float pf = float(pp[u][t].v[j]);
+                            hi[j] = fmaxf(hi[j], d + pf);
+                            hp[j] = fmaxf(hp[j], pf);
+                        } else {
+                            hi[j] += d;
+                        }
+                    }
+                }
+            }
+            Vec<T, N> r;
+            const float area = float(K * K);
+#pragma unroll
+            for (int j = 0; j < N; ++j) r.v[j] = MAX ? T(hi[j] - hp[j]) : T(hi[j] / area);
+            vstore<T, N>(out + (size_t)pix[u] * C + c, r);
         }
     }
 }
@@ -289,13 +432,26 @@ hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, c
             pool_global_kernel<T, false><<<grid, 256, 0, s>>>(p, q, in, prev, (float *)out, mask, out_mask);
         return hipGetLastError();
     }
-    note_kernel("pool_window_kernel");
     dim3 grid(ceil_div(g.out_w, TILE), ceil_div(g.out_h, TILE), g.batch);
     const bool vec = g.in_c % N == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
                      ((uintptr_t)prev & 15) == 0;
     int G = pow2_ceil(vec ? g.in_c / N : g.in_c);
     if (G > WAVE) G = WAVE;
     const int ksq = (g.kernel_h == g.kernel_w && (g.kernel_h == 2 || g.kernel_h == 3)) ? g.kernel_h : 0;
+    const int64_t po = (int64_t)g.batch * g.out_h * g.out_w;
+    if (ksq > 0 && vec && g.in_c / N <= WAVE && po >= (1 << 18) && po < (1ll << 31) && g.out_h < 65536 && g.out_w < 65536 &&
+        (int64_t)g.batch * g.in_h * g.in_w < (1ll << 31)) {
+        note_kernel("pool_scan_kernel");
+        const dim3 sgrid((unsigned)ceil_div64(po, 4 * WAVE));
+        int lg = 0;
+        while ((1 << lg) < G) ++lg;
+#define DC_PS(MX, KV) pool_scan_kernel<T, N, MX, KV><<<sgrid, 256, 0, s>>>(p, q, in, prev, (T *)out, mask, out_mask, lg)
+        if (mode == DC_POOL_MAX) { if (ksq == 2) DC_PS(true, 2); else DC_PS(true, 3); }
+        else { if (ksq == 2) DC_PS(false, 2); else DC_PS(false, 3); }
+#undef DC_PS
+        return hipGetLastError();
+    }
+    note_kernel("pool_window_kernel");
 #define DC_POOL(NN, MX)                                                                                           \
     do {                                                                                                          \
         if (ksq == 2) pool_window_kernel<T, NN, MX, 2><<<grid, 256, 0, s>>>(p, q, in, prev, (T *)out, mask, out_mask, G); \

@@ -45,6 +45,7 @@ from __future__ import annotations
 import math
 from typing import Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 import torch.nn.functional as F
 
@@ -74,6 +75,15 @@ def activation(x: torch.Tensor, act: int) -> torch.Tensor:
     if act == ACT_SWISH:
         return (x.float() * (1.0 / (1.0 + torch.exp(-x.float())))).to(x.dtype)
     raise ValueError(f"activation id {act}")
+
+
+def _round_f64(value: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """One rounding from float64 to `dtype`.  torch converts float64 to float16 by way of
+    float32, which rounds twice (about one value in 10^5 of a fused multiply-add ends one ulp
+    off); numpy converts directly."""
+    if dtype == torch.float16:
+        return torch.from_numpy(value.contiguous().numpy().astype(np.float16)).view(value.shape)
+    return value.to(dtype)
 
 
 def _active(mask: torch.Tensor) -> torch.Tensor:
@@ -296,7 +306,7 @@ def add(a, mask_a, b, mask_b, prev_out: Optional[torch.Tensor], weight_a: float 
     zero = torch.zeros_like(a)
     s = torch.where(ma, a * wa, zero)
     # single-rounding fma: the fp64 product and sum are exact for fp16 operands
-    sb = (torch.where(mb, b, zero).double() * wb.double() + s.double()).to(a.dtype)
+    sb = _round_f64(torch.where(mb, b, zero).double() * wb.double() + s.double(), a.dtype)
     s = torch.where(mb, sb, s)
     if dense_out:
         new = s + prev_out
@@ -333,5 +343,5 @@ def mul_add(x, mask, scale, bias: Optional[torch.Tensor]):
         y = x * sc
     else:
         # single-rounding fma (``__hfma2``, :3861): exact in fp64 for fp16 operands
-        y = (x.double() * sc.double() + bias.reshape(1, -1, 1, 1).to(x.dtype).double()).to(x.dtype)
+        y = _round_f64(x.double() * sc.double() + bias.reshape(1, -1, 1, 1).to(x.dtype).double(), x.dtype)
     return torch.where(_active(mask), y, torch.zeros_like(y)), (mask != 0).to(torch.int32)

@@ -711,6 +711,105 @@ def test_pool_global(lib, dtype, mode, C, H, W, density):
     assert_masked_close(out2, want, want_mask, tol, tol, "out (float32 accumulator)")
 
 
+# ------------------------------------------------ the scanning forms of the simple operators
+def _last_kernel():
+    from deltacnn_amd import _lib
+    return _lib.load().dc_last_kernels().decode()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("density", [0.0, 0.03, 0.5, 1.0])
+def test_scanned_simple_operators(lib, dtype, density):
+    """mul_add, add_to_dense, concat and upsample on maps large enough for their mask-scanning
+    kernels (channel counts that fill, underfill and split a lane group)."""
+    g = _gen(int(1500 + 100 * density))
+    B, H, W = 2, 397, 333
+    for C in (24, 64) if dtype == torch.float16 else (12, 40):
+        mask = rand_mask(g, B, H, W, density)
+        x = torch.randn(B, C, H, W, generator=g).to(dtype)
+        scale, bias = torch.randn(C, generator=g).to(dtype), torch.randn(C, generator=g).to(dtype)
+        for bi in (None, bias):
+            want, want_mask = ops.mul_add(x, mask, scale, bi)
+            d_x, d_m = cl(poison(x, mask)), cl(mask)
+            out, om = torch.full_like(d_x, float("nan")), torch.full_like(d_m, -3)
+            hk().sparse_mul_add(d_x, d_m, out, om, scale.to(DEV), None if bi is None else bi.to(DEV))
+            assert _last_kernel() == "mul_add_scan_kernel"
+            assert torch.equal(om.cpu(), want_mask)
+            if dtype == torch.float32 and bi is not None:
+                assert_masked_close(out, want, want_mask, 1e-6, 1e-6, "mul_add")
+            else:
+                assert_masked_equal(out, want, want_mask, "mul_add")
+            if density == 0.0:
+                assert bool(out.isnan().all())
+            # in place, as the batch-norm layer calls it
+            hk().sparse_mul_add(d_x, d_m, d_x, d_m, scale.to(DEV), None if bi is None else bi.to(DEV))
+            if not (dtype == torch.float32 and bi is not None):
+                assert_masked_equal(d_x, want, want_mask, "mul_add in place")
+            assert torch.equal(d_m.cpu(), mask)
+
+        b = torch.randn(B, C, H, W, generator=g).to(dtype)
+        w_b = b.clone()
+        ops.add_to_dense(x, w_b, mask)
+        d_b = cl(b)
+        hk().sparse_add_to_dense_tensor(cl(poison(x, mask)), d_b, cl(mask), 0)
+        assert _last_kernel() == "add_to_dense_scan_kernel"
+        assert torch.equal(d_b.cpu(), w_b)
+
+        Cb = C - (4 if dtype == torch.float32 else 8)
+        mb = rand_mask(g, B, H, W, density / 2)
+        y = torch.randn(B, Cb, H, W, generator=g).to(dtype)
+        want, want_mask = ops.concatenate(x, mask, y, mb)
+        d_out = torch.full((B, C + Cb, H, W), float("nan"), dtype=dtype, device=DEV).contiguous(
+            memory_format=torch.channels_last)
+        d_om = torch.full((B, 1, H, W), -3, dtype=torch.int32, device=DEV)
+        hk().sparse_concatenate((cl(poison(x, mask)), cl(mask)), (cl(poison(y, mb)), cl(mb)), out=(d_out, d_om))
+        assert _last_kernel() == "concat_scan_kernel"
+        assert torch.equal(d_om.cpu(), want_mask)
+        assert_masked_equal(d_out, want, want_mask, "concat")
+
+        for s in (2, 3):
+            want, want_mask = ops.upsample(x, mask, s)
+            d_out = torch.full((B, C, H * s, W * s), float("nan"), dtype=dtype, device=DEV).contiguous(
+                memory_format=torch.channels_last)
+            d_om = torch.full((B, 1, H * s, W * s), -3, dtype=torch.int32, device=DEV)
+            hk().sparse_upsample(cl(poison(x, mask)), cl(mask), s, out=(d_out, d_om))
+            assert _last_kernel() == "upsample_scan_kernel"
+            assert torch.equal(d_om.cpu(), want_mask)
+            assert_masked_equal(d_out, want, want_mask, "upsample")
+            if density == 0.0:
+                assert bool(d_out.isnan().all())
+
+
+SCANNED_POOLS = [
+    # C, K, stride, padding, H, W
+    (16, 2, 2, 0, 1023, 1031),
+    (24, 3, 2, 1, 1021, 1035),
+    (8, 3, 1, 1, 515, 513),
+    (32, 2, 2, (0, 1, 0, 1), 1023, 1031),   # asymmetric: zero joins the maximum
+    (16, 2, 1, 0, 520, 511),               # overlapping 2x2 windows
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", SCANNED_POOLS, ids=lambda c: "-".join(str(v).replace(" ", "") for v in c))
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("density", [0.0, 0.02, 0.6])
+def test_pool_scanned_map(lib, dtype, cfg, mode, density):
+    C, K, s, p, H, W = cfg
+    K, s, p = _pair(K), _pair(s), _pair(p)
+    g = _gen(1600 + C)
+    B = 1
+    mask = rand_mask(g, B, H, W, density)
+    x = torch.randn(B, C, H, W, generator=g).to(dtype)
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+    want, want_mask = ops.pool(x, prev if mode == 0 else None, mask, K, s, p, (1, 1), mode)
+    out, om = hk().sparse_pooling(cl(poison(x, mask)), cl(prev) if mode == 0 else None, K, cl(mask), s, p, (1, 1),
+                                  pooling_mode_int=mode)
+    assert _last_kernel() == "pool_scan_kernel"
+    assert torch.equal(om.cpu(), want_mask)
+    assert_masked_equal(out, want, want_mask, "out")
+
+
 # ------------------------------------------------------------- upsample / concat / mul_add
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("C", [3, 32, 72])

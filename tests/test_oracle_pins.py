@@ -367,3 +367,40 @@ def test_multibranch_networks_threshold_zero_equal_dense(which):
                 want, got = {"out": want}, {"out": got}
             for k in want:
                 assert torch.allclose(got[k], want[k], rtol=1e-3, atol=1e-4 * max(1.0, float(want[k].abs().max()))), (t, k)
+
+
+def test_fused_multiply_add_rounds_once_in_half_precision():
+    """The fp16 fused multiply-adds of the oracle (DCAdd's second operand, mul_add with a bias)
+    must be a nearest representable value of the EXACT a*b+c, checked in rational arithmetic
+    -- a conversion from float64 by way of float32 is one ulp off about once in 10^5 values."""
+    from fractions import Fraction
+    g = torch.Generator().manual_seed(0)
+    n = 400_000
+    x = torch.randn(1, 1, 1, n, generator=g).half().permute(0, 3, 1, 2)  # [1, n, 1, 1]: a channel each
+    scale, shift = torch.randn(n, generator=g).half(), torch.randn(n, generator=g).half()
+    mask = torch.ones(1, 1, 1, 1, dtype=torch.int32)
+    got, _ = O.mul_add(x, mask, scale, shift)
+    got = got.flatten()
+    exact64 = x.flatten().double() * scale.double() + shift.double()  # exact: 22 + 11 bits, close exponents
+    # candidates: every value where the two-step conversion and the direct one disagree, plus a sample
+    two_step = exact64.float().half()
+    idx = (two_step != torch.from_numpy(exact64.numpy().astype(np.float16))).nonzero().flatten().tolist()
+    assert len(idx) >= 1, "no double-rounding candidate among the inputs: the test pins nothing"
+    idx += list(range(0, n, 997))
+    for i in idx:
+        ex = Fraction(float(x.flatten()[i])) * Fraction(float(scale[i])) + Fraction(float(shift[i]))
+        r = np.float16(float(got[i]))
+        err = abs(Fraction(float(r)) - ex)
+        for nb in (np.nextafter(r, np.float16(np.inf)), np.nextafter(r, np.float16(-np.inf))):
+            assert err <= abs(Fraction(float(nb)) - ex), (i, float(r), float(nb))
+    # DCAdd: s = a*wa, then fma(b, wb, s)
+    a, b = x, torch.randn(1, n, 1, 1, generator=g).half()
+    out, _ = O.add(a, mask, b, mask, None, 0.5, -1.25, 0, False)
+    out = out.flatten()
+    s = (a.flatten() * torch.tensor(0.5).half())
+    for i in idx[:200]:
+        ex = Fraction(float(b.flatten()[i])) * Fraction(-1.25) + Fraction(float(s[i]))
+        r = np.float16(float(out[i]))
+        err = abs(Fraction(float(r)) - ex)
+        for nb in (np.nextafter(r, np.float16(np.inf)), np.nextafter(r, np.float16(-np.inf))):
+            assert err <= abs(Fraction(float(nb)) - ex), (i, float(r), float(nb))
