@@ -835,14 +835,47 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
         for (int i = 0; i < 4; ++i) bv[r][i] = bias != nullptr ? bias[min(co + i, p.Co - 1)] : half_t(0);
     }
 
+    // Staging of channels [kbase * 32, (kbase + kcur) * 32) of the halo: 2^lgv lanes per pixel, SU
+    // pixels per lane in flight (a 10 x 10 halo is one pass); inactive pixels read one shared
+    // dummy address and are stored as zeros.  The first pass of the first channel chunk is
+    // requested here, so that it travels while the first wavefront dilates the mask.
+    constexpr int SU = 8;
+    const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+    const int sv = tid & ((1 << lgv) - 1), hstep = nthr >> lgv;
+    auto stage_load = [&](int kbase, int h0, half8_t (&val)[SU], int (&px)[SU]) {
+        const int c = min((kbase << 5) + sv * 8, p.Ci - 8);
+#pragma unroll
+        for (int u = 0; u < SU; ++u) {
+            px[u] = s_hpix[min(h0 + u * hstep, hpx - 1)];
+            val[u] = *reinterpret_cast<const half8_t *>(inb + (size_t)max(px[u], 0) * p.Ci + c);
+        }
+    };
+    auto stage_store = [&](int kbase, int kcur, int h0, const half8_t (&val)[SU], const int (&px)[SU]) {
+        const bool vok = sv < kcur * 4 && (kbase << 5) + sv * 8 < p.Ci;
+#pragma unroll
+        for (int u = 0; u < SU; ++u) {
+            const int hp = h0 + u * hstep;
+            if (hp < hpx && sv < kcur * 4)
+                *reinterpret_cast<half8_t *>(s_halo + hp * row + sv * 16) = keep8(val[u], vok && px[u] >= 0);
+        }
+    };
+    half8_t val0[SU];
+    int px0[SU];
+    stage_load(0, tid >> lgv, val0, px0);
+
     if (tid < WAVE) {  // dilate the mask over the window, compact the updated pixels
         const int ly = tid >> 3, lx = tid & 7;
         const int oy = out_y(ly), ox = out_x(lx);
         const bool inb = oy < p.Ho && ox < p.Wo;
         bool upd = false;
         const int base = ly * vsy * hal_w + lx * vsx;
-        for (int ta = 0; ta < A; ++ta)
-            for (int tb = 0; tb < Bt; ++tb) upd |= s_hpix[base + tap_off(ta, tb)] >= 0;
+        if (!TR && p.Kh == 3 && p.Kw == 3) {  // the common window: nine independent reads
+#pragma unroll
+            for (int t = 0; t < 9; ++t) upd |= s_hpix[base + (t / 3) * p.dh * hal_w + (t % 3) * p.dw] >= 0;
+        } else {
+            for (int ta = 0; ta < A; ++ta)
+                for (int tb = 0; tb < Bt; ++tb) upd |= s_hpix[base + tap_off(ta, tb)] >= 0;
+        }
         upd = upd && inb;
         if (inb && cb == 0) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = upd ? 1 : 0;
         int n;
@@ -850,12 +883,12 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
         if (upd) s_list[rank] = tid;
         if (tid == 0) s_n = n;
     }
+    stage_store(0, min(kcc, ksteps), tid >> lgv, val0, px0);
     __syncthreads();
     const int n = s_n;
     if (n == 0) return;
 
     const int n_tiles = (n + 15) >> 4;
-    const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
     int hbase[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -875,29 +908,14 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
             __syncthreads();
             build_steps(kbase, kcur);
         }
-        {   // stage channels [kbase * 32, (kbase + kcur) * 32) of the halo: 2^lgv lanes per pixel,
-            // four pixels per lane in flight; inactive pixels read one shared dummy address
-            const int v = tid & ((1 << lgv) - 1);
-            const int hstep = nthr >> lgv;
-            const int c = min((kbase << 5) + v * 8, p.Ci - 8);
-            const bool vok = v < kcur * 4 && (kbase << 5) + v * 8 < p.Ci;
-            for (int h0 = tid >> lgv; h0 < hpx; h0 += 4 * hstep) {
-                half8_t val[4];
-                int px[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    px[u] = s_hpix[min(h0 + u * hstep, hpx - 1)];
-                    val[u] = *reinterpret_cast<const half8_t *>(inb + (size_t)max(px[u], 0) * p.Ci + c);
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int hp = h0 + u * hstep;
-                    if (hp < hpx && v < kcur * 4)
-                        *reinterpret_cast<half8_t *>(s_halo + hp * row + v * 16) = keep8(val[u], vok && px[u] >= 0);
-                }
-            }
+        // remaining staging passes (all of them for the channel chunks after the first)
+        for (int h0 = (tid >> lgv) + (kbase == 0 ? SU * hstep : 0); h0 < hpx; h0 += SU * hstep) {
+            half8_t val[SU];
+            int px[SU];
+            stage_load(kbase, h0, val, px);
+            stage_store(kbase, kcur, h0, val, px);
         }
-        __syncthreads();
+        if (kbase > 0 || hpx > SU * hstep) __syncthreads();  // uniform: something was staged here
         const int nsteps = VK2 * kcur;
         const int groups = (nsteps + S * D * KS - 1) / (S * D * KS);  // of D chunks of S steps per slice
         if (kbase > 0) {
@@ -940,11 +958,18 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
                     // already reloaded below
                     compute_chunk(a[d], xo[d], xo[(d + 1) % D][0], std::false_type{}, 0);
                     load_chunk(a[d], xo[d]);
+                    // the refill stays here, D - 1 chunks ahead of its use: left to itself the
+                    // scheduler gathers the requests of all chunks at the end of the iteration,
+                    // where they overlap nothing
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
 #pragma unroll
-            for (int d = 0; d < D; ++d)
-                compute_chunk(a[d], xo[d], xo[(d + 1) % D][0], std::true_type{}, ((groups - 1) * D + d) * S);
+            for (int d = 0; d < D; ++d) {
+                const int j0 = ((groups - 1) * D + d) * S;
+                if (j0 * KS + kz >= nsteps) break;  // wave-uniform: chunks past the last step
+                compute_chunk(a[d], xo[d], xo[(d + 1) % D][0], std::true_type{}, j0);
+            }
         };
         switch (n_tiles) {
             case 1: reduce(std::integral_constant<int, 1>{}); break;
@@ -1482,17 +1507,17 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
             const int lty = transposed ? ceil_div(ceil_div(g.out_h, g.stride_h), TILE) * g.stride_h : ty;
             const int hpx = hal_h * hal_w;
             const int ksteps_all = ci_p / 32;
-            const int kmax = hpx <= LDS_MAX_HALO ? ((48 << 10) / hpx - 16) / 64 : 0;
-            const int kcc = kmax >= 1 ? ceil_div(ksteps_all, ceil_div(ksteps_all, kmax)) : 0;
-            // the step table holds all steps of a channel chunk plus the ring's run-out
-            if (kmax >= 1 && vkh * vkw * kcc + 48 <= LDS_MAX_STEPS) {
-                const int64_t tiles = (int64_t)ltx * lty * g.batch;
-                // Arrangements (R channel tiles per wavefront, KS reduction slices, channel groups):
-                // wide outputs on many tiles: R = 2, four channel groups; otherwise, with enough
-                // steps to split, R = 2 and two or four slices (x two or one channel groups); short
-                // reductions: R = 1, up to four channel groups.
+            // Arrangements (R channel tiles per wavefront, KS reduction slices, channel groups):
+            // wide outputs on many tiles: R = 2, four channel groups; otherwise, with enough
+            // steps to split, R = 2 and two or four slices (x two or one channel groups); short
+            // reductions: R = 1, up to four channel groups.
+            const int64_t tiles = (int64_t)ltx * lty * g.batch;
+            int kcc = 0, rl = 1, ksl = 1, ncw = 1;
+            auto plan = [&](int lds_budget) {
+                const int kmax = hpx <= LDS_MAX_HALO ? (lds_budget / hpx - 16) / 64 : 0;
+                kcc = kmax >= 1 ? ceil_div(ksteps_all, ceil_div(ksteps_all, kmax)) : 0;
                 const int nsteps_chunk = vkh * vkw * kcc;
-                int rl = 1, ksl = 1, ncw = std::min(4, co_tiles);
+                rl = 1; ksl = 1; ncw = std::min(4, co_tiles);
                 if (co_tiles >= 16 && tiles * ceil_div(co_tiles, 8) >= 512) { rl = 2; ncw = 4; }
                 else if (nsteps_chunk >= 16 && co_tiles >= 4) {
                     // no more workgroups than compute units and a long reduction: eight wavefronts
@@ -1500,6 +1525,19 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                     ksl = (nsteps_chunk >= 36 && tiles * ceil_div(co_tiles, 4) <= 256) ? 4 : 2;
                 }
                 else if (nsteps_chunk >= 16 && co_tiles >= 2) { rl = 2; ksl = 4; ncw = 1; }
+            };
+            // Fewer LDS passes over the input channels (each costs a table, a staging round trip
+            // and a ring start-up) where a larger halo does not cost residency: a compute unit
+            // holds one workgroup of this launch anyway.  Otherwise 48 KB, two workgroups per
+            // compute unit.
+            plan(48 << 10);
+            const int passes_small = kcc >= 1 ? ceil_div(ksteps_all, kcc) : 1 << 30;
+            plan(112 << 10);
+            if (!(kcc >= 1 && ceil_div(ksteps_all, kcc) < passes_small &&
+                  tiles * ceil_div(co_tiles, ncw * rl) <= 256))
+                plan(48 << 10);
+            // the step table holds all steps of a channel chunk plus the ring's run-out
+            if (kcc >= 1 && vkh * vkw * kcc + 48 <= LDS_MAX_STEPS) {
                 const int nwv = ncw * ksl;  // wavefronts per workgroup
                 const int cbl = ceil_div(co_tiles, ncw * rl);
                 const size_t lds = std::max((size_t)hpx * (kcc * 64 + 16), (size_t)(ksl - 1) * ncw * rl * 4 * 1024);
@@ -1507,16 +1545,25 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                 dim3 lgrid(ltx, lty, g.batch * cbl);
                 note_kernel("conv_lds_mfma_kernel");
 #define DC_LDS_ARGS (p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
+#define DC_LDS_K(RV, SV, DV, KV, TV)                                                                        \
+    do {                                                                                                    \
+        static const hipError_t big = hipFuncSetAttribute(                                                  \
+            reinterpret_cast<const void *>(&conv_lds_mfma_kernel<RV, SV, DV, KV, TV>),                      \
+            hipFuncAttributeMaxDynamicSharedMemorySize, 112 << 10);                                         \
+        if (lds > (48u << 10) && big != hipSuccess) return big;                                             \
+        conv_lds_mfma_kernel<RV, SV, DV, KV, TV><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS;                 \
+    } while (0)
 #define DC_LDS_L(RV, SV, DV, KV)                                                                            \
     do {                                                                                                    \
-        if (transposed) conv_lds_mfma_kernel<RV, SV, DV, KV, true><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS; \
-        else conv_lds_mfma_kernel<RV, SV, DV, KV, false><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS;         \
+        if (transposed) DC_LDS_K(RV, SV, DV, KV, true);                                                     \
+        else DC_LDS_K(RV, SV, DV, KV, false);                                                               \
     } while (0)
                 if (rl == 1) DC_LDS_L(1, 2, 3, 1);
-                else if (ksl == 1) DC_LDS_L(2, 2, 2, 1);
-                else if (ksl == 2) DC_LDS_L(2, 2, 2, 2);
-                else DC_LDS_L(2, 2, 2, 4);
+                else if (ksl == 1) DC_LDS_L(2, 2, 3, 1);
+                else if (ksl == 2) DC_LDS_L(2, 2, 3, 2);
+                else DC_LDS_L(2, 2, 3, 4);
 #undef DC_LDS_L
+#undef DC_LDS_K
 #undef DC_LDS_ARGS
                 hipError_t le = hipGetLastError();
                 if (le != hipSuccess || epi == nullptr) return le;
