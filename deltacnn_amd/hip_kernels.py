@@ -124,8 +124,9 @@ def _conv_like(transposed, x, filter, mask, bias, stride, padding, dilation, gro
     if out_mask is None:
         out_mask = new_mask(g.batch, g.out_h, g.out_w, x.device)
     dt = _dtype(x)
+    # `keep`: the tracer replays recorded calls later; buffers allocated here must outlive them
     meta = dict(g=g, esize=x.element_size(), in_mask=mask, out_mask=out_mask,
-                mfma=packed_filter is not None)
+                mfma=packed_filter is not None, keep=(x, filter, packed_filter, bias, out))
     if epilogue is not None:
         prev, trunc, thr, act, mode = epilogue
         _call("conv_act", lib.dc_conv_act,
@@ -243,7 +244,8 @@ def sparse_pooling(x, prev_x, kernel_size, mask=None, stride=(1, 1), padding=(0,
     _call("pool", lib.dc_pool,
           (g, x.data_ptr(), _ptr(prev_x), out.data_ptr(), _mask(mask, "mask").data_ptr(),
            out_mask.data_ptr(), int(pooling_mode_int), _dtype(x), _dtype(out), _stream()),
-          g=g, esize=x.element_size(), in_mask=mask, out_mask=out_mask, mode=int(pooling_mode_int))
+          g=g, esize=x.element_size(), in_mask=mask, out_mask=out_mask, mode=int(pooling_mode_int),
+          keep=(x, prev_x, out))
     if out.dtype != x.dtype:
         out = out.to(dtype=x.dtype)
     if create_out_mask:
@@ -338,7 +340,8 @@ def sparse_upsample(input, mask_in, scale, out=None):
     _call("upsample", lib.dc_upsample,
           (input.data_ptr(), out_t.data_ptr(), _mask(mask_in, "mask_in").data_ptr(),
            mask_out.data_ptr(), b, h, w, c, scale, _dtype(input), _stream()),
-          P=b * h * w, C=c, esize=input.element_size(), in_mask=mask_in, scale=scale)
+          P=b * h * w, C=c, esize=input.element_size(), in_mask=mask_in, scale=scale,
+          keep=(input, out_t, mask_out))
     return out_t, mask_out
 
 
@@ -360,5 +363,5 @@ def sparse_concatenate(a, b, out=None):
            _mask(mask_b, "mask_b").data_ptr(), mask_out.data_ptr(), _pixels(a), a.shape[1],
            b.shape[1], _dtype(a), _stream()),
           P=_pixels(a), C=a.shape[1], Cb=b.shape[1], esize=a.element_size(), in_mask=mask_a,
-          in_mask_b=mask_b, out_mask=mask_out)
+          in_mask_b=mask_b, out_mask=mask_out, keep=(a, b, out_t))
     return out_t, mask_out

@@ -70,7 +70,10 @@ class Tracer:
         two events.  Returns microseconds per call, one per record; a call that launches two
         kernels (convolution, then activation/truncation) also gets ``split_us`` per kernel.
 
-        Every call has to see the masks of the traced frame, so
+        The replays pass the recorded device pointers again: operands of the traced calls
+        must still be allocated (the records hold references to the masks and to every buffer
+        the wrappers allocated themselves; tensors the caller passed in are the caller's to
+        keep).  Every call has to see the masks of the traced frame, so
           * records are replayed last to first: a replay only disturbs its own outputs, whose
             consumers have been timed already;
           * an operator that works in place is replayed behind its producer (which restores the
