@@ -1247,6 +1247,185 @@ __global__ void pack_filter_kernel(const half_t *__restrict__ f, half_t *__restr
     }
 }
 
+
+// ------------------------------------------------------- few input channels on the matrix cores
+// Stems of large frames (Cin <= 4, window up to 8 x 8, stride <= 2, Cout <= 64, fp16).  With the
+// input channels padded to 4 in LDS, the 32 reduction elements of one MFMA step are one window
+// ROW: k = kx * 4 + ci for kx = 0..7, so the input fragment of lane (pixel, kq) -- elements
+// kq * 8 .. kq * 8 + 7 -- is simply the two neighbouring halo pixels kx = 2 kq, 2 kq + 1 of that
+// row, 16 contiguous bytes; no im2col copy exists.  Window columns past Kw and channel 3 of an
+// RGB input meet zero weights in the packed filter ([Cout tile][ky][lane][8], see
+// pack_stem_filter_kernel); inactive and out-of-bounds pixels are staged as zeros.
+// Workgroup = 8 x 8 output pixels, wavefront w = rows 2w, 2w + 1 x all R channel tiles, so the
+// keep decision of the fused activation stays inside the wavefront.  The halo's update mask is
+// kept as one bit row per halo row; an output is updated if its window meets a set bit.
+constexpr int STEM_K = 8;
+template <int R, int ACT>
+__global__ void __launch_bounds__(256)
+conv_stem_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
+                      const half_t *__restrict__ bias, half_t *__restrict__ out,
+                      const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, EpiP epi,
+                      int hal_h, int hal_wp) {
+    extern __shared__ __align__(16) unsigned char s_mem[];
+    half_t *s_x = reinterpret_cast<half_t *>(s_mem);                       // [hal_h][hal_wp][4]
+    unsigned *s_row = reinterpret_cast<unsigned *>(s_x + hal_h * hal_wp * 4);  // [hal_h]
+    const int b = blockIdx.z, ty0 = blockIdx.y * TILE, tx0 = blockIdx.x * TILE;
+    const int tid = threadIdx.x, wave = wave_id(), lane = lane_id();
+    const int l16 = lane & 15, kq = lane >> 4;
+    const int iy0 = ty0 * p.sh - p.pt, ix0 = tx0 * p.sw - p.pl;
+    // filter fragments of the wavefront's R channel tiles: requested first, used last (surplus
+    // tiles re-read the last one and are not stored)
+    const int co_tiles = (p.Co + 15) >> 4;
+    half8_t a[R][STEM_K];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int ky = 0; ky < STEM_K; ++ky)
+            a[r][ky] = *reinterpret_cast<const half8_t *>(wp + ((size_t)(min(r, co_tiles - 1) * p.Kh + min(ky, p.Kh - 1)) * WAVE + lane) * 8);
+    half4_t bv[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        bv[r] = half4_t{0, 0, 0, 0};
+        if (bias != nullptr) bv[r] = *reinterpret_cast<const half4_t *>(bias + min(r * 16 + kq * 4, p.Co - 4));
+    }
+    if (tid < hal_h) s_row[tid] = 0;
+    __syncthreads();
+    const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+    const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
+    for (int hp = tid; hp < hal_h * hal_wp; hp += 256) {
+        const int hy = hp / hal_wp, hx = hp - hy * hal_wp;
+        const int iy = iy0 + hy, ix = ix0 + hx;
+        const bool ok = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
+        const size_t pix = ok ? (size_t)iy * p.Wi + ix : 0;
+        const int word = mb[pix];
+        half4_t v;
+#pragma unroll
+        for (int ci = 0; ci < 4; ++ci) v[ci] = inb[pix * p.Ci + min(ci, p.Ci - 1)];
+        const bool m = ok && word != 0;
+#pragma unroll
+        for (int ci = 0; ci < 4; ++ci) v[ci] = (m && ci < p.Ci) ? v[ci] : half_t(0);
+        *reinterpret_cast<half4_t *>(s_x + hp * 4) = v;
+        if (m) atomicOr(&s_row[hy], 1u << hx);
+    }
+    __syncthreads();
+
+    const int ly = wave * 2 + (l16 >> 3), lx = l16 & 7;
+    const int oy = ty0 + ly, ox = tx0 + lx;
+    const bool inside = oy < p.Ho && ox < p.Wo;
+    unsigned any = 0;
+    for (int ky = 0; ky < p.Kh; ++ky) any |= (s_row[ly * p.sh + ky] >> (lx * p.sw)) & ((1u << p.Kw) - 1u);
+    const bool upd = inside && any != 0;
+    const size_t po = ((size_t)b * p.Ho + oy) * p.Wo + ox;
+    if (inside && kq == 0 && (ACT < 0 || !upd)) out_mask[po] = upd ? 1 : 0;
+    if (ballot(upd) == 0) return;
+
+    // cached state of the fused epilogue, requested before the contraction
+    half4_t q[R], tr[R];
+    if (ACT >= 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const size_t off = (upd ? po : 0) * p.Co + min(r * 16 + kq * 4, p.Co - 4);
+            q[r] = *reinterpret_cast<const half4_t *>((const half_t *)epi.prev + off);
+            tr[r] = *reinterpret_cast<const half4_t *>((const half_t *)epi.trunc + off);
+        }
+    }
+    float4_t acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ky = 0; ky < STEM_K; ++ky) {
+        if (ky < p.Kh) {  // uniform
+            const half_t *xp = s_x + ((ly * p.sh + ky) * hal_wp + lx * p.sw + 2 * kq) * 4;
+            const half4_t x0 = *reinterpret_cast<const half4_t *>(xp), x1 = *reinterpret_cast<const half4_t *>(xp + 4);
+            const half8_t x = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[r][ky], x, acc[r], 0, 0, 0);
+        }
+    }
+    half4_t v[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[r][i] = half_t(acc[r][i] + float(bv[r][i]));
+    if (ACT < 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int co = r * 16 + kq * 4;
+            if (upd && co < p.Co) *reinterpret_cast<half4_t *>(out + po * p.Co + co) = v[r];
+        }
+        return;
+    }
+    // activation + truncation, the operations and roundings of act_trunc_pixel; the statistics
+    // of a pixel are combined over its four kq lanes
+    constexpr int ACTC = ACT < 0 ? 0 : ACT;
+    const half_t thr = half_t(epi.thr);
+    half4_t t[R], sm[R], d[R];
+    bool hit = false;
+    float sq = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const bool live = upd && r * 16 + kq * 4 < p.Co;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            t[r][i] = tr[r][i] + v[r][i];
+            sm[r][i] = t[r][i] + q[r][i];
+            d[r][i] = act_apply<half_t>(sm[r][i], ACTC) - act_apply<half_t>(q[r][i], ACTC);
+            if (live) {
+                hit |= tabs(d[r][i]) > thr;
+                sq += float(d[r][i]) * float(d[r][i]);
+            }
+        }
+    }
+    bool keep;
+    if (epi.mode == DC_TRUNC_MAX) {
+        const uint64_t bl = ballot(hit);
+        keep = ((bl >> l16) & 0x0001000100010001ull) != 0;
+    } else {
+        sq += __shfl_xor(sq, 16, WAVE);
+        sq += __shfl_xor(sq, 32, WAVE);
+        if (epi.mode == DC_TRUNC_RMS) sq /= float(p.Co);
+        keep = sqrtf(sq) > float(thr);
+    }
+    if (!upd) return;
+    if (kq == 0) out_mask[po] = keep ? 1 : 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int co = r * 16 + kq * 4;
+        if (co >= p.Co) continue;
+        const size_t off = po * p.Co + co;
+        if (keep) {
+            *reinterpret_cast<half4_t *>((half_t *)epi.prev + off) = sm[r];
+            *reinterpret_cast<half4_t *>(out + off) = d[r];
+            *reinterpret_cast<half4_t *>((half_t *)epi.trunc + off) = half4_t{0, 0, 0, 0};
+        } else {
+            *reinterpret_cast<half4_t *>((half_t *)epi.trunc + off) = t[r];
+        }
+    }
+}
+
+// Filter of conv_stem_mfma_kernel: fragment (channel tile, ky) holds, for lane (l16, kq) and
+// element e, W[co = tile * 16 + l16][ky][kx = (kq * 8 + e) / 4][ci = (kq * 8 + e) % 4], zero past
+// Kw, Cin and Cout.  Reads the processed fp16 layout (rows swizzled by the output parity).
+__global__ void pack_stem_filter_kernel(const half_t *__restrict__ f, half_t *__restrict__ wp, int Ci,
+                                        int Co, int Kh, int Kw, int w_co, int co_tiles) {
+    const int total = co_tiles * Kh * 512;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        const int e = i & 7, lane = (i >> 3) & 63, frag = i >> 9;
+        const int ky = frag % Kh, ct = frag / Kh;
+        const int co = ct * 16 + (lane & 15), k = (lane >> 4) * 8 + e;
+        const int kx = k >> 2, ci = k & 3;
+        half_t v = half_t(0);
+        if (kx < Kw && ci < Ci && co < Co) v = f[((size_t)(ci ^ (co & 1)) * Kh * Kw + ky * Kw + kx) * w_co + co];
+        wp[i] = v;
+    }
+}
+
+inline bool stem_eligible(const dc_geometry &g, int dtype) {
+    return dtype == DC_F16 && g.groups == 1 && g.in_c <= 4 && g.kernel_h <= STEM_K && g.kernel_w <= STEM_K &&
+           g.dilation_h == 1 && g.dilation_w == 1 && g.stride_h <= 2 && g.stride_w <= 2 && g.out_c % 4 == 0 &&
+           g.out_c <= 64;
+}
+
 inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 inline bool mfma_eligible(const dc_geometry &g, int dtype) {
@@ -1270,14 +1449,21 @@ ConvP make_params(const dc_geometry &g, int dtype) {
 }  // namespace
 
 int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed) {
-    (void)transposed;
+    if (!transposed && stem_eligible(g, dtype)) return (int64_t)ceil_div(g.out_c, 16) * g.kernel_h * 1024;
     if (!mfma_eligible(g, dtype)) return 0;
     return (int64_t)round_up(g.out_c, 16) * g.kernel_h * g.kernel_w * round_up(g.in_c, 32) * 2;
 }
 
 hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *packed, int dtype,
                               bool transposed, hipStream_t s) {
-    (void)transposed;
+    if (!transposed && stem_eligible(g, dtype)) {
+        note_kernel("pack_stem_filter_kernel");
+        const int co_tiles = ceil_div(g.out_c, 16);
+        pack_stem_filter_kernel<<<ceil_div(co_tiles * g.kernel_h * 512, 256), 256, 0, s>>>(
+            (const half_t *)filter, (half_t *)packed, g.in_c, g.out_c, g.kernel_h, g.kernel_w,
+            g.out_c + (g.out_c & 1), co_tiles);
+        return hipGetLastError();
+    }
     if (!mfma_eligible(g, dtype)) return hipSuccess;
     const int K2 = g.kernel_h * g.kernel_w;
     const int ci_p = round_up(g.in_c, 32), co_p = round_up(g.out_c, 16);
@@ -1367,6 +1553,44 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
         case 2: dw_launch<T, 2>(grid, block, eager, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
         default: dw_launch<T, 4>(grid, block, false, s, act, p, in, filter, bias, out, mask, out_mask, e, lg); break;
     }
+    return true;
+}
+
+// Stems of large frames on the matrix cores (see conv_stem_mfma_kernel); false if the shape, the
+// operands' alignment or the map size do not qualify.
+bool try_stem_mfma(const dc_geometry &g, const ConvP &p, const half_t *in, const half_t *packed,
+                   const half_t *bias, half_t *out, const int32_t *mask, int32_t *out_mask,
+                   const ActEpilogue *epi, hipStream_t s) {
+    const auto al8 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 7u) == 0; };
+    if (packed == nullptr || !stem_eligible(g, DC_F16)) return false;
+    // many channel tiles on a large map: the per-pixel kernel's wide stores win (measured)
+    if (g.out_c > 32 && (int64_t)g.batch * g.out_h * g.out_w > 65536) return false;
+    if (!al8(out) || (bias && !al8(bias)) || (reinterpret_cast<uintptr_t>(packed) & 15u) != 0) return false;
+    if (epi && (epi->mode < 0 || epi->trunc == nullptr || !al8(epi->prev) || !al8(epi->trunc))) return false;
+    const int hal_h = (TILE - 1) * g.stride_h + g.kernel_h;
+    const int hal_wp = (TILE - 1) * g.stride_w + STEM_K;  // every lane reads 8 window columns
+    const size_t lds = (size_t)hal_h * hal_wp * 8 + (size_t)hal_h * 4;
+    dim3 grid(ceil_div(g.out_w, TILE), ceil_div(g.out_h, TILE), g.batch);
+    EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f, epi ? epi->mode : 0};
+    const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
+    const int co_tiles = ceil_div(g.out_c, 16);
+    note_kernel("conv_stem_mfma_kernel");
+#define DC_ST_R(A)                                                                                                   \
+    do {                                                                                                             \
+        if (co_tiles == 1) conv_stem_mfma_kernel<1, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
+        else if (co_tiles == 2) conv_stem_mfma_kernel<2, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
+        else conv_stem_mfma_kernel<4, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
+    } while (0)
+    switch (act) {
+        case DC_ACT_LINEAR: DC_ST_R(DC_ACT_LINEAR); break;
+        case DC_ACT_RELU: DC_ST_R(DC_ACT_RELU); break;
+        case DC_ACT_RELU6: DC_ST_R(DC_ACT_RELU6); break;
+        case DC_ACT_LEAKY: DC_ST_R(DC_ACT_LEAKY); break;
+        case DC_ACT_SIGMOID: DC_ST_R(DC_ACT_SIGMOID); break;
+        case DC_ACT_SWISH: DC_ST_R(DC_ACT_SWISH); break;
+        default: DC_ST_R(-1); break;
+    }
+#undef DC_ST_R
     return true;
 }
 
@@ -1472,6 +1696,9 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
             ? try_depthwise<float>(g, p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, epi, s)
             : try_depthwise<half_t>(g, p, (const half_t *)in, (const half_t *)filter, (const half_t *)bias, (half_t *)out, mask, out_mask, epi, s);
         if (done) return hipGetLastError();
+        if (dtype == DC_F16 && try_stem_mfma(g, p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias,
+                                             (half_t *)out, mask, out_mask, epi, s))
+            return hipGetLastError();
         const bool few = dtype == DC_F32
             ? try_fewcin<float>(g, p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, epi, s)
             : try_fewcin<half_t>(g, p, (const half_t *)in, (const half_t *)filter, (const half_t *)bias, (half_t *)out, mask, out_mask, epi, s);

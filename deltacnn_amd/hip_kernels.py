@@ -203,7 +203,8 @@ def sparse_deconv(x, filter, mask=None, bias=None, stride=(1, 1), padding=(0, 0)
 def pack_filter(filter: torch.Tensor, c_in: int, c_out: int, groups: int = 1,
                 transposed: bool = False) -> Optional[torch.Tensor]:
     """One-time relayout of a processed fp16 filter for the MFMA kernels; None if the shape
-    has no packed form (fp32, grouped, Cin % 8 != 0)."""
+    has no packed form (fp32, grouped, or an input channel count that is neither a multiple
+    of 8 nor a stem's: Cin <= 4 with a window up to 8 x 8 and Cout <= 64)."""
     lib = _lib.load()
     if filter.dtype != torch.float16:
         return None

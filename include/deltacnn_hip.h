@@ -128,8 +128,12 @@ int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filt
 /* Number of bytes dc_pack_filter writes for this geometry (0 if the shape has no packed
  * form).  One-time weight relayout for the MFMA kernels, fp16, un-swizzled, in fragment order
  * [Cout tile of 16][Kh][Kw][Cin step of 32][lane 0..63][8] (lane kq*16+r holds input channels
- * kq*8..+8 of output channel r): round_up(Cout,16) * Kh * Kw * round_up(Cin,32) halves.  The
- * buffer is opaque to callers: only dc_pack_filter writes it and only this library reads it. */
+ * kq*8..+8 of output channel r): round_up(Cout,16) * Kh * Kw * round_up(Cin,32) halves.
+ * Stems (Cin <= 4, window up to 8 x 8, Cout <= 64 and a multiple of 4, not transposed) pack as
+ * [Cout tile of 16][Kh][lane][8] with reduction element k = kx * 4 + ci of a window row,
+ * ceil(Cout / 16) * Kh * 512 halves.  The buffer is opaque to callers: only dc_pack_filter
+ * writes it and only this library reads it; it has to be made from the same Cin, Cout and
+ * window as the convolution it is handed to. */
 int64_t dc_packed_filter_bytes(const dc_geometry *g, int dtype, int transposed);
 int dc_pack_filter(const dc_geometry *g, const void *filter, void *packed_filter, int dtype,
                    int transposed, void *stream);

@@ -319,6 +319,13 @@ CONVS = [
     (40, 24, (1, 3), (1, 2), (0, 1), 1, 1, 8, 16),
     (12, 18, 3, 1, 1, 1, 3, 8, 8),          # general groups (fp32 only)
     (5, 7, 3, 1, 1, 1, 1, 9, 9),            # odd channels: fp16 padding rows/cols of the swizzle
+    # stems on the matrix cores (fp16 packed): window rows as reduction steps
+    (3, 16, 7, 1, 3, 1, 1, 37, 45),
+    (3, 64, 3, 2, 1, 1, 1, 40, 41),
+    (4, 24, 5, 1, 2, 1, 1, 19, 23),
+    (1, 8, 3, 1, 1, 1, 1, 16, 16),
+    (3, 48, 7, 2, 3, 1, 1, 33, 35),
+    (2, 64, 8, 2, 3, 1, 1, 30, 30),
     # layers large enough for the LDS-halo MFMA kernel (fp16 packed), one per arrangement / corner
     (64, 64, 3, 1, 1, 1, 1, 72, 70),        # two channel tiles per wave, steps split over two waves
     (64, 32, 3, 1, 1, 1, 1, 100, 100),      # ... over four waves (one channel group)
@@ -401,7 +408,9 @@ def test_conv(lib, dtype, cfg, density, use_bias, packed):
     ((64, 256, 1, 1, 0, 1, 1, 20, 20), "pw_mfma_kernel"),
     ((32, 32, 3, 1, 1, 1, 32, 15, 18), "conv_dw_kernel"),
     ((16, 16, 3, 1, 1, 1, 16, 726, 727), "conv_dw_strip_kernel"),
-    ((3, 32, 3, 2, 1, 1, 1, 33, 31), "conv_fewcin_kernel"),
+    ((3, 32, 3, 2, 1, 1, 1, 33, 31), "conv_stem_mfma_kernel"),
+    ((3, 64, 3, 2, 1, 1, 1, 600, 520), "conv_fewcin_kernel"),     # many channel tiles on a large map
+    ((3, 32, 3, 2, 1, 2, 1, 33, 31), "conv_fewcin_kernel"),       # dilation: no matrix-core form
 ], ids=lambda v: v if isinstance(v, str) else "-".join(str(x) for x in v))
 def test_conv_dispatch(lib, cfg, kernel):
     """The shapes the parity cases above are chosen for reach the kernel they are meant to cover
@@ -481,6 +490,9 @@ FUSED = [
     (64, 64, 3, 2, 1, 1, 64, 13, 13),       # depthwise stride 2
     (24, 24, 5, 1, 2, 1, 24, 12, 12),       # depthwise 5x5 (generic tap loop)
     (3, 32, 3, 2, 1, 1, 1, 24, 24),         # RGB stem
+    (3, 16, 7, 1, 3, 1, 1, 37, 45),         # 7x7 RGB stem
+    (3, 64, 3, 2, 1, 1, 1, 40, 41),         # four channel tiles per wavefront
+    (4, 24, 5, 1, 2, 1, 1, 19, 23),         # partial channel tile
     (96, 96, 3, 1, 1, 1, 96, 96, 96),       # large map: two vectors per lane
     (24, 24, 3, 1, 1, 1, 24, 192, 192),     # large map: three vectors per lane
     (16, 16, 3, 1, 1, 1, 16, 726, 727),     # very large map: strips of four pixels per lane group
