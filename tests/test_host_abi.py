@@ -93,6 +93,14 @@ def test_packed_filter_size_is_host_arithmetic(lib):
     assert lib.dc_packed_filter_bytes(ctypes.byref(g), 0, 0) == 0
     g = _geom(groups=16)
     assert lib.dc_packed_filter_bytes(ctypes.byref(g), 1, 0) == 0
+    # stems (Cin <= 4, window <= 8 x 8, Cout <= 64 and a multiple of 4): one KB per (channel tile, row)
+    g = _geom(in_c=3, out_c=24, kernel_h=7, kernel_w=7)
+    assert lib.dc_packed_filter_bytes(ctypes.byref(g), 1, 0) == 2 * 7 * 1024
+    assert lib.dc_packed_filter_bytes(ctypes.byref(g), 1, 1) == 0      # not for transposed convolutions
+    assert lib.dc_packed_filter_bytes(ctypes.byref(g), 0, 0) == 0      # fp32
+    for bad in (dict(in_c=5), dict(out_c=22), dict(out_c=80), dict(kernel_h=9, kernel_w=9)):
+        g = _geom(**{**dict(in_c=3, out_c=24, kernel_h=7, kernel_w=7), **bad})
+        assert lib.dc_packed_filter_bytes(ctypes.byref(g), 1, 0) == 0, bad
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
