@@ -792,13 +792,23 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
         }
         return;
     }
-    build_steps(0, min(kcc, ksteps));
-    // halo table: global pixel index of every active in-bounds halo pixel, -1 otherwise
-    for (int i = tid; i < hpx; i += nthr) {
+    // halo table: global pixel index of every active in-bounds halo pixel, -1 otherwise.  The
+    // mask word of a thread's first halo pixel is requested before the step table is built, so
+    // the table's arithmetic runs while it travels.
+    auto halo_pixel = [&](int i, bool &ok) {
         const int hy = i / hal_w, hx = i - hy * hal_w;
         const int iy = iy0 + hy, ix = ix0 + hx;
-        const bool ok = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
-        const int px = ok ? iy * p.Wi + ix : 0;
+        ok = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
+        return ok ? iy * p.Wi + ix : 0;
+    };
+    bool ok0;
+    const int hpix0 = halo_pixel(min(tid, hpx - 1), ok0);
+    const int hword0 = mb[hpix0];
+    build_steps(0, min(kcc, ksteps));
+    if (tid < hpx) s_hpix[tid] = (ok0 && hword0 != 0) ? hpix0 : -1;
+    for (int i = tid + nthr; i < hpx; i += nthr) {
+        bool ok;
+        const int px = halo_pixel(i, ok);
         const int word = mb[px];
         s_hpix[i] = (ok && word != 0) ? px : -1;
     }
