@@ -324,7 +324,7 @@ __device__ __forceinline__ void pw_epilogue_store(const half4_t (&q)[CTW], const
 // the stores.  Longer reductions stream two steps per round trip in ascending order (the same
 // summation order as the convolution-only kernel without reduction split).  What is loaded
 // for inactive pixels is dropped.  Requires Cout % 4 == 0.
-template <int NW, int CTW, int ACT, bool EAGER>
+template <int NW, int CTW, int ACT>
 __global__ void __launch_bounds__(NW * WAVE)
 pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                    const half_t *__restrict__ bias, half_t *__restrict__ out,
@@ -338,20 +338,10 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
     const int px = blockIdx.x * 16 + l16;
     const int pxc = min(px, p.P - 1);
     const int m = mask[pxc];
-    // EAGER (small maps): every operand is requested before the mask word has arrived.  On large
-    // maps that would read the cached state of every pixel, active or not; there the mask is
-    // waited for first, a workgroup without active pixels leaves at once, and an inactive lane
-    // shadows the first active pixel of its tile, so it adds no memory traffic.
-    int pl = pxc;
-    if (!EAGER) {
-        const bool on0 = px < p.P && m != 0;
-        const uint64_t act16 = ballot(on0) & 0xffffull;
-        if (act16 == 0) {
-            if (wave == 0 && kq == 0 && px < p.P) out_mask[px] = 0;
-            return;
-        }
-        if (!on0) pl = blockIdx.x * 16 + (__ffsll((unsigned long long)act16) - 1);
-    }
+    // Every operand is requested before the mask word has arrived (the host uses this kernel
+    // while the cached state of the whole map is a few MB: reading it for inactive pixels too
+    // costs less than a second memory round trip).
+    const int pl = pxc;
     const half_t *wrow[CTW];
 #pragma unroll
     for (int j = 0; j < CTW; ++j)
@@ -504,10 +494,13 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     // over many workgroups) is faster.
     const bool fusable = res == nullptr && epi != nullptr && epi->mode >= 0 && g.out_c % 4 == 0 && al8(epi->prev) &&
                          al8(epi->trunc) && al8(out);
-    // ... and not for large problems either (>= 4096 output tiles of 16x16 with a reduction of
-    // several steps): there fragment traffic dominates, and the convolution-only kernel reuses
-    // every fragment 4 times where a 16-pixel workgroup cannot.
-    const bool large = (int64_t)ceil_div(p.P, 16) * p.co_tiles >= 4096 && ksteps >= 2;
+    // ... and not for large problems either: >= 4096 output tiles of 16x16 with a reduction of
+    // several steps (there fragment traffic dominates, and the convolution-only kernel reuses
+    // every fragment 4 times where a 16-pixel workgroup cannot), or an output map beyond 4 MB
+    // (as with many streams in a batch: there the epilogue's 8-byte accesses per lane hold the
+    // fused kernel at a quarter of the bandwidth the separate activation kernel reaches).
+    const bool large = ((int64_t)ceil_div(p.P, 16) * p.co_tiles >= 4096 && ksteps >= 2) ||
+                       (int64_t)p.P * p.Co * 2 > (4 << 20);
     if (fusable && ksteps <= PW_FUSED_MAX_STEPS && p.P >= 512 && !large) {
         dim3 grid(ceil_div(p.P, 16));
         const int act = epi->act < 0 ? 0 : epi->act;
@@ -515,21 +508,12 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
         // as many wavefronts as channel tiles, up to 16; then several tiles per wavefront
         const int nw = p.co_tiles <= 4 ? 4 : p.co_tiles <= 8 ? 8 : 16;
         const int ctw = ceil_div(p.co_tiles, nw);
-        // eager operand requests while the cached state of the whole map is small (stays in L2)
-        const bool eager = (int64_t)p.P * p.Co * 2 <= (4 << 20);
 #define DC_GO(NW, CTW)                                                                                \
     do {                                                                                              \
-        if (eager) {                                                                                  \
-            DC_ACT_SWITCH(act, (pw_act_mfma_kernel<NW, CTW, A, true><<<grid, NW * WAVE, 0, s>>>(      \
-                                   p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, \
-                                   (half_t *)out, mask, out_mask, (half_t *)epi->prev,                \
-                                   (half_t *)epi->trunc, epi->thr, epi->mode)));                      \
-        } else {                                                                                      \
-            DC_ACT_SWITCH(act, (pw_act_mfma_kernel<NW, CTW, A, false><<<grid, NW * WAVE, 0, s>>>(     \
-                                   p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, \
-                                   (half_t *)out, mask, out_mask, (half_t *)epi->prev,                \
-                                   (half_t *)epi->trunc, epi->thr, epi->mode)));                      \
-        }                                                                                             \
+        DC_ACT_SWITCH(act, (pw_act_mfma_kernel<NW, CTW, A><<<grid, NW * WAVE, 0, s>>>(                \
+                               p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias,   \
+                               (half_t *)out, mask, out_mask, (half_t *)epi->prev,                    \
+                               (half_t *)epi->trunc, epi->thr, epi->mode)));                          \
         *epilogue_done = true;                                                                        \
         return hipGetLastError();                                                                     \
     } while (0)

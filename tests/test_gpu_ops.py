@@ -496,7 +496,7 @@ FUSED = [
     (96, 96, 3, 1, 1, 1, 96, 96, 96),       # large map: two vectors per lane
     (24, 24, 3, 1, 1, 1, 24, 192, 192),     # large map: three vectors per lane
     (16, 16, 3, 1, 1, 1, 16, 726, 727),     # very large map: strips of four pixels per lane group
-    (16, 96, 1, 1, 0, 1, 1, 110, 111),      # pointwise on a large map: operands requested after the mask
+    (16, 96, 1, 1, 0, 1, 1, 110, 111),      # pointwise on a large map: convolution and activation as two launches
 ]
 
 
