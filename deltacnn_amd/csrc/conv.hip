@@ -381,6 +381,120 @@ conv_dw_strip_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ fi
     }
 }
 
+
+// Depthwise 3x3 on maps of at least 2^18 outputs, any update density: a wavefront owns 64
+// consecutive output pixels, one per lane while the nine mask words of the window are read and
+// the output mask is written; the updated outputs are listed in LDS -- pixel, coordinates and the
+// set of updated taps -- and served two at a time per lane group (one 16-byte vector per lane).
+// A sparse map costs no idle lane groups, and the delta of a tap that was not updated is not
+// fetched (its request goes to an updated tap's row, which is being read anyway).  The filter
+// of the lane's channels is loaded once.  Per pixel the arithmetic is that of conv_dw_kernel.
+template <typename T, int ACT>
+__global__ void __launch_bounds__(256)
+conv_dw_scan_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
+                    const T *__restrict__ bias, T *__restrict__ out,
+                    const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, EpiP epi,
+                    int lg) {
+    constexpr int N = Vec16<T>::N;
+    __shared__ int s_pix[4][WAVE], s_yx[4][WAVE], s_img[4][WAVE], s_taps[4][WAVE];
+    const int Po = p.B * p.Ho * p.Wo, C = p.Ci;
+    const int wave = wave_id(), lane = lane_id();
+    const int po = (blockIdx.x * 4 + wave) * WAVE + lane;
+    int taps = 0;  // bit t: tap t is inside the map and updated
+    int yx, img;
+    {
+        const int pc = min(po, Po - 1);
+        const int row = pc / p.Wo, ox = pc - row * p.Wo;
+        const int b = row / p.Ho, oy = row - b * p.Ho;
+        yx = (oy << 16) | ox;
+        img = b * p.Hi * p.Wi;
+        int mw[9];
+        bool inside[9];
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const int iy = oy * p.sh - p.pt + (t / 3) * p.dh, ix = ox * p.sw - p.pl + (t % 3) * p.dw;
+            inside[t] = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
+            mw[t] = mask[(size_t)img + min(max(iy, 0), p.Hi - 1) * p.Wi + min(max(ix, 0), p.Wi - 1)];
+        }
+#pragma unroll
+        for (int t = 0; t < 9; ++t) taps |= (inside[t] && mw[t] != 0) ? 1 << t : 0;
+    }
+    if (po >= Po) taps = 0;
+    if (po < Po) out_mask[po] = taps != 0 ? 1 : 0;
+    int n;
+    const int rank = wave_rank(taps != 0, n);
+    if (n == 0) return;
+    if (taps != 0) {
+        s_pix[wave][rank] = po;
+        s_yx[wave][rank] = yx;
+        s_img[wave][rank] = img;
+        s_taps[wave][rank] = taps;
+    }
+    const int G = 1 << lg, gl = lane & (G - 1), grp = lane >> lg, ppi = WAVE >> lg;
+    const bool mine = gl * N < C;
+    const int c = min(gl * N, C - N);
+    Vec<T, N> w[9], bv;
+#pragma unroll
+    for (int t = 0; t < 9; ++t) w[t] = vload<T, N>(filter + (size_t)t * C + c);
+    if (bias != nullptr) bv = vload<T, N>(bias + c);
+    constexpr int U = 2;
+    for (int k = 0; k < n; k += U * ppi) {
+        Vec<T, N> x[U][9], q[U][1], tr[U][1];
+        bool valid[U];
+        int pix[U], tp[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int idx = k + u * ppi + grp, e = min(idx, n - 1);
+            valid[u] = idx < n && mine;
+            pix[u] = s_pix[wave][e];
+            tp[u] = s_taps[wave][e];
+            const int oy = s_yx[wave][e] >> 16, ox = s_yx[wave][e] & 0xffff;
+            const size_t base = (size_t)s_img[wave][e];
+            const int first = __builtin_ctz(tp[u]);  // an updated tap: the list holds no other pixels
+            size_t ip[9];
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                const int iy = min(max(oy * p.sh - p.pt + (t / 3) * p.dh, 0), p.Hi - 1);
+                const int ix = min(max(ox * p.sw - p.pl + (t % 3) * p.dw, 0), p.Wi - 1);
+                ip[t] = base + (size_t)iy * p.Wi + ix;
+            }
+            size_t ifirst = ip[0];
+#pragma unroll
+            for (int t = 1; t < 9; ++t) ifirst = first == t ? ip[t] : ifirst;
+#pragma unroll
+            for (int t = 0; t < 9; ++t) x[u][t] = vload<T, N>(in + (((tp[u] >> t) & 1) ? ip[t] : ifirst) * C + c);
+            if (ACT >= 0)
+                load_state<T, 1>(q[u], tr[u], valid[u], (size_t)pix[u], gl, G, C, (const T *)epi.prev, (const T *)epi.trunc);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (k + u * ppi >= n) continue;  // wave-uniform
+            float acc[N];
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc[e] = 0.f;
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                const Vec<T, N> xs = vkeep<T, N>(x[u][t], (tp[u] >> t) & 1);
+#pragma unroll
+                for (int e = 0; e < N; ++e) acc[e] = __builtin_fmaf(float(xs.v[e]), float(w[t].v[e]), acc[e]);
+            }
+            Vec<T, N> dl[1];
+            if (bias != nullptr) {
+#pragma unroll
+                for (int e = 0; e < N; ++e) acc[e] += float(bv.v[e]);
+            }
+#pragma unroll
+            for (int e = 0; e < N; ++e) dl[0].v[e] = T(acc[e]);
+            if (ACT < 0) {
+                if (valid[u]) vstore<T, N>(out + (size_t)pix[u] * C + c, dl[0]);
+            } else {
+                act_trunc_pixel<T, 1, (ACT < 0 ? 0 : ACT)>(dl, q[u], tr[u], valid[u], (size_t)pix[u], gl, G, C, out,
+                                                            (T *)epi.prev, (T *)epi.trunc, out_mask, T(epi.thr), epi.mode);
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------ few input channels
 // Network stems (RGB input): groups == 1, Cin <= 4.  Same one-group-per-output-pixel shape as
 // the depthwise kernel; a lane owns N consecutive output channels, input values are scalar
@@ -1522,6 +1636,31 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
     if (epi && (!al(epi->prev) || (epi->trunc && !al(epi->trunc)) || epi->mode < 0)) return false;
     const int64_t P_out = (int64_t)g.batch * g.out_h * g.out_w;
     const int nvec = g.in_c / N;
+    // very large maps: mask scan and compaction per wavefront (see conv_dw_scan_kernel)
+    // (measured against the strip kernel and the per-pixel kernel on sparse and dense maps: it
+    // wins from 2^18 outputs on, with a stride -- where no strip kernel exists -- from 2^16)
+    const bool strided = g.stride_h > 1 || g.stride_w > 1;
+    if (g.kernel_h == 3 && g.kernel_w == 3 && nvec <= WAVE && P_out >= (strided ? 1 << 16 : 1 << 18) && P_out < (1ll << 31) &&
+        (int64_t)g.batch * g.in_h * g.in_w < (1ll << 31) && g.out_h < 65536 && g.out_w < 65536 &&
+        (epi == nullptr || epi->trunc != nullptr)) {
+        const int lg = log2i(group_lanes(nvec, 1));
+        dim3 grid((unsigned)ceil_div64(P_out, 4 * WAVE));
+        EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f, epi ? epi->mode : 0};
+        const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
+        note_kernel("conv_dw_scan_kernel");
+#define DC_DWN(A) conv_dw_scan_kernel<T, A><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg)
+        switch (act) {
+            case DC_ACT_LINEAR: DC_DWN(DC_ACT_LINEAR); break;
+            case DC_ACT_RELU: DC_DWN(DC_ACT_RELU); break;
+            case DC_ACT_RELU6: DC_DWN(DC_ACT_RELU6); break;
+            case DC_ACT_LEAKY: DC_DWN(DC_ACT_LEAKY); break;
+            case DC_ACT_SIGMOID: DC_DWN(DC_ACT_SIGMOID); break;
+            case DC_ACT_SWISH: DC_DWN(DC_ACT_SWISH); break;
+            default: DC_DWN(-1); break;
+        }
+#undef DC_DWN
+        return true;
+    }
     // large maps: strips of four output pixels per group of lanes (see conv_dw_strip_kernel)
     if (g.kernel_h == 3 && g.kernel_w == 3 && g.stride_h == 1 && g.stride_w == 1 && g.dilation_h == 1 &&
         g.dilation_w == 1 && nvec <= WAVE && P_out * g.in_c * (int64_t)sizeof(T) >= (4 << 20)) {

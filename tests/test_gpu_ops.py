@@ -337,8 +337,11 @@ CONVS = [
     (64, 48, 3, 1, 2, 2, 1, 80, 81),        # dilation 2
     (32, 64, 5, 1, 2, 1, 1, 64, 66),        # 5x5
     (24, 40, 3, 1, 1, 1, 1, 128, 130),      # partial reduction step and partial channel tile
-    (16, 16, 3, 1, 1, 1, 16, 726, 727),     # depthwise on a large map: strips of four pixels per lane group
+    (16, 16, 3, 1, 1, 1, 16, 726, 727),     # depthwise on a very large map: mask scan and compaction per wavefront
     (24, 24, 3, 1, 1, 1, 24, 600, 601),     # ... with idle lanes in the group
+    (16, 16, 3, 2, 1, 1, 16, 600, 521),     # ... with a stride
+    (16, 16, 3, 1, 1, 1, 16, 300, 301),     # depthwise on a large map: strips of four pixels per lane group
+    (24, 24, 3, 1, 1, 1, 24, 250, 251),     # ... with idle lanes in the group
 ]
 
 
@@ -407,7 +410,9 @@ def test_conv(lib, dtype, cfg, density, use_bias, packed):
     ((320, 32, 3, 1, 1, 1, 1, 40, 40), "conv_lds_mfma_kernel"),
     ((64, 256, 1, 1, 0, 1, 1, 20, 20), "pw_mfma_kernel"),
     ((32, 32, 3, 1, 1, 1, 32, 15, 18), "conv_dw_kernel"),
-    ((16, 16, 3, 1, 1, 1, 16, 726, 727), "conv_dw_strip_kernel"),
+    ((16, 16, 3, 1, 1, 1, 16, 726, 727), "conv_dw_scan_kernel"),
+    ((16, 16, 3, 1, 1, 1, 16, 300, 301), "conv_dw_strip_kernel"),
+    ((16, 16, 3, 2, 1, 1, 16, 600, 521), "conv_dw_scan_kernel"),
     ((3, 32, 3, 2, 1, 1, 1, 33, 31), "conv_stem_mfma_kernel"),
     ((3, 64, 3, 2, 1, 1, 1, 600, 520), "conv_fewcin_kernel"),     # many channel tiles on a large map
     ((3, 32, 3, 2, 1, 2, 1, 33, 31), "conv_fewcin_kernel"),       # dilation: no matrix-core form
@@ -495,7 +500,9 @@ FUSED = [
     (4, 24, 5, 1, 2, 1, 1, 19, 23),         # partial channel tile
     (96, 96, 3, 1, 1, 1, 96, 96, 96),       # large map: two vectors per lane
     (24, 24, 3, 1, 1, 1, 24, 192, 192),     # large map: three vectors per lane
-    (16, 16, 3, 1, 1, 1, 16, 726, 727),     # very large map: strips of four pixels per lane group
+    (16, 16, 3, 1, 1, 1, 16, 726, 727),     # very large map: mask scan and compaction per wavefront
+    (24, 24, 3, 2, 1, 1, 24, 600, 521),     # the same with a stride
+    (16, 16, 3, 1, 1, 1, 16, 300, 301),     # large map: strips of four pixels per lane group
     (16, 96, 1, 1, 0, 1, 1, 110, 111),      # pointwise on a large map: convolution and activation as two launches
 ]
 
@@ -613,7 +620,8 @@ def test_conv_add_fused_small_layers(lib, cfg, act, weights):
     (64, 64, 3, 1, 1, 1, 1, 72, 70),        # LDS-halo kernel
     (64, 256, 1, 1, 0, 1, 1, 20, 20),       # pointwise
     (32, 32, 3, 1, 1, 1, 32, 15, 18),       # depthwise
-    (16, 16, 3, 1, 1, 1, 16, 726, 727),     # depthwise strips
+    (16, 16, 3, 1, 1, 1, 16, 726, 727),     # depthwise, mask scan
+    (16, 16, 3, 1, 1, 1, 16, 300, 301),     # depthwise strips
     (3, 32, 3, 2, 1, 1, 1, 33, 31),         # stem
 ], ids=lambda c: "-".join(str(v) for v in c))
 def test_conv_uniform_masks(lib, cfg, fill):
