@@ -13,6 +13,8 @@
 //                     [Cout][tap][Cin]) and columns = compacted pixels (NHWC rows), so both
 //                     operands are 16-byte row loads and the accumulator tile stores 4
 //                     consecutive channels per lane
+#include <atomic>
+
 #include "epilogue.hpp"
 #include "tile.hpp"
 
@@ -1552,6 +1554,20 @@ inline bool stem_eligible(const dc_geometry &g, int dtype) {
 
 inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
+// Raises a kernel's dynamic LDS limit to 112 KB, once per kernel and device (the attribute belongs
+// to the device's copy of the function); a plain host call, nothing is put on a stream.
+template <typename K>
+hipError_t allow_large_lds(K *kernel) {
+    static std::atomic<uint64_t> done{0};  // one bit per device; devices past 63 ask every time
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 64 && ((done.load(std::memory_order_relaxed) >> dev) & 1ull)) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 112 << 10);
+    if (e == hipSuccess && dev < 64) done.fetch_or(1ull << dev, std::memory_order_relaxed);
+    return e;
+}
+
 inline bool mfma_eligible(const dc_geometry &g, int dtype) {
     return dtype == DC_F16 && g.groups == 1 && g.in_c % 8 == 0 && g.in_c >= 8;
 }
@@ -1923,10 +1939,10 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
 #define DC_LDS_ARGS (p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
 #define DC_LDS_K(RV, SV, DV, KV, TV)                                                                        \
     do {                                                                                                    \
-        static const hipError_t big = hipFuncSetAttribute(                                                  \
-            reinterpret_cast<const void *>(&conv_lds_mfma_kernel<RV, SV, DV, KV, TV>),                      \
-            hipFuncAttributeMaxDynamicSharedMemorySize, 112 << 10);                                         \
-        if (lds > (48u << 10) && big != hipSuccess) return big;                                             \
+        if (lds > (48u << 10)) {                                                                            \
+            const hipError_t big = allow_large_lds(&conv_lds_mfma_kernel<RV, SV, DV, KV, TV>);              \
+            if (big != hipSuccess) return big;                                                              \
+        }                                                                                                   \
         conv_lds_mfma_kernel<RV, SV, DV, KV, TV><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS;                 \
     } while (0)
 #define DC_LDS_L(RV, SV, DV, KV)                                                                            \
