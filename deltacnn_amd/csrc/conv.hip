@@ -1170,12 +1170,24 @@ struct PatchRes {  // DCAdd fused behind the convolution: a = residual, b = conv
 // activation the sum is accumulated in `prev` and its activated difference is emitted -- the
 // arithmetic of add_kernel applied to the convolution result rounded to fp16, so the output
 // equals that of the two separate launches bit for bit.
-template <bool TR, int KW, int R, int S, bool ADD, bool K3>
+// MODE 2 (one wavefront holding every output channel of its 16 pixels: KW == 1, one channel
+// block): the activation and truncation of DCActivation applied to the accumulators -- T = trunc
+// + v, S = T + prev, D = act(S) - act(prev), one rounding each, the sequence of act_trunc_pixel;
+// the keep statistics of a pixel are combined over its four k-quarter lanes.
+struct PatchEpi {
+    half_t *prev, *trunc;
+    float thr;
+    int mode, act;
+};
+
+template <bool TR, int KW, int R, int S, int MODE, bool K3>
 __global__ void __launch_bounds__(KW * WAVE)
 conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                        const half_t *__restrict__ bias, half_t *__restrict__ out,
                        const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
-                       int co_blocks, int ci_p, PatchRes rs) {
+                       int co_blocks, int ci_p, PatchRes rs, PatchEpi ep) {
+    constexpr bool ADD = MODE == 1, EPI = MODE == 2;
+    static_assert(!EPI || KW == 1, "the fused activation needs all channels in one wavefront");
     __shared__ float4_t s_red[KW > 1 ? KW * R * WAVE : 1];
     __shared__ int s_src[KW * MFMA_MAX_TAPS * 16];
     const int b = blockIdx.z / co_blocks, cb = blockIdx.z % co_blocks;
@@ -1252,9 +1264,19 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     bits |= __shfl_xor(bits, 32, WAVE);
     const bool upd = bits != 0;
     const bool radd = ADD && inside && rword != 0;
-    if (cb == 0 && kw == 0 && kq == 0 && inside) out_mask[opix] = (upd || radd) ? 1 : 0;
+    // with the fused activation the mask word of an updated pixel is its keep decision, below
+    if (cb == 0 && kw == 0 && kq == 0 && inside && !(EPI && upd)) out_mask[opix] = (upd || radd) ? 1 : 0;
     const bool reduce = ballot(upd) != 0;  // the same in every wavefront of the workgroup
     if (!reduce && ballot(radd) == 0) return;
+    half4_t eq[R], etr[R];  // cached state of the fused activation, requested before the reduction
+    if (EPI) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const size_t off = (upd ? opix : 0) * p.Co + min((cb * R + r) * 16 + kq * 4, p.Co - 4);
+            eq[r] = *reinterpret_cast<const half4_t *>(ep.prev + off);
+            etr[r] = *reinterpret_cast<const half4_t *>(ep.trunc + off);
+        }
+    }
     // operands of the fused sum, requested now so that they arrive during the reduction
     half4_t rv[R], qv[R];
     if (ADD) {
@@ -1301,6 +1323,67 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
             for (int q = 1; q < KW; ++q) sum += s_red[(q * R + r) * WAVE + lane];
             acc[r] = sum;
         }
+    }
+    if (EPI) {
+        const half_t thr = half_t(ep.thr);
+        auto finish = [&](auto act_c) {  // the activation as a compile-time constant
+            constexpr int ACTC = decltype(act_c)::value;
+            half4_t t[R], sm[R], d[R];
+            bool hit = false;
+            float sq = 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int co = (cb * R + r) * 16 + kq * 4;
+                const bool live = upd && cb * R + r < co_tiles && co < p.Co;
+                half4_t bh = half4_t{0, 0, 0, 0};
+                if (bias != nullptr) bh = *reinterpret_cast<const half4_t *>(bias + min(co, p.Co - 4));
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const half_t v = half_t(acc[r][i] + float(bh[i]));
+                    t[r][i] = etr[r][i] + v;
+                    sm[r][i] = t[r][i] + eq[r][i];
+                    d[r][i] = act_apply<half_t>(sm[r][i], ACTC) - act_apply<half_t>(eq[r][i], ACTC);
+                    if (live) {
+                        hit |= tabs(d[r][i]) > thr;
+                        sq += float(d[r][i]) * float(d[r][i]);
+                    }
+                }
+            }
+            bool keep;
+            if (ep.mode == DC_TRUNC_MAX) {
+                const uint64_t bl = ballot(hit);
+                keep = ((bl >> l16) & 0x0001000100010001ull) != 0;
+            } else {
+                sq += __shfl_xor(sq, 16, WAVE);
+                sq += __shfl_xor(sq, 32, WAVE);
+                if (ep.mode == DC_TRUNC_RMS) sq /= float(p.Co);
+                keep = sqrtf(sq) > float(thr);
+            }
+            if (!upd) return;
+            if (kq == 0) out_mask[opix] = keep ? 1 : 0;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int co = (cb * R + r) * 16 + kq * 4;
+                if (cb * R + r >= co_tiles || co >= p.Co) continue;
+                const size_t off = opix * p.Co + co;
+                if (keep) {
+                    *reinterpret_cast<half4_t *>(ep.prev + off) = sm[r];
+                    *reinterpret_cast<half4_t *>(out + off) = d[r];
+                    *reinterpret_cast<half4_t *>(ep.trunc + off) = half4_t{0, 0, 0, 0};
+                } else {
+                    *reinterpret_cast<half4_t *>(ep.trunc + off) = t[r];
+                }
+            }
+        };
+        switch (ep.act) {
+            case DC_ACT_RELU: finish(std::integral_constant<int, DC_ACT_RELU>{}); break;
+            case DC_ACT_RELU6: finish(std::integral_constant<int, DC_ACT_RELU6>{}); break;
+            case DC_ACT_LEAKY: finish(std::integral_constant<int, DC_ACT_LEAKY>{}); break;
+            case DC_ACT_SIGMOID: finish(std::integral_constant<int, DC_ACT_SIGMOID>{}); break;
+            case DC_ACT_SWISH: finish(std::integral_constant<int, DC_ACT_SWISH>{}); break;
+            default: finish(std::integral_constant<int, DC_ACT_LINEAR>{}); break;
+        }
+        return;
     }
     if (!(upd || radd)) return;
     half_t *o = out + opix * p.Co;
@@ -1814,7 +1897,8 @@ bool patch_eligible(const dc_geometry &g, int dtype) {
 
 hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *packed,
                              const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
-                             bool transposed, const Residual *res, hipStream_t s) {
+                             bool transposed, const Residual *res, hipStream_t s,
+                             const ActEpilogue *epi, bool *epilogue_done) {
     ConvP p = make_params(g, DC_F16);
     const int co_tiles = ceil_div(g.out_c, 16);
     const int ci_p = round_up(g.in_c, 32);
@@ -1828,8 +1912,16 @@ hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *p
     if (res != nullptr)
         rs = PatchRes{(const half_t *)res->values, res->mask, (half_t *)res->prev, res->wa, res->wb, res->act};
     const bool k3 = g.kernel_h == 3 && g.kernel_w == 3;
+    // activation + truncation inside the kernel where one wavefront holds all channels of a pixel
+    const auto al8 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 7u) == 0; };
+    const bool fuse = epi != nullptr && epilogue_done != nullptr && res == nullptr && !transposed && kwv == 1 &&
+                      cbk == 1 && epi->mode >= 0 && epi->trunc != nullptr && g.out_c % 4 == 0 && al8(epi->prev) &&
+                      al8(epi->trunc) && al8(out) && (bias == nullptr || al8(bias));
+    if (epilogue_done != nullptr) *epilogue_done = fuse;
+    PatchEpi pe{nullptr, nullptr, 0.f, 0, 0};
+    if (fuse) pe = PatchEpi{(half_t *)epi->prev, (half_t *)epi->trunc, epi->thr, epi->mode, epi->act < 0 ? 0 : epi->act};
     note_kernel("conv_patch_mfma_kernel");
-#define DC_PATCH_ARGS (p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbk, ci_p, rs)
+#define DC_PATCH_ARGS (p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbk, ci_p, rs, pe)
 #define DC_PATCH_L(TRF, KWV, RV, SV, AV)                                                                      \
     do {                                                                                                      \
         if (k3) conv_patch_mfma_kernel<TRF, KWV, RV, SV, AV, true><<<pgrid, KWV * WAVE, 0, s>>> DC_PATCH_ARGS; \
@@ -1841,9 +1933,10 @@ hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *p
         else if (kwv == 4) { if (rv == 2) DC_PATCH_L(TRF, 4, 2, 6, AV); else DC_PATCH_L(TRF, 4, 1, 12, AV); } \
         else { if (rv == 2) DC_PATCH_L(TRF, 8, 2, 6, AV); else DC_PATCH_L(TRF, 8, 1, 12, AV); } \
     } while (0)
-    if (res != nullptr) DC_PATCH(false, true);  // the fused sum exists for plain convolutions only
-    else if (transposed) DC_PATCH(true, false);
-    else DC_PATCH(false, false);
+    if (res != nullptr) DC_PATCH(false, 1);  // the fused sum exists for plain convolutions only
+    else if (transposed) DC_PATCH(true, 0);
+    else if (fuse) { if (rv == 2) DC_PATCH_L(false, 1, 2, 6, 2); else DC_PATCH_L(false, 1, 1, 12, 2); }
+    else DC_PATCH(false, 0);
 #undef DC_PATCH
 #undef DC_PATCH_L
 #undef DC_PATCH_ARGS
@@ -1882,8 +1975,9 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
         const int steps = g.kernel_h * g.kernel_w * (ci_p / 32);
         // Small layers: one 4x4 output patch per workgroup (see conv_patch_mfma_kernel).
         if (patch_eligible(g, dtype)) {
-            hipError_t pe = launch_patch_conv(g, in, packed, bias, out, mask, out_mask, transposed, nullptr, s);
-            if (pe != hipSuccess || epi == nullptr) return pe;
+            bool fused = false;
+            hipError_t pe = launch_patch_conv(g, in, packed, bias, out, mask, out_mask, transposed, nullptr, s, epi, &fused);
+            if (pe != hipSuccess || epi == nullptr || fused) return pe;
             return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
                                             epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
         }

@@ -494,6 +494,10 @@ FUSED = [
     (32, 32, 3, 1, 1, 1, 32, 12, 12),       # depthwise 3x3, epilogue in the kernel
     (64, 64, 3, 2, 1, 1, 64, 13, 13),       # depthwise stride 2
     (24, 24, 5, 1, 2, 1, 24, 12, 12),       # depthwise 5x5 (generic tap loop)
+    (32, 32, 3, 1, 1, 1, 1, 64, 64),        # small 3x3 layer: epilogue in the patch kernel, two tiles per wavefront
+    (32, 24, 3, 1, 1, 1, 1, 64, 62),        # ... partial channel tile, ragged map
+    (16, 16, 3, 1, 1, 1, 1, 24, 24),        # ... one tile per wavefront
+    (32, 32, 3, 2, 1, 1, 1, 64, 64),        # two channel blocks: separate epilogue launch
     (3, 32, 3, 2, 1, 1, 1, 24, 24),         # RGB stem
     (3, 16, 7, 1, 3, 1, 1, 37, 45),         # 7x7 RGB stem
     (3, 64, 3, 2, 1, 1, 1, 40, 41),         # four channel tiles per wavefront
