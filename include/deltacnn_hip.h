@@ -98,7 +98,8 @@ int dc_conv(const dc_geometry *g, const void *input, const void *filter,
             int32_t *out_mask, int dtype, void *stream);
 
 /* Conv + activation/truncation in one call: dc_conv followed by dc_activate_truncate on the
- * conv output.  Depthwise, few-input-channel and large-map pointwise shapes run as ONE launch
+ * conv output.  Depthwise, few-input-channel, mid-size pointwise and small KxK shapes of up
+ * to 32 output channels run as ONE launch
  * (the epilogue works on the accumulators, the conv output never travels through memory);
  * every other shape runs the two kernels back to back inside the call.  No counterpart in
  * the reference (it launches the two kernels separately, sparse_layers.py:636-638); results
