@@ -168,6 +168,9 @@ hipError_t launch_activate_truncate(void *delta, void *prev, void *trunc, int32_
 hipError_t launch_add(const void *a, const void *b, void *prev, void *out, const int32_t *ma,
                       const int32_t *mb, int32_t *mo, float wa, float wb, int act, int dense_out,
                       int32_t P, int32_t C, int dtype, hipStream_t s);
+hipError_t launch_add_upsampled(const void *a, const void *b, void *prev, void *out, const int32_t *ma,
+                                const int32_t *mb, int32_t *mo, float wa, float wb, int act, int32_t B,
+                                int32_t H, int32_t W, int32_t C, int32_t scale, int dtype, hipStream_t s);
 hipError_t launch_add_to_dense(void *a, void *b, const int32_t *ma, int act, int32_t P, int32_t C,
                                int dtype, hipStream_t s);
 hipError_t launch_upsample(const void *in, void *out, const int32_t *mi, int32_t *mo, int32_t B,

@@ -326,6 +326,37 @@ int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_
                                  (hipStream_t)stream), "dc_add");
 }
 
+int dc_add_upsampled(const void *a, const void *b, void *prev_out, void *out, const int32_t *mask_a,
+                     const int32_t *mask_b, int32_t *mask_out, float weight_a, float weight_b,
+                     int activation, int32_t batch, int32_t height, int32_t width, int32_t channels,
+                     int32_t scale, int dtype, void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_add_upsampled");
+    if (batch <= 0 || height <= 0 || width <= 0 || scale <= 0)
+        return fail(DC_ERR_SHAPE, "dc_add_upsampled: batch, height, width and scale must be positive");
+    if (height % scale != 0 || width % scale != 0)
+        return fail(DC_ERR_SHAPE, "dc_add_upsampled: %d x %d is not a multiple of scale %d", height, width, scale);
+    if ((int64_t)batch * height * width > INT32_MAX)
+        return fail(DC_ERR_SHAPE, "dc_add_upsampled: more than 2^31 pixels");
+    int rc = check_pc("dc_add_upsampled", batch * height * width, channels);
+    if (rc != DC_OK) return rc;
+    if (activation > DC_ACT_SWISH) return fail(DC_ERR_UNSUPPORTED, "dc_add_upsampled: activation id %d", activation);
+    DC_REQUIRE_PTR("dc_add_upsampled", a);
+    DC_REQUIRE_PTR("dc_add_upsampled", b);
+    DC_REQUIRE_PTR("dc_add_upsampled", out);
+    DC_REQUIRE_PTR("dc_add_upsampled", mask_a);
+    DC_REQUIRE_PTR("dc_add_upsampled", mask_b);
+    DC_REQUIRE_PTR("dc_add_upsampled", mask_out);
+    if (activation > 0) DC_REQUIRE_PTR("dc_add_upsampled", prev_out);
+    DC_REQUIRE_ALIGNED("dc_add_upsampled", a, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_add_upsampled", b, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_add_upsampled", out, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_add_upsampled", prev_out, esize(dtype));
+    return finish(dc::launch_add_upsampled(a, b, prev_out, out, mask_a, mask_b, mask_out, weight_a, weight_b,
+                                           activation, batch, height, width, channels, scale, dtype,
+                                           (hipStream_t)stream), "dc_add_upsampled");
+}
+
 int dc_densify(const void *delta, void *prev_out, void *out, const int32_t *mask, int32_t pixels,
                int32_t channels, int dtype, void *stream) {
     dc::kernel_log_reset();

@@ -324,6 +324,55 @@ add_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ pre
     }
 }
 
+// add_kernel whose second operand lives on a map S times smaller in both directions and is
+// read through nearest upsampling: pixel (y, x) takes b and its mask word at (y / S, x / S).
+// The upsampled tensor never exists in memory.
+template <typename T, int N>
+__global__ void __launch_bounds__(256)
+add_up_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ prev,
+              T *__restrict__ out, const int32_t *__restrict__ ma, const int32_t *__restrict__ mb,
+              int32_t *__restrict__ mo, float wa_f, float wb_f, int act, int B, int H, int W, int C,
+              int S, int lg) {
+    const T wa = T(wa_f), wb = T(wb_f);
+    const int G = 1 << lg, P = B * H * W;
+    int p, gl;
+    group_coords(lg, p, gl);
+    if (p >= P) return;
+    const int row = p / W, x = p - row * W;  // row = image * H + y
+    const int img = row / H, y = row - img * H;
+    const size_t pb = ((size_t)img * (H / S) + y / S) * (W / S) + x / S;
+    const bool aa = ma[p] != 0, ab = mb[pb] != 0;
+    if (gl == 0) mo[p] = (aa || ab) ? 1 : 0;
+    if (!(aa || ab)) return;
+    for (int c = gl * N; c < C; c += G * N) {
+        const size_t off = (size_t)p * C + c;
+        Vec<T, N> s;
+#pragma unroll
+        for (int j = 0; j < N; ++j) s.v[j] = T(0);
+        if (aa) {
+            Vec<T, N> va = vload<T, N>(a + off);
+#pragma unroll
+            for (int j = 0; j < N; ++j) s.v[j] = va.v[j] * wa;
+        }
+        if (ab) {
+            Vec<T, N> vb = vload<T, N>(b + pb * C + c);
+#pragma unroll
+            for (int j = 0; j < N; ++j) s.v[j] = fma_t(vb.v[j], wb, s.v[j]);
+        }
+        if (act > 0) {
+            Vec<T, N> q = vload<T, N>(prev + off);
+            Vec<T, N> n;
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                n.v[j] = s.v[j] + q.v[j];
+                s.v[j] = act_apply<T>(n.v[j], act) - act_apply<T>(q.v[j], act);
+            }
+            vstore<T, N>(prev + off, n);
+        }
+        vstore<T, N>(out + off, s);
+    }
+}
+
 // add_kernel for large maps: mask scan and compaction per wavefront (see act_trunc_scan_kernel).
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
@@ -925,6 +974,31 @@ hipError_t launch_densify(const void *delta, void *prev, void *out, const int32_
                           int dtype, hipStream_t s) {
     if (dtype == DC_F32) return densify_t<float>((const float *)delta, (float *)prev, (float *)out, mask, P, C, s);
     return densify_t<half_t>((const half_t *)delta, (half_t *)prev, (half_t *)out, mask, P, C, s);
+}
+
+namespace {
+template <typename T>
+hipError_t add_up_t(const T *a, const T *b, T *prev, T *out, const int32_t *ma, const int32_t *mb,
+                    int32_t *mo, float wa, float wb, int act, int B, int H, int W, int C, int S,
+                    hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    if (act < 0) act = 0;
+    const int P = B * H * W;
+    const bool vec = can_vec<T>(C, {a, b, prev, out});
+    GroupLaunch L(P, vec ? pick_group(C / N, P, 4) : group_lanes(C, 1));
+    note_kernel("add_up_kernel");
+    if (vec) add_up_kernel<T, N><<<L.grid, L.block, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, B, H, W, C, S, L.lg);
+    else add_up_kernel<T, 1><<<L.grid, L.block, 0, s>>>(a, b, prev, out, ma, mb, mo, wa, wb, act, B, H, W, C, S, L.lg);
+    return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_add_upsampled(const void *a, const void *b, void *prev, void *out, const int32_t *ma,
+                                const int32_t *mb, int32_t *mo, float wa, float wb, int act, int32_t B,
+                                int32_t H, int32_t W, int32_t C, int32_t scale, int dtype, hipStream_t s) {
+    if (dtype == DC_F32)
+        return add_up_t<float>((const float *)a, (const float *)b, (float *)prev, (float *)out, ma, mb, mo, wa, wb, act, B, H, W, C, scale, s);
+    return add_up_t<half_t>((const half_t *)a, (const half_t *)b, (half_t *)prev, (half_t *)out, ma, mb, mo, wa, wb, act, B, H, W, C, scale, s);
 }
 
 hipError_t launch_add(const void *a, const void *b, void *prev, void *out, const int32_t *ma,

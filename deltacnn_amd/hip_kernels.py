@@ -305,6 +305,24 @@ def sparse_add_tensors(a, b, prev_out, out, mask_a, mask_b, mask_out, weight_a, 
           dense_out=bool(dense_out))
 
 
+def sparse_add_upsampled(a, b, prev_out, out, mask_a, mask_b, mask_out, weight_a, weight_b, activation, scale):
+    """``sparse_add_tensors(a, sparse_upsample(b, scale))`` without the upsampled tensor
+    (cuda_kernels.py:132-141 after :152-167): b and mask_b are `scale` times smaller."""
+    lib = _lib.load()
+    _nhwc(a, "a")
+    _nhwc(b, "b")
+    bt, c, h, w = a.shape
+    scale = int(scale)
+    if tuple(b.shape) != (bt, c, h // scale, w // scale) or h % scale or w % scale:
+        raise _lib.DeltaCNNError(-2, f"sparse_add_upsampled: {tuple(b.shape)} x{scale} does not give {tuple(a.shape)}")
+    _call("add", lib.dc_add_upsampled,
+          (a.data_ptr(), b.data_ptr(), _ptr(prev_out), out.data_ptr(), _mask(mask_a, "mask_a").data_ptr(),
+           _mask(mask_b, "mask_b").data_ptr(), mask_out.data_ptr(), float(weight_a), float(weight_b),
+           int(activation), bt, h, w, c, scale, _dtype(a), _stream()),
+          P=_pixels(a), C=c, esize=a.element_size(), in_mask=mask_a, in_mask_b=mask_b, out_mask=mask_out,
+          with_prev=prev_out is not None, dense_out=False, b_scale=scale)
+
+
 def sparse_add_to_dense_tensor(a, b, mask_a, activation=0):
     """cuda_kernels.py:144-145: ``b[px] += a[px]`` on active pixels."""
     lib = _lib.load()

@@ -355,7 +355,12 @@ class _HRModule(nn.Module):
         for row, adds in zip(self.fuse, self.adds):
             y = row[0](xs[0])
             for j in range(1, len(xs)):
-                y = adds[j - 1](y, row[j](xs[j]))
+                add, branch = adds[j - 1], row[j]
+                if j > len(outs) and hasattr(add, "after_upsample"):
+                    # 1x1 convolution + upsampling: the upsampling is folded into the sum
+                    y = add.after_upsample(y, branch[0](xs[j]), branch[1])
+                else:
+                    y = add(y, branch(xs[j]))
             outs.append(y)
         return outs
 

@@ -442,6 +442,25 @@ class DCAdd(DCModule):
                     return res
         return self(a, conv(conv_input))
 
+    def after_upsample(self, a, b, upsample):
+        """``self(a, upsample(b))`` with the nearest upsampling folded into the addition's kernel
+        (the upsampled tensor is never stored) when both operands are delta tensors and this
+        layer has no dense_out; otherwise exactly the two separate layer calls."""
+        fusable = (DCAdd.fuse_into_conv and type(a) != Tensor and type(b) != Tensor and not self.first_iter
+                   and not self.dense_out and isinstance(upsample, DCUpsamplingNearest2d))
+        if not fusable:
+            return self(a, upsample(b))
+        val_a, mask_a = a
+        val_b, mask_b = b
+        if self.out is None or self.out.shape != val_a.shape or self.out.dtype != val_a.dtype:
+            self.out = torch.empty_like(val_a)
+        if self.mask_out is None or self.mask_out.shape != mask_a.shape:
+            self.mask_out = torch.empty_like(mask_a)
+        hk.sparse_add_upsampled(val_a, val_b, self.prev_out if self.activation is not None else None, self.out,
+                                mask_a, mask_b, self.mask_out, self.weight_a, self.weight_b,
+                                self.activation_int if self.activation is not None else 0, upsample.scale_factor)
+        return self.out, self.mask_out
+
     def reset(self):
         super().reset()
         self.idx = -1

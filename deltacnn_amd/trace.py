@@ -201,9 +201,10 @@ class Tracer:
                 elif op == "add":
                     n_o = n_out if n_out is not None else P
                     ext = n_o * C * s if meta["with_prev"] else 0
-                    rd = 2 * P * m + (n_in + n_in_b) * C * s + ext
+                    bs = meta.get("b_scale", 1) ** 2  # second operand read from a smaller map
+                    rd = (P + P // bs) * m + (n_in + n_in_b) * C * s + ext
                     wr = n_o * C * s + ext + P * m
-                    dens = ((n_in + n_in_b) / (2 * P), n_o / P)
+                    dens = ((n_in + n_in_b * bs) / (2 * P), n_o / P)
                 elif op == "add_to_dense":
                     rd, wr = P * m + 2 * n_in * C * s, n_in * C * s
                     dens = (n_in / P, n_in / P)

@@ -163,6 +163,17 @@ int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_
            int activation, int dense_out, int32_t pixels, int32_t channels, int dtype,
            void *stream);
 
+/* dc_add whose operand b lives on a map `scale` times smaller in both directions and enters
+ * through nearest upsampling: out(y, x) = weight_a * a(y, x) + weight_b * b(y / scale, x / scale),
+ * mask_out = mask_a | upsampled mask_b.  height and width are those of a and out and must be
+ * multiples of scale; no dense_out form.  No counterpart in the reference, which runs
+ * sparse_upsample_wrapper (conv_torch_wrapper.cpp:484-513) and sparse_add_tensors_wrapper
+ * (:387-444) one after the other; results are identical, the upsampled tensor is never stored. */
+int dc_add_upsampled(const void *a, const void *b, void *prev_out, void *out, const int32_t *mask_a,
+                     const int32_t *mask_b, int32_t *mask_out, float weight_a, float weight_b,
+                     int activation, int32_t batch, int32_t height, int32_t width, int32_t channels,
+                     int32_t scale, int dtype, void *stream);
+
 /* DCDensify in one launch (sparse_layers.py:1287-1329): prev_out += delta on active pixels,
  * then out = prev_out for EVERY pixel (the dense clone of :1324-1325).  No counterpart in the
  * reference, which runs deltacnn_activate_truncate(..., truncation_mode -1) and a torch clone;

@@ -850,6 +850,33 @@ def test_upsample(lib, dtype, C, scale):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [5, 32, 72])
+@pytest.mark.parametrize("scale", [2, 4])
+@pytest.mark.parametrize("act", [-1, 1])
+def test_add_upsampled(lib, dtype, C, scale, act):
+    """dc_add_upsampled == DCAdd(a, DCUpsamplingNearest2d(b)) of the oracle, bit for bit."""
+    g = _gen(1250 + C + scale)
+    B, h, w = 2, 5, 7
+    H, W = h * scale, w * scale
+    ma, mb = rand_mask(g, B, H, W, 0.3), rand_mask(g, B, h, w, 0.4)
+    a = torch.randn(B, C, H, W, generator=g).to(dtype)
+    b = torch.randn(B, C, h, w, generator=g).to(dtype)
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype) if act > 0 else None
+    up, up_mask = ops.upsample(b, mb, scale)
+    w_prev = prev.clone() if act > 0 else None
+    want, want_mask = ops.add(a, ma, up, up_mask, w_prev, 0.75, -0.5, act, False)
+    d_prev = cl(prev) if act > 0 else None
+    d_out = torch.full((B, C, H, W), float("nan"), dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+    d_mo = torch.full((B, 1, H, W), -3, dtype=torch.int32, device=DEV)
+    hk().sparse_add_upsampled(cl(poison(a, ma)), cl(poison(b, mb)), d_prev, d_out, cl(ma), cl(mb), d_mo,
+                              0.75, -0.5, act, scale)
+    assert torch.equal(d_mo.cpu(), want_mask)
+    assert_masked_equal(d_out, want, want_mask, "out")
+    if act > 0:
+        assert torch.equal(d_prev.cpu(), w_prev)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("Ca,Cb", [(3, 5), (16, 32), (64, 24), (8, 3)])
 def test_concat(lib, dtype, Ca, Cb):
     g = _gen(1300 + Ca)
