@@ -1189,7 +1189,8 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     constexpr bool ADD = MODE == 1, EPI = MODE == 2;
     static_assert(!EPI || KW == 1, "the fused activation needs all channels in one wavefront");
     __shared__ float4_t s_red[KW > 1 ? KW * R * WAVE : 1];
-    __shared__ int s_src[KW * MFMA_MAX_TAPS * 16];
+    constexpr int TAB_TAPS = MFMA_MAX_TAPS + 12;  // a pass writes up to 11 surplus taps
+    __shared__ int s_src[KW * TAB_TAPS * 16];
     const int b = blockIdx.z / co_blocks, cb = blockIdx.z % co_blocks;
     const int kw = wave_id(), lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;
@@ -1211,22 +1212,22 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     // the lane's output pixel through `tap`, or -1 if it is out of bounds.  The four k-quarter
     // lanes of a pixel share the taps (kq, kq + 4, ...), each also fetches the mask word of its
     // taps; the activity bits are then combined across the four lanes.
-    int *src_tab = s_src + kw * (MFMA_MAX_TAPS * 16);
+    int *src_tab = s_src + kw * (TAB_TAPS * 16);
     unsigned long long bits = 0;
     for (int t0 = 0; t0 < K2; t0 += 12) {
         int word[3], src[3];
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
+            // straight-line (selects instead of branches): the three mask words of a lane are
+            // requested back to back; the table has room for the surplus taps of the last pass
             const int tap = t0 + kq + 4 * j;
-            src[j] = -1;
-            if (tap < K2) {
-                const int ky = tap / Kw, kx = tap - ky * Kw;
-                int iy = 0, ix = 0;
-                if (inside && tap_src<TR>(oy, ky, p.sh, p.dh, p.pt, p.Hi, iy) &&
-                    tap_src<TR>(ox, kx, p.sw, p.dw, p.pl, p.Wi, ix))
-                    src[j] = iy * p.Wi + ix;
-                src_tab[tap * 16 + l16] = src[j];
-            }
+            const int tc = min(tap, K2 - 1);
+            const int ky = tc / Kw, kx = tc - ky * Kw;
+            int iy = 0, ix = 0;
+            const bool oky = tap_src<TR>(oy, ky, p.sh, p.dh, p.pt, p.Hi, iy);
+            const bool okx = tap_src<TR>(ox, kx, p.sw, p.dw, p.pl, p.Wi, ix);
+            src[j] = (tap < K2 && inside && oky && okx) ? iy * p.Wi + ix : -1;
+            src_tab[tap * 16 + l16] = src[j];
             word[j] = mb[max(src[j], 0)];
         }
 #pragma unroll
