@@ -83,6 +83,12 @@ def test_bad_arguments_are_rejected_before_any_launch(lib):
     g = _geom(in_h=6, in_w=6, out_h=1, out_w=1, kernel_h=8, kernel_w=8)
     assert lib.dc_pool(ctypes.byref(g), p, p, p, p, p, 1, 1, 1, None) == -3
     assert lib.dc_densify(p, p, None, p, 16, 4, 0, None) == -4
+    # the sum with an upsampled operand: sizes must be multiples of the scale
+    assert lib.dc_add_upsampled(p, p, None, p, p, p, p, 1.0, 1.0, 0, 1, 6, 8, 4, 4, 0, None) == -2
+    assert b"multiple of scale" in lib.dc_last_error()
+    assert lib.dc_add_upsampled(p, p, None, p, p, p, p, 1.0, 1.0, 0, 1, 8, 8, 4, 0, 0, None) == -2
+    assert lib.dc_add_upsampled(p, p, None, p, p, p, p, 1.0, 1.0, 1, 1, 8, 8, 4, 2, 0, None) == -4   # activation needs prev_out
+    assert lib.dc_add_upsampled(p, p, None, p, p, p, None, 1.0, 1.0, 0, 1, 8, 8, 4, 2, 0, None) == -4
 
 
 def test_packed_filter_size_is_host_arithmetic(lib):
