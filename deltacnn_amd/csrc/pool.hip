@@ -3,6 +3,9 @@
 //   avg: out = sum_w M*delta / (Kh*Kw)
 // Arithmetic is fp32 for both tensor types with one rounding on store.
 //
+// pool_pixel_kernel   2x2 / 3x3 windows on small and mid-size maps: a lane group per output
+//                     pixel, everything requested at once
+// pool_scan_kernel    2x2 / 3x3 windows on very large maps: mask scan and compaction per wavefront
 // pool_window_kernel  8x8 output tile per workgroup, mask dilation + compaction as for the
 //                     convolutions; each compacted pixel is then handled by a group of G lanes
 //                     that run along the channels with 16-byte vectors
@@ -263,6 +266,105 @@ pool_scan_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restrict
     }
 }
 
+// The K x K window kernel for maps that give pool_window_kernel too few tiles to fill the chip:
+// one group of G lanes per OUTPUT pixel; every lane requests the window's mask words, the deltas
+// and (for the maximum) the cached inputs of all taps at once from clamped addresses and selects
+// afterwards -- one memory round trip, no workgroup barrier, no serial walk over a tile's pixels.
+// Same operations in the same order as pool_window_kernel.
+template <typename T, int N, bool MAX, int K>
+__global__ void __launch_bounds__(256)
+pool_pixel_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restrict__ prev,
+                  T *__restrict__ out, const int32_t *__restrict__ mask,
+                  int32_t *__restrict__ out_mask, int lg) {
+    constexpr int KK = K * K;
+    const int Po = p.B * p.Ho * p.Wo, C = p.Ci;
+    const int G = 1 << lg;
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int po = gid >> lg, gl = gid & (G - 1);
+    if (po >= Po) return;
+    const int row = po / p.Wo, ox = po - row * p.Wo;
+    const int b = row / p.Ho, oy = row - b * p.Ho;
+    const size_t base = (size_t)b * p.Hi * p.Wi;
+    size_t ip[KK];
+    int mw[KK];
+    bool inside[KK];
+#pragma unroll
+    for (int t = 0; t < KK; ++t) {
+        const int iy = oy * p.sh - p.pt + (t / K) * p.dh, ix = ox * p.sw - p.pl + (t % K) * p.dw;
+        inside[t] = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
+        ip[t] = base + (size_t)min(max(iy, 0), p.Hi - 1) * p.Wi + min(max(ix, 0), p.Wi - 1);
+        mw[t] = mask[ip[t]];
+    }
+    for (int c0 = gl * N; c0 < C; c0 += G * N) {  // one pass unless C > 64 vectors
+        Vec<T, N> pd[KK], pp[KK];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) {
+            pd[t] = vload<T, N>(in + ip[t] * C + c0);
+            if (MAX) pp[t] = vload<T, N>(prev + ip[t] * C + c0);
+        }
+        int taps = 0;
+#pragma unroll
+        for (int t = 0; t < KK; ++t) taps |= (inside[t] && mw[t] != 0) ? 1 << t : 0;
+        if (c0 == gl * N && gl == 0) out_mask[po] = taps != 0 ? 1 : 0;
+        if (taps == 0) return;  // the same for every lane of the group
+        float hi[N], hp[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            hi[j] = MAX ? -INFINITY : 0.f;
+            hp[j] = -INFINITY;
+        }
+#pragma unroll
+        for (int ky = 0; ky < K; ++ky) {
+            const int iy = oy * p.sh - p.pt + ky * p.dh;
+            if (iy < 0) continue;
+            if (iy >= p.Hi) {
+                if (MAX && q.zero_bottom && iy < p.Hi + q.pb) {
+#pragma unroll
+                    for (int j = 0; j < N; ++j) {
+                        hi[j] = fmaxf(hi[j], 0.f);
+                        hp[j] = fmaxf(hp[j], 0.f);
+                    }
+                }
+                continue;
+            }
+#pragma unroll
+            for (int kx = 0; kx < K; ++kx) {
+                const int ix = ox * p.sw - p.pl + kx * p.dw;
+                if (ix < 0) continue;
+                if (ix >= p.Wi) {
+                    if (MAX && q.zero_right && ix < p.Wi + q.pr) {
+#pragma unroll
+                        for (int j = 0; j < N; ++j) {
+                            hi[j] = fmaxf(hi[j], 0.f);
+                            hp[j] = fmaxf(hp[j], 0.f);
+                        }
+                    }
+                    continue;
+                }
+                const int t = ky * K + kx;
+                const bool act = (taps >> t) & 1;
+                if (!MAX && !act) continue;
+#pragma unroll
+                for (int j = 0; j < N; ++j) {
+                    const float d = act ? float(pd[t].v[j]) : 0.f;
+                    if (MAX) {
+                        const float pf = float(pp[t].v[j]);
+                        hi[j] = fmaxf(hi[j], d + pf);
+                        hp[j] = fmaxf(hp[j], pf);
+                    } else {
+                        hi[j] += d;
+                    }
+                }
+            }
+        }
+        Vec<T, N> r;
+        const float area = float(K * K);
+#pragma unroll
+        for (int j = 0; j < N; ++j) r.v[j] = MAX ? T(hi[j] - hp[j]) : T(hi[j] / area);
+        vstore<T, N>(out + (size_t)po * C + c0, r);
+    }
+}
+
 // 1x1 output: grid (channel slices, batch); a workgroup's 4 wavefronts stride over the window
 // taps, each lane owns one channel, partial results meet in LDS.
 template <typename T, bool MAX>
@@ -449,6 +551,21 @@ hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, c
         if (mode == DC_POOL_MAX) { if (ksq == 2) DC_PS(true, 2); else DC_PS(true, 3); }
         else { if (ksq == 2) DC_PS(false, 2); else DC_PS(false, 3); }
 #undef DC_PS
+        return hipGetLastError();
+    }
+    // small and mid-size maps: a lane group per output pixel, one memory round trip (measured
+    // against the tile kernel, whose few workgroups walk their pixels one after the other)
+    if (ksq > 0 && vec && po * G <= (1 << 20) && (int64_t)g.batch * g.in_h * g.in_w < (1ll << 31)) {
+        note_kernel("pool_pixel_kernel");
+        const int64_t lanes = po * G;
+        const int block = lanes <= 2048 * WAVE ? WAVE : 256;
+        const dim3 pgrid((unsigned)ceil_div64(lanes, block));
+        int lg = 0;
+        while ((1 << lg) < G) ++lg;
+#define DC_PP(MX, KV) pool_pixel_kernel<T, N, MX, KV><<<pgrid, block, 0, s>>>(p, q, in, prev, (T *)out, mask, out_mask, lg)
+        if (mode == DC_POOL_MAX) { if (ksq == 2) DC_PP(true, 2); else DC_PP(true, 3); }
+        else { if (ksq == 2) DC_PP(false, 2); else DC_PP(false, 3); }
+#undef DC_PP
         return hipGetLastError();
     }
     note_kernel("pool_window_kernel");
