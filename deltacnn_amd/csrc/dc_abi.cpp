@@ -209,10 +209,10 @@ int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filt
     if (rc != DC_OK) return rc;
     if (activation < 0 || activation > DC_ACT_SWISH)
         return fail(DC_ERR_UNSUPPORTED, "dc_conv_add: activation %d", activation);
-    const bool pointwise = activation == 0 && dc::pointwise_eligible(*g, dtype);
+    const bool pointwise = dc::pointwise_eligible(*g, dtype);
     if (!pointwise && !dc::patch_eligible(*g, dtype))
         return fail(DC_ERR_UNSUPPORTED, "dc_conv_add: only fp16 1x1 stride-1 convolutions with "
-                                        "Cin %% 8 == 0 and Cout %% 4 == 0 (no activation) and small "
+                                        "Cin %% 8 == 0 and Cout %% 4 == 0 and small "
                                         "fp16 layers with Cin %% 8 == 0 have the fused form");
     DC_REQUIRE_PTR("dc_conv_add", input);
     DC_REQUIRE_PTR("dc_conv_add", packed_filter);

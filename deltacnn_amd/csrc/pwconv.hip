@@ -45,6 +45,8 @@ struct ResP {
     const half_t *res;
     const int32_t *mask;
     float wa, wb;
+    half_t *prev;  // MODE 2: the sum is accumulated here and its activated difference is emitted
+    int act;
 };
 
 // A workgroup takes 64 consecutive pixels (4 pixel tiles of 16) x CBW * R channel tiles of 16.
@@ -59,12 +61,14 @@ struct ResP {
 // fragments are then shared by R channel tiles instead of being fetched again by other
 // workgroups).  S = reduction steps per memory round trip: all fragment loads of S steps are in
 // flight together.
-template <int KW, int CBW, int NBW, int R, int NTW, int S, bool ADD, bool EAGER>
+// MODE: 0 convolution only, 1 fused sum, 2 fused sum with the DCAdd layer's activation.
+template <int KW, int CBW, int NBW, int R, int NTW, int S, int MODE, bool EAGER>
 __global__ void __launch_bounds__(KW * CBW * NBW * WAVE)
 pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
                const half_t *__restrict__ bias, half_t *__restrict__ out,
                const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, ResP rp) {
     static_assert(NBW * NTW <= 4, "a workgroup covers at most 64 pixels");
+    constexpr bool ADD = MODE > 0, ADDACT = MODE == 2;
     constexpr int NW = KW * CBW * NBW, TILES = R * NTW, FT = (TILES + KW - 1) / KW;
     constexpr int PXW = NBW * NTW * 16;  // pixels per workgroup
     __shared__ float4_t s_red[KW > 1 ? NW * TILES * WAVE : 1];
@@ -125,7 +129,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
 
     // tiles this wavefront finishes: all of its own (KW == 1) or tiles kw, kw + KW, ... of
     // its group after the reduction
-    half4_t res[FT], bh[FT];
+    half4_t res[FT], bh[FT], qv[FT];
 #pragma unroll
     for (int m = 0; m < FT; ++m) {
         const int t = KW > 1 ? kw + m * KW : m;
@@ -137,6 +141,10 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
             const int bit = (nw * NTW + j) * 16 + l16;
             const bool on_r = t < TILES && ((br >> bit) & 1);
             res[m] = *reinterpret_cast<const half4_t *>(rp.res + (size_t)(on_r ? pbase + bit : 0) * p.Co + co);
+            if (ADDACT) {
+                const bool on_o = t < TILES && ((bo >> bit) & 1);
+                qv[m] = *reinterpret_cast<const half4_t *>(rp.prev + (size_t)(on_o ? pbase + bit : 0) * p.Co + co);
+            }
         }
     }
 
@@ -227,13 +235,19 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
         if (!(on || on_r)) continue;
         const float4_t v = fin[m] + float4_t{float(bh[m][0]), float(bh[m][1]), float(bh[m][2]), float(bh[m][3])};
         half4_t o = half4_t{half_t(v[0]), half_t(v[1]), half_t(v[2]), half_t(v[3])};
-        if (ADD) {
+        if (ADD) {  // add_kernel's sequence: s = a * wa; s = fma(b, wb, s); n = s + prev; ...
+            half4_t qn;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 half_t sum = on_r ? half_t(res[m][i] * wa) : half_t(0);
                 if (on) sum = fma_t(o[i], wb, sum);
+                if (ADDACT) {
+                    qn[i] = sum + qv[m][i];
+                    sum = act_apply<half_t>(qn[i], rp.act) - act_apply<half_t>(qv[m][i], rp.act);
+                }
                 o[i] = sum;
             }
+            if (ADDACT) *reinterpret_cast<half4_t *>(rp.prev + (size_t)(pbase + bit) * p.Co + co) = qn;
         }
         *reinterpret_cast<half4_t *>(out + (size_t)(pbase + bit) * p.Co + co) = o;
     }
@@ -533,8 +547,8 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
         if (ctw == 5) DC_GO(16, 5);
 #undef DC_GO
     }
-    ResP rp{nullptr, nullptr, 1.f, 1.f};
-    if (res != nullptr) rp = ResP{(const half_t *)res->values, res->mask, res->wa, res->wb};
+    ResP rp{nullptr, nullptr, 1.f, 1.f, nullptr, 0};
+    if (res != nullptr) rp = ResP{(const half_t *)res->values, res->mask, res->wa, res->wb, (half_t *)res->prev, res->act};
     const int cfg = pick_config(p, ksteps);
     note_kernel("pw_mfma_kernel");
 #define DC_PW_S(KW, CBW, NBW, R, NTW, EA, SS)                                                        \
@@ -544,11 +558,14 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
         /* filter bytes dominate and the plain order would spread a channel group over XCDs */      \
         p.xcd = (p.nx % 8 != 0 && p.ny > 1 && (int64_t)p.ci_p * p.Co > (int64_t)p.P * p.Ci) ? 1 : 0; \
         dim3 grid(p.xcd ? p.nx * ((p.ny + 7) / 8 * 8) : p.nx, p.xcd ? 1 : p.ny);                     \
-        if (res != nullptr)                                                                          \
-            pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, true, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(  \
+        if (res != nullptr && res->act > 0)                                                          \
+            pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, 2, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
+                p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
+        else if (res != nullptr)                                                                     \
+            pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, 1, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
                 p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
         else                                                                                         \
-            pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, false, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>( \
+            pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, 0, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
                 p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
     } while (0)
 #define DC_PW(ID, KW, CBW, NBW, R, NTW, EA)                                                          \

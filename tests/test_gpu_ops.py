@@ -575,7 +575,10 @@ def test_conv_add_fused(lib, cfg, weights):
 
 @pytest.mark.parametrize("cfg", [(32, 32, 3, 1, 1, 1, 1, 16, 16), (64, 64, 3, 1, 1, 1, 1, 12, 13),
                                  (128, 128, 3, 1, 1, 1, 1, 8, 8), (24, 20, 3, 2, 1, 1, 1, 17, 19),
-                                 (16, 18, 5, 1, 2, 1, 1, 9, 9), (48, 32, 1, 1, 0, 1, 1, 10, 10)],
+                                 (16, 18, 5, 1, 2, 1, 1, 9, 9), (48, 32, 1, 1, 0, 1, 1, 10, 10),
+                                 # pointwise arrangements: 64x64 tiles, reduction split over 4 and 8 wavefronts
+                                 (64, 256, 1, 1, 0, 1, 1, 64, 64), (576, 96, 1, 1, 0, 1, 1, 14, 14),
+                                 (960, 160, 1, 1, 0, 1, 1, 7, 7)],
                          ids=lambda c: "-".join(str(v) for v in c))
 @pytest.mark.parametrize("act", [0, 1, 3])
 @pytest.mark.parametrize("weights", [(1.0, 1.0), (0.5, -1.5)])
