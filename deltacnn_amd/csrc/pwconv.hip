@@ -509,7 +509,7 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     *epilogue_done = false;
     const auto al8 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 7u) == 0; };
     // Fused epilogue: a workgroup owns all output channels of its 16 pixels (up to 16
-    // wavefronts x 5 channel tiles), so it takes the keep / drop decision itself.  Only for maps
+    // wavefronts x 2 channel tiles), so it takes the keep / drop decision itself.  Only for maps
     // of at least 512 pixels: a smaller map gives too few workgroups, the whole filter then
     // streams through a handful of compute units and the two-launch form (channel tiles spread
     // over many workgroups) is faster.
@@ -522,7 +522,9 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     // fused kernel at a quarter of the bandwidth the separate activation kernel reaches).
     const bool large = ((int64_t)ceil_div(p.P, 16) * p.co_tiles >= 4096 && ksteps >= 2) ||
                        (int64_t)p.P * p.Co * 2 > (4 << 20);
-    if (fusable && ksteps <= PW_FUSED_MAX_STEPS && p.P >= 512 && !large) {
+    // ... nor for filters beyond 32 KB, which every 16-pixel workgroup would stream in full
+    const bool small_filter = (int64_t)p.ci_p * p.Co * 2 <= (32 << 10);
+    if (fusable && ksteps <= PW_FUSED_MAX_STEPS && p.P >= 512 && !large && small_filter) {
         dim3 grid(ceil_div(p.P, 16));
         const int act = epi->act < 0 ? 0 : epi->act;
         note_kernel("pw_act_mfma_kernel");
@@ -541,10 +543,7 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
         if (nw == 4) DC_GO(4, 1);
         if (nw == 8) DC_GO(8, 1);
         if (ctw == 1) DC_GO(16, 1);
-        if (ctw == 2) DC_GO(16, 2);
-        if (ctw == 3) DC_GO(16, 3);
-        if (ctw == 4) DC_GO(16, 4);
-        if (ctw == 5) DC_GO(16, 5);
+        if (ctw == 2) DC_GO(16, 2);  // 32 KB of filter: at most 32 channel tiles
 #undef DC_GO
     }
     ResP rp{nullptr, nullptr, 1.f, 1.f, nullptr, 0};

@@ -484,12 +484,14 @@ FUSED = [
     (16, 96, 1, 1, 0, 1, 1, 40, 40),        # pointwise, epilogue in the kernel: 2 tiles/wave, 1 step
     (64, 192, 1, 1, 0, 1, 1, 40, 40),       # 3 tiles/wave, 2 steps
     (32, 384, 1, 1, 0, 1, 1, 40, 40),       # 6 tiles/wave, 1 step
-    (64, 512, 1, 1, 0, 1, 1, 40, 40),       # 8 tiles/wave, 2 steps
+    (64, 512, 1, 1, 0, 1, 1, 40, 40),       # a filter too large for the fused kernel: two launches
+    (32, 512, 1, 1, 0, 1, 1, 40, 40),       # 2 tiles/wave on 16 wavefronts
     (24, 40, 1, 1, 0, 1, 1, 40, 40),        # partial channel tile and partial reduction step
-    (64, 384, 1, 1, 0, 1, 1, 14, 14),       # small map, 8 wavefronts: 3 tiles/wave, 2 steps
-    (96, 576, 1, 1, 0, 1, 1, 14, 14),       # 5 tiles/wave, 3 steps, two filter batches
-    (160, 960, 1, 1, 0, 1, 1, 7, 7),        # 8 tiles/wave, 5 steps
-    (128, 256, 1, 1, 0, 1, 1, 7, 7),        # 2 tiles/wave, 4 steps
+    (64, 384, 1, 1, 0, 1, 1, 14, 14),       # small maps: two launches
+    (96, 576, 1, 1, 0, 1, 1, 14, 14),
+    (160, 960, 1, 1, 0, 1, 1, 7, 7),
+    (128, 256, 1, 1, 0, 1, 1, 7, 7),
+    (128, 64, 1, 1, 0, 1, 1, 40, 40),       # epilogue in the kernel: 4 reduction steps
     (320, 1280, 1, 1, 0, 1, 1, 7, 7),       # too long a reduction: two launches
     (32, 32, 3, 1, 1, 1, 32, 12, 12),       # depthwise 3x3, epilogue in the kernel
     (64, 64, 3, 2, 1, 1, 64, 13, 13),       # depthwise stride 2
