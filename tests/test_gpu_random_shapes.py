@@ -1,0 +1,170 @@
+"""Random-shape parity sweep: operators of the HIP library against the CPU oracle on shapes,
+strides, paddings, densities and channel counts drawn from a fixed seed per case, so that
+corners nobody thought of listing by hand (ragged maps, partial channel tiles, windows larger
+than the map's remainder) are visited too.  Masks bit-exact, elementwise operators bit-exact,
+contractions within the fp16 tolerance (2e-2 absolute)."""
+import os
+import random
+import sys
+
+import pytest
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+from oracle import delta_ops as ops  # noqa: E402
+from util import DEV, assert_masked_close, assert_masked_equal, cl, poison, rand_mask  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+KINDS = ["stem", "stem_act", "depthwise", "pool", "add_upsampled", "pointwise", "conv", "deconv", "small_conv_act"]
+
+
+def hk():
+    from deltacnn_amd import hip_kernels
+    return hip_kernels
+
+
+def _half_filter(wt, transposed=False, depthwise=False):
+    from deltacnn_amd.filter_conversion import convert_half_filter
+    return convert_half_filter(wt, pixel_wise=depthwise, transposed=transposed).to(DEV)
+
+
+def _conv_and_fused_activation(x, mask, wt, filt, pk, stride, pad, cout, rnd, g):
+    """dc_conv against the oracle, then dc_conv_act against dc_conv + dc_activate_truncate."""
+    want, wm = ops.conv(x, mask, wt, None, stride, pad, (1, 1), 1)
+    dx, dm = cl(poison(x, mask)), cl(mask)
+    o1, m1 = hk().sparse_conv(dx, filt, dm, None, stride, pad, (1, 1), 1, c_out=cout, create_out_mask=True, packed_filter=pk)
+    assert torch.equal(m1.cpu(), wm)
+    assert_masked_close(o1, want, wm, 0, 2e-2, "conv")
+    act, mode = rnd.choice([(1, 0), (2, 0), (3, 1), (1, 2)])
+    prev = torch.randn(want.shape, generator=g).half()
+    trunc = (torch.randn(want.shape, generator=g) * 0.01).half()
+    p1, t1 = cl(prev), cl(trunc)
+    hk().sparse_activation(o1, p1, t1, m1, 0.3, act, mode)
+    p2, t2 = cl(prev), cl(trunc)
+    o2, m2 = hk().sparse_conv_activation(dx, filt, dm, None, p2, t2, 0.3, act, mode, stride, pad, (1, 1), 1, cout, packed_filter=pk)
+    assert torch.equal(m1, m2) and torch.equal(p1, p2) and torch.equal(t1, t2)
+    assert_masked_equal(o2, o1.cpu(), m1.cpu(), "fused activation")
+
+
+@pytest.mark.parametrize("case", range(72))
+def test_random_shape(lib, case):
+    rnd = random.Random(7000 + case)
+    g = torch.Generator().manual_seed(9000 + case)
+    kind = KINDS[case % len(KINDS)]
+    B = rnd.choice([1, 2])
+    density = rnd.choice([0.0, 0.05, 0.5, 1.0])
+    if kind in ("stem", "stem_act"):
+        cin, cout = rnd.choice([1, 2, 3, 4]), rnd.choice([4, 8, 16, 20, 32, 48, 64])
+        k, st = rnd.choice([1, 2, 3, 5, 7, 8]), rnd.choice([1, 2])
+        pad = rnd.choice([0, k // 2, max(0, k // 2 - 1)])
+        H, W = rnd.randint(k + 1, 70), rnd.randint(k + 1, 70)
+        mask = rand_mask(g, B, H, W, max(density, 0.05))
+        x = (torch.randn(B, cin, H, W, generator=g) * (0.01 + rand_mask(g, B, H, W, 0.5).float())).half()
+        wt = (torch.randn(cout, cin, k, k, generator=g) / (cin * k * k) ** 0.5).half()
+        filt = _half_filter(wt)
+        pk = hk().pack_filter(filt, cin, cout, 1)
+        if kind == "stem":
+            want, wm = ops.conv(x, mask, wt, None, (st, st), (pad, pad), (1, 1), 1)
+            out, om = hk().sparse_conv(cl(poison(x, mask)), filt, cl(mask), None, (st, st), (pad, pad), (1, 1), 1,
+                                       c_out=cout, create_out_mask=True, packed_filter=pk)
+            assert torch.equal(om.cpu(), wm)
+            assert_masked_close(out, want, wm, 0, 2e-2, "out")
+        else:
+            _conv_and_fused_activation(x, mask, wt, filt, pk, (st, st), (pad, pad), cout, rnd, g)
+    elif kind == "depthwise":
+        C, st = rnd.choice([8, 16, 24, 40, 64, 136]), rnd.choice([1, 2])
+        H, W = rnd.choice([(rnd.randint(5, 40), rnd.randint(5, 40)), (rnd.randint(380, 420), rnd.randint(380, 420))])
+        mask = rand_mask(g, B, H, W, density)
+        x = torch.randn(B, C, H, W, generator=g).half()
+        wt = (torch.randn(C, 1, 3, 3, generator=g) / 3).half()
+        filt = _half_filter(wt, depthwise=True)
+        want, wm = ops.conv(x, mask, wt, None, (st, st), (1, 1), (1, 1), C)
+        out, om = hk().sparse_conv(cl(poison(x, mask)), filt, cl(mask), None, (st, st), (1, 1), (1, 1), C, c_out=C,
+                                   create_out_mask=True)
+        assert torch.equal(om.cpu(), wm)
+        assert_masked_close(out, want, wm, 0, 2e-2, "out")
+    elif kind == "pool":
+        C, K, st, mode = rnd.choice([8, 16, 24, 64, 128, 520]), rnd.choice([2, 3]), rnd.choice([1, 2]), rnd.choice([0, 1])
+        pad = rnd.choice([0, 1]) if K == 3 else 0
+        H, W = rnd.randint(K + 1, 40), rnd.randint(K + 1, 40)
+        mask = rand_mask(g, B, H, W, density)
+        x, prev = torch.randn(B, C, H, W, generator=g).half(), torch.randn(B, C, H, W, generator=g).half()
+        want, wm = ops.pool(x, prev if mode == 0 else None, mask, (K, K), (st, st), (pad, pad), (1, 1), mode)
+        out, om = hk().sparse_pooling(cl(poison(x, mask)), cl(prev) if mode == 0 else None, (K, K), cl(mask), (st, st),
+                                      (pad, pad), (1, 1), pooling_mode_int=mode)
+        assert torch.equal(om.cpu(), wm)
+        assert_masked_equal(out, want, wm, "out")
+    elif kind == "add_upsampled":
+        C, sc, act = rnd.choice([3, 8, 32, 72, 136]), rnd.choice([2, 4, 8]), rnd.choice([-1, 1, 3])
+        h, w = rnd.randint(1, 9), rnd.randint(1, 9)
+        H, W = h * sc, w * sc
+        ma, mb = rand_mask(g, B, H, W, 0.3), rand_mask(g, B, h, w, 0.5)
+        a, b = torch.randn(B, C, H, W, generator=g).half(), torch.randn(B, C, h, w, generator=g).half()
+        prev = torch.randn(B, C, H, W, generator=g).half() if act > 0 else None
+        up, um = ops.upsample(b, mb, sc)
+        wp = prev.clone() if act > 0 else None
+        want, wm = ops.add(a, ma, up, um, wp, 0.75, -0.5, act, False)
+        dp = cl(prev) if act > 0 else None
+        out = torch.full((B, C, H, W), float("nan"), dtype=torch.half, device=DEV).contiguous(memory_format=torch.channels_last)
+        mo = torch.full((B, 1, H, W), -3, dtype=torch.int32, device=DEV)
+        hk().sparse_add_upsampled(cl(poison(a, ma)), cl(poison(b, mb)), dp, out, cl(ma), cl(mb), mo, 0.75, -0.5, act, sc)
+        assert torch.equal(mo.cpu(), wm)
+        assert_masked_equal(out, want, wm, "out")
+        if act > 0:
+            assert torch.equal(dp.cpu(), wp)
+    elif kind == "pointwise":
+        cin, cout = rnd.choice([8, 24, 64, 136, 320, 448]), rnd.choice([4, 20, 64, 80, 128, 256])
+        H, W = rnd.randint(5, 70), rnd.randint(5, 70)
+        mask = rand_mask(g, B, H, W, density)
+        x = torch.randn(B, cin, H, W, generator=g).half()
+        wt = (torch.randn(cout, cin, 1, 1, generator=g) / cin ** 0.5).half()
+        filt = _half_filter(wt)
+        pk = hk().pack_filter(filt, cin, cout, 1)
+        want, wm = ops.conv(x, mask, wt, None, (1, 1), (0, 0), (1, 1), 1)
+        out, om = hk().sparse_conv(cl(poison(x, mask)), filt, cl(mask), None, (1, 1), (0, 0), (1, 1), 1, c_out=cout,
+                                   create_out_mask=True, packed_filter=pk)
+        assert torch.equal(om.cpu(), wm)
+        assert_masked_close(out, want, wm, 0, 2e-2, "out")
+    elif kind == "conv":
+        cin, cout = rnd.choice([16, 32, 64, 128, 256, 320]), rnd.choice([16, 24, 64, 128, 256])
+        k, st, dil = rnd.choice([3, 3, 5]), rnd.choice([1, 1, 2]), rnd.choice([1, 1, 2])
+        H, W = rnd.randint(20, 90), rnd.randint(20, 90)
+        pad = dil * (k // 2)
+        mask = rand_mask(g, 1, H, W, density)
+        x = torch.randn(1, cin, H, W, generator=g).half()
+        wt = (torch.randn(cout, cin, k, k, generator=g) / (cin * k * k) ** 0.5).half()
+        filt = _half_filter(wt)
+        pk = hk().pack_filter(filt, cin, cout, 1)
+        want, wm = ops.conv(x, mask, wt, None, (st, st), (pad, pad), (dil, dil), 1)
+        out, om = hk().sparse_conv(cl(poison(x, mask)), filt, cl(mask), None, (st, st), (pad, pad), (dil, dil), 1,
+                                   c_out=cout, create_out_mask=True, packed_filter=pk)
+        assert torch.equal(om.cpu(), wm)
+        assert_masked_close(out, want, wm, 0, 2e-2, "out")
+    elif kind == "deconv":
+        cin, cout = rnd.choice([8, 16, 64, 128, 256]), rnd.choice([8, 16, 64, 128])
+        k, st = rnd.choice([(4, 2), (2, 2), (3, 2), (8, 4), (6, 4), (3, 1), (2, 4)])
+        H, W = rnd.randint(3, 40), rnd.randint(3, 40)
+        pad = rnd.choice([0, max(0, (k - st) // 2)])
+        mask = rand_mask(g, B, H, W, density)
+        x = torch.randn(B, cin, H, W, generator=g).half()
+        wt = (torch.randn(cin, cout, k, k, generator=g) / (cin * k * k / st / st) ** 0.5).half()
+        filt = _half_filter(wt, transposed=True)
+        pk = hk().pack_filter(filt, cin, cout, 1, transposed=True)
+        want, wm = ops.deconv(x, mask, wt, None, (st, st), (pad, pad), (1, 1), 1)
+        out, om = hk().sparse_deconv(cl(poison(x, mask)), filt, cl(mask), None, (st, st), (pad, pad), (1, 1), 1,
+                                     c_out=cout, create_out_mask=True, packed_filter=pk)
+        assert torch.equal(om.cpu(), wm)
+        assert_masked_close(out, want, wm, 0, 2e-2, "out")
+    else:  # small K x K layers with the activation fused where one wavefront holds all channels
+        cin, cout = rnd.choice([8, 16, 32, 64]), rnd.choice([4, 16, 24, 32, 64])
+        k, st = rnd.choice([3, 3, 5]), rnd.choice([1, 2])
+        H, W = rnd.randint(6, 70), rnd.randint(6, 70)
+        mask = rand_mask(g, B, H, W, max(density, 0.05))
+        x = (torch.randn(B, cin, H, W, generator=g) * (0.01 + rand_mask(g, B, H, W, 0.5).float())).half()
+        wt = (torch.randn(cout, cin, k, k, generator=g) / (cin * k * k) ** 0.5).half()
+        filt = _half_filter(wt)
+        pk = hk().pack_filter(filt, cin, cout, 1)
+        _conv_and_fused_activation(x, mask, wt, filt, pk, (st, st), (k // 2, k // 2), cout, rnd, g)
