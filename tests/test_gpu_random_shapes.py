@@ -168,3 +168,58 @@ def test_random_shape(lib, case):
         filt = _half_filter(wt)
         pk = hk().pack_filter(filt, cin, cout, 1)
         _conv_and_fused_activation(x, mask, wt, filt, pk, (st, st), (k // 2, k // 2), cout, rnd, g)
+
+
+@pytest.mark.parametrize("case", range(48))
+def test_random_rectangular_fp32(lib, case):
+    """fp32 with everything unequal in y and x (window, stride, padding, dilation), grouped
+    channels and a bias: the generic kernels' index arithmetic.  1e-4 relative."""
+    from deltacnn_amd.filter_conversion import convert_filter_out_channels_last
+    rnd = random.Random(17000 + case)
+    g = torch.Generator().manual_seed(19000 + case)
+    kind = ["conv", "deconv", "pool"][case % 3]
+    B = rnd.choice([1, 2, 3])
+    density = rnd.choice([0.05, 0.3, 1.0])
+    K = (rnd.randint(1, 5), rnd.randint(1, 5))
+    H, W = rnd.randint(6, 33), rnd.randint(6, 33)
+    mask = rand_mask(g, B, H, W, density)
+    if kind == "conv":
+        groups = rnd.choice([1, 1, 2, 4])
+        cin, cout = groups * rnd.choice([1, 3, 4, 9]), groups * rnd.choice([1, 2, 4, 7])
+        st, dil = (rnd.randint(1, 3), rnd.randint(1, 3)), (rnd.randint(1, 2), rnd.randint(1, 2))
+        pad = (rnd.randint(0, dil[0] * (K[0] - 1)), rnd.randint(0, dil[1] * (K[1] - 1)))
+        if H + 2 * pad[0] < dil[0] * (K[0] - 1) + 1 or W + 2 * pad[1] < dil[1] * (K[1] - 1) + 1:
+            pytest.skip("window larger than the padded map")
+        x = torch.randn(B, cin, H, W, generator=g)
+        wt = torch.randn(cout, cin // groups, *K, generator=g) / (cin // groups * K[0] * K[1]) ** 0.5
+        bias = torch.randn(cout, generator=g) if rnd.random() < 0.5 else None
+        want, wm = ops.conv(x, mask, wt, bias, st, pad, dil, groups)
+        out, om = hk().sparse_conv(cl(poison(x, mask)), convert_filter_out_channels_last(wt).to(DEV), cl(mask),
+                                   bias.to(DEV) if bias is not None else None, st, pad, dil, groups, c_out=cout,
+                                   create_out_mask=True)
+        assert out.shape == want.shape and torch.equal(om.cpu(), wm)
+        assert_masked_close(out, want, wm, 1e-4, 1e-5, "out")
+    elif kind == "deconv":
+        cin, cout = rnd.choice([1, 3, 8, 17]), rnd.choice([1, 4, 6, 13])
+        st = (rnd.randint(1, 3), rnd.randint(1, 3))
+        p = rnd.randint(0, min(K[0], K[1]) - 1)
+        x = torch.randn(B, cin, H, W, generator=g)
+        wt = torch.randn(cin, cout, *K, generator=g) / (cin * K[0] * K[1]) ** 0.5
+        bias = torch.randn(cout, generator=g) if rnd.random() < 0.5 else None
+        want, wm = ops.deconv(x, mask, wt, bias, st, (p, p), (1, 1), 1)
+        out, om = hk().sparse_deconv(cl(poison(x, mask)), convert_filter_out_channels_last(wt, transposed=True).to(DEV),
+                                     cl(mask), bias.to(DEV) if bias is not None else None, st, (p, p), (1, 1), 1,
+                                     c_out=cout, create_out_mask=True)
+        assert out.shape == want.shape and torch.equal(om.cpu(), wm)
+        assert_masked_close(out, want, wm, 1e-4, 1e-5, "out")
+    else:
+        C, mode = rnd.choice([1, 4, 5, 12, 68]), rnd.choice([0, 1])
+        K = (max(K[0], 2), max(K[1], 2))
+        st = (rnd.randint(1, K[0]), rnd.randint(1, K[1]))
+        pad = (rnd.randint(0, K[0] // 2), rnd.randint(0, K[1] // 2))
+        x, prev = torch.randn(B, C, H, W, generator=g), torch.randn(B, C, H, W, generator=g)
+        want, wm = ops.pool(x, prev if mode == 0 else None, mask, K, st, pad, (1, 1), mode)
+        out, om = hk().sparse_pooling(cl(poison(x, mask)), cl(prev) if mode == 0 else None, K, cl(mask), st, pad, (1, 1),
+                                      pooling_mode_int=mode)
+        assert out.shape == want.shape and torch.equal(om.cpu(), wm)
+        assert_masked_close(out, want, wm, 1e-5, 1e-6, "out")
