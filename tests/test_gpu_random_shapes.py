@@ -223,3 +223,111 @@ def test_random_rectangular_fp32(lib, case):
                                       pooling_mode_int=mode)
         assert out.shape == want.shape and torch.equal(om.cpu(), wm)
         assert_masked_close(out, want, wm, 1e-5, 1e-6, "out")
+
+
+ELEMENTWISE = ["sparsify", "activate_truncate", "accumulate", "densify", "add", "add_to_dense", "mul_add", "concat",
+               "upsample"]
+
+
+@pytest.mark.parametrize("case", range(108))
+def test_random_elementwise(lib, case):
+    """The bandwidth operators in both types on any channel count (odd ones included) and on maps
+    on either side of 2^18 pixels, where the per-pixel kernels hand over to the scanning ones.
+    Bit-exact (fp32 multiply-add with a bias: 1e-6, the oracle fuses in fp64)."""
+    rnd = random.Random(27000 + case)
+    g = torch.Generator().manual_seed(29000 + case)
+    kind = ELEMENTWISE[case % len(ELEMENTWISE)]
+    dtype = rnd.choice([torch.float32, torch.float16])
+    big = rnd.random() < 0.25
+    if big:
+        B, H, W = 2, rnd.randint(300, 340), rnd.randint(440, 480)
+        C = rnd.choice([3, 8, 12, 24, 33, 40])
+    else:
+        B, H, W = rnd.choice([1, 2, 3]), rnd.randint(1, 40), rnd.randint(1, 40)
+        C = rnd.randint(1, 140)
+    density = rnd.choice([0.0, 0.03, 0.3, 1.0])
+    mask = rand_mask(g, B, H, W, density)
+    x = torch.randn(B, C, H, W, generator=g).to(dtype)
+    nan_like = lambda t: torch.full_like(t, float("nan"))  # noqa: E731
+    if kind == "sparsify":
+        prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+        xin = torch.where(mask != 0, (prev.float() + torch.randn(B, C, H, W, generator=g) * 0.5).to(dtype), prev)
+        wp = prev.clone()
+        want, wm = ops.sparsify(xin, wp, 0.25)
+        dp, dx = cl(prev), cl(xin)
+        dd, dm = nan_like(dx), torch.full((B, 1, H, W), -7, dtype=torch.int32, device=DEV)
+        hk().sparsify(dx, dp, dd, dm, 0.25)
+        assert torch.equal(dm.cpu(), wm) and torch.equal(dp.cpu(), wp)
+        assert_masked_equal(dd, want, wm, "delta")
+    elif kind in ("activate_truncate", "accumulate"):
+        act = rnd.choice([1, 2, 3])
+        mode = 0 if kind == "activate_truncate" else -1
+        prev = (torch.randn(B, C, H, W, generator=g) * 2).to(dtype)
+        trunc = (torch.randn(B, C, H, W, generator=g) * 0.005).to(dtype)
+        delta = (x.float() * (0.005 + 0.5 * rand_mask(g, B, H, W, 0.5).float())).to(dtype)
+        w = [delta.clone(), prev.clone(), trunc.clone(), mask.clone()]
+        ops.activate_truncate(*w, 0.1, act, mode)
+        d = [cl(poison(delta, mask)), cl(prev), cl(trunc), cl(mask)]
+        hk().sparse_activation(*d, 0.1, act, mode)
+        assert torch.equal(d[3].cpu(), w[3])
+        assert_masked_equal(d[0], w[0], w[3], "delta")
+        assert torch.equal(d[1].cpu(), w[1]) and torch.equal(d[2].cpu(), w[2])
+    elif kind == "densify":
+        prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+        wp = prev.clone()
+        ops.activate_truncate(x.clone(), wp, None, mask.clone(), 0.0, 0, -1)
+        dp = cl(prev)
+        out = nan_like(dp)
+        hk().densify(cl(poison(x, mask)), dp, out, cl(mask))
+        assert torch.equal(dp.cpu(), wp) and torch.equal(out.cpu(), wp)
+    elif kind == "add":
+        act = rnd.choice([-1, 1, 2])
+        wa, wb = rnd.choice([(1.0, 1.0), (0.5, -1.25), (2.0, 0.3)])
+        mb = rand_mask(g, B, H, W, rnd.choice([0.0, 0.2, 1.0]))
+        b = torch.randn(B, C, H, W, generator=g).to(dtype)
+        prev = torch.randn(B, C, H, W, generator=g).to(dtype) if act > 0 else None
+        wp = prev.clone() if act > 0 else None
+        want, wm = ops.add(x, mask, b, mb, wp, wa, wb, act, False)
+        dp = cl(prev) if act > 0 else None
+        out = nan_like(cl(x))
+        mo = torch.full((B, 1, H, W), -3, dtype=torch.int32, device=DEV)
+        hk().sparse_add_tensors(cl(poison(x, mask)), cl(poison(b, mb)), dp, out, cl(mask), cl(mb), mo, wa, wb, act, False)
+        assert torch.equal(mo.cpu(), wm)
+        assert_masked_equal(out, want, wm, "out")
+        if act > 0:
+            assert torch.equal(dp.cpu(), wp)
+    elif kind == "add_to_dense":
+        b = torch.randn(B, C, H, W, generator=g).to(dtype)
+        wb = b.clone()
+        ops.add_to_dense(x, wb, mask)
+        db = cl(b)
+        hk().sparse_add_to_dense_tensor(cl(poison(x, mask)), db, cl(mask))
+        assert torch.equal(db.cpu(), wb)
+    elif kind == "mul_add":
+        scale = torch.randn(C, generator=g).to(dtype)
+        bias = torch.randn(C, generator=g).to(dtype) if rnd.random() < 0.5 else None
+        want, wm = ops.mul_add(x, mask, scale, bias)
+        dx, dm = cl(poison(x, mask)), cl(mask)
+        out, om = nan_like(dx), torch.zeros_like(dm)
+        hk().sparse_mul_add(dx, dm, out, om, scale.to(DEV), None if bias is None else bias.to(DEV))
+        assert torch.equal(om.cpu(), wm)
+        if dtype == torch.float32 and bias is not None:
+            assert_masked_close(out, want, wm, 1e-6, 1e-6, "out")
+        else:
+            assert_masked_equal(out, want, wm, "out")
+    elif kind == "concat":
+        Cb = rnd.randint(1, 40) if big else rnd.randint(1, 140)
+        mb = rand_mask(g, B, H, W, rnd.choice([0.0, 0.2, 1.0]))
+        b = torch.randn(B, Cb, H, W, generator=g).to(dtype)
+        want, wm = ops.concatenate(x, mask, b, mb)
+        out, om = hk().sparse_concatenate((cl(poison(x, mask)), cl(mask)), (cl(poison(b, mb)), cl(mb)))
+        assert torch.equal(om.cpu(), wm)
+        assert_masked_equal(out, want, wm, "out")
+    else:
+        scale = rnd.choice([2, 2, 4]) if big else rnd.choice([2, 3, 4, 8])
+        if big:
+            x, mask = x[:, :, ::2, ::2].contiguous(), mask[:, :, ::2, ::2].contiguous()
+        want, wm = ops.upsample(x, mask, scale)
+        out, om = hk().sparse_upsample(cl(poison(x, mask)), cl(mask), scale)
+        assert torch.equal(om.cpu(), wm)
+        assert_masked_equal(out, want, wm, "out")
