@@ -109,3 +109,18 @@ def test_toy_cnn_teacher_forced(lib, dtype):
     video = noise_block_video(frames=10, size=64, fraction=0.05)
     ref, dut = _build(ToyCNN, dtype, 0.05)
     assert run_teacher_forced(ref, dut, video, dtype) == 10 * (1 + 3 + 2 + 1)
+
+
+@pytest.mark.parametrize("network", ["hrnet", "dla34"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_multibranch_teacher_forced(lib, network, dtype):
+    """Every layer call of HRNet (strided exchange convolutions, nearest upsampling, chained sums
+    with ReLU) and of DLA-34 + CenterNet heads (max-pooling, concatenating roots, transposed
+    convolutions, dense heads) over 8 frames, each HIP layer fed the oracle's inputs."""
+    from deltacnn_amd.video import moving_rectangles_video
+    from test_gpu_network import _calibrated, _dla, _hrnet
+    builder, size = {"hrnet": (_hrnet, (64, 64)), "dla34": (_dla, (64, 96))}[network]
+    video = moving_rectangles_video(frames=8, height=size[0], width=size[1], n_rect=2, min_size=8, max_size=24)
+    ref, dut = _build(builder, dtype, 0.05, _calibrated(builder, video[:3]))
+    n = run_teacher_forced(ref, dut, video, dtype)
+    assert n % 8 == 0 and n // 8 > 100
