@@ -276,3 +276,51 @@ def test_multibranch_networks(lib, builder, size, dtype):
                 assert _out_err(got, want) <= 1e-4 * _out_scale(want), f"frame {t}"
     print(f"{dtype}: |oracle-dense| {e_ref:.4f}  |hip-dense| {e_dut:.4f}")
     assert e_dut <= 1.5 * e_ref + 2e-2
+
+
+def _two_hip_models(builder, state):
+    from deltacnn_amd import sparse_layers as SL
+    SL.DCThreshold.t_default = 0.05
+    pair = []
+    for _ in range(2):
+        m = builder(SL).eval()
+        m.load_state_dict(state)
+        m = m.to(DEV, memory_format=torch.channels_last).half()
+        m.process_filters()
+        pair.append(m)
+    return pair
+
+
+def _same(a, b):
+    if isinstance(a, dict):
+        return all(_same(a[k], b[k]) for k in a)
+    return torch.equal(a, b)
+
+
+@pytest.mark.parametrize("network,size", [("mobilenet", (224, 224)), ("hrnet", (256, 256)), ("dla34", (192, 320))])
+def test_fused_layer_calls_change_nothing(lib, network, size):
+    """One-launch forms (convolution + activation, convolution + residual sum, sum with an
+    upsampled operand) against the same model issuing the separate layer calls, fp16, at map
+    sizes where the fused kernels are the ones chosen: outputs bit-identical on every frame."""
+    from deltacnn_amd import sparse_layers as SL
+    from deltacnn_amd.video import moving_rectangles_video
+    video = moving_rectangles_video(frames=8, height=size[0], width=size[1], n_rect=3, min_size=16, max_size=60)
+    small = moving_rectangles_video(frames=3, height=64, width=96, n_rect=2, min_size=8, max_size=24)
+    if network == "mobilenet":
+        builder, state = _mobilenet, _calibrated_state(small)
+    else:
+        builder = {"hrnet": _hrnet, "dla34": _dla}[network]
+        state = _calibrated(builder, small)
+    fused, plain = _two_hip_models(builder, state)
+    try:
+        with torch.no_grad():
+            for t in range(video.shape[0]):
+                frame = cl(video[t:t + 1].half())
+                SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = True
+                got = fused(frame)
+                got = {k: v.clone() for k, v in got.items()} if isinstance(got, dict) else got.clone()
+                SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = False
+                want = plain(frame)
+                assert _same(got, want), f"frame {t}"
+    finally:
+        SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = True
