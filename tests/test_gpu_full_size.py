@@ -1,0 +1,100 @@
+"""The configurations the measurements are quoted on, at their full sizes, checked through
+properties that need no CPU restatement of that size:
+
+  * threshold 0: the delta model's densified output equals the dense PyTorch model's (the same
+    weights, fp32, on the GPU) on every frame -- MobileNetV2 224x224, HRNet-W32 256x256,
+    DLA-34 + CenterNet 544x960;
+  * idempotence: a repeated frame is an empty update -- the output does not change by a bit;
+  * the single-layer shapes on 64x64 maps (3x3 256->256, 1x1 256->1024, depthwise 3x3 on 512
+    channels, fp16) against torch's fp32 convolution of the masked delta, masks against the
+    dilation of the input mask; 2e-2 absolute.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from util import DEV, cl, rand_mask
+
+pytestmark = pytest.mark.gpu
+
+
+def _builders():
+    from deltacnn_amd.networks import DLA34CenterNet, HRNet, MobileNetV2
+    return {"mobilenetv2": (MobileNetV2, (224, 224)), "hrnet_w32": (HRNet, (256, 256)),
+            "dla34_centernet": (DLA34CenterNet, (544, 960))}
+
+
+def _pair(name, dtype, thr):
+    from deltacnn_amd import sparse_layers as SL
+    from deltacnn_amd.networks import DenseLayers, fold_data_statistics
+    from deltacnn_amd.video import moving_rectangles_video
+    builder, size = _builders()[name]
+    SL.DCThreshold.t_default = thr
+    torch.manual_seed(0)
+    dense = builder(DenseLayers).eval()
+    with torch.no_grad():  # keeps activations of the random-init model in a sane range
+        fold_data_statistics(dense, moving_rectangles_video(frames=2, height=64, width=96, n_rect=2, min_size=8, max_size=24))
+    if dtype == torch.float16:
+        dense = dense.half().float()
+    model = builder(SL).eval()
+    model.load_state_dict(dense.state_dict())
+    model = model.to(DEV, memory_format=torch.channels_last).to(dtype)
+    model.process_filters()
+    video = moving_rectangles_video(frames=5, height=size[0], width=size[1], n_rect=3, min_size=20, max_size=80)
+    return dense.to(DEV), model, video
+
+
+def _items(out):
+    return out.items() if isinstance(out, dict) else [("out", out)]
+
+
+@pytest.mark.parametrize("name", ["mobilenetv2", "hrnet_w32", "dla34_centernet"])
+def test_threshold_zero_equals_dense_model(lib, name):
+    dense, model, video = _pair(name, torch.float32, 0.0)
+    with torch.no_grad():
+        for t in range(video.shape[0]):
+            frame = video[t:t + 1].to(DEV)
+            want = dict(_items(dense(frame)))
+            got = dict(_items(model(cl(frame))))
+            for k in want:
+                err = float((got[k].float() - want[k]).abs().max())
+                assert err <= 1e-4 * max(1.0, float(want[k].abs().max())), f"frame {t} {k}: {err}"
+
+
+@pytest.mark.parametrize("name", ["mobilenetv2", "hrnet_w32", "dla34_centernet"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_repeated_frame_is_an_empty_update(lib, name, dtype):
+    _, model, video = _pair(name, dtype, 0.05)
+    with torch.no_grad():
+        for t in range(3):
+            first = {k: v.clone() for k, v in _items(model(cl(video[t:t + 1].to(DEV, dtype))))}
+        again = dict(_items(model(cl(video[2:3].to(DEV, dtype)))))
+        for k in first:
+            assert torch.equal(first[k], again[k]), k
+            assert bool(torch.isfinite(first[k].float()).all()), k
+
+
+SINGLE_LAYERS = [("3x3_256_256", 256, 256, 3, 1), ("1x1_256_1024", 256, 1024, 1, 1), ("dw3x3_512", 512, 512, 3, 512)]
+
+
+@pytest.mark.parametrize("layer", SINGLE_LAYERS, ids=lambda c: c[0])
+@pytest.mark.parametrize("density", [0.01, 0.1, 1.0])
+def test_single_layer_shapes_against_torch(lib, layer, density):
+    from deltacnn_amd import hip_kernels as hk
+    from deltacnn_amd.filter_conversion import convert_half_filter
+    _, cin, cout, k, groups = layer
+    g = torch.Generator().manual_seed(4100 + cin + cout + k)
+    mask = rand_mask(g, 1, 64, 64, density).to(DEV)
+    x = torch.randn(1, cin, 64, 64, generator=g).half().to(DEV)
+    wt = (torch.randn(cout, cin // groups, k, k, generator=g) / (cin // groups * k * k) ** 0.5).half().to(DEV)
+    active = mask != 0
+    want = F.conv2d(torch.where(active, x, torch.zeros_like(x)).float(), wt.float(), padding=k // 2, groups=groups)
+    want_mask = (F.max_pool2d(active.float(), k, stride=1, padding=k // 2) > 0)
+    filt = convert_half_filter(wt, pixel_wise=groups > 1).to(DEV)
+    pk = hk.pack_filter(filt, cin, cout, groups)
+    xin = torch.where(active, x, torch.full_like(x, float("nan")))
+    out, om = hk.sparse_conv(cl(xin), filt, cl(mask), None, (1, 1), (k // 2, k // 2), (1, 1), groups, c_out=cout,
+                             create_out_mask=True, packed_filter=pk)
+    assert torch.equal(om != 0, want_mask)
+    diff = torch.where(want_mask, (out.float() - want).abs(), torch.zeros_like(want))
+    assert float(diff.max()) <= 2e-2, float(diff.max())
