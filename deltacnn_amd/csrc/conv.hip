@@ -280,7 +280,7 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
 // which cuts load instructions and conversions per output pixel by more than half.  Per pixel
 // the arithmetic (tap order, zero-select of inactive taps, bias, epilogue) is that of
 // conv_dw_kernel, so the results are identical.
-template <typename T, int ACT>
+template <typename T, int ACT, bool LW>
 __global__ void __launch_bounds__(256)
 conv_dw_strip_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
                      const T *__restrict__ bias, T *__restrict__ out,
@@ -303,6 +303,17 @@ conv_dw_strip_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ fi
     const int glo = lane_id() & ~(G - 1);
     const uint64_t gmask = G >= WAVE ? ~0ull : ((1ull << G) - 1ull);
     const int iy0 = oy - p.pt, ix0 = ox0 - p.pl;
+
+    // LW: the filter goes through LDS once per workgroup, 36 registers less per lane (a third
+    // wavefront per SIMD); costs a barrier, which small maps do not earn back
+    __shared__ Vec<T, N> s_w[LW ? 9 : 1][WAVE];
+    if (LW) {
+        const int nv = C / N;
+        for (int i = threadIdx.x; i < 9 * nv; i += 256) {
+            const int t = i / nv, v = i - t * nv;
+            s_w[t][v] = vload<T, N>(filter + (size_t)t * C + v * N);
+        }
+    }
 
     // activity of the 3 x COLS input pixels of the strip, one mask word per lane and pass
     uint32_t words = 0;
@@ -327,6 +338,7 @@ conv_dw_strip_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ fi
         any |= active[j];
         if (valid && ox0 + j < p.Wo && gl == 0) out_mask[po0 + j] = active[j] ? 1 : 0;
     }
+    if (LW) __syncthreads();
     if (ballot(any) == 0) return;
 
     const int c = min(gl * N, C - N);
@@ -339,7 +351,7 @@ conv_dw_strip_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ fi
     }
     // all rows of the strip and the filter are requested together (clamped, always valid
     // addresses); inactive taps are zeroed by selection afterwards
-    Vec<T, N> x[3][COLS], w[9];
+    Vec<T, N> x[3][COLS];
     const T *inb = in + (size_t)b * p.Hi * p.Wi * C;
 #pragma unroll
     for (int wy = 0; wy < 3; ++wy) {
@@ -350,8 +362,11 @@ conv_dw_strip_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ fi
             x[wy][wx] = vload<T, N>(inb + (size_t)(iy * p.Wi + ix) * C + c);
         }
     }
+    Vec<T, N> w[LW ? 1 : 9];
+    if (!LW) {
 #pragma unroll
-    for (int t = 0; t < 9; ++t) w[t] = vload<T, N>(filter + (size_t)t * C + c);
+        for (int t = 0; t < 9; ++t) w[LW ? 0 : t] = vload<T, N>(filter + (size_t)t * C + c);
+    }
     Vec<T, N> bv;
     if (bias != nullptr) bv = vload<T, N>(bias + c);
 
@@ -363,8 +378,9 @@ conv_dw_strip_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ fi
 #pragma unroll
         for (int t = 0; t < 9; ++t) {
             const Vec<T, N> xs = vkeep<T, N>(x[t / 3][j + t % 3], (taps[j] >> t) & 1u);
+            const Vec<T, N> wt = LW ? s_w[LW ? t : 0][c / N] : w[LW ? 0 : t];
 #pragma unroll
-            for (int e = 0; e < N; ++e) acc[e] = __builtin_fmaf(float(xs.v[e]), float(w[t].v[e]), acc[e]);
+            for (int e = 0; e < N; ++e) acc[e] = __builtin_fmaf(float(xs.v[e]), float(wt.v[e]), acc[e]);
         }
         Vec<T, N> dl[1];
         if (bias != nullptr) {
@@ -1792,7 +1808,13 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
         EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f, epi ? epi->mode : 0};
         const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
         note_kernel("conv_dw_strip_kernel");
-#define DC_DWS(A) conv_dw_strip_kernel<T, A><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg)
+        // filter in LDS (measured): from 8 MB of output on with rows of more than 8 vectors
+        const bool lw = nvec > 8 && P_out * g.in_c * (int64_t)sizeof(T) >= (8 << 20);
+#define DC_DWS(A)                                                                                              \
+    do {                                                                                                       \
+        if (lw) conv_dw_strip_kernel<T, A, true><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg);   \
+        else conv_dw_strip_kernel<T, A, false><<<grid, 256, 0, s>>>(p, in, filter, bias, out, mask, out_mask, e, lg);     \
+    } while (0)
         switch (act) {
             case DC_ACT_LINEAR: DC_DWS(DC_ACT_LINEAR); break;
             case DC_ACT_RELU: DC_DWS(DC_ACT_RELU); break;

@@ -342,6 +342,7 @@ CONVS = [
     (16, 16, 3, 2, 1, 1, 16, 600, 521),     # ... with a stride
     (16, 16, 3, 1, 1, 1, 16, 300, 301),     # depthwise on a large map: strips of four pixels per lane group
     (24, 24, 3, 1, 1, 1, 24, 250, 251),     # ... with idle lanes in the group
+    (144, 144, 3, 1, 1, 1, 144, 130, 131),  # ... wide rows on 8 MB and more: filter through LDS
 ]
 
 
@@ -412,6 +413,7 @@ def test_conv(lib, dtype, cfg, density, use_bias, packed):
     ((32, 32, 3, 1, 1, 1, 32, 15, 18), "conv_dw_kernel"),
     ((16, 16, 3, 1, 1, 1, 16, 726, 727), "conv_dw_scan_kernel"),
     ((16, 16, 3, 1, 1, 1, 16, 300, 301), "conv_dw_strip_kernel"),
+    ((144, 144, 3, 1, 1, 1, 144, 130, 131), "conv_dw_strip_kernel"),
     ((16, 16, 3, 2, 1, 1, 16, 600, 521), "conv_dw_scan_kernel"),
     ((3, 32, 3, 2, 1, 1, 1, 33, 31), "conv_stem_mfma_kernel"),
     ((3, 64, 3, 2, 1, 1, 1, 600, 520), "conv_fewcin_kernel"),     # many channel tiles on a large map
@@ -509,6 +511,7 @@ FUSED = [
     (16, 16, 3, 1, 1, 1, 16, 726, 727),     # very large map: mask scan and compaction per wavefront
     (24, 24, 3, 2, 1, 1, 24, 600, 521),     # the same with a stride
     (16, 16, 3, 1, 1, 1, 16, 300, 301),     # large map: strips of four pixels per lane group
+    (144, 144, 3, 1, 1, 1, 144, 130, 131),  # ... wide rows, filter through LDS
     (16, 96, 1, 1, 0, 1, 1, 110, 111),      # pointwise on a large map: convolution and activation as two launches
 ]
 
