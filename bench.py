@@ -6,7 +6,9 @@ folded) at a controlled input update density, on one MI355X.
 
 A step is one video frame through the whole network (sparsify -> 52 delta convolutions with
 activation/truncation -> residual adds -> global average pooling -> densify -> classifier).
-All frames are resident in HBM before the timed region.  One JSON line is printed with
+All frames are resident in HBM before the timed region.  The JSON line is printed as soon as the
+headline is known and again, enriched, after each group of sections (the last line printed is
+the result; a section that fails is named under "errors" and the run goes on).  It holds
   value            delta-path frames/sec at the requested density (default 10 %)
   dense_gpu        the same model dense (plain PyTorch / MIOpen) on the same GPU, eager and
                    graph-replayed, and the speed-up over the faster of the two
@@ -82,15 +84,65 @@ def time_steps(step, warmup, steps):
 UNROLL = 8  # frames per graph launch (processed one after the other)
 
 
+def launch_plan(steps, warmup, unroll=UNROLL):
+    """How `warmup` untimed and EXACTLY `steps` timed frames are cut into graph launches.
+
+    The frames of one launch are processed strictly one after the other, so the cut changes no
+    result, only how often the host launches.  `steps` is split into steps // unroll launches
+    of a graph that holds `unroll` frames plus, when that leaves a remainder, one launch of a
+    second graph that holds the `tail` remaining frames.  Warm-up runs ceil(warmup / unroll)
+    launches of the first graph and one launch of the tail graph, so both have run before
+    the clock starts.  Pure arithmetic (no GPU), returned as a dict:
+      unroll, tail, timed_main, warm_main, warm_tail   launches as described
+      warm_frames      frames the warm-up consumes (>= warmup)
+      frames_after_start   frames the clip must hold from the first graph frame on
+    """
+    if steps < 1 or warmup < 0:
+        raise ValueError("steps must be >= 1 and warmup >= 0")
+    unroll = max(1, min(unroll, steps))
+    tail = steps % unroll
+    warm_main = -(-warmup // unroll)
+    warm_tail = 1 if tail else 0
+    warm_frames = warm_main * unroll + warm_tail * tail
+    return {"unroll": unroll, "tail": tail, "timed_main": steps // unroll, "warm_main": warm_main,
+            "warm_tail": warm_tail, "warm_frames": warm_frames, "frames_after_start": warm_frames + steps}
+
+
+def clip_frames(steps, warmup, lead=2):
+    """Length of the clip the headline run needs: `lead` eager frames (the dense first frame and
+    one eager delta frame), the warm-up and timed frames of launch_plan, one spare."""
+    return lead + launch_plan(steps, warmup)["frames_after_start"] + 1
+
+
 def time_graph(model, frames, start, warmup, steps):
-    """Seconds per frame of model(frame) replayed from a HIP graph that holds UNROLL consecutive
-    frames per launch (exactly `steps` timed frames after at least `warmup` untimed ones)."""
+    """Seconds per frame of model(frame) on consecutive frames of the clip from frame `start`
+    on, replayed from HIP graphs cut as launch_plan says (exactly `steps` timed frames after
+    at least `warmup` untimed ones)."""
+    import torch
     from deltacnn_amd.graph import VideoGraph
-    unroll = UNROLL if steps % UNROLL == 0 else 1
-    vg = VideoGraph(model, frames, start=start, unroll=unroll)
-    warm = -(-warmup // unroll)
-    assert start + (warm + steps // unroll) * unroll <= frames.shape[0]
-    return time_steps(vg.step, warm, steps // unroll) / unroll
+    plan = launch_plan(steps, warmup)
+    if start + plan["frames_after_start"] > frames.shape[0]:
+        raise ValueError(f"clip of {frames.shape[0]} frames is too short: start {start} + "
+                         f"{plan['frames_after_start']} frames needed")
+    main = VideoGraph(model, frames, start=start, unroll=plan["unroll"])
+    tail = VideoGraph(model, frames, start=start, unroll=plan["tail"]) if plan["tail"] else None
+    for _ in range(plan["warm_main"]):
+        main.step()
+    pos = start + plan["warm_main"] * plan["unroll"]
+    if tail is not None:
+        tail.seek(pos)
+        tail.step()
+        pos += plan["tail"]
+        tail.seek(pos + plan["timed_main"] * plan["unroll"])
+    main.seek(pos)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(plan["timed_main"]):
+        main.step()
+    if tail is not None:
+        tail.step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
 
 
 def run_delta(delta, frames, warmup, steps, mode):
@@ -122,18 +174,30 @@ def run_dense(dense, frames, warmup, steps):
     return eager, graph
 
 
-def streams_bench(delta, dense, frames, batch=8, steps=64, warmup=16):
-    """Supplementary: `batch` independent video streams (the same clip at different offsets)
-    through ONE model instance as a batch, i.e. the same kernels on maps `batch` times larger.
-    Every stream keeps its own caches (they are the batch dimension of the layers' state).
-    Returns total frames/s for the delta path and for the dense model, both from HIP graphs."""
+STREAM_UNROLL = 4   # frames per graph launch of the batched-streams runs
+STREAM_STRIDE = 2   # clip offset between neighbouring streams, in frames
+
+
+def streams_clip_frames(batch, steps, warmup, unroll=STREAM_UNROLL, stride=STREAM_STRIDE):
+    """Frames a clip must hold for streams_bench: the last stream starts (batch-1)*stride frames
+    in, then 2 eager frames, ceil(warmup/unroll)*unroll warm-up and `steps` timed frames."""
+    return (batch - 1) * stride + 2 + -(-warmup // unroll) * unroll + (steps // unroll) * unroll + 1
+
+
+def streams_bench(delta, dense, batch=8, steps=64, warmup=16, density=0.10, with_dense=True):
+    """Supplementary: `batch` independent video streams (one clip of its own, read at different
+    offsets) through ONE model instance as a batch, i.e. the same kernels on maps `batch` times
+    larger.  Every stream keeps its own caches (they are the batch dimension of the layers'
+    state).  Returns total frames/s for the delta path and for the dense model, both from HIP
+    graphs."""
     import torch
+    from deltacnn_amd.video import controlled_density_video
+    unroll = STREAM_UNROLL
+    steps = max(unroll, steps - steps % unroll)
+    frames = gpu_frames(controlled_density_video(frames=streams_clip_frames(batch, steps, warmup), density=density))
     t, c, h, w = frames.shape
     rows = frames.permute(0, 2, 3, 1).reshape(t, h * w * c)
-    unroll = 4
-    span = t - (2 + warmup + steps + unroll)
-    offsets = torch.arange(batch, device=frames.device) * max(1, span // batch)
-    assert int(offsets[-1]) + 2 + warmup + steps + unroll <= t
+    offsets = torch.arange(batch, device=frames.device) * STREAM_STRIDE
 
     def fetch(index):
         return rows.index_select(0, index).view(-1, batch, h, w, c).permute(0, 1, 4, 2, 3)
@@ -152,11 +216,13 @@ def streams_bench(delta, dense, frames, batch=8, steps=64, warmup=16):
         for i in range(2):  # dense first frame of every stream, one eager delta frame
             delta(fetch(offsets + i)[0])
         d = timed(delta, 2)
-        dense(fetch(offsets)[0])
-        dn = timed(dense, 2)
         delta.reset_layers()
-    return {"streams": batch, "delta_fps_total": round(batch / d, 1), "dense_graph_fps_total": round(batch / dn, 1),
-            "ms_per_step": round(d * 1e3, 4)}
+        out = {"streams": batch, "update_density": density, "delta_fps_total": round(batch / d, 1),
+               "ms_per_step": round(d * 1e3, 4), "steps": steps}
+        if with_dense:
+            dense(fetch(offsets)[0])
+            out["dense_graph_fps_total"] = round(batch / timed(dense, 2), 1)
+    return out
 
 
 def trace_kernels(delta, frames):
@@ -321,7 +387,7 @@ def network_bench(which, steps, warmup):
         "hrnet": (HRNet, (256, 256), dict(n_rect=1, min_size=100, max_size=180, min_speed=2, max_speed=6)),
         "dla34": (DLA34CenterNet, (544, 960), dict(n_rect=12, min_size=30, max_size=200, min_speed=1, max_speed=5)),
     }[which]
-    video = moving_rectangles_video(frames=steps + warmup + 3 + UNROLL, height=size[0], width=size[1],
+    video = moving_rectangles_video(frames=clip_frames(steps, warmup), height=size[0], width=size[1],
                                     noise_sigma=0.0, **kw)
     torch.manual_seed(0)
     dense = builder(DenseLayers).eval().to("cuda", memory_format=torch.channels_last)
@@ -418,12 +484,11 @@ def main():
         print(json.dumps({"micro": micro_bench(), "scaled": scaled_bench()}), flush=True)
         return
     if args.network != "mobilenetv2":
-        steps = args.steps - args.steps % UNROLL if args.steps >= UNROLL else args.steps
-        print(json.dumps(network_bench(args.network, min(steps, 64), min(args.warmup, 16))), flush=True)
+        print(json.dumps(network_bench(args.network, min(args.steps, 64), min(args.warmup, 16))), flush=True)
         return
 
-    n_frames = args.warmup + args.steps + 3 + UNROLL
-    video = controlled_density_video(frames=n_frames, density=args.density)
+    plan = launch_plan(args.steps, args.warmup)
+    video = controlled_density_video(frames=clip_frames(args.steps, args.warmup), density=args.density)
     stats_video = moving_rectangles_video(frames=4)
     dense, delta, state = build_models(stats_video.to("cuda").contiguous(memory_format=torch.channels_last))
     frames = gpu_frames(video)
@@ -441,60 +506,9 @@ def main():
         print(json.dumps({"value": round(fps, 2), "unit": "frames/s", "ms_per_step": round(sec * 1e3, 4),
                           "steps": args.steps, "update_density": args.density}), flush=True)
         return
-    with torch.no_grad():
-        ref_logits = dense(frames[-1:]).float()
-    dense_eager, dense_graph = run_dense(dense, frames, args.warmup, args.steps)
-    dense_best = min(dense_eager, dense_graph)
-    log(f"dense GPU: eager {1 / dense_eager:.1f} fps, graph {1 / dense_graph:.1f} fps")
 
-    sweep = []
-    if not args.no_sweep:
-        for rho in SWEEP:
-            sw_steps = min(args.steps, 12 * UNROLL)
-            v = gpu_frames(controlled_density_video(frames=sw_steps + 13 + UNROLL, density=rho))
-            s = run_delta(delta, v, 10, sw_steps, args.mode)
-            sweep.append({"density": rho, "fps": round(1.0 / s, 1), "ms_per_frame": round(s * 1e3, 4),
-                          "speedup_vs_dense_gpu": round(dense_best / s, 3)})
-            log(f"  density {rho:4.2f}: {1 / s:9.1f} fps")
-
-    agg, rows = trace_kernels(delta, frames)
-    dom_name = max(agg, key=lambda k: agg[k]["ms"])
-    dom = agg[dom_name]
-    kernels = {k: {"launches_per_frame": round(a["launches_per_frame"], 2),
-                   "us_per_launch": round(a["us_per_launch"], 3),
-                   "ms_per_frame": round(a["ms_per_frame"], 4),
-                   "alg_bytes_per_launch": round(a["bytes_per_launch"], 1),
-                   "alg_GBps": round(a["GBps"], 2), "alg_TFLOPs": round(a["TFLOPs"], 3)}
-               for k, a in sorted(agg.items(), key=lambda kv: -kv[1]["ms"])}
-    alg_frame_bytes = sum(a["bytes"] for a in agg.values())
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
-    if os.path.exists(tpath):  # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-        with open(tpath) as f:
-            traffic = json.load(f).get(dom_name, {}).get("bytes_per_launch")
-    streams = None
-    if not args.no_micro:
-        streams = [streams_bench(delta, dense, frames, batch=nb) for nb in (8, 32)]
-        for st in streams:
-            log(f"{st['streams']} streams as a batch: delta {st['delta_fps_total']:.0f} frames/s in total, "
-                f"dense graph {st['dense_graph_fps_total']:.0f}")
-    micro = scaled = None
-    if not args.no_micro:
-        log("single-layer sweeps (64x64 fp16):")
-        micro = micro_bench()
-        log("scaled shapes (512x512, batch 8, C=64 fp16):")
-        scaled = scaled_bench()
-
-    cpu = None
-    if not args.no_cpu:
-        threads = min(16, os.cpu_count() or 1)
-        cpu_frames = max(1, min(args.cpu_frames, video.shape[0] - 1))
-        d_fps, dn_fps = cpu_baseline(state, video, cpu_frames, threads)
-        cpu = {"value": round(d_fps, 3), "unit": "frames/s", "cores": threads, "kind": "port",
-               "sample": f"{cpu_frames} delta frames of the same video through the fp32 CPU "
-                         f"oracle (pure PyTorch layers) after the dense first frame",
-               "dense_cpu_fps": round(dn_fps, 3)}
-
+    graph_launches = ([plan["unroll"]] * plan["timed_main"] + ([plan["tail"]] if plan["tail"] else [])
+                      if args.mode == "graph" else [])
     result = {
         "metric": "frames/sec vs update density (MobileNetV2 224^2); HBM GB/s % of peak",
         "value": round(fps, 2), "unit": "frames/s", "n_gpus": 1, "steps": args.steps,
@@ -503,33 +517,139 @@ def main():
         "config": {"workload": "MobileNetV2 w1.0 (BN folded, 1000-way head) 224x224 fp16 channels-last "
                                "batch 1, threshold 0.05 on all layers, controlled-density video",
                    "update_density": args.density, "launch_mode": args.mode,
-                   "frames_per_graph_launch": UNROLL if args.mode == "graph" and args.steps % UNROLL == 0 else 1,
+                   "frames_per_graph_launch": plan["unroll"] if args.mode == "graph" else 0,
+                   "timed_graph_launches": graph_launches,
                    "weights": "random init (seed 0) rescaled per conv to unit output variance"},
-        "dense_gpu": {"eager_fps": round(1 / dense_eager, 1), "graph_fps": round(1 / dense_graph, 1),
-                      "speedup_vs_dense_gpu": round(dense_best / sec, 3)},
-        "frame_alg_GBps": round(alg_frame_bytes / sec / 1e9, 2),
-        "kernel_time_sum_ms": round(sum(a["ms"] for a in agg.values()), 4),
-        "sweep": sweep,
-        "kernels": kernels,
-        "roofline": {"bound": "hbm", "kernel": dom_name,
-                     "achieved": round(dom["GBps"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom["GBps"] / HBM_PEAK_GBS, 5), "traffic": traffic,
-                     "bytes_per_launch": round(dom["bytes_per_launch"], 1),
-                     "us_per_launch": round(dom["us_per_launch"], 3),
-                     "note": "latency-bound regime: the feature maps of this workload are <= 2.4 MB and "
-                             "an empty dependent kernel in a HIP graph already costs ~1.6 us"},
-        "cpu_baseline": cpu,
-        "streams_as_batch": streams,
-        "micro": micro,
-        "scaled": scaled,
+        "roofline": None, "cpu_baseline": None,
     }
-    with torch.no_grad():
-        delta.reset_layers()
-        for i in range(frames.shape[0]):
-            out = delta(frames[i:i + 1])
-        result["logit_max_abs_diff_vs_dense"] = round(float((out.float() - ref_logits).abs().max()), 4)
-        result["logit_max_abs"] = round(float(ref_logits.abs().max()), 4)
-    print(json.dumps(result), flush=True)
+    errors = {}
+
+    def emit():
+        """One JSON line with everything known so far; the LAST line printed is the result.  It
+        is printed as soon as the headline exists and again after each group of sections, so a
+        failure further down cannot erase it."""
+        if errors:
+            result["errors"] = errors
+        print(json.dumps(result), flush=True)
+
+    def section(name, fn):
+        """Run one report section; a failure is recorded under errors[name] and the run goes on."""
+        try:
+            return fn()
+        except Exception as e:  # noqa: BLE001 -- the report must survive any one section
+            import traceback
+            errors[name] = f"{type(e).__name__}: {e}"
+            log(f"section {name} failed:\n{traceback.format_exc()}")
+            return None
+
+    emit()
+
+    # -- the dominant kernel's roofline: per-call device times of one traced frame ------------
+    def roofline_section():
+        agg, rows = trace_kernels(delta, frames)
+        dom_name = max(agg, key=lambda k: agg[k]["ms"])
+        dom = agg[dom_name]
+        result["kernels"] = {k: {"launches_per_frame": round(a["launches_per_frame"], 2),
+                                 "us_per_launch": round(a["us_per_launch"], 3),
+                                 "ms_per_frame": round(a["ms_per_frame"], 4),
+                                 "alg_bytes_per_launch": round(a["bytes_per_launch"], 1),
+                                 "alg_GBps": round(a["GBps"], 2), "alg_TFLOPs": round(a["TFLOPs"], 3)}
+                             for k, a in sorted(agg.items(), key=lambda kv: -kv[1]["ms"])}
+        result["library_launches_per_frame"] = sum(a["launches"] for a in agg.values())
+        result["frame_alg_GBps"] = round(sum(a["bytes"] for a in agg.values()) / sec / 1e9, 2)
+        result["kernel_time_sum_ms"] = round(sum(a["ms"] for a in agg.values()), 4)
+        traffic = None
+        tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
+        if os.path.exists(tpath):  # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+            with open(tpath) as f:
+                traffic = json.load(f).get(dom_name, {}).get("bytes_per_launch")
+        result["roofline"] = {
+            "bound": "hbm", "kernel": dom_name, "achieved": round(dom["GBps"], 2), "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": round(dom["GBps"] / HBM_PEAK_GBS, 5), "traffic": traffic,
+            "bytes_per_launch": round(dom["bytes_per_launch"], 1),
+            "us_per_launch": round(dom["us_per_launch"], 3),
+            "duration_source": "live: every library call of one traced frame replayed back to back from a HIP "
+                               "graph between two events on the stream it runs on, averaged over this kernel's "
+                               "launches (the committed rocprofv3 average includes the profiler's dispatch "
+                               "interception)",
+            "note": "latency-bound regime: the feature maps of this workload are <= 2.4 MB and "
+                    "an empty dependent kernel in a HIP graph already costs ~1.6 us"}
+    section("roofline", roofline_section)
+
+    # -- the CPU restatement of the same path on this host's cores (bounded sample) -----------
+    def cpu_section():
+        # 16 = the CPU share a one-GPU box grants one job here, whatever os.cpu_count() shows
+        threads = min(16, os.cpu_count() or 1)
+        n = max(1, args.cpu_frames)
+        clip = video if video.shape[0] > n else controlled_density_video(frames=n + 1, density=args.density)
+        d_fps, dn_fps = cpu_baseline(state, clip, n, threads)
+        result["cpu_baseline"] = {
+            "value": round(d_fps, 3), "unit": "frames/s", "cores": threads, "kind": "port",
+            "sample": f"{n} delta frames of the same synthetic video (same generator and seed) through the "
+                      f"fp32 CPU oracle (pure PyTorch layers) after the dense first frame",
+            "dense_cpu_fps": round(dn_fps, 3)}
+        log(f"CPU oracle: {d_fps:.1f} frames/s delta, {dn_fps:.1f} dense, {threads} threads")
+    if not args.no_cpu:
+        section("cpu_baseline", cpu_section)
+
+    dense_best = [None]
+
+    def dense_section():
+        dense_eager, dense_graph = run_dense(dense, frames, args.warmup, args.steps)
+        dense_best[0] = min(dense_eager, dense_graph)
+        log(f"dense GPU: eager {1 / dense_eager:.1f} fps, graph {1 / dense_graph:.1f} fps")
+        result["dense_gpu"] = {"eager_fps": round(1 / dense_eager, 1), "graph_fps": round(1 / dense_graph, 1),
+                               "speedup_vs_dense_gpu": round(dense_best[0] / sec, 3)}
+    section("dense_gpu", dense_section)
+    emit()
+
+    def sweep_section():
+        sweep = result["sweep"] = []
+        sw_steps, sw_warm = min(args.steps, 12 * UNROLL), min(args.warmup, 10)
+        for rho in SWEEP:
+            v = gpu_frames(controlled_density_video(frames=clip_frames(sw_steps, sw_warm), density=rho))
+            s = run_delta(delta, v, sw_warm, sw_steps, args.mode)
+            sweep.append({"density": rho, "fps": round(1.0 / s, 1), "ms_per_frame": round(s * 1e3, 4)})
+            if dense_best[0]:
+                sweep[-1]["speedup_vs_dense_gpu"] = round(dense_best[0] / s, 3)
+            log(f"  density {rho:4.2f}: {1 / s:9.1f} fps")
+    if not args.no_sweep:
+        section("sweep", sweep_section)
+
+    def logits_section():
+        with torch.no_grad():
+            ref_logits = dense(frames[-1:]).float()
+            delta.reset_layers()
+            for i in range(frames.shape[0]):
+                out = delta(frames[i:i + 1])
+            result["logit_max_abs_diff_vs_dense"] = round(float((out.float() - ref_logits).abs().max()), 4)
+            result["logit_max_abs"] = round(float(ref_logits.abs().max()), 4)
+    section("logits", logits_section)
+    emit()
+
+    if not args.no_micro:
+        def streams_section():
+            out = result["streams_as_batch"] = []
+            for nb in (8, 32):
+                out.append(streams_bench(delta, dense, batch=nb))
+                log(f"{nb} streams as a batch: delta {out[-1]['delta_fps_total']:.0f} frames/s in total, "
+                    f"dense graph {out[-1]['dense_graph_fps_total']:.0f}")
+            sw = result["streams_32_sweep"] = []
+            for rho in SWEEP:
+                sw.append(streams_bench(delta, dense, batch=32, steps=32, warmup=8, density=rho, with_dense=False))
+                log(f"  32 streams, density {rho:4.2f}: {sw[-1]['delta_fps_total']:9.0f} frames/s in total")
+        section("streams_as_batch", streams_section)
+
+        def micro_section():
+            log("single-layer sweeps (64x64 fp16):")
+            result["micro"] = micro_bench()
+        section("micro", micro_section)
+
+        def scaled_section():
+            log("scaled shapes (512x512, batch 8, C=64 fp16):")
+            result["scaled"] = scaled_bench()
+        section("scaled", scaled_section)
+        emit()
 
 
 if __name__ == "__main__":
