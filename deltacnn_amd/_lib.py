@@ -25,6 +25,21 @@ class Geometry(ctypes.Structure):
         "pad_right", "groups")]
 
 
+class BlockArgs(ctypes.Structure):
+    """struct dc_block_args."""
+    _fields_ = [
+        ("input", c_void_p), ("mask", c_void_p), ("dw_filter", c_void_p), ("dw_prev_out", c_void_p),
+        ("dw_truncated", c_void_p), ("dw_threshold", c_float), ("dw_activation", c_int32),
+        ("dw_truncation_mode", c_int32),
+        ("project_packed_filter", c_void_p), ("project_channels", c_int32), ("residual", c_void_p),
+        ("residual_mask", c_void_p), ("weight_residual", c_float), ("weight_conv", c_float),
+        ("out", c_void_p), ("out_mask", c_void_p),
+        ("expand_packed_filter", c_void_p), ("expand_channels", c_int32), ("expand_prev_out", c_void_p),
+        ("expand_truncated", c_void_p), ("expand_threshold", c_float), ("expand_activation", c_int32),
+        ("expand_truncation_mode", c_int32), ("expand_out", c_void_p), ("expand_out_mask", c_void_p),
+        ("flags", c_int32)]
+
+
 _P = c_void_p
 _G = POINTER(Geometry)
 _SIGNATURES = {
@@ -36,6 +51,7 @@ _SIGNATURES = {
     "dc_conv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),
     "dc_conv_act": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_float, c_int, c_int, c_int, _P]),
     "dc_conv_add": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, _P, c_float, c_float, _P, c_int, c_int, _P]),
+    "dc_block": (c_int, [_G, POINTER(BlockArgs), c_int, _P]),
     "dc_packed_filter_bytes": (c_int64, [_G, c_int, c_int]),
     "dc_pack_filter": (c_int, [_G, _P, _P, c_int, c_int, _P]),
     "dc_deconv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),

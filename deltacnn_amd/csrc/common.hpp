@@ -224,4 +224,12 @@ hipError_t launch_pool(const dc_geometry &g, const void *in, const void *prev, v
 // Whether a 1x1-output pooling of this shape can write its result in the tensor's own type.
 bool pool_global_casts(const dc_geometry &g, const void *in, const void *prev, int dtype);
 
+// Fused depthwise -> projection (-> expansion) block.  block_unsupported names the reason a
+// shape is outside the kernel's range (nullptr: supported as far as the shape check goes);
+// launch_block may still decline (*why != nullptr, nothing launched).
+const char *block_unsupported(const dc_geometry &g, const dc_block_args &b, int dtype);
+hipError_t launch_block(const dc_geometry &g, const dc_block_args &b, hipStream_t s, const char **why);
+// Reduction slices (KW) the stand-alone pointwise kernel uses for this layer.
+int pointwise_reduction_slices(int pixels, int in_c, int out_c);
+
 }  // namespace dc

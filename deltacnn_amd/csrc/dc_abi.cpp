@@ -374,6 +374,52 @@ int dc_densify(const void *delta, void *prev_out, void *out, const int32_t *mask
                                      (hipStream_t)stream), "dc_densify");
 }
 
+int dc_block(const dc_geometry *g, const dc_block_args *block, int dtype, void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_block");
+    int rc = check_geometry("dc_block", g, false, false);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_PTR("dc_block", block);
+    const dc_block_args &b = *block;
+    const char *why = dc::block_unsupported(*g, b, dtype);
+    if (why != nullptr) return fail(DC_ERR_UNSUPPORTED, "dc_block: %s", why);
+    DC_REQUIRE_PTR("dc_block", b.input);
+    DC_REQUIRE_PTR("dc_block", b.mask);
+    DC_REQUIRE_PTR("dc_block", b.dw_filter);
+    DC_REQUIRE_PTR("dc_block", b.dw_prev_out);
+    DC_REQUIRE_PTR("dc_block", b.dw_truncated);
+    DC_REQUIRE_PTR("dc_block", b.project_packed_filter);
+    DC_REQUIRE_PTR("dc_block", b.out);
+    DC_REQUIRE_PTR("dc_block", b.out_mask);
+    if (b.residual != nullptr) DC_REQUIRE_PTR("dc_block", b.residual_mask);
+    if (b.expand_channels > 0) {
+        DC_REQUIRE_PTR("dc_block", b.expand_packed_filter);
+        DC_REQUIRE_PTR("dc_block", b.expand_prev_out);
+        DC_REQUIRE_PTR("dc_block", b.expand_truncated);
+        DC_REQUIRE_PTR("dc_block", b.expand_out);
+        DC_REQUIRE_PTR("dc_block", b.expand_out_mask);
+    }
+    // 16-byte vectors on the depthwise side, 8-byte cells behind the matrix cores
+    DC_REQUIRE_ALIGNED("dc_block", b.input, 16);
+    DC_REQUIRE_ALIGNED("dc_block", b.dw_filter, 16);
+    DC_REQUIRE_ALIGNED("dc_block", b.dw_prev_out, 16);
+    DC_REQUIRE_ALIGNED("dc_block", b.dw_truncated, 16);
+    DC_REQUIRE_ALIGNED("dc_block", b.project_packed_filter, 16);
+    DC_REQUIRE_ALIGNED("dc_block", b.expand_packed_filter, 16);
+    DC_REQUIRE_ALIGNED("dc_block", b.residual, 8);
+    DC_REQUIRE_ALIGNED("dc_block", b.out, 8);
+    DC_REQUIRE_ALIGNED("dc_block", b.expand_prev_out, 8);
+    DC_REQUIRE_ALIGNED("dc_block", b.expand_truncated, 8);
+    DC_REQUIRE_ALIGNED("dc_block", b.expand_out, 8);
+    DC_REQUIRE_ALIGNED("dc_block", b.mask, 4);
+    DC_REQUIRE_ALIGNED("dc_block", b.out_mask, 4);
+    DC_REQUIRE_ALIGNED("dc_block", b.residual_mask, 4);
+    DC_REQUIRE_ALIGNED("dc_block", b.expand_out_mask, 4);
+    hipError_t e = dc::launch_block(*g, b, (hipStream_t)stream, &why);
+    if (e == hipSuccess && why != nullptr) return fail(DC_ERR_UNSUPPORTED, "dc_block: %s", why);
+    return finish(e, "dc_block");
+}
+
 int dc_add_to_dense(void *a, void *b, const int32_t *mask_a, int activation, int32_t pixels,
                     int32_t channels, int dtype, void *stream) {
     dc::kernel_log_reset();

@@ -570,8 +570,8 @@ concat_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ 
 // -------------------------------------------------------------------------------- mul_add
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
-mul_add_kernel(const T *__restrict__ in, const int32_t *__restrict__ mask, T *__restrict__ out,
-               int32_t *__restrict__ mo, const T *__restrict__ scale,
+mul_add_kernel(const T *in, const int32_t *mask, T *out,  // in == out, mask == mo when in place
+               int32_t *mo, const T *__restrict__ scale,
                const T *__restrict__ bias, int P, int C, int lg) {
     const int G = 1 << lg;
     int p, gl;

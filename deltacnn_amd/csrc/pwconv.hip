@@ -493,6 +493,22 @@ int pick_config(const PwP &p, int ksteps) {
     return 2;
 }
 
+int pointwise_reduction_slices(int pixels, int in_c, int out_c) {
+    PwP p;
+    p.P = pixels;
+    p.Ci = in_c;
+    p.Co = out_c;
+    p.ci_p = (in_c + 31) / 32 * 32;
+    p.co_tiles = ceil_div(out_c, 16);
+    p.xcd = p.nx = p.ny = 0;
+    const int cfg = pick_config(p, p.ci_p / 32);
+#define DC_PW_KW(ID, KW, CBW, NBW, R, NTW, EA) \
+    if (cfg == ID) return KW;
+    DC_PW_CONFIGS(DC_PW_KW)
+#undef DC_PW_KW
+    return 1;
+}
+
 hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *packed,
                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
                             const ActEpilogue *epi, bool *epilogue_done, const Residual *res,

@@ -6,6 +6,7 @@ synchronises.
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional, Sequence
 
 import torch
@@ -188,6 +189,49 @@ def sparse_conv_add(x, packed_filter, mask, bias, residual, mask_residual, geome
             return None
         raise
     return out, out_mask
+
+
+def sparse_block(x, mask, dw_filter, dw_geometry, dw_prev_out, dw_truncated, dw_threshold, dw_activation,
+                 project_packed, project_channels, out, out_mask, residual=None, residual_mask=None,
+                 weight_residual=1.0, weight_conv=1.0, expand=None, truncation_mode=0, late_loads=False):
+    """Depthwise 3x3 convolution + activation/truncation, 1x1 projection (+ residual sum) and,
+    with ``expand = (packed_filter, channels, prev_out, truncated, threshold, activation, out,
+    out_mask)``, the following 1x1 expansion + activation/truncation, in ONE launch (``dc_block``).
+    Identical to the separate calls bit for bit; the depthwise output is never stored.  Returns
+    ``False`` (nothing launched) for shapes the kernel does not take, so the caller can issue the
+    separate calls.  ``late_loads``: fetch operands only once the masks are known (for large,
+    mostly inactive maps; the default requests everything up front where the filters are small)."""
+    lib = _lib.load()
+    _nhwc(x, "x")
+    if x.dtype != torch.float16 or project_packed is None:
+        return False
+    a = _lib.BlockArgs()
+    a.flags = 1 if late_loads else 0
+    a.input, a.mask, a.dw_filter = x.data_ptr(), _mask(mask, "mask").data_ptr(), dw_filter.data_ptr()
+    a.dw_prev_out, a.dw_truncated = dw_prev_out.data_ptr(), dw_truncated.data_ptr()
+    a.dw_threshold, a.dw_activation, a.dw_truncation_mode = float(dw_threshold), int(dw_activation), int(truncation_mode)
+    a.project_packed_filter, a.project_channels = project_packed.data_ptr(), int(project_channels)
+    a.residual, a.residual_mask = _ptr(residual), _ptr(residual_mask)
+    a.weight_residual, a.weight_conv = float(weight_residual), float(weight_conv)
+    a.out, a.out_mask = out.data_ptr(), out_mask.data_ptr()
+    ex_mask, ce = None, 0
+    if expand is not None:
+        packed, ce, prev, trunc, thr, act, eout, ex_mask = expand
+        if packed is None:
+            return False
+        a.expand_packed_filter, a.expand_channels = packed.data_ptr(), int(ce)
+        a.expand_prev_out, a.expand_truncated = prev.data_ptr(), trunc.data_ptr()
+        a.expand_threshold, a.expand_activation, a.expand_truncation_mode = float(thr), int(act), int(truncation_mode)
+        a.expand_out, a.expand_out_mask = eout.data_ptr(), ex_mask.data_ptr()
+    meta = dict(g=dw_geometry, esize=2, in_mask=mask, in_mask_b=residual_mask, out_mask=out_mask, ex_mask=ex_mask,
+                Cp=int(project_channels), Ce=int(ce), keep=(a, x, dw_filter, project_packed, residual, expand))
+    try:
+        _call("block", lib.dc_block, (dw_geometry, ctypes.byref(a), DC_F16, _stream()), **meta)
+    except _lib.DeltaCNNError as e:
+        if e.code == -3:
+            return False
+        raise
+    return True
 
 
 def sparse_deconv(x, filter, mask=None, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),

@@ -182,15 +182,45 @@ class _InvertedResidual(nn.Module):
         layers.append(_ConvBNAct(L, hidden, hidden, stride=stride, groups=hidden, fold_bn=fold_bn))
         layers.append(_ConvBNAct(L, hidden, oup, kernel_size=1, fold_bn=fold_bn, act=None))
         self.conv = nn.Sequential(*layers)
+        self.has_expansion = expand_ratio != 1
 
-    def forward(self, x):
+    def _tail(self, x, hidden):
+        """Depthwise convolution and projection (+ residual sum) of the block, layer by layer;
+        ``hidden`` is the output of the expansion layer (the block input itself without one)."""
+        start = 1 if self.has_expansion else 0
         if not self.use_res_connect:
-            return self.conv(x)
+            return self.conv[start:](hidden)
         fused = getattr(self.sparse_add, "after_conv", None)
         if fused is None or len(self.conv[-1]) != 1:
-            return self.sparse_add(x, self.conv(x))
+            return self.sparse_add(x, self.conv[start:](hidden))
         # the layer namespace can add the residual inside the last convolution's kernel
-        return fused(x, self.conv[-1][0], self.conv[:-1](x))
+        return fused(x, self.conv[-1][0], self.conv[start:-1](hidden))
+
+    def forward(self, x):
+        return self._tail(x, self.conv[0](x) if self.has_expansion else x)
+
+    def single_layers(self):
+        """(expansion or None, depthwise, projection) when each is ONE layer (batch norm folded),
+        else None."""
+        if any(len(seq) != 1 for seq in self.conv):
+            return None
+        convs = [seq[0] for seq in self.conv]
+        return ([None] + convs) if not self.has_expansion else convs
+
+    def forward_ahead(self, x, expanded, fused_block, next_expansion):
+        """The block when a layer namespace offers ``fused_block``: ``expanded`` is this block's
+        expansion output if the previous block's launch already produced it; the block's own
+        launch runs the next block's expansion ahead in turn.  Returns (block output, expansion
+        output of the next block or None)."""
+        layers = self.single_layers()
+        if expanded is None:
+            expanded = self.conv[0](x) if self.has_expansion else x
+        if layers is not None:
+            add = self.sparse_add if self.use_res_connect else None
+            done = fused_block(expanded, layers[1], layers[2], add, x if add is not None else None, next_expansion)
+            if done is not None:
+                return done
+        return self._tail(x, expanded), None
 
 
 MOBILENET_V2_SETTING = [  # t, c, n, s  (example/mobilenet_deltacnn.py:160-170)
@@ -216,6 +246,8 @@ class MobileNetV2(_Net):
                 input_channel = output_channel
         features.append(_ConvBNAct(L, input_channel, self.last_channel, kernel_size=1, fold_bn=fold_bn))
         self.features = nn.Sequential(*features)
+        self._fused_block = getattr(L, "fused_block", None)
+        self.fuse_head = True
         self.sparsify = L.DCSparsify()
         self.densify = L.DCDensify()
         self.adaptive_avg_pooling = L.DCAdaptiveAveragePooling(output_size=(1, 1))
@@ -232,9 +264,29 @@ class MobileNetV2(_Net):
                 nn.init.normal_(m.weight, 0, 0.01)
                 nn.init.zeros_(m.bias)
 
+    def _features(self, x):
+        """``self.features(x)``; with a layer namespace that has ``fused_block``, every inverted
+        residual block runs as one launch that also carries the next block's expansion (or the
+        final 1x1 convolution)."""
+        fused_block = self._fused_block
+        if fused_block is None or isinstance(x, torch.Tensor):
+            return self.features(x)
+        stages = list(self.features)
+        x = stages[0](x)
+        expanded = None
+        for i in range(1, len(stages) - 1):
+            nxt = stages[i + 1]
+            if isinstance(nxt, _InvertedResidual):
+                layers = nxt.single_layers()
+                ahead = layers[0] if layers is not None else None
+            else:  # the final 1x1 convolution
+                ahead = nxt[0] if len(nxt) == 1 and self.fuse_head else None
+            x, expanded = stages[i].forward_ahead(x, expanded, fused_block, ahead)
+        return expanded if expanded is not None else stages[-1](x)
+
     def forward(self, x):
         x = self.sparsify(x)
-        x = self.features(x)
+        x = self._features(x)
         x = self.adaptive_avg_pooling(x)
         x = self.densify(x)
         x = x.reshape(x.shape[0], -1)

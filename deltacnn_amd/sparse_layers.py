@@ -19,6 +19,7 @@ from enum import Enum
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 from torch import Tensor
 
 from . import hip_kernels as hk
@@ -43,44 +44,61 @@ def convert_activation_string(name, **kwargs):
     raise Exception(f"Activation {name} not implemented")
 
 
-class DCBackend(Enum):
-    cudnn = 0
-    deltacnn = 1
-    delta_cudnn = 2
+class _NamedChoice:
+    """Enum mix-in: look a member up by its (case-insensitive) name."""
 
     @classmethod
-    def parse_string(cls, x):
-        try:
-            return cls[x.lower()]
-        except KeyError:
-            raise Exception(f"invalid backend {x}")
+    def parse_string(cls, text):
+        member = cls.__members__.get(str(text).lower())
+        if member is None:
+            raise Exception(f"invalid {cls.__name__} value {text!r}; one of {', '.join(cls.__members__)}")
+        return member
 
 
-class DCTruncation(Enum):
+class DCBackend(_NamedChoice, Enum):
+    """Which implementation a convolution layer runs (sparse_layers.py:64-75)."""
+    cudnn = 0        # dense torch layers
+    deltacnn = 1     # the delta kernels
+    delta_cudnn = 2  # the reference's training aid; not provided here
+
+
+class DCTruncation(_NamedChoice, Enum):
+    """How an activation layer decides that an update is too small to pass on
+    (sparse_layers.py:102-117)."""
     none = -1
     max = 0
     norm = 1
     rms = 2
 
-    @classmethod
-    def parse_string(cls, x):
-        try:
-            return cls[x.lower()]
-        except KeyError:
-            raise Exception(f"invalid truncation mode {x}")
+
+class _ThresholdFile:
+    """Per-layer thresholds on disk: one JSON object {"0": t0, "1": t1, ...} numbered in the
+    order the layers registered (the file format of the reference, sparse_layers.py:157-186)."""
+
+    def __init__(self, path):
+        self.path = path
+
+    def read(self):
+        with open(self.path) as f:
+            table = json.load(f)
+        return [table[str(i)] for i in range(len(table))]
+
+    def write(self, values):
+        with open(self.path, "w+") as f:
+            json.dump(dict(enumerate(values)), f)
 
 
 class DCThreshold:
     """Registry of per-layer thresholds keyed by module (sparse_layers.py:122-208).
 
-    Layers register their threshold on their first frame and look it up on every later
-    frame, so a JSON file loaded after frame 0 overrides the defaults.
+    A layer registers its threshold on its first frame (`set` never overwrites) and looks it
+    up on every later frame, so a file loaded after frame 0 overrides the defaults.
     """
-    t_default = 0.0
-    t = OrderedDict()
-    path = None
-    initialized = False
-    scale = 1.0
+    t = OrderedDict()    # layer -> threshold, in registration order
+    t_default = 0.0      # what a layer without a delta_threshold of its own registers
+    path = None          # JSON file for load_thresholds
+    scale = 1.0          # factor applied to the file's values
+    initialized = False  # load_thresholds has run since the last reset
 
     @classmethod
     def get(cls, key, default=0.0):
@@ -88,43 +106,42 @@ class DCThreshold:
 
     @classmethod
     def set(cls, key, val):
-        if key not in cls.t:
-            cls.t[key] = val
+        cls.t.setdefault(key, val)
 
     @classmethod
     def load_thresholds(cls):
-        if cls.initialized:
+        """Once per reset: overwrite the registered thresholds with `path`'s values times
+        `scale`.  File and registry are aligned at their ENDS: a shorter file describes the
+        layers registered last, a longer one loses its leading entries."""
+        already, cls.initialized = cls.initialized, True
+        if already or cls.path is None:
             return
-        cls.initialized = True
-        if cls.path is None:
-            return
-        with open(cls.path) as f:
-            thresholds = json.load(f)
-        if len(thresholds) != len(cls.t):
-            print(f"WARNING: thresholds file contains different number of thresholds. "
-                  f"file: {len(thresholds)} expected {len(cls.t)}")
-        skip = len(cls.t) - len(thresholds)
-        for i, key in enumerate(cls.t.keys()):
-            if i >= skip:
-                cls.t[key] = thresholds[str(i - skip)] * cls.scale
+        values = _ThresholdFile(cls.path).read()
+        layers = list(cls.t)
+        if len(values) != len(layers):
+            print(f"WARNING: {cls.path} holds {len(values)} thresholds, the model registered {len(layers)}")
+        for layer, value in zip(reversed(layers), reversed(values)):
+            cls.t[layer] = value * cls.scale
 
     @classmethod
     def save_thresholds(cls, name):
-        with open(f"thresholds_{name}.json", "w+") as f:
-            json.dump({i: v for i, v in enumerate(cls.t.values())}, f)
+        _ThresholdFile(f"thresholds_{name}.json").write(list(cls.t.values()))
 
     @classmethod
     def reset(cls):
+        """Forget every registered layer and the file."""
+        cls.path, cls.initialized = None, False
         cls.t.clear()
-        cls.initialized = False
-        cls.path = None
 
 
 class DCModule(nn.Module):
+    """Base of every stateful layer.  `temp_buffers` lists all cache tensors of all layers
+    (class level, sparse_layers.py:212), `reset_layers` returns a model to "no frame seen"."""
     temp_buffers = []
-    # Layers keep their output / mask buffers between frames instead of allocating per call
-    # (the reference allocates with torch.empty on every call, cuda_kernels.py:34-37).  A
-    # returned delta tensor is therefore valid until the same layer runs its next frame.
+    # Intermediate (delta, mask) outputs live in per-layer buffers that are reused frame after
+    # frame (the reference allocates with torch.empty on every call, cuda_kernels.py:34-37):
+    # a returned delta tuple is valid until the same layer runs its next frame.  Dense results
+    # (DCDensify, dense_out) are fresh tensors per call like in the reference.
     reuse_buffers = True
 
     def __init__(self):
@@ -132,33 +149,53 @@ class DCModule(nn.Module):
 
     @classmethod
     def get_temp_buffer_numel(cls):
-        return sum(x.numel() for x in cls.temp_buffers)
+        return sum(buf.numel() for buf in cls.temp_buffers)
+
+    @staticmethod
+    def _cache(tensor):
+        """Book a per-layer cache tensor in the class-level list and hand it back."""
+        DCModule.temp_buffers.append(tensor)
+        return tensor
+
+    def _take_index(self, owner):
+        """First frame of a layer: number it within `owner`, the class that holds the `idx`
+        counter of its kind."""
+        owner.idx += 1
+        self.idx = owner.idx
 
     def reset(self):
         DCModule.temp_buffers = []
 
     def process_filters(self):
-        for mod in list(self.modules()):
-            if type(mod) in [DCConv2d, DCConvTranspose2d]:
-                mod.process_filters()
+        for layer in self.modules():
+            if type(layer) in (DCConv2d, DCConvTranspose2d):
+                layer.process_filters()
 
     def reset_layers(self):
-        for module in self.modules():
-            if module is not self and isinstance(module, DCModule):
-                module.reset()
+        # nn.Module.modules() walks the whole tree and yields each module once
+        for layer in self.modules():
+            if layer is not self and isinstance(layer, DCModule):
+                layer.reset()
         DCModule.temp_buffers.clear()
 
 
+def _pair(v):
+    if isinstance(v, int):
+        return (v, v)
+    v = tuple(v)
+    return v + v if len(v) == 1 else v
+
+
 def to_tuple(*args):
-    result = []
-    for x in args:
-        if type(x) == int:
-            result.append((x, x))
-        elif len(x) == 1:
-            result.append((x[0], x[0]))
-        else:
-            result.append(tuple(x))
-    return result[0] if len(result) == 1 else result
+    """ints and 1-sequences become (v, v); longer sequences pass as tuples.  One argument
+    returns its pair, several return the list of pairs (sparse_layers.py:241-253)."""
+    pairs = [_pair(a) for a in args]
+    return pairs[0] if len(pairs) == 1 else pairs
+
+
+def _matches(buf, like) -> bool:
+    """A reusable buffer still fits: same shape, dtype and device as `like`."""
+    return buf is not None and buf.shape == like.shape and buf.dtype == like.dtype and buf.device == like.device
 
 
 def _is_depthwise(m) -> bool:
@@ -197,38 +234,59 @@ class _DeltaConvBase:
             "Leaky ReLU implementation uses hard coded negative slope of 0.1"
 
     def init_first_iter(self, input):
+        """First call: take the layer's number from the class-level call counter
+        (sparse_layers.py:341), note what kind of input arrives and register the threshold of a
+        fused activation."""
+        dense = isinstance(input, Tensor)
+        self.dense_in = dense
+        self.in_shape = (input if dense else input[0]).shape
         self.conv_idx = DCConv2d.conv_idx
-        self.dense_in = type(input) == Tensor
-        self.in_shape = input.shape if type(input) == Tensor else input[0].shape
-        if self.activation is not None and self.backend != DCBackend.cudnn:
+        if self.backend != DCBackend.cudnn and self.activation is not None:
             DCThreshold.set(self, self.delta_threshold)
 
     def forward(self, input):
+        # the class-level counter advances on every call of every convolution (:425); a layer
+        # is on its first frame while it has not copied a number from it yet (:427)
         DCConv2d.conv_idx += 1
         self.frame_idx += 1
-        first_iter = self.conv_idx == -1
+        first_iter = self.conv_idx < 0
         if first_iter:
             self.init_first_iter(input)
+        if self.backend == DCBackend.deltacnn:
+            return self._forward_delta_conv(input, first_iter)
         if self.backend == DCBackend.cudnn:
             return self._forward_dense(input)
-        if self.backend == DCBackend.delta_cudnn:
-            raise NotImplementedError("the delta_cudnn training backend is not part of this package")
-        return self._forward_delta_conv(input, first_iter)
+        raise NotImplementedError("the delta_cudnn training backend is not part of this package")
 
     def _forward_dense(self, input):
         out = self._conv_forward_dense(input)
         return self.activation(out) if self.activation is not None else out
 
-    def _make_plan(self, x):
+    def _make_plan(self, shape, dtype, device):
         pad = self.padding4 if getattr(self, "padding4", None) is not None else self.padding
         w = self.weight
-        g = hk.conv_geometry(x.shape, (w.shape[1], w.shape[2]), self.out_channels, self.stride, pad,
+        g = hk.conv_geometry(shape, (w.shape[1], w.shape[2]), self.out_channels, self.stride, pad,
                              self.dilation, self.groups, self._transposed)
-        plan = {"shape": tuple(x.shape), "dtype": x.dtype, "g": g, "out": None, "out_mask": None}
+        plan = {"shape": tuple(shape), "dtype": dtype, "g": g, "out": None, "out_mask": None}
         if DCModule.reuse_buffers:
-            plan["out"] = hk.new_features(g.batch, g.out_c, g.out_h, g.out_w, x.dtype, x.device)
-            plan["out_mask"] = hk.new_mask(g.batch, g.out_h, g.out_w, x.device)
+            plan["out"] = hk.new_features(g.batch, g.out_c, g.out_h, g.out_w, dtype, device)
+            plan["out_mask"] = hk.new_mask(g.batch, g.out_h, g.out_w, device)
         return plan
+
+    def _plan_for(self, shape, dtype, device):
+        """Geometry and reusable output buffers for an input of this shape."""
+        if self._plan is None or self._plan["shape"] != tuple(shape) or self._plan["dtype"] != dtype:
+            self._plan = self._make_plan(shape, dtype, device)
+            self.in_shape = torch.Size(shape)
+        return self._plan
+
+    def _packed_filter(self):
+        """The filter in matrix-core fragment order (made once), or None if it has no such form."""
+        if self._packed is None:
+            made = hk.pack_filter(self.weight.data, self.in_channels, self.out_channels, self.groups,
+                                  self._transposed)
+            self._packed = False if made is None else made
+        return None if self._packed is False else self._packed
 
     def _prepare(self, input):
         if type(input) == Tensor:
@@ -238,18 +296,10 @@ class _DeltaConvBase:
             raise RuntimeError("call process_filters() on the model (after moving it to the GPU "
                                "in channels_last) before the first frame")
         x, mask = input
-        if self._plan is None or self._plan["shape"] != tuple(x.shape) or self._plan["dtype"] != x.dtype:
-            self._plan = self._make_plan(x)
-            self.in_shape = x.shape
-        if self._packed is None:
-            self._packed = hk.pack_filter(self.weight.data, self.in_channels, self.out_channels,
-                                          self.groups, self._transposed)
-            if self._packed is None:
-                self._packed = False
-        packed = self._packed if self._packed is not False else None
+        plan = self._plan_for(x.shape, x.dtype, x.device)
         bias = self.bias if self.frame_idx <= 0 else None
         pad = self.padding4 if getattr(self, "padding4", None) is not None else self.padding
-        return x, mask, self._plan, packed, bias, pad
+        return x, mask, plan, self._packed_filter(), bias, pad
 
     def conv_delta(self, input):
         """The convolution alone: ``(delta, mask) -> (out, out_mask)`` without the layer's
@@ -282,39 +332,39 @@ class _DeltaConvBase:
 
     def reset(self):
         DCModule.reset(self)
-        self.frame_idx = -1
-        self.conv_idx = -1
-        self.prev_out = None
-        self.prev_in = None
-        self.out_shape = []
         DCConv2d.conv_idx = -1
-
-    def process_filters_half(self):
-        self.orig_weights = self.weight.data.clone()
-        result = self.half()
-        if self.backend == DCBackend.deltacnn:
-            result.weight.data = convert_half_filter(result.weight.data, pixel_wise=_is_depthwise(self),
-                                                     transposed=self._transposed)
-            self.filters_processed = True
-            self._packed = None
-        return result
-
-    def process_filters_single(self):
-        self.orig_weights = self.weight.data.clone()
-        if self.backend == DCBackend.deltacnn:
-            self.weight.data = convert_filter_out_channels_last(self.weight.data,
-                                                                transposed=self._transposed)
-            self.filters_processed = True
-            self._packed = None
-        return self
+        self.conv_idx = self.frame_idx = -1
+        self.prev_in = self.prev_out = None
+        self.out_shape = []
 
     def process_filters(self):
+        """Once per layer: move the weights into the layout the kernels read
+        (filter_conversion.py; sparse_layers.py:648-675).  The torch layout is kept in
+        ``orig_weights``; fp16 weights are padded to even channel counts and pair-swizzled,
+        fp32 weights become [Cin][Kh][Kw][Cout]."""
         if self.filters_processed:
             return
-        if self.weight.data.dtype == torch.float16:
-            self.process_filters_half()
-        else:
-            self.process_filters_single()
+        self.orig_weights = self.weight.data.clone()
+        half = self.weight.data.dtype == torch.float16
+        (self.process_filters_half if half else self.process_filters_single)()
+
+    def process_filters_half(self):
+        layer = self.half()
+        if self.backend == DCBackend.deltacnn:
+            layer.weight.data = convert_half_filter(layer.weight.data, pixel_wise=_is_depthwise(self),
+                                                    transposed=self._transposed)
+            self._filters_ready()
+        return layer
+
+    def process_filters_single(self):
+        if self.backend == DCBackend.deltacnn:
+            self.weight.data = convert_filter_out_channels_last(self.weight.data, transposed=self._transposed)
+            self._filters_ready()
+        return self
+
+    def _filters_ready(self):
+        self.filters_processed = True
+        self._packed = None
 
 
 class DCConv2d(_DeltaConvBase, nn.Conv2d, DCModule):
@@ -322,6 +372,12 @@ class DCConv2d(_DeltaConvBase, nn.Conv2d, DCModule):
     backend = DCBackend.deltacnn
     conv_idx = -1
     fuse_activation = True
+    fuse_blocks = True  # fused_block(): depthwise -> projection (-> expansion) in one launch
+    # ... while the two 1x1 filters together stay below this many bytes: every 16-pixel workgroup
+    # of that launch reads both in full, and one compute unit pulls only a few GB/s out of the
+    # far caches, so larger layers are faster as separate launches that spread their filter over
+    # many workgroups
+    fuse_blocks_max_filter_bytes = 32 << 10
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
                  groups=1, bias=True, padding_mode="zeros", delta_threshold=None, name=None,
@@ -365,52 +421,56 @@ class DCConvTranspose2d(_DeltaConvBase, nn.ConvTranspose2d, DCModule):
 
 
 class DCAdd(DCModule):
-    """Sum of two delta tensors with union mask (sparse_layers.py:1086-1182)."""
+    """Weighted sum of two delta tensors over the union of their masks, optionally followed by
+    an activation on the accumulated sum or by a dense output (sparse_layers.py:1086-1182)."""
     idx = -1
     fuse_into_conv = True
 
     def __init__(self, activation: str = None, dense_out=False, weight_a=None, weight_b=None, name=""):
         super().__init__()
-        self.name = name
-        self.dense_out = dense_out
         self.activation, self.activation_int = convert_activation_string(activation)
+        self.name, self.dense_out = name, dense_out
+        self.weight_a, self.weight_b = (1.0 if w is None else w for w in (weight_a, weight_b))
+        self._forget()
+
+    def _forget(self):
         self.idx = -1
-        self.prev_out = None
-        self.mask_out = None
-        self.out = None
-        self.weight_a = 1.0 if weight_a is None else weight_a
-        self.weight_b = 1.0 if weight_b is None else weight_b
         self.first_iter = True
+        self.prev_out = self.out = self.mask_out = None
+
+    def _needs_sum_cache(self):
+        """An activation or a dense output works on the accumulated sum of all frames."""
+        return self.dense_out or self.activation is not None
+
+    def _result_buffers(self, like, like_mask):
+        """(delta, mask) buffers for the result: per-layer and reused between frames, except the
+        dense_out result, which is a fresh tensor per call."""
+        if not DCModule.reuse_buffers:
+            return torch.empty_like(like), torch.empty_like(like_mask)
+        if not _matches(self.mask_out, like_mask):
+            self.mask_out = torch.empty_like(like_mask)
+        if self.dense_out:
+            return torch.empty_like(like), self.mask_out
+        if not _matches(self.out, like):
+            self.out = torch.empty_like(like)
+        return self.out, self.mask_out
 
     def forward(self, a, b, weight_a=None, weight_b=None):
-        w_a = self.weight_a if weight_a is None else weight_a
-        w_b = self.weight_b if weight_b is None else weight_b
-        if type(a) == Tensor:
-            c = w_a * a + w_b * b
-            return self.activation(c) if self.activation is not None else c
-        val_a, mask_a = a
-        val_b, mask_b = b
+        wa = self.weight_a if weight_a is None else weight_a
+        wb = self.weight_b if weight_b is None else weight_b
+        if isinstance(a, Tensor):  # dense operands: plain arithmetic
+            total = wa * a + wb * b
+            return total if self.activation is None else self.activation(total)
+        (delta_a, mask_a), (delta_b, mask_b) = a, b
         if self.first_iter:
             self.first_iter = False
-            DCAdd.idx += 1
-            self.idx = DCAdd.idx
-            if self.dense_out or self.activation is not None:
-                self.prev_out = torch.zeros_like(val_a)
-                DCModule.temp_buffers.append(self.prev_out)
-        if self.mask_out is None or self.mask_out.shape != mask_a.shape:
-            self.mask_out = torch.empty_like(mask_a)
-        if DCModule.reuse_buffers and not self.dense_out:
-            if self.out is None or self.out.shape != val_a.shape or self.out.dtype != val_a.dtype:
-                self.out = torch.empty_like(val_a)
-            out = self.out
-        else:
-            out = torch.empty_like(val_a)
-        mask_out = self.mask_out if DCModule.reuse_buffers else torch.empty_like(mask_a)
-        hk.sparse_add_tensors(val_a, val_b, self.prev_out, out, mask_a, mask_b, mask_out, w_a, w_b,
+            self._take_index(DCAdd)
+            if self._needs_sum_cache():
+                self.prev_out = self._cache(torch.zeros_like(delta_a))
+        out, mask_out = self._result_buffers(delta_a, mask_a)
+        hk.sparse_add_tensors(delta_a, delta_b, self.prev_out, out, mask_a, mask_b, mask_out, wa, wb,
                               self.activation_int, self.dense_out)
-        if self.dense_out:
-            return out
-        return out, mask_out
+        return out if self.dense_out else (out, mask_out)
 
     def after_conv(self, a, conv, conv_input):
         """``self(a, conv(conv_input))`` with the addition fused into the convolution's kernel
@@ -428,9 +488,9 @@ class DCAdd(DCModule):
             x, mask, plan, packed, _, _ = conv._prepare(conv_input)
             g = plan["g"]
             if packed is not None and tuple(val_a.shape) == (g.batch, g.out_c, g.out_h, g.out_w):
-                if self.out is None or self.out.shape != val_a.shape or self.out.dtype != val_a.dtype:
+                if not _matches(self.out, val_a):
                     self.out = torch.empty_like(val_a)
-                if self.mask_out is None or self.mask_out.shape != mask_a.shape:
+                if not _matches(self.mask_out, mask_a):
                     self.mask_out = torch.empty_like(mask_a)
                 res = hk.sparse_conv_add(x, packed, mask, None, val_a, mask_a, plan["g"], self.out,
                                          self.mask_out, self.weight_a, self.weight_b,
@@ -452,9 +512,9 @@ class DCAdd(DCModule):
             return self(a, upsample(b))
         val_a, mask_a = a
         val_b, mask_b = b
-        if self.out is None or self.out.shape != val_a.shape or self.out.dtype != val_a.dtype:
+        if not _matches(self.out, val_a):
             self.out = torch.empty_like(val_a)
-        if self.mask_out is None or self.mask_out.shape != mask_a.shape:
+        if not _matches(self.mask_out, mask_a):
             self.mask_out = torch.empty_like(mask_a)
         hk.sparse_add_upsampled(val_a, val_b, self.prev_out if self.activation is not None else None, self.out,
                                 mask_a, mask_b, self.mask_out, self.weight_a, self.weight_b,
@@ -463,12 +523,90 @@ class DCAdd(DCModule):
 
     def reset(self):
         super().reset()
-        self.idx = -1
-        self.mask_out = None
-        self.out = None
-        self.prev_out = None
-        self.first_iter = True
+        self._forget()
         DCAdd.idx = -1
+
+
+def _steady(conv) -> bool:
+    """A convolution layer of the delta backend that has seen its first frame (no bias from here
+    on) and owns processed fp16 filters."""
+    return (isinstance(conv, DCConv2d) and conv.backend == DCBackend.deltacnn and conv.frame_idx >= 0
+            and conv.filters_processed and conv.weight.dtype == torch.float16 and not conv.dense_out)
+
+
+def _steady_activation(conv):
+    """The convolution's fused activation layer if it can run inside another kernel: past its
+    first frame, in place, truncation mode max."""
+    act = conv.activation_layer
+    if act is None or act.first_iter or not act.inplace or act.truncation_mode != DCTruncation.max:
+        return None
+    return act
+
+
+def fused_block(dw_input, depthwise, project, add=None, residual=None, expand=None):
+    """One launch for ``depthwise`` (3x3 depthwise DCConv2d with activation) -> ``project`` (1x1
+    DCConv2d without activation) [-> ``add(residual, .)``, a DCAdd without activation]
+    [-> ``expand`` (1x1 DCConv2d with the same activation)], on frames after the first.
+
+    Returns ``(block_output, expanded)`` -- two ``(delta, mask)`` tuples, ``expanded`` is None
+    without ``expand`` -- exactly what the separate layer calls return, or ``None`` when the
+    layers are not in a state or of a shape the kernel takes; nothing has happened then and the
+    caller runs the layers one by one.  Switch: ``DCConv2d.fuse_blocks``."""
+    if not DCConv2d.fuse_blocks or isinstance(dw_input, Tensor):
+        return None
+    if not (_steady(depthwise) and _steady(project) and (expand is None or _steady(expand))):
+        return None
+    act_a = _steady_activation(depthwise)
+    if act_a is None or project.activation is not None or not _is_depthwise(depthwise):
+        return None
+    if add is not None and (add.first_iter or add.dense_out or add.activation is not None
+                            or residual is None or isinstance(residual, Tensor)):
+        return None
+    act_c = None
+    if expand is not None:
+        act_c = _steady_activation(expand)
+        if act_c is None or act_c.activation_int != act_a.activation_int:
+            return None
+    x, mask = dw_input
+    if x.dtype != torch.float16 or depthwise.padding4 is not None:
+        return None
+    filter_bytes = 2 * project.out_channels * (project.in_channels + (expand.out_channels if expand is not None else 0))
+    if filter_bytes > DCConv2d.fuse_blocks_max_filter_bytes:
+        return None
+    plan_a = depthwise._plan_for(x.shape, x.dtype, x.device)
+    g = plan_a["g"]
+    hidden_shape = (g.batch, g.out_c, g.out_h, g.out_w)
+    plan_b = project._plan_for(hidden_shape, x.dtype, x.device)
+    if plan_b["out"] is None or (project.kernel_size, project.stride, project.padding) != ((1, 1), (1, 1), (0, 0)):
+        return None
+    out, out_mask = plan_b["out"], plan_b["out_mask"]
+    res_delta = res_mask = None
+    if add is not None:
+        res_delta, res_mask = residual
+        if tuple(res_delta.shape) != tuple(out.shape):
+            return None
+        if not _matches(add.out, res_delta):
+            add.out = torch.empty_like(res_delta)
+        if not _matches(add.mask_out, res_mask):
+            add.mask_out = torch.empty_like(res_mask)
+        out, out_mask = add.out, add.mask_out
+    ex = None
+    if expand is not None:
+        plan_c = expand._plan_for(out.shape, x.dtype, x.device)
+        if plan_c["out"] is None or (expand.kernel_size, expand.stride, expand.padding) != ((1, 1), (1, 1), (0, 0)):
+            return None
+        ex = (expand._packed_filter(), expand.out_channels, act_c.prev_out, act_c.out_truncated,
+              DCThreshold.get(act_c), act_c.activation_int, plan_c["out"], plan_c["out_mask"])
+    done = hk.sparse_block(x, mask, depthwise.weight, g, act_a.prev_out, act_a.out_truncated,
+                           DCThreshold.get(act_a), act_a.activation_int, project._packed_filter(),
+                           project.out_channels, out, out_mask, res_delta, res_mask,
+                           add.weight_a if add is not None else 1.0, add.weight_b if add is not None else 1.0, ex)
+    if not done:
+        return None
+    for conv in (depthwise, project) + ((expand,) if expand is not None else ()):
+        DCConv2d.conv_idx += 1  # what the layers' own forward calls would have counted
+        conv.frame_idx += 1
+    return (out, out_mask), ((ex[6], ex[7]) if ex is not None else None)
 
 
 class DCConcatenate(DCModule):
@@ -498,125 +636,126 @@ class DCConcatenate(DCModule):
 
 class DCSparsify(DCModule):
     """Dense frame -> (delta, mask) against the cached accumulated input
-    (sparse_layers.py:1197-1273)."""
+    (sparse_layers.py:1197-1273).  With ``dilation > 1`` the per-pixel test is replaced by a
+    torch expression over a dilation x dilation neighbourhood (:1233-1244)."""
     idx = -1
 
     def __init__(self, name="", delta_threshold=None, dilation=-1):
         super().__init__()
         self.name = name
-        self.prev_in = None
-        self.idx = -1
-        self.delta_threshold = delta_threshold if delta_threshold is not None else DCThreshold.t_default
         self.dilation = dilation
+        self.delta_threshold = DCThreshold.t_default if delta_threshold is None else delta_threshold
+        self._forget()
+
+    def _forget(self):
+        self.idx = -1
         self.frame_idx = -1
+        self.prev_in = None
         self.mask = None
         self.delta = None
+
+    def _first_frame(self, frame):
+        """Everything is new: the frame itself is the delta, every pixel is active."""
+        DCThreshold.set(self, self.delta_threshold)
+        self._take_index(DCSparsify)
+        self.prev_in = self._cache(frame.clone())
+        b, _, h, w = frame.shape
+        return frame, torch.ones((b, 1, h, w), dtype=torch.int32, device=frame.device)
+
+    def _neighbourhood_delta(self, frame, threshold):
+        k = self.dilation
+        delta = frame - self.prev_in
+        peak = F.max_pool2d(delta.abs().amax(dim=1, keepdim=True), k, stride=1, padding=(k - 1) // 2)
+        active = peak > threshold
+        self.prev_in = torch.where(active, frame, self.prev_in)
+        return delta, active.to(torch.int32)
 
     def forward(self, input):
         if DCConv2d.backend != DCBackend.deltacnn:
             return input
-        first_iter = self.idx == -1
         self.frame_idx += 1
-        if first_iter:
-            if self not in DCThreshold.t:
-                DCThreshold.set(self, self.delta_threshold)
-            DCSparsify.idx += 1
-            self.idx = DCSparsify.idx
-            self.prev_in = input.clone()
-            DCModule.temp_buffers.append(self.prev_in)
-            return input, torch.ones_like(input[:, :1], dtype=torch.int)
+        if self.idx < 0:
+            return self._first_frame(input)
         threshold = DCThreshold.get(self)
         if self.dilation > 1:
-            x = input - self.prev_in
-            mask = torch.max(torch.abs(x), dim=1, keepdim=True)[0]
-            k = self.dilation
-            mask = torch.max_pool2d(mask, (k, k), stride=(1, 1), padding=((k - 1) // 2, (k - 1) // 2)) > threshold
-            self.prev_in = torch.where(mask, input, self.prev_in)
-            return x, mask.int()
-        if self.mask is None or self.mask.shape[2:] != input.shape[2:] or self.mask.shape[0] != input.shape[0]:
-            self.mask = torch.empty_like(input[:, :1], dtype=torch.int)
-        if DCModule.reuse_buffers:
-            if self.delta is None or self.delta.shape != input.shape or self.delta.dtype != input.dtype:
-                self.delta = torch.empty_like(input)
-            x = self.delta
+            return self._neighbourhood_delta(input, threshold)
+        b, _, h, w = input.shape
+        if self.mask is None or self.mask.shape != (b, 1, h, w) or self.mask.device != input.device:
+            self.mask = hk.new_mask(b, h, w, input.device)
+        if not DCModule.reuse_buffers:
+            delta = torch.empty_like(input)
         else:
-            x = torch.empty_like(input)
-        hk.sparsify(input, self.prev_in, x, self.mask, threshold)
-        return x, self.mask
+            if not _matches(self.delta, input):
+                self.delta = torch.empty_like(input)
+            delta = self.delta
+        hk.sparsify(input, self.prev_in, delta, self.mask, threshold)
+        return delta, self.mask
 
     def reset(self):
         super().reset()
-        self.idx = -1
-        self.frame_idx = -1
-        self.prev_in = None
-        self.mask = None
-        self.delta = None
+        self._forget()
         DCSparsify.idx = -1
 
 
 class DCDensify(DCModule):
-    """(delta, mask) -> dense accumulated tensor (sparse_layers.py:1276-1333)."""
+    """(delta, mask) -> dense accumulated tensor (sparse_layers.py:1276-1333).  With
+    ``clone_out`` (default) every call returns a NEW tensor, so results collected over frames
+    stay distinct; ``clone_out=False`` returns the accumulator itself."""
     idx = -1
 
     def __init__(self, activation: str = None, name="", clone_out=True):
         super().__init__()
         self.name = name
         self.activation, self.activation_int = convert_activation_string(activation)
-        self.prev_out = None
-        self.out = None
-        self.idx = -1
         self.clone_out = clone_out
+        self.prev_out = None
+        self.idx = -1
 
     def forward(self, input):
-        if type(input) == Tensor:
+        if isinstance(input, Tensor):
             return input
-        input, mask = input
-        if self.prev_out is None:
-            DCDensify.idx += 1
-            self.idx = DCDensify.idx
-            self.prev_out = torch.zeros_like(input)
-            DCModule.temp_buffers.append(self.prev_out)
-        if self.clone_out:  # accumulate and copy in one launch
-            out = self.out if DCModule.reuse_buffers and self.out is not None else torch.empty_like(self.prev_out)
-            if DCModule.reuse_buffers:
-                self.out = out
-            hk.densify(input, self.prev_out, out, mask)
+        delta, mask = input
+        if self.prev_out is None or not _matches(self.prev_out, delta):
+            if self.prev_out is None:
+                self._take_index(DCDensify)
+            self.prev_out = self._cache(torch.zeros_like(delta))  # bias arrives with the frame-0 delta
+        if self.clone_out:
+            dense = torch.empty_like(self.prev_out)
+            hk.densify(delta, self.prev_out, dense, mask)  # accumulate and copy in one launch
         else:
-            hk.sparse_activation(input, self.prev_out, None, mask, -1, -1, DCTruncation.none.value)
-            out = self.prev_out
-        if self.activation is not None:
-            return self.activation(out)
-        return out
+            hk.sparse_activation(delta, self.prev_out, None, mask, -1, -1, DCTruncation.none.value)
+            dense = self.prev_out
+        return dense if self.activation is None else self.activation(dense)
 
     def reset(self):
         super().reset()
         self.prev_out = None
-        self.out = None
 
 
 class DCUpsamplingNearest2d(DCModule):
-    """Nearest upsampling by an integer factor (sparse_layers.py:1336-1359)."""
+    """Nearest upsampling by an integer factor (sparse_layers.py:1336-1359): an updated pixel
+    updates its scale x scale copies."""
     idx = -1
 
     def __init__(self, scale_factor=2, name=""):
         super().__init__()
-        self.name = name
         self.scale_factor = int(scale_factor)
+        self.torch_upsample = nn.UpsamplingNearest2d(scale_factor=scale_factor)
+        self.name = name
         self.idx = -1
         self.out = None
-        self.torch_upsample = nn.UpsamplingNearest2d(scale_factor=scale_factor)
 
     def forward(self, input):
-        if type(input) == Tensor:
+        if isinstance(input, Tensor):
             return self.torch_upsample(input)
-        val, mask = input
-        if self.out is not None and (self.out[0].shape[0] != val.shape[0]
-                                     or self.out[0].shape[1] != val.shape[1]
-                                     or self.out[0].shape[2] != val.shape[2] * self.scale_factor
-                                     or self.out[0].shape[3] != val.shape[3] * self.scale_factor
-                                     or self.out[0].dtype != val.dtype):
-            self.out = None
-        self.out = hk.sparse_upsample(val, mask, self.scale_factor, self.out)
+        delta, mask = input
+        b, c, h, w = delta.shape
+        k = self.scale_factor
+        if self.out is not None:
+            have = self.out[0]
+            if have.shape != (b, c, h * k, w * k) or have.dtype != delta.dtype or have.device != delta.device:
+                self.out = None
+        self.out = hk.sparse_upsample(delta, mask, k, self.out)
         return self.out
 
     def reset(self):
@@ -626,86 +765,90 @@ class DCUpsamplingNearest2d(DCModule):
 
 class DCActivation(DCModule):
     """Non-linearity on accumulated values with truncation of small updates
-    (sparse_layers.py:1362-1425)."""
+    (sparse_layers.py:1362-1425).  State: ``prev_out`` = accumulated pre-activation values,
+    ``out_truncated`` = updates withheld so far."""
     idx = -1
     truncation_default = DCTruncation.max
 
     def __init__(self, name="", inplace=True, delta_threshold=None, activation="relu",
                  truncation_mode: DCTruncation = None):
         super().__init__()
-        self.name = name
-        self.idx = -1
-        self.prev_out = None
-        self.inplace = inplace
-        self.out_truncated = None
         self.activation, self.activation_int = convert_activation_string(activation)
         if self.activation is None:
             raise ValueError("DCActivation needs a non-linear activation")
-        self.delta_threshold = delta_threshold if delta_threshold is not None else DCThreshold.t_default
+        self.name = name
+        self.inplace = inplace
+        self.delta_threshold = DCThreshold.t_default if delta_threshold is None else delta_threshold
+        self.truncation_mode = DCActivation.truncation_default if truncation_mode is None else truncation_mode
+        self.idx = -1
+        self._forget()
+
+    def _forget(self):
         self.first_iter = True
-        self.truncation_mode = truncation_mode if truncation_mode is not None else DCActivation.truncation_default
+        self.prev_out = None
+        self.out_truncated = None
+
+    def _first_frame(self, values, mask):
+        """Dense frame: remember the pre-activation values, nothing withheld yet; the mask
+        passes through untouched."""
+        self.first_iter = False
+        DCThreshold.set(self, self.delta_threshold)
+        if self.idx < 0:
+            self._take_index(DCActivation)
+        self.prev_out = self._cache(values.clone())
+        self.out_truncated = self._cache(torch.zeros_like(values))
+        return self.activation(values), mask
 
     def forward(self, input):
-        if type(input) == Tensor:
+        if isinstance(input, Tensor):
             return self.activation(input)
-        val, mask = input
+        values, mask = input
         if self.first_iter:
-            self.first_iter = False
-            if self not in DCThreshold.t:
-                DCThreshold.set(self, self.delta_threshold)
-            if self.idx < 0:
-                DCActivation.idx += 1
-                self.idx = DCActivation.idx
-            self.prev_out = val.clone()
-            self.out_truncated = torch.zeros_like(val)
-            DCModule.temp_buffers.append(self.prev_out)
-            DCModule.temp_buffers.append(self.out_truncated)
-            return self.activation(val), mask
-        threshold = DCThreshold.get(self)
+            return self._first_frame(values, mask)
         if not self.inplace:
-            val = val.clone()
-            mask = mask.clone()
-        hk.sparse_activation(val, self.prev_out, self.out_truncated, mask, threshold,
+            values, mask = values.clone(), mask.clone()
+        hk.sparse_activation(values, self.prev_out, self.out_truncated, mask, DCThreshold.get(self),
                              self.activation_int, self.truncation_mode.value)
-        return val, mask
+        return values, mask
 
     def reset(self):
         super().reset()
         self.idx = -1
-        self.prev_out = None
-        self.out_truncated = None
-        self.first_iter = True
+        self._forget()
         DCActivation.idx = -1
 
 
 class DCMaxPooling(nn.MaxPool2d, DCModule):
-    """Delta max pooling; caches the accumulated input (sparse_layers.py:1428-1474)."""
+    """Delta max pooling; caches the accumulated input (sparse_layers.py:1428-1474).
+    ``padding`` may be a pair or (left, right, top, bottom) as torch.nn.functional.pad takes it
+    (:1439-1441)."""
 
     def __init__(self, kernel_size, stride=(1, 1), padding=(0, 0), dilation=(1, 1)):
         kernel_size, stride, padding, dilation = to_tuple(kernel_size, stride, padding, dilation)
         nn.MaxPool2d.__init__(self, kernel_size, stride=stride, padding=padding, dilation=dilation)
-        self.first_iter = True
         self.out_shape = []
+        self.first_iter = True
         self.prev_in = None
 
+    def _dense(self, x):
+        """Plain tensors: torch pooling; four-sided padding is applied beforehand (zeros, as the
+        reference pads) and the window then runs unpadded."""
+        pad = self.padding
+        if len(pad) == 4:
+            x, pad = F.pad(x, pad), 0
+        return F.max_pool2d(x, self.kernel_size, self.stride, pad, self.dilation, self.ceil_mode)
+
     def forward(self, input):
-        if type(input) == Tensor:
-            old_padding = self.padding
-            if len(self.padding) == 4:
-                input = torch.nn.functional.pad(input, self.padding)
-                self.padding = 0
-            out = nn.MaxPool2d.forward(self, input)
-            self.padding = old_padding
-            return out
-        x, mask = input
+        if isinstance(input, Tensor):
+            return self._dense(input)
+        delta, mask = input
         if self.first_iter:
             self.first_iter = False
-            self.prev_in = torch.zeros_like(x)
-            DCModule.temp_buffers.append(self.prev_in)
-        out = hk.sparse_pooling(x, self.prev_in, self.kernel_size, mask, self.stride, self.padding,
-                                self.dilation, create_out_mask=True, pooling_mode_int=0)
-        hk.sparse_add_to_dense_tensor(x, self.prev_in, mask)
-        return out
+            self.prev_in = self._cache(torch.zeros_like(delta))
+        pooled = hk.sparse_pooling(delta, self.prev_in, self.kernel_size, mask, self.stride, self.padding,
+                                   self.dilation, create_out_mask=True, pooling_mode_int=0)
+        hk.sparse_add_to_dense_tensor(delta, self.prev_in, mask)  # the cache follows the input
+        return pooled
 
     def reset(self):
         DCModule.reset(self)
@@ -714,26 +857,29 @@ class DCMaxPooling(nn.MaxPool2d, DCModule):
 
 
 class DCAdaptiveAveragePooling(nn.AdaptiveAvgPool2d, DCModule):
-    """Global average pooling of deltas (sparse_layers.py:1477-1513); output size 1x1 only."""
+    """Global average pooling of deltas (sparse_layers.py:1477-1513): the mean is linear, so the
+    delta of the mean is the mean of the deltas and no cache is needed.  Output size 1x1 only."""
 
     def __init__(self, output_size=None):
         output_size = to_tuple(output_size)
         nn.AdaptiveAvgPool2d.__init__(self, output_size=output_size)
-        self.first_iter = True
         self.out_shape = output_size
+        self.first_iter = True
         self.prev_in = None
 
     def get_target_size(self, input):
-        assert self.output_size[0] == 1 and self.output_size[1] == 1
+        """(window, stride, padding, dilation) of the pooling call that produces one pixel."""
+        if tuple(self.output_size) != (1, 1):
+            raise AssertionError("only output_size 1x1 is supported on delta tensors")
         return tuple(input.shape[2:]), (1, 1), (0, 0), (1, 1)
 
     def forward(self, input):
-        if type(input) == Tensor:
+        if isinstance(input, Tensor):
             return nn.AdaptiveAvgPool2d.forward(self, input)
-        x, mask = input
+        delta, mask = input
         self.first_iter = False
-        kernel_size, stride, padding, dilation = self.get_target_size(x)
-        return hk.sparse_pooling(x, None, kernel_size, mask, stride, padding, dilation,
+        window, stride, padding, dilation = self.get_target_size(delta)
+        return hk.sparse_pooling(delta, None, window, mask, stride, padding, dilation,
                                  create_out_mask=True, pooling_mode_int=1)
 
     def reset(self):
@@ -743,47 +889,41 @@ class DCAdaptiveAveragePooling(nn.AdaptiveAvgPool2d, DCModule):
 
 
 class DCBatchNorm2d(nn.BatchNorm2d, DCModule):
-    """Inference batch norm on deltas: scale on every frame, offset on the first only
-    (sparse_layers.py:1516-1585)."""
+    """Inference batch norm on deltas (sparse_layers.py:1516-1585).  y = x * scale + offset is
+    affine: a delta only needs the scale, the offset enters once with the first frame (and on
+    every dense tensor)."""
 
     def __init__(self, num_features, eps=1e-5, momentum=0.1, affine=True,
                  track_running_stats=True, inplace=True):
         nn.BatchNorm2d.__init__(self, num_features, eps, momentum, affine, track_running_stats)
-        self.first_iter = True
-        self.scale = None
-        self.offset = None
         self.inplace = inplace
+        self.first_iter = True
+        self.scale = self.offset = None
 
-    def convert_to_scale_offset(self, input):
-        bn_scale = self.weight * torch.rsqrt(self.running_var + self.eps)
-        self.scale = bn_scale[None, :, None, None]
-        self.offset = (-self.running_mean * bn_scale + self.bias)[None, :, None, None]
+    def convert_to_scale_offset(self, input=None):
+        """Fold running statistics and affine parameters into per-channel scale and offset,
+        shaped [1, C, 1, 1]."""
+        inv_std = torch.rsqrt(self.running_var + self.eps)
+        gain = self.weight * inv_std
+        shift = self.bias - self.running_mean * gain
+        self.scale, self.offset = gain.view(1, -1, 1, 1), shift.view(1, -1, 1, 1)
 
     def forward(self, input):
-        use_offset = False
-        mask = None
-        dense = True
-        if type(input) == tuple:
-            input, mask = input
-            dense = False
-        else:
-            use_offset = True
-        if self.first_iter:
-            self.first_iter = False
-            use_offset = True
-            self.convert_to_scale_offset(input)
-        if dense:
+        is_delta = isinstance(input, tuple)
+        first, self.first_iter = self.first_iter, False
+        if first:
+            self.convert_to_scale_offset()
+        with_offset = first or not is_delta
+        if not is_delta:
             out = input.mul_(self.scale) if self.inplace else input * self.scale
-            if use_offset:
-                out.add_(self.offset)
-            return out
-        bias = self.offset if use_offset else None
+            return out.add_(self.offset) if with_offset else out
+        delta, mask = input
+        shift = self.offset if with_offset else None
         if self.inplace:
-            hk.sparse_mul_add(input, mask, input, mask, self.scale, bias)
-            return input, mask
-        out = torch.empty_like(input)
-        out_mask = mask.clone()
-        hk.sparse_mul_add(input, mask, out, out_mask, self.scale, bias)
+            out, out_mask = delta, mask
+        else:
+            out, out_mask = torch.empty_like(delta), mask.clone()
+        hk.sparse_mul_add(delta, mask, out, out_mask, self.scale, shift)
         return out, out_mask
 
     def reset(self):

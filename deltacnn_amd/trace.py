@@ -20,6 +20,16 @@ m = 4-byte mask word, P pixels, n_x = number of active pixels of mask x):
   upsample           R = P*m + n*C*s                      W = S*S*(n*C*s + P*m)
   concat             R = 2*P*m + (n_a*Ca + n_b*Cb)*s      W = n_out*(Ca+Cb)*s + P*m
   mul_add            R = P*m + n*C*s + C*s                W = n*C*s
+  block              (depthwise 3x3 + activation -> projection (+ residual) -> expansion + activation in
+                     one launch; Ch hidden, Cp projection, Ce expansion channels; n_mid = updated
+                     depthwise outputs before truncation, n_out / n_ex = pixels of the block output /
+                     expansion output mask; the hidden mask is never stored, so the depthwise layer's
+                     kept pixels are counted as min(n_mid, n_out))
+                     R = P_in*m + n_in*Ch*s + 9*Ch*s + n_mid*2*Ch*s + Ch*Cp*s [+ P*m + n_res*Cp*s]
+                         [+ Cp*Ce*s + n_out*2*Ce*s]
+                     W = n_keep*2*Ch*s + (n_mid-n_keep)*Ch*s + n_out*Cp*s + P*m
+                         [+ n_ex*3*Ce*s + (n_out-n_ex)*Ce*s + P*m]
+                     flops = 2*9*Ch*n_mid (as tap pairs) + 2*Ch*Cp*n_keep + 2*Cp*Ce*n_out
 """
 from __future__ import annotations
 
@@ -46,7 +56,7 @@ class Tracer:
         rec = {"op": op, "meta": meta}
         rec["n_in"] = self._count(meta.get("in_mask"))
         rec["n_in_b"] = self._count(meta.get("in_mask_b"))
-        if self.count_pairs and op in ("conv", "deconv", "conv_act", "conv_add"):
+        if self.count_pairs and op in ("conv", "deconv", "conv_act", "conv_add", "block"):
             rec["pairs"], rec["n_mid"] = self._pairs(meta["g"], meta["in_mask"], op == "deconv")
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
@@ -57,6 +67,7 @@ class Tracer:
         rec["events"] = (start, end)
         rec["kernels"] = _lib.load().dc_last_kernels().decode().split("+")
         rec["n_out"] = self._count(meta.get("out_mask"))
+        rec["n_ex"] = self._count(meta.get("ex_mask"))
         rec["call"] = (fn, args)
         self.records.append(rec)
         return rc
@@ -176,6 +187,24 @@ class Tracer:
                     extra = {"kernel": r["kernels"][1], "call": op, "shape": f"C{C} P{p_out}", "ms": t_act * 1e-3,
                              "bytes": p_out * m + n_mid * 3 * C * s + n_out * 3 * C * s + (n_mid - n_out) * (C * s + m),
                              "flops": 0, "density_in": n_mid / p_out, "density_out": n_out / p_out}
+            elif op == "block":
+                g = meta["g"]
+                ch, cp, ce = g.in_c, meta["Cp"], meta["Ce"]
+                p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
+                n_mid = int(r["n_mid"]) if "n_mid" in r else n_out
+                n_keep = min(n_mid, n_out)
+                rd = p_in * m + n_in * ch * s + 9 * ch * s + n_mid * 2 * ch * s + ch * cp * s
+                wr = n_keep * 2 * ch * s + (n_mid - n_keep) * ch * s + n_out * cp * s + p_out * m
+                if n_in_b is not None:
+                    rd += p_out * m + n_in_b * cp * s
+                flops = 2 * ch * cp * n_keep + (2 * ch * int(r["pairs"]) if "pairs" in r else 0)
+                if ce:
+                    n_ex = int(r["n_ex"])
+                    rd += cp * ce * s + n_out * 2 * ce * s
+                    wr += n_ex * 3 * ce * s + (n_out - n_ex) * ce * s + p_out * m
+                    flops += 2 * cp * ce * n_out
+                shape = f"dw{ch} s{g.stride_h} -> {cp} -> {ce} @{g.out_h}x{g.out_w}"
+                dens = (n_in / p_in, n_out / p_out)
             elif op == "pool":
                 g = meta["g"]
                 p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w

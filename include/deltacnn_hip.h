@@ -126,6 +126,60 @@ int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filt
                 const int32_t *mask_residual, void *out, int32_t *out_mask, float weight_residual,
                 float weight_conv, void *prev_out, int activation, int dtype, void *stream);
 
+/* Operands of dc_block beyond the depthwise geometry.  Feature pointers are fp16 NHWC; the
+ * packed filters come from dc_pack_filter (1x1 geometry of that convolution). */
+typedef struct dc_block_args {
+    /* A: depthwise 3x3 convolution (geometry argument) + activation/truncation */
+    const void *input;              /* [B][in_h][in_w][C] delta */
+    const int32_t *mask;            /* its update mask */
+    const void *dw_filter;          /* reference depthwise layout [3][3][C] */
+    void *dw_prev_out;              /* activation state [B][out_h][out_w][C], in place */
+    void *dw_truncated;
+    float dw_threshold;
+    int32_t dw_activation;          /* DC_ACT_RELU / RELU6 / LEAKY */
+    int32_t dw_truncation_mode;     /* DC_TRUNC_MAX */
+    /* B: 1x1 projection C -> project_channels (+ residual sum, a DCAdd without activation) */
+    const void *project_packed_filter;
+    int32_t project_channels;
+    const void *residual;           /* [P][project_channels] delta or NULL */
+    const int32_t *residual_mask;   /* required with residual */
+    float weight_residual, weight_conv;
+    void *out;                      /* [P][project_channels], written where out_mask is 1 */
+    int32_t *out_mask;              /* [P], written for every pixel */
+    /* C (expand_channels > 0): 1x1 expansion project_channels -> expand_channels + activation/truncation */
+    const void *expand_packed_filter;
+    int32_t expand_channels;
+    void *expand_prev_out;          /* [P][expand_channels], in place */
+    void *expand_truncated;
+    float expand_threshold;
+    int32_t expand_activation;      /* must equal dw_activation */
+    int32_t expand_truncation_mode; /* DC_TRUNC_MAX */
+    void *expand_out;               /* [P][expand_channels], written where expand_out_mask is 1 */
+    int32_t *expand_out_mask;       /* [P], written for every pixel */
+    int32_t flags;                  /* DC_BLOCK_* bits */
+} dc_block_args;
+
+/* dc_block_args.flags.  By default layers with small filters request every operand before the
+ * update masks are known (one memory round trip; what was fetched for inactive pixels is
+ * dropped): right for small batches, which are bound by latency.  DC_BLOCK_LATE_LOADS fetches
+ * only what active pixels need, one round trip later: right when the maps are large and mostly
+ * inactive.  Results do not depend on it. */
+enum { DC_BLOCK_LATE_LOADS = 1 };
+
+/* The layers between two spatial convolutions of an inverted-residual network in ONE launch:
+ * depthwise 3x3 convolution + activation/truncation, 1x1 projection (+ residual sum) and,
+ * optionally, the next block's 1x1 expansion + activation/truncation.  `g` describes the
+ * depthwise convolution (groups == in_c == out_c); P = batch * out_h * out_w.  Neither the
+ * depthwise output nor, on its way into the expansion, the block output passes through memory.
+ * Results (all outputs, masks and layer states) are identical, bit for bit, to
+ * dc_conv_act(depthwise) -> dc_conv / dc_conv_add(projection) -> dc_conv_act(expansion), none
+ * of them with a bias (a layer's bias belongs to its first frame, which takes the separate
+ * calls).  fp16 only.  Shapes outside the kernel's range (see dc_last_error) return
+ * DC_ERR_UNSUPPORTED before any launch so that the caller can issue the separate calls.  No
+ * counterpart in the reference, which launches every layer and every activation on its own
+ * (sparse_layers.py:636-638). */
+int dc_block(const dc_geometry *g, const dc_block_args *block, int dtype, void *stream);
+
 /* Number of bytes dc_pack_filter writes for this geometry (0 if the shape has no packed
  * form).  One-time weight relayout for the MFMA kernels, fp16, un-swizzled, in fragment order
  * [Cout tile of 16][Kh][Kw][Cin step of 32][lane 0..63][8] (lane kq*16+r holds input channels

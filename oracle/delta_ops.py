@@ -17,28 +17,37 @@ Conventions
 
 Paths are relative to the reference tree (``src/cuda/...``, ``src/deltacnn/...``).
 
-Pinning status (what fixes each function besides re-reading the source)
+Pinning status (what fixes each function besides re-reading the source; tests are in
+tests/test_oracle_pins.py unless another file is named)
 ----------------------------------------------------------------------
-sparsify            witness ``sparse_layers.py:1250-1255`` (amax|x-prev| > thr) as a
-                    library expression + cache invariants; the fp16 even-C ``>=``
-                    tie rule (``other_nn_layers.cu:1289``) is source-derived only:
+activation          ids 1-3: scalar loops (test_activate_truncate_against_loops); ids 4/5:
+                    torch.sigmoid / F.silu (test_sigmoid_and_swish_against_library).  The
+                    reference's fp16 ``hexp``/``hrcp`` rounding is source-derived only:
+                    parity unpinned for the last fp16 ulp of sigmoid / swish.
+sparsify            loops (test_sparsify_against_loops) + cache invariants; the fp16 even-C
+                    ``>=`` tie rule (``other_nn_layers.cu:1289``) is source-derived only:
                     parity unpinned for that tie case.
-activate_truncate   witness ``differentiable_threshold(mode="clamp")``
-                    ``sparse_layers.py:44-54`` + conservation invariant
-                    prev + trunc == running pre-activation; modes norm/rms:
-                    parity unpinned (lane-order float sums in the reference).
-                    sigmoid/swish in fp16: parity unpinned (``hexp``/``hrcp``).
-conv / deconv       ``F.conv2d`` / ``F.conv_transpose2d`` on zero-filled deltas,
-                    brute-force loops on tiny inputs; mask = dilation closed form
-                    (same formula as ``utils.py:123-134``).  The fp16 rounding
-                    sequence of the reference accumulation (``conv_kernel.cu:1390``)
-                    cannot be run: parity unpinned beyond the 2e-2 tolerance.
-pooling             witness ``sparse_layers.py:1452-1454`` (max) and linearity
-                    (avg); asymmetric-padding zero quirk is source-derived only:
-                    parity unpinned for that quirk.  Global max follows the
-                    windowed definition, not the reference's per-block atomicMax.
-add / densify       witnesses ``sparse_layers.py:1140-1165`` / ``:1311-1320``.
-upsample / concat / mul_add   library routines (repeat_interleave, cat, affine).
+sparsify_dilated    window loops (test_sparsify_dilated_against_window_loops).
+activate_truncate   mode max: loops + conservation invariant prev + trunc == running
+                    pre-activation; modes norm / rms: loops away from ties
+                    (test_norm_rms_truncation_against_loops; at a tie the reference's
+                    lane-order sum in the tensor's type decides: parity unpinned there);
+                    mode < 0 with an activation: telescoping sum
+                    (test_accumulate_with_activation_telescopes).
+conv / deconv       brute-force loops on tiny inputs, all 2^9 3x3 mask patterns, frame sums =
+                    dense conv.  The fp16 rounding sequence of the reference accumulation
+                    (``conv_kernel.cu:1390``) cannot be run: parity unpinned beyond the 2e-2
+                    tolerance.  deconv with dilation / groups: library call only (the
+                    reference has no such path).
+pool                loops incl. dilation (test_pool_against_loops,
+                    test_pool_with_dilation_against_loops_and_library) and library pooling;
+                    the asymmetric-padding zero quirk is source-derived only: parity
+                    unpinned for that quirk.  Global max follows the windowed definition,
+                    not the reference's per-block atomicMax.
+add                 loops (test_add_against_loops), dense-sum tracking with activation,
+                    dense_out by indexing (test_add_dense_out_against_indexing).
+add_to_dense        indexing loops (test_add_to_dense_against_indexing).
+upsample / concat / mul_add   indexing (test_upsample_concat_mul_add_against_indexing).
 """
 from __future__ import annotations
 
@@ -116,7 +125,8 @@ def sparsify_dilated(x, prev, threshold: float, dilation: int):
     """Torch-side option of DCSparsify, sparse_layers.py:1233-1244."""
     d = x - prev
     a = d.abs().amax(dim=1, keepdim=True)
-    m = F.max_pool2d(a.float(), dilation, stride=1, padding=(dilation - 1) // 2) > threshold
+    # a tensor compared with a Python number is compared in the tensor's type
+    m = F.max_pool2d(a.float(), dilation, stride=1, padding=(dilation - 1) // 2) > float(_scalar(threshold, x))
     prev.copy_(torch.where(m, x, prev))
     return torch.where(m, d, torch.zeros_like(d)), m.to(torch.int32)
 
@@ -208,7 +218,9 @@ def deconv(delta: torch.Tensor, mask: torch.Tensor, weight: torch.Tensor,
     """Delta transposed convolution, deconv_kernel.cu:296-336,460-481.
 
     ``weight`` is in torch layout ``[Cin, Cout/g, Kh, Kw]``; output size ignores
-    ``output_padding`` (cuda_kernels.py:56-57).
+    ``output_padding`` (cuda_kernels.py:56-57).  Pinned by scatter loops for dilation 1 and
+    one group (all the reference supports, deconv_kernel.cu:857); with dilation or groups this
+    is the library call alone, there is no reference behaviour to match.
     """
     x = torch.where(_active(mask), delta, torch.zeros_like(delta)).float()
     out = F.conv_transpose2d(x, weight.float(), None if bias is None else bias.float(),
@@ -286,8 +298,11 @@ def pool(delta: torch.Tensor, prev: Optional[torch.Tensor], mask: torch.Tensor, 
 
 
 def add_to_dense(a: torch.Tensor, b: torch.Tensor, mask_a: torch.Tensor, act: int = 0) -> None:
-    """``b[px] += a[px]`` on active pixels, other_nn_layers.cu:1731-1957."""
+    """``b[px] += a[px]`` on active pixels, other_nn_layers.cu:1731-1957; with ``act > 0``
+    (the USE_ACTIVATION variant) ``a`` additionally becomes ``act(b)`` on every pixel."""
     b.copy_(torch.where(_active(mask_a), b + a, b))
+    if act > 0:
+        a.copy_(activation(b, act))
 
 
 # ------------------------------------------------------------------------------- add

@@ -147,16 +147,16 @@ def activate_truncate(delta, prev, trunc, mask, thr, act):
     return delta, prev, trunc, mask
 
 
-def pool(delta, prev, mask, kernel, stride, padding, mode):
+def pool(delta, prev, mask, kernel, stride, padding, mode, dilation=(1, 1)):
     """Delta pooling over in-bounds window pixels (src/cuda/other_nn_layers.cu:2390-2459).
     mode 0 (max): max_w(prev + M*delta) - max_w(prev); with asymmetric padding a literal 0
     joins both maxima for window positions beyond the bottom (right) edge when
     top != bottom (left != right) (:2404-2406, :2418-2420).
-    mode 1 (avg): sum_w(M*delta) / (Kh*Kw) (:2456)."""
+    mode 1 (avg): sum_w(M*delta) / (Kh*Kw) (:2456).  Window taps are `dilation` pixels apart."""
     B, C, H, W = delta.shape
     t, b, l, r = pad4(padding)
-    Ho = conv_out_size(H, kernel[0], stride[0], t, b, 1)
-    Wo = conv_out_size(W, kernel[1], stride[1], l, r, 1)
+    Ho = conv_out_size(H, kernel[0], stride[0], t, b, dilation[0])
+    Wo = conv_out_size(W, kernel[1], stride[1], l, r, dilation[1])
     out = np.zeros((B, C, Ho, Wo), np.float64)
     om = np.zeros((B, 1, Ho, Wo), np.int32)
     for n in range(B):
@@ -167,7 +167,7 @@ def pool(delta, prev, mask, kernel, stride, padding, mode):
                 sm = np.zeros(C)
                 hit = False
                 for ky in range(kernel[0]):
-                    iy = oy * stride[0] - t + ky
+                    iy = oy * stride[0] - t + ky * dilation[0]
                     if iy < 0:
                         continue
                     if iy >= H:  # one zero per padded bottom row, whatever the column
@@ -176,7 +176,7 @@ def pool(delta, prev, mask, kernel, stride, padding, mode):
                             hp = np.maximum(hp, 0.0)
                         continue
                     for kx in range(kernel[1]):
-                        ix = ox * stride[1] - l + kx
+                        ix = ox * stride[1] - l + kx * dilation[1]
                         if ix < 0:
                             continue
                         if ix >= W:
@@ -218,3 +218,99 @@ def add(a, mask_a, b, mask_b, wa, wb):
                         s = dt(np.float64(b[n, c, y, x]) * np.float64(dt(wb)) + np.float64(s))
                     out[n, c, y, x] = s
     return out, om
+
+
+def activate_truncate_sum(delta, prev, trunc, mask, thr, act, mode):
+    """Modes `norm` (1) and `rms` (2) (src/cuda/other_nn_layers.cu:664-719): as mode `max`, but a
+    pixel is kept when sqrt(sum_c D_c^2) > thr, resp. sqrt(sum_c D_c^2 / C) > thr.  T, S and D
+    round in the tensor's type; the sum of squares is taken in float64 here (the reference adds
+    in lane order in the tensor's type), so inputs must keep the statistic away from thr.
+    Returns new (delta, prev, trunc, mask) and the per-pixel statistic."""
+    B, C, H, W = delta.shape
+    dt = delta.dtype.type
+    delta, prev, trunc, mask = delta.copy(), prev.copy(), trunc.copy(), mask.copy()
+    stat = np.full((B, 1, H, W), np.nan)
+    for n in range(B):
+        for y in range(H):
+            for x in range(W):
+                if mask[n, 0, y, x] == 0:
+                    continue
+                T, S, D = (np.zeros(C, delta.dtype) for _ in range(3))
+                total = 0.0
+                for c in range(C):
+                    T[c] = dt(trunc[n, c, y, x] + delta[n, c, y, x])
+                    S[c] = dt(T[c] + prev[n, c, y, x])
+                    D[c] = dt(_act(S[c], act) - _act(prev[n, c, y, x], act))
+                    total += float(D[c]) * float(D[c])
+                value = np.sqrt(total) if mode == 1 else np.sqrt(total / C)
+                stat[n, 0, y, x] = value
+                if value > thr:
+                    prev[n, :, y, x] = S
+                    delta[n, :, y, x] = D
+                    trunc[n, :, y, x] = 0
+                else:
+                    trunc[n, :, y, x] = T
+                    mask[n, 0, y, x] = 0
+    return delta, prev, trunc, mask, stat
+
+
+def sparsify_neighbourhood(x, prev, thr, k):
+    """DCSparsify's `dilation` option (src/deltacnn/sparse_layers.py:1233-1244): a pixel is
+    active when the largest |x - prev| over all channels of any pixel of the k x k window
+    around it (window offset (k-1)//2 up/left, out-of-image positions ignored) exceeds thr.
+    The delta is x - prev on EVERY pixel; the cache takes x on active pixels.
+    Returns (delta, mask, new_prev)."""
+    B, C, H, W = x.shape
+    delta = (x - prev).astype(x.dtype)
+    peak = np.abs(delta).max(axis=1)
+    mask = np.zeros((B, 1, H, W), np.int32)
+    new_prev = prev.copy()
+    off = (k - 1) // 2
+    # torch's max_pool2d output size for stride 1, padding off: H + 2*off - k + 1
+    Ho, Wo = H + 2 * off - k + 1, W + 2 * off - k + 1
+    for n in range(B):
+        for y in range(Ho):
+            for xx in range(Wo):
+                best = -np.inf
+                for dy in range(k):
+                    for dx in range(k):
+                        yy, xc = y - off + dy, xx - off + dx
+                        if 0 <= yy < H and 0 <= xc < W:
+                            best = max(best, float(peak[n, yy, xc]))
+                if best > thr:
+                    mask[n, 0, y, xx] = 1
+                    new_prev[n, :, y, xx] = x[n, :, y, xx]
+    return delta, mask, new_prev
+
+
+def add_dense_out(a, mask_a, b, mask_b, prev, wa, wb, act):
+    """DCAdd with dense_out (src/deltacnn/sparse_layers.py:1140-1172): the accumulated sum takes
+    wa*a where Ma and wb*b where Mb; the result is act(accumulated sum) on EVERY pixel.
+    float64 arithmetic.  Returns (dense result, new accumulated sum)."""
+    B, C, H, W = a.shape
+    new_prev = prev.astype(np.float64).copy()
+    for n in range(B):
+        for y in range(H):
+            for x in range(W):
+                if mask_a[n, 0, y, x] != 0:
+                    new_prev[n, :, y, x] += wa * a[n, :, y, x].astype(np.float64)
+                if mask_b[n, 0, y, x] != 0:
+                    new_prev[n, :, y, x] += wb * b[n, :, y, x].astype(np.float64)
+    out = np.empty_like(new_prev)
+    for idx in np.ndindex(*new_prev.shape):
+        out[idx] = _act(np.float64(new_prev[idx]), act)
+    return out, new_prev
+
+
+def add_to_dense(a, b, mask_a):
+    """src/cuda/other_nn_layers.cu:1731-1957: b[pixel] += a[pixel] where the mask is set, b
+    untouched elsewhere (rounded in the tensor's type).  Returns the new b."""
+    out = b.copy()
+    B, C, H, W = a.shape
+    for n in range(B):
+        for y in range(H):
+            for x in range(W):
+                if mask_a[n, 0, y, x] != 0:
+                    for c in range(C):
+                        out[n, c, y, x] = a.dtype.type(b[n, c, y, x] + a[n, c, y, x])
+    return out

@@ -1,0 +1,247 @@
+"""dc_block (depthwise 3x3 + activation/truncation -> 1x1 projection (+ residual sum) -> 1x1
+expansion + activation/truncation in one launch) against
+
+  * the separate library calls on the same operands: every output, mask and layer state equal
+    bit for bit (the kernel repeats their arithmetic operation for operation), and
+  * the CPU oracle chained the same way: masks equal except where a truncation decision sits
+    within one fp16 step of the threshold (counted and bounded), values within 2e-2 absolute on
+    pixels both agree on.
+"""
+import pytest
+import torch
+
+from oracle import delta_ops as ops
+from util import DEV, cl, poison, rand_mask
+
+pytestmark = pytest.mark.gpu
+
+THR = 0.05
+RELU6 = 2
+
+# hidden, project, expand (0: none), H, W, stride, residual, density
+CASES = [
+    (32, 16, 96, 20, 23, 1, False, 0.3),     # 4 lanes per pixel, one wavefront per workgroup
+    (64, 24, 0, 17, 9, 1, False, 0.5),       # 8 lanes per pixel, no expansion
+    (96, 24, 144, 30, 31, 2, False, 0.2),    # stride 2, partial channel tile (24 = 16 + 8)
+    (144, 24, 144, 28, 28, 1, True, 0.1),    # residual sum; 144 = 4.5 reduction steps
+    (192, 32, 192, 28, 28, 1, True, 0.05),
+    (192, 64, 384, 29, 27, 2, False, 0.3),
+    (384, 64, 384, 14, 14, 1, True, 0.3),    # reduction split over 4 wavefronts (12 steps)
+    (384, 96, 576, 14, 14, 1, False, 1.0),
+    (576, 96, 576, 14, 14, 1, True, 0.2),    # two vectors per lane, 18 steps in 4 slices
+    (576, 160, 960, 15, 13, 2, False, 0.4),
+    (960, 160, 960, 7, 7, 1, True, 0.5),     # 30 steps in 8 slices, 10 projection tiles
+    (960, 320, 1280, 7, 7, 1, False, 1.0),   # two passes of projection tiles, 80 expansion tiles
+    (960, 160, 0, 7, 7, 1, True, 0.02),      # hardly anything active
+    (128, 40, 200, 11, 50, 1, True, 0.3),    # channel counts off the tile grid (40 = 2.5 tiles, 200 = 12.5)
+]
+
+
+def _case(cfg, seed, batch=2):
+    from deltacnn_amd import hip_kernels as hk
+    from deltacnn_amd.filter_conversion import convert_half_filter
+    ch, cp, ce, H, W, stride, residual, density = cfg
+    g = torch.Generator().manual_seed(seed)
+    geo = hk.conv_geometry((batch, ch, H, W), (3, 3), ch, (stride, stride), (1, 1), (1, 1), ch)
+    Ho, Wo = geo.out_h, geo.out_w
+    c = {"cfg": cfg, "geo": geo}
+    c["mask"] = rand_mask(g, batch, H, W, density)
+    c["x"] = (torch.randn(batch, ch, H, W, generator=g) * 0.5).half()
+    c["w_dw"] = (torch.randn(ch, 1, 3, 3, generator=g) / 3).half()
+    c["w_pj"] = (torch.randn(cp, ch, 1, 1, generator=g) / ch ** 0.5).half()
+    c["prev_a"] = torch.randn(batch, ch, Ho, Wo, generator=g).half()
+    c["trunc_a"] = (torch.randn(batch, ch, Ho, Wo, generator=g) * 0.02).half()
+    if residual:
+        c["res"] = (torch.randn(batch, cp, Ho, Wo, generator=g) * 0.3).half()
+        c["res_mask"] = rand_mask(g, batch, Ho, Wo, density)
+    if ce:
+        c["w_ex"] = (torch.randn(ce, cp, 1, 1, generator=g) / cp ** 0.5).half()
+        c["prev_c"] = torch.randn(batch, ce, Ho, Wo, generator=g).half()
+        c["trunc_c"] = (torch.randn(batch, ce, Ho, Wo, generator=g) * 0.02).half()
+    c["f_dw"] = convert_half_filter(c["w_dw"], pixel_wise=True).to(DEV)
+    c["f_pj"] = convert_half_filter(c["w_pj"]).to(DEV)
+    c["p_pj"] = hk.pack_filter(c["f_pj"], ch, cp, 1)
+    if ce:
+        c["f_ex"] = convert_half_filter(c["w_ex"]).to(DEV)
+        c["p_ex"] = hk.pack_filter(c["f_ex"], cp, ce, 1)
+    return c
+
+
+def _device_state(c):
+    """Fresh device copies of everything a run modifies or reads (NaN at inactive input pixels)."""
+    d = {"x": cl(poison(c["x"], c["mask"])), "mask": cl(c["mask"]),
+         "prev_a": cl(c["prev_a"]), "trunc_a": cl(c["trunc_a"])}
+    if "res" in c:
+        d["res"], d["res_mask"] = cl(poison(c["res"], c["res_mask"])), cl(c["res_mask"])
+    if "w_ex" in c:
+        d["prev_c"], d["trunc_c"] = cl(c["prev_c"]), cl(c["trunc_c"])
+    return d
+
+
+def _run_separate(c, d):
+    from deltacnn_amd import hip_kernels as hk
+    ch, cp, ce, H, W, stride, residual, density = c["cfg"]
+    hid, hid_mask = hk.sparse_conv_activation(d["x"], c["f_dw"], d["mask"], None, d["prev_a"], d["trunc_a"], THR, RELU6,
+                                              0, (stride, stride), (1, 1), (1, 1), ch, ch)
+    if residual:
+        out, out_mask = hk.sparse_conv(hid, c["f_pj"], hid_mask, None, (1, 1), (0, 0), (1, 1), 1, c_out=cp,
+                                       create_out_mask=True, packed_filter=c["p_pj"])
+        summed, sum_mask = torch.empty_like(out), torch.empty_like(out_mask)
+        hk.sparse_add_tensors(d["res"], out, None, summed, d["res_mask"], out_mask, sum_mask, 1.0, 1.0, 0, False)
+        out, out_mask = summed, sum_mask
+    else:
+        out, out_mask = hk.sparse_conv(hid, c["f_pj"], hid_mask, None, (1, 1), (0, 0), (1, 1), 1, c_out=cp,
+                                       create_out_mask=True, packed_filter=c["p_pj"])
+    res = {"out": out, "out_mask": out_mask}
+    if ce:
+        eo, em = hk.sparse_conv_activation(out, c["f_ex"], out_mask, None, d["prev_c"], d["trunc_c"], THR, RELU6, 0,
+                                           (1, 1), (0, 0), (1, 1), 1, ce, packed_filter=c["p_ex"])
+        res["eout"], res["eout_mask"] = eo, em
+    return res
+
+
+def _run_fused(c, d, late_loads=False):
+    from deltacnn_amd import hip_kernels as hk
+    ch, cp, ce, H, W, stride, residual, density = c["cfg"]
+    geo = c["geo"]
+    B, Ho, Wo = geo.batch, geo.out_h, geo.out_w
+    nan = float("nan")
+    out = torch.full((B, cp, Ho, Wo), nan, dtype=torch.half, device=DEV).contiguous(memory_format=torch.channels_last)
+    out_mask = torch.full((B, 1, Ho, Wo), -7, dtype=torch.int32, device=DEV)
+    expand = None
+    res = {"out": out, "out_mask": out_mask}
+    if ce:
+        eo = torch.full((B, ce, Ho, Wo), nan, dtype=torch.half, device=DEV).contiguous(memory_format=torch.channels_last)
+        em = torch.full((B, 1, Ho, Wo), -7, dtype=torch.int32, device=DEV)
+        expand = (c["p_ex"], ce, d["prev_c"], d["trunc_c"], THR, RELU6, eo, em)
+        res["eout"], res["eout_mask"] = eo, em
+    done = hk.sparse_block(d["x"], d["mask"], c["f_dw"], geo, d["prev_a"], d["trunc_a"], THR, RELU6, c["p_pj"], cp,
+                           out, out_mask, d.get("res"), d.get("res_mask"), 1.0, 1.0, expand, late_loads=late_loads)
+    assert done, "the kernel declined a shape of its own test"
+    return res
+
+
+def _equal_on(a, b, mask, what):
+    m = (mask != 0).expand_as(a)
+    assert torch.equal(a[m], b[m]), f"{what}: {int((a[m] != b[m]).sum())} of {int(m.sum())} active values differ"
+
+
+# the shapes of CASES small enough for the form that requests every operand up front
+EAGER = {(32, 16, 96), (64, 24, 0), (96, 24, 144), (144, 24, 144), (192, 32, 192)}
+
+
+@pytest.mark.parametrize("late_loads", [False, True], ids=["default", "late_loads"])
+@pytest.mark.parametrize("cfg", CASES, ids=lambda c: "-".join(str(v) for v in c))
+def test_block_equals_separate_calls(lib, cfg, late_loads):
+    from deltacnn_amd import _lib
+    c = _case(cfg, 5000 + cfg[0] + cfg[1])
+    ds, df = _device_state(c), _device_state(c)
+    want = _run_separate(c, ds)
+    got = _run_fused(c, df, late_loads)
+    eager = tuple(cfg[:3]) in EAGER and not late_loads
+    assert _lib.load().dc_last_kernels().decode() == ("block_eager_kernel" if eager else "block_dw_pw_kernel")
+    assert torch.equal(got["out_mask"], want["out_mask"])
+    _equal_on(got["out"], want["out"], want["out_mask"], "block output")
+    for k in ("prev_a", "trunc_a"):
+        assert torch.equal(df[k], ds[k]), f"depthwise activation state {k}"
+    if cfg[2]:
+        assert torch.equal(got["eout_mask"], want["eout_mask"])
+        _equal_on(got["eout"], want["eout"], want["eout_mask"], "expansion output")
+        for k in ("prev_c", "trunc_c"):
+            assert torch.equal(df[k], ds[k]), f"expansion activation state {k}"
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("cfg", [CASES[3], CASES[5], CASES[8], CASES[10]], ids=lambda c: "-".join(str(v) for v in c))
+def test_block_against_oracle_chain(lib, cfg):
+    """The same chain through the CPU oracle.  A convolution output differs from the oracle's in
+    its last fp16 bit now and then, which can flip a truncation decision that sits on the
+    threshold; such pixels are counted (and must be rare), everything else has to agree."""
+    ch, cp, ce, H, W, stride, residual, density = cfg
+    c = _case(cfg, 6000 + ch)
+    got = _run_fused(c, _device_state(c))
+    hid, hm = ops.conv(c["x"], c["mask"], c["w_dw"], None, (stride, stride), (1, 1), (1, 1), ch)
+    prev_a, trunc_a = c["prev_a"].clone(), c["trunc_a"].clone()
+    hm = hm.clone()
+    ops.activate_truncate(hid, prev_a, trunc_a, hm, THR, RELU6, 0)
+    out, om = ops.conv(hid, hm, c["w_pj"])
+    if residual:
+        out, om = ops.add(c["res"], c["res_mask"], out, om, None)
+    flips = int((got["out_mask"].cpu() != om).sum())
+    both = (got["out_mask"].cpu() != 0) & (om != 0)
+    zero = torch.zeros(())
+    err = torch.where(both, (got["out"].cpu().float() - out.float()).abs(), zero).max()
+    assert flips <= max(2, om.numel() // 200), f"{flips} of {om.numel()} block output mask words differ"
+    print(f"block output: {flips} mask words of {om.numel()} differ, max |diff| on common pixels {float(err):.4f}")
+    # a flipped decision upstream changes what reaches a pixel; compare only where the hidden masks agree
+    if flips == 0:
+        assert float(err) <= 2e-2
+        if ce:
+            eo, em = ops.conv(out, om, c["w_ex"])
+            prev_c, trunc_c = c["prev_c"].clone(), c["trunc_c"].clone()
+            em = em.clone()
+            ops.activate_truncate(eo, prev_c, trunc_c, em, THR, RELU6, 0)
+            eflips = int((got["eout_mask"].cpu() != em).sum())
+            assert eflips <= max(2, em.numel() // 200), f"{eflips} expansion mask words differ"
+            both = (got["eout_mask"].cpu() != 0) & (em != 0)
+            assert float(torch.where(both, (got["eout"].cpu().float() - eo.float()).abs(), zero).max()) <= 2e-2
+
+
+def test_block_declines_what_it_cannot_do(lib):
+    from deltacnn_amd import hip_kernels as hk
+    c = _case((64, 24, 0, 9, 9, 1, False, 0.5), 1)
+    d = _device_state(c)
+    geo = c["geo"]
+    out = torch.empty(2, 24, 9, 9, dtype=torch.half, device=DEV).contiguous(memory_format=torch.channels_last)
+    om = torch.empty(2, 1, 9, 9, dtype=torch.int32, device=DEV)
+    # norm truncation has no fused form: nothing is launched, the caller takes the separate calls
+    assert hk.sparse_block(d["x"], d["mask"], c["f_dw"], geo, d["prev_a"], d["trunc_a"], THR, RELU6, c["p_pj"], 24,
+                           out, om, truncation_mode=1) is False
+    assert hk.sparse_block(d["x"], d["mask"], c["f_dw"], geo, d["prev_a"], d["trunc_a"], THR, 4, c["p_pj"], 24,
+                           out, om) is False  # sigmoid
+
+
+def test_mobilenet_block_fusion_keeps_every_layer_state(lib):
+    """MobileNetV2 224x224, 6 frames: the model that runs one launch per block against the model
+    that issues every layer call on its own -- logits, every activation layer's cached state and
+    every layer's last output mask equal bit for bit."""
+    from deltacnn_amd import sparse_layers as SL
+    from deltacnn_amd.video import moving_rectangles_video
+    from test_gpu_network import _calibrated_state, _mobilenet, _two_hip_models
+    video = moving_rectangles_video(frames=6, height=224, width=224, n_rect=3, min_size=16, max_size=60)
+    small = moving_rectangles_video(frames=3, height=64, width=96, n_rect=2, min_size=8, max_size=24)
+    from deltacnn_amd import hip_kernels as hk
+    fused, plain = _two_hip_models(_mobilenet, _calibrated_state(small))
+    launches = []
+    original = hk.sparse_block
+
+    def counted(*a, **k):
+        done = original(*a, **k)
+        launches.append(done)
+        return done
+    hk.sparse_block = counted
+    limit = SL.DCConv2d.fuse_blocks_max_filter_bytes
+    SL.DCConv2d.fuse_blocks_max_filter_bytes = 1 << 30  # every block, whatever its filter size
+    try:
+        with torch.no_grad():
+            for t in range(video.shape[0]):
+                frame = cl(video[t:t + 1].half())
+                SL.DCConv2d.fuse_blocks = True
+                got = fused(frame).clone()
+                SL.DCConv2d.fuse_blocks = False
+                want = plain(frame)
+                assert torch.equal(got, want), f"frame {t}"
+        fm, pm = dict(fused.named_modules()), dict(plain.named_modules())
+        n = 0
+        for name, mod in fm.items():
+            if isinstance(mod, SL.DCActivation):
+                assert torch.equal(mod.prev_out, pm[name].prev_out), name
+                assert torch.equal(mod.out_truncated, pm[name].out_truncated), name
+                n += 1
+        assert n == 35
+        # every inverted residual block of every frame after the first took the one-launch form
+        assert len(launches) == 17 * (video.shape[0] - 1) and all(launches), (len(launches), sum(launches))
+    finally:
+        SL.DCConv2d.fuse_blocks = True
+        SL.DCConv2d.fuse_blocks_max_filter_bytes = limit
+        hk.sparse_block = original

@@ -316,11 +316,11 @@ def test_fused_layer_calls_change_nothing(lib, network, size):
         with torch.no_grad():
             for t in range(video.shape[0]):
                 frame = cl(video[t:t + 1].half())
-                SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = True
+                SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = SL.DCConv2d.fuse_blocks = True
                 got = fused(frame)
                 got = {k: v.clone() for k, v in got.items()} if isinstance(got, dict) else got.clone()
-                SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = False
+                SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = SL.DCConv2d.fuse_blocks = False
                 want = plain(frame)
                 assert _same(got, want), f"frame {t}"
     finally:
-        SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = True
+        SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = SL.DCConv2d.fuse_blocks = True

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import delta_ops as ops
-from util import DEV, assert_masked_close, assert_masked_equal, cl, poison, rand_mask
+from util import DEV, assert_masked_close, assert_masked_equal, cl, packed_form_exists, poison, rand_mask
 
 pytestmark = pytest.mark.gpu
 
@@ -379,24 +379,31 @@ def _check_conv(dtype, got, want, want_mask):
         assert_masked_close(got, want, want_mask, 0, 2e-2, "out")
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("cfg", CONVS, ids=lambda c: "-".join(str(v).replace(" ", "") for v in c))
+def _conv_params(cfgs, transposed=False):
+    """(dtype, cfg, packed) for every combination that exists: fp16 filters are defined for one
+    group and depthwise only, and `packed` needs a packed form of the filter."""
+    out = []
+    for cfg in cfgs:
+        cin, cout, k, groups = cfg[0], cfg[1], cfg[2], cfg[6]
+        for dtype in DTYPES:
+            if dtype == torch.float16 and groups > 1 and not (groups == cin == cout):
+                continue
+            out.append(pytest.param(dtype, cfg, False, id=f"{str(dtype)[6:]}-{'-'.join(str(v).replace(' ', '') for v in cfg)}"))
+            if packed_form_exists(dtype, cin, cout, k, groups, transposed):
+                out.append(pytest.param(dtype, cfg, True, id=f"{str(dtype)[6:]}-{'-'.join(str(v).replace(' ', '') for v in cfg)}-packed"))
+    return out
+
+
+@pytest.mark.parametrize("dtype,cfg,packed", _conv_params(CONVS))
 @pytest.mark.parametrize("density", [0.05, 0.5, 1.0])
 @pytest.mark.parametrize("use_bias", [False, True])
-@pytest.mark.parametrize("packed", [False, True])
 def test_conv(lib, dtype, cfg, density, use_bias, packed):
     groups, Cin, Cout = cfg[6], cfg[0], cfg[1]
-    general_groups = groups > 1 and not (groups == Cin == Cout)
-    if general_groups and dtype == torch.float16:
-        pytest.skip("fp16 filter layout is defined for groups == 1 and depthwise only")
     x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 800 + Cin + Cout, density)
     want, want_mask = ops.conv(x, mask, wt, bias if use_bias else None, s, p, d, groups)
     d_filt = filt.to(DEV)
-    pk = None
-    if packed:
-        pk = hk().pack_filter(d_filt, Cin, Cout, groups)
-        if pk is None:
-            pytest.skip("no packed form for this shape")
+    pk = hk().pack_filter(d_filt, Cin, Cout, groups) if packed else None
+    assert (pk is not None) == packed
     out, om = hk().sparse_conv(cl(poison(x, mask)), d_filt, cl(mask), bias.to(DEV) if use_bias else None,
                                s, p, d, groups, c_out=Cout, create_out_mask=True, packed_filter=pk)
     assert out.shape == want.shape
@@ -460,20 +467,15 @@ DECONVS = [
 ]
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("cfg", DECONVS, ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("dtype,cfg,packed", _conv_params(DECONVS, transposed=True))
 @pytest.mark.parametrize("density", [0.1, 1.0])
-@pytest.mark.parametrize("packed", [False, True])
 def test_deconv(lib, dtype, cfg, density, packed):
     Cin, Cout = cfg[0], cfg[1]
     x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 900 + Cin, density, True)
     want, want_mask = ops.deconv(x, mask, wt, bias, s, p, d, groups)
     d_filt = filt.to(DEV)
-    pk = None
-    if packed:
-        pk = hk().pack_filter(d_filt, Cin, Cout, groups, transposed=True)
-        if pk is None:
-            pytest.skip("no packed form for this shape")
+    pk = hk().pack_filter(d_filt, Cin, Cout, groups, transposed=True) if packed else None
+    assert (pk is not None) == packed
     out, om = hk().sparse_deconv(cl(poison(x, mask)), d_filt, cl(mask), bias.to(DEV), s, p, d, groups,
                                  c_out=Cout, create_out_mask=True, packed_filter=pk)
     assert out.shape == want.shape

@@ -188,8 +188,10 @@ def test_random_rectangular_fp32(lib, case):
         cin, cout = groups * rnd.choice([1, 3, 4, 9]), groups * rnd.choice([1, 2, 4, 7])
         st, dil = (rnd.randint(1, 3), rnd.randint(1, 3)), (rnd.randint(1, 2), rnd.randint(1, 2))
         pad = (rnd.randint(0, dil[0] * (K[0] - 1)), rnd.randint(0, dil[1] * (K[1] - 1)))
-        if H + 2 * pad[0] < dil[0] * (K[0] - 1) + 1 or W + 2 * pad[1] < dil[1] * (K[1] - 1) + 1:
-            pytest.skip("window larger than the padded map")
+        # a window larger than the padded map has no output: grow the map instead
+        H = max(H, dil[0] * (K[0] - 1) + 1 - 2 * pad[0])
+        W = max(W, dil[1] * (K[1] - 1) + 1 - 2 * pad[1])
+        mask = rand_mask(g, B, H, W, density)
         x = torch.randn(B, cin, H, W, generator=g)
         wt = torch.randn(cout, cin // groups, *K, generator=g) / (cin // groups * K[0] * K[1]) ** 0.5
         bias = torch.randn(cout, generator=g) if rnd.random() < 0.5 else None

@@ -404,3 +404,188 @@ def test_fused_multiply_add_rounds_once_in_half_precision():
         err = abs(Fraction(float(r)) - ex)
         for nb in (np.nextafter(r, np.float16(np.inf)), np.nextafter(r, np.float16(-np.inf))):
             assert err <= abs(Fraction(float(nb)) - ex), (i, float(r), float(nb))
+
+
+# --------------------------------------------------------------------------------------------
+# Branches that the operator-level loops above do not reach
+# --------------------------------------------------------------------------------------------
+def test_sigmoid_and_swish_against_library():
+    """Activation ids 4 / 5 (other_nn_layers.cu:36-44, 106-121) against torch.sigmoid / F.silu:
+    fp32 to a few ulp; fp16 = the fp32 value rounded once (at most one fp16 ulp apart from the
+    library's own rounding of its fp32 result, and equal almost everywhere)."""
+    g = torch.Generator().manual_seed(41)
+    x = torch.cat([torch.randn(4000, generator=g) * 4, torch.tensor([0.0, -0.0, 20.0, -20.0, 1e-4, -1e-4])])
+    for act, lib in ((O.ACT_SIGMOID, torch.sigmoid), (O.ACT_SWISH, F.silu)):
+        got = O.activation(x.clone(), act)
+        want = lib(x.double())
+        assert torch.allclose(got.double(), want, rtol=3e-7, atol=1e-9), act
+        xh = x.half()
+        got_h = O.activation(xh.clone(), act)
+        assert got_h.dtype == torch.float16
+        want_h = lib(xh.double())
+        # spacing of fp16 at the result's magnitude: 2^-10 relative (2^-24 absolute floor)
+        ulp = torch.maximum(want_h.abs() * 2.0 ** -10, torch.tensor(2.0 ** -24, dtype=torch.float64))
+        assert ((got_h.double() - want_h).abs() <= 0.5 * ulp * (1 + 1e-3)).all(), act  # correctly rounded
+    # a sign error or a missing "x *" would fail these closed forms
+    assert O.activation(torch.tensor([0.0]), O.ACT_SIGMOID).item() == 0.5
+    assert O.activation(torch.tensor([2.0]), O.ACT_SWISH).item() == pytest.approx(2.0 / (1.0 + np.exp(-2.0)), rel=1e-6)
+    assert O.activation(torch.tensor([-30.0]), O.ACT_SIGMOID).item() < 1e-12
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("mode", [O.TRUNC_NORM, O.TRUNC_RMS])
+@pytest.mark.parametrize("act", [1, 3])
+def test_norm_rms_truncation_against_loops(dtype, mode, act):
+    """other_nn_layers.cu:664-719: keep iff sqrt(sum D^2) (norm) or sqrt(sum D^2 / C) (rms)
+    exceeds the threshold.  The loop statement sums in float64; pixels whose statistic lies
+    within 2 % of the threshold are left out of the case (there the summation order of the
+    tensor's type decides)."""
+    rng = np.random.default_rng(77 + mode)
+    B, C, H, W = 1, 6, 6, 7
+    thr = 0.45 if mode == O.TRUNC_NORM else 0.2
+    delta = (rng.standard_normal((B, C, H, W)) * 0.25).astype(dtype)
+    prev = rng.standard_normal((B, C, H, W)).astype(dtype)
+    trunc = (rng.standard_normal((B, C, H, W)) * 0.05).astype(dtype)
+    mask = (rng.random((B, 1, H, W)) < 0.7).astype(np.int32)
+    _, _, _, _, stat = bf.activate_truncate_sum(delta, prev, trunc, mask, thr, act, mode)
+    near = np.abs(stat - thr) < 0.02 * thr
+    mask = np.where(near, 0, mask).astype(np.int32)   # drop near-tie pixels from the case
+    wd, wp, wt, wm, stat = bf.activate_truncate_sum(delta, prev, trunc, mask, thr, act, mode)
+    kept, dropped = int(wm.sum()), int(mask.sum() - wm.sum())
+    assert kept >= 5 and dropped >= 5, (kept, dropped)  # both branches are exercised
+    d, p, t, m = (torch.from_numpy(v.copy()) for v in (delta, prev, trunc, mask))
+    O.activate_truncate(d, p, t, m, thr, act, mode)
+    assert np.array_equal(_np(m), wm)
+    assert np.array_equal(_np(p), wp)
+    assert np.array_equal(_np(t), wt)
+    on = np.broadcast_to(wm != 0, wd.shape)
+    assert np.array_equal(_np(d)[on], wd[on])
+    # the two modes differ by exactly the factor sqrt(C): the same input under the other mode
+    # with the threshold scaled accordingly takes the same decisions
+    other = O.TRUNC_RMS if mode == O.TRUNC_NORM else O.TRUNC_NORM
+    thr2 = thr / np.sqrt(C) if mode == O.TRUNC_NORM else thr * np.sqrt(C)
+    d2, p2, t2, m2 = (torch.from_numpy(v.copy()) for v in (delta, prev, trunc, mask))
+    O.activate_truncate(d2, p2, t2, m2, float(thr2), act, other)
+    assert np.array_equal(_np(m2), wm)
+
+
+@pytest.mark.parametrize("act", [1, 2, 3, 5])
+def test_accumulate_with_activation_telescopes(act):
+    """mode < 0 with an activation (activate_no_truncation, other_nn_layers.cu:378-394):
+    prev += delta and delta := act(prev_new) - act(prev_old) on active pixels.  Over T frames
+    the emitted deltas of a pixel telescope to act(prev_T) - act(prev_0), the cache is the plain
+    sum of the incoming deltas, and an inactive pixel changes nothing."""
+    g = torch.Generator().manual_seed(5 + act)
+    B, C, H, W, T = 1, 3, 5, 6, 6
+    prev0 = torch.randn(B, C, H, W, generator=g, dtype=torch.float64) * 2
+    prev = prev0.clone()
+    emitted = torch.zeros_like(prev)
+    incoming = torch.zeros_like(prev)
+    for _ in range(T):
+        delta = torch.randn(B, C, H, W, generator=g, dtype=torch.float64)
+        mask = (torch.rand(B, 1, H, W, generator=g) < 0.6).to(torch.int32)
+        raw = delta.clone()
+        before = prev.clone()
+        O.activate_truncate(delta, prev, None, mask, 0.0, act, O.TRUNC_NONE)
+        on = (mask != 0).expand_as(delta)
+        assert torch.equal(delta[~on], raw[~on]) and torch.equal(prev[~on], before[~on])
+        emitted += torch.where(on, delta, torch.zeros_like(delta))
+        incoming += torch.where(on, raw, torch.zeros_like(raw))
+    lib = {1: torch.relu, 2: lambda v: v.clamp(0, 6), 3: lambda v: F.leaky_relu(v, float(np.float32(0.1))),  # the slope is a C float
+           5: F.silu}[act]
+    assert torch.allclose(prev, prev0 + incoming, rtol=0, atol=1e-12)
+    # sigmoid / swish are evaluated in float32 whatever the tensor's type
+    assert torch.allclose(emitted, lib(prev) - lib(prev0), rtol=0, atol=1e-12 if act < 4 else 1e-5)
+
+
+@pytest.mark.parametrize("act", [0, 1, 2])
+def test_add_dense_out_against_indexing(act):
+    """DCAdd(dense_out=True), sparse_layers.py:1140-1172: the cache takes the weighted sum on
+    the union of the masks and act(cache) is returned for EVERY pixel, as a plain tensor."""
+    rng = np.random.default_rng(11 + act)
+    B, C, H, W = 2, 3, 5, 4
+    a, b, prev = (rng.standard_normal((B, C, H, W)).astype(np.float32) * 3 for _ in range(3))
+    ma = (rng.random((B, 1, H, W)) < 0.5).astype(np.int32)
+    mb = (rng.random((B, 1, H, W)) < 0.5).astype(np.int32)
+    a_p = np.where(ma != 0, a, np.nan).astype(np.float32)   # inactive operands must not be read
+    b_p = np.where(mb != 0, b, np.nan).astype(np.float32)
+    want, want_prev = bf.add_dense_out(a, ma, b, mb, prev, 0.5, -2.0, act)
+    p = torch.from_numpy(prev.copy())
+    out, mask = O.add(torch.from_numpy(a_p), torch.from_numpy(ma), torch.from_numpy(b_p), torch.from_numpy(mb),
+                      p, 0.5, -2.0, act, dense_out=True)
+    assert mask is None
+    assert np.allclose(_np(p), want_prev, rtol=1e-6, atol=1e-6)
+    assert np.allclose(_np(out), want, rtol=1e-6, atol=1e-6)
+    assert ((ma | mb) == 0).any() and ((ma & mb) != 0).any()   # all four mask combinations occur
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_add_to_dense_against_indexing(dtype):
+    rng = np.random.default_rng(3)
+    B, C, H, W = 2, 5, 4, 6
+    a = rng.standard_normal((B, C, H, W)).astype(dtype)
+    b = rng.standard_normal((B, C, H, W)).astype(dtype)
+    m = (rng.random((B, 1, H, W)) < 0.5).astype(np.int32)
+    want = bf.add_to_dense(a, b, m)
+    a_p = np.where(m != 0, a, np.nan).astype(dtype)
+    tb = torch.from_numpy(b.copy())
+    O.add_to_dense(torch.from_numpy(a_p), tb, torch.from_numpy(m))
+    assert np.array_equal(_np(tb), want)
+    # the activation variant also turns `a` into act(b) on every pixel
+    ta, tb = torch.from_numpy(a.copy()), torch.from_numpy(b.copy())
+    O.add_to_dense(ta, tb, torch.from_numpy(m), act=1)
+    assert np.array_equal(_np(tb), want)
+    assert np.array_equal(_np(ta), np.maximum(want, 0))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("k", [3, 5])
+def test_sparsify_dilated_against_window_loops(dtype, k):
+    """DCSparsify(dilation=k), sparse_layers.py:1233-1244."""
+    rng = np.random.default_rng(19 + k)
+    B, C, H, W = 1, 3, 9, 8
+    prev = rng.random((B, C, H, W)).astype(dtype)
+    x = prev.copy()
+    for _ in range(3):  # a few isolated changed pixels, one of them in a corner
+        y0, x0 = rng.integers(0, H), rng.integers(0, W)
+        x[0, :, y0, x0] += dtype(0.5)
+    x[0, 1, 0, 0] -= dtype(0.4)
+    x = (x + (rng.standard_normal(x.shape) * 0.004).astype(dtype)).astype(dtype)  # sub-threshold noise
+    thr = 0.1
+    wd, wm, wp = bf.sparsify_neighbourhood(x, prev, thr, k)
+    assert 0 < wm.sum() < wm.size
+    tp = torch.from_numpy(prev.copy())
+    d, m = O.sparsify_dilated(torch.from_numpy(x), tp, thr, k)
+    assert np.array_equal(_np(m), wm)
+    assert np.array_equal(_np(tp), wp)
+    on = np.broadcast_to(wm != 0, wd.shape)
+    assert np.array_equal(_np(d)[on], wd[on])
+
+
+@pytest.mark.parametrize("kernel,stride,padding,dilation", [
+    ((2, 2), (1, 1), (0, 0), (2, 2)), ((3, 3), (1, 1), (2, 2), (2, 2)), ((3, 2), (2, 1), (2, 1), (2, 3)),
+    ((2, 2), (2, 2), (1, 1), (3, 3))])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_pool_with_dilation_against_loops_and_library(kernel, stride, padding, dilation, mode):
+    """Window taps `dilation` pixels apart: against the dilated loop statement on a sparse mask,
+    and (max) against F.max_pool2d(..., dilation=) with every pixel active."""
+    rng = np.random.default_rng(23)
+    B, C, H, W = 1, 3, 10, 10
+    delta = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    prev = rng.standard_normal((B, C, H, W)).astype(np.float32)
+    mask = (rng.random((B, 1, H, W)) < 0.3).astype(np.int32)
+    want, wm = bf.pool(delta, prev, mask, kernel, stride, padding, mode, dilation)
+    d_p = np.where(mask != 0, delta, np.nan).astype(np.float32)
+    out, om = O.pool(torch.from_numpy(d_p), torch.from_numpy(prev), torch.from_numpy(mask), kernel, stride,
+                     padding, dilation, mode)
+    assert np.array_equal(_np(om), wm)
+    on = np.broadcast_to(wm != 0, want.shape)
+    assert np.allclose(_np(out)[on], want[on], rtol=1e-6, atol=1e-6)
+    # torch's pooling refuses padding beyond half the window
+    if mode == 0 and all(2 * p <= k for p, k in zip(padding, kernel)):
+        ones = torch.ones(B, 1, H, W, dtype=torch.int32)
+        d, p = torch.from_numpy(delta), torch.from_numpy(prev)
+        out, om = O.pool(d, p, ones, kernel, stride, padding, dilation, 0)
+        lib = (F.max_pool2d(p + d, kernel, stride, padding, dilation) - F.max_pool2d(p, kernel, stride, padding, dilation))
+        assert out.shape == lib.shape and bool((om != 0).all())
+        assert torch.allclose(out, lib, rtol=1e-6, atol=1e-6)
