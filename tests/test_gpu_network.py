@@ -78,6 +78,48 @@ def _calibrated_state(frames):
     return dense.state_dict()
 
 
+class MaskCensus:
+    """Counts, per layer, the update-mask words on which two free-running models differ.  Hooks
+    every layer of both models that returns a (delta, mask) tuple; call `frame()` after each frame."""
+
+    def __init__(self, ref, dut):
+        self.masks = ({}, {})
+        self.hooks = []
+        self.words = 0
+        self.differ = 0
+        self.per_layer = {}
+        for side, model in enumerate((ref, dut)):
+            for name, mod in model.named_modules():
+                self.hooks.append(mod.register_forward_hook(
+                    lambda m, inp, out, name=name, side=side: self._note(side, name, out)))
+
+    def _note(self, side, name, out):
+        if isinstance(out, tuple) and len(out) == 2 and torch.is_tensor(out[1]) and out[1].dtype == torch.int32:
+            self.masks[side][name] = (out[1] != 0).cpu().clone()
+
+    def frame(self):
+        for name, a in self.masks[0].items():
+            b = self.masks[1].get(name)
+            if b is None or b.shape != a.shape:
+                continue
+            d = int((a != b).sum())
+            self.words += a.numel()
+            self.differ += d
+            if d:
+                self.per_layer[name] = self.per_layer.get(name, 0) + d
+        self.masks[0].clear()
+        self.masks[1].clear()
+
+    def close(self):
+        for h in self.hooks:
+            h.remove()
+
+    def report(self):
+        worst = sorted(self.per_layer.items(), key=lambda kv: -kv[1])[:3]
+        return (f"{self.differ} of {self.words} mask words differ ({100.0 * self.differ / max(1, self.words):.3f} %), "
+                f"{len(self.per_layer)} layers affected, worst {worst}")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_mobilenet_32_frames(lib, dtype):
     """MobileNetV2 (BN folded) at 96x96, 33 frames of a moving-rectangle video, threshold 0.05:
@@ -92,22 +134,37 @@ def test_mobilenet_32_frames(lib, dtype):
     from deltacnn_amd.video import moving_rectangles_video
     video = moving_rectangles_video(frames=33, height=96, width=96, n_rect=2, min_size=10, max_size=30)
     state = _calibrated_state(video[:4])
+    from deltacnn_amd import sparse_layers as SL
     dense, ref, dut = _models(_mobilenet, dtype, 0.05, state)
     e_ref = e_dut = e_pair = 0.0
-    with torch.no_grad():
-        for t in range(video.shape[0]):
-            frame = video[t:t + 1].to(dtype)
-            full = dense(frame.float())
-            want = ref(frame).float()
-            got = dut(cl(frame)).float().cpu()
-            e_ref = max(e_ref, float((want - full).abs().max()))
-            e_dut = max(e_dut, float((got - full).abs().max()))
-            e_pair = max(e_pair, float((got - want).abs().max()))
-            if dtype == torch.float32:
-                assert float((got - want).abs().max()) <= 1e-4 * max(1.0, float(want.abs().max())), f"frame {t}"
+    census = MaskCensus(ref, dut)
+    SL.DCConv2d.fuse_blocks = False  # every layer returns its own mask (the one-launch form is bit-identical)
+    try:
+        with torch.no_grad():
+            for t in range(video.shape[0]):
+                frame = video[t:t + 1].to(dtype)
+                full = dense(frame.float())
+                want = ref(frame).float()
+                got = dut(cl(frame)).float().cpu()
+                census.frame()
+                e_ref = max(e_ref, float((want - full).abs().max()))
+                e_dut = max(e_dut, float((got - full).abs().max()))
+                e_pair = max(e_pair, float((got - want).abs().max()))
+                if dtype == torch.float32:
+                    assert float((got - want).abs().max()) <= 1e-4 * max(1.0, float(want.abs().max())), f"frame {t}"
+    finally:
+        SL.DCConv2d.fuse_blocks = True
+        census.close()
     print(f"{dtype}: |oracle-dense| {e_ref:.4f}  |hip-dense| {e_dut:.4f}  |hip-oracle| {e_pair:.4f}  "
           f"|dense| {float(full.abs().max()):.3f}")
+    print(f"{dtype}: free-running update masks, HIP against oracle: {census.report()}")
     assert e_dut <= 1.5 * e_ref + 2e-2
+    # Free-running masks: in fp32 a convolution output would have to land within 1e-6 of a
+    # threshold for a decision to differ; in fp16 a flipped decision changes the truncation state
+    # of that pixel for good (both states are valid), so differences accumulate along the clip --
+    # bounded here, exact equality at identical inputs is the teacher-forced test.
+    assert census.words > 0
+    assert census.differ <= (1e-5 if dtype == torch.float32 else 2e-3) * census.words, census.report()  # measured: 0 / 6e-5 .. 2e-4
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
@@ -262,20 +319,31 @@ def test_multibranch_networks(lib, builder, size, dtype):
     from deltacnn_amd.video import moving_rectangles_video
     video = moving_rectangles_video(frames=8, height=size[0], width=size[1], n_rect=2, min_size=8, max_size=24)
     state = _calibrated(builder, video[:3])
+    from deltacnn_amd import sparse_layers as SL
     dense, ref, dut = _models(builder, dtype, 0.05, state)
     e_ref = e_dut = 0.0
-    with torch.no_grad():
-        for t in range(video.shape[0]):
-            frame = video[t:t + 1].to(dtype)
-            full = dense(frame.float())
-            want = ref(frame)
-            got = dut(cl(frame))
-            e_ref = max(e_ref, _out_err(want, full))
-            e_dut = max(e_dut, _out_err(got, full))
-            if dtype == torch.float32:
-                assert _out_err(got, want) <= 1e-4 * _out_scale(want), f"frame {t}"
+    census = MaskCensus(ref, dut)
+    SL.DCAdd.fuse_into_conv = False  # every layer returns its own mask (the fused forms are bit-identical)
+    try:
+        with torch.no_grad():
+            for t in range(video.shape[0]):
+                frame = video[t:t + 1].to(dtype)
+                full = dense(frame.float())
+                want = ref(frame)
+                got = dut(cl(frame))
+                census.frame()
+                e_ref = max(e_ref, _out_err(want, full))
+                e_dut = max(e_dut, _out_err(got, full))
+                if dtype == torch.float32:
+                    assert _out_err(got, want) <= 1e-4 * _out_scale(want), f"frame {t}"
+    finally:
+        SL.DCAdd.fuse_into_conv = True
+        census.close()
     print(f"{dtype}: |oracle-dense| {e_ref:.4f}  |hip-dense| {e_dut:.4f}")
+    print(f"{dtype}: free-running update masks, HIP against oracle: {census.report()}")
     assert e_dut <= 1.5 * e_ref + 2e-2
+    assert census.words > 0
+    assert census.differ <= (1e-5 if dtype == torch.float32 else 2e-3) * census.words, census.report()  # measured: 0 / 6e-5 .. 2e-4
 
 
 def _two_hip_models(builder, state):

@@ -6,8 +6,10 @@ fed the oracle's inputs for that call.  With identical inputs every frame, the b
 
   * update masks (and therefore active-pixel index sets) equal bit for bit at every layer
   * elementwise layers (sparsify, activation/truncation, add, densify) equal bit for bit
-  * contractions (conv, transposed conv) within 1e-4 relative (fp32) / 2e-2 absolute (fp16);
-    global average pooling within float-sum reordering
+  * contractions (conv, transposed conv) within 1e-4 relative (fp32) / 2e-2 absolute (fp16; for
+    values beyond +-10, where one fp16 step alone exceeds that, two steps of the value: 2^-9
+    relative -- the random-init HRNet reaches +-300); global average pooling within float-sum
+    reordering
 
 Free-running models cannot be held to mask equality in fp16: one last-bit difference of a
 convolution output next to a threshold legitimately flips a truncation decision.
@@ -42,7 +44,7 @@ def _compare(kind, got, want, dtype, where):
         elif dtype == torch.float32:
             assert_masked_close(g, w, wm, 1e-4, 1e-5, where)
         else:
-            assert_masked_close(g, w, wm, 0, 2e-2, where)
+            assert_masked_close(g, w, wm, 2.0 ** -9, 2e-2, where)
     else:
         if kind == "exact":
             assert torch.equal(got.cpu(), want), f"{where}: max diff {float((got.cpu().float() - want.float()).abs().max())}"
@@ -124,3 +126,47 @@ def test_multibranch_teacher_forced(lib, network, dtype):
     ref, dut = _build(builder, dtype, 0.05, _calibrated(builder, video[:3]))
     n = run_teacher_forced(ref, dut, video, dtype)
     assert n % 8 == 0 and n // 8 > 100
+
+
+# --------------------------------------------------------------------------------------------
+# The measured configurations at their real sizes, fp16 (the type they are measured in)
+# --------------------------------------------------------------------------------------------
+def test_mobilenet_224_fp16_teacher_forced_34_frames(lib):
+    """MobileNetV2 w1.0 at 224x224, fp16, on the synthetic clip of the headline configuration
+    (smooth-noise background, three textured rectangles moving 1-4 px per frame, sensor noise
+    sigma 0.01, threshold 0.05 on all layers): 34 frames, every layer call of every frame fed the
+    CPU oracle's input.  Masks bit for bit, elementwise layers bit for bit, convolutions within
+    2e-2 absolute -- after 33 frames of delta accumulation in every layer's caches."""
+    from deltacnn_amd.networks import MobileNetV2
+    from deltacnn_amd.video import moving_rectangles_video
+    from test_gpu_network import _calibrated
+    video = moving_rectangles_video(frames=34)  # the generator's defaults are that configuration
+    assert tuple(video.shape[1:]) == (3, 224, 224)
+
+    def full(L, **kw):
+        return MobileNetV2(L, **kw)  # 1000-way head
+    ref, dut = _build(full, torch.float16, 0.05, _calibrated(full, video[:3]))
+    n = run_teacher_forced(ref, dut, video, torch.float16)
+    assert n == 34 * (1 + 52 + 35 + 10 + 1 + 1)
+
+
+@pytest.mark.parametrize("network", ["hrnet_w32", "dla34_centernet"])
+def test_full_depth_networks_fp16_teacher_forced(lib, network):
+    """HRNet-W32 (full depth: 1 / 4 / 3 modules of 4 blocks, 17 heat maps) at 256x256 and DLA-34 +
+    CenterNet heads (80 classes, 256-channel heads) at 544x960, fp16, threshold 0.05: every layer
+    call of 5 resp. 4 frames fed the CPU oracle's input, bar as above."""
+    from deltacnn_amd.networks import DLA34CenterNet, HRNet
+    from deltacnn_amd.video import moving_rectangles_video
+    from test_gpu_network import _calibrated
+    if network == "hrnet_w32":
+        builder, frames = HRNet, 5
+        video = moving_rectangles_video(frames=frames, height=256, width=256, n_rect=1, min_size=100,
+                                        max_size=180, min_speed=2, max_speed=6)
+    else:
+        builder, frames = DLA34CenterNet, 4
+        video = moving_rectangles_video(frames=frames, height=544, width=960, n_rect=12, min_size=30,
+                                        max_size=200, min_speed=1, max_speed=5)
+    small = moving_rectangles_video(frames=2, height=64, width=96, n_rect=2, min_size=8, max_size=24)
+    ref, dut = _build(builder, torch.float16, 0.05, _calibrated(builder, small))
+    n = run_teacher_forced(ref, dut, video, torch.float16)
+    assert n % frames == 0 and n // frames >= (400 if network == "hrnet_w32" else 150), n
