@@ -15,7 +15,9 @@ m = 4-byte mask word, P pixels, n_x = number of active pixels of mask x):
                      truncation; conv_act in two launches: a conv row and an activate_truncate row)
                      flops = 2*(Cin/g)*Cout*N_pairs, N_pairs = sum over updated outputs of the
                      active inputs in their window (computed exactly from the masks)
-  pool               R = P_in*m + n_in*C*s (x2 for max)   W = n_out*C*s + P_out*m
+  pool               R = P_in*m + n_in*C*s [max: + n_cov*C*s]   W = n_out*C*s + P_out*m
+                     (the maximum of an updated window needs the cached input of EVERY pixel of the
+                     window, updated or not: n_cov = input pixels covered by updated windows)
   add_to_dense       R = P*m + 2*n*C*s                    W = n*C*s
   upsample           R = P*m + n*C*s                      W = S*S*(n*C*s + P*m)
   concat             R = 2*P*m + (n_a*Ca + n_b*Cb)*s      W = n_out*(Ca+Cb)*s + P*m
@@ -68,6 +70,8 @@ class Tracer:
         rec["kernels"] = _lib.load().dc_last_kernels().decode().split("+")
         rec["n_out"] = self._count(meta.get("out_mask"))
         rec["n_ex"] = self._count(meta.get("ex_mask"))
+        if op == "pool" and meta.get("mode") == 0:
+            rec["n_cov"] = self._covered(meta["g"], meta["out_mask"])
         rec["call"] = (fn, args)
         self.records.append(rec)
         return rc
@@ -131,6 +135,15 @@ class Tracer:
                 t_conv = min(timed([conv_only]), times[i])
                 rec["split_us"] = [t_conv, times[i] - t_conv]
         return times
+
+    @staticmethod
+    def _covered(g, out_mask):
+        """Input pixels that lie in the window of at least one updated output pixel."""
+        m = (out_mask != 0).float()
+        ones = torch.ones(1, 1, g.kernel_h, g.kernel_w, device=m.device)
+        cov = F.conv_transpose2d(m, ones, stride=(g.stride_h, g.stride_w), dilation=(g.dilation_h, g.dilation_w))
+        cov = cov[:, :, g.pad_top:g.pad_top + g.in_h, g.pad_left:g.pad_left + g.in_w]
+        return (cov > 0).sum()
 
     @staticmethod
     def _pairs(g, mask, transposed):
@@ -208,7 +221,9 @@ class Tracer:
             elif op == "pool":
                 g = meta["g"]
                 p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
-                rd = p_in * m + n_in * g.in_c * s * (2 if meta["mode"] == 0 else 1)
+                rd = p_in * m + n_in * g.in_c * s
+                if meta["mode"] == 0:  # + the cached input of every pixel under an updated window
+                    rd += int(r["n_cov"]) * g.in_c * s if "n_cov" in r else n_in * g.in_c * s
                 wr = n_out * g.in_c * s + p_out * m
                 shape = f"C{g.in_c} k{g.kernel_h} @{g.in_h}x{g.in_w}"
                 dens = (n_in / p_in, n_out / p_out)
