@@ -188,3 +188,43 @@ def test_packed_form_rule_matches_the_library(lib):
                             have = lib.dc_packed_filter_bytes(g, code, int(transposed)) != 0
                             assert have == packed_form_exists(dtype, cin, cout, k, groups, transposed), \
                                 (cin, cout, k, groups, transposed, dtype)
+
+
+def test_block_arguments_are_checked_before_any_launch(lib):
+    """dc_block: shape rules -> -3 (the caller then issues the separate calls), missing operands
+    -> -4, misaligned feature pointers -> -5; all without touching a device."""
+    from deltacnn_amd._lib import BlockArgs
+    buf = (ctypes.c_char * 8192)()
+    p = (ctypes.addressof(buf) + 255) // 256 * 256
+    g = _geom(in_c=64, out_c=64, groups=64)   # depthwise 3x3, stride 1, padding 1
+
+    def args(**kw):
+        a = BlockArgs()
+        for name in ("input", "mask", "dw_filter", "dw_prev_out", "dw_truncated", "project_packed_filter", "out",
+                     "out_mask"):
+            setattr(a, name, p)
+        a.dw_threshold, a.dw_activation, a.dw_truncation_mode = 0.05, 2, 0
+        a.project_channels, a.weight_residual, a.weight_conv = 24, 1.0, 1.0
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+
+    def call(geom, a, dtype=1):
+        return lib.dc_block(ctypes.byref(geom), ctypes.byref(a), dtype, None)
+
+    assert call(g, args(), dtype=0) == -3 and b"fp16 only" in lib.dc_last_error()
+    assert call(g, args(), dtype=7) == -1
+    assert call(_geom(in_c=64, out_c=64, groups=1), args()) == -3          # not depthwise
+    assert call(_geom(in_c=60, out_c=60, groups=60), args()) == -3         # hidden channels not a multiple of 8
+    assert call(g, args(project_channels=20)) == -3                       # projection channels not a multiple of 8
+    assert call(g, args(dw_activation=4)) == -3                           # sigmoid
+    assert call(g, args(dw_truncation_mode=1)) == -3                      # norm truncation
+    assert call(g, args(expand_channels=96, expand_activation=1, expand_truncation_mode=0)) == -3  # activations differ
+    assert call(_geom(in_c=64, out_c=64, groups=64, out_h=7), args()) == -2
+    assert lib.dc_block(None, ctypes.byref(args()), 1, None) == -4
+    assert lib.dc_block(ctypes.byref(g), None, 1, None) == -4
+    assert call(g, args(out=None)) == -4
+    assert call(g, args(residual=p)) == -4                                # a residual needs its mask
+    assert call(g, args(expand_channels=96, expand_activation=2)) == -4   # expansion operands missing
+    assert call(g, args(input=p + 2)) == -5
+    assert call(g, args(out=p + 4)) == -5
