@@ -12,7 +12,7 @@ from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdeltacnn_hip.so")
 
-DC_F32, DC_F16 = 0, 1
+DC_F32, DC_F16, DC_BF16 = 0, 1, 2
 ERROR_NAMES = {0: "DC_OK", -1: "DC_ERR_DTYPE", -2: "DC_ERR_SHAPE", -3: "DC_ERR_UNSUPPORTED",
                -4: "DC_ERR_NULL", -5: "DC_ERR_ALIGN", -6: "DC_ERR_LAUNCH"}
 

@@ -16,6 +16,34 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+// The two 16-bit element types of the matrix-core kernels: vector types and the MFMA
+// instruction (16 x 16 outputs, 32 reduction elements, fp32 accumulate).
+template <typename E>
+struct Elem16;
+template <>
+struct Elem16<half_t> {
+    typedef half4_t v4;
+    typedef half8_t v8;
+    static __device__ __forceinline__ float4_t mfma(v8 a, v8 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct Elem16<bf16_t> {
+    typedef bf16x4_t v4;
+    typedef bf16x8_t v8;
+    static __device__ __forceinline__ float4_t mfma(v8 a, v8 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <typename E>
+__device__ __forceinline__ typename Elem16<E>::v4 zero4() {
+    return typename Elem16<E>::v4{E(0), E(0), E(0), E(0)};
+}
 
 // N elements of T moved with one naturally aligned load / store.
 template <typename T, int N>
@@ -51,6 +79,17 @@ __device__ __forceinline__ Vec<T, N> vkeep(const Vec<T, N> &x, bool on) {
 __device__ __forceinline__ half8_t keep8(half8_t x, bool on) {
     union {
         half8_t v;
+        uint32_t u[4];
+    } c;
+    c.v = x;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) c.u[k] = on ? c.u[k] : 0u;
+    return c.v;
+}
+
+__device__ __forceinline__ bf16x8_t keep8(bf16x8_t x, bool on) {
+    union {
+        bf16x8_t v;
         uint32_t u[4];
     } c;
     c.v = x;
@@ -107,6 +146,12 @@ __device__ __attribute__((noinline)) half_t sigmoid_t(half_t x) {
 __device__ __attribute__((noinline)) half_t swish_t(half_t x) {
     return half_t(float(x) * (1.0f / (1.0f + expf(-float(x)))));
 }
+__device__ __attribute__((noinline)) bf16_t sigmoid_t(bf16_t x) {
+    return bf16_t(1.0f / (1.0f + expf(-float(x))));
+}
+__device__ __attribute__((noinline)) bf16_t swish_t(bf16_t x) {
+    return bf16_t(float(x) * (1.0f / (1.0f + expf(-float(x)))));
+}
 
 // max / min as single instructions (v_max_f16, v_max_f32, ...).  For finite operands they give
 // the values of the compare-and-select form `x < 0 ? 0 : x`; the two differ only for NaN (here
@@ -116,6 +161,10 @@ __device__ __forceinline__ float tmax(float a, float b) { return __builtin_fmaxf
 __device__ __forceinline__ float tmin(float a, float b) { return __builtin_fminf(a, b); }
 __device__ __forceinline__ half_t tmax(half_t a, half_t b) { return __builtin_fmaxf16(a, b); }
 __device__ __forceinline__ half_t tmin(half_t a, half_t b) { return __builtin_fminf16(a, b); }
+// bfloat16 arithmetic is fp32 arithmetic on the widened operands followed by one rounding
+// (v_cvt_pk_bf16_f32); max / min / abs of bfloat16 values are exact in either type
+__device__ __forceinline__ bf16_t tmax(bf16_t a, bf16_t b) { return bf16_t(__builtin_fmaxf(float(a), float(b))); }
+__device__ __forceinline__ bf16_t tmin(bf16_t a, bf16_t b) { return bf16_t(__builtin_fminf(float(a), float(b))); }
 
 template <typename T>
 __device__ __forceinline__ T act_apply(T x, int act) {
@@ -134,9 +183,15 @@ __device__ __forceinline__ float fma_t(float a, float b, float c) { return __bui
 __device__ __forceinline__ half_t fma_t(half_t a, half_t b, half_t c) {
     return __builtin_fmaf16(a, b, c);
 }
+// the fp32 fused multiply-add of bfloat16 operands is exact up to its own rounding (the product
+// has 16 significant bits), then rounded to bfloat16
+__device__ __forceinline__ bf16_t fma_t(bf16_t a, bf16_t b, bf16_t c) {
+    return bf16_t(__builtin_fmaf(float(a), float(b), float(c)));
+}
 
 __device__ __forceinline__ float tabs(float x) { return __builtin_fabsf(x); }
 __device__ __forceinline__ half_t tabs(half_t x) { return __builtin_fabsf16(x); }
+__device__ __forceinline__ bf16_t tabs(bf16_t x) { return bf16_t(__builtin_fabsf(float(x))); }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -212,7 +267,7 @@ hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *p
 hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *packed,
                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
                             const ActEpilogue *epi, bool *epilogue_done, const Residual *res,
-                            hipStream_t s);
+                            int dtype, hipStream_t s);
 hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *packed, int dtype,
                               bool transposed, hipStream_t s);
 int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed);

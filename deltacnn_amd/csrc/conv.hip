@@ -1462,13 +1462,14 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
 }
 
 // One-time relayout of a reference-layout fp16 filter [Cin pad 2][K][K][Cout pad 2] (channel
-// pairs swizzled: W[ci][co] is stored at row ci ^ (co & 1)) into MFMA fragment order
+// pairs swizzled: W[ci][co] is stored at row ci ^ (co & 1); swz == 0: the plain [Cin][K][K][Cout]
+// layout of bfloat16 filters) into MFMA fragment order
 // [Cout tile of 16][tap][Cin step of 32][lane 0..63][8]: lane (kq * 16 + r) of a fragment holds
 // input channels kq * 8 .. + 8 of output channel r, so one A operand of
 // v_mfma_f32_16x16x32_f16 is a single contiguous 1 KB read (16 bytes per lane, consecutive
 // lanes at consecutive addresses).  Channels past Cin / Cout are zero.
-__global__ void pack_filter_kernel(const half_t *__restrict__ f, half_t *__restrict__ wp, int Ci,
-                                   int Co, int K2, int w_co, int ci_p, int co_p) {
+__global__ void pack_filter_kernel(const uint16_t *__restrict__ f, uint16_t *__restrict__ wp, int Ci,
+                                   int Co, int K2, int w_co, int ci_p, int co_p, int swz) {
     const size_t total = (size_t)co_p * K2 * ci_p;
     const int ksteps = ci_p >> 5;
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total;
@@ -1480,8 +1481,8 @@ __global__ void pack_filter_kernel(const half_t *__restrict__ f, half_t *__restr
         const int ct = int(frag / ((size_t)ksteps * K2));
         const int co = ct * 16 + (lane & 15);
         const int ci = step * 32 + (lane >> 4) * 8 + e;
-        half_t v = half_t(0);
-        if (ci < Ci && co < Co) v = f[((size_t)(ci ^ (co & 1)) * K2 + tap) * w_co + co];
+        uint16_t v = 0;  // 16-bit elements of either type are moved as they are
+        if (ci < Ci && co < Co) v = f[((size_t)(ci ^ (swz ? (co & 1) : 0)) * K2 + tap) * w_co + co];
         wp[i] = v;
     }
 }
@@ -1701,9 +1702,15 @@ ConvP make_params(const dc_geometry &g, int dtype) {
 
 }  // namespace
 
+// bfloat16 has matrix-core kernels for pointwise convolutions only (K x K windows take the
+// generic kernel); its filters are in the fp32 layout, unswizzled.
+inline bool bf16_packable(const dc_geometry &g, int dtype, bool transposed) {
+    return dtype == DC_BF16 && !transposed && pointwise_eligible(g, dtype);
+}
+
 int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed) {
     if (!transposed && stem_eligible(g, dtype)) return (int64_t)ceil_div(g.out_c, 16) * g.kernel_h * 1024;
-    if (!mfma_eligible(g, dtype)) return 0;
+    if (!mfma_eligible(g, dtype) && !bf16_packable(g, dtype, transposed)) return 0;
     return (int64_t)round_up(g.out_c, 16) * g.kernel_h * g.kernel_w * round_up(g.in_c, 32) * 2;
 }
 
@@ -1717,15 +1724,16 @@ hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *pa
             g.out_c + (g.out_c & 1), co_tiles);
         return hipGetLastError();
     }
-    if (!mfma_eligible(g, dtype)) return hipSuccess;
+    if (!mfma_eligible(g, dtype) && !bf16_packable(g, dtype, transposed)) return hipSuccess;
     const int K2 = g.kernel_h * g.kernel_w;
     const int ci_p = round_up(g.in_c, 32), co_p = round_up(g.out_c, 16);
     const size_t total = (size_t)co_p * K2 * ci_p;
     int blocks = (int)((total + 255) / 256);
     if (blocks > 4096) blocks = 4096;
     note_kernel("pack_filter_kernel");
-    pack_filter_kernel<<<blocks, 256, 0, s>>>((const half_t *)filter, (half_t *)packed, g.in_c,
-                                              g.out_c, K2, g.out_c + (g.out_c & 1), ci_p, co_p);
+    const int swz = dtype == DC_F16 ? 1 : 0;  // the fp16 reference layout: rows padded to even, pairs swizzled
+    pack_filter_kernel<<<blocks, 256, 0, s>>>((const uint16_t *)filter, (uint16_t *)packed, g.in_c, g.out_c, K2,
+                                              swz ? g.out_c + (g.out_c & 1) : g.out_c, ci_p, co_p, swz);
     return hipGetLastError();
 }
 
@@ -1996,6 +2004,8 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
     if (!transposed) {
         const bool done = dtype == DC_F32
             ? try_depthwise<float>(g, p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, epi, s)
+            : dtype == DC_BF16
+            ? try_depthwise<bf16_t>(g, p, (const bf16_t *)in, (const bf16_t *)filter, (const bf16_t *)bias, (bf16_t *)out, mask, out_mask, epi, s)
             : try_depthwise<half_t>(g, p, (const half_t *)in, (const half_t *)filter, (const half_t *)bias, (half_t *)out, mask, out_mask, epi, s);
         if (done) return hipGetLastError();
         if (dtype == DC_F16 && try_stem_mfma(g, p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias,
@@ -2003,12 +2013,14 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
             return hipGetLastError();
         const bool few = dtype == DC_F32
             ? try_fewcin<float>(g, p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, epi, s)
+            : dtype == DC_BF16
+            ? try_fewcin<bf16_t>(g, p, (const bf16_t *)in, (const bf16_t *)filter, (const bf16_t *)bias, (bf16_t *)out, mask, out_mask, epi, s)
             : try_fewcin<half_t>(g, p, (const half_t *)in, (const half_t *)filter, (const half_t *)bias, (half_t *)out, mask, out_mask, epi, s);
         if (few) return hipGetLastError();
     }
     if (packed != nullptr && !transposed && pointwise_eligible(g, dtype)) {
         bool epilogue_done = false;
-        hipError_t e = launch_pointwise(g, in, packed, bias, out, mask, out_mask, epi, &epilogue_done, nullptr, s);
+        hipError_t e = launch_pointwise(g, in, packed, bias, out, mask, out_mask, epi, &epilogue_done, nullptr, dtype, s);
         if (e != hipSuccess || epi == nullptr || epilogue_done) return e;
         return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
                                         epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
@@ -2139,6 +2151,11 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                 conv_direct_kernel<float, true><<<grid, 256, 0, s>>>(p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, COT);
             else
                 conv_direct_kernel<float, false><<<grid, 256, 0, s>>>(p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, COT);
+        } else if (dtype == DC_BF16) {
+            if (transposed)
+                conv_direct_kernel<bf16_t, true><<<grid, 256, 0, s>>>(p, (const bf16_t *)in, (const bf16_t *)filter, (const bf16_t *)bias, (bf16_t *)out, mask, out_mask, COT);
+            else
+                conv_direct_kernel<bf16_t, false><<<grid, 256, 0, s>>>(p, (const bf16_t *)in, (const bf16_t *)filter, (const bf16_t *)bias, (bf16_t *)out, mask, out_mask, COT);
         } else {
             if (transposed)
                 conv_direct_kernel<half_t, true><<<grid, 256, 0, s>>>(p, (const half_t *)in, (const half_t *)filter, (const half_t *)bias, (half_t *)out, mask, out_mask, COT);

@@ -27,7 +27,7 @@ int finish(hipError_t e, const char *what) {
 inline size_t esize(int dtype) { return dtype == DC_F32 ? 4 : 2; }
 
 #define DC_REQUIRE_DTYPE(fn) \
-    if (dtype != DC_F32 && dtype != DC_F16) return fail(DC_ERR_DTYPE, fn ": unsupported dtype %d", dtype)
+    if (dtype != DC_F32 && dtype != DC_F16 && dtype != DC_BF16) return fail(DC_ERR_DTYPE, fn ": unsupported dtype %d", dtype)
 #define DC_REQUIRE_PTR(fn, p) \
     if ((p) == nullptr) return fail(DC_ERR_NULL, fn ": " #p " is NULL")
 #define DC_REQUIRE_ALIGNED(fn, p, a) \
@@ -89,7 +89,7 @@ int check_geometry(const char *fn, const dc_geometry *g, bool transposed, bool p
 int check_conv(const char *fn, const dc_geometry *g, const void *input, const void *filter,
                const void *out, const int32_t *mask, const int32_t *out_mask, int dtype,
                bool transposed) {
-    if (dtype != DC_F32 && dtype != DC_F16) return fail(DC_ERR_DTYPE, "%s: unsupported dtype %d", fn, dtype);
+    if (dtype != DC_F32 && dtype != DC_F16 && dtype != DC_BF16) return fail(DC_ERR_DTYPE, "%s: unsupported dtype %d", fn, dtype);
     int rc = check_geometry(fn, g, transposed, false);
     if (rc != DC_OK) return rc;
     if (!input || !filter || !out || !mask || !out_mask)
@@ -232,7 +232,7 @@ int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filt
     if (pointwise) {
         bool unused = false;
         return finish(dc::launch_pointwise(*g, input, packed_filter, bias, out, mask, out_mask, nullptr,
-                                           &unused, &res, (hipStream_t)stream), "dc_conv_add");
+                                           &unused, &res, dtype, (hipStream_t)stream), "dc_conv_add");
     }
     return finish(dc::launch_patch_conv(*g, input, packed_filter, bias, out, mask, out_mask, false, &res,
                                         (hipStream_t)stream), "dc_conv_add");

@@ -943,6 +943,8 @@ hipError_t launch_sparsify(const void *in, void *prev, void *delta, int32_t *mas
                            int32_t P, int32_t C, int dtype, hipStream_t s) {
     if (dtype == DC_F32)
         return sparsify_t<float>((const float *)in, (float *)prev, (float *)delta, mask, thr, P, C, false, s);
+    if (dtype == DC_BF16)
+        return sparsify_t<bf16_t>((const bf16_t *)in, (bf16_t *)prev, (bf16_t *)delta, mask, thr, P, C, false, s);
     return sparsify_t<half_t>((const half_t *)in, (half_t *)prev, (half_t *)delta, mask, thr, P, C,
                               C % 2 == 0, s);
 }
@@ -952,6 +954,8 @@ hipError_t launch_activate_truncate(void *delta, void *prev, void *trunc, int32_
                                     hipStream_t s) {
     if (dtype == DC_F32)
         return act_trunc_t<float>((float *)delta, (float *)prev, (float *)trunc, mask, thr, act, mode, P, C, s);
+    if (dtype == DC_BF16)
+        return act_trunc_t<bf16_t>((bf16_t *)delta, (bf16_t *)prev, (bf16_t *)trunc, mask, thr, act, mode, P, C, s);
     return act_trunc_t<half_t>((half_t *)delta, (half_t *)prev, (half_t *)trunc, mask, thr, act, mode, P, C, s);
 }
 
@@ -973,6 +977,8 @@ hipError_t densify_t(const T *delta, T *prev, T *out, const int32_t *mask, int P
 hipError_t launch_densify(const void *delta, void *prev, void *out, const int32_t *mask, int P, int C,
                           int dtype, hipStream_t s) {
     if (dtype == DC_F32) return densify_t<float>((const float *)delta, (float *)prev, (float *)out, mask, P, C, s);
+    if (dtype == DC_BF16)
+        return densify_t<bf16_t>((const bf16_t *)delta, (bf16_t *)prev, (bf16_t *)out, mask, P, C, s);
     return densify_t<half_t>((const half_t *)delta, (half_t *)prev, (half_t *)out, mask, P, C, s);
 }
 
@@ -998,6 +1004,8 @@ hipError_t launch_add_upsampled(const void *a, const void *b, void *prev, void *
                                 int32_t H, int32_t W, int32_t C, int32_t scale, int dtype, hipStream_t s) {
     if (dtype == DC_F32)
         return add_up_t<float>((const float *)a, (const float *)b, (float *)prev, (float *)out, ma, mb, mo, wa, wb, act, B, H, W, C, scale, s);
+    if (dtype == DC_BF16)
+        return add_up_t<bf16_t>((const bf16_t *)a, (const bf16_t *)b, (bf16_t *)prev, (bf16_t *)out, ma, mb, mo, wa, wb, act, B, H, W, C, scale, s);
     return add_up_t<half_t>((const half_t *)a, (const half_t *)b, (half_t *)prev, (half_t *)out, ma, mb, mo, wa, wb, act, B, H, W, C, scale, s);
 }
 
@@ -1006,6 +1014,8 @@ hipError_t launch_add(const void *a, const void *b, void *prev, void *out, const
                       int32_t P, int32_t C, int dtype, hipStream_t s) {
     if (dtype == DC_F32)
         return add_t<float>((const float *)a, (const float *)b, (float *)prev, (float *)out, ma, mb, mo, wa, wb, act, dense_out != 0, P, C, s);
+    if (dtype == DC_BF16)
+        return add_t<bf16_t>((const bf16_t *)a, (const bf16_t *)b, (bf16_t *)prev, (bf16_t *)out, ma, mb, mo, wa, wb, act, dense_out != 0, P, C, s);
     return add_t<half_t>((const half_t *)a, (const half_t *)b, (half_t *)prev, (half_t *)out, ma, mb, mo, wa, wb, act, dense_out != 0, P, C, s);
 }
 
@@ -1097,6 +1107,8 @@ hipError_t mul_add_t(const T *in, const int32_t *mask, T *out, int32_t *mo, cons
 hipError_t launch_add_to_dense(void *a, void *b, const int32_t *ma, int act, int32_t P, int32_t C,
                                int dtype, hipStream_t s) {
     if (dtype == DC_F32) return add_to_dense_t<float>((float *)a, (float *)b, ma, act, P, C, s);
+    if (dtype == DC_BF16)
+        return add_to_dense_t<bf16_t>((bf16_t *)a, (bf16_t *)b, ma, act, P, C, s);
     return add_to_dense_t<half_t>((half_t *)a, (half_t *)b, ma, act, P, C, s);
 }
 
@@ -1104,6 +1116,8 @@ hipError_t launch_upsample(const void *in, void *out, const int32_t *mi, int32_t
                            int32_t H, int32_t W, int32_t C, int32_t scale, int dtype,
                            hipStream_t s) {
     if (dtype == DC_F32) return upsample_t<float>((const float *)in, (float *)out, mi, mo, B, H, W, C, scale, s);
+    if (dtype == DC_BF16)
+        return upsample_t<bf16_t>((const bf16_t *)in, (bf16_t *)out, mi, mo, B, H, W, C, scale, s);
     return upsample_t<half_t>((const half_t *)in, (half_t *)out, mi, mo, B, H, W, C, scale, s);
 }
 
@@ -1111,6 +1125,8 @@ hipError_t launch_concat(const void *a, const void *b, void *out, const int32_t 
                          const int32_t *mb, int32_t *mo, int32_t P, int32_t Ca, int32_t Cb,
                          int dtype, hipStream_t s) {
     if (dtype == DC_F32) return concat_t<float>((const float *)a, (const float *)b, (float *)out, ma, mb, mo, P, Ca, Cb, s);
+    if (dtype == DC_BF16)
+        return concat_t<bf16_t>((const bf16_t *)a, (const bf16_t *)b, (bf16_t *)out, ma, mb, mo, P, Ca, Cb, s);
     return concat_t<half_t>((const half_t *)a, (const half_t *)b, (half_t *)out, ma, mb, mo, P, Ca, Cb, s);
 }
 
@@ -1118,6 +1134,8 @@ hipError_t launch_mul_add(const void *in, const int32_t *mask, void *out, int32_
                           const void *scale, const void *bias, int32_t P, int32_t C, int dtype,
                           hipStream_t s) {
     if (dtype == DC_F32) return mul_add_t<float>((const float *)in, mask, (float *)out, mo, (const float *)scale, (const float *)bias, P, C, s);
+    if (dtype == DC_BF16)
+        return mul_add_t<bf16_t>((const bf16_t *)in, mask, (bf16_t *)out, mo, (const bf16_t *)scale, (const bf16_t *)bias, P, C, s);
     return mul_add_t<half_t>((const half_t *)in, mask, (half_t *)out, mo, (const half_t *)scale, (const half_t *)bias, P, C, s);
 }
 

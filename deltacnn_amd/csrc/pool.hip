@@ -598,6 +598,8 @@ hipError_t launch_pool(const dc_geometry &g, const void *in, const void *prev, v
                        hipStream_t s) {
     if (dtype == DC_F32)
         return pool_t<float>(g, (const float *)in, (const float *)prev, out, mask, out_mask, mode, true, s);
+    if (dtype == DC_BF16)
+        return pool_t<bf16_t>(g, (const bf16_t *)in, (const bf16_t *)prev, out, mask, out_mask, mode, out_f32, s);
     return pool_t<half_t>(g, (const half_t *)in, (const half_t *)prev, out, mask, out_mask, mode, out_f32, s);
 }
 

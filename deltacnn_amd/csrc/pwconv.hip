@@ -41,11 +41,12 @@ struct PwP {
 // (mask Ma) and b = convolution output rounded to fp16 (mask Mb = input mask),
 // out = fma(b, wb, a * wa) on pixels of Ma | Mb, each term present only where its mask is set --
 // the same operations, in the same order and precision, as the stand-alone add kernel.
+template <typename E>
 struct ResP {
-    const half_t *res;
+    const E *res;
     const int32_t *mask;
     float wa, wb;
-    half_t *prev;  // MODE 2: the sum is accumulated here and its activated difference is emitted
+    E *prev;  // MODE 2: the sum is accumulated here and its activated difference is emitted
     int act;
 };
 
@@ -62,11 +63,13 @@ struct ResP {
 // workgroups).  S = reduction steps per memory round trip: all fragment loads of S steps are in
 // flight together.
 // MODE: 0 convolution only, 1 fused sum, 2 fused sum with the DCAdd layer's activation.
-template <int KW, int CBW, int NBW, int R, int NTW, int S, int MODE, bool EAGER>
+template <typename E, int KW, int CBW, int NBW, int R, int NTW, int S, int MODE, bool EAGER>
 __global__ void __launch_bounds__(KW * CBW * NBW * WAVE)
-pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
-               const half_t *__restrict__ bias, half_t *__restrict__ out,
-               const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, ResP rp) {
+pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
+               const E *__restrict__ bias, E *__restrict__ out,
+               const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, ResP<E> rp) {
+    typedef typename Elem16<E>::v4 E4;
+    typedef typename Elem16<E>::v8 E8;
     static_assert(NBW * NTW <= 4, "a workgroup covers at most 64 pixels");
     constexpr bool ADD = MODE > 0, ADDACT = MODE == 2;
     constexpr int NW = KW * CBW * NBW, TILES = R * NTW, FT = (TILES + KW - 1) / KW;
@@ -93,22 +96,22 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
     int rword = 0;
     if (ADD) rword = rp.mask[min(mp, p.P - 1)];
     const int ct0 = (by * CBW + cw) * R;
-    const half_t *wrow[R];  // fragment order: one contiguous KB per (channel tile, step)
+    const E *wrow[R];  // fragment order: one contiguous KB per (channel tile, step)
 #pragma unroll
     for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
         wrow[r] = wp + (size_t)min(ct0 + r, p.co_tiles - 1) * ksteps * 512 + lane * 8;
-    half8_t a[S][R];
+    E8 a[S][R];
 #pragma unroll
     for (int i = 0; i < S; ++i) {
         const int s = min(kw + i * KW, ksteps - 1);
 #pragma unroll
-        for (int r = 0; r < R; ++r) a[i][r] = *reinterpret_cast<const half8_t *>(wrow[r] + (s << 9));
+        for (int r = 0; r < R; ++r) a[i][r] = *reinterpret_cast<const E8 *>(wrow[r] + (s << 9));
     }
     // EAGER: the input fragments of the first chunk are requested before the masks are known
     // (one memory round trip less in the dependency chain; what inactive pixels return is
     // never stored)
-    const half_t *xrow[NTW];
-    half8_t x[S][NTW];
+    const E *xrow[NTW];
+    E8 x[S][NTW];
     if (EAGER) {
 #pragma unroll
         for (int j = 0; j < NTW; ++j)
@@ -118,7 +121,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
             const int s = min(kw + i * KW, ksteps - 1);
             const int k = min((s << 5) + kq * 8, p.Ci - 8);
 #pragma unroll
-            for (int j = 0; j < NTW; ++j) x[i][j] = *reinterpret_cast<const half8_t *>(xrow[j] + k);
+            for (int j = 0; j < NTW; ++j) x[i][j] = *reinterpret_cast<const E8 *>(xrow[j] + k);
         }
     }
     const uint64_t bm = ballot(mine && mword != 0);
@@ -129,21 +132,21 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
 
     // tiles this wavefront finishes: all of its own (KW == 1) or tiles kw, kw + KW, ... of
     // its group after the reduction
-    half4_t res[FT], bh[FT], qv[FT];
+    E4 res[FT], bh[FT], qv[FT];
 #pragma unroll
     for (int m = 0; m < FT; ++m) {
         const int t = KW > 1 ? kw + m * KW : m;
         const int r = t / NTW, j = t % NTW;
         const int co = min((ct0 + r) * 16 + kq * 4, p.Co - 4);
-        bh[m] = half4_t{0, 0, 0, 0};
-        if (bias != nullptr) bh[m] = *reinterpret_cast<const half4_t *>(bias + co);
+        bh[m] = zero4<E>();
+        if (bias != nullptr) bh[m] = *reinterpret_cast<const E4 *>(bias + co);
         if (ADD) {
             const int bit = (nw * NTW + j) * 16 + l16;
             const bool on_r = t < TILES && ((br >> bit) & 1);
-            res[m] = *reinterpret_cast<const half4_t *>(rp.res + (size_t)(on_r ? pbase + bit : 0) * p.Co + co);
+            res[m] = *reinterpret_cast<const E4 *>(rp.res + (size_t)(on_r ? pbase + bit : 0) * p.Co + co);
             if (ADDACT) {
                 const bool on_o = t < TILES && ((bo >> bit) & 1);
-                qv[m] = *reinterpret_cast<const half4_t *>(rp.prev + (size_t)(on_o ? pbase + bit : 0) * p.Co + co);
+                qv[m] = *reinterpret_cast<const E4 *>(rp.prev + (size_t)(on_o ? pbase + bit : 0) * p.Co + co);
             }
         }
     }
@@ -172,7 +175,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
                     const int s = min(s0 + i * KW, ksteps - 1);
 #pragma unroll
                     for (int r = 0; r < R; ++r)
-                        a[i][r] = *reinterpret_cast<const half8_t *>(wrow[r] + (s << 9));
+                        a[i][r] = *reinterpret_cast<const E8 *>(wrow[r] + (s << 9));
                 }
             }
             if (!EAGER || s0 != kw) {
@@ -181,7 +184,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
                     const int s = min(s0 + i * KW, ksteps - 1);
                     const int k = min((s << 5) + kq * 8, p.Ci - 8);
 #pragma unroll
-                    for (int j = 0; j < NTW; ++j) x[i][j] = *reinterpret_cast<const half8_t *>(xrow[j] + k);
+                    for (int j = 0; j < NTW; ++j) x[i][j] = *reinterpret_cast<const E8 *>(xrow[j] + k);
                 }
             }
             // No zero-fill is needed: columns of inactive pixels are never stored, and where a
@@ -195,7 +198,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
                         if (nt_on[j]) {  // wave-uniform
 #pragma unroll
                             for (int r = 0; r < R; ++r)
-                                acc[r][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][r], x[i][j], acc[r][j], 0, 0, 0);
+                                acc[r][j] = Elem16<E>::mfma(a[i][r], x[i][j], acc[r][j]);
                         }
                 }
             }
@@ -222,7 +225,7 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
         for (int m = 0; m < FT; ++m) fin[m] = acc[m / NTW][m % NTW];
     }
 
-    const half_t wa = half_t(rp.wa), wb = half_t(rp.wb);
+    const E wa = E(rp.wa), wb = E(rp.wb);
 #pragma unroll
     for (int m = 0; m < FT; ++m) {
         const int t = KW > 1 ? kw + m * KW : m;
@@ -234,22 +237,22 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
         const bool on = (bm >> bit) & 1, on_r = (br >> bit) & 1;
         if (!(on || on_r)) continue;
         const float4_t v = fin[m] + float4_t{float(bh[m][0]), float(bh[m][1]), float(bh[m][2]), float(bh[m][3])};
-        half4_t o = half4_t{half_t(v[0]), half_t(v[1]), half_t(v[2]), half_t(v[3])};
+        E4 o = E4{E(v[0]), E(v[1]), E(v[2]), E(v[3])};
         if (ADD) {  // add_kernel's sequence: s = a * wa; s = fma(b, wb, s); n = s + prev; ...
-            half4_t qn;
+            E4 qn;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                half_t sum = on_r ? half_t(res[m][i] * wa) : half_t(0);
+                E sum = on_r ? E(res[m][i] * wa) : E(0);
                 if (on) sum = fma_t(o[i], wb, sum);
                 if (ADDACT) {
                     qn[i] = sum + qv[m][i];
-                    sum = act_apply<half_t>(qn[i], rp.act) - act_apply<half_t>(qv[m][i], rp.act);
+                    sum = act_apply<E>(qn[i], rp.act) - act_apply<E>(qv[m][i], rp.act);
                 }
                 o[i] = sum;
             }
-            if (ADDACT) *reinterpret_cast<half4_t *>(rp.prev + (size_t)(pbase + bit) * p.Co + co) = qn;
+            if (ADDACT) *reinterpret_cast<E4 *>(rp.prev + (size_t)(pbase + bit) * p.Co + co) = qn;
         }
-        *reinterpret_cast<half4_t *>(out + (size_t)(pbase + bit) * p.Co + co) = o;
+        *reinterpret_cast<E4 *>(out + (size_t)(pbase + bit) * p.Co + co) = o;
     }
 }
 
@@ -261,11 +264,11 @@ pw_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ 
 // the filter stream of a wavefront is one uninterrupted run of loads.  Requires Cout % 4 == 0.
 // Pass 1 of the epilogue: conv output v (rounded to fp16), T = trunc + v, S = T + prev,
 // D = act(S) - act(prev), one rounding each; collects the keep statistics of this lane.
-template <int CTW, int ACT>
-__device__ __forceinline__ void pw_epilogue_stats(const float4_t (&acc)[CTW], const half4_t (&q)[CTW],
-                                                  const half4_t (&tr)[CTW], half4_t (&v)[CTW],
-                                                  const half4_t (&bh)[CTW], bool on, int wave,
-                                                  int NW, int kq, const PwP &p, half_t thr, bool norm,
+template <typename E, int CTW, int ACT>
+__device__ __forceinline__ void pw_epilogue_stats(const float4_t (&acc)[CTW], const typename Elem16<E>::v4 (&q)[CTW],
+                                                  const typename Elem16<E>::v4 (&tr)[CTW], typename Elem16<E>::v4 (&v)[CTW],
+                                                  const typename Elem16<E>::v4 (&bh)[CTW], bool on, int wave,
+                                                  int NW, int kq, const PwP &p, E thr, bool norm,
                                                   bool &hit, float &sq) {
 #pragma unroll
     for (int j = 0; j < CTW; ++j) {
@@ -276,10 +279,10 @@ __device__ __forceinline__ void pw_epilogue_stats(const float4_t (&acc)[CTW], co
         const float4_t r = acc[j] + float4_t{float(bh[j][0]), float(bh[j][1]), float(bh[j][2]), float(bh[j][3])};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            v[j][i] = half_t(r[i]);
-            const half_t t = tr[j][i] + v[j][i];
-            const half_t s = t + q[j][i];
-            const half_t d = act_apply<half_t>(s, ACT) - act_apply<half_t>(q[j][i], ACT);
+            v[j][i] = E(r[i]);
+            const E t = tr[j][i] + v[j][i];
+            const E s = t + q[j][i];
+            const E d = act_apply<E>(s, ACT) - act_apply<E>(q[j][i], ACT);
             if (live && on) {
                 hit |= tabs(d) > thr;
                 if (norm) sq += float(d) * float(d);  // uniform: only the norm modes need it
@@ -290,12 +293,13 @@ __device__ __forceinline__ void pw_epilogue_stats(const float4_t (&acc)[CTW], co
 
 // Pass 2: recompute T, S, D (a handful of ALU operations, cheaper than keeping them in
 // registers across the workgroup barrier) and write the kept / dropped state.
-template <int CTW, int ACT>
-__device__ __forceinline__ void pw_epilogue_store(const half4_t (&q)[CTW], const half4_t (&tr)[CTW],
-                                                  const half4_t (&v)[CTW], bool keep, int wave, int NW,
+template <typename E, int CTW, int ACT>
+__device__ __forceinline__ void pw_epilogue_store(const typename Elem16<E>::v4 (&q)[CTW], const typename Elem16<E>::v4 (&tr)[CTW],
+                                                  const typename Elem16<E>::v4 (&v)[CTW], bool keep, int wave, int NW,
                                                   int kq, int px, const PwP &p,
-                                                  half_t *__restrict__ out, half_t *__restrict__ prev,
-                                                  half_t *__restrict__ trunc) {
+                                                  E *__restrict__ out, E *__restrict__ prev,
+                                                  E *__restrict__ trunc) {
+    typedef typename Elem16<E>::v4 E4;
 #pragma unroll
     for (int j = 0; j < CTW; ++j) {
         const int ct = wave + j * NW;
@@ -303,19 +307,19 @@ __device__ __forceinline__ void pw_epilogue_store(const half4_t (&q)[CTW], const
         const int co = ct * 16 + kq * 4;
         if (co >= p.Co) continue;
         const size_t off = (size_t)px * p.Co + co;
-        half4_t t, s, d;
+        E4 t, s, d;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             t[i] = tr[j][i] + v[j][i];
             s[i] = t[i] + q[j][i];
-            d[i] = act_apply<half_t>(s[i], ACT) - act_apply<half_t>(q[j][i], ACT);
+            d[i] = act_apply<E>(s[i], ACT) - act_apply<E>(q[j][i], ACT);
         }
         if (keep) {
-            *reinterpret_cast<half4_t *>(prev + off) = s;
-            *reinterpret_cast<half4_t *>(out + off) = d;
-            *reinterpret_cast<half4_t *>(trunc + off) = half4_t{0, 0, 0, 0};
+            *reinterpret_cast<E4 *>(prev + off) = s;
+            *reinterpret_cast<E4 *>(out + off) = d;
+            *reinterpret_cast<E4 *>(trunc + off) = zero4<E>();
         } else {
-            *reinterpret_cast<half4_t *>(trunc + off) = t;
+            *reinterpret_cast<E4 *>(trunc + off) = t;
         }
     }
 }
@@ -338,12 +342,14 @@ __device__ __forceinline__ void pw_epilogue_store(const half4_t (&q)[CTW], const
 // the stores.  Longer reductions stream two steps per round trip in ascending order (the same
 // summation order as the convolution-only kernel without reduction split).  What is loaded
 // for inactive pixels is dropped.  Requires Cout % 4 == 0.
-template <int NW, int CTW, int ACT>
+template <typename E, int NW, int CTW, int ACT>
 __global__ void __launch_bounds__(NW * WAVE)
-pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
-                   const half_t *__restrict__ bias, half_t *__restrict__ out,
+pw_act_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
+                   const E *__restrict__ bias, E *__restrict__ out,
                    const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
-                   half_t *__restrict__ prev, half_t *__restrict__ trunc, float thr_f, int mode) {
+                   E *__restrict__ prev, E *__restrict__ trunc, float thr_f, int mode) {
+    typedef typename Elem16<E>::v4 E4;
+    typedef typename Elem16<E>::v8 E8;
     constexpr int S = 2;
     __shared__ float s_stat[NW][16];
     const int wave = wave_id(), lane = lane_id();
@@ -356,28 +362,28 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
     // while the cached state of the whole map is a few MB: reading it for inactive pixels too
     // costs less than a second memory round trip).
     const int pl = pxc;
-    const half_t *wrow[CTW];
+    const E *wrow[CTW];
 #pragma unroll
     for (int j = 0; j < CTW; ++j)
         wrow[j] = wp + (size_t)min(wave + j * NW, p.co_tiles - 1) * ksteps * 512 + lane * 8;
-    const half_t *xrow = in + (size_t)pl * p.Ci;
-    half8_t a[S][CTW], x[S];
+    const E *xrow = in + (size_t)pl * p.Ci;
+    E8 a[S][CTW], x[S];
 #pragma unroll
     for (int i = 0; i < S; ++i) {
         const int s = min(i, ksteps - 1);
-        x[i] = *reinterpret_cast<const half8_t *>(xrow + min((s << 5) + kq * 8, p.Ci - 8));
+        x[i] = *reinterpret_cast<const E8 *>(xrow + min((s << 5) + kq * 8, p.Ci - 8));
 #pragma unroll
-        for (int j = 0; j < CTW; ++j) a[i][j] = *reinterpret_cast<const half8_t *>(wrow[j] + (s << 9));
+        for (int j = 0; j < CTW; ++j) a[i][j] = *reinterpret_cast<const E8 *>(wrow[j] + (s << 9));
     }
-    half4_t q[CTW], tr[CTW], bh[CTW];
+    E4 q[CTW], tr[CTW], bh[CTW];
 #pragma unroll
     for (int j = 0; j < CTW; ++j) {
         const int co = min(min(wave + j * NW, p.co_tiles - 1) * 16 + kq * 4, p.Co - 4);
         const size_t off = (size_t)pl * p.Co + co;
-        q[j] = *reinterpret_cast<const half4_t *>(prev + off);
-        tr[j] = *reinterpret_cast<const half4_t *>(trunc + off);
-        bh[j] = half4_t{0, 0, 0, 0};
-        if (bias != nullptr) bh[j] = *reinterpret_cast<const half4_t *>(bias + co);
+        q[j] = *reinterpret_cast<const E4 *>(prev + off);
+        tr[j] = *reinterpret_cast<const E4 *>(trunc + off);
+        bh[j] = zero4<E>();
+        if (bias != nullptr) bh[j] = *reinterpret_cast<const E4 *>(bias + co);
     }
     // all of the above is in flight before anything is waited for
 #pragma unroll
@@ -406,10 +412,10 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
 #pragma unroll
             for (int i = 0; i < S; ++i) {
                 const int s = min(s0 + i, ksteps - 1);
-                x[i] = *reinterpret_cast<const half8_t *>(xrow + min((s << 5) + kq * 8, p.Ci - 8));
+                x[i] = *reinterpret_cast<const E8 *>(xrow + min((s << 5) + kq * 8, p.Ci - 8));
 #pragma unroll
                 for (int j = 0; j < CTW; ++j)
-                    a[i][j] = *reinterpret_cast<const half8_t *>(wrow[j] + (s << 9));
+                    a[i][j] = *reinterpret_cast<const E8 *>(wrow[j] + (s << 9));
             }
 #pragma unroll
             for (int i = 0; i < S; ++i) {
@@ -423,15 +429,15 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
             if (s0 + i < ksteps) {  // uniform
 #pragma unroll
                 for (int j = 0; j < CTW; ++j)
-                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][j], x[i], acc[j], 0, 0, 0);
+                    acc[j] = Elem16<E>::mfma(a[i][j], x[i], acc[j]);
             }
         }
     }
-    const half_t thr = half_t(thr_f);
-    half4_t v[CTW];
+    const E thr = E(thr_f);
+    E4 v[CTW];
     bool hit = false;
     float sq = 0.f;
-    pw_epilogue_stats<CTW, ACT>(acc, q, tr, v, bh, on, wave, NW, kq, p, thr, mode != DC_TRUNC_MAX, hit, sq);
+    pw_epilogue_stats<E, CTW, ACT>(acc, q, tr, v, bh, on, wave, NW, kq, p, thr, mode != DC_TRUNC_MAX, hit, sq);
     // per pixel: combine the four k-quarter lanes, then the wavefronts
     float stat;
     if (mode == DC_TRUNC_MAX) {
@@ -452,13 +458,13 @@ pw_act_mfma_kernel(PwP p, const half_t *__restrict__ in, const half_t *__restric
     else keep = sqrtf(mode == DC_TRUNC_RMS ? tot / float(p.Co) : tot) > float(thr);
     if (wave == 0 && kq == 0 && px < p.P) out_mask[px] = (on && keep) ? 1 : 0;
     if (!on) return;
-    pw_epilogue_store<CTW, ACT>(q, tr, v, keep, wave, NW, kq, px, p, out, prev, trunc);
+    pw_epilogue_store<E, CTW, ACT>(q, tr, v, keep, wave, NW, kq, px, p, out, prev, trunc);
 }
 
 }  // namespace
 
 bool pointwise_eligible(const dc_geometry &g, int dtype) {
-    return dtype == DC_F16 && g.groups == 1 && g.in_c % 8 == 0 && g.in_c >= 8 && g.out_c % 4 == 0 &&
+    return (dtype == DC_F16 || dtype == DC_BF16) && g.groups == 1 && g.in_c % 8 == 0 && g.in_c >= 8 && g.out_c % 4 == 0 &&
            g.kernel_h == 1 &&
            g.kernel_w == 1 && g.stride_h == 1 && g.stride_w == 1 && g.pad_top == 0 &&
            g.pad_left == 0 && g.pad_bottom == 0 && g.pad_right == 0;
@@ -509,10 +515,12 @@ int pointwise_reduction_slices(int pixels, int in_c, int out_c) {
     return 1;
 }
 
-hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *packed,
-                            const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
-                            const ActEpilogue *epi, bool *epilogue_done, const Residual *res,
-                            hipStream_t s) {
+namespace {
+template <typename E>
+hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *packed,
+                              const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
+                              const ActEpilogue *epi, bool *epilogue_done, const Residual *res,
+                              hipStream_t s) {
     PwP p;
     p.P = g.batch * g.in_h * g.in_w;
     p.Ci = g.in_c;
@@ -549,10 +557,10 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
         const int ctw = ceil_div(p.co_tiles, nw);
 #define DC_GO(NW, CTW)                                                                                \
     do {                                                                                              \
-        DC_ACT_SWITCH(act, (pw_act_mfma_kernel<NW, CTW, A><<<grid, NW * WAVE, 0, s>>>(                \
-                               p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias,   \
-                               (half_t *)out, mask, out_mask, (half_t *)epi->prev,                    \
-                               (half_t *)epi->trunc, epi->thr, epi->mode)));                          \
+        DC_ACT_SWITCH(act, (pw_act_mfma_kernel<E, NW, CTW, A><<<grid, NW * WAVE, 0, s>>>(                \
+                               p, (const E *)in, (const E *)packed, (const E *)bias,   \
+                               (E *)out, mask, out_mask, (E *)epi->prev,                    \
+                               (E *)epi->trunc, epi->thr, epi->mode)));                          \
         *epilogue_done = true;                                                                        \
         return hipGetLastError();                                                                     \
     } while (0)
@@ -562,8 +570,8 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
         if (ctw == 2) DC_GO(16, 2);  // 32 KB of filter: at most 32 channel tiles
 #undef DC_GO
     }
-    ResP rp{nullptr, nullptr, 1.f, 1.f, nullptr, 0};
-    if (res != nullptr) rp = ResP{(const half_t *)res->values, res->mask, res->wa, res->wb, (half_t *)res->prev, res->act};
+    ResP<E> rp{nullptr, nullptr, 1.f, 1.f, nullptr, 0};
+    if (res != nullptr) rp = ResP<E>{(const E *)res->values, res->mask, res->wa, res->wb, (E *)res->prev, res->act};
     const int cfg = pick_config(p, ksteps);
     note_kernel("pw_mfma_kernel");
 #define DC_PW_S(KW, CBW, NBW, R, NTW, EA, SS)                                                        \
@@ -574,14 +582,14 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
         p.xcd = (p.nx % 8 != 0 && p.ny > 1 && (int64_t)p.ci_p * p.Co > (int64_t)p.P * p.Ci) ? 1 : 0; \
         dim3 grid(p.xcd ? p.nx * ((p.ny + 7) / 8 * 8) : p.nx, p.xcd ? 1 : p.ny);                     \
         if (res != nullptr && res->act > 0)                                                          \
-            pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, 2, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
-                p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
+            pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 2, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
         else if (res != nullptr)                                                                     \
-            pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, 1, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
-                p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
+            pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 1, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
         else                                                                                         \
-            pw_mfma_kernel<KW, CBW, NBW, R, NTW, SS, 0, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
-                p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, rp); \
+            pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 0, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
     } while (0)
 #define DC_PW(ID, KW, CBW, NBW, R, NTW, EA)                                                          \
     case ID: {                                                                                       \
@@ -598,6 +606,16 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
 #undef DC_PW
 #undef DC_PW_S
     return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *packed,
+                            const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
+                            const ActEpilogue *epi, bool *epilogue_done, const Residual *res,
+                            int dtype, hipStream_t s) {
+    if (dtype == DC_BF16)
+        return launch_pointwise_t<bf16_t>(g, in, packed, bias, out, mask, out_mask, epi, epilogue_done, res, s);
+    return launch_pointwise_t<half_t>(g, in, packed, bias, out, mask, out_mask, epi, epilogue_done, res, s);
 }
 
 }  // namespace dc

@@ -9,6 +9,8 @@ either implementation are interchangeable:
 * fp16 otherwise Cin and Cout padded to even with zeros, then every 2x2 block of
   (input pair, output pair) is swizzled so that ``W[ci, co]`` lives at row
   ``ci ^ (co & 1)``                                                     (filter_conversion.py:26-37)
+* bfloat16       (no counterpart in the reference) the fp32 layouts in bfloat16: no padding, no
+  swizzle -- ``convert_filter_out_channels_last`` on the bfloat16 weights
 """
 from __future__ import annotations
 

@@ -12,9 +12,9 @@ from typing import Optional, Sequence
 import torch
 
 from . import _lib
-from ._lib import DC_F16, DC_F32, Geometry
+from ._lib import DC_BF16, DC_F16, DC_F32, Geometry
 
-_DTYPES = {torch.float32: DC_F32, torch.float16: DC_F16}
+_DTYPES = {torch.float32: DC_F32, torch.float16: DC_F16, torch.bfloat16: DC_BF16}
 
 # Optional per-call tracer (see deltacnn_amd/trace.py): when set, every library call goes
 # through ``tracer.run(op, fn, args, meta)`` which brackets it with events and records the
@@ -38,7 +38,7 @@ def _dtype(t: torch.Tensor) -> int:
     try:
         return _DTYPES[t.dtype]
     except KeyError:
-        raise _lib.DeltaCNNError(-1, f"unsupported dtype {t.dtype} (float32 and float16 only)")
+        raise _lib.DeltaCNNError(-1, f"unsupported dtype {t.dtype} (float32, float16 and bfloat16 only)")
 
 
 def _nhwc(t: torch.Tensor, name: str) -> torch.Tensor:
@@ -174,13 +174,13 @@ def sparse_conv_add(x, packed_filter, mask, bias, residual, mask_residual, geome
     lib = _lib.load()
     _nhwc(x, "x")
     _nhwc(residual, "residual")
-    if packed_filter is None or x.dtype != torch.float16:
+    if packed_filter is None or x.dtype not in (torch.float16, torch.bfloat16):
         return None
     activation = max(int(activation), 0)
     args = (geometry, x.data_ptr(), packed_filter.data_ptr(), _ptr(bias), _mask(mask, "mask").data_ptr(),
             residual.data_ptr(), _mask(mask_residual, "mask_residual").data_ptr(), out.data_ptr(),
             out_mask.data_ptr(), float(weight_residual), float(weight_conv), _ptr(prev_out), activation,
-            DC_F16, _stream())
+            _dtype(x), _stream())
     meta = dict(g=geometry, esize=2, in_mask=mask, in_mask_b=mask_residual, out_mask=out_mask, mfma=True)
     try:
         _call("conv_add", lib.dc_conv_add, args, **meta)
@@ -248,18 +248,19 @@ def pack_filter(filter: torch.Tensor, c_in: int, c_out: int, groups: int = 1,
                 transposed: bool = False) -> Optional[torch.Tensor]:
     """One-time relayout of a processed fp16 filter for the MFMA kernels; None if the shape
     has no packed form (fp32, grouped, or an input channel count that is neither a multiple
-    of 8 nor a stem's: Cin <= 4 with a window up to 8 x 8 and Cout <= 64)."""
+    of 8 nor a stem's: Cin <= 4 with a window up to 8 x 8 and Cout <= 64).  bfloat16 filters
+    (fp32 layout) have a packed form for 1x1 convolutions only."""
     lib = _lib.load()
-    if filter.dtype != torch.float16:
+    if filter.dtype not in (torch.float16, torch.bfloat16):
         return None
+    dt = _dtype(filter)
     g = Geometry(1, 1, 1, c_in, 1, 1, c_out, filter.shape[1], filter.shape[2], 1, 1, 1, 1, 0, 0, 0,
                  0, groups)
-    nbytes = lib.dc_packed_filter_bytes(g, DC_F16, int(transposed))
+    nbytes = lib.dc_packed_filter_bytes(g, dt, int(transposed))
     if nbytes == 0:
         return None
-    packed = torch.empty(nbytes // 2, dtype=torch.float16, device=filter.device)
-    _lib.check(lib.dc_pack_filter(g, filter.data_ptr(), packed.data_ptr(), DC_F16, int(transposed),
-                                  _stream()))
+    packed = torch.empty(nbytes // 2, dtype=filter.dtype, device=filter.device)
+    _lib.check(lib.dc_pack_filter(g, filter.data_ptr(), packed.data_ptr(), dt, int(transposed), _stream()))
     return packed
 
 

@@ -6,7 +6,7 @@
  * `deltacnn.cuda` (src/cuda/conv_torch_wrapper.cpp:640-655).  Conventions:
  *
  *   - feature tensors are NHWC (torch.channels_last) device pointers, element type
- *     given by `dtype` (DC_F32 or DC_F16); masks are dense int32 [B*H*W] device
+ *     given by `dtype` (DC_F32, DC_F16 or DC_BF16); masks are dense int32 [B*H*W] device
  *     pointers, a pixel is active iff its word != 0
  *   - the library never allocates, frees or retains memory; pointers are borrowed
  *     for the duration of the asynchronous launch on `stream` (a hipStream_t, NULL =
@@ -31,7 +31,7 @@ extern "C" {
 
 typedef enum dc_status {
     DC_OK = 0,
-    DC_ERR_DTYPE = -1,       /* dtype not DC_F32 / DC_F16 */
+    DC_ERR_DTYPE = -1,       /* dtype not DC_F32 / DC_F16 / DC_BF16 */
     DC_ERR_SHAPE = -2,       /* non-positive or inconsistent dimensions */
     DC_ERR_UNSUPPORTED = -3, /* valid but not implemented configuration */
     DC_ERR_NULL = -4,        /* required pointer is NULL */
@@ -39,7 +39,10 @@ typedef enum dc_status {
     DC_ERR_LAUNCH = -6       /* HIP reported a launch error */
 } dc_status;
 
-enum { DC_F32 = 0, DC_F16 = 1 };
+/* DC_BF16: bfloat16 has no counterpart in the reference (readme.md:228, fp16 and fp32 only); every
+ * operator follows the fp16 rules with two exceptions: sparsify compares with > for any channel
+ * count, and filters use the fp32 layout [Cin/g][Kh][Kw][Cout] (no padding, no pair swizzle). */
+enum { DC_F32 = 0, DC_F16 = 1, DC_BF16 = 2 };
 
 /* activation ids of convert_activation_string (sparse_layers.py:20-34); <= 0 is linear */
 enum { DC_ACT_LINEAR = 0, DC_ACT_RELU = 1, DC_ACT_RELU6 = 2, DC_ACT_LEAKY = 3,

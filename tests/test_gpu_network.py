@@ -21,16 +21,16 @@ def _models(builder, dtype, thr, state=None, **kw):
     dense = builder(DenseLayers, **kw).eval()
     if state is not None:
         dense.load_state_dict(state)
-    if dtype == torch.float16:  # oracle and HIP model share weights that are exact in fp16
-        dense = dense.half().float()
+    if dtype != torch.float32:  # oracle and HIP model share weights that are exact in the 16-bit type
+        dense = dense.to(dtype).float()
     ref = builder(OL, **kw).eval()
     ref.load_state_dict(dense.state_dict())
     dut = builder(SL, **kw).eval()
     dut.load_state_dict(dense.state_dict())
     dut = dut.to(DEV, memory_format=torch.channels_last)
-    if dtype == torch.float16:
-        ref = ref.half()
-        dut = dut.half()
+    if dtype != torch.float32:
+        ref = ref.to(dtype)
+        dut = dut.to(dtype)
     dut.process_filters()
     return dense, ref, dut
 

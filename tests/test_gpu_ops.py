@@ -11,7 +11,9 @@ from util import DEV, assert_masked_close, assert_masked_equal, cl, packed_form_
 
 pytestmark = pytest.mark.gpu
 
-DTYPES = [torch.float32, torch.float16]
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+# tolerance of results that pass through a transcendental or a reordered float sum: a few steps of the type
+LOOSE = {torch.float32: 1e-5, torch.float16: 2e-3, torch.bfloat16: 1.6e-2}
 CHANNELS = [1, 3, 4, 8, 16, 31, 32, 33, 64, 96, 130, 256, 960, 1280, 2100]
 
 
@@ -186,7 +188,7 @@ def test_activate_truncate_transcendental(lib, dtype, act):
     d_delta, d_prev, d_trunc, d_mask = cl(poison(delta, mask)), cl(prev), cl(trunc), cl(mask)
     hk().sparse_activation(d_delta, d_prev, d_trunc, d_mask, thr, act, 0)
     assert torch.equal(d_mask.cpu(), w_mask)
-    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    tol = LOOSE[dtype]
     assert_masked_close(d_delta, w_delta, w_mask, tol, tol, "delta")
 
 
@@ -375,6 +377,8 @@ def _conv_case(dtype, cfg, seed, density, transposed=False):
 def _check_conv(dtype, got, want, want_mask):
     if dtype == torch.float32:
         assert_masked_close(got, want, want_mask, 1e-4, 1e-5, "out")
+    elif dtype == torch.bfloat16:  # one bfloat16 step is 2^-8 of the value: 2e-2 absolute or two steps
+        assert_masked_close(got, want, want_mask, 2.0 ** -7, 2e-2, "out")
     else:
         assert_masked_close(got, want, want_mask, 0, 2e-2, "out")
 
@@ -434,6 +438,24 @@ def test_conv_dispatch(lib, cfg, kernel):
     x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(torch.float16, cfg, 5, 0.5)
     d_filt = filt.to(DEV)
     pk = hk().pack_filter(d_filt, Cin, Cout, groups)
+    hk().sparse_conv(cl(x), d_filt, cl(mask), None, s, p, d, groups, c_out=Cout, create_out_mask=True, packed_filter=pk)
+    assert _lib.load().dc_last_kernels().decode() == kernel
+
+
+@pytest.mark.parametrize("cfg,kernel", [
+    ((64, 256, 1, 1, 0, 1, 1, 20, 20), "pw_mfma_kernel"),          # 1x1: the matrix cores (v_mfma_f32_16x16x32_bf16)
+    ((576, 96, 1, 1, 0, 1, 1, 14, 14), "pw_mfma_kernel"),
+    ((64, 64, 3, 1, 1, 1, 1, 40, 40), "conv_direct_kernel"),       # K x K windows: the generic kernel
+    ((32, 32, 3, 1, 1, 1, 32, 15, 18), "conv_dw_kernel"),
+    ((3, 32, 3, 2, 1, 1, 1, 33, 31), "conv_fewcin_kernel"),
+], ids=lambda v: v if isinstance(v, str) else "-".join(str(x) for x in v))
+def test_conv_dispatch_bfloat16(lib, cfg, kernel):
+    from deltacnn_amd import _lib
+    Cin, Cout, groups = cfg[0], cfg[1], cfg[6]
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(torch.bfloat16, cfg, 5, 0.5)
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, Cin, Cout, groups)
+    assert (pk is not None) == (K == (1, 1))
     hk().sparse_conv(cl(x), d_filt, cl(mask), None, s, p, d, groups, c_out=Cout, create_out_mask=True, packed_filter=pk)
     assert _lib.load().dc_last_kernels().decode() == kernel
 
@@ -550,12 +572,12 @@ def test_conv_activation_fused(lib, dtype, cfg, act, mode):
 @pytest.mark.parametrize("cfg", [(96, 24, 56, 56), (144, 32, 28, 28), (384, 64, 14, 14), (960, 160, 7, 7),
                                  (32, 20, 9, 9)], ids=lambda c: "-".join(str(v) for v in c))
 @pytest.mark.parametrize("weights", [(1.0, 1.0), (0.5, -1.5)])
-def test_conv_add_fused(lib, cfg, weights):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_conv_add_fused(lib, cfg, weights, dtype):
     """dc_conv_add == DCAdd(residual, conv(x)) of the oracle, and bit-identical to the two
     separate library calls."""
     from deltacnn_amd.hip_kernels import conv_geometry
     Cin, Cout, H, W = cfg
-    dtype = torch.float16
     x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, (Cin, Cout, 1, 1, 0, 1, 1, H, W), 91, 0.3)
     g = _gen(92)
     mres = rand_mask(g, 2, H, W, 0.3)
@@ -571,7 +593,7 @@ def test_conv_add_fused(lib, cfg, weights):
     got = hk().sparse_conv_add(dx, pk, dm, None, dres, dmres, geo, out, om, weights[0], weights[1])
     assert got is not None
     assert torch.equal(om.cpu(), want_mask)
-    assert_masked_close(out, want, want_mask, 0, 2e-2, "out")
+    _check_conv(dtype, out, want, want_mask)
     c_out, c_mask = hk().sparse_conv(dx, d_filt, dm, None, s, p, d, 1, c_out=Cout, create_out_mask=True, packed_filter=pk)
     two = torch.empty_like(out)
     two_mask = torch.empty_like(om)
@@ -734,7 +756,7 @@ def test_pool_global(lib, dtype, mode, C, H, W, density):
     assert out.dtype == dtype and out.shape == (B, C, 1, 1)
     assert torch.equal(om.cpu(), want_mask)
     # the average is a float sum over up to H*W values in a different order than the oracle's
-    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    tol = LOOSE[dtype]
     assert_masked_close(out, want, want_mask, tol, tol, "out")
     # the reference's protocol: float32 accumulator handed in by the caller, cast afterwards
     acc = torch.full((B, C, 1, 1), float("nan"), dtype=torch.float32, device=DEV).contiguous(
@@ -758,7 +780,7 @@ def test_scanned_simple_operators(lib, dtype, density):
     kernels (channel counts that fill, underfill and split a lane group)."""
     g = _gen(int(1500 + 100 * density))
     B, H, W = 2, 397, 333
-    for C in (24, 64) if dtype == torch.float16 else (12, 40):
+    for C in (24, 64) if dtype != torch.float32 else (12, 40):
         mask = rand_mask(g, B, H, W, density)
         x = torch.randn(B, C, H, W, generator=g).to(dtype)
         scale, bias = torch.randn(C, generator=g).to(dtype), torch.randn(C, generator=g).to(dtype)

@@ -43,13 +43,15 @@ def _compare(kind, got, want, dtype, where):
             assert_masked_equal(g, w, wm, where)
         elif dtype == torch.float32:
             assert_masked_close(g, w, wm, 1e-4, 1e-5, where)
+        elif dtype == torch.bfloat16:  # one bfloat16 step is 2^-8 of the value
+            assert_masked_close(g, w, wm, 2.0 ** -7, 2e-2, where)
         else:
             assert_masked_close(g, w, wm, 2.0 ** -9, 2e-2, where)
     else:
         if kind == "exact":
             assert torch.equal(got.cpu(), want), f"{where}: max diff {float((got.cpu().float() - want.float()).abs().max())}"
         else:
-            tol = 1e-4 if dtype == torch.float32 else 2e-2
+            tol = {torch.float32: 1e-4, torch.float16: 2e-2, torch.bfloat16: 4e-2}[dtype]
             assert float((got.cpu().float() - want.float()).abs().max()) <= tol * max(1.0, float(want.abs().max())), where
 
 
@@ -94,7 +96,7 @@ def _build(builder, dtype, thr, state=None, **kw):
     return ref, dut
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_mobilenet_teacher_forced_32_frames(lib, dtype):
     from deltacnn_amd.video import moving_rectangles_video
     from test_gpu_network import _calibrated_state, _mobilenet
@@ -104,7 +106,7 @@ def test_mobilenet_teacher_forced_32_frames(lib, dtype):
     assert n == 33 * (1 + 52 + 35 + 10 + 1 + 1)  # sparsify, convs, activations, adds, pool, densify
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_toy_cnn_teacher_forced(lib, dtype):
     from deltacnn_amd.networks import ToyCNN
     from deltacnn_amd.video import noise_block_video
@@ -114,7 +116,7 @@ def test_toy_cnn_teacher_forced(lib, dtype):
 
 
 @pytest.mark.parametrize("network", ["hrnet", "dla34"])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_multibranch_teacher_forced(lib, network, dtype):
     """Every layer call of HRNet (strided exchange convolutions, nearest upsampling, chained sums
     with ReLU) and of DLA-34 + CenterNet heads (max-pooling, concatenating roots, transposed

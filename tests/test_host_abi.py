@@ -175,7 +175,7 @@ def test_packed_form_rule_matches_the_library(lib):
     import sys
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     from util import packed_form_exists
-    from deltacnn_amd._lib import DC_F16, DC_F32, Geometry
+    from deltacnn_amd._lib import DC_BF16, DC_F16, DC_F32, Geometry
     for cin in (1, 3, 4, 5, 8, 12, 16, 24, 40, 320):
         for cout in (2, 4, 16, 30, 64, 68, 256):
             for k in (1, 3, 7, 8, 9):
@@ -183,7 +183,7 @@ def test_packed_form_rule_matches_the_library(lib):
                     if cin % groups or cout % groups:
                         continue
                     for transposed in (False, True):
-                        for dtype, code in ((torch.float16, DC_F16), (torch.float32, DC_F32)):
+                        for dtype, code in ((torch.float16, DC_F16), (torch.float32, DC_F32), (torch.bfloat16, DC_BF16)):
                             g = Geometry(1, 1, 1, cin, 1, 1, cout, k, k, 1, 1, 1, 1, 0, 0, 0, 0, groups)
                             have = lib.dc_packed_filter_bytes(g, code, int(transposed)) != 0
                             assert have == packed_form_exists(dtype, cin, cout, k, groups, transposed), \
