@@ -262,7 +262,7 @@ bool pointwise_eligible(const dc_geometry &g, int dtype);
 bool patch_eligible(const dc_geometry &g, int dtype);
 hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *packed,
                              const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
-                             bool transposed, const Residual *res, hipStream_t s,
+                             bool transposed, const Residual *res, int dtype, hipStream_t s,
                              const ActEpilogue *epi = nullptr, bool *epilogue_done = nullptr);
 hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *packed,
                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,

@@ -726,12 +726,14 @@ conv_fewcin_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filt
 //     selection afterwards -- unlike the pointwise case they would reach valid outputs.
 constexpr int MFMA_MAX_TAPS = 64;
 
-template <bool TR, int KW, int R, int S>
+template <typename E, bool TR, int KW, int R, int S>
 __global__ void __launch_bounds__(KW * WAVE)
-conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
-                 const half_t *__restrict__ bias, half_t *__restrict__ out,
+conv_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp,
+                 const E *__restrict__ bias, E *__restrict__ out,
                  const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, int co_blocks,
                  int ci_p) {
+    typedef typename Elem16<E>::v4 E4;
+    typedef typename Elem16<E>::v8 E8;
     constexpr int NT = 4;
     __shared__ int s_list[TILE_PX];
     __shared__ int s_n;
@@ -754,7 +756,7 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
     const int K2 = p.Kh * p.Kw;
     const int n_tiles = (n + 15) >> 4;
     const int co_tiles = (p.Co + 15) >> 4;
-    const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+    const E *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
 
     float4_t acc[R][NT];
 #pragma unroll
@@ -763,13 +765,13 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
         for (int nt = 0; nt < NT; ++nt) acc[r][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
     const int ksteps = ci_p >> 5;
     const int total = s_ntaps * ksteps;  // steps over the taps in use only
-    const half_t *wfrag[R];
+    const E *wfrag[R];
 #pragma unroll
     for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
         wfrag[r] = wp + (size_t)min(cb * R + r, co_tiles - 1) * K2 * ksteps * 512 + lane * 8;
 
     for (int s0 = kw; s0 < total; s0 += S * KW) {
-        half8_t a[S][R], x[S][NT];
+        E8 a[S][R], x[S][NT];
         int src[S][NT];
         bool use[S];
 #pragma unroll
@@ -781,11 +783,11 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
             use[i] = s0 + i * KW < total;  // wave-uniform
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                a[i][r] = *reinterpret_cast<const half8_t *>(wfrag[r] + (size_t)(tap * ksteps + ks) * 512);
+                a[i][r] = *reinterpret_cast<const E8 *>(wfrag[r] + (size_t)(tap * ksteps + ks) * 512);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 src[i][nt] = s_src[(tap << 6) + nt * 16 + l16];
-                x[i][nt] = *reinterpret_cast<const half8_t *>(inb + (size_t)max(src[i][nt], 0) * p.Ci + k);
+                x[i][nt] = *reinterpret_cast<const E8 *>(inb + (size_t)max(src[i][nt], 0) * p.Ci + k);
             }
         }
 #pragma unroll
@@ -794,10 +796,10 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 if (nt >= n_tiles) continue;  // wave-uniform
-                const half8_t xz = keep8(x[i][nt], src[i][nt] >= 0);
+                const E8 xz = keep8(x[i][nt], src[i][nt] >= 0);
 #pragma unroll
                 for (int r = 0; r < R; ++r)
-                    acc[r][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][r], xz, acc[r][nt], 0, 0, 0);
+                    acc[r][nt] = Elem16<E>::mfma(a[i][r], xz, acc[r][nt]);
             }
         }
     }
@@ -835,16 +837,16 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
             const int pix = nt * 16 + l16;
             if (pix >= n) continue;
             const int code = s_list[pix];
-            half_t *o = out + (((size_t)b * p.Ho + (code >> 16)) * p.Wo + (code & 0xffff)) * p.Co + co;
+            E *o = out + (((size_t)b * p.Ho + (code >> 16)) * p.Wo + (code & 0xffff)) * p.Co + co;
             if (co + 3 < p.Co && (p.Co & 3) == 0) {
-                half4_t v;
+                E4 v;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v[i] = half_t(acc[r][nt][i] + bv[i]);
-                *reinterpret_cast<half4_t *>(o) = v;
+                for (int i = 0; i < 4; ++i) v[i] = E(acc[r][nt][i] + bv[i]);
+                *reinterpret_cast<E4 *>(o) = v;
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (co + i < p.Co) o[i] = half_t(acc[r][nt][i] + bv[i]);
+                    if (co + i < p.Co) o[i] = E(acc[r][nt][i] + bv[i]);
             }
         }
     }
@@ -869,12 +871,14 @@ conv_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restric
 constexpr int LDS_MAX_HALO = 1024;
 constexpr int LDS_MAX_STEPS = 1024;
 
-template <int R, int S, int D, int KS, bool TR>
+template <typename E, int R, int S, int D, int KS, bool TR>
 __global__ void __launch_bounds__(8 * WAVE)
-conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
-                     const half_t *__restrict__ bias, half_t *__restrict__ out,
+conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp,
+                     const E *__restrict__ bias, E *__restrict__ out,
                      const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
                      int co_blocks, int ci_p, int hal_h, int hal_w, int kcc, int lgv) {
+    typedef typename Elem16<E>::v4 E4;
+    typedef typename Elem16<E>::v8 E8;
     constexpr int NT = 4;
     extern __shared__ __align__(16) unsigned char s_halo[];
     __shared__ int s_hpix[LDS_MAX_HALO];
@@ -966,28 +970,28 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
 #pragma unroll
     for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
         wfrag[r] = (unsigned)min((cb * ncw + cw) * R + r, co_tiles - 1) * K2 * ksteps * 512 + lane * 8;
-    half8_t a[D][S][R];
+    E8 a[D][S][R];
     int xo[D][S];
     int jl = 0;
-    auto load_chunk = [&](half8_t (&ac)[S][R], int (&xc)[S]) {
+    auto load_chunk = [&](E8 (&ac)[S][R], int (&xc)[S]) {
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             const int2 e = s_step[(jl + i) * KS + kz];
             xc[i] = e.x;
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                ac[i][r] = *reinterpret_cast<const half8_t *>(wp + (wfrag[r] + (unsigned)e.y));
+                ac[i][r] = *reinterpret_cast<const E8 *>(wp + (wfrag[r] + (unsigned)e.y));
         }
         jl += S;
     };
 #pragma unroll
     for (int d = 0; d < D; ++d) load_chunk(a[d], xo[d]);
-    half_t bv[R][4];  // bias of the lane's four channels per tile, requested early as well
+    E bv[R][4];  // bias of the lane's four channels per tile, requested early as well
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int co = ((cb * ncw + cw) * R + r) * 16 + kq * 4;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) bv[r][i] = bias != nullptr ? bias[min(co + i, p.Co - 1)] : half_t(0);
+        for (int i = 0; i < 4; ++i) bv[r][i] = bias != nullptr ? bias[min(co + i, p.Co - 1)] : E(0);
     }
 
     // Staging of channels [kbase * 32, (kbase + kcur) * 32) of the halo: 2^lgv lanes per pixel, SU
@@ -995,26 +999,26 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
     // dummy address and are stored as zeros.  The first pass of the first channel chunk is
     // requested here, so that it travels while the first wavefront dilates the mask.
     constexpr int SU = 8;
-    const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+    const E *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
     const int sv = tid & ((1 << lgv) - 1), hstep = nthr >> lgv;
-    auto stage_load = [&](int kbase, int h0, half8_t (&val)[SU], int (&px)[SU]) {
+    auto stage_load = [&](int kbase, int h0, E8 (&val)[SU], int (&px)[SU]) {
         const int c = min((kbase << 5) + sv * 8, p.Ci - 8);
 #pragma unroll
         for (int u = 0; u < SU; ++u) {
             px[u] = s_hpix[min(h0 + u * hstep, hpx - 1)];
-            val[u] = *reinterpret_cast<const half8_t *>(inb + (size_t)max(px[u], 0) * p.Ci + c);
+            val[u] = *reinterpret_cast<const E8 *>(inb + (size_t)max(px[u], 0) * p.Ci + c);
         }
     };
-    auto stage_store = [&](int kbase, int kcur, int h0, const half8_t (&val)[SU], const int (&px)[SU]) {
+    auto stage_store = [&](int kbase, int kcur, int h0, const E8 (&val)[SU], const int (&px)[SU]) {
         const bool vok = sv < kcur * 4 && (kbase << 5) + sv * 8 < p.Ci;
 #pragma unroll
         for (int u = 0; u < SU; ++u) {
             const int hp = h0 + u * hstep;
             if (hp < hpx && sv < kcur * 4)
-                *reinterpret_cast<half8_t *>(s_halo + hp * row + sv * 16) = keep8(val[u], vok && px[u] >= 0);
+                *reinterpret_cast<E8 *>(s_halo + hp * row + sv * 16) = keep8(val[u], vok && px[u] >= 0);
         }
     };
-    half8_t val0[SU];
+    E8 val0[SU];
     int px0[SU];
     stage_load(0, tid >> lgv, val0, px0);
 
@@ -1065,7 +1069,7 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
         }
         // remaining staging passes (all of them for the channel chunks after the first)
         for (int h0 = (tid >> lgv) + (kbase == 0 ? SU * hstep : 0); h0 < hpx; h0 += SU * hstep) {
-            half8_t val[SU];
+            E8 val[SU];
             int px[SU];
             stage_load(kbase, h0, val, px);
             stage_store(kbase, kcur, h0, val, px);
@@ -1083,23 +1087,23 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
         auto reduce = [&](auto nta_tag) {
             constexpr int NTA = decltype(nta_tag)::value;
             // input fragments are read from LDS one step ahead of the MFMAs that consume them
-            half8_t xq[NTA];
-            auto read_x = [&](half8_t (&x)[NTA], int off) {
+            E8 xq[NTA];
+            auto read_x = [&](E8 (&x)[NTA], int off) {
 #pragma unroll
                 for (int nt = 0; nt < NTA; ++nt)
-                    x[nt] = *reinterpret_cast<const half8_t *>(s_halo + hbase[nt] + off);
+                    x[nt] = *reinterpret_cast<const E8 *>(s_halo + hbase[nt] + off);
             };
-            auto compute_chunk = [&](const half8_t (&ac)[S][R], const int (&xc)[S], int next_off, auto tail_tag, int j0) {
+            auto compute_chunk = [&](const E8 (&ac)[S][R], const int (&xc)[S], int next_off, auto tail_tag, int j0) {
 #pragma unroll
                 for (int i = 0; i < S; ++i) {
-                    half8_t xn[NTA];
+                    E8 xn[NTA];
                     read_x(xn, i + 1 < S ? xc[i + 1] : next_off);
 #pragma unroll
                     for (int nt = 0; nt < NTA; ++nt) {
                         if (decltype(tail_tag)::value) xq[nt] = keep8(xq[nt], (j0 + i) * KS + kz < nsteps);
 #pragma unroll
                         for (int r = 0; r < R; ++r)
-                            acc[r][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ac[i][r], xq[nt], acc[r][nt], 0, 0, 0);
+                            acc[r][nt] = Elem16<E>::mfma(ac[i][r], xq[nt], acc[r][nt]);
                     }
 #pragma unroll
                     for (int nt = 0; nt < NTA; ++nt) xq[nt] = xn[nt];
@@ -1164,16 +1168,16 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
             const int pix = nt * 16 + l16;
             if (pix >= n) continue;
             const int loc = s_list[pix];
-            half_t *o = out + (((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7)) * p.Co + co;
+            E *o = out + (((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7)) * p.Co + co;
             if (co + 3 < p.Co && (p.Co & 3) == 0) {
-                half4_t v;
+                E4 v;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v[i] = half_t(acc[r][nt][i] + float(bv[r][i]));
-                *reinterpret_cast<half4_t *>(o) = v;
+                for (int i = 0; i < 4; ++i) v[i] = E(acc[r][nt][i] + float(bv[r][i]));
+                *reinterpret_cast<E4 *>(o) = v;
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (co + i < p.Co) o[i] = half_t(acc[r][nt][i] + float(bv[r][i]));
+                    if (co + i < p.Co) o[i] = E(acc[r][nt][i] + float(bv[r][i]));
             }
         }
     }
@@ -1187,10 +1191,11 @@ conv_lds_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__res
 // Fragments of taps that are out of bounds or inactive are zeroed by selection (every step is
 // computed: at this size the instruction stream, not the MFMA count, is the kernel time);
 // outputs are stored for updated pixels only.  KW wavefronts split the reduction steps round-robin.
+template <typename E>
 struct PatchRes {  // DCAdd fused behind the convolution: a = residual, b = convolution
-    const half_t *values;
+    const E *values;
     const int32_t *mask;
-    half_t *prev;
+    E *prev;
     float wa, wb;
     int act;
 };
@@ -1203,18 +1208,21 @@ struct PatchRes {  // DCAdd fused behind the convolution: a = residual, b = conv
 // block): the activation and truncation of DCActivation applied to the accumulators -- T = trunc
 // + v, S = T + prev, D = act(S) - act(prev), one rounding each, the sequence of act_trunc_pixel;
 // the keep statistics of a pixel are combined over its four k-quarter lanes.
+template <typename E>
 struct PatchEpi {
-    half_t *prev, *trunc;
+    E *prev, *trunc;
     float thr;
     int mode, act;
 };
 
-template <bool TR, int KW, int R, int S, int MODE, bool K3>
+template <typename E, bool TR, int KW, int R, int S, int MODE, bool K3>
 __global__ void __launch_bounds__(KW * WAVE)
-conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
-                       const half_t *__restrict__ bias, half_t *__restrict__ out,
+conv_patch_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp,
+                       const E *__restrict__ bias, E *__restrict__ out,
                        const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
-                       int co_blocks, int ci_p, PatchRes rs, PatchEpi ep) {
+                       int co_blocks, int ci_p, PatchRes<E> rs, PatchEpi<E> ep) {
+    typedef typename Elem16<E>::v4 E4;
+    typedef typename Elem16<E>::v8 E8;
     constexpr bool ADD = MODE == 1, EPI = MODE == 2;
     static_assert(!EPI || KW == 1, "the fused activation needs all channels in one wavefront");
     __shared__ float4_t s_red[KW > 1 ? KW * R * WAVE : 1];
@@ -1230,9 +1238,9 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     const int co_tiles = (p.Co + 15) >> 4;
     const int ksteps = ci_p >> 5;
     const int total = K2 * ksteps;
-    const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+    const E *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
     const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
-    const half_t *wfrag[R];
+    const E *wfrag[R];
 #pragma unroll
     for (int r = 0; r < R; ++r)  // surplus channel tiles re-read the last one and are not stored
         wfrag[r] = wp + (size_t)min(cb * R + r, co_tiles - 1) * total * 512 + lane * 8;
@@ -1270,7 +1278,7 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     // wave-uniform, so they live in scalar registers.
     int n_tap = 0, n_ks = kw;
     while (n_ks >= ksteps) { n_ks -= ksteps; ++n_tap; }
-    auto load_chunk = [&](half8_t (&a)[S][R], half8_t (&x)[S], int (&tp)[S]) {
+    auto load_chunk = [&](E8 (&a)[S][R], E8 (&x)[S], int (&tp)[S]) {
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             const int tap = min(n_tap, K2 - 1), ks = n_tap < K2 ? n_ks : ksteps - 1;  // past the end: last step again
@@ -1279,15 +1287,15 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
             const int sp = src_tab[tap * 16 + l16];
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                a[i][r] = *reinterpret_cast<const half8_t *>(wfrag[r] + (size_t)(tap * ksteps + ks) * 512);
-            x[i] = *reinterpret_cast<const half8_t *>(inb + (size_t)max(sp, 0) * p.Ci + k);
+                a[i][r] = *reinterpret_cast<const E8 *>(wfrag[r] + (size_t)(tap * ksteps + ks) * 512);
+            x[i] = *reinterpret_cast<const E8 *>(inb + (size_t)max(sp, 0) * p.Ci + k);
             n_ks += KW;
             while (n_ks >= ksteps) { n_ks -= ksteps; ++n_tap; }
         }
     };
 
     // eager: the first chunk of fragments is requested while the mask words are in flight
-    half8_t a[S][R], x[S];
+    E8 a[S][R], x[S];
     int tp[S];
     load_chunk(a, x, tp);
     bits |= __shfl_xor(bits, 16, WAVE);
@@ -1298,24 +1306,24 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
     if (cb == 0 && kw == 0 && kq == 0 && inside && !(EPI && upd)) out_mask[opix] = (upd || radd) ? 1 : 0;
     const bool reduce = ballot(upd) != 0;  // the same in every wavefront of the workgroup
     if (!reduce && ballot(radd) == 0) return;
-    half4_t eq[R], etr[R];  // cached state of the fused activation, requested before the reduction
+    E4 eq[R], etr[R];  // cached state of the fused activation, requested before the reduction
     if (EPI) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const size_t off = (upd ? opix : 0) * p.Co + min((cb * R + r) * 16 + kq * 4, p.Co - 4);
-            eq[r] = *reinterpret_cast<const half4_t *>(ep.prev + off);
-            etr[r] = *reinterpret_cast<const half4_t *>(ep.trunc + off);
+            eq[r] = *reinterpret_cast<const E4 *>(ep.prev + off);
+            etr[r] = *reinterpret_cast<const E4 *>(ep.trunc + off);
         }
     }
     // operands of the fused sum, requested now so that they arrive during the reduction
-    half4_t rv[R], qv[R];
+    E4 rv[R], qv[R];
     if (ADD) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int co = min((cb * R + r) * 16 + kq * 4, ((p.Co + 3) & ~3) - 4);
             if ((p.Co & 3) == 0) {
-                rv[r] = *reinterpret_cast<const half4_t *>(rs.values + opix * p.Co + co);
-                if (rs.act > 0) qv[r] = *reinterpret_cast<const half4_t *>(rs.prev + opix * p.Co + co);
+                rv[r] = *reinterpret_cast<const E4 *>(rs.values + opix * p.Co + co);
+                if (rs.act > 0) qv[r] = *reinterpret_cast<const E4 *>(rs.prev + opix * p.Co + co);
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -1335,10 +1343,10 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             // straight-line: a step past the end or an invalid (tap, pixel) pair multiplies zeros
-            const half8_t xz = keep8(x[i], s0 + i * KW < total && ((bits >> tp[i]) & 1ull));
+            const E8 xz = keep8(x[i], s0 + i * KW < total && ((bits >> tp[i]) & 1ull));
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][r], xz, acc[r], 0, 0, 0);
+                acc[r] = Elem16<E>::mfma(a[i][r], xz, acc[r]);
         }
     }
     if (KW > 1 && reduce) {
@@ -1355,24 +1363,24 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
         }
     }
     if (EPI) {
-        const half_t thr = half_t(ep.thr);
+        const E thr = E(ep.thr);
         auto finish = [&](auto act_c) {  // the activation as a compile-time constant
             constexpr int ACTC = decltype(act_c)::value;
-            half4_t t[R], sm[R], d[R];
+            E4 t[R], sm[R], d[R];
             bool hit = false;
             float sq = 0.f;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const int co = (cb * R + r) * 16 + kq * 4;
                 const bool live = upd && cb * R + r < co_tiles && co < p.Co;
-                half4_t bh = half4_t{0, 0, 0, 0};
-                if (bias != nullptr) bh = *reinterpret_cast<const half4_t *>(bias + min(co, p.Co - 4));
+                E4 bh = zero4<E>();
+                if (bias != nullptr) bh = *reinterpret_cast<const E4 *>(bias + min(co, p.Co - 4));
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const half_t v = half_t(acc[r][i] + float(bh[i]));
+                    const E v = E(acc[r][i] + float(bh[i]));
                     t[r][i] = etr[r][i] + v;
                     sm[r][i] = t[r][i] + eq[r][i];
-                    d[r][i] = act_apply<half_t>(sm[r][i], ACTC) - act_apply<half_t>(eq[r][i], ACTC);
+                    d[r][i] = act_apply<E>(sm[r][i], ACTC) - act_apply<E>(eq[r][i], ACTC);
                     if (live) {
                         hit |= tabs(d[r][i]) > thr;
                         sq += float(d[r][i]) * float(d[r][i]);
@@ -1397,11 +1405,11 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
                 if (cb * R + r >= co_tiles || co >= p.Co) continue;
                 const size_t off = opix * p.Co + co;
                 if (keep) {
-                    *reinterpret_cast<half4_t *>(ep.prev + off) = sm[r];
-                    *reinterpret_cast<half4_t *>(out + off) = d[r];
-                    *reinterpret_cast<half4_t *>(ep.trunc + off) = half4_t{0, 0, 0, 0};
+                    *reinterpret_cast<E4 *>(ep.prev + off) = sm[r];
+                    *reinterpret_cast<E4 *>(out + off) = d[r];
+                    *reinterpret_cast<E4 *>(ep.trunc + off) = zero4<E>();
                 } else {
-                    *reinterpret_cast<half4_t *>(ep.trunc + off) = t[r];
+                    *reinterpret_cast<E4 *>(ep.trunc + off) = t[r];
                 }
             }
         };
@@ -1416,7 +1424,7 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
         return;
     }
     if (!(upd || radd)) return;
-    half_t *o = out + opix * p.Co;
+    E *o = out + opix * p.Co;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (KW > 1 && (r % KW) != kw) continue;
@@ -1428,28 +1436,28 @@ conv_patch_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__r
             for (int i = 0; i < 4; ++i)
                 if (co + i < p.Co) bv[i] = float(bias[co + i]);
         }
-        half4_t v;
+        E4 v;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = half_t(acc[r][i] + bv[i]);
-        half4_t q;
+        for (int i = 0; i < 4; ++i) v[i] = E(acc[r][i] + bv[i]);
+        E4 q;
         if (ADD) {  // add_kernel's sequence: s = a * wa; s = fma(b, wb, s); n = s + prev; ...
-            const half_t wa = half_t(rs.wa), wb = half_t(rs.wb);
+            const E wa = E(rs.wa), wb = E(rs.wb);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                half_t sum = half_t(0);
+                E sum = E(0);
                 if (radd) sum = rv[r][i] * wa;
                 if (upd) sum = fma_t(v[i], wb, sum);
                 if (rs.act > 0) {
-                    const half_t n = sum + qv[r][i];
-                    sum = act_apply<half_t>(n, rs.act) - act_apply<half_t>(qv[r][i], rs.act);
+                    const E n = sum + qv[r][i];
+                    sum = act_apply<E>(n, rs.act) - act_apply<E>(qv[r][i], rs.act);
                     q[i] = n;
                 }
                 v[i] = sum;
             }
         }
         if (co + 3 < p.Co && (p.Co & 3) == 0) {
-            *reinterpret_cast<half4_t *>(o + co) = v;
-            if (ADD && rs.act > 0) *reinterpret_cast<half4_t *>(rs.prev + opix * p.Co + co) = q;
+            *reinterpret_cast<E4 *>(o + co) = v;
+            if (ADD && rs.act > 0) *reinterpret_cast<E4 *>(rs.prev + opix * p.Co + co) = q;
         } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -1500,14 +1508,16 @@ __global__ void pack_filter_kernel(const uint16_t *__restrict__ f, uint16_t *__r
 // keep decision of the fused activation stays inside the wavefront.  The halo's update mask is
 // kept as one bit row per halo row; an output is updated if its window meets a set bit.
 constexpr int STEM_K = 8;
-template <int R, int ACT>
+template <typename E, int R, int ACT>
 __global__ void __launch_bounds__(256)
-conv_stem_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__restrict__ wp,
-                      const half_t *__restrict__ bias, half_t *__restrict__ out,
+conv_stem_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp,
+                      const E *__restrict__ bias, E *__restrict__ out,
                       const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, EpiP epi,
                       int hal_h, int hal_wp) {
+    typedef typename Elem16<E>::v4 E4;
+    typedef typename Elem16<E>::v8 E8;
     extern __shared__ __align__(16) unsigned char s_mem[];
-    half_t *s_x = reinterpret_cast<half_t *>(s_mem);                       // [hal_h][hal_wp][4]
+    E *s_x = reinterpret_cast<E *>(s_mem);                       // [hal_h][hal_wp][4]
     unsigned *s_row = reinterpret_cast<unsigned *>(s_x + hal_h * hal_wp * 4);  // [hal_h]
     const int b = blockIdx.z, ty0 = blockIdx.y * TILE, tx0 = blockIdx.x * TILE;
     const int tid = threadIdx.x, wave = wave_id(), lane = lane_id();
@@ -1516,21 +1526,21 @@ conv_stem_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__re
     // filter fragments of the wavefront's R channel tiles: requested first, used last (surplus
     // tiles re-read the last one and are not stored)
     const int co_tiles = (p.Co + 15) >> 4;
-    half8_t a[R][STEM_K];
+    E8 a[R][STEM_K];
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
         for (int ky = 0; ky < STEM_K; ++ky)
-            a[r][ky] = *reinterpret_cast<const half8_t *>(wp + ((size_t)(min(r, co_tiles - 1) * p.Kh + min(ky, p.Kh - 1)) * WAVE + lane) * 8);
-    half4_t bv[R];
+            a[r][ky] = *reinterpret_cast<const E8 *>(wp + ((size_t)(min(r, co_tiles - 1) * p.Kh + min(ky, p.Kh - 1)) * WAVE + lane) * 8);
+    E4 bv[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        bv[r] = half4_t{0, 0, 0, 0};
-        if (bias != nullptr) bv[r] = *reinterpret_cast<const half4_t *>(bias + min(r * 16 + kq * 4, p.Co - 4));
+        bv[r] = zero4<E>();
+        if (bias != nullptr) bv[r] = *reinterpret_cast<const E4 *>(bias + min(r * 16 + kq * 4, p.Co - 4));
     }
     if (tid < hal_h) s_row[tid] = 0;
     __syncthreads();
-    const half_t *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+    const E *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
     const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
     for (int hp = tid; hp < hal_h * hal_wp; hp += 256) {
         const int hy = hp / hal_wp, hx = hp - hy * hal_wp;
@@ -1538,13 +1548,13 @@ conv_stem_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__re
         const bool ok = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
         const size_t pix = ok ? (size_t)iy * p.Wi + ix : 0;
         const int word = mb[pix];
-        half4_t v;
+        E4 v;
 #pragma unroll
         for (int ci = 0; ci < 4; ++ci) v[ci] = inb[pix * p.Ci + min(ci, p.Ci - 1)];
         const bool m = ok && word != 0;
 #pragma unroll
-        for (int ci = 0; ci < 4; ++ci) v[ci] = (m && ci < p.Ci) ? v[ci] : half_t(0);
-        *reinterpret_cast<half4_t *>(s_x + hp * 4) = v;
+        for (int ci = 0; ci < 4; ++ci) v[ci] = (m && ci < p.Ci) ? v[ci] : E(0);
+        *reinterpret_cast<E4 *>(s_x + hp * 4) = v;
         if (m) atomicOr(&s_row[hy], 1u << hx);
     }
     __syncthreads();
@@ -1560,13 +1570,13 @@ conv_stem_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__re
     if (ballot(upd) == 0) return;
 
     // cached state of the fused epilogue, requested before the contraction
-    half4_t q[R], tr[R];
+    E4 q[R], tr[R];
     if (ACT >= 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const size_t off = (upd ? po : 0) * p.Co + min(r * 16 + kq * 4, p.Co - 4);
-            q[r] = *reinterpret_cast<const half4_t *>((const half_t *)epi.prev + off);
-            tr[r] = *reinterpret_cast<const half4_t *>((const half_t *)epi.trunc + off);
+            q[r] = *reinterpret_cast<const E4 *>((const E *)epi.prev + off);
+            tr[r] = *reinterpret_cast<const E4 *>((const E *)epi.trunc + off);
         }
     }
     float4_t acc[R];
@@ -1575,31 +1585,31 @@ conv_stem_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__re
 #pragma unroll
     for (int ky = 0; ky < STEM_K; ++ky) {
         if (ky < p.Kh) {  // uniform
-            const half_t *xp = s_x + ((ly * p.sh + ky) * hal_wp + lx * p.sw + 2 * kq) * 4;
-            const half4_t x0 = *reinterpret_cast<const half4_t *>(xp), x1 = *reinterpret_cast<const half4_t *>(xp + 4);
-            const half8_t x = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+            const E *xp = s_x + ((ly * p.sh + ky) * hal_wp + lx * p.sw + 2 * kq) * 4;
+            const E4 x0 = *reinterpret_cast<const E4 *>(xp), x1 = *reinterpret_cast<const E4 *>(xp + 4);
+            const E8 x = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
 #pragma unroll
-            for (int r = 0; r < R; ++r) acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[r][ky], x, acc[r], 0, 0, 0);
+            for (int r = 0; r < R; ++r) acc[r] = Elem16<E>::mfma(a[r][ky], x, acc[r]);
         }
     }
-    half4_t v[R];
+    E4 v[R];
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[r][i] = half_t(acc[r][i] + float(bv[r][i]));
+        for (int i = 0; i < 4; ++i) v[r][i] = E(acc[r][i] + float(bv[r][i]));
     if (ACT < 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int co = r * 16 + kq * 4;
-            if (upd && co < p.Co) *reinterpret_cast<half4_t *>(out + po * p.Co + co) = v[r];
+            if (upd && co < p.Co) *reinterpret_cast<E4 *>(out + po * p.Co + co) = v[r];
         }
         return;
     }
     // activation + truncation, the operations and roundings of act_trunc_pixel; the statistics
     // of a pixel are combined over its four kq lanes
     constexpr int ACTC = ACT < 0 ? 0 : ACT;
-    const half_t thr = half_t(epi.thr);
-    half4_t t[R], sm[R], d[R];
+    const E thr = E(epi.thr);
+    E4 t[R], sm[R], d[R];
     bool hit = false;
     float sq = 0.f;
 #pragma unroll
@@ -1609,7 +1619,7 @@ conv_stem_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__re
         for (int i = 0; i < 4; ++i) {
             t[r][i] = tr[r][i] + v[r][i];
             sm[r][i] = t[r][i] + q[r][i];
-            d[r][i] = act_apply<half_t>(sm[r][i], ACTC) - act_apply<half_t>(q[r][i], ACTC);
+            d[r][i] = act_apply<E>(sm[r][i], ACTC) - act_apply<E>(q[r][i], ACTC);
             if (live) {
                 hit |= tabs(d[r][i]) > thr;
                 sq += float(d[r][i]) * float(d[r][i]);
@@ -1634,34 +1644,35 @@ conv_stem_mfma_kernel(ConvP p, const half_t *__restrict__ in, const half_t *__re
         if (co >= p.Co) continue;
         const size_t off = po * p.Co + co;
         if (keep) {
-            *reinterpret_cast<half4_t *>((half_t *)epi.prev + off) = sm[r];
-            *reinterpret_cast<half4_t *>(out + off) = d[r];
-            *reinterpret_cast<half4_t *>((half_t *)epi.trunc + off) = half4_t{0, 0, 0, 0};
+            *reinterpret_cast<E4 *>((E *)epi.prev + off) = sm[r];
+            *reinterpret_cast<E4 *>(out + off) = d[r];
+            *reinterpret_cast<E4 *>((E *)epi.trunc + off) = zero4<E>();
         } else {
-            *reinterpret_cast<half4_t *>((half_t *)epi.trunc + off) = t[r];
+            *reinterpret_cast<E4 *>((E *)epi.trunc + off) = t[r];
         }
     }
 }
 
 // Filter of conv_stem_mfma_kernel: fragment (channel tile, ky) holds, for lane (l16, kq) and
 // element e, W[co = tile * 16 + l16][ky][kx = (kq * 8 + e) / 4][ci = (kq * 8 + e) % 4], zero past
-// Kw, Cin and Cout.  Reads the processed fp16 layout (rows swizzled by the output parity).
-__global__ void pack_stem_filter_kernel(const half_t *__restrict__ f, half_t *__restrict__ wp, int Ci,
-                                        int Co, int Kh, int Kw, int w_co, int co_tiles) {
+// Kw, Cin and Cout.  Reads the processed fp16 layout (rows swizzled by the output parity) or,
+// swz == 0, the plain layout of bfloat16 filters; 16-bit elements of either type move as they are.
+__global__ void pack_stem_filter_kernel(const uint16_t *__restrict__ f, uint16_t *__restrict__ wp, int Ci,
+                                        int Co, int Kh, int Kw, int w_co, int co_tiles, int swz) {
     const int total = co_tiles * Kh * 512;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
         const int e = i & 7, lane = (i >> 3) & 63, frag = i >> 9;
         const int ky = frag % Kh, ct = frag / Kh;
         const int co = ct * 16 + (lane & 15), k = (lane >> 4) * 8 + e;
         const int kx = k >> 2, ci = k & 3;
-        half_t v = half_t(0);
-        if (kx < Kw && ci < Ci && co < Co) v = f[((size_t)(ci ^ (co & 1)) * Kh * Kw + ky * Kw + kx) * w_co + co];
+        uint16_t v = 0;
+        if (kx < Kw && ci < Ci && co < Co) v = f[((size_t)(ci ^ (swz ? (co & 1) : 0)) * Kh * Kw + ky * Kw + kx) * w_co + co];
         wp[i] = v;
     }
 }
 
 inline bool stem_eligible(const dc_geometry &g, int dtype) {
-    return dtype == DC_F16 && g.groups == 1 && g.in_c <= 4 && g.kernel_h <= STEM_K && g.kernel_w <= STEM_K &&
+    return (dtype == DC_F16 || dtype == DC_BF16) && g.groups == 1 && g.in_c <= 4 && g.kernel_h <= STEM_K && g.kernel_w <= STEM_K &&
            g.dilation_h == 1 && g.dilation_w == 1 && g.stride_h <= 2 && g.stride_w <= 2 && g.out_c % 4 == 0 &&
            g.out_c <= 64;
 }
@@ -1683,7 +1694,7 @@ hipError_t allow_large_lds(K *kernel) {
 }
 
 inline bool mfma_eligible(const dc_geometry &g, int dtype) {
-    return dtype == DC_F16 && g.groups == 1 && g.in_c % 8 == 0 && g.in_c >= 8;
+    return (dtype == DC_F16 || dtype == DC_BF16) && g.groups == 1 && g.in_c % 8 == 0 && g.in_c >= 8;
 }
 
 ConvP make_params(const dc_geometry &g, int dtype) {
@@ -1702,15 +1713,9 @@ ConvP make_params(const dc_geometry &g, int dtype) {
 
 }  // namespace
 
-// bfloat16 has matrix-core kernels for pointwise convolutions only (K x K windows take the
-// generic kernel); its filters are in the fp32 layout, unswizzled.
-inline bool bf16_packable(const dc_geometry &g, int dtype, bool transposed) {
-    return dtype == DC_BF16 && !transposed && pointwise_eligible(g, dtype);
-}
-
 int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed) {
     if (!transposed && stem_eligible(g, dtype)) return (int64_t)ceil_div(g.out_c, 16) * g.kernel_h * 1024;
-    if (!mfma_eligible(g, dtype) && !bf16_packable(g, dtype, transposed)) return 0;
+    if (!mfma_eligible(g, dtype)) return 0;
     return (int64_t)round_up(g.out_c, 16) * g.kernel_h * g.kernel_w * round_up(g.in_c, 32) * 2;
 }
 
@@ -1720,11 +1725,11 @@ hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *pa
         note_kernel("pack_stem_filter_kernel");
         const int co_tiles = ceil_div(g.out_c, 16);
         pack_stem_filter_kernel<<<ceil_div(co_tiles * g.kernel_h * 512, 256), 256, 0, s>>>(
-            (const half_t *)filter, (half_t *)packed, g.in_c, g.out_c, g.kernel_h, g.kernel_w,
-            g.out_c + (g.out_c & 1), co_tiles);
+            (const uint16_t *)filter, (uint16_t *)packed, g.in_c, g.out_c, g.kernel_h, g.kernel_w,
+            dtype == DC_F16 ? g.out_c + (g.out_c & 1) : g.out_c, co_tiles, dtype == DC_F16 ? 1 : 0);
         return hipGetLastError();
     }
-    if (!mfma_eligible(g, dtype) && !bf16_packable(g, dtype, transposed)) return hipSuccess;
+    if (!mfma_eligible(g, dtype)) return hipSuccess;
     const int K2 = g.kernel_h * g.kernel_w;
     const int ci_p = round_up(g.in_c, 32), co_p = round_up(g.out_c, 16);
     const size_t total = (size_t)co_p * K2 * ci_p;
@@ -1858,8 +1863,9 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
 
 // Stems of large frames on the matrix cores (see conv_stem_mfma_kernel); false if the shape, the
 // operands' alignment or the map size do not qualify.
-bool try_stem_mfma(const dc_geometry &g, const ConvP &p, const half_t *in, const half_t *packed,
-                   const half_t *bias, half_t *out, const int32_t *mask, int32_t *out_mask,
+template <typename E>
+bool try_stem_mfma(const dc_geometry &g, const ConvP &p, const E *in, const E *packed,
+                   const E *bias, E *out, const int32_t *mask, int32_t *out_mask,
                    const ActEpilogue *epi, hipStream_t s) {
     const auto al8 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 7u) == 0; };
     if (packed == nullptr || !stem_eligible(g, DC_F16)) return false;
@@ -1877,9 +1883,9 @@ bool try_stem_mfma(const dc_geometry &g, const ConvP &p, const half_t *in, const
     note_kernel("conv_stem_mfma_kernel");
 #define DC_ST_R(A)                                                                                                   \
     do {                                                                                                             \
-        if (co_tiles == 1) conv_stem_mfma_kernel<1, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
-        else if (co_tiles == 2) conv_stem_mfma_kernel<2, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
-        else conv_stem_mfma_kernel<4, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
+        if (co_tiles == 1) conv_stem_mfma_kernel<E, 1, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
+        else if (co_tiles == 2) conv_stem_mfma_kernel<E, 2, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
+        else conv_stem_mfma_kernel<E, 4, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
     } while (0)
     switch (act) {
         case DC_ACT_LINEAR: DC_ST_R(DC_ACT_LINEAR); break;
@@ -1947,11 +1953,13 @@ bool patch_eligible(const dc_geometry &g, int dtype) {
     return patches * ceil_div(g.out_c, 16) * steps <= 32768;
 }
 
-hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *packed,
-                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
-                             bool transposed, const Residual *res, hipStream_t s,
-                             const ActEpilogue *epi, bool *epilogue_done) {
-    ConvP p = make_params(g, DC_F16);
+namespace {
+template <typename E>
+hipError_t launch_patch_conv_t(const dc_geometry &g, const void *in, const void *packed,
+                               const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
+                               bool transposed, const Residual *res, hipStream_t s,
+                               const ActEpilogue *epi, bool *epilogue_done) {
+    ConvP p = make_params(g, DC_F16);  // the packed filter's layout does not depend on the type
     const int co_tiles = ceil_div(g.out_c, 16);
     const int ci_p = round_up(g.in_c, 32);
     const int steps = g.kernel_h * g.kernel_w * (ci_p / 32);
@@ -1960,9 +1968,9 @@ hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *p
     const int rv = (co_tiles >= 2 && patches * co_tiles >= 512) ? 2 : 1;
     const int cbk = ceil_div(co_tiles, rv);
     dim3 pgrid(ceil_div(g.out_w, 4), ceil_div(g.out_h, 4), g.batch * cbk);
-    PatchRes rs{nullptr, nullptr, nullptr, 0.f, 0.f, 0};
+    PatchRes<E> rs{nullptr, nullptr, nullptr, 0.f, 0.f, 0};
     if (res != nullptr)
-        rs = PatchRes{(const half_t *)res->values, res->mask, (half_t *)res->prev, res->wa, res->wb, res->act};
+        rs = PatchRes<E>{(const E *)res->values, res->mask, (E *)res->prev, res->wa, res->wb, res->act};
     const bool k3 = g.kernel_h == 3 && g.kernel_w == 3;
     // activation + truncation inside the kernel where one wavefront holds all channels of a pixel
     const auto al8 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 7u) == 0; };
@@ -1970,14 +1978,14 @@ hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *p
                       cbk == 1 && epi->mode >= 0 && epi->trunc != nullptr && g.out_c % 4 == 0 && al8(epi->prev) &&
                       al8(epi->trunc) && al8(out) && (bias == nullptr || al8(bias));
     if (epilogue_done != nullptr) *epilogue_done = fuse;
-    PatchEpi pe{nullptr, nullptr, 0.f, 0, 0};
-    if (fuse) pe = PatchEpi{(half_t *)epi->prev, (half_t *)epi->trunc, epi->thr, epi->mode, epi->act < 0 ? 0 : epi->act};
+    PatchEpi<E> pe{nullptr, nullptr, 0.f, 0, 0};
+    if (fuse) pe = PatchEpi<E>{(E *)epi->prev, (E *)epi->trunc, epi->thr, epi->mode, epi->act < 0 ? 0 : epi->act};
     note_kernel("conv_patch_mfma_kernel");
-#define DC_PATCH_ARGS (p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbk, ci_p, rs, pe)
+#define DC_PATCH_ARGS (p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, cbk, ci_p, rs, pe)
 #define DC_PATCH_L(TRF, KWV, RV, SV, AV)                                                                      \
     do {                                                                                                      \
-        if (k3) conv_patch_mfma_kernel<TRF, KWV, RV, SV, AV, true><<<pgrid, KWV * WAVE, 0, s>>> DC_PATCH_ARGS; \
-        else conv_patch_mfma_kernel<TRF, KWV, RV, SV, AV, false><<<pgrid, KWV * WAVE, 0, s>>> DC_PATCH_ARGS;  \
+        if (k3) conv_patch_mfma_kernel<E, TRF, KWV, RV, SV, AV, true><<<pgrid, KWV * WAVE, 0, s>>> DC_PATCH_ARGS; \
+        else conv_patch_mfma_kernel<E, TRF, KWV, RV, SV, AV, false><<<pgrid, KWV * WAVE, 0, s>>> DC_PATCH_ARGS;  \
     } while (0)
 #define DC_PATCH(TRF, AV)                                                                       \
     do {                                                                                        \
@@ -1994,11 +2002,25 @@ hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *p
 #undef DC_PATCH_ARGS
     return hipGetLastError();
 }
+}  // namespace
 
-hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
-                       const void *packed, const void *bias, void *out, const int32_t *mask,
-                       int32_t *out_mask, int dtype, bool transposed, const ActEpilogue *epi,
-                       hipStream_t s) {
+hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *packed,
+                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
+                             bool transposed, const Residual *res, int dtype, hipStream_t s,
+                             const ActEpilogue *epi, bool *epilogue_done) {
+    if (dtype == DC_BF16)
+        return launch_patch_conv_t<bf16_t>(g, in, packed, bias, out, mask, out_mask, transposed, res, s, epi, epilogue_done);
+    return launch_patch_conv_t<half_t>(g, in, packed, bias, out, mask, out_mask, transposed, res, s, epi, epilogue_done);
+}
+
+namespace {
+// E16: the 16-bit element type of the matrix-core paths (half_t where dtype is fp32 -- those
+// paths are not eligible then).
+template <typename E16>
+hipError_t launch_conv_t(const dc_geometry &g, const void *in, const void *filter,
+                         const void *packed, const void *bias, void *out, const int32_t *mask,
+                         int32_t *out_mask, int dtype, bool transposed, const ActEpilogue *epi,
+                         hipStream_t s) {
     ConvP p = make_params(g, dtype);
     const int tx = ceil_div(g.out_w, TILE), ty = ceil_div(g.out_h, TILE);
     if (!transposed) {
@@ -2008,8 +2030,8 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
             ? try_depthwise<bf16_t>(g, p, (const bf16_t *)in, (const bf16_t *)filter, (const bf16_t *)bias, (bf16_t *)out, mask, out_mask, epi, s)
             : try_depthwise<half_t>(g, p, (const half_t *)in, (const half_t *)filter, (const half_t *)bias, (half_t *)out, mask, out_mask, epi, s);
         if (done) return hipGetLastError();
-        if (dtype == DC_F16 && try_stem_mfma(g, p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias,
-                                             (half_t *)out, mask, out_mask, epi, s))
+        if (dtype != DC_F32 && try_stem_mfma<E16>(g, p, (const E16 *)in, (const E16 *)packed, (const E16 *)bias,
+                                                  (E16 *)out, mask, out_mask, epi, s))
             return hipGetLastError();
         const bool few = dtype == DC_F32
             ? try_fewcin<float>(g, p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, epi, s)
@@ -2032,7 +2054,7 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
         // Small layers: one 4x4 output patch per workgroup (see conv_patch_mfma_kernel).
         if (patch_eligible(g, dtype)) {
             bool fused = false;
-            hipError_t pe = launch_patch_conv(g, in, packed, bias, out, mask, out_mask, transposed, nullptr, s, epi, &fused);
+            hipError_t pe = launch_patch_conv_t<E16>(g, in, packed, bias, out, mask, out_mask, transposed, nullptr, s, epi, &fused);
             if (pe != hipSuccess || epi == nullptr || fused) return pe;
             return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
                                             epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
@@ -2086,14 +2108,14 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                 const int lgv = log2i(pow2_ceil(kcc * 4));  // lanes per halo pixel while staging
                 dim3 lgrid(ltx, lty, g.batch * cbl);
                 note_kernel("conv_lds_mfma_kernel");
-#define DC_LDS_ARGS (p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
+#define DC_LDS_ARGS (p, (const E16 *)in, (const E16 *)packed, (const E16 *)bias, (E16 *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
 #define DC_LDS_K(RV, SV, DV, KV, TV)                                                                        \
     do {                                                                                                    \
         if (lds > (48u << 10)) {                                                                            \
-            const hipError_t big = allow_large_lds(&conv_lds_mfma_kernel<RV, SV, DV, KV, TV>);              \
+            const hipError_t big = allow_large_lds(&conv_lds_mfma_kernel<E16, RV, SV, DV, KV, TV>);              \
             if (big != hipSuccess) return big;                                                              \
         }                                                                                                   \
-        conv_lds_mfma_kernel<RV, SV, DV, KV, TV><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS;                 \
+        conv_lds_mfma_kernel<E16, RV, SV, DV, KV, TV><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS;                 \
     } while (0)
 #define DC_LDS_L(RV, SV, DV, KV)                                                                            \
     do {                                                                                                    \
@@ -2125,7 +2147,7 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
         const int co_blocks = ceil_div(co_tiles, R);
         dim3 grid(gtx, gty, g.batch * co_blocks);
         note_kernel("conv_mfma_kernel");
-#define DC_MFMA_L(TRF, KWV, RV, SV) conv_mfma_kernel<TRF, KWV, RV, SV><<<grid, KWV * WAVE, 0, s>>>(p, (const half_t *)in, (const half_t *)packed, (const half_t *)bias, (half_t *)out, mask, out_mask, co_blocks, ci_p)
+#define DC_MFMA_L(TRF, KWV, RV, SV) conv_mfma_kernel<E16, TRF, KWV, RV, SV><<<grid, KWV * WAVE, 0, s>>>(p, (const E16 *)in, (const E16 *)packed, (const E16 *)bias, (E16 *)out, mask, out_mask, co_blocks, ci_p)
 #define DC_MFMA(TRF)                                                                   \
     do {                                                                               \
         if (ksplit) {                                                                  \
@@ -2167,6 +2189,16 @@ hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
     if (e != hipSuccess || epi == nullptr) return e;
     return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
                                     epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
+}
+}  // namespace
+
+hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
+                       const void *packed, const void *bias, void *out, const int32_t *mask,
+                       int32_t *out_mask, int dtype, bool transposed, const ActEpilogue *epi,
+                       hipStream_t s) {
+    if (dtype == DC_BF16)
+        return launch_conv_t<bf16_t>(g, in, filter, packed, bias, out, mask, out_mask, dtype, transposed, epi, s);
+    return launch_conv_t<half_t>(g, in, filter, packed, bias, out, mask, out_mask, dtype, transposed, epi, s);
 }
 
 }  // namespace dc

@@ -211,9 +211,9 @@ int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filt
         return fail(DC_ERR_UNSUPPORTED, "dc_conv_add: activation %d", activation);
     const bool pointwise = dc::pointwise_eligible(*g, dtype);
     if (!pointwise && !dc::patch_eligible(*g, dtype))
-        return fail(DC_ERR_UNSUPPORTED, "dc_conv_add: only fp16 1x1 stride-1 convolutions with "
+        return fail(DC_ERR_UNSUPPORTED, "dc_conv_add: only 16-bit 1x1 stride-1 convolutions with "
                                         "Cin %% 8 == 0 and Cout %% 4 == 0 and small "
-                                        "fp16 layers with Cin %% 8 == 0 have the fused form");
+                                        "16-bit layers with Cin %% 8 == 0 have the fused form");
     DC_REQUIRE_PTR("dc_conv_add", input);
     DC_REQUIRE_PTR("dc_conv_add", packed_filter);
     DC_REQUIRE_PTR("dc_conv_add", mask);
@@ -235,7 +235,7 @@ int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filt
                                            &unused, &res, dtype, (hipStream_t)stream), "dc_conv_add");
     }
     return finish(dc::launch_patch_conv(*g, input, packed_filter, bias, out, mask, out_mask, false, &res,
-                                        (hipStream_t)stream), "dc_conv_add");
+                                        dtype, (hipStream_t)stream), "dc_conv_add");
 }
 
 int64_t dc_packed_filter_bytes(const dc_geometry *g, int dtype, int transposed) {

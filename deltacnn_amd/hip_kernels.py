@@ -246,10 +246,10 @@ def sparse_deconv(x, filter, mask=None, bias=None, stride=(1, 1), padding=(0, 0)
 
 def pack_filter(filter: torch.Tensor, c_in: int, c_out: int, groups: int = 1,
                 transposed: bool = False) -> Optional[torch.Tensor]:
-    """One-time relayout of a processed fp16 filter for the MFMA kernels; None if the shape
-    has no packed form (fp32, grouped, or an input channel count that is neither a multiple
-    of 8 nor a stem's: Cin <= 4 with a window up to 8 x 8 and Cout <= 64).  bfloat16 filters
-    (fp32 layout) have a packed form for 1x1 convolutions only."""
+    """One-time relayout of a processed fp16 filter, or of a bfloat16 filter in the fp32 layout,
+    for the MFMA kernels; None if the shape has no packed form (fp32, grouped, or an input
+    channel count that is neither a multiple of 8 nor a stem's: Cin <= 4 with a window up to
+    8 x 8 and Cout <= 64)."""
     lib = _lib.load()
     if filter.dtype not in (torch.float16, torch.bfloat16):
         return None

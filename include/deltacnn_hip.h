@@ -117,8 +117,8 @@ int dc_conv_act(const dc_geometry *g, const void *input, const void *filter,
  * s = weight_residual * a [mask_residual] + weight_conv * b [mask]; activation == 0: out = s;
  * activation > 0 (other_nn_layers.cu:1379-1559): prev_out += s, out = act(prev_out) - act(old
  * prev_out).  out_mask = mask | mask_residual.  Results are identical to dc_conv followed by
- * dc_add(residual, conv).  No counterpart in the reference.  Two forms exist: fp16 1x1 stride-1
- * convolutions without padding (Cin % 8 == 0, Cout % 4 == 0), and small fp16
+ * dc_add(residual, conv).  No counterpart in the reference.  Two forms exist, both for the
+ * 16-bit types: 1x1 stride-1 convolutions without padding (Cin % 8 == 0, Cout % 4 == 0), and small
  * layers of any kernel size (Cin % 8 == 0, groups 1, at most 64 taps,
  * ceil(W/4) * ceil(H/4) * B * ceil(Cout/16) * Kh * Kw * ceil(Cin/32) <= 32768), both with or
  * without activation.  Both need a packed filter; anything else returns DC_ERR_UNSUPPORTED before any
@@ -184,7 +184,7 @@ enum { DC_BLOCK_LATE_LOADS = 1 };
 int dc_block(const dc_geometry *g, const dc_block_args *block, int dtype, void *stream);
 
 /* Number of bytes dc_pack_filter writes for this geometry (0 if the shape has no packed
- * form).  One-time weight relayout for the MFMA kernels, fp16, un-swizzled, in fragment order
+ * form).  One-time weight relayout for the MFMA kernels, fp16 or bfloat16, un-swizzled, in fragment order
  * [Cout tile of 16][Kh][Kw][Cin step of 32][lane 0..63][8] (lane kq*16+r holds input channels
  * kq*8..+8 of output channel r): round_up(Cout,16) * Kh * Kw * round_up(Cin,32) halves.
  * Stems (Cin <= 4, window up to 8 x 8, Cout <= 64 and a multiple of 4, not transposed) pack as

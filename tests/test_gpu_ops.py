@@ -429,33 +429,17 @@ def test_conv(lib, dtype, cfg, density, use_bias, packed):
     ((3, 32, 3, 2, 1, 1, 1, 33, 31), "conv_stem_mfma_kernel"),
     ((3, 64, 3, 2, 1, 1, 1, 600, 520), "conv_fewcin_kernel"),     # many channel tiles on a large map
     ((3, 32, 3, 2, 1, 2, 1, 33, 31), "conv_fewcin_kernel"),       # dilation: no matrix-core form
+    ((12, 64, 3, 1, 1, 1, 1, 40, 40), "conv_direct_kernel"),      # Cin not a multiple of 8: the generic kernel
 ], ids=lambda v: v if isinstance(v, str) else "-".join(str(x) for x in v))
-def test_conv_dispatch(lib, cfg, kernel):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["float16", "bfloat16"])
+def test_conv_dispatch(lib, cfg, kernel, dtype):
     """The shapes the parity cases above are chosen for reach the kernel they are meant to cover
-    (the library names the kernels of the last call)."""
+    (the library names the kernels of the last call), in both 16-bit types."""
     from deltacnn_amd import _lib
     Cin, Cout, groups = cfg[0], cfg[1], cfg[6]
-    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(torch.float16, cfg, 5, 0.5)
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 5, 0.5)
     d_filt = filt.to(DEV)
     pk = hk().pack_filter(d_filt, Cin, Cout, groups)
-    hk().sparse_conv(cl(x), d_filt, cl(mask), None, s, p, d, groups, c_out=Cout, create_out_mask=True, packed_filter=pk)
-    assert _lib.load().dc_last_kernels().decode() == kernel
-
-
-@pytest.mark.parametrize("cfg,kernel", [
-    ((64, 256, 1, 1, 0, 1, 1, 20, 20), "pw_mfma_kernel"),          # 1x1: the matrix cores (v_mfma_f32_16x16x32_bf16)
-    ((576, 96, 1, 1, 0, 1, 1, 14, 14), "pw_mfma_kernel"),
-    ((64, 64, 3, 1, 1, 1, 1, 40, 40), "conv_direct_kernel"),       # K x K windows: the generic kernel
-    ((32, 32, 3, 1, 1, 1, 32, 15, 18), "conv_dw_kernel"),
-    ((3, 32, 3, 2, 1, 1, 1, 33, 31), "conv_fewcin_kernel"),
-], ids=lambda v: v if isinstance(v, str) else "-".join(str(x) for x in v))
-def test_conv_dispatch_bfloat16(lib, cfg, kernel):
-    from deltacnn_amd import _lib
-    Cin, Cout, groups = cfg[0], cfg[1], cfg[6]
-    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(torch.bfloat16, cfg, 5, 0.5)
-    d_filt = filt.to(DEV)
-    pk = hk().pack_filter(d_filt, Cin, Cout, groups)
-    assert (pk is not None) == (K == (1, 1))
     hk().sparse_conv(cl(x), d_filt, cl(mask), None, s, p, d, groups, c_out=Cout, create_out_mask=True, packed_filter=pk)
     assert _lib.load().dc_last_kernels().decode() == kernel
 
@@ -465,10 +449,11 @@ def test_conv_dispatch_bfloat16(lib, cfg, kernel):
     ((64, 48, 4, 2, 1, 1, 1, 37, 41), "conv_lds_mfma_kernel"),
     ((64, 64, 3, 2, 1, 2, 1, 40, 41), "conv_mfma_kernel"),
 ], ids=lambda v: v if isinstance(v, str) else "-".join(str(x) for x in v))
-def test_deconv_dispatch(lib, cfg, kernel):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["float16", "bfloat16"])
+def test_deconv_dispatch(lib, cfg, kernel, dtype):
     from deltacnn_amd import _lib
     Cin, Cout = cfg[0], cfg[1]
-    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(torch.float16, cfg, 6, 0.5, True)
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 6, 0.5, True)
     d_filt = filt.to(DEV)
     pk = hk().pack_filter(d_filt, Cin, Cout, groups, transposed=True)
     hk().sparse_deconv(cl(x), d_filt, cl(mask), None, s, p, d, groups, c_out=Cout, create_out_mask=True, packed_filter=pk)
@@ -611,12 +596,13 @@ def test_conv_add_fused(lib, cfg, weights, dtype):
                          ids=lambda c: "-".join(str(v) for v in c))
 @pytest.mark.parametrize("act", [0, 1, 3])
 @pytest.mark.parametrize("weights", [(1.0, 1.0), (0.5, -1.5)])
-def test_conv_add_fused_small_layers(lib, cfg, act, weights):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["float16", "bfloat16"])
+def test_conv_add_fused_small_layers(lib, cfg, act, weights, dtype):
     """dc_conv_add on small KxK layers, with the DCAdd's activation and accumulated sum: equal to
     the oracle's conv + add, bit-identical to dc_conv followed by dc_add (outputs and state)."""
     from deltacnn_amd.hip_kernels import conv_geometry
     Cin, Cout = cfg[0], cfg[1]
-    dtype = torch.float16
+    tol = 2e-2 if dtype == torch.float16 else 8e-2  # one bfloat16 step at |x| <= 8 is 3e-2
     x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 93, 0.05)
     want_conv, want_cm = ops.conv(x, mask, wt, None, s, p, d, groups)
     B, _, Ho, Wo = want_conv.shape
@@ -638,7 +624,7 @@ def test_conv_add_fused_small_layers(lib, cfg, act, weights):
                                p1 if act else None, act)
     assert got is not None
     assert torch.equal(om.cpu(), want_mask)
-    assert_masked_close(out, want, want_mask, 0, 2e-2, "out")
+    assert_masked_close(out, want, want_mask, 0, tol, "out")
     c_out, c_mask = hk().sparse_conv(dx, d_filt, dm, None, s, p, d, 1, c_out=Cout, create_out_mask=True, packed_filter=pk)
     two, two_mask, p2 = torch.empty_like(out), torch.empty_like(om), cl(prev)
     hk().sparse_add_tensors(dres, c_out, p2 if act else None, two, dmres, c_mask, two_mask, weights[0], weights[1], act, False)
@@ -646,7 +632,7 @@ def test_conv_add_fused_small_layers(lib, cfg, act, weights):
     assert_masked_equal(out, two.cpu(), want_mask, "fused vs two calls")
     assert torch.equal(p1, p2)
     if act:
-        assert_masked_close(p1, want_prev, torch.ones_like(want_mask), 0, 2e-2, "prev_out")
+        assert_masked_close(p1, want_prev, torch.ones_like(want_mask), 0, tol, "prev_out")
 
 
 # ------------------------------------------------------------------ nothing active / all active

@@ -37,15 +37,13 @@ def assert_masked_close(got, want, mask, rtol, atol, what=""):
 
 
 def packed_form_exists(dtype, c_in, c_out, kernel, groups=1, transposed=False) -> bool:
-    """Whether dc_pack_filter has a form for this filter (include/deltacnn_hip.h): fp16, one
-    group, and either input channels in multiples of 8 or a stem (Cin <= 4, window up to 8 x 8,
-    Cout <= 64 and a multiple of 4, not transposed); bfloat16: 1x1 convolutions with Cin a multiple of
-    8 and Cout a multiple of 4.  tests/test_host_abi.py checks this rule
-    against dc_packed_filter_bytes, so parametrisations can be built without the library."""
+    """Whether dc_pack_filter has a form for this filter (include/deltacnn_hip.h): a 16-bit type
+    (fp16 or bfloat16), one group, and either input channels in multiples of 8 or a stem
+    (Cin <= 4, window up to 8 x 8, Cout <= 64 and a multiple of 4, not transposed).
+    tests/test_host_abi.py checks this rule against dc_packed_filter_bytes, so parametrisations
+    can be built without the library."""
     kh, kw = (kernel, kernel) if isinstance(kernel, int) else kernel
-    if dtype == torch.bfloat16:  # matrix-core kernels for 1x1 convolutions only
-        return groups == 1 and not transposed and (kh, kw) == (1, 1) and c_in % 8 == 0 and c_in >= 8 and c_out % 4 == 0
-    if dtype != torch.float16 or groups != 1:
+    if dtype not in (torch.float16, torch.bfloat16) or groups != 1:
         return False
     if c_in % 8 == 0 and c_in >= 8:
         return True
