@@ -57,6 +57,8 @@ _SIGNATURES = {
     "dc_deconv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),
     "dc_pool": (c_int, [_G, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P]),
     "dc_densify": (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int, _P]),
+    "dc_pool_densify": (c_int, [_G, _P, _P, _P, _P, c_int, _P]),
+    "dc_linear": (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int32, c_int, _P]),
     "dc_add": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_float, c_float, c_int, c_int, c_int32, c_int32, c_int, _P]),
     "dc_add_upsampled": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_float, c_float, c_int, c_int32, c_int32, c_int32, c_int32, c_int32, c_int, _P]),
     "dc_add_to_dense": (c_int, [_P, _P, _P, c_int, c_int32, c_int32, c_int, _P]),

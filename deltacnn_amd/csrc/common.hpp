@@ -278,6 +278,11 @@ hipError_t launch_pool(const dc_geometry &g, const void *in, const void *prev, v
                        hipStream_t s);
 // Whether a 1x1-output pooling of this shape can write its result in the tensor's own type.
 bool pool_global_casts(const dc_geometry &g, const void *in, const void *prev, int dtype);
+hipError_t launch_pool_densify(const dc_geometry &g, const void *in, const int32_t *mask, void *acc,
+                               void *dense, int dtype, hipStream_t s);
+bool linear_eligible(int in_features, int dtype);
+hipError_t launch_linear(const void *x, const void *w, const void *bias, void *out, int rows,
+                         int in_features, int out_features, int dtype, hipStream_t s);
 
 // Fused depthwise -> projection (-> expansion) block.  block_unsupported names the reason a
 // shape is outside the kernel's range (nullptr: supported as far as the shape check goes);

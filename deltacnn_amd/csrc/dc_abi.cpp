@@ -374,6 +374,48 @@ int dc_densify(const void *delta, void *prev_out, void *out, const int32_t *mask
                                      (hipStream_t)stream), "dc_densify");
 }
 
+int dc_pool_densify(const dc_geometry *g, const void *input, const int32_t *mask, void *prev_out,
+                    void *out, int dtype, void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_pool_densify");
+    int rc = check_geometry("dc_pool_densify", g, false, true);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_PTR("dc_pool_densify", input);
+    DC_REQUIRE_PTR("dc_pool_densify", mask);
+    DC_REQUIRE_PTR("dc_pool_densify", prev_out);
+    DC_REQUIRE_PTR("dc_pool_densify", out);
+    DC_REQUIRE_ALIGNED("dc_pool_densify", prev_out, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_pool_densify", out, esize(dtype));
+    if (!dc::pool_global_casts(*g, input, nullptr, dtype))
+        return fail(DC_ERR_UNSUPPORTED, "dc_pool_densify: needs a window covering the whole unpadded map, "
+                                        "channels in whole 16-byte vectors and a 16-byte aligned input");
+    return finish(dc::launch_pool_densify(*g, input, mask, prev_out, out, dtype, (hipStream_t)stream),
+                  "dc_pool_densify");
+}
+
+int dc_linear(const void *x, const void *weight, const void *bias, void *out, int32_t rows,
+              int32_t in_features, int32_t out_features, int dtype, void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_linear");
+    if (rows <= 0 || in_features <= 0 || out_features <= 0)
+        return fail(DC_ERR_SHAPE, "dc_linear: rows=%d in_features=%d out_features=%d must be positive", rows,
+                    in_features, out_features);
+    if ((int64_t)rows * in_features >= (int64_t)1 << 31 || (int64_t)rows * out_features >= (int64_t)1 << 31 ||
+        (int64_t)in_features * out_features >= (int64_t)1 << 40)
+        return fail(DC_ERR_SHAPE, "dc_linear: operands too large");
+    if (!dc::linear_eligible(in_features, dtype))
+        return fail(DC_ERR_UNSUPPORTED, "dc_linear: in_features=%d does not fill whole 16-byte vectors", in_features);
+    DC_REQUIRE_PTR("dc_linear", x);
+    DC_REQUIRE_PTR("dc_linear", weight);
+    DC_REQUIRE_PTR("dc_linear", out);
+    DC_REQUIRE_ALIGNED("dc_linear", x, 16);
+    DC_REQUIRE_ALIGNED("dc_linear", weight, 16);
+    DC_REQUIRE_ALIGNED("dc_linear", bias, esize(dtype));
+    DC_REQUIRE_ALIGNED("dc_linear", out, esize(dtype));
+    return finish(dc::launch_linear(x, weight, bias, out, rows, in_features, out_features, dtype,
+                                    (hipStream_t)stream), "dc_linear");
+}
+
 int dc_block(const dc_geometry *g, const dc_block_args *block, int dtype, void *stream) {
     dc::kernel_log_reset();
     DC_REQUIRE_DTYPE("dc_block");

@@ -435,14 +435,22 @@ pool_global_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restri
 // load is unconditional (the mask word selects afterwards), partial results meet in LDS and
 // are combined slice by slice in ascending order, so the sum has a fixed order and needs no
 // atomics.  OutT is float (the reference's accumulator protocol) or T (cast fused).
-template <typename T, typename OutT, bool MAX>
+// DENS (average, OutT == T): the DCDensify that follows a network's global pooling runs on the
+// pooled delta as it leaves the reduction -- acc += delta if any pixel of the map was updated,
+// dense = acc -- with the pooled delta rounded to T first, as the separate launches have it;
+// the delta itself and its one-pixel mask are not stored.
+template <typename T, typename OutT, bool MAX, bool DENS = false>
 __global__ void __launch_bounds__(256)
 pool_global_vec_kernel(int npx, int C, const T *__restrict__ in, const T *__restrict__ prev,
                        OutT *__restrict__ out, const int32_t *__restrict__ mask,
-                       int32_t *__restrict__ out_mask) {
+                       int32_t *__restrict__ out_mask, T *__restrict__ acc = nullptr,
+                       T *__restrict__ dense = nullptr) {
     constexpr int N = Vec16<T>::N, VPB = 8, SL = 256 / VPB;
     __shared__ float s_hi[SL][VPB * N], s_hp[MAX ? SL : 1][VPB * N];
     const int b = blockIdx.y;
+    T held = T(0);  // the accumulated value of this thread's channel, requested with the map
+    if (DENS && threadIdx.x < VPB * N && blockIdx.x * VPB * N + threadIdx.x < C)
+        held = acc[(size_t)b * C + blockIdx.x * VPB * N + threadIdx.x];
     const int vl = threadIdx.x % VPB, sl = threadIdx.x / VPB;
     const int c = (blockIdx.x * VPB + vl) * N;
     const int cc = min(c, C - N);
@@ -490,9 +498,20 @@ pool_global_vec_kernel(int npx, int C, const T *__restrict__ in, const T *__rest
                 r += s_hi[s2][threadIdx.x];
             }
         }
-        if (ch < C) out[(size_t)b * C + ch] = OutT(wg_any ? (MAX ? r - rp : r / float(npx)) : 0.f);
+        if (ch < C) {
+            const OutT pooled = OutT(wg_any ? (MAX ? r - rp : r / float(npx)) : 0.f);
+            if (DENS) {
+                if (wg_any) {
+                    held = T(pooled) + held;
+                    acc[(size_t)b * C + ch] = held;
+                }
+                dense[(size_t)b * C + ch] = held;
+            } else {
+                out[(size_t)b * C + ch] = pooled;
+            }
+        }
     }
-    if (blockIdx.x == 0 && threadIdx.x == 0 && out_mask != nullptr) out_mask[b] = wg_any ? 1 : 0;
+    if (!DENS && blockIdx.x == 0 && threadIdx.x == 0 && out_mask != nullptr) out_mask[b] = wg_any ? 1 : 0;
 }
 
 template <typename T>
@@ -591,6 +610,27 @@ bool pool_global_casts(const dc_geometry &g, const void *in, const void *prev, i
     return g.out_h == 1 && g.out_w == 1 && g.kernel_h == g.in_h && g.kernel_w == g.in_w && g.pad_top == 0 &&
            g.pad_left == 0 && g.pad_bottom == 0 && g.pad_right == 0 && g.dilation_h == 1 &&
            g.dilation_w == 1 && g.in_c % n == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)prev & 15) == 0;
+}
+
+namespace {
+template <typename T>
+hipError_t pool_densify_t(const dc_geometry &g, const T *in, const int32_t *mask, T *acc, T *dense,
+                          hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    note_kernel("pool_global_vec_kernel");
+    dim3 vgrid(ceil_div(g.in_c / N, 8), g.batch);
+    pool_global_vec_kernel<T, T, false, true><<<vgrid, 256, 0, s>>>(g.in_h * g.in_w, g.in_c, in, nullptr, nullptr, mask,
+                                                                    nullptr, acc, dense);
+    return hipGetLastError();
+}
+}  // namespace
+
+// Global average pooling + DCDensify in one launch; the caller has checked pool_global_casts.
+hipError_t launch_pool_densify(const dc_geometry &g, const void *in, const int32_t *mask, void *acc,
+                               void *dense, int dtype, hipStream_t s) {
+    if (dtype == DC_F32) return pool_densify_t<float>(g, (const float *)in, mask, (float *)acc, (float *)dense, s);
+    if (dtype == DC_BF16) return pool_densify_t<bf16_t>(g, (const bf16_t *)in, mask, (bf16_t *)acc, (bf16_t *)dense, s);
+    return pool_densify_t<half_t>(g, (const half_t *)in, mask, (half_t *)acc, (half_t *)dense, s);
 }
 
 hipError_t launch_pool(const dc_geometry &g, const void *in, const void *prev, void *out,

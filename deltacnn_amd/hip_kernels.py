@@ -321,6 +321,46 @@ def densify(delta, prev_out, out, mask):
           P=_pixels(delta), C=delta.shape[1], esize=delta.element_size(), in_mask=mask, dense_copy=True)
 
 
+def pooled_densify(x, mask, prev_out, out) -> bool:
+    """Global average pooling of the delta ``x`` [B, C, H, W] followed by DCDensify on the pooled
+    pixel, in one launch: ``prev_out`` [B, C, 1, 1] accumulates the pooled delta if any pixel of
+    the map was updated, ``out`` receives the accumulated value.  Identical to
+    ``sparse_pooling`` (average, whole map) followed by ``densify``.  False if the shape has no
+    such form (nothing was launched): issue the two calls."""
+    lib = _lib.load()
+    _nhwc(x, "x")
+    g = conv_geometry(x.shape, tuple(x.shape[2:]), x.shape[1], (1, 1), (0, 0), (1, 1), 1)
+    try:
+        _call("pool_densify", lib.dc_pool_densify,
+              (g, x.data_ptr(), _mask(mask, "mask").data_ptr(), prev_out.data_ptr(), out.data_ptr(),
+               _dtype(x), _stream()),
+              g=g, esize=x.element_size(), in_mask=mask, keep=(x, prev_out, out))
+    except _lib.DeltaCNNError as e:
+        if e.code == -3:
+            return False
+        raise
+    return True
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x @ weight.T + bias`` for a few rows ``x`` [rows, in_features] with torch.nn.Linear's
+    weight layout [out_features, in_features]: fp32 accumulation, one rounding to the input
+    type; returns a new [rows, out_features] tensor.  The library's kernel for the classifier
+    behind DCDensify (which the reference leaves to torch, example/mobilenet_deltacnn.py:225)."""
+    lib = _lib.load()
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+        raise _lib.DeltaCNNError(-2, f"linear: x {tuple(x.shape)} against weight {tuple(weight.shape)}")
+    if not (x.is_cuda and x.is_contiguous() and weight.is_contiguous() and weight.dtype == x.dtype
+            and (bias is None or (bias.dtype == x.dtype and bias.is_contiguous()))):
+        raise _lib.DeltaCNNError(-2, "linear: contiguous GPU operands of one dtype expected")
+    out = torch.empty((x.shape[0], weight.shape[0]), dtype=x.dtype, device=x.device)
+    _call("linear", lib.dc_linear,
+          (x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), x.shape[0], x.shape[1],
+           weight.shape[0], _dtype(x), _stream()),
+          rows=x.shape[0], in_f=x.shape[1], out_f=weight.shape[0], esize=x.element_size(), keep=(x, out))
+    return out
+
+
 def sparsify(input, prev_in, delta, mask, threshold):
     """cuda_kernels.py:136-137."""
     lib = _lib.load()

@@ -251,7 +251,8 @@ class MobileNetV2(_Net):
         self.sparsify = L.DCSparsify()
         self.densify = L.DCDensify()
         self.adaptive_avg_pooling = L.DCAdaptiveAveragePooling(output_size=(1, 1))
-        self.classifier = nn.Sequential(nn.Dropout(0.2), nn.Linear(self.last_channel, num_classes))
+        self._pooled_dense = getattr(L, "pooled_dense", None)
+        self.classifier = nn.Sequential(nn.Dropout(0.2), getattr(L, "Linear", nn.Linear)(self.last_channel, num_classes))
         for m in self.modules():
             if isinstance(m, nn.Conv2d):
                 nn.init.kaiming_normal_(m.weight, mode="fan_out")
@@ -287,8 +288,10 @@ class MobileNetV2(_Net):
     def forward(self, x):
         x = self.sparsify(x)
         x = self._features(x)
-        x = self.adaptive_avg_pooling(x)
-        x = self.densify(x)
+        dense = None
+        if self._pooled_dense is not None:  # pooling and densify as one launch where the namespace has it
+            dense = self._pooled_dense(self.adaptive_avg_pooling, self.densify, x)
+        x = dense if dense is not None else self.densify(self.adaptive_avg_pooling(x))
         x = x.reshape(x.shape[0], -1)
         return self.classifier(x)
 

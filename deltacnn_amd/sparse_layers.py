@@ -709,6 +709,7 @@ class DCDensify(DCModule):
     ``clone_out`` (default) every call returns a NEW tensor, so results collected over frames
     stay distinct; ``clone_out=False`` returns the accumulator itself."""
     idx = -1
+    fuse_pooling = True  # pooled_dense(): a preceding global average pooling joins the launch
 
     def __init__(self, activation: str = None, name="", clone_out=True):
         super().__init__()
@@ -737,6 +738,51 @@ class DCDensify(DCModule):
     def reset(self):
         super().reset()
         self.prev_out = None
+
+
+def pooled_dense(pool, densify, input):
+    """``densify(pool(input))`` for a global average pooling followed by a DCDensify, in one
+    launch on frames after the first: the pooled delta goes straight into the densify layer's
+    accumulator and never exists in memory.  Returns the dense ``[B, C, 1, 1]`` tensor (a new
+    tensor per call, as DCDensify returns), or ``None`` when the layers are not in a state or
+    of a shape the kernel takes; nothing has happened then and the caller runs the two layers.
+    Switch: ``DCDensify.fuse_pooling``."""
+    if not DCDensify.fuse_pooling or isinstance(input, Tensor):
+        return None
+    if not isinstance(pool, DCAdaptiveAveragePooling) or tuple(pool.output_size) != (1, 1):
+        return None
+    if not isinstance(densify, DCDensify) or densify.activation is not None or not densify.clone_out:
+        return None
+    delta, mask = input
+    acc = densify.prev_out
+    if (acc is None or tuple(acc.shape) != (delta.shape[0], delta.shape[1], 1, 1) or acc.dtype != delta.dtype
+            or acc.device != delta.device):
+        return None
+    dense = torch.empty_like(acc)
+    if not hk.pooled_densify(delta, mask, acc, dense):
+        return None
+    pool.first_iter = False
+    return dense
+
+
+class Linear(nn.Linear):
+    """torch.nn.Linear (same parameters, same state dict) whose forward runs the library's
+    dense-layer kernel on a few rows of a GPU tensor -- the classifier behind DCDensify, which
+    the reference leaves to torch (example/mobilenet_deltacnn.py:196-199, 225) and which a GEMM
+    library serves with several launch latencies at one row per stream.  Everything else
+    (CPU tensors, training, more than ``max_rows`` rows, feature counts that do not fill 16-byte
+    vectors) goes to torch.  Switch: ``Linear.use_library``."""
+    use_library = True
+    max_rows = 64
+
+    def forward(self, input):
+        w = self.weight
+        if (Linear.use_library and input.is_cuda and input.dim() == 2 and input.dtype == w.dtype
+                and input.dtype in (torch.float16, torch.bfloat16, torch.float32)
+                and input.shape[0] <= Linear.max_rows and input.shape[1] % (16 // input.element_size()) == 0
+                and not (torch.is_grad_enabled() and (input.requires_grad or w.requires_grad))):
+            return hk.linear(input.contiguous(), w.contiguous(), self.bias)
+        return F.linear(input, w, self.bias)
 
 
 class DCUpsamplingNearest2d(DCModule):

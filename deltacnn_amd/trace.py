@@ -218,6 +218,19 @@ class Tracer:
                     flops += 2 * cp * ce * n_out
                 shape = f"dw{ch} s{g.stride_h} -> {cp} -> {ce} @{g.out_h}x{g.out_w}"
                 dens = (n_in / p_in, n_out / p_out)
+            elif op == "pool_densify":  # the map's updated pixels in, accumulator in and out, dense copy out
+                g = meta["g"]
+                p_in = g.batch * g.in_h * g.in_w
+                rd = p_in * m + n_in * g.in_c * s + g.batch * g.in_c * s
+                wr = 2 * g.batch * g.in_c * s
+                shape = f"C{g.in_c} k{g.kernel_h} @{g.in_h}x{g.in_w}"
+                dens = (n_in / p_in, 1.0)
+            elif op == "linear":
+                rows, fi, fo = meta["rows"], meta["in_f"], meta["out_f"]
+                rd, wr = (rows * fi + fo * fi + fo) * s, rows * fo * s
+                flops = 2 * rows * fi * fo
+                shape = f"{fi}->{fo} rows {rows}"
+                dens = (1.0, 1.0)
             elif op == "pool":
                 g = meta["g"]
                 p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w

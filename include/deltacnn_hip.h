@@ -238,6 +238,27 @@ int dc_add_upsampled(const void *a, const void *b, void *prev_out, void *out, co
 int dc_densify(const void *delta, void *prev_out, void *out, const int32_t *mask, int32_t pixels,
                int32_t channels, int dtype, void *stream);
 
+/* The tail of a classification network in one launch: global average pooling over the whole
+ * unpadded map (sparse_pooling_wrapper_masked with a 1x1 output, conv_torch_wrapper.cpp:213-293)
+ * followed by DCDensify (sparse_layers.py:1287-1329) on its one-pixel result: with
+ * d = mean of the deltas of the map's updated pixels, rounded to the tensor type, prev_out += d
+ * if any pixel was updated, out = prev_out.  input is [B, H, W, C] with g->in_h x g->in_w the
+ * window, prev_out and out are [B, C].  Results are identical to dc_pool (mode average, output
+ * in the tensor type) followed by dc_densify; the pooled delta and its mask are not stored.
+ * Needs C in whole 16-byte vectors and a 16-byte aligned input, else DC_ERR_UNSUPPORTED before
+ * any launch (the caller then issues the two calls).  No counterpart in the reference. */
+int dc_pool_densify(const dc_geometry *g, const void *input, const int32_t *mask, void *prev_out,
+                    void *out, int dtype, void *stream);
+
+/* Dense layer on a few rows: out[r][o] = bias[o] + sum_i x[r][i] * weight[o][i], weight in
+ * torch.nn.Linear's [out_features][in_features] layout, bias may be NULL; fp32 accumulation
+ * in a fixed order, one rounding.  For the classifier behind DCDensify, which the reference
+ * leaves to torch (example/mobilenet_deltacnn.py:196-199, 225): at one row per stream it is a
+ * matrix-vector product of launch-latency size.  in_features must fill whole 16-byte vectors
+ * (DC_ERR_UNSUPPORTED otherwise); x, weight 16-byte aligned.  No counterpart in the reference. */
+int dc_linear(const void *x, const void *weight, const void *bias, void *out, int32_t rows,
+              int32_t in_features, int32_t out_features, int dtype, void *stream);
+
 /* Replaces sparse_add_to_dense_tensor_wrapper (conv_torch_wrapper.cpp:447-482):
  * b[px] += a[px] on active pixels.  With activation > 0 it also writes a = act(b) on every
  * pixel (the USE_ACTIVATION variant, other_nn_layers.cu:1731-1957). */

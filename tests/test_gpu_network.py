@@ -368,7 +368,7 @@ def _same(a, b):
 @pytest.mark.parametrize("network,size", [("mobilenet", (224, 224)), ("hrnet", (256, 256)), ("dla34", (192, 320))])
 def test_fused_layer_calls_change_nothing(lib, network, size):
     """One-launch forms (convolution + activation, convolution + residual sum, sum with an
-    upsampled operand) against the same model issuing the separate layer calls, fp16, at map
+    upsampled operand, inverted residual blocks, global pooling + densify) against the same model issuing the separate layer calls, fp16, at map
     sizes where the fused kernels are the ones chosen: outputs bit-identical on every frame."""
     from deltacnn_amd import sparse_layers as SL
     from deltacnn_amd.video import moving_rectangles_video
@@ -385,10 +385,13 @@ def test_fused_layer_calls_change_nothing(lib, network, size):
             for t in range(video.shape[0]):
                 frame = cl(video[t:t + 1].half())
                 SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = SL.DCConv2d.fuse_blocks = True
+                SL.DCDensify.fuse_pooling = True
                 got = fused(frame)
                 got = {k: v.clone() for k, v in got.items()} if isinstance(got, dict) else got.clone()
                 SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = SL.DCConv2d.fuse_blocks = False
+                SL.DCDensify.fuse_pooling = False
                 want = plain(frame)
                 assert _same(got, want), f"frame {t}"
     finally:
         SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = SL.DCConv2d.fuse_blocks = True
+        SL.DCDensify.fuse_pooling = True

@@ -753,6 +753,70 @@ def test_pool_global(lib, dtype, mode, C, H, W, density):
     assert_masked_close(out2, want, want_mask, tol, tol, "out (float32 accumulator)")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C,H,W", [(1280, 7, 7), (64, 16, 16), (24, 3, 5), (2048, 1, 1)])
+@pytest.mark.parametrize("density", [0.0, 0.2, 1.0])
+def test_pool_densify_fused(lib, dtype, C, H, W, density):
+    """dc_pool_densify == global average pooling followed by densify: bit-identical to the two
+    library calls (dense result and accumulator), within the pooling tolerance of the oracle's;
+    one stream of the batch without any update keeps its accumulator bit for bit."""
+    g = _gen(1150 + C)
+    B = 3
+    mask = rand_mask(g, B, H, W, density)
+    mask[2] = 0  # a stream whose frame did not change
+    x = torch.randn(B, C, H, W, generator=g).to(dtype)
+    acc0 = torch.randn(B, C, 1, 1, generator=g).to(dtype)
+    dx, dm = cl(poison(x, mask)), cl(mask)
+    acc, dense = cl(acc0), torch.full((B, C, 1, 1), float("nan"), dtype=dtype, device=DEV).contiguous(
+        memory_format=torch.channels_last)
+    assert hk().pooled_densify(dx, dm, acc, dense)
+    assert _last_kernel() == "pool_global_vec_kernel"
+    pooled, pm = hk().sparse_pooling(dx, None, (H, W), dm, pooling_mode_int=1)
+    acc2, dense2 = cl(acc0), torch.empty_like(dense)
+    hk().densify(pooled, acc2, dense2, pm)
+    assert torch.equal(acc, acc2) and torch.equal(dense, dense2) and torch.equal(dense, acc)
+    assert torch.equal(acc[2].cpu(), acc0[2])
+    want, want_mask = ops.pool(x, None, mask, (H, W), (1, 1), (0, 0), (1, 1), 1)
+    w_acc = acc0.clone()
+    ops.activate_truncate(want.clone(), w_acc, None, want_mask, -1, -1, -1)
+    tol = LOOSE[dtype]
+    assert float((dense.cpu().float() - w_acc.float()).abs().max()) <= tol * max(1.0, float(w_acc.float().abs().max()))
+
+
+def test_pool_densify_declines_other_shapes(lib):
+    """Channel counts that do not fill 16-byte vectors have no one-launch form: False, nothing
+    launched, operands untouched."""
+    g = _gen(1199)
+    mask = rand_mask(g, 1, 4, 4, 0.5)
+    x = torch.randn(1, 20, 4, 4, generator=g).half()
+    acc = cl(torch.randn(1, 20, 1, 1, generator=g).half())
+    before, dense = acc.clone(), torch.zeros_like(acc)
+    assert not hk().pooled_densify(cl(x), cl(mask), acc, dense)
+    assert torch.equal(acc, before) and not bool(dense.any())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows", [1, 3, 8, 9, 32])
+@pytest.mark.parametrize("fi,fo", [(1280, 1000), (64, 10), (520, 7), (4104, 33)])
+@pytest.mark.parametrize("use_bias", [True, False])
+def test_linear(lib, dtype, rows, fi, fo, use_bias):
+    """dc_linear against torch's linear evaluated in fp64 on the same (rounded) operands: fp32
+    accumulation and one rounding, so the error is half a unit of the output type plus the
+    accumulation error of fi fp32 products."""
+    g = _gen(1300 + fi + rows)
+    x = torch.randn(rows, fi, generator=g).to(dtype)
+    w = (torch.randn(fo, fi, generator=g) / fi ** 0.5).to(dtype)
+    b = torch.randn(fo, generator=g).to(dtype) if use_bias else None
+    want = torch.nn.functional.linear(x.double(), w.double(), None if b is None else b.double())
+    got = hk().linear(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV))
+    assert _last_kernel() == "linear_kernel"
+    assert got.dtype == dtype and got.shape == (rows, fo)
+    step = {torch.float32: 2.0 ** -23, torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    err = (got.cpu().double() - want).abs()
+    bound = step * want.abs().clamp(min=1.0) + 1e-5
+    assert bool((err <= bound).all()), float((err / bound).max())
+
+
 # ------------------------------------------------ the scanning forms of the simple operators
 def _last_kernel():
     from deltacnn_amd import _lib

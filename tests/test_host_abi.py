@@ -228,3 +228,36 @@ def test_block_arguments_are_checked_before_any_launch(lib):
     assert call(g, args(expand_channels=96, expand_activation=2)) == -4   # expansion operands missing
     assert call(g, args(input=p + 2)) == -5
     assert call(g, args(out=p + 4)) == -5
+
+
+def test_head_entry_points_check_their_arguments(lib):
+    """dc_pool_densify and dc_linear: shapes without the one-launch form -> -3 (the caller issues
+    the separate calls / torch's linear), bad sizes -> -2, missing operands -> -4, alignment -> -5."""
+    buf = (ctypes.c_char * 8192)()
+    p = (ctypes.addressof(buf) + 255) // 256 * 256
+    whole = _geom(in_h=7, in_w=7, in_c=64, out_h=1, out_w=1, out_c=64, kernel_h=7, kernel_w=7, pad_top=0,
+                  pad_left=0, pad_bottom=0, pad_right=0)
+
+    def pool(g, x=p, m=p, acc=p, out=p, dtype=1):
+        return lib.dc_pool_densify(ctypes.byref(g), x, m, acc, out, dtype, None)
+
+    assert pool(whole, dtype=9) == -1
+    assert pool(whole, x=None) == -4 and pool(whole, acc=None) == -4 and pool(whole, out=None) == -4
+    assert pool(whole, acc=p + 1) == -5
+    assert pool(whole, x=p + 2) == -3                                    # input not 16-byte aligned
+    window = _geom(in_h=8, in_w=8, in_c=64, out_h=4, out_w=4, out_c=64, kernel_h=2, kernel_w=2, stride_h=2,
+                   stride_w=2, pad_top=0, pad_left=0, pad_bottom=0, pad_right=0)
+    assert pool(window) == -3                                            # not a global pooling
+    odd = _geom(in_h=7, in_w=7, in_c=60, out_h=1, out_w=1, out_c=60, kernel_h=7, kernel_w=7, pad_top=0,
+                pad_left=0, pad_bottom=0, pad_right=0)
+    assert pool(odd) == -3                                               # 60 halves do not fill 16-byte vectors
+    assert lib.dc_pool_densify(None, p, p, p, p, 1, None) == -4
+
+    def linear(x=p, w=p, b=p, out=p, rows=1, fi=64, fo=10, dtype=1):
+        return lib.dc_linear(x, w, b, out, rows, fi, fo, dtype, None)
+
+    assert linear(dtype=5) == -1
+    assert linear(rows=0) == -2 and linear(fi=0) == -2 and linear(fo=-3) == -2
+    assert linear(fi=36) == -3 and b"16-byte" in lib.dc_last_error()     # 36 halves
+    assert linear(x=None) == -4 and linear(w=None) == -4 and linear(out=None) == -4
+    assert linear(x=p + 8) == -5 and linear(w=p + 2) == -5 and linear(out=p + 1) == -5
