@@ -1513,7 +1513,7 @@ __global__ void __launch_bounds__(256)
 conv_stem_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp,
                       const E *__restrict__ bias, E *__restrict__ out,
                       const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, EpiP epi,
-                      int hal_h, int hal_wp) {
+                      int hal_h, int hal_wp, int lazy) {
     typedef typename Elem16<E>::v4 E4;
     typedef typename Elem16<E>::v8 E8;
     extern __shared__ __align__(16) unsigned char s_mem[];
@@ -1527,11 +1527,14 @@ conv_stem_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ w
     // tiles re-read the last one and are not stored)
     const int co_tiles = (p.Co + 15) >> 4;
     E8 a[R][STEM_K];
+    auto load_filter = [&]() {
 #pragma unroll
-    for (int r = 0; r < R; ++r)
+        for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int ky = 0; ky < STEM_K; ++ky)
-            a[r][ky] = *reinterpret_cast<const E8 *>(wp + ((size_t)(min(r, co_tiles - 1) * p.Kh + min(ky, p.Kh - 1)) * WAVE + lane) * 8);
+            for (int ky = 0; ky < STEM_K; ++ky)
+                a[r][ky] = *reinterpret_cast<const E8 *>(wp + ((size_t)(min(r, co_tiles - 1) * p.Kh + min(ky, p.Kh - 1)) * WAVE + lane) * 8);
+    };
+    if (!lazy) load_filter();  // lazy: a tile without an update does not fetch its 16 KB per wavefront
     E4 bv[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -1548,9 +1551,14 @@ conv_stem_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ w
         const bool ok = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
         const size_t pix = ok ? (size_t)iy * p.Wi + ix : 0;
         const int word = mb[pix];
-        E4 v;
+        E4 v = zero4<E>();
+        // small maps: the pixel is requested together with its mask word (one round trip);
+        // lazy (large maps, where instructions and bytes count, not the latency chain): only
+        // updated pixels are read at all
+        if (!lazy || (ok && word != 0)) {
 #pragma unroll
-        for (int ci = 0; ci < 4; ++ci) v[ci] = inb[pix * p.Ci + min(ci, p.Ci - 1)];
+            for (int ci = 0; ci < 4; ++ci) v[ci] = inb[pix * p.Ci + min(ci, p.Ci - 1)];
+        }
         const bool m = ok && word != 0;
 #pragma unroll
         for (int ci = 0; ci < 4; ++ci) v[ci] = (m && ci < p.Ci) ? v[ci] : E(0);
@@ -1568,6 +1576,7 @@ conv_stem_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ w
     const size_t po = ((size_t)b * p.Ho + oy) * p.Wo + ox;
     if (inside && kq == 0 && (ACT < 0 || !upd)) out_mask[po] = upd ? 1 : 0;
     if (ballot(upd) == 0) return;
+    if (lazy) load_filter();
 
     // cached state of the fused epilogue, requested before the contraction
     E4 q[R], tr[R];
@@ -1880,12 +1889,14 @@ bool try_stem_mfma(const dc_geometry &g, const ConvP &p, const E *in, const E *p
     EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f, epi ? epi->mode : 0};
     const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
     const int co_tiles = ceil_div(g.out_c, 16);
+    // maps of 2^18 pixels and more: only updated pixels and the filters of updated tiles are read
+    const int lazy = (int64_t)g.batch * g.in_h * g.in_w >= (1 << 18) ? 1 : 0;
     note_kernel("conv_stem_mfma_kernel");
 #define DC_ST_R(A)                                                                                                   \
     do {                                                                                                             \
-        if (co_tiles == 1) conv_stem_mfma_kernel<E, 1, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
-        else if (co_tiles == 2) conv_stem_mfma_kernel<E, 2, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
-        else conv_stem_mfma_kernel<E, 4, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp); \
+        if (co_tiles == 1) conv_stem_mfma_kernel<E, 1, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp, lazy); \
+        else if (co_tiles == 2) conv_stem_mfma_kernel<E, 2, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp, lazy); \
+        else conv_stem_mfma_kernel<E, 4, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_wp, lazy); \
     } while (0)
     switch (act) {
         case DC_ACT_LINEAR: DC_ST_R(DC_ACT_LINEAR); break;

@@ -461,6 +461,178 @@ pw_act_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
     pw_epilogue_store<E, CTW, ACT>(q, tr, v, keep, wave, NW, kq, px, p, out, prev, trunc);
 }
 
+
+// ----------------------------------------------------------- large maps: active-pixel gather
+// On maps of tens of thousands of pixels and more (many video streams in a batch, large frames)
+// the fixed runs of 64 pixels above spend most of their workgroups on runs without an update,
+// and their 8-byte accesses per lane (the MFMA accumulator layout) reach a fraction of the
+// memory bandwidth.  Here a workgroup of four wavefronts scans a span of the update mask,
+// compacts the updated pixels into an LDS list, and every wavefront then takes 16 LISTED pixels
+// at a time: their rows are gathered by index, contracted against the whole filter -- staged
+// in LDS once per workgroup, at most 32 KB -- so a wavefront holds ALL output channels of its
+// 16 pixels; the result is rounded, transposed through a wavefront-private LDS tile into pixel
+// rows, and the rest runs on rows in 16-byte pieces: the plain store (MODE 0), or the
+// activation / truncation of DCActivation with its keep decision per pixel (MODE 2, maximum-norm
+// truncation: T = trunc + v, S = T + prev, D = act(S) - act(prev), one rounding each, the
+// sequence of act_trunc_pixel).  Reduction steps run in ascending order in one accumulator, the
+// order of pw_mfma_kernel without reduction slices, which is the arrangement the host would
+// otherwise pick for the layers this kernel takes.  Requires Cout % 8 == 0.
+constexpr int PWG_WAVES = 4;
+constexpr int PWG_MAX_STEPS = 8;
+
+template <typename E, int CT, int KSM, int MODE, int ACT>
+__global__ void __launch_bounds__(PWG_WAVES * WAVE)
+pw_gather_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp, const E *__restrict__ bias,
+                 E *__restrict__ out, const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
+                 E *__restrict__ prev, E *__restrict__ trunc, float thr_f, int span) {
+    typedef typename Elem16<E>::v4 E4;
+    typedef typename Elem16<E>::v8 E8;
+    constexpr int NT = PWG_WAVES * WAVE;
+    constexpr int RC = CT * 2;  // 16-byte pieces of a pixel row held by CT channel tiles
+    extern __shared__ __align__(16) unsigned char s_dyn[];
+    __shared__ int s_n;
+    __shared__ int s_keep[PWG_WAVES][16];
+    const int ksteps = p.ci_p >> 5;
+    const int wbytes = p.co_tiles * ksteps * 1024;
+    const int rowb = CT * 32 + 16;  // bytes of a staged pixel row: padded, rows start in different banks
+    E *s_w = reinterpret_cast<E *>(s_dyn);
+    unsigned char *s_v = s_dyn + wbytes + wave_id() * 16 * rowb;
+    int *s_list = reinterpret_cast<int *>(s_dyn + wbytes + PWG_WAVES * 16 * rowb);
+    const int tid = threadIdx.x, wave = wave_id(), lane = lane_id();
+    const int l16 = lane & 15, kq = lane >> 4;
+    const int p0 = blockIdx.x * span;
+    if (tid == 0) s_n = 0;
+    // the filter, in fragment order as packed (contiguous), requested before the mask words
+    for (int i = tid * 8; i < wbytes / 2; i += NT * 8)
+        *reinterpret_cast<E8 *>(s_w + i) = *reinterpret_cast<const E8 *>(wp + i);
+    __syncthreads();
+    for (int q0 = 0; q0 < span; q0 += NT) {
+        const int px = p0 + q0 + tid;
+        const bool in_map = q0 + tid < span && px < p.P;
+        const bool on = in_map && mask[min(px, p.P - 1)] != 0;
+        if (in_map && (MODE == 0 || !on)) out_mask[px] = on ? 1 : 0;
+        int cnt;
+        const int rank = wave_rank(on, cnt);
+        int base = 0;
+        if (lane == 0 && cnt > 0) base = atomicAdd(&s_n, cnt);
+        base = __shfl(base, 0, WAVE);
+        if (on) s_list[base + rank] = px;
+    }
+    __syncthreads();
+    const int n = s_n;
+    const E thr = E(thr_f);
+    for (int t0 = wave * 16; t0 < n; t0 += PWG_WAVES * 16) {
+        const int nt = min(16, n - t0);            // listed pixels of this tile
+        const int pix = s_list[t0 + min(l16, nt - 1)];  // surplus columns repeat a listed pixel and are dropped
+        const E *xrow = in + (size_t)pix * p.Ci;
+        E8 x[KSM];
+#pragma unroll
+        for (int ks = 0; ks < KSM; ++ks)
+            if (ks < ksteps) x[ks] = *reinterpret_cast<const E8 *>(xrow + min((ks << 5) + kq * 8, p.Ci - 8));
+        // rows of the cached state, in the 16-byte pieces the epilogue works on: piece c of the
+        // tile is piece c % RC of pixel c / RC; requested now, used after the contraction
+        constexpr int PIECES = (16 * RC + WAVE - 1) / WAVE;
+        E8 qrow[MODE == 2 ? PIECES : 1], trow[MODE == 2 ? PIECES : 1];
+        int ppix[PIECES], pcol[PIECES];
+        bool pon[PIECES];
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int c = lane + i * WAVE;
+            const int r = c / RC, cc = c - r * RC;
+            pon[i] = r < nt && cc * 8 < p.Co;
+            ppix[i] = s_list[t0 + min(r, nt - 1)];
+            pcol[i] = min(cc * 8, p.Co - 8);
+            if (MODE == 2) {
+                const size_t off = (size_t)ppix[i] * p.Co + pcol[i];
+                qrow[i] = *reinterpret_cast<const E8 *>(prev + off);
+                trow[i] = *reinterpret_cast<const E8 *>(trunc + off);
+            }
+        }
+        float4_t acc[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc[ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KSM; ++ks) {
+            if (ks < ksteps) {  // uniform
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    const int ctc = min(ct, p.co_tiles - 1);  // surplus tiles repeat the last one and are dropped
+                    const E8 a = *reinterpret_cast<const E8 *>(s_w + (size_t)(ctc * ksteps + ks) * 512 + lane * 8);
+                    acc[ct] = Elem16<E>::mfma(a, x[ks], acc[ct]);
+                }
+            }
+        }
+        // rounded result into the wavefront's LDS tile, pixel rows contiguous
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            const int co = min(ct, p.co_tiles - 1) * 16 + kq * 4;
+            E4 bh = zero4<E>();
+            if (bias != nullptr) bh = *reinterpret_cast<const E4 *>(bias + min(co, p.Co - 4));
+            E4 v;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = E(acc[ct][i] + float(bh[i]));
+            *reinterpret_cast<E4 *>(s_v + l16 * rowb + ct * 32 + kq * 8) = v;
+        }
+        if (MODE == 2 && lane < 16) s_keep[wave][lane] = 0;
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        E8 vrow[PIECES];
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int r = min(lane + i * WAVE, 16 * RC - 1) / RC;
+            vrow[i] = *reinterpret_cast<const E8 *>(s_v + r * rowb + pcol[i] * 2);
+        }
+        if (MODE == 0) {
+#pragma unroll
+            for (int i = 0; i < PIECES; ++i)
+                if (pon[i]) *reinterpret_cast<E8 *>(out + (size_t)ppix[i] * p.Co + pcol[i]) = vrow[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < PIECES; ++i) {
+                bool hit = false;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const E t = trow[i][j] + vrow[i][j];
+                    const E sm = t + qrow[i][j];
+                    const E d = act_apply<E>(sm, ACT) - act_apply<E>(qrow[i][j], ACT);
+                    hit |= tabs(d) > thr;
+                }
+                if (pon[i] && hit) s_keep[wave][(lane + i * WAVE) / RC] = 1;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            // second pass: T, S, D again (a handful of operations, cheaper than holding them)
+#pragma unroll
+            for (int i = 0; i < PIECES; ++i) {
+                const int c = lane + i * WAVE;
+                const int r = min(c, 16 * RC - 1) / RC;
+                const bool keep = s_keep[wave][r] != 0;
+                if (!pon[i]) continue;
+                const size_t off = (size_t)ppix[i] * p.Co + pcol[i];
+                if (c - r * RC == 0) out_mask[ppix[i]] = keep ? 1 : 0;
+                E8 tv, sv, dv, z;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    tv[j] = trow[i][j] + vrow[i][j];
+                    sv[j] = tv[j] + qrow[i][j];
+                    dv[j] = act_apply<E>(sv[j], ACT) - act_apply<E>(qrow[i][j], ACT);
+                    z[j] = E(0);
+                }
+                if (keep) {
+                    *reinterpret_cast<E8 *>(prev + off) = sv;
+                    *reinterpret_cast<E8 *>(out + off) = dv;
+                    *reinterpret_cast<E8 *>(trunc + off) = z;
+                } else {
+                    *reinterpret_cast<E8 *>(trunc + off) = tv;
+                }
+            }
+        }
+        // the tile's LDS row buffer and keep flags are reused by the next tile of this wavefront
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 }  // namespace
 
 bool pointwise_eligible(const dc_geometry &g, int dtype) {
@@ -499,6 +671,33 @@ int pick_config(const PwP &p, int ksteps) {
     return 2;
 }
 
+namespace {
+int config_slices(int cfg) {
+#define DC_PW_KW(ID, KW, CBW, NBW, R, NTW, EA) \
+    if (cfg == ID) return KW;
+    DC_PW_CONFIGS(DC_PW_KW)
+#undef DC_PW_KW
+    return 1;
+}
+
+// Shapes pw_gather_kernel takes: maps of 2^16 pixels and more, a filter of at most 32 KB with
+// up to 8 reduction steps and 16 channel tiles, output rows in whole 16-byte pieces, LDS within
+// 64 KB -- and only layers whose pw_mfma_kernel arrangement has no reduction slices, so that a
+// layer keeps one summation order whichever kernel serves it (fused sums stay with pw_mfma_kernel).
+int gather_tiles(const PwP &p, int ksteps) {
+    if (p.P < (1 << 16) || p.Co % 8 != 0 || p.co_tiles > 16 || ksteps > PWG_MAX_STEPS) return 0;
+    if (p.co_tiles * ksteps * 1024 > (32 << 10)) return 0;
+    if (config_slices(pick_config(p, ksteps)) != 1) return 0;
+    const int ct = p.co_tiles <= 4 ? p.co_tiles : p.co_tiles <= 6 ? 6 : p.co_tiles <= 8 ? 8 : p.co_tiles == 9 ? 9
+                   : p.co_tiles <= 12 ? 12 : 16;
+    return ct;
+}
+int gather_span(const PwP &p) { return p.P >= (1 << 19) ? 1024 : p.P >= (1 << 18) ? 512 : 256; }
+size_t gather_lds(const PwP &p, int ksteps, int ct) {
+    return (size_t)p.co_tiles * ksteps * 1024 + (size_t)PWG_WAVES * 16 * (ct * 32 + 16) + (size_t)gather_span(p) * 4;
+}
+}  // namespace
+
 int pointwise_reduction_slices(int pixels, int in_c, int out_c) {
     PwP p;
     p.P = pixels;
@@ -507,12 +706,7 @@ int pointwise_reduction_slices(int pixels, int in_c, int out_c) {
     p.ci_p = (in_c + 31) / 32 * 32;
     p.co_tiles = ceil_div(out_c, 16);
     p.xcd = p.nx = p.ny = 0;
-    const int cfg = pick_config(p, p.ci_p / 32);
-#define DC_PW_KW(ID, KW, CBW, NBW, R, NTW, EA) \
-    if (cfg == ID) return KW;
-    DC_PW_CONFIGS(DC_PW_KW)
-#undef DC_PW_KW
-    return 1;
+    return config_slices(pick_config(p, p.ci_p / 32));
 }
 
 namespace {
@@ -532,6 +726,51 @@ hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *
     const int ksteps = p.ci_p / 32;
     *epilogue_done = false;
     const auto al8 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 7u) == 0; };
+    // Large maps: active-pixel gather, with the activation / truncation as its epilogue where the
+    // layer has one with maximum-norm truncation.
+    const auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    const int gct = (res == nullptr && al16(in) && al16(out) && al16(packed)) ? gather_tiles(p, ksteps) : 0;
+    if (gct > 0 && gather_lds(p, ksteps, gct) <= (64u << 10)) {
+        const bool with_act = epi != nullptr && epi->mode == DC_TRUNC_MAX && epi->trunc != nullptr && al16(epi->prev) &&
+                              al16(epi->trunc);
+        const int span = gather_span(p);
+        const size_t lds = gather_lds(p, ksteps, gct);
+        dim3 grid(ceil_div(p.P, span));
+        note_kernel("pw_gather_kernel");
+#define DC_PWG_K(CTV, KSV)                                                                                        \
+    do {                                                                                                         \
+        if (with_act) {                                                                                          \
+            DC_ACT_SWITCH(act, (pw_gather_kernel<E, CTV, KSV, 2, A><<<grid, PWG_WAVES * WAVE, lds, s>>>(          \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, (E *)epi->prev,  \
+                (E *)epi->trunc, epi->thr, span)));                                                              \
+        } else {                                                                                                 \
+            pw_gather_kernel<E, CTV, KSV, 0, 0><<<grid, PWG_WAVES * WAVE, lds, s>>>(                             \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, nullptr,         \
+                nullptr, 0.f, span);                                                                             \
+        }                                                                                                        \
+    } while (0)
+#define DC_PWG(CTV)                                                                                              \
+    do {                                                                                                         \
+        if (ksteps <= 2) DC_PWG_K(CTV, 2);                                                                       \
+        else DC_PWG_K(CTV, PWG_MAX_STEPS);                                                                       \
+    } while (0)
+        const int act = epi != nullptr && epi->act > 0 ? epi->act : 0;
+        switch (gct) {
+            case 1: DC_PWG(1); break;
+            case 2: DC_PWG(2); break;
+            case 3: DC_PWG(3); break;
+            case 4: DC_PWG(4); break;
+            case 6: DC_PWG(6); break;
+            case 8: DC_PWG(8); break;
+            case 9: DC_PWG(9); break;
+            case 12: DC_PWG(12); break;
+            default: DC_PWG(16); break;
+        }
+#undef DC_PWG_K
+#undef DC_PWG
+        *epilogue_done = with_act;
+        return hipGetLastError();
+    }
     // Fused epilogue: a workgroup owns all output channels of its 16 pixels (up to 16
     // wavefronts x 2 channel tiles), so it takes the keep / drop decision itself.  Only for maps
     // of at least 512 pixels: a smaller map gives too few workgroups, the whole filter then

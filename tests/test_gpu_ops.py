@@ -328,6 +328,7 @@ CONVS = [
     (1, 8, 3, 1, 1, 1, 1, 16, 16),
     (3, 48, 7, 2, 3, 1, 1, 33, 35),
     (2, 64, 8, 2, 3, 1, 1, 30, 30),
+    (3, 32, 3, 2, 1, 1, 1, 400, 380),       # ... on a map of 2^18 pixels and more: only updated pixels are staged
     # layers large enough for the LDS-halo MFMA kernel (fp16 packed), one per arrangement / corner
     (64, 64, 3, 1, 1, 1, 1, 72, 70),        # two channel tiles per wave, steps split over two waves
     (64, 32, 3, 1, 1, 1, 1, 100, 100),      # ... over four waves (one channel group)
@@ -427,6 +428,7 @@ def test_conv(lib, dtype, cfg, density, use_bias, packed):
     ((144, 144, 3, 1, 1, 1, 144, 130, 131), "conv_dw_strip_kernel"),
     ((16, 16, 3, 2, 1, 1, 16, 600, 521), "conv_dw_scan_kernel"),
     ((3, 32, 3, 2, 1, 1, 1, 33, 31), "conv_stem_mfma_kernel"),
+    ((3, 32, 3, 2, 1, 1, 1, 400, 380), "conv_stem_mfma_kernel"),
     ((3, 64, 3, 2, 1, 1, 1, 600, 520), "conv_fewcin_kernel"),     # many channel tiles on a large map
     ((3, 32, 3, 2, 1, 2, 1, 33, 31), "conv_fewcin_kernel"),       # dilation: no matrix-core form
     ((12, 64, 3, 1, 1, 1, 1, 40, 40), "conv_direct_kernel"),      # Cin not a multiple of 8: the generic kernel
@@ -550,6 +552,83 @@ def test_conv_activation_fused(lib, dtype, cfg, act, mode):
                                             packed_filter=pk)
     assert torch.equal(om1, om2)
     assert 0 < int(om1.sum()) and (mode != 0 or int(om1.sum()) < int(want_mask.sum()))
+    assert torch.equal(p1, p2) and torch.equal(t1, t2)
+    assert_masked_equal(out2, out1.cpu(), om1.cpu(), "out")
+
+
+# ------------------------------------------- pointwise convolutions of large maps: active-pixel gather
+GATHER_SHAPES = [(16, 96), (24, 144), (144, 24), (32, 16), (96, 24), (32, 192), (192, 32), (64, 128), (256, 40),
+                 (8, 8)]
+
+
+def _gather_case(dtype, cin, cout, density, seed):
+    """Two 192 x 192 maps (73 728 pixels: the gather kernel's range), masks in runs as a video's."""
+    g = _gen(seed)
+    B, H, W = 2, 192, 192
+    mask = (torch.nn.functional.interpolate((torch.rand(B, 1, H // 4, W // 8, generator=g) < density).float(),
+                                            size=(H, W)) > 0).to(torch.int32)
+    mask[0, 0, 5, 7] = 1                      # a lone pixel, and a map border
+    mask[1, 0, H - 1, W - 3:] = 1
+    x = torch.randn(B, cin, H, W, generator=g).to(dtype)
+    wt = (torch.randn(cout, cin, 1, 1, generator=g) / cin ** 0.5).to(dtype)
+    from deltacnn_amd.filter_conversion import convert_filter_out_channels_last, convert_half_filter
+    filt = convert_half_filter(wt) if dtype == torch.float16 else convert_filter_out_channels_last(wt)
+    return x, mask, wt, filt
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["float16", "bfloat16"])
+@pytest.mark.parametrize("cin,cout", GATHER_SHAPES, ids=lambda v: str(v))
+@pytest.mark.parametrize("density", [0.0, 0.02, 0.4, 1.0])
+def test_pointwise_gather(lib, dtype, cin, cout, density):
+    """1x1 convolutions of maps from 2^16 pixels on run on pw_gather_kernel: masks equal to the
+    oracle's, values within the convolution tolerance, and bit-identical to the same pixels
+    convolved as two smaller maps (which take pw_mfma_kernel): one summation order per layer."""
+    x, mask, wt, filt = _gather_case(dtype, cin, cout, density, 1400 + cin + cout)
+    want, want_mask = ops.conv(x, mask, wt, None, (1, 1), (0, 0), (1, 1), 1)
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, cin, cout, 1)
+    dx, dm = cl(poison(x, mask)), cl(mask)
+    out, om = hk().sparse_conv(dx, d_filt, dm, None, (1, 1), (0, 0), (1, 1), 1, c_out=cout, create_out_mask=True,
+                               packed_filter=pk)
+    assert _last_kernel() == "pw_gather_kernel"
+    assert torch.equal(om.cpu(), want_mask)
+    _check_conv(dtype, out, want, want_mask)
+    for b in range(2):
+        part, pm = hk().sparse_conv(cl(dx[b:b + 1]), d_filt, cl(dm[b:b + 1]), None, (1, 1), (0, 0), (1, 1), 1,
+                                    c_out=cout, create_out_mask=True, packed_filter=pk)
+        assert _last_kernel() == "pw_mfma_kernel"
+        assert_masked_equal(out[b:b + 1], part.cpu(), want_mask[b:b + 1], f"map {b}: gather vs 64-pixel runs")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["float16", "bfloat16"])
+@pytest.mark.parametrize("cin,cout", GATHER_SHAPES, ids=lambda v: str(v))
+@pytest.mark.parametrize("act", [1, 2, 5])
+@pytest.mark.parametrize("density", [0.02, 0.4, 1.0])
+def test_pointwise_gather_with_activation(lib, dtype, cin, cout, act, density):
+    """dc_conv_act on a large map (gather kernel with the activation / truncation as its
+    epilogue) == dc_conv (gather kernel) followed by dc_activate_truncate: output, both cached
+    tensors and the mask bit for bit; some pixels kept, some dropped."""
+    x, mask, wt, filt = _gather_case(dtype, cin, cout, density, 1500 + cin + cout)
+    g = _gen(1501 + cin)
+    # half of the pixels carry a change far below the threshold: their updates are truncated
+    x = (x.float() * torch.where(torch.rand(2, 1, 192, 192, generator=g) < 0.5, 1.0, 1e-3)).to(dtype)
+    prev = torch.randn(2, cout, 192, 192, generator=g).to(dtype)
+    trunc = (torch.randn(2, cout, 192, 192, generator=g) * 0.05).to(dtype)
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, cin, cout, 1)
+    dx, dm = cl(poison(x, mask)), cl(mask)
+    thr = 0.9 if act != 5 else 0.6
+    p1, t1 = cl(prev), cl(trunc)
+    out1, om1 = hk().sparse_conv(dx, d_filt, dm, None, (1, 1), (0, 0), (1, 1), 1, c_out=cout, create_out_mask=True,
+                                 packed_filter=pk)
+    hk().sparse_activation(out1, p1, t1, om1, thr, act, 0)
+    p2, t2 = cl(prev), cl(trunc)
+    out2, om2 = hk().sparse_conv_activation(dx, d_filt, dm, None, p2, t2, thr, act, 0, (1, 1), (0, 0), (1, 1), 1, cout,
+                                            packed_filter=pk)
+    assert _last_kernel() == "pw_gather_kernel"
+    assert torch.equal(om1, om2)
+    kept, reached = int(om1.sum()), int(mask.sum())
+    assert 0 < kept < reached, (kept, reached)
     assert torch.equal(p1, p2) and torch.equal(t1, t2)
     assert_masked_equal(out2, out1.cpu(), om1.cpu(), "out")
 
