@@ -462,6 +462,143 @@ pw_act_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
 }
 
 
+// ------------------------------------------- fused conv + act/trunc, epilogue on pixel rows
+// The fused form for layers too large for pw_act_mfma_kernel's 8-byte epilogue accesses (many
+// streams in a batch: output maps beyond 4 MB) and too wide for pw_gather_kernel (more than 256
+// output channels, filters beyond LDS): 16 consecutive pixels x all output channels per
+// workgroup, NW wavefronts x CTW channel tiles each, filter fragments streamed by the wavefront
+// that owns the tile (reduction steps ascending, one accumulator: the order of pw_mfma_kernel
+// without reduction slices).  The rounded result is transposed through LDS into pixel rows and
+// the activation / truncation (maximum norm) runs on rows in 16-byte pieces, the keep decision of
+// a pixel meeting in an LDS flag.  The masks are read first and only updated pixels are touched:
+// this kernel serves throughput, not the latency chain.  Requires Cout % 8 == 0.
+template <typename E, int NW, int CTW, int ACT>
+__global__ void __launch_bounds__(NW * WAVE)
+pw_rows_act_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
+                   const E *__restrict__ bias, E *__restrict__ out,
+                   const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
+                   E *__restrict__ prev, E *__restrict__ trunc, float thr_f) {
+    typedef typename Elem16<E>::v4 E4;
+    typedef typename Elem16<E>::v8 E8;
+    constexpr int NT = NW * WAVE, S = 2;
+    constexpr int PIECES = (16 * CTW * NW * 2 + NT - 1) / NT;  // 16-byte pieces of the tile per thread
+    extern __shared__ __align__(16) unsigned char s_rows[];   // [16][rowb]
+    __shared__ int s_keep[16];
+    const int tid = threadIdx.x, wave = wave_id(), lane = lane_id();
+    const int l16 = lane & 15, kq = lane >> 4;
+    const int ksteps = p.ci_p >> 5;
+    const int rc = p.Co >> 3;                 // pieces per pixel row
+    const int rowb = p.Co * 2 + 16;           // padded: rows start in different banks
+    const int px = blockIdx.x * 16 + l16;
+    const int pxc = min(px, p.P - 1);
+    const bool on = px < p.P && mask[pxc] != 0;
+    const uint64_t bon = ballot(on) & 0xffffull;  // the same 16 pixels in every wavefront
+    if (bon == 0) {
+        if (wave == 0 && kq == 0 && px < p.P) out_mask[px] = 0;
+        return;
+    }
+    if (tid < 16) s_keep[tid] = 0;
+    // rows of the cached state of updated pixels, requested before the contraction
+    E8 qrow[PIECES], trow[PIECES];
+    int64_t poff[PIECES];  // element offset of the piece in the map, -1: nothing to do
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+        const int c = tid + i * NT;
+        const int r = c / rc, cc = c - r * rc;
+        const bool live = r < 16 && ((bon >> r) & 1);
+        poff[i] = live ? ((int64_t)blockIdx.x * 16 + r) * p.Co + cc * 8 : -1;
+        if (live) {
+            qrow[i] = *reinterpret_cast<const E8 *>(prev + poff[i]);
+            trow[i] = *reinterpret_cast<const E8 *>(trunc + poff[i]);
+        }
+    }
+    const E *wrow[CTW];
+#pragma unroll
+    for (int j = 0; j < CTW; ++j)
+        wrow[j] = wp + (size_t)min(wave + j * NW, p.co_tiles - 1) * ksteps * 512 + lane * 8;
+    // inactive pixels read an updated pixel's row (finite values; their columns are dropped)
+    const int src = on ? pxc : blockIdx.x * 16 + (__ffsll((long long)bon) - 1);
+    const E *xrow = in + (size_t)src * p.Ci;
+    float4_t acc[CTW];
+#pragma unroll
+    for (int j = 0; j < CTW; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < ksteps; s0 += S) {
+        E8 a[S][CTW], x[S];
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            const int sidx = min(s0 + i, ksteps - 1);
+            x[i] = *reinterpret_cast<const E8 *>(xrow + min((sidx << 5) + kq * 8, p.Ci - 8));
+#pragma unroll
+            for (int j = 0; j < CTW; ++j) a[i][j] = *reinterpret_cast<const E8 *>(wrow[j] + (sidx << 9));
+        }
+#pragma unroll
+        for (int i = 0; i < S; ++i) {
+            if (s0 + i < ksteps) {  // uniform
+#pragma unroll
+                for (int j = 0; j < CTW; ++j) acc[j] = Elem16<E>::mfma(a[i][j], x[i], acc[j]);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < CTW; ++j) {
+        const int ct = wave + j * NW;
+        if (ct >= p.co_tiles) break;  // uniform
+        const int co = ct * 16 + kq * 4;
+        if (co >= p.Co) continue;
+        E4 bh = zero4<E>();
+        if (bias != nullptr) bh = *reinterpret_cast<const E4 *>(bias + co);
+        E4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = E(acc[j][i] + float(bh[i]));
+        *reinterpret_cast<E4 *>(s_rows + l16 * rowb + co * 2) = v;
+    }
+    __syncthreads();
+    const E thr = E(thr_f);
+    E8 vrow[PIECES];
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+        if (poff[i] < 0) continue;
+        const int c = tid + i * NT;
+        const int r = c / rc, cc = c - r * rc;
+        vrow[i] = *reinterpret_cast<const E8 *>(s_rows + r * rowb + cc * 16);
+        bool hit = false;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const E t = trow[i][j] + vrow[i][j];
+            const E sm = t + qrow[i][j];
+            const E d = act_apply<E>(sm, ACT) - act_apply<E>(qrow[i][j], ACT);
+            hit |= tabs(d) > thr;
+        }
+        if (hit) s_keep[r] = 1;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+        if (poff[i] < 0) continue;
+        const int c = tid + i * NT;
+        const int r = c / rc, cc = c - r * rc;
+        const bool keep = s_keep[r] != 0;
+        if (cc == 0) out_mask[blockIdx.x * 16 + r] = keep ? 1 : 0;
+        E8 tv, sv, dv, z;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            tv[j] = trow[i][j] + vrow[i][j];
+            sv[j] = tv[j] + qrow[i][j];
+            dv[j] = act_apply<E>(sv[j], ACT) - act_apply<E>(qrow[i][j], ACT);
+            z[j] = E(0);
+        }
+        if (keep) {
+            *reinterpret_cast<E8 *>(prev + poff[i]) = sv;
+            *reinterpret_cast<E8 *>(out + poff[i]) = dv;
+            *reinterpret_cast<E8 *>(trunc + poff[i]) = z;
+        } else {
+            *reinterpret_cast<E8 *>(trunc + poff[i]) = tv;
+        }
+    }
+    // pixels of the tile without an update: mask word 0
+    if (wave == 0 && kq == 0 && px < p.P && !on) out_mask[px] = 0;
+}
+
 // ----------------------------------------------------------- large maps: active-pixel gather
 // On maps of tens of thousands of pixels and more (many video streams in a batch, large frames)
 // the fixed runs of 64 pixels above spend most of their workgroups on runs without an update,
@@ -787,6 +924,33 @@ hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *
                        (int64_t)p.P * p.Co * 2 > (4 << 20);
     // ... nor for filters beyond 32 KB, which every 16-pixel workgroup would stream in full
     const bool small_filter = (int64_t)p.ci_p * p.Co * 2 <= (32 << 10);
+    // large layers with a filter of up to 128 KB: the fused form with its epilogue on pixel rows
+    if (fusable && large && epi->mode == DC_TRUNC_MAX && p.Co % 8 == 0 && al16(epi->prev) && al16(epi->trunc) &&
+        al16(out) && ksteps <= PW_FUSED_MAX_STEPS && p.P >= 4096 && p.co_tiles <= 64 &&
+        (int64_t)p.ci_p * p.Co * 2 <= (128 << 10) && config_slices(pick_config(p, ksteps)) == 1) {
+        dim3 grid(ceil_div(p.P, 16));
+        const int act = epi->act < 0 ? 0 : epi->act;
+        const size_t lds = (size_t)16 * (p.Co * 2 + 16);
+        note_kernel("pw_rows_act_kernel");
+#define DC_ROWS(NWV, CTWV)                                                                              \
+    do {                                                                                              \
+        DC_ACT_SWITCH(act, (pw_rows_act_kernel<E, NWV, CTWV, A><<<grid, NWV * WAVE, lds, s>>>(          \
+                               p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask,  \
+                               out_mask, (E *)epi->prev, (E *)epi->trunc, epi->thr)));                \
+        *epilogue_done = true;                                                                        \
+        return hipGetLastError();                                                                     \
+    } while (0)
+        if (p.co_tiles <= 4) DC_ROWS(4, 1);
+        if (p.co_tiles <= 8) DC_ROWS(4, 2);
+        if (p.co_tiles <= 12) DC_ROWS(4, 3);
+        if (p.co_tiles <= 16) DC_ROWS(4, 4);
+        if (p.co_tiles <= 24) DC_ROWS(8, 3);
+        if (p.co_tiles <= 32) DC_ROWS(16, 2);
+        if (p.co_tiles <= 40) DC_ROWS(8, 5);
+        if (p.co_tiles <= 48) DC_ROWS(16, 3);
+        DC_ROWS(16, 4);
+#undef DC_ROWS
+    }
     if (fusable && ksteps <= PW_FUSED_MAX_STEPS && p.P >= 512 && !large && small_filter) {
         dim3 grid(ceil_div(p.P, 16));
         const int act = epi->act < 0 ? 0 : epi->act;

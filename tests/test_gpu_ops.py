@@ -633,6 +633,47 @@ def test_pointwise_gather_with_activation(lib, dtype, cin, cout, act, density):
     assert_masked_equal(out2, out1.cpu(), om1.cpu(), "out")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["float16", "bfloat16"])
+@pytest.mark.parametrize("cfg", [(64, 384, 56, 56), (96, 576, 56, 56), (32, 192, 112, 112), (64, 1024, 48, 48),
+                                 (24, 40, 170, 170), (96, 264, 64, 64)], ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("act", [1, 2, 4])
+@pytest.mark.parametrize("density", [0.03, 0.6, 1.0])
+def test_pointwise_rows_epilogue(lib, dtype, cfg, act, density):
+    """dc_conv_act on layers whose output map exceeds 4 MB (as with many streams in a batch) and
+    whose filter stays below 128 KB: one launch (pw_rows_act_kernel), bit-identical -- output,
+    both cached tensors, mask -- to dc_conv followed by dc_activate_truncate, and the convolution
+    within tolerance of the oracle's."""
+    cin, cout, H, W = cfg
+    g = _gen(1600 + cin + cout)
+    B = 2
+    mask = rand_mask(g, B, H, W, density)
+    x = torch.randn(B, cin, H, W, generator=g)
+    x = (x * torch.where(torch.rand(B, 1, H, W, generator=g) < 0.5, 1.0, 1e-3)).to(dtype)  # half of the updates get truncated
+    wt = (torch.randn(cout, cin, 1, 1, generator=g) / cin ** 0.5).to(dtype)
+    prev = torch.randn(B, cout, H, W, generator=g).to(dtype)
+    trunc = (torch.randn(B, cout, H, W, generator=g) * 0.05).to(dtype)
+    from deltacnn_amd.filter_conversion import convert_filter_out_channels_last, convert_half_filter
+    d_filt = (convert_half_filter(wt) if dtype == torch.float16 else convert_filter_out_channels_last(wt)).to(DEV)
+    pk = hk().pack_filter(d_filt, cin, cout, 1)
+    dx, dm = cl(poison(x, mask)), cl(mask)
+    thr = 0.9 if act != 4 else 0.2
+    p1, t1 = cl(prev), cl(trunc)
+    out1, om1 = hk().sparse_conv(dx, d_filt, dm, None, (1, 1), (0, 0), (1, 1), 1, c_out=cout, create_out_mask=True,
+                                 packed_filter=pk)
+    assert _last_kernel() == "pw_mfma_kernel"
+    want, want_mask = ops.conv(x, mask, wt, None, (1, 1), (0, 0), (1, 1), 1)
+    _check_conv(dtype, out1, want, want_mask)
+    hk().sparse_activation(out1, p1, t1, om1, thr, act, 0)
+    p2, t2 = cl(prev), cl(trunc)
+    out2, om2 = hk().sparse_conv_activation(dx, d_filt, dm, None, p2, t2, thr, act, 0, (1, 1), (0, 0), (1, 1), 1, cout,
+                                            packed_filter=pk)
+    assert _last_kernel() == "pw_rows_act_kernel"
+    assert torch.equal(om1, om2)
+    assert 0 < int(om1.sum()) < int(mask.sum())
+    assert torch.equal(p1, p2) and torch.equal(t1, t2)
+    assert_masked_equal(out2, out1.cpu(), om1.cpu(), "out")
+
+
 @pytest.mark.parametrize("cfg", [(96, 24, 56, 56), (144, 32, 28, 28), (384, 64, 14, 14), (960, 160, 7, 7),
                                  (32, 20, 9, 9)], ids=lambda c: "-".join(str(v) for v in c))
 @pytest.mark.parametrize("weights", [(1.0, 1.0), (0.5, -1.5)])
