@@ -797,15 +797,18 @@ constexpr int PW_FUSED_MAX_STEPS = 10;
 int pick_config(const PwP &p, int ksteps) {
     const int64_t tiles = (int64_t)ceil_div(p.P, 16) * p.co_tiles;
     // 64 pixels x 64 channels per workgroup (every fragment used four times) from 2048 output
-    // tiles on; for reductions short enough for the fused kernel only where that kernel is not
-    // used (>= 4096 tiles), so that a layer keeps one summation order
-    if (p.co_tiles >= 4 && ((ksteps > PW_FUSED_MAX_STEPS && tiles >= 2048) || (ksteps >= 4 && tiles >= 4096))) return 5;
+    // tiles on (from 1536 for reductions of 16 steps and more); for reductions short enough for
+    // the fused kernel only where that kernel is not used (>= 4096 tiles), so that a layer keeps
+    // one summation order
+    if (p.co_tiles >= 4 && ((ksteps > PW_FUSED_MAX_STEPS && tiles >= 2048) || (ksteps >= 16 && tiles >= 1536) ||
+                            (ksteps >= 4 && tiles >= 4096)))
+        return 5;
     if (tiles >= 4096 && ksteps >= 2 && p.co_tiles >= 4) return 4;
     if (ksteps <= PW_FUSED_MAX_STEPS) return (ksteps <= 2 && p.P >= 4096 && p.co_tiles >= 2) ? 1 : 0;
     // long reductions: split over wavefronts while there are few tiles, one wavefront per tile
     // once the tiles alone fill the chip
     if (ksteps > 24) return tiles >= 1024 ? 0 : 3;
-    return 2;
+    return tiles >= 1024 ? 0 : 2;
 }
 
 namespace {
