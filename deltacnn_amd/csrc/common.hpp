@@ -260,6 +260,10 @@ struct Residual {  // optional DCAdd fused behind a convolution
 
 bool pointwise_eligible(const dc_geometry &g, int dtype);
 bool patch_eligible(const dc_geometry &g, int dtype);
+bool lds_add_eligible(const dc_geometry &g, int dtype, int activation);
+hipError_t launch_lds_conv_add(const dc_geometry &g, const void *in, const void *packed, const void *bias,
+                               void *out, const int32_t *mask, int32_t *out_mask, const Residual *res,
+                               int dtype, hipStream_t s);
 hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *packed,
                              const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
                              bool transposed, const Residual *res, int dtype, hipStream_t s,

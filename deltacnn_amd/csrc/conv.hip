@@ -868,23 +868,37 @@ conv_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp,
 //   * filter fragments (contiguous 1 KB reads) stream through a ring of D register buffers of
 //     S steps each, so D - 1 chunks are in flight while one is consumed: 4 LDS reads and
 //     4 * R MFMAs per step.
+// Operands of a DCAdd fused behind a convolution: a = residual, b = convolution.
+template <typename E>
+struct PatchRes {  // DCAdd fused behind the convolution: a = residual, b = convolution
+    const E *values;
+    const int32_t *mask;
+    E *prev;
+    float wa, wb;
+    int act;
+};
+
 constexpr int LDS_MAX_HALO = 1024;
 constexpr int LDS_MAX_STEPS = 1024;
 
-template <typename E, int R, int S, int D, int KS, bool TR>
+template <typename E, int R, int S, int D, int KS, bool TR, bool ADD>
 __global__ void __launch_bounds__(8 * WAVE)
 conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp,
                      const E *__restrict__ bias, E *__restrict__ out,
                      const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
-                     int co_blocks, int ci_p, int hal_h, int hal_w, int kcc, int lgv) {
+                     int co_blocks, int ci_p, int hal_h, int hal_w, int kcc, int lgv, PatchRes<E> rs) {
+    // ADD: the sum of a DCAdd without activation rides on the accumulators.  (With an activation the
+    // accumulated sum has to be read and written as well; in this kernel's 8-byte-per-lane epilogue
+    // that costs what the separate add kernel costs -- measured -- so that form is not offered.)
+    static_assert(!(ADD && TR), "the fused sum exists for plain convolutions only");
     typedef typename Elem16<E>::v4 E4;
     typedef typename Elem16<E>::v8 E8;
     constexpr int NT = 4;
     extern __shared__ __align__(16) unsigned char s_halo[];
     __shared__ int s_hpix[LDS_MAX_HALO];
     __shared__ int2 s_step[LDS_MAX_STEPS];
-    __shared__ int s_list[TILE_PX];
-    __shared__ int s_n;
+    __shared__ int s_list[TILE_PX];  // compacted tile pixels: index | 64 if updated | 128 if the residual is
+    __shared__ int s_n, s_nupd;
     const int b = blockIdx.z / co_blocks, cb = blockIdx.z % co_blocks;
     // TR (transposed, dilation 1): the outputs of one stride phase (py, px) form an ordinary
     // convolution of the input with the A x Bt filter taps ky = ry + a * stride, kx = rx + b * stride:
@@ -1026,6 +1040,8 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
         const int ly = tid >> 3, lx = tid & 7;
         const int oy = out_y(ly), ox = out_x(lx);
         const bool inb = oy < p.Ho && ox < p.Wo;
+        int rword = 0;  // ADD: the residual's mask word, requested before the window is examined
+        if (ADD) rword = rs.mask[((size_t)b * p.Ho + min(oy, p.Ho - 1)) * p.Wo + min(ox, p.Wo - 1)];
         bool upd = false;
         const int base = ly * vsy * hal_w + lx * vsx;
         if (!TR && p.Kh == 3 && p.Kw == 3) {  // the common window: nine independent reads
@@ -1036,11 +1052,17 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
                 for (int tb = 0; tb < Bt; ++tb) upd |= s_hpix[base + tap_off(ta, tb)] >= 0;
         }
         upd = upd && inb;
-        if (inb && cb == 0) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = upd ? 1 : 0;
+        const bool radd = ADD && inb && rword != 0;
+        const bool any = upd || radd;  // ADD: the union of both masks is written and compacted
+        if (inb && cb == 0) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = any ? 1 : 0;
         int n;
-        const int rank = wave_rank(upd, n);
-        if (upd) s_list[rank] = tid;
-        if (tid == 0) s_n = n;
+        const int rank = wave_rank(any, n);
+        if (any) s_list[rank] = tid | (upd ? 64 : 0) | (radd ? 128 : 0);
+        const bool tile_upd = ballot(upd) != 0;
+        if (tid == 0) {
+            s_n = n;
+            s_nupd = tile_upd ? 1 : 0;
+        }
     }
     stage_store(0, min(kcc, ksteps), tid >> lgv, val0, px0);
     __syncthreads();
@@ -1052,8 +1074,36 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int slot = nt * 16 + l16;
-        const int loc = slot < n ? s_list[slot] : 0;
+        const int loc = slot < n ? (s_list[slot] & 63) : 0;
         hbase[nt] = ((loc >> 3) * vsy * hal_w + (loc & 7) * vsx) * row + kq * 16;
+    }
+    // ADD: the operands of the sum for all tiles of this lane, requested before the reduction,
+    // which they overlap
+    E4 rv[ADD ? R : 1][ADD ? NT : 1];
+    if (ADD && kz == 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int co = ((cb * ncw + cw) * R + r) * 16 + kq * 4;
+            const bool vec = co + 3 < p.Co && (p.Co & 3) == 0;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                rv[r][nt] = zero4<E>();
+                const int pix = nt * 16 + l16;
+                if (pix >= n || co >= p.Co) continue;
+                const int code = s_list[pix], loc = code & 63;
+                const size_t off = (((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7)) * p.Co;
+                const bool radd = (code & 128) != 0;
+                if (vec) {
+                    if (radd) rv[r][nt] = *reinterpret_cast<const E4 *>(rs.values + off + co);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int c = min(co + i, p.Co - 1);
+                        if (radd) rv[r][nt][i] = rs.values[off + c];
+                    }
+                }
+            }
+        }
     }
     float4_t acc[R][NT];
 #pragma unroll
@@ -1061,7 +1111,9 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[r][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int kbase = 0; kbase < ksteps; kbase += kcc) {
+    // ADD: a tile reached by the residual only has nothing to contract (uniform)
+    const int kend = (ADD && s_nupd == 0) ? 0 : ksteps;
+    for (int kbase = 0; kbase < kend; kbase += kcc) {
         const int kcur = min(kcc, ksteps - kbase);
         if (kbase > 0) {
             __syncthreads();
@@ -1167,17 +1219,30 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
         for (int nt = 0; nt < NT; ++nt) {
             const int pix = nt * 16 + l16;
             if (pix >= n) continue;
-            const int loc = s_list[pix];
-            E *o = out + (((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7)) * p.Co + co;
-            if (co + 3 < p.Co && (p.Co & 3) == 0) {
-                E4 v;
+            const int code = s_list[pix], loc = code & 63;
+            const size_t opix = ((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7);
+            E *o = out + opix * p.Co + co;
+            const bool vec = co + 3 < p.Co && (p.Co & 3) == 0;
+            E4 v;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v[i] = E(acc[r][nt][i] + float(bv[r][i]));
+            for (int i = 0; i < 4; ++i) v[i] = E(acc[r][nt][i] + float(bv[r][i]));
+            if (ADD) {  // add_kernel's sequence on the rounded convolution result: s = a * wa; s = fma(b, wb, s)
+                const bool upd = (code & 64) != 0, radd = (code & 128) != 0;
+                const E wa = E(rs.wa), wb = E(rs.wb);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    E sum = E(0);
+                    if (radd) sum = rv[r][nt][i] * wa;
+                    if (upd) sum = fma_t(v[i], wb, sum);
+                    v[i] = sum;
+                }
+            }
+            if (vec) {
                 *reinterpret_cast<E4 *>(o) = v;
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (co + i < p.Co) o[i] = E(acc[r][nt][i] + float(bv[r][i]));
+                    if (co + i < p.Co) o[i] = v[i];
             }
         }
     }
@@ -1191,14 +1256,6 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
 // Fragments of taps that are out of bounds or inactive are zeroed by selection (every step is
 // computed: at this size the instruction stream, not the MFMA count, is the kernel time);
 // outputs are stored for updated pixels only.  KW wavefronts split the reduction steps round-robin.
-template <typename E>
-struct PatchRes {  // DCAdd fused behind the convolution: a = residual, b = convolution
-    const E *values;
-    const int32_t *mask;
-    E *prev;
-    float wa, wb;
-    int act;
-};
 
 // ADD: out = wa * residual [its mask] + wb * conv [updated pixels], out_mask = the union; with an
 // activation the sum is accumulated in `prev` and its activated difference is emitted -- the
@@ -1965,6 +2022,106 @@ bool patch_eligible(const dc_geometry &g, int dtype) {
 }
 
 namespace {
+// Launch plan of conv_lds_mfma_kernel for a layer the 4x4-patch kernel does not take; !ok: the
+// halo or the step table does not fit (or a transposed convolution is dilated).
+struct LdsPlan {
+    bool ok;
+    int hal_h, hal_w, ltx, lty, vk2, kcc, rl, ksl, ncw;
+};
+
+LdsPlan lds_plan(const dc_geometry &g, bool transposed) {
+    LdsPlan lp{};
+    if (transposed && !(g.dilation_h == 1 && g.dilation_w == 1)) return lp;
+    const int co_tiles = ceil_div(g.out_c, 16);
+    const int ksteps_all = round_up(g.in_c, 32) / 32;
+    // taps per dimension seen by a tile: all of them, or those of one stride phase
+    const int vkh = transposed ? ceil_div(g.kernel_h, g.stride_h) : g.kernel_h;
+    const int vkw = transposed ? ceil_div(g.kernel_w, g.stride_w) : g.kernel_w;
+    lp.vk2 = vkh * vkw;
+    lp.hal_h = transposed ? TILE + vkh - 1 : (TILE - 1) * g.stride_h + (g.kernel_h - 1) * g.dilation_h + 1;
+    lp.hal_w = transposed ? TILE + vkw - 1 : (TILE - 1) * g.stride_w + (g.kernel_w - 1) * g.dilation_w + 1;
+    // transposed: one tile per (8x8 block of pixels one stride apart, stride phase)
+    lp.ltx = transposed ? ceil_div(ceil_div(g.out_w, g.stride_w), TILE) * g.stride_w : ceil_div(g.out_w, TILE);
+    lp.lty = transposed ? ceil_div(ceil_div(g.out_h, g.stride_h), TILE) * g.stride_h : ceil_div(g.out_h, TILE);
+    const int hpx = lp.hal_h * lp.hal_w;
+    // Arrangements (R channel tiles per wavefront, KS reduction slices, channel groups):
+    // wide outputs on many tiles: R = 2, four channel groups; otherwise, with enough
+    // steps to split, R = 2 and two or four slices (x two or one channel groups); short
+    // reductions: R = 1, up to four channel groups.
+    const int64_t tiles = (int64_t)lp.ltx * lp.lty * g.batch;
+    auto plan = [&](int lds_budget) {
+        const int kmax = hpx <= LDS_MAX_HALO ? (lds_budget / hpx - 16) / 64 : 0;
+        lp.kcc = kmax >= 1 ? ceil_div(ksteps_all, ceil_div(ksteps_all, kmax)) : 0;
+        const int nsteps_chunk = lp.vk2 * lp.kcc;
+        lp.rl = 1; lp.ksl = 1; lp.ncw = std::min(4, co_tiles);
+        if (co_tiles >= 16 && tiles * ceil_div(co_tiles, 8) >= 512) { lp.rl = 2; lp.ncw = 4; }
+        else if (nsteps_chunk >= 16 && co_tiles >= 4) {
+            // no more workgroups than compute units and a long reduction: eight wavefronts
+            lp.rl = 2; lp.ncw = 2;
+            lp.ksl = (nsteps_chunk >= 36 && tiles * ceil_div(co_tiles, 4) <= 256) ? 4 : 2;
+        }
+        else if (nsteps_chunk >= 16 && co_tiles >= 2) { lp.rl = 2; lp.ksl = 4; lp.ncw = 1; }
+    };
+    // Fewer LDS passes over the input channels (each costs a table, a staging round trip
+    // and a ring start-up) where a larger halo does not cost residency: a compute unit
+    // holds one workgroup of this launch anyway.  Otherwise 48 KB, two workgroups per
+    // compute unit.
+    plan(48 << 10);
+    const int passes_small = lp.kcc >= 1 ? ceil_div(ksteps_all, lp.kcc) : 1 << 30;
+    plan(112 << 10);
+    if (!(lp.kcc >= 1 && ceil_div(ksteps_all, lp.kcc) < passes_small &&
+          tiles * ceil_div(co_tiles, lp.ncw * lp.rl) <= 256))
+        plan(48 << 10);
+    // the step table holds all steps of a channel chunk plus the ring's run-out
+    lp.ok = lp.kcc >= 1 && lp.vk2 * lp.kcc + 48 <= LDS_MAX_STEPS;
+    return lp;
+}
+
+// res != nullptr (plain convolutions only): the DCAdd behind the convolution runs on the
+// accumulators, see conv_lds_mfma_kernel.
+template <typename E>
+hipError_t launch_lds_conv(const dc_geometry &g, const ConvP &p, const LdsPlan &lp, const void *in, const void *packed,
+                           const void *bias, void *out, const int32_t *mask, int32_t *out_mask, bool transposed,
+                           const Residual *res, hipStream_t s) {
+    const int co_tiles = ceil_div(g.out_c, 16);
+    const int ci_p = round_up(g.in_c, 32);
+    const int hpx = lp.hal_h * lp.hal_w;
+    const int kcc = lp.kcc, hal_h = lp.hal_h, hal_w = lp.hal_w;
+    const int nwv = lp.ncw * lp.ksl;  // wavefronts per workgroup
+    const int cbl = ceil_div(co_tiles, lp.ncw * lp.rl);
+    const size_t lds = std::max((size_t)hpx * (kcc * 64 + 16), (size_t)(lp.ksl - 1) * lp.ncw * lp.rl * 4 * 1024);
+    const int lgv = log2i(pow2_ceil(kcc * 4));  // lanes per halo pixel while staging
+    dim3 lgrid(lp.ltx, lp.lty, g.batch * cbl);
+    PatchRes<E> rs{nullptr, nullptr, nullptr, 0.f, 0.f, 0};
+    if (res != nullptr) rs = PatchRes<E>{(const E *)res->values, res->mask, (E *)res->prev, res->wa, res->wb, res->act};
+    note_kernel("conv_lds_mfma_kernel");
+#define DC_LDS_ARGS (p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv, rs)
+#define DC_LDS_K(RV, SV, DV, KV, TV, AV)                                                                    \
+    do {                                                                                                    \
+        if (lds > (48u << 10)) {                                                                            \
+            const hipError_t big = allow_large_lds(&conv_lds_mfma_kernel<E, RV, SV, DV, KV, TV, AV>);       \
+            if (big != hipSuccess) return big;                                                              \
+        }                                                                                                   \
+        conv_lds_mfma_kernel<E, RV, SV, DV, KV, TV, AV><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS;          \
+    } while (0)
+#define DC_LDS_L(RV, SV, DV, KV)                                                                            \
+    do {                                                                                                    \
+        if (res != nullptr) DC_LDS_K(RV, SV, DV, KV, false, true);                                          \
+        else if (transposed) DC_LDS_K(RV, SV, DV, KV, true, false);                                         \
+        else DC_LDS_K(RV, SV, DV, KV, false, false);                                                        \
+    } while (0)
+    if (lp.rl == 1) DC_LDS_L(1, 2, 3, 1);
+    else if (lp.ksl == 1) DC_LDS_L(2, 2, 3, 1);
+    else if (lp.ksl == 2) DC_LDS_L(2, 2, 3, 2);
+    else DC_LDS_L(2, 2, 3, 4);
+#undef DC_LDS_L
+#undef DC_LDS_K
+#undef DC_LDS_ARGS
+    return hipGetLastError();
+}
+}  // namespace
+
+namespace {
 template <typename E>
 hipError_t launch_patch_conv_t(const dc_geometry &g, const void *in, const void *packed,
                                const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
@@ -2014,6 +2171,22 @@ hipError_t launch_patch_conv_t(const dc_geometry &g, const void *in, const void 
     return hipGetLastError();
 }
 }  // namespace
+
+// Layers of the LDS-halo kernel (larger K x K convolutions) have the fused residual sum too, for a
+// DCAdd without activation.
+bool lds_add_eligible(const dc_geometry &g, int dtype, int activation) {
+    return activation <= 0 && mfma_eligible(g, dtype) && g.kernel_h * g.kernel_w <= MFMA_MAX_TAPS && !patch_eligible(g, dtype) &&
+           lds_plan(g, false).ok;
+}
+
+hipError_t launch_lds_conv_add(const dc_geometry &g, const void *in, const void *packed, const void *bias,
+                               void *out, const int32_t *mask, int32_t *out_mask, const Residual *res,
+                               int dtype, hipStream_t s) {
+    const ConvP p = make_params(g, DC_F16);  // the packed filter's layout does not depend on the type
+    const LdsPlan lp = lds_plan(g, false);
+    if (dtype == DC_BF16) return launch_lds_conv<bf16_t>(g, p, lp, in, packed, bias, out, mask, out_mask, false, res, s);
+    return launch_lds_conv<half_t>(g, p, lp, in, packed, bias, out, mask, out_mask, false, res, s);
+}
 
 hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *packed,
                              const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
@@ -2071,80 +2244,12 @@ hipError_t launch_conv_t(const dc_geometry &g, const void *in, const void *filte
                                             epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
         }
         // Larger layers: halo staged in LDS (see conv_lds_mfma_kernel).
-        if (!transposed || (g.dilation_h == 1 && g.dilation_w == 1)) {
-            // taps per dimension seen by a tile: all of them, or those of one stride phase
-            const int vkh = transposed ? ceil_div(g.kernel_h, g.stride_h) : g.kernel_h;
-            const int vkw = transposed ? ceil_div(g.kernel_w, g.stride_w) : g.kernel_w;
-            const int hal_h = transposed ? TILE + vkh - 1 : (TILE - 1) * g.stride_h + (g.kernel_h - 1) * g.dilation_h + 1;
-            const int hal_w = transposed ? TILE + vkw - 1 : (TILE - 1) * g.stride_w + (g.kernel_w - 1) * g.dilation_w + 1;
-            // transposed: one tile per (8x8 block of pixels one stride apart, stride phase)
-            const int ltx = transposed ? ceil_div(ceil_div(g.out_w, g.stride_w), TILE) * g.stride_w : tx;
-            const int lty = transposed ? ceil_div(ceil_div(g.out_h, g.stride_h), TILE) * g.stride_h : ty;
-            const int hpx = hal_h * hal_w;
-            const int ksteps_all = ci_p / 32;
-            // Arrangements (R channel tiles per wavefront, KS reduction slices, channel groups):
-            // wide outputs on many tiles: R = 2, four channel groups; otherwise, with enough
-            // steps to split, R = 2 and two or four slices (x two or one channel groups); short
-            // reductions: R = 1, up to four channel groups.
-            const int64_t tiles = (int64_t)ltx * lty * g.batch;
-            int kcc = 0, rl = 1, ksl = 1, ncw = 1;
-            auto plan = [&](int lds_budget) {
-                const int kmax = hpx <= LDS_MAX_HALO ? (lds_budget / hpx - 16) / 64 : 0;
-                kcc = kmax >= 1 ? ceil_div(ksteps_all, ceil_div(ksteps_all, kmax)) : 0;
-                const int nsteps_chunk = vkh * vkw * kcc;
-                rl = 1; ksl = 1; ncw = std::min(4, co_tiles);
-                if (co_tiles >= 16 && tiles * ceil_div(co_tiles, 8) >= 512) { rl = 2; ncw = 4; }
-                else if (nsteps_chunk >= 16 && co_tiles >= 4) {
-                    // no more workgroups than compute units and a long reduction: eight wavefronts
-                    rl = 2; ncw = 2;
-                    ksl = (nsteps_chunk >= 36 && tiles * ceil_div(co_tiles, 4) <= 256) ? 4 : 2;
-                }
-                else if (nsteps_chunk >= 16 && co_tiles >= 2) { rl = 2; ksl = 4; ncw = 1; }
-            };
-            // Fewer LDS passes over the input channels (each costs a table, a staging round trip
-            // and a ring start-up) where a larger halo does not cost residency: a compute unit
-            // holds one workgroup of this launch anyway.  Otherwise 48 KB, two workgroups per
-            // compute unit.
-            plan(48 << 10);
-            const int passes_small = kcc >= 1 ? ceil_div(ksteps_all, kcc) : 1 << 30;
-            plan(112 << 10);
-            if (!(kcc >= 1 && ceil_div(ksteps_all, kcc) < passes_small &&
-                  tiles * ceil_div(co_tiles, ncw * rl) <= 256))
-                plan(48 << 10);
-            // the step table holds all steps of a channel chunk plus the ring's run-out
-            if (kcc >= 1 && vkh * vkw * kcc + 48 <= LDS_MAX_STEPS) {
-                const int nwv = ncw * ksl;  // wavefronts per workgroup
-                const int cbl = ceil_div(co_tiles, ncw * rl);
-                const size_t lds = std::max((size_t)hpx * (kcc * 64 + 16), (size_t)(ksl - 1) * ncw * rl * 4 * 1024);
-                const int lgv = log2i(pow2_ceil(kcc * 4));  // lanes per halo pixel while staging
-                dim3 lgrid(ltx, lty, g.batch * cbl);
-                note_kernel("conv_lds_mfma_kernel");
-#define DC_LDS_ARGS (p, (const E16 *)in, (const E16 *)packed, (const E16 *)bias, (E16 *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv)
-#define DC_LDS_K(RV, SV, DV, KV, TV)                                                                        \
-    do {                                                                                                    \
-        if (lds > (48u << 10)) {                                                                            \
-            const hipError_t big = allow_large_lds(&conv_lds_mfma_kernel<E16, RV, SV, DV, KV, TV>);              \
-            if (big != hipSuccess) return big;                                                              \
-        }                                                                                                   \
-        conv_lds_mfma_kernel<E16, RV, SV, DV, KV, TV><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS;                 \
-    } while (0)
-#define DC_LDS_L(RV, SV, DV, KV)                                                                            \
-    do {                                                                                                    \
-        if (transposed) DC_LDS_K(RV, SV, DV, KV, true);                                                     \
-        else DC_LDS_K(RV, SV, DV, KV, false);                                                               \
-    } while (0)
-                if (rl == 1) DC_LDS_L(1, 2, 3, 1);
-                else if (ksl == 1) DC_LDS_L(2, 2, 3, 1);
-                else if (ksl == 2) DC_LDS_L(2, 2, 3, 2);
-                else DC_LDS_L(2, 2, 3, 4);
-#undef DC_LDS_L
-#undef DC_LDS_K
-#undef DC_LDS_ARGS
-                hipError_t le = hipGetLastError();
-                if (le != hipSuccess || epi == nullptr) return le;
-                return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
-                                                epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
-            }
+        const LdsPlan lp = lds_plan(g, transposed);
+        if (lp.ok) {
+            hipError_t le = launch_lds_conv<E16>(g, p, lp, in, packed, bias, out, mask, out_mask, transposed, nullptr, s);
+            if (le != hipSuccess || epi == nullptr) return le;
+            return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
+                                            epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
         }
         // transposed: one tile per (8x8 block of pixels one stride apart, stride phase)
         const int gtx = transposed ? ceil_div(ceil_div(g.out_w, g.stride_w), TILE) * g.stride_w : tx;

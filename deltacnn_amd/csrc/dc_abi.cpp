@@ -210,10 +210,11 @@ int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filt
     if (activation < 0 || activation > DC_ACT_SWISH)
         return fail(DC_ERR_UNSUPPORTED, "dc_conv_add: activation %d", activation);
     const bool pointwise = dc::pointwise_eligible(*g, dtype);
-    if (!pointwise && !dc::patch_eligible(*g, dtype))
+    const bool patch = !pointwise && dc::patch_eligible(*g, dtype);
+    if (!pointwise && !patch && !dc::lds_add_eligible(*g, dtype, activation))
         return fail(DC_ERR_UNSUPPORTED, "dc_conv_add: only 16-bit 1x1 stride-1 convolutions with "
-                                        "Cin %% 8 == 0 and Cout %% 4 == 0 and small "
-                                        "16-bit layers with Cin %% 8 == 0 have the fused form");
+                                        "Cin %% 8 == 0 and Cout %% 4 == 0 and 16-bit K x K layers "
+                                        "with Cin %% 8 == 0 and at most 64 taps have the fused form");
     DC_REQUIRE_PTR("dc_conv_add", input);
     DC_REQUIRE_PTR("dc_conv_add", packed_filter);
     DC_REQUIRE_PTR("dc_conv_add", mask);
@@ -234,6 +235,9 @@ int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filt
         return finish(dc::launch_pointwise(*g, input, packed_filter, bias, out, mask, out_mask, nullptr,
                                            &unused, &res, dtype, (hipStream_t)stream), "dc_conv_add");
     }
+    if (!patch)
+        return finish(dc::launch_lds_conv_add(*g, input, packed_filter, bias, out, mask, out_mask, &res, dtype,
+                                              (hipStream_t)stream), "dc_conv_add");
     return finish(dc::launch_patch_conv(*g, input, packed_filter, bias, out, mask, out_mask, false, &res,
                                         dtype, (hipStream_t)stream), "dc_conv_add");
 }

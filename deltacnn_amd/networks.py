@@ -414,6 +414,12 @@ class _HRModule(nn.Module):
                 if j > len(outs) and hasattr(add, "after_upsample"):
                     # 1x1 convolution + upsampling: the upsampling is folded into the sum
                     y = add.after_upsample(y, branch[0](xs[j]), branch[1])
+                elif isinstance(branch, nn.Sequential):
+                    # strided 3x3 convolutions: the sum rides in the last one's kernel where it can
+                    mid = xs[j]
+                    for step in list(branch)[:-1]:
+                        mid = step(mid)
+                    y = _residual_sum(add, y, branch[-1], mid)
                 else:
                     y = add(y, branch(xs[j]))
             outs.append(y)

@@ -117,11 +117,12 @@ int dc_conv_act(const dc_geometry *g, const void *input, const void *filter,
  * s = weight_residual * a [mask_residual] + weight_conv * b [mask]; activation == 0: out = s;
  * activation > 0 (other_nn_layers.cu:1379-1559): prev_out += s, out = act(prev_out) - act(old
  * prev_out).  out_mask = mask | mask_residual.  Results are identical to dc_conv followed by
- * dc_add(residual, conv).  No counterpart in the reference.  Two forms exist, both for the
- * 16-bit types: 1x1 stride-1 convolutions without padding (Cin % 8 == 0, Cout % 4 == 0), and small
- * layers of any kernel size (Cin % 8 == 0, groups 1, at most 64 taps,
- * ceil(W/4) * ceil(H/4) * B * ceil(Cout/16) * Kh * Kw * ceil(Cin/32) <= 32768), both with or
- * without activation.  Both need a packed filter; anything else returns DC_ERR_UNSUPPORTED before any
+ * dc_add(residual, conv).  No counterpart in the reference.  For the 16-bit types: 1x1 stride-1
+ * convolutions without padding (Cin % 8 == 0, Cout % 4 == 0), and K x K layers (Cin % 8 == 0,
+ * groups 1, at most 64 taps) whose input window of an 8 x 8 output tile fits the kernel's LDS
+ * staging (any layer of up to 32 x 32 halo pixels does), with or
+ * without activation (layers beyond ceil(W/4) * ceil(H/4) * B * ceil(Cout/16) * Kh * Kw *
+ * ceil(Cin/32) = 32768: without activation only).  All need a packed filter; anything else returns DC_ERR_UNSUPPORTED before any
  * launch so that the caller can issue the two separate calls.  prev_out may be NULL when
  * activation == 0. */
 int dc_conv_add(const dc_geometry *g, const void *input, const void *packed_filter,
