@@ -342,6 +342,9 @@ def scaled_bench():
     h1, h2 = (torch.randn(B, C // 2, H, W, device="cuda", dtype=torch.half, generator=gen).contiguous(
         memory_format=torch.channels_last) for _ in range(2))
     scale, shift = (torch.randn(C, device="cuda", dtype=torch.half, generator=gen) for _ in range(2))
+    from deltacnn_amd.filter_conversion import convert_half_filter
+    wpw = convert_half_filter((torch.randn(C, C, 1, 1, generator=torch.Generator().manual_seed(8)) / C ** 0.5).half()).cuda()
+    wpw_packed = hk.pack_filter(wpw, C, C, 1)
     for rho in (0.1, 1.0):
         mask = (torch.rand(B, 1, H, W, device="cuda", generator=gen) < rho).to(torch.int32)
         mask2 = mask.clone()
@@ -360,6 +363,11 @@ def scaled_bench():
             "concat": (lambda: hk.sparse_concatenate((h1, mask), (h2, mask), out=(d, mask2)), None),
             "mul_add": (lambda: hk.sparse_mul_add(a, mask, d, mask2, scale, shift), None),
             "add_to_dense": (lambda: hk.sparse_add_to_dense_tensor(a, d, mask), None),
+            "pointwise64->64": (lambda: hk.sparse_conv(a, wpw, mask, None, (1, 1), (0, 0), (1, 1), 1, c_out=C, out=d,
+                                                         out_mask=mask2, packed_filter=wpw_packed), None),
+            "pointwise64->64+relu": (lambda: hk.sparse_conv_activation(a, wpw, mask, None, b, c, 0.0, 1, 0, (1, 1), (0, 0),
+                                                                         (1, 1), 1, C, out=d, out_mask=mask2,
+                                                                         packed_filter=wpw_packed), None),
         })
         qmask_in = (torch.rand(B, 1, H // 2, W // 2, device="cuda", generator=gen) < rho).to(torch.int32)
         if rho < 1:
