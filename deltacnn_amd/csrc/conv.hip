@@ -1846,9 +1846,10 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
     const int nvec = g.in_c / N;
     // very large maps: mask scan and compaction per wavefront (see conv_dw_scan_kernel)
     // (measured against the strip kernel and the per-pixel kernel on sparse and dense maps: it
-    // wins from 2^18 outputs on, with a stride -- where no strip kernel exists -- from 2^16)
+    // wins from 2^18 outputs on; with a stride -- where no strip kernel exists -- and with rows of
+    // up to 8 vectors, where it serves one pixel per lane group out of LDS-held filters, from 2^16)
     const bool strided = g.stride_h > 1 || g.stride_w > 1;
-    if (g.kernel_h == 3 && g.kernel_w == 3 && nvec <= WAVE && P_out >= (strided ? 1 << 16 : 1 << 18) && P_out < (1ll << 31) &&
+    if (g.kernel_h == 3 && g.kernel_w == 3 && nvec <= WAVE && P_out >= ((strided || nvec <= 8) ? 1 << 16 : 1 << 18) && P_out < (1ll << 31) &&
         (int64_t)g.batch * g.in_h * g.in_w < (1ll << 31) && g.out_h < 65536 && g.out_w < 65536 &&
         (epi == nullptr || epi->trunc != nullptr)) {
         const int lg = log2i(group_lanes(nvec, 1));

@@ -343,8 +343,9 @@ CONVS = [
     (16, 16, 3, 1, 1, 1, 16, 726, 727),     # depthwise on a very large map: mask scan and compaction per wavefront
     (24, 24, 3, 1, 1, 1, 24, 600, 601),     # ... with idle lanes in the group
     (16, 16, 3, 2, 1, 1, 16, 600, 521),     # ... with a stride
-    (16, 16, 3, 1, 1, 1, 16, 300, 301),     # depthwise on a large map: strips of four pixels per lane group
-    (24, 24, 3, 1, 1, 1, 24, 250, 251),     # ... with idle lanes in the group
+    (16, 16, 3, 1, 1, 1, 16, 300, 301),     # ... narrow rows take the scan from 2^16 outputs on
+    (64, 64, 3, 1, 1, 1, 64, 180, 181),     # depthwise on a large map: strips of four pixels per lane group
+    (40, 40, 3, 1, 1, 1, 40, 180, 181),     # ... with idle lanes in the group
     (144, 144, 3, 1, 1, 1, 144, 130, 131),  # ... wide rows on 8 MB and more: filter through LDS
 ]
 
@@ -424,7 +425,9 @@ def test_conv(lib, dtype, cfg, density, use_bias, packed):
     ((64, 256, 1, 1, 0, 1, 1, 20, 20), "pw_mfma_kernel"),
     ((32, 32, 3, 1, 1, 1, 32, 15, 18), "conv_dw_kernel"),
     ((16, 16, 3, 1, 1, 1, 16, 726, 727), "conv_dw_scan_kernel"),
-    ((16, 16, 3, 1, 1, 1, 16, 300, 301), "conv_dw_strip_kernel"),
+    ((16, 16, 3, 1, 1, 1, 16, 300, 301), "conv_dw_scan_kernel"),
+    ((64, 64, 3, 1, 1, 1, 64, 180, 181), "conv_dw_strip_kernel"),
+    ((40, 40, 3, 1, 1, 1, 40, 180, 181), "conv_dw_strip_kernel"),
     ((144, 144, 3, 1, 1, 1, 144, 130, 131), "conv_dw_strip_kernel"),
     ((16, 16, 3, 2, 1, 1, 16, 600, 521), "conv_dw_scan_kernel"),
     ((3, 32, 3, 2, 1, 1, 1, 33, 31), "conv_stem_mfma_kernel"),
@@ -521,7 +524,7 @@ FUSED = [
     (24, 24, 3, 1, 1, 1, 24, 192, 192),     # large map: three vectors per lane
     (16, 16, 3, 1, 1, 1, 16, 726, 727),     # very large map: mask scan and compaction per wavefront
     (24, 24, 3, 2, 1, 1, 24, 600, 521),     # the same with a stride
-    (16, 16, 3, 1, 1, 1, 16, 300, 301),     # large map: strips of four pixels per lane group
+    (64, 64, 3, 1, 1, 1, 64, 180, 181),     # large map: strips of four pixels per lane group
     (144, 144, 3, 1, 1, 1, 144, 130, 131),  # ... wide rows, filter through LDS
     (16, 96, 1, 1, 0, 1, 1, 110, 111),      # pointwise on a large map: convolution and activation as two launches
 ]
@@ -774,7 +777,7 @@ def test_conv_add_fused_small_layers(lib, cfg, act, weights, dtype):
     (64, 256, 1, 1, 0, 1, 1, 20, 20),       # pointwise
     (32, 32, 3, 1, 1, 1, 32, 15, 18),       # depthwise
     (16, 16, 3, 1, 1, 1, 16, 726, 727),     # depthwise, mask scan
-    (16, 16, 3, 1, 1, 1, 16, 300, 301),     # depthwise strips
+    (64, 64, 3, 1, 1, 1, 64, 180, 181),     # depthwise strips
     (3, 32, 3, 2, 1, 1, 1, 33, 31),         # stem
 ], ids=lambda c: "-".join(str(v) for v in c))
 def test_conv_uniform_masks(lib, cfg, fill):
