@@ -40,6 +40,18 @@ class BlockArgs(ctypes.Structure):
         ("flags", c_int32)]
 
 
+class ExpandDwArgs(ctypes.Structure):
+    """struct dc_expand_dw_args."""
+    _fields_ = [
+        ("input", c_void_p), ("mask", c_void_p), ("expand_packed_filter", c_void_p),
+        ("expand_in_channels", c_int32), ("expand_prev_out", c_void_p), ("expand_truncated", c_void_p),
+        ("expand_threshold", c_float), ("expand_activation", c_int32), ("expand_truncation_mode", c_int32),
+        ("expand_out", c_void_p), ("expand_out_mask", c_void_p),
+        ("dw_filter", c_void_p), ("dw_prev_out", c_void_p), ("dw_truncated", c_void_p),
+        ("dw_threshold", c_float), ("dw_activation", c_int32), ("dw_truncation_mode", c_int32),
+        ("out", c_void_p), ("out_mask", c_void_p)]
+
+
 _P = c_void_p
 _G = POINTER(Geometry)
 _SIGNATURES = {
@@ -52,6 +64,7 @@ _SIGNATURES = {
     "dc_conv_act": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_float, c_int, c_int, c_int, _P]),
     "dc_conv_add": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, _P, c_float, c_float, _P, c_int, c_int, _P]),
     "dc_block": (c_int, [_G, POINTER(BlockArgs), c_int, _P]),
+    "dc_expand_depthwise": (c_int, [_G, POINTER(ExpandDwArgs), c_int, _P]),
     "dc_packed_filter_bytes": (c_int64, [_G, c_int, c_int]),
     "dc_pack_filter": (c_int, [_G, _P, _P, c_int, c_int, _P]),
     "dc_deconv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),

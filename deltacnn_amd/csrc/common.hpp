@@ -60,6 +60,44 @@ __device__ __forceinline__ void vstore(T *p, const Vec<T, N> &x) {
     *reinterpret_cast<Vec<T, N> *>(p) = x;
 }
 
+// DC_PIN (below) for a 16-byte Vec: the load that produced `x` is issued before this program
+// point instead of where the compiler would sink it to -- next to its first use, possibly behind
+// a barrier or a run of stores, where its latency would be paid on its own.  Place it where
+// the value has arrived anyway (behind a wait for a request issued later).
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+template <typename T, int N>
+__device__ __forceinline__ void pin_vec(Vec<T, N> &x) {
+    static_assert(sizeof(Vec<T, N>) == 16, "16-byte vectors only");
+    union {
+        Vec<T, N> v;
+        u32x4_t r;
+    } c;
+    c.v = x;
+    asm volatile("" : "+v"(c.r));
+    x = c.v;
+}
+
+// Largest magnitude of a 16-byte vector's elements (NaN elements are skipped, as a comparison
+// against a threshold would skip them); halves take the packed instructions.
+__device__ __forceinline__ float vec_absmax(const Vec<half_t, 8> &x) {
+    union {
+        Vec<half_t, 8> v;
+        half8_t h;
+    } c;
+    c.v = x;
+    const half8_t a = __builtin_elementwise_abs(c.h);
+    const half4_t m4 = __builtin_elementwise_max(a.lo, a.hi);
+    const half2_t m2 = __builtin_elementwise_max(m4.lo, m4.hi);
+    return float(__builtin_fmaxf16(m2[0], m2[1]));
+}
+template <typename T, int N>
+__device__ __forceinline__ float vec_absmax(const Vec<T, N> &x) {
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < N; ++j) m = fmaxf(m, __builtin_fabsf(float(x.v[j])));
+    return m;
+}
+
 // A 16-byte vector kept if `on`, else all-zero bits: four 32-bit selects whatever the element
 // type (a per-element select on halves costs twice as many instructions).
 template <typename T, int N>
@@ -258,6 +296,23 @@ struct Residual {  // optional DCAdd fused behind a convolution
     int act = 0;           // its activation (0: none)
 };
 
+// A layer's activation / truncation left open by its convolution and finished by the depthwise
+// layer that consumes it: the layer's cached state (its truncated values receive T = truncated + v
+// from the convolution), its threshold and activation.
+struct OpenAct {
+    void *prev = nullptr;
+    void *trunc = nullptr;
+    float thr = 0.f;
+    int act = 0;
+};
+bool depthwise_closing_eligible(const dc_geometry &g, const ActEpilogue *epi, int dtype);
+hipError_t launch_depthwise_closing(const dc_geometry &g, const void *in, const void *filter, void *out,
+                                    const int32_t *mask, int32_t *out_mask, const ActEpilogue *epi,
+                                    const OpenAct &open, int dtype, hipStream_t s);
+bool pointwise_open_eligible(const dc_geometry &g, int dtype, int activation);
+hipError_t launch_pointwise_open(const dc_geometry &g, const void *in, const void *packed, void *out,
+                                 const int32_t *mask, int32_t *out_mask, const OpenAct &open, int dtype,
+                                 hipStream_t s);
 bool pointwise_eligible(const dc_geometry &g, int dtype);
 bool patch_eligible(const dc_geometry &g, int dtype);
 bool lds_add_eligible(const dc_geometry &g, int dtype, int activation);

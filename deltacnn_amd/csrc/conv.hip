@@ -103,14 +103,33 @@ struct EpiP {
     int mode;
 };
 
+// The activation / truncation of the layer that PRODUCED this kernel's input, left open by
+// that layer (see pw_mfma_kernel MODE 3): `in` holds D = act(S) - act(prev) for every pixel the
+// producer's convolution updated (mask = its update mask), and the layer's truncated values
+// already hold T = truncated + v for those pixels.
+struct OpenActP {
+    void *prev;
+    void *trunc;
+    float thr;
+};
+
 // EAGER (3x3 only, small maps): the nine input rows, the filter and the cached state are
 // requested before the mask words have arrived -- their addresses depend on coordinates only --
 // so the whole kernel is one memory round trip; what is loaded for inactive pixels is dropped.
-template <typename T, int ITERS, int ACT, bool K3, bool EAGER>
+// FIN (EAGER, stride 1, padding 1): the producing layer's activation / truncation is finished
+// here, which saves that layer's activation launch.  A window pixel counts as updated only if
+// the producer's keep decision holds for it -- any |D| above the producer's threshold over all
+// channels, which this lane group sees since it reads the pixel's whole row anyway -- and the
+// group commits the producer's cached state of its CENTRE pixel (every pixel is the centre of
+// exactly one group): kept: prev += T, truncated = 0; dropped: truncated = T, which it holds
+// already.  Neighbouring groups read D and the update mask only, never that state, so nothing
+// races.
+template <typename T, int ITERS, int ACT, bool K3, bool EAGER, bool FIN = false>
 __global__ void __launch_bounds__(256)
 conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
                const T *__restrict__ bias, T *__restrict__ out, const int32_t *__restrict__ mask,
-               int32_t *__restrict__ out_mask, EpiP epi, int lg) {
+               int32_t *__restrict__ out_mask, EpiP epi, int lg, OpenActP fin = OpenActP{}) {
+    static_assert(!FIN || (K3 && EAGER), "the open activation is finished by the eager 3x3 form only");
     constexpr int N = Vec16<T>::N;
     const int G = 1 << lg;
     const int C = p.Ci;
@@ -154,6 +173,18 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
             }
         }
     }
+    // FIN: T and the accumulated value of the centre pixel (stride 1, padding 1: input pixel
+    // (oy, ox)), requested with everything else
+    Vec<T, N> ft[FIN ? ITERS : 1], fq[FIN ? ITERS : 1];
+    const size_t centre = ((size_t)b * p.Hi + oy) * p.Wi + ox;
+    if (FIN) {
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int c = min((it * G + gl) * N, C - N);
+            ft[it] = vload<T, N>((const T *)fin.trunc + centre * C + c);
+            fq[it] = vload<T, N>((const T *)fin.prev + centre * C + c);
+        }
+    }
 
     uint64_t taps = 0;
     const int GW = G > WAVE ? WAVE : G;  // a group wider than a wavefront: every wavefront scans
@@ -166,6 +197,60 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
             if (iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi) m = mb[iy * p.Wi + ix] != 0;
         }
         taps |= ((ballot(m) >> glo) & gmask) << j;
+    }
+    if (FIN) {
+        // (the centre pixel's state was requested with everything else and has arrived with the
+        // mask words: keep the compiler from moving those requests down to the commit below)
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            pin_vec(ft[it]);
+            pin_vec(fq[it]);
+        }
+        // the producer's keep decision for the nine window pixels: this lane's share first (what
+        // was loaded for a pixel without update is dropped), then the group's, straight-line
+        const float fthr = float(T(fin.thr));
+        uint32_t mine = 0;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            float big = 0.f;
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) big = fmaxf(big, vec_absmax(ex[t][it]));
+            mine |= (big > fthr ? 1u : 0u) << t;
+        }
+        mine &= (uint32_t)taps;
+        uint64_t kept = 0;
+        if (G >= WAVE) {
+#pragma unroll
+            for (int t = 0; t < 9; ++t) kept |= (ballot((mine >> t) & 1u) != 0 ? 1ull : 0ull) << t;
+        } else {
+#pragma unroll
+            for (int t = 0; t < 9; ++t) kept |= (((ballot((mine >> t) & 1u) >> glo) & gmask) != 0 ? 1ull : 0ull) << t;
+        }
+        if (G > WAVE) {  // one pixel per workgroup: the wavefronts hold different channels
+            __shared__ uint32_t s_kept[4];
+            if (lane_id() == 0) s_kept[wave_id()] = (uint32_t)kept;
+            __syncthreads();
+            kept = 0;
+            for (int w = 0; w < (int)(blockDim.x / WAVE); ++w) kept |= s_kept[w];
+        }
+        const bool centre_updated = (taps >> 4) & 1ull;
+        taps &= kept;
+        if (valid && centre_updated && ((taps >> 4) & 1ull)) {  // kept
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int c = (it * G + gl) * N;
+                if (c < C) {
+                    Vec<T, N> z, sum;
+#pragma unroll
+                    for (int j = 0; j < N; ++j) {
+                        z.v[j] = T(0);
+                        sum.v[j] = ft[it].v[j] + fq[it].v[j];
+                    }
+                    vstore<T, N>((T *)fin.prev + centre * C + c, sum);
+                    vstore<T, N>((T *)fin.trunc + centre * C + c, z);
+                }
+            }
+        }
     }
     const bool active = valid && taps != 0;
     if (valid && gl == 0) out_mask[po] = active ? 1 : 0;
@@ -1928,6 +2013,55 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
     return true;
 }
 
+// The depthwise layer that finishes its producer's open activation (conv_dw_kernel<FIN>): 3x3,
+// stride 1, padding 1, on maps small enough for the eager per-pixel form (where launches, not
+// bytes, are the cost).  Returns false if the shape does not qualify; nothing is launched then.
+template <typename T>
+bool try_depthwise_closing(const dc_geometry &g, const ConvP &p, const T *in, const T *filter, T *out,
+                           const int32_t *mask, int32_t *out_mask, const ActEpilogue *epi, const OpenAct &open,
+                           bool launch, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    const auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (g.groups != g.in_c || g.groups != g.out_c || g.groups == 1) return false;
+    if (g.kernel_h != 3 || g.kernel_w != 3 || g.stride_h != 1 || g.stride_w != 1 || g.dilation_h != 1 ||
+        g.dilation_w != 1 || g.pad_top != 1 || g.pad_left != 1 || g.pad_bottom != 1 || g.pad_right != 1)
+        return false;
+    if (g.in_c % N != 0 || g.in_c / N > WAVE * 4) return false;
+    if (epi == nullptr || epi->trunc == nullptr || epi->mode < 0) return false;
+    const int64_t P_out = (int64_t)g.batch * g.out_h * g.out_w;
+    const int nvec = g.in_c / N;
+    if (P_out >= (1 << 16) || P_out * g.in_c * (int64_t)sizeof(T) >= (4 << 20)) return false;  // scan / strip kernels
+    const int wide = epi->mode == DC_TRUNC_MAX ? wide_group(nvec, P_out) : 0;
+    const int G = wide ? wide : pick_group(nvec, P_out, 4);
+    const int iters = ceil_div(nvec, G);
+    if (iters > 2 || P_out * g.in_c * (int64_t)sizeof(T) > (2 << 20)) return false;  // the eager form only
+    if (!launch) return true;
+    if (!al(in) || !al(filter) || !al(out) || !al(epi->prev) || !al(epi->trunc) || !al(open.prev) || !al(open.trunc))
+        return false;
+    const int block = wide ? wide : group_block(P_out * G);
+    note_kernel("conv_dw_kernel");
+    dim3 grid((unsigned)ceil_div64(P_out * G, block));
+    EpiP e{epi->prev, epi->trunc, epi->thr, epi->mode};
+    OpenActP f{open.prev, open.trunc, open.thr};
+    const int act = epi->act < 0 ? 0 : epi->act;
+    const int lg = log2i(G);
+#define DC_DWF(A)                                                                                                      \
+    do {                                                                                                               \
+        if (iters == 1) conv_dw_kernel<T, 1, A, true, true, true><<<grid, block, 0, s>>>(p, in, filter, nullptr, out, mask, out_mask, e, lg, f); \
+        else conv_dw_kernel<T, 2, A, true, true, true><<<grid, block, 0, s>>>(p, in, filter, nullptr, out, mask, out_mask, e, lg, f); \
+    } while (0)
+    switch (act) {
+        case DC_ACT_RELU: DC_DWF(DC_ACT_RELU); break;
+        case DC_ACT_RELU6: DC_DWF(DC_ACT_RELU6); break;
+        case DC_ACT_LEAKY: DC_DWF(DC_ACT_LEAKY); break;
+        case DC_ACT_SIGMOID: DC_DWF(DC_ACT_SIGMOID); break;
+        case DC_ACT_SWISH: DC_DWF(DC_ACT_SWISH); break;
+        default: DC_DWF(DC_ACT_LINEAR); break;
+    }
+#undef DC_DWF
+    return true;
+}
+
 // Stems of large frames on the matrix cores (see conv_stem_mfma_kernel); false if the shape, the
 // operands' alignment or the map size do not qualify.
 template <typename E>
@@ -2314,6 +2448,26 @@ hipError_t launch_conv_t(const dc_geometry &g, const void *in, const void *filte
                                     epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
 }
 }  // namespace
+
+bool depthwise_closing_eligible(const dc_geometry &g, const ActEpilogue *epi, int dtype) {
+    const ConvP p = make_params(g, dtype);
+    const OpenAct none{};
+    if (dtype == DC_F16)
+        return try_depthwise_closing<half_t>(g, p, nullptr, nullptr, nullptr, nullptr, nullptr, epi, none, false, nullptr);
+    if (dtype == DC_BF16)
+        return try_depthwise_closing<bf16_t>(g, p, nullptr, nullptr, nullptr, nullptr, nullptr, epi, none, false, nullptr);
+    return false;
+}
+
+hipError_t launch_depthwise_closing(const dc_geometry &g, const void *in, const void *filter, void *out,
+                                    const int32_t *mask, int32_t *out_mask, const ActEpilogue *epi,
+                                    const OpenAct &open, int dtype, hipStream_t s) {
+    const ConvP p = make_params(g, dtype);
+    const bool ok = dtype == DC_BF16
+        ? try_depthwise_closing<bf16_t>(g, p, (const bf16_t *)in, (const bf16_t *)filter, (bf16_t *)out, mask, out_mask, epi, open, true, s)
+        : try_depthwise_closing<half_t>(g, p, (const half_t *)in, (const half_t *)filter, (half_t *)out, mask, out_mask, epi, open, true, s);
+    return ok ? hipGetLastError() : hipErrorInvalidValue;
+}
 
 hipError_t launch_conv(const dc_geometry &g, const void *in, const void *filter,
                        const void *packed, const void *bias, void *out, const int32_t *mask,

@@ -378,6 +378,71 @@ int dc_densify(const void *delta, void *prev_out, void *out, const int32_t *mask
                                      (hipStream_t)stream), "dc_densify");
 }
 
+int dc_expand_depthwise(const dc_geometry *g, const dc_expand_dw_args *args, int dtype, void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_expand_depthwise");
+    int rc = check_geometry("dc_expand_depthwise", g, false, false);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_PTR("dc_expand_depthwise", args);
+    const dc_expand_dw_args &a = *args;
+    if (dtype != DC_F16 && dtype != DC_BF16)
+        return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: 16-bit types only");
+    if (a.expand_in_channels <= 0)
+        return fail(DC_ERR_SHAPE, "dc_expand_depthwise: expand_in_channels=%d must be positive", a.expand_in_channels);
+    if (a.expand_activation > DC_ACT_SWISH || a.dw_activation > DC_ACT_SWISH || a.dw_truncation_mode > DC_TRUNC_RMS)
+        return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: activation or truncation mode out of range");
+    if (a.expand_truncation_mode != DC_TRUNC_MAX)
+        return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: the expansion's truncation has to be the maximum norm");
+    // the expansion as a 1x1 convolution on the depthwise layer's input map
+    dc_geometry ge = *g;
+    ge.in_c = a.expand_in_channels;
+    ge.out_h = g->in_h; ge.out_w = g->in_w; ge.out_c = g->in_c;
+    ge.kernel_h = ge.kernel_w = 1;
+    ge.stride_h = ge.stride_w = ge.dilation_h = ge.dilation_w = 1;
+    ge.pad_top = ge.pad_left = ge.pad_bottom = ge.pad_right = 0;
+    ge.groups = 1;
+    if (!dc::pointwise_open_eligible(ge, dtype, a.expand_activation))
+        return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: the expansion needs input channels in multiples of 8, "
+                                        "output channels in multiples of 4 and ReLU or ReLU6");
+    dc::ActEpilogue dw_epi{a.dw_prev_out, a.dw_truncated, a.dw_threshold, a.dw_activation, a.dw_truncation_mode};
+    if (!dc::depthwise_closing_eligible(*g, &dw_epi, dtype))
+        return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: needs a depthwise 3x3 convolution with stride 1 and "
+                                        "padding 1 on a map small enough for the per-pixel kernel (input of at "
+                                        "most 2 MB, at most two 16-byte vectors per lane) with a truncating activation");
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.input);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.mask);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.expand_packed_filter);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.expand_prev_out);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.expand_truncated);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.expand_out);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.expand_out_mask);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.dw_filter);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.dw_prev_out);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.dw_truncated);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.out);
+    DC_REQUIRE_PTR("dc_expand_depthwise", a.out_mask);
+    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.input, 16);
+    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.expand_packed_filter, 16);
+    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.expand_prev_out, 16);
+    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.expand_truncated, 16);
+    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.expand_out, 16);
+    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.dw_filter, 16);
+    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.dw_prev_out, 16);
+    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.dw_truncated, 16);
+    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.out, 16);
+    dc::OpenAct open;
+    open.prev = a.expand_prev_out;
+    open.trunc = a.expand_truncated;
+    open.thr = a.expand_threshold;
+    open.act = a.expand_activation;
+    hipError_t e = dc::launch_pointwise_open(ge, a.input, a.expand_packed_filter, a.expand_out, a.mask,
+                                             a.expand_out_mask, open, dtype, (hipStream_t)stream);
+    if (e != hipSuccess) return finish(e, "dc_expand_depthwise");
+    return finish(dc::launch_depthwise_closing(*g, a.expand_out, a.dw_filter, a.out, a.expand_out_mask, a.out_mask,
+                                               &dw_epi, open, dtype, (hipStream_t)stream),
+                  "dc_expand_depthwise");
+}
+
 int dc_pool_densify(const dc_geometry *g, const void *input, const int32_t *mask, void *prev_out,
                     void *out, int dtype, void *stream) {
     dc::kernel_log_reset();

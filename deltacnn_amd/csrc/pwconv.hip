@@ -43,11 +43,12 @@ struct PwP {
 // the same operations, in the same order and precision, as the stand-alone add kernel.
 template <typename E>
 struct ResP {
-    const E *res;
+    const E *res;  // MODE 3: the layer's truncated values (read; T is written back through `tmp`)
     const int32_t *mask;
     float wa, wb;
-    E *prev;  // MODE 2: the sum is accumulated here and its activated difference is emitted
+    E *prev;  // MODE 2: the sum is accumulated here and its activated difference is emitted; MODE 3: read only
     int act;
+    E *tmp = nullptr;  // MODE 3: the layer's truncated values again, which receive T = truncated + v
 };
 
 // A workgroup takes 64 consecutive pixels (4 pixel tiles of 16) x CBW * R channel tiles of 16.
@@ -62,8 +63,16 @@ struct ResP {
 // fragments are then shared by R channel tiles instead of being fetched again by other
 // workgroups).  S = reduction steps per memory round trip: all fragment loads of S steps are in
 // flight together.
-// MODE: 0 convolution only, 1 fused sum, 2 fused sum with the DCAdd layer's activation.
-template <typename E, int KW, int CBW, int NBW, int R, int NTW, int S, int MODE, bool EAGER>
+// MODE: 0 convolution only, 1 fused sum, 2 fused sum with the DCAdd layer's activation,
+// 3 the layer's own activation left OPEN: with v the convolution result, T = truncated + v,
+// S = T + prev, D = act(S) - act(prev) (one rounding each, the sequence of act_trunc_pixel), the
+// kernel emits D as its output, replaces the layer's truncated values by T for every updated pixel
+// (what they have to hold if the pixel is dropped) and leaves the accumulated values alone; whether a pixel is kept -- any |D| of its channels above the threshold -- is
+// decided by the depthwise kernel that consumes D (conv_dw_kernel<FIN>), which also commits
+// the state.  A workgroup holds a slice of a pixel's channels, so it cannot decide itself.
+// ACTC >= 0: the activation of MODE 2 / 3 as a compile-time constant (a run-time id costs a chain
+// of scalar branches per element, half a microsecond in a kernel of this size); -1: rp.act.
+template <typename E, int KW, int CBW, int NBW, int R, int NTW, int S, int MODE, bool EAGER, int ACTC = -1>
 __global__ void __launch_bounds__(KW * CBW * NBW * WAVE)
 pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
                const E *__restrict__ bias, E *__restrict__ out,
@@ -71,7 +80,7 @@ pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
     typedef typename Elem16<E>::v4 E4;
     typedef typename Elem16<E>::v8 E8;
     static_assert(NBW * NTW <= 4, "a workgroup covers at most 64 pixels");
-    constexpr bool ADD = MODE > 0, ADDACT = MODE == 2;
+    constexpr bool ADD = MODE == 1 || MODE == 2, ADDACT = MODE == 2, OPEN = MODE == 3;
     constexpr int NW = KW * CBW * NBW, TILES = R * NTW, FT = (TILES + KW - 1) / KW;
     constexpr int PXW = NBW * NTW * 16;  // pixels per workgroup
     __shared__ float4_t s_red[KW > 1 ? NW * TILES * WAVE : 1];
@@ -124,15 +133,33 @@ pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
             for (int j = 0; j < NTW; ++j) x[i][j] = *reinterpret_cast<const E8 *>(xrow[j] + k);
         }
     }
+    // tiles this wavefront finishes: all of its own (KW == 1) or tiles kw, kw + KW, ... of
+    // its group after the reduction
+    E4 res[FT], bh[FT], qv[FT];
+    if (OPEN && EAGER) {  // the activation's cached state of the lane's pixels, before the masks are known
+#pragma unroll
+        for (int m = 0; m < FT; ++m) {
+            const int t = min(KW > 1 ? kw + m * KW : m, TILES - 1);
+            const int r = t / NTW, j = t % NTW;
+            const int co = min((ct0 + r) * 16 + kq * 4, p.Co - 4);
+            const size_t off = (size_t)min(pbase + (nw * NTW + j) * 16 + l16, p.P - 1) * p.Co + co;
+            res[m] = *reinterpret_cast<const E4 *>(rp.res + off);
+            qv[m] = *reinterpret_cast<const E4 *>(rp.prev + off);
+        }
+    }
     const uint64_t bm = ballot(mine && mword != 0);
     const uint64_t br = ADD ? ballot(mine && rword != 0) : 0;
     const uint64_t bo = bm | br;
     if (by == 0 && wave == 0 && mine) out_mask[mp] = int((bo >> lane) & 1);
     if (bo == 0) return;  // the same for every wavefront of the workgroup
+    if (OPEN && EAGER) {  // requested above, arrived with the mask words: not to be moved down to the epilogue
+#pragma unroll
+        for (int m = 0; m < FT; ++m) {
+            DC_PIN(res[m]);
+            DC_PIN(qv[m]);
+        }
+    }
 
-    // tiles this wavefront finishes: all of its own (KW == 1) or tiles kw, kw + KW, ... of
-    // its group after the reduction
-    E4 res[FT], bh[FT], qv[FT];
 #pragma unroll
     for (int m = 0; m < FT; ++m) {
         const int t = KW > 1 ? kw + m * KW : m;
@@ -148,6 +175,13 @@ pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
                 const bool on_o = t < TILES && ((bo >> bit) & 1);
                 qv[m] = *reinterpret_cast<const E4 *>(rp.prev + (size_t)(on_o ? pbase + bit : 0) * p.Co + co);
             }
+        }
+        if (OPEN && !EAGER) {  // cached state of the layer's activation, for updated pixels
+            const int bit = (nw * NTW + j) * 16 + l16;
+            const bool on_c = t < TILES && ((bm >> bit) & 1);
+            const size_t off = (size_t)(on_c ? pbase + bit : 0) * p.Co + co;
+            res[m] = *reinterpret_cast<const E4 *>(rp.res + off);
+            qv[m] = *reinterpret_cast<const E4 *>(rp.prev + off);
         }
     }
 
@@ -226,6 +260,7 @@ pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
     }
 
     const E wa = E(rp.wa), wb = E(rp.wb);
+    const int act = ACTC >= 0 ? ACTC : rp.act;
 #pragma unroll
     for (int m = 0; m < FT; ++m) {
         const int t = KW > 1 ? kw + m * KW : m;
@@ -246,11 +281,21 @@ pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
                 if (on) sum = fma_t(o[i], wb, sum);
                 if (ADDACT) {
                     qn[i] = sum + qv[m][i];
-                    sum = act_apply<E>(qn[i], rp.act) - act_apply<E>(qv[m][i], rp.act);
+                    sum = act_apply<E>(qn[i], act) - act_apply<E>(qv[m][i], act);
                 }
                 o[i] = sum;
             }
             if (ADDACT) *reinterpret_cast<E4 *>(rp.prev + (size_t)(pbase + bit) * p.Co + co) = qn;
+        }
+        if (OPEN) {
+            E4 tq;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                tq[i] = res[m][i] + o[i];
+                const E sm = tq[i] + qv[m][i];
+                o[i] = act_apply<E>(sm, act) - act_apply<E>(qv[m][i], act);
+            }
+            *reinterpret_cast<E4 *>(rp.tmp + (size_t)(pbase + bit) * p.Co + co) = tq;
         }
         *reinterpret_cast<E4 *>(out + (size_t)(pbase + bit) * p.Co + co) = o;
     }
@@ -854,7 +899,7 @@ template <typename E>
 hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *packed,
                               const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
                               const ActEpilogue *epi, bool *epilogue_done, const Residual *res,
-                              hipStream_t s) {
+                              hipStream_t s, const OpenAct *open = nullptr) {
     PwP p;
     p.P = g.batch * g.in_h * g.in_w;
     p.Ci = g.in_c;
@@ -869,7 +914,7 @@ hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *
     // Large maps: active-pixel gather, with the activation / truncation as its epilogue where the
     // layer has one with maximum-norm truncation.
     const auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
-    const int gct = (res == nullptr && al16(in) && al16(out) && al16(packed)) ? gather_tiles(p, ksteps) : 0;
+    const int gct = (res == nullptr && open == nullptr && al16(in) && al16(out) && al16(packed)) ? gather_tiles(p, ksteps) : 0;
     if (gct > 0 && gather_lds(p, ksteps, gct) <= (64u << 10)) {
         const bool with_act = epi != nullptr && epi->mode == DC_TRUNC_MAX && epi->trunc != nullptr && al16(epi->prev) &&
                               al16(epi->trunc);
@@ -978,6 +1023,8 @@ hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *
     }
     ResP<E> rp{nullptr, nullptr, 1.f, 1.f, nullptr, 0};
     if (res != nullptr) rp = ResP<E>{(const E *)res->values, res->mask, res->wa, res->wb, (E *)res->prev, res->act};
+    if (open != nullptr)
+        rp = ResP<E>{(const E *)open->trunc, nullptr, 1.f, 1.f, (E *)open->prev, open->act < 0 ? 0 : open->act, (E *)open->trunc};
     const int cfg = pick_config(p, ksteps);
     note_kernel("pw_mfma_kernel");
 #define DC_PW_S(KW, CBW, NBW, R, NTW, EA, SS)                                                        \
@@ -987,7 +1034,16 @@ hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *
         /* filter bytes dominate and the plain order would spread a channel group over XCDs */      \
         p.xcd = (p.nx % 8 != 0 && p.ny > 1 && (int64_t)p.ci_p * p.Co > (int64_t)p.P * p.Ci) ? 1 : 0; \
         dim3 grid(p.xcd ? p.nx * ((p.ny + 7) / 8 * 8) : p.nx, p.xcd ? 1 : p.ny);                     \
-        if (res != nullptr && res->act > 0)                                                          \
+        if (open != nullptr && open->act == DC_ACT_RELU6)                                            \
+            pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 3, EA, DC_ACT_RELU6><<<grid, KW * CBW * NBW * WAVE, 0, s>>>( \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
+        else if (open != nullptr)                                                                    \
+            pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 3, EA, DC_ACT_RELU><<<grid, KW * CBW * NBW * WAVE, 0, s>>>( \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
+        else if (res != nullptr && res->act == DC_ACT_RELU)                                          \
+            pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 2, EA, DC_ACT_RELU><<<grid, KW * CBW * NBW * WAVE, 0, s>>>( \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
+        else if (res != nullptr && res->act > 0)                                                     \
             pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 2, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
                 p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
         else if (res != nullptr)                                                                     \
@@ -1024,5 +1080,20 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     return launch_pointwise_t<half_t>(g, in, packed, bias, out, mask, out_mask, epi, epilogue_done, res, s);
 }
 
-}  // namespace dc
+// ReLU and ReLU6 (what the layers in front of depthwise convolutions use) are instantiated.
+bool pointwise_open_eligible(const dc_geometry &g, int dtype, int activation) {
+    return pointwise_eligible(g, dtype) && (activation == DC_ACT_RELU || activation == DC_ACT_RELU6);
+}
 
+// The pointwise convolution of a layer whose activation / truncation is left open (MODE 3 of
+// pw_mfma_kernel): out = D, truncated = T on updated pixels, out_mask = the update mask.
+hipError_t launch_pointwise_open(const dc_geometry &g, const void *in, const void *packed, void *out,
+                                 const int32_t *mask, int32_t *out_mask, const OpenAct &open, int dtype,
+                                 hipStream_t s) {
+    bool unused = false;
+    if (dtype == DC_BF16)
+        return launch_pointwise_t<bf16_t>(g, in, packed, nullptr, out, mask, out_mask, nullptr, &unused, nullptr, s, &open);
+    return launch_pointwise_t<half_t>(g, in, packed, nullptr, out, mask, out_mask, nullptr, &unused, nullptr, s, &open);
+}
+
+}  // namespace dc

@@ -234,6 +234,39 @@ def sparse_block(x, mask, dw_filter, dw_geometry, dw_prev_out, dw_truncated, dw_
     return True
 
 
+def sparse_expand_depthwise(x, mask, expand_packed, expand_prev_out, expand_truncated, expand_threshold,
+                            expand_activation, expand_out, expand_out_mask, dw_filter, dw_geometry, dw_prev_out,
+                            dw_truncated, dw_threshold, dw_activation, dw_truncation_mode, out, out_mask):
+    """A 1x1 expansion with activation / maximum-norm truncation followed by a depthwise 3x3
+    (stride 1, padding 1) with activation / truncation as TWO launches instead of three
+    (``dc_expand_depthwise``): the expansion leaves its keep decision to the depthwise kernel,
+    which reads whole pixel rows anyway and commits the expansion's cached state.  Layer states
+    and the depthwise output are identical, bit for bit, to the separate calls.  Returns ``False``
+    (nothing launched) for shapes without this form, so the caller can issue the separate calls."""
+    lib = _lib.load()
+    _nhwc(x, "x")
+    if x.dtype not in (torch.float16, torch.bfloat16) or expand_packed is None:
+        return False
+    a = _lib.ExpandDwArgs()
+    a.input, a.mask, a.expand_packed_filter = x.data_ptr(), _mask(mask, "mask").data_ptr(), expand_packed.data_ptr()
+    a.expand_in_channels = int(x.shape[1])
+    a.expand_prev_out, a.expand_truncated = expand_prev_out.data_ptr(), expand_truncated.data_ptr()
+    a.expand_threshold, a.expand_activation, a.expand_truncation_mode = float(expand_threshold), int(expand_activation), 0
+    a.expand_out, a.expand_out_mask = expand_out.data_ptr(), expand_out_mask.data_ptr()
+    a.dw_filter, a.dw_prev_out, a.dw_truncated = dw_filter.data_ptr(), dw_prev_out.data_ptr(), dw_truncated.data_ptr()
+    a.dw_threshold, a.dw_activation, a.dw_truncation_mode = float(dw_threshold), int(dw_activation), int(dw_truncation_mode)
+    a.out, a.out_mask = out.data_ptr(), out_mask.data_ptr()
+    meta = dict(g=dw_geometry, esize=x.element_size(), in_mask=mask, out_mask=out_mask, Ci=int(x.shape[1]),
+                keep=(a, x, expand_packed, dw_filter))
+    try:
+        _call("expand_dw", lib.dc_expand_depthwise, (dw_geometry, ctypes.byref(a), _dtype(x), _stream()), **meta)
+    except _lib.DeltaCNNError as e:
+        if e.code == -3:
+            return False
+        raise
+    return True
+
+
 def sparse_deconv(x, filter, mask=None, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
                   groups=1, c_out: int = None, create_out_mask=False, sub_tile_sparsity=True,
                   out_mask=None, out_shape=None, *, packed_filter=None, out=None, geometry=None):

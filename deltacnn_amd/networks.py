@@ -183,6 +183,8 @@ class _InvertedResidual(nn.Module):
         layers.append(_ConvBNAct(L, hidden, oup, kernel_size=1, fold_bn=fold_bn, act=None))
         self.conv = nn.Sequential(*layers)
         self.has_expansion = expand_ratio != 1
+        self._expand_depthwise = getattr(L, "expand_depthwise", None)
+        self._block_wanted = getattr(L, "fused_block_wanted", None) or (lambda *a: False)
 
     def _tail(self, x, hidden):
         """Depthwise convolution and projection (+ residual sum) of the block, layer by layer;
@@ -195,6 +197,16 @@ class _InvertedResidual(nn.Module):
             return self.sparse_add(x, self.conv[start:](hidden))
         # the layer namespace can add the residual inside the last convolution's kernel
         return fused(x, self.conv[-1][0], self.conv[start:-1](hidden))
+
+    def _project(self, x, hidden):
+        """The projection (+ residual sum) behind the depthwise layer's output ``hidden``."""
+        last = self.conv[2 if self.has_expansion else 1:]
+        if not self.use_res_connect:
+            return last(hidden)
+        fused = getattr(self.sparse_add, "after_conv", None)
+        if fused is None or len(last) != 1 or len(last[0]) != 1:
+            return self.sparse_add(x, last(hidden))
+        return fused(x, last[0][0], hidden)
 
     def forward(self, x):
         return self._tail(x, self.conv[0](x) if self.has_expansion else x)
@@ -213,6 +225,15 @@ class _InvertedResidual(nn.Module):
         launch runs the next block's expansion ahead in turn.  Returns (block output, expansion
         output of the next block or None)."""
         layers = self.single_layers()
+        if expanded is None and self.has_expansion and layers is not None and self._expand_depthwise is not None \
+                and not isinstance(x, torch.Tensor):
+            # where the block launch below would not take the block anyway: expansion and depthwise
+            # layer as two launches (the expansion's activation is finished by the depthwise kernel)
+            hidden_shape = (x[0].shape[0], layers[0].out_channels) + tuple(x[0].shape[2:])
+            if not self._block_wanted(layers[1], layers[2], next_expansion, hidden_shape, x[0].dtype):
+                hidden = self._expand_depthwise(layers[0], layers[1], x)
+                if hidden is not None:
+                    return self._project(x, hidden), None
         if expanded is None:
             expanded = self.conv[0](x) if self.has_expansion else x
         if layers is not None:

@@ -372,6 +372,7 @@ class DCConv2d(_DeltaConvBase, nn.Conv2d, DCModule):
     backend = DCBackend.deltacnn
     conv_idx = -1
     fuse_activation = True
+    fuse_expansion = True  # expand_depthwise(): 1x1 expansion + activation -> depthwise 3x3 + activation in two launches
     fuse_blocks = True  # fused_block(): depthwise -> projection (-> expansion) in one launch
     # ... while the two 1x1 filters together stay below this many bytes: every 16-pixel workgroup
     # of that launch reads both in full, and one compute unit pulls only a few GB/s out of the
@@ -546,6 +547,65 @@ def _steady_activation(conv):
     if act is None or act.first_iter or not act.inplace or act.truncation_mode != DCTruncation.max:
         return None
     return act
+
+
+def fused_block_wanted(depthwise, project, expand, hidden_shape, dtype) -> bool:
+    """The policy part of :func:`fused_block`, decidable before the block's hidden tensor exists:
+    the class switches, the layers' steady state, filter bytes and pixel count."""
+    if not DCConv2d.fuse_blocks or dtype != torch.float16:
+        return False
+    if not (_steady(depthwise) and _steady(project) and (expand is None or _steady(expand))):
+        return False
+    if _steady_activation(depthwise) is None or project.activation is not None or not _is_depthwise(depthwise):
+        return False
+    filter_bytes = 2 * project.out_channels * (project.in_channels + (expand.out_channels if expand is not None else 0))
+    if filter_bytes > DCConv2d.fuse_blocks_max_filter_bytes:
+        return False
+    g = depthwise._plan_for(hidden_shape, dtype, depthwise.weight.device)["g"]
+    return g.batch * g.out_h * g.out_w <= DCConv2d.fuse_blocks_max_pixels
+
+
+def expand_depthwise(expand, depthwise, input):
+    """``depthwise(expand(input))`` for a 1x1 expansion DCConv2d and a 3x3 stride-1 depthwise
+    DCConv2d, both with a truncating activation, as TWO launches instead of three on frames
+    after the first: the expansion's convolution leaves its keep decision to the depthwise
+    kernel (``dc_expand_depthwise``).  Returns the depthwise layer's ``(delta, mask)`` -- exactly
+    what the separate layer calls return, all layer states included -- or ``None`` when the
+    layers are not in a state or of a shape the kernels take; nothing has happened then and the
+    caller runs the layers one by one.  Switch: ``DCConv2d.fuse_expansion``."""
+    if not DCConv2d.fuse_expansion or isinstance(input, Tensor):
+        return None
+    for conv in (expand, depthwise):
+        if not (isinstance(conv, DCConv2d) and conv.backend == DCBackend.deltacnn and conv.frame_idx >= 0
+                and conv.filters_processed and not conv.dense_out):
+            return None
+    act_e, act_d = expand.activation_layer, depthwise.activation_layer
+    if (act_e is None or act_e.first_iter or not act_e.inplace or act_e.truncation_mode != DCTruncation.max
+            or act_d is None or act_d.first_iter or not act_d.inplace):
+        return None
+    if (not _is_depthwise(depthwise) or depthwise.padding4 is not None
+            or (expand.kernel_size, expand.stride, expand.padding, expand.groups) != ((1, 1), (1, 1), (0, 0), 1)):
+        return None
+    x, mask = input
+    if x.dtype not in (torch.float16, torch.bfloat16) or x.dtype != expand.weight.dtype:
+        return None
+    plan_e = expand._plan_for(x.shape, x.dtype, x.device)
+    packed = expand._packed_filter()
+    if packed is None or plan_e["out"] is None:
+        return None
+    plan_d = depthwise._plan_for(plan_e["out"].shape, x.dtype, x.device)
+    if plan_d["out"] is None:
+        return None
+    done = hk.sparse_expand_depthwise(
+        x, mask, packed, act_e.prev_out, act_e.out_truncated, DCThreshold.get(act_e), act_e.activation_int,
+        plan_e["out"], plan_e["out_mask"], depthwise.weight, plan_d["g"], act_d.prev_out, act_d.out_truncated,
+        DCThreshold.get(act_d), act_d.activation_int, act_d.truncation_mode.value, plan_d["out"], plan_d["out_mask"])
+    if not done:
+        return None
+    for conv in (expand, depthwise):
+        DCConv2d.conv_idx += 1  # what the layers' own forward calls would have counted
+        conv.frame_idx += 1
+    return plan_d["out"], plan_d["out_mask"]
 
 
 def fused_block(dw_input, depthwise, project, add=None, residual=None, expand=None):

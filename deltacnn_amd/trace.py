@@ -218,6 +218,21 @@ class Tracer:
                     flops += 2 * cp * ce * n_out
                 shape = f"dw{ch} s{g.stride_h} -> {cp} -> {ce} @{g.out_h}x{g.out_w}"
                 dens = (n_in / p_in, n_out / p_out)
+            elif op == "expand_dw":  # 1x1 expansion with its activation left open + the depthwise layer that finishes it
+                g = meta["g"]
+                ci, ch = meta["Ci"], g.in_c
+                p_px = g.batch * g.in_h * g.in_w
+                rd = p_px * m + n_in * ci * s + ci * ch * s + n_in * 2 * ch * s
+                wr = n_in * 2 * ch * s + p_px * m
+                flops = 2 * ci * ch * n_in
+                shape = f"{ci}->{ch} k1 s1 @{g.in_h}x{g.in_w} (open)"
+                dens = (n_in / p_px, n_in / p_px)
+                ms = ms / 2  # the call's two launches share its time
+                extra = {"kernel": r["kernels"][1], "call": op, "shape": f"dw{ch} k3 s1 @{g.in_h}x{g.in_w} (closing)",
+                         "ms": ms,
+                         "bytes": p_px * m + n_in * 3 * ch * s + 9 * ch * s + n_out * 2 * ch * s
+                                  + n_in * 2 * ch * s + n_out * 3 * ch * s + p_px * m,
+                         "flops": 2 * 9 * ch * n_out, "density_in": n_in / p_px, "density_out": n_out / p_px}
             elif op == "pool_densify":  # the map's updated pixels in, accumulator in and out, dense copy out
                 g = meta["g"]
                 p_in = g.batch * g.in_h * g.in_w

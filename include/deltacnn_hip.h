@@ -184,6 +184,48 @@ enum { DC_BLOCK_LATE_LOADS = 1 };
  * (sparse_layers.py:636-638). */
 int dc_block(const dc_geometry *g, const dc_block_args *block, int dtype, void *stream);
 
+/* Operands of dc_expand_depthwise beyond the depthwise geometry. */
+typedef struct dc_expand_dw_args {
+    /* A: 1x1 expansion expand_in_channels -> C (the depthwise layer's channels) + activation/truncation */
+    const void *input;              /* [B][H][W][expand_in_channels] delta */
+    const int32_t *mask;            /* its update mask */
+    const void *expand_packed_filter;
+    int32_t expand_in_channels;
+    void *expand_prev_out;          /* [P][C] activation state of the expansion, in place */
+    void *expand_truncated;
+    float expand_threshold;
+    int32_t expand_activation;
+    int32_t expand_truncation_mode; /* DC_TRUNC_MAX */
+    void *expand_out;               /* [P][C] the expansion's output delta, valid on the pixels it keeps */
+    int32_t *expand_out_mask;       /* [P] receives the UPDATE mask of the expansion's convolution (= mask) */
+    /* B: depthwise 3x3, stride 1, padding 1 (geometry argument) + activation/truncation */
+    const void *dw_filter;          /* reference depthwise layout [3][3][C] */
+    void *dw_prev_out;              /* [P][C], in place */
+    void *dw_truncated;
+    float dw_threshold;
+    int32_t dw_activation;
+    int32_t dw_truncation_mode;
+    void *out;                      /* [P][C], written where out_mask is 1 */
+    int32_t *out_mask;              /* [P], written for every pixel */
+} dc_expand_dw_args;
+
+/* A 1x1 expansion with activation / maximum-norm truncation followed by a depthwise 3x3
+ * (stride 1, padding 1) with activation / truncation, as two launches instead of three: the
+ * expansion's convolution computes T = truncated + v, S = T + prev, D = act(S) - act(prev) for
+ * every updated pixel, stores D and T, and leaves the keep decision -- any |D| of a pixel's
+ * channels above the threshold, which no workgroup of that kernel can see -- to the depthwise
+ * kernel, whose lane groups read whole pixel rows anyway: a window pixel counts only if the
+ * decision holds for it, and every group commits the expansion's state of its centre pixel.
+ * All layer states and the depthwise output are identical, bit for bit, to
+ * dc_conv_act(expansion) followed by dc_conv_act(depthwise); of the expansion's own output only
+ * the pixels it keeps are meaningful (as always), and expand_out_mask receives its convolution's
+ * update mask rather than the keep mask.  For the small maps where launches are the cost:
+ * shapes outside the range (see dc_last_error) return DC_ERR_UNSUPPORTED before any launch so
+ * that the caller can issue the separate calls.  16-bit types; no bias (a layer's bias belongs
+ * to its first frame, which takes the separate calls).  No counterpart in the reference, which
+ * launches every layer and every activation on its own (sparse_layers.py:636-638). */
+int dc_expand_depthwise(const dc_geometry *g, const dc_expand_dw_args *args, int dtype, void *stream);
+
 /* Number of bytes dc_pack_filter writes for this geometry (0 if the shape has no packed
  * form).  One-time weight relayout for the MFMA kernels, fp16 or bfloat16, un-swizzled, in fragment order
  * [Cout tile of 16][Kh][Kw][Cin step of 32][lane 0..63][8] (lane kq*16+r holds input channels

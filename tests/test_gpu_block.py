@@ -228,8 +228,9 @@ def test_mobilenet_block_fusion_keeps_every_layer_state(lib):
                 frame = cl(video[t:t + 1].half())
                 SL.DCConv2d.fuse_blocks = True
                 got = fused(frame).clone()
-                SL.DCConv2d.fuse_blocks = False
+                SL.DCConv2d.fuse_blocks = SL.DCConv2d.fuse_expansion = False
                 want = plain(frame)
+                SL.DCConv2d.fuse_expansion = True
                 assert torch.equal(got, want), f"frame {t}"
         fm, pm = dict(fused.named_modules()), dict(plain.named_modules())
         n = 0

@@ -1,0 +1,139 @@
+"""dc_expand_depthwise: a 1x1 expansion whose activation / truncation is left open by its
+convolution and finished by the depthwise 3x3 kernel that consumes it -- two launches instead of
+three.  Everything the separate calls leave behind (depthwise output and mask, both layers' cached
+states) has to come out bit for bit; the expansion's own output is meaningful on kept pixels."""
+import pytest
+import torch
+
+from util import DEV, assert_masked_equal, cl, poison, rand_mask
+
+pytestmark = pytest.mark.gpu
+
+CASES = [  # Cin, hidden channels, H, W, batch
+    (64, 384, 14, 14, 1), (96, 576, 14, 14, 1), (160, 960, 7, 7, 1), (24, 144, 28, 28, 1), (32, 192, 20, 23, 2),
+    (8, 8, 9, 11, 1), (64, 1024, 5, 6, 1), (16, 96, 56, 56, 1),
+]
+
+
+def _case(dtype, cin, ch, H, W, B, density, seed):
+    from deltacnn_amd.filter_conversion import convert_filter_out_channels_last, convert_half_filter
+    g = torch.Generator().manual_seed(seed)
+    mask = rand_mask(g, B, H, W, density)
+    x = torch.randn(B, cin, H, W, generator=g)
+    # half of the updates are far below the expansion's threshold: they get truncated
+    x = (x * torch.where(torch.rand(B, 1, H, W, generator=g) < 0.5, 1.0, 1e-3)).to(dtype)
+    we = (torch.randn(ch, cin, 1, 1, generator=g) / cin ** 0.5).to(dtype)
+    wd = (torch.randn(ch, 1, 3, 3, generator=g) / 3).to(dtype)
+    if dtype == torch.float16:
+        fe, fd = convert_half_filter(we), convert_half_filter(wd, pixel_wise=True)
+    else:
+        fe, fd = convert_filter_out_channels_last(we), convert_filter_out_channels_last(wd)
+    states = [torch.randn(B, ch, H, W, generator=g).to(dtype) * s for s in (1.0, 0.05, 1.0, 0.05)]
+    return x, mask, fe.to(DEV), fd.to(DEV), states
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["float16", "bfloat16"])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("density", [0.15, 1.0])
+@pytest.mark.parametrize("acts", [(2, 2), (1, 3)], ids=["relu6", "relu-leaky"])
+def test_expand_depthwise_equals_separate_calls(lib, dtype, case, density, acts):
+    from deltacnn_amd import _lib
+    from deltacnn_amd import hip_kernels as hk
+    cin, ch, H, W, B = case
+    x, mask, fe, fd, states = _case(dtype, cin, ch, H, W, B, density, 1700 + cin + ch)
+    pk = hk.pack_filter(fe, cin, ch, 1)
+    dx, dm = cl(poison(x, mask)), cl(mask)
+    thr_e, thr_d = 0.9, 0.3
+    # separate calls
+    pe1, te1, pd1, td1 = (cl(t) for t in states)
+    e_out, e_mask = hk.sparse_conv_activation(dx, fe, dm, None, pe1, te1, thr_e, acts[0], 0, (1, 1), (0, 0), (1, 1), 1, ch,
+                                              packed_filter=pk)
+    kept, reached = int(e_mask.sum()), int(mask.sum())
+    assert reached < 16 or 0 < kept < reached, (kept, reached)  # some kept, some truncated
+    d_out, d_mask = hk.sparse_conv_activation(e_out, fd, e_mask, None, pd1, td1, thr_d, acts[1], 0, (1, 1), (1, 1), (1, 1),
+                                              ch, ch)
+    # the two-launch form
+    pe2, te2, pd2, td2 = (cl(t) for t in states)
+    geo = hk.conv_geometry((B, ch, H, W), (3, 3), ch, (1, 1), (1, 1), (1, 1), ch)
+    nan = float("nan")
+    e2 = torch.full((B, ch, H, W), nan, dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+    out2 = torch.full_like(e2, nan)
+    em2 = torch.full((B, 1, H, W), -7, dtype=torch.int32, device=DEV)
+    om2 = torch.full_like(em2, -7)
+    assert hk.sparse_expand_depthwise(dx, dm, pk, pe2, te2, thr_e, acts[0], e2, em2, fd, geo, pd2, td2, thr_d, acts[1], 0,
+                                      out2, om2)
+    assert _lib.load().dc_last_kernels().decode() == "pw_mfma_kernel+conv_dw_kernel"
+    assert torch.equal(om2, d_mask)
+    assert_masked_equal(out2, d_out.cpu(), d_mask.cpu(), "depthwise output")
+    assert torch.equal(pe1, pe2) and torch.equal(te1, te2), "expansion state"
+    assert torch.equal(pd1, pd2) and torch.equal(td1, td2), "depthwise state"
+    assert torch.equal(em2.cpu(), mask)  # the expansion's convolution mask, not its keep mask
+    assert_masked_equal(e2, e_out.cpu(), e_mask.cpu(), "expansion output on kept pixels")
+
+
+def test_expand_depthwise_declines_what_it_cannot_do(lib):
+    """Strided depthwise layers, maps beyond the per-pixel kernel's range and fp32 have no such
+    form: False, nothing launched, nothing touched."""
+    from deltacnn_amd import hip_kernels as hk
+    dtype = torch.float16
+    for (cin, ch, H, W, B, stride, dt) in [(64, 384, 14, 14, 1, 2, dtype), (32, 192, 112, 112, 2, 1, dtype),
+                                           (64, 384, 14, 14, 1, 1, torch.float32)]:
+        x, mask, fe, fd, states = _case(dtype, cin, ch, H, W, B, 0.5, 1800 + H)
+        pk = hk.pack_filter(fe, cin, ch, 1)
+        Ho, Wo = (H - 1) // stride + 1, (W - 1) // stride + 1
+        geo = hk.conv_geometry((B, ch, H, W), (3, 3), ch, (stride, stride), (1, 1), (1, 1), ch)
+        pe, te = cl(states[0]), cl(states[1])
+        pd = cl(states[2][:, :, :Ho, :Wo].contiguous())
+        td = cl(states[3][:, :, :Ho, :Wo].contiguous())
+        before = [t.clone() for t in (pe, te, pd, td)]
+        e = torch.zeros(B, ch, H, W, dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+        out = torch.zeros(B, ch, Ho, Wo, dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+        em = torch.zeros(B, 1, H, W, dtype=torch.int32, device=DEV)
+        om = torch.zeros(B, 1, Ho, Wo, dtype=torch.int32, device=DEV)
+        dx = cl(x).to(dt) if dt != dtype else cl(x)
+        assert hk.sparse_expand_depthwise(dx, cl(mask), pk, pe, te, 0.5, 2, e, em, fd, geo, pd, td, 0.5, 2, 0, out, om) is False
+        assert all(torch.equal(a, b) for a, b in zip(before, (pe, te, pd, td)))
+        assert not bool(out.any()) and not bool(e.any())
+
+
+def test_mobilenet_open_expansions_keep_every_layer_state(lib):
+    """MobileNetV2 224x224, 6 frames: the model whose expansions leave their activation to the
+    depthwise kernels against the model that issues every layer call on its own -- logits and
+    every activation layer's cached state equal bit for bit; nine blocks of every frame after
+    the first take the two-launch form (the 14x14 and 7x7 blocks with a stride-1 depthwise layer)."""
+    from deltacnn_amd import hip_kernels as hk
+    from deltacnn_amd import sparse_layers as SL
+    from deltacnn_amd.video import moving_rectangles_video
+    from test_gpu_network import _calibrated_state, _mobilenet, _two_hip_models
+    video = moving_rectangles_video(frames=6, height=224, width=224, n_rect=3, min_size=16, max_size=60)
+    small = moving_rectangles_video(frames=3, height=64, width=96, n_rect=2, min_size=8, max_size=24)
+    fused, plain = _two_hip_models(_mobilenet, _calibrated_state(small))
+    launches = []
+    original = hk.sparse_expand_depthwise
+
+    def counted(*a, **k):
+        done = original(*a, **k)
+        launches.append(done)
+        return done
+    hk.sparse_expand_depthwise = counted
+    try:
+        with torch.no_grad():
+            for t in range(video.shape[0]):
+                frame = cl(video[t:t + 1].half())
+                SL.DCConv2d.fuse_expansion = SL.DCConv2d.fuse_blocks = True
+                got = fused(frame).clone()
+                SL.DCConv2d.fuse_expansion = SL.DCConv2d.fuse_blocks = False
+                want = plain(frame)
+                assert torch.equal(got, want), f"frame {t}"
+        fm, pm = dict(fused.named_modules()), dict(plain.named_modules())
+        n = 0
+        for name, mod in fm.items():
+            if isinstance(mod, SL.DCActivation):
+                assert torch.equal(mod.prev_out, pm[name].prev_out), name
+                assert torch.equal(mod.out_truncated, pm[name].out_truncated), name
+                n += 1
+        assert n == 35
+        assert sum(launches) == 9 * (video.shape[0] - 1), (len(launches), sum(launches))
+    finally:
+        SL.DCConv2d.fuse_expansion = SL.DCConv2d.fuse_blocks = True
+        hk.sparse_expand_depthwise = original

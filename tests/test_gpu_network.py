@@ -385,13 +385,13 @@ def test_fused_layer_calls_change_nothing(lib, network, size):
             for t in range(video.shape[0]):
                 frame = cl(video[t:t + 1].half())
                 SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = SL.DCConv2d.fuse_blocks = True
-                SL.DCDensify.fuse_pooling = True
+                SL.DCDensify.fuse_pooling = SL.DCConv2d.fuse_expansion = True
                 got = fused(frame)
                 got = {k: v.clone() for k, v in got.items()} if isinstance(got, dict) else got.clone()
                 SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = SL.DCConv2d.fuse_blocks = False
-                SL.DCDensify.fuse_pooling = False
+                SL.DCDensify.fuse_pooling = SL.DCConv2d.fuse_expansion = False
                 want = plain(frame)
                 assert _same(got, want), f"frame {t}"
     finally:
         SL.DCConv2d.fuse_activation = SL.DCAdd.fuse_into_conv = SL.DCConv2d.fuse_blocks = True
-        SL.DCDensify.fuse_pooling = True
+        SL.DCDensify.fuse_pooling = SL.DCConv2d.fuse_expansion = True

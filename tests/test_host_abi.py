@@ -261,3 +261,41 @@ def test_head_entry_points_check_their_arguments(lib):
     assert linear(fi=36) == -3 and b"16-byte" in lib.dc_last_error()     # 36 halves
     assert linear(x=None) == -4 and linear(w=None) == -4 and linear(out=None) == -4
     assert linear(x=p + 8) == -5 and linear(w=p + 2) == -5 and linear(out=p + 1) == -5
+
+
+def test_expand_depthwise_arguments_are_checked_before_any_launch(lib):
+    """dc_expand_depthwise: shapes without the two-launch form -> -3 (the caller issues the
+    separate calls), missing operands -> -4, misaligned pointers -> -5; nothing touches a device."""
+    from deltacnn_amd._lib import ExpandDwArgs
+    buf = (ctypes.c_char * 8192)()
+    p = (ctypes.addressof(buf) + 255) // 256 * 256
+    g = _geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=384, out_c=384, groups=384)
+
+    def args(**kw):
+        a = ExpandDwArgs()
+        for name in ("input", "mask", "expand_packed_filter", "expand_prev_out", "expand_truncated", "expand_out",
+                     "expand_out_mask", "dw_filter", "dw_prev_out", "dw_truncated", "out", "out_mask"):
+            setattr(a, name, p)
+        a.expand_in_channels, a.expand_threshold, a.expand_activation, a.expand_truncation_mode = 64, 0.05, 2, 0
+        a.dw_threshold, a.dw_activation, a.dw_truncation_mode = 0.05, 2, 0
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+
+    def call(geom, a, dtype=1):
+        return lib.dc_expand_depthwise(ctypes.byref(geom), ctypes.byref(a), dtype, None)
+
+    assert call(g, args(), dtype=0) == -3 and b"16-bit" in lib.dc_last_error()
+    assert call(g, args(), dtype=9) == -1
+    assert call(g, args(expand_in_channels=0)) == -2
+    assert call(g, args(expand_in_channels=20)) == -3                      # not a multiple of 8
+    assert call(g, args(expand_truncation_mode=1)) == -3                   # norm truncation of the expansion
+    assert call(g, args(dw_truncation_mode=-1)) == -3                      # a depthwise layer without truncation
+    assert call(_geom(in_h=14, in_w=14, out_h=7, out_w=7, in_c=384, out_c=384, groups=384, stride_h=2, stride_w=2),
+                args()) == -3                                              # strided
+    assert call(_geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=384, out_c=384, groups=1), args()) == -3  # not depthwise
+    assert call(_geom(in_h=224, in_w=224, out_h=224, out_w=224, in_c=96, out_c=96, groups=96), args()) == -3  # too large
+    assert lib.dc_expand_depthwise(None, ctypes.byref(args()), 1, None) == -4
+    assert lib.dc_expand_depthwise(ctypes.byref(g), None, 1, None) == -4
+    assert call(g, args(out=None)) == -4 and call(g, args(expand_truncated=None)) == -4
+    assert call(g, args(input=p + 2)) == -5 and call(g, args(dw_prev_out=p + 8)) == -5
