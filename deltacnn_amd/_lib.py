@@ -52,6 +52,18 @@ class ExpandDwArgs(ctypes.Structure):
         ("out", c_void_p), ("out_mask", c_void_p)]
 
 
+class ProjectExpandArgs(ctypes.Structure):
+    """struct dc_project_expand_args."""
+    _fields_ = [
+        ("input", c_void_p), ("mask", c_void_p), ("project_packed_filter", c_void_p),
+        ("residual", c_void_p), ("residual_mask", c_void_p), ("weight_residual", c_float), ("weight_conv", c_float),
+        ("out", c_void_p), ("out_mask", c_void_p),
+        ("expand_packed_filter", c_void_p), ("expand_channels", c_int32), ("expand_prev_out", c_void_p),
+        ("expand_truncated", c_void_p), ("expand_activation", c_int32), ("expand_out", c_void_p),
+        ("expand_out_mask", c_void_p),
+        ("dw_geometry", POINTER(Geometry)), ("dw_activation", c_int32), ("dw_truncation_mode", c_int32)]
+
+
 _P = c_void_p
 _G = POINTER(Geometry)
 _SIGNATURES = {
@@ -65,6 +77,7 @@ _SIGNATURES = {
     "dc_conv_add": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, _P, c_float, c_float, _P, c_int, c_int, _P]),
     "dc_block": (c_int, [_G, POINTER(BlockArgs), c_int, _P]),
     "dc_expand_depthwise": (c_int, [_G, POINTER(ExpandDwArgs), c_int, _P]),
+    "dc_project_expand": (c_int, [_G, POINTER(ProjectExpandArgs), c_int, _P]),
     "dc_packed_filter_bytes": (c_int64, [_G, c_int, c_int]),
     "dc_pack_filter": (c_int, [_G, _P, _P, c_int, c_int, _P]),
     "dc_deconv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),

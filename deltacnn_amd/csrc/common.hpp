@@ -313,6 +313,12 @@ bool pointwise_open_eligible(const dc_geometry &g, int dtype, int activation);
 hipError_t launch_pointwise_open(const dc_geometry &g, const void *in, const void *packed, void *out,
                                  const int32_t *mask, int32_t *out_mask, const OpenAct &open, int dtype,
                                  hipStream_t s);
+// Projection (+ residual sum) and the next 1x1 expansion with its activation left open, one launch.
+bool pointwise_pair_eligible(const dc_geometry &gp, int expand_channels, int activation, int dtype);
+hipError_t launch_pointwise_pair(const dc_geometry &gp, const void *in, const int32_t *mask,
+                                 const void *project_packed, const Residual *res, void *out, int32_t *out_mask,
+                                 const void *expand_packed, int expand_channels, const OpenAct &open,
+                                 void *expand_out, int32_t *expand_out_mask, int dtype, hipStream_t s);
 bool pointwise_eligible(const dc_geometry &g, int dtype);
 bool patch_eligible(const dc_geometry &g, int dtype);
 bool lds_add_eligible(const dc_geometry &g, int dtype, int activation);

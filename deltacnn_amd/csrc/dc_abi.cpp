@@ -401,7 +401,8 @@ int dc_expand_depthwise(const dc_geometry *g, const dc_expand_dw_args *args, int
     ge.stride_h = ge.stride_w = ge.dilation_h = ge.dilation_w = 1;
     ge.pad_top = ge.pad_left = ge.pad_bottom = ge.pad_right = 0;
     ge.groups = 1;
-    if (!dc::pointwise_open_eligible(ge, dtype, a.expand_activation))
+    const bool opened = a.expand_packed_filter == nullptr;  // dc_project_expand ran the convolution
+    if (!opened && !dc::pointwise_open_eligible(ge, dtype, a.expand_activation))
         return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: the expansion needs input channels in multiples of 8, "
                                         "output channels in multiples of 4 and ReLU or ReLU6");
     dc::ActEpilogue dw_epi{a.dw_prev_out, a.dw_truncated, a.dw_threshold, a.dw_activation, a.dw_truncation_mode};
@@ -409,9 +410,12 @@ int dc_expand_depthwise(const dc_geometry *g, const dc_expand_dw_args *args, int
         return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: needs a depthwise 3x3 convolution with stride 1 and "
                                         "padding 1 on a map small enough for the per-pixel kernel (input of at "
                                         "most 2 MB, at most two 16-byte vectors per lane) with a truncating activation");
-    DC_REQUIRE_PTR("dc_expand_depthwise", a.input);
-    DC_REQUIRE_PTR("dc_expand_depthwise", a.mask);
-    DC_REQUIRE_PTR("dc_expand_depthwise", a.expand_packed_filter);
+    if (!opened) {
+        DC_REQUIRE_PTR("dc_expand_depthwise", a.input);
+        DC_REQUIRE_PTR("dc_expand_depthwise", a.mask);
+        DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.input, 16);
+        DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.expand_packed_filter, 16);
+    }
     DC_REQUIRE_PTR("dc_expand_depthwise", a.expand_prev_out);
     DC_REQUIRE_PTR("dc_expand_depthwise", a.expand_truncated);
     DC_REQUIRE_PTR("dc_expand_depthwise", a.expand_out);
@@ -421,8 +425,6 @@ int dc_expand_depthwise(const dc_geometry *g, const dc_expand_dw_args *args, int
     DC_REQUIRE_PTR("dc_expand_depthwise", a.dw_truncated);
     DC_REQUIRE_PTR("dc_expand_depthwise", a.out);
     DC_REQUIRE_PTR("dc_expand_depthwise", a.out_mask);
-    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.input, 16);
-    DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.expand_packed_filter, 16);
     DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.expand_prev_out, 16);
     DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.expand_truncated, 16);
     DC_REQUIRE_ALIGNED("dc_expand_depthwise", a.expand_out, 16);
@@ -435,12 +437,75 @@ int dc_expand_depthwise(const dc_geometry *g, const dc_expand_dw_args *args, int
     open.trunc = a.expand_truncated;
     open.thr = a.expand_threshold;
     open.act = a.expand_activation;
-    hipError_t e = dc::launch_pointwise_open(ge, a.input, a.expand_packed_filter, a.expand_out, a.mask,
-                                             a.expand_out_mask, open, dtype, (hipStream_t)stream);
-    if (e != hipSuccess) return finish(e, "dc_expand_depthwise");
+    if (!opened) {
+        hipError_t e = dc::launch_pointwise_open(ge, a.input, a.expand_packed_filter, a.expand_out, a.mask,
+                                                 a.expand_out_mask, open, dtype, (hipStream_t)stream);
+        if (e != hipSuccess) return finish(e, "dc_expand_depthwise");
+    }
     return finish(dc::launch_depthwise_closing(*g, a.expand_out, a.dw_filter, a.out, a.expand_out_mask, a.out_mask,
                                                &dw_epi, open, dtype, (hipStream_t)stream),
                   "dc_expand_depthwise");
+}
+
+int dc_project_expand(const dc_geometry *g, const dc_project_expand_args *args, int dtype, void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_project_expand");
+    int rc = check_geometry("dc_project_expand", g, false, false);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_PTR("dc_project_expand", args);
+    const dc_project_expand_args &a = *args;
+    if (dtype != DC_F16 && dtype != DC_BF16)
+        return fail(DC_ERR_UNSUPPORTED, "dc_project_expand: 16-bit types only");
+    if (a.expand_channels <= 0)
+        return fail(DC_ERR_SHAPE, "dc_project_expand: expand_channels=%d must be positive", a.expand_channels);
+    if (a.expand_activation > DC_ACT_SWISH || a.dw_activation > DC_ACT_SWISH || a.dw_truncation_mode > DC_TRUNC_RMS)
+        return fail(DC_ERR_UNSUPPORTED, "dc_project_expand: activation or truncation mode out of range");
+    if (!dc::pointwise_pair_eligible(*g, a.expand_channels, a.expand_activation, dtype))
+        return fail(DC_ERR_UNSUPPORTED, "dc_project_expand: needs 1x1 layers with block output channels in multiples "
+                                        "of 32 up to 96, a projection filter of at most 128 KB, ReLU or ReLU6 and a "
+                                        "map small enough for the reduction-slice form of the projection");
+    DC_REQUIRE_PTR("dc_project_expand", a.dw_geometry);
+    rc = check_geometry("dc_project_expand", a.dw_geometry, false, false);
+    if (rc != DC_OK) return rc;
+    const dc_geometry &gd = *a.dw_geometry;
+    if (gd.batch != g->batch || gd.in_h != g->out_h || gd.in_w != g->out_w || gd.in_c != a.expand_channels)
+        return fail(DC_ERR_SHAPE, "dc_project_expand: dw_geometry does not describe a layer on the expansion's output");
+    DC_REQUIRE_PTR("dc_project_expand", a.input);
+    DC_REQUIRE_PTR("dc_project_expand", a.mask);
+    DC_REQUIRE_PTR("dc_project_expand", a.project_packed_filter);
+    DC_REQUIRE_PTR("dc_project_expand", a.out);
+    DC_REQUIRE_PTR("dc_project_expand", a.out_mask);
+    if (a.residual != nullptr) DC_REQUIRE_PTR("dc_project_expand", a.residual_mask);
+    DC_REQUIRE_PTR("dc_project_expand", a.expand_packed_filter);
+    DC_REQUIRE_PTR("dc_project_expand", a.expand_prev_out);
+    DC_REQUIRE_PTR("dc_project_expand", a.expand_truncated);
+    DC_REQUIRE_PTR("dc_project_expand", a.expand_out);
+    DC_REQUIRE_PTR("dc_project_expand", a.expand_out_mask);
+    DC_REQUIRE_ALIGNED("dc_project_expand", a.input, 16);
+    DC_REQUIRE_ALIGNED("dc_project_expand", a.project_packed_filter, 16);
+    DC_REQUIRE_ALIGNED("dc_project_expand", a.residual, 16);
+    DC_REQUIRE_ALIGNED("dc_project_expand", a.out, 16);
+    DC_REQUIRE_ALIGNED("dc_project_expand", a.expand_packed_filter, 16);
+    DC_REQUIRE_ALIGNED("dc_project_expand", a.expand_prev_out, 16);
+    DC_REQUIRE_ALIGNED("dc_project_expand", a.expand_truncated, 16);
+    DC_REQUIRE_ALIGNED("dc_project_expand", a.expand_out, 16);
+    {
+        // the state pointers do not enter the decision; placeholders that pass its alignment tests
+        dc::ActEpilogue probe{a.expand_prev_out, a.expand_truncated, 0.f, a.dw_activation, a.dw_truncation_mode};
+        if (!dc::depthwise_closing_eligible(gd, &probe, dtype))
+            return fail(DC_ERR_UNSUPPORTED, "dc_project_expand: the depthwise layer behind the expansion cannot finish "
+                                            "its activation (needs 3x3, stride 1, padding 1 on a small map)");
+    }
+    dc::Residual res{a.residual, a.residual_mask, a.weight_residual, a.weight_conv};
+    dc::OpenAct open;
+    open.prev = a.expand_prev_out;
+    open.trunc = a.expand_truncated;
+    open.act = a.expand_activation;
+    return finish(dc::launch_pointwise_pair(*g, a.input, a.mask, a.project_packed_filter,
+                                            a.residual != nullptr ? &res : nullptr, a.out, a.out_mask,
+                                            a.expand_packed_filter, a.expand_channels, open, a.expand_out,
+                                            a.expand_out_mask, dtype, (hipStream_t)stream),
+                  "dc_project_expand");
 }
 
 int dc_pool_densify(const dc_geometry *g, const void *input, const int32_t *mask, void *prev_out,

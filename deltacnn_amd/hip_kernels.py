@@ -236,19 +236,28 @@ def sparse_block(x, mask, dw_filter, dw_geometry, dw_prev_out, dw_truncated, dw_
 
 def sparse_expand_depthwise(x, mask, expand_packed, expand_prev_out, expand_truncated, expand_threshold,
                             expand_activation, expand_out, expand_out_mask, dw_filter, dw_geometry, dw_prev_out,
-                            dw_truncated, dw_threshold, dw_activation, dw_truncation_mode, out, out_mask):
+                            dw_truncated, dw_threshold, dw_activation, dw_truncation_mode, out, out_mask,
+                            opened: bool = False):
     """A 1x1 expansion with activation / maximum-norm truncation followed by a depthwise 3x3
     (stride 1, padding 1) with activation / truncation as TWO launches instead of three
     (``dc_expand_depthwise``): the expansion leaves its keep decision to the depthwise kernel,
     which reads whole pixel rows anyway and commits the expansion's cached state.  Layer states
     and the depthwise output are identical, bit for bit, to the separate calls.  Returns ``False``
-    (nothing launched) for shapes without this form, so the caller can issue the separate calls."""
+    (nothing launched) for shapes without this form, so the caller can issue the separate calls.
+
+    ``opened``: :func:`sparse_project_expand` has already run the expansion's convolution into
+    ``expand_out`` / ``expand_truncated`` / ``expand_out_mask``; only the depthwise launch runs
+    (``x`` is then the expansion's INPUT shape donor only and ``mask``, ``expand_packed`` are unused)."""
     lib = _lib.load()
     _nhwc(x, "x")
-    if x.dtype not in (torch.float16, torch.bfloat16) or expand_packed is None:
+    if x.dtype not in (torch.float16, torch.bfloat16) or (expand_packed is None and not opened):
         return False
     a = _lib.ExpandDwArgs()
-    a.input, a.mask, a.expand_packed_filter = x.data_ptr(), _mask(mask, "mask").data_ptr(), expand_packed.data_ptr()
+    if opened:
+        a.input, a.mask, a.expand_packed_filter = None, None, None
+        mask = expand_out_mask
+    else:
+        a.input, a.mask, a.expand_packed_filter = x.data_ptr(), _mask(mask, "mask").data_ptr(), expand_packed.data_ptr()
     a.expand_in_channels = int(x.shape[1])
     a.expand_prev_out, a.expand_truncated = expand_prev_out.data_ptr(), expand_truncated.data_ptr()
     a.expand_threshold, a.expand_activation, a.expand_truncation_mode = float(expand_threshold), int(expand_activation), 0
@@ -257,9 +266,46 @@ def sparse_expand_depthwise(x, mask, expand_packed, expand_prev_out, expand_trun
     a.dw_threshold, a.dw_activation, a.dw_truncation_mode = float(dw_threshold), int(dw_activation), int(dw_truncation_mode)
     a.out, a.out_mask = out.data_ptr(), out_mask.data_ptr()
     meta = dict(g=dw_geometry, esize=x.element_size(), in_mask=mask, out_mask=out_mask, Ci=int(x.shape[1]),
-                keep=(a, x, expand_packed, dw_filter))
+                opened=opened, keep=(a, x, expand_packed, dw_filter))
     try:
         _call("expand_dw", lib.dc_expand_depthwise, (dw_geometry, ctypes.byref(a), _dtype(x), _stream()), **meta)
+    except _lib.DeltaCNNError as e:
+        if e.code == -3:
+            return False
+        raise
+    return True
+
+
+def sparse_project_expand(x, mask, project_packed, project_geometry, residual, residual_mask, out, out_mask,
+                          expand_packed, expand_prev_out, expand_truncated, expand_activation, expand_out,
+                          expand_out_mask, dw_geometry, dw_activation, dw_truncation_mode,
+                          weight_residual: float = 1.0, weight_conv: float = 1.0):
+    """The 1x1 projection that ends an inverted-residual block (+ the block's residual sum) and the
+    next block's 1x1 expansion in ONE launch (``dc_project_expand``).  The expansion's activation is
+    left open: the next call on its buffers has to be :func:`sparse_expand_depthwise` with
+    ``opened=True``, which this call has verified to be accepted for ``dw_geometry``.  Together
+    the two are identical, bit for bit, to the separate layer calls.  Returns ``False`` (nothing
+    launched) for shapes without this form."""
+    lib = _lib.load()
+    _nhwc(x, "x")
+    if x.dtype not in (torch.float16, torch.bfloat16) or project_packed is None or expand_packed is None:
+        return False
+    a = _lib.ProjectExpandArgs()
+    a.input, a.mask, a.project_packed_filter = x.data_ptr(), _mask(mask, "mask").data_ptr(), project_packed.data_ptr()
+    if residual is not None:
+        a.residual, a.residual_mask = _nhwc(residual, "residual").data_ptr(), _mask(residual_mask, "residual_mask").data_ptr()
+    a.weight_residual, a.weight_conv = float(weight_residual), float(weight_conv)
+    a.out, a.out_mask = out.data_ptr(), out_mask.data_ptr()
+    a.expand_packed_filter, a.expand_channels = expand_packed.data_ptr(), int(expand_out.shape[1])
+    a.expand_prev_out, a.expand_truncated = expand_prev_out.data_ptr(), expand_truncated.data_ptr()
+    a.expand_activation = int(expand_activation)
+    a.expand_out, a.expand_out_mask = expand_out.data_ptr(), expand_out_mask.data_ptr()
+    a.dw_geometry = ctypes.pointer(dw_geometry)
+    a.dw_activation, a.dw_truncation_mode = int(dw_activation), int(dw_truncation_mode)
+    meta = dict(g=project_geometry, esize=x.element_size(), in_mask=mask, in_mask_b=residual_mask, out_mask=out_mask,
+                Ce=int(expand_out.shape[1]), keep=(a, x, project_packed, expand_packed, residual, dw_geometry))
+    try:
+        _call("project_expand", lib.dc_project_expand, (project_geometry, ctypes.byref(a), _dtype(x), _stream()), **meta)
     except _lib.DeltaCNNError as e:
         if e.code == -3:
             return False

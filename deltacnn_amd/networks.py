@@ -185,6 +185,7 @@ class _InvertedResidual(nn.Module):
         self.has_expansion = expand_ratio != 1
         self._expand_depthwise = getattr(L, "expand_depthwise", None)
         self._block_wanted = getattr(L, "fused_block_wanted", None) or (lambda *a: False)
+        self._project_expand = getattr(L, "project_expand", None)
 
     def _tail(self, x, hidden):
         """Depthwise convolution and projection (+ residual sum) of the block, layer by layer;
@@ -219,29 +220,45 @@ class _InvertedResidual(nn.Module):
         convs = [seq[0] for seq in self.conv]
         return ([None] + convs) if not self.has_expansion else convs
 
-    def forward_ahead(self, x, expanded, fused_block, next_expansion):
-        """The block when a layer namespace offers ``fused_block``: ``expanded`` is this block's
-        expansion output if the previous block's launch already produced it; the block's own
-        launch runs the next block's expansion ahead in turn.  Returns (block output, expansion
-        output of the next block or None)."""
+    def forward_ahead(self, x, expanded, fused_block, next_layers):
+        """The block when a layer namespace offers fused forms.  ``expanded`` is this block's
+        expansion output if the previous block's launch already produced it (an ``OpenExpansion``
+        if its activation still has to be finished by this block's depthwise layer);
+        ``next_layers`` = (expansion, depthwise) of the next block, or (final 1x1 convolution,
+        None), or None.  The block's own last launch runs the next block's expansion ahead in
+        turn where a form for that exists.  Returns (block output, expansion output of the next
+        block or None)."""
         layers = self.single_layers()
-        if expanded is None and self.has_expansion and layers is not None and self._expand_depthwise is not None \
-                and not isinstance(x, torch.Tensor):
+        next_expansion = next_layers[0] if next_layers is not None else None
+        opened = expanded is not None and not isinstance(expanded, (tuple, torch.Tensor))
+        hidden = None
+        if opened:
+            hidden = self._expand_depthwise(layers[0], layers[1], x, opened=expanded)
+        elif (expanded is None and self.has_expansion and layers is not None and self._expand_depthwise is not None
+                and not isinstance(x, torch.Tensor)):
             # where the block launch below would not take the block anyway: expansion and depthwise
             # layer as two launches (the expansion's activation is finished by the depthwise kernel)
             hidden_shape = (x[0].shape[0], layers[0].out_channels) + tuple(x[0].shape[2:])
             if not self._block_wanted(layers[1], layers[2], next_expansion, hidden_shape, x[0].dtype):
                 hidden = self._expand_depthwise(layers[0], layers[1], x)
-                if hidden is not None:
-                    return self._project(x, hidden), None
-        if expanded is None:
-            expanded = self.conv[0](x) if self.has_expansion else x
-        if layers is not None:
+        if hidden is None:
+            if expanded is None:
+                expanded = self.conv[0](x) if self.has_expansion else x
+            if layers is not None:
+                add = self.sparse_add if self.use_res_connect else None
+                done = fused_block(expanded, layers[1], layers[2], add, x if add is not None else None, next_expansion)
+                if done is not None:
+                    return done
+            hidden = self.conv[1 if self.has_expansion else 0](expanded)
+        if (layers is not None and self._project_expand is not None and next_layers is not None
+                and next_layers[1] is not None and not isinstance(hidden, torch.Tensor)):
+            # projection (+ residual sum) and the next block's expansion in one launch
             add = self.sparse_add if self.use_res_connect else None
-            done = fused_block(expanded, layers[1], layers[2], add, x if add is not None else None, next_expansion)
+            done = self._project_expand(layers[2], add, x if add is not None else None, next_layers[0],
+                                        next_layers[1], hidden)
             if done is not None:
                 return done
-        return self._tail(x, expanded), None
+        return self._project(x, hidden), None
 
 
 MOBILENET_V2_SETTING = [  # t, c, n, s  (example/mobilenet_deltacnn.py:160-170)
@@ -300,9 +317,9 @@ class MobileNetV2(_Net):
             nxt = stages[i + 1]
             if isinstance(nxt, _InvertedResidual):
                 layers = nxt.single_layers()
-                ahead = layers[0] if layers is not None else None
+                ahead = (layers[0], layers[1]) if layers is not None and layers[0] is not None else None
             else:  # the final 1x1 convolution
-                ahead = nxt[0] if len(nxt) == 1 and self.fuse_head else None
+                ahead = (nxt[0], None) if len(nxt) == 1 and self.fuse_head else None
             x, expanded = stages[i].forward_ahead(x, expanded, fused_block, ahead)
         return expanded if expanded is not None else stages[-1](x)
 

@@ -373,6 +373,7 @@ class DCConv2d(_DeltaConvBase, nn.Conv2d, DCModule):
     conv_idx = -1
     fuse_activation = True
     fuse_expansion = True  # expand_depthwise(): 1x1 expansion + activation -> depthwise 3x3 + activation in two launches
+    fuse_projection = True  # project_expand(): projection (+ residual sum) + next expansion (left open) in one launch
     fuse_blocks = True  # fused_block(): depthwise -> projection (-> expansion) in one launch
     # ... while the two 1x1 filters together stay below this many bytes: every 16-pixel workgroup
     # of that launch reads both in full, and one compute unit pulls only a few GB/s out of the
@@ -565,16 +566,17 @@ def fused_block_wanted(depthwise, project, expand, hidden_shape, dtype) -> bool:
     return g.batch * g.out_h * g.out_w <= DCConv2d.fuse_blocks_max_pixels
 
 
-def expand_depthwise(expand, depthwise, input):
-    """``depthwise(expand(input))`` for a 1x1 expansion DCConv2d and a 3x3 stride-1 depthwise
-    DCConv2d, both with a truncating activation, as TWO launches instead of three on frames
-    after the first: the expansion's convolution leaves its keep decision to the depthwise
-    kernel (``dc_expand_depthwise``).  Returns the depthwise layer's ``(delta, mask)`` -- exactly
-    what the separate layer calls return, all layer states included -- or ``None`` when the
-    layers are not in a state or of a shape the kernels take; nothing has happened then and the
-    caller runs the layers one by one.  Switch: ``DCConv2d.fuse_expansion``."""
-    if not DCConv2d.fuse_expansion or isinstance(input, Tensor):
-        return None
+class OpenExpansion:
+    """What :func:`project_expand` hands to the next block in place of its expansion's output: the
+    expansion's convolution has run with its activation left open, and :func:`expand_depthwise`
+    has to finish it (``opened=`` this object) before anything else touches the two layers."""
+
+    def __init__(self, expand, depthwise):
+        self.expand, self.depthwise = expand, depthwise
+
+
+def _closing_pair(expand, depthwise, dtype):
+    """The conditions of :func:`expand_depthwise` on the two layers themselves."""
     for conv in (expand, depthwise):
         if not (isinstance(conv, DCConv2d) and conv.backend == DCBackend.deltacnn and conv.frame_idx >= 0
                 and conv.filters_processed and not conv.dense_out):
@@ -586,9 +588,89 @@ def expand_depthwise(expand, depthwise, input):
     if (not _is_depthwise(depthwise) or depthwise.padding4 is not None
             or (expand.kernel_size, expand.stride, expand.padding, expand.groups) != ((1, 1), (1, 1), (0, 0), 1)):
         return None
-    x, mask = input
-    if x.dtype not in (torch.float16, torch.bfloat16) or x.dtype != expand.weight.dtype:
+    if dtype not in (torch.float16, torch.bfloat16) or dtype != expand.weight.dtype:
         return None
+    return act_e, act_d
+
+
+def project_expand(project, add, residual, expand, depthwise, input):
+    """``add(residual, project(input))`` (``add`` / ``residual`` may be None) and the convolution of
+    the NEXT block's 1x1 expansion ``expand`` in one launch (``dc_project_expand``), on frames after
+    the first.  The expansion's activation is left open; ``depthwise`` is the layer behind it, which
+    finishes it.  Returns ``(block_output, opened)`` -- the block's ``(delta, mask)`` exactly as
+    the separate layer calls return it, and an :class:`OpenExpansion` that MUST be the next thing
+    handed to :func:`expand_depthwise` -- or ``None`` when the layers are not in a state or of a
+    shape the kernel takes; nothing has happened then.  Switch: ``DCConv2d.fuse_projection``."""
+    if not (DCConv2d.fuse_projection and DCConv2d.fuse_expansion) or isinstance(input, Tensor):
+        return None
+    x, mask = input
+    acts = _closing_pair(expand, depthwise, x.dtype)
+    if acts is None:
+        return None
+    act_e, act_d = acts
+    if not (isinstance(project, DCConv2d) and project.backend == DCBackend.deltacnn and project.frame_idx >= 0
+            and project.filters_processed and not project.dense_out and project.activation is None
+            and project.weight.dtype == x.dtype
+            and (project.kernel_size, project.stride, project.padding, project.groups) == ((1, 1), (1, 1), (0, 0), 1)):
+        return None
+    if add is not None and (not DCAdd.fuse_into_conv or add.first_iter or add.dense_out or add.activation is not None
+                            or residual is None or isinstance(residual, Tensor)):
+        return None
+    plan_p = project._plan_for(x.shape, x.dtype, x.device)
+    packed_p, packed_e = project._packed_filter(), expand._packed_filter()
+    if packed_p is None or packed_e is None or plan_p["out"] is None:
+        return None
+    plan_e = expand._plan_for(plan_p["out"].shape, x.dtype, x.device)
+    if plan_e["out"] is None:
+        return None
+    plan_d = depthwise._plan_for(plan_e["out"].shape, x.dtype, x.device)
+    out, out_mask = plan_p["out"], plan_p["out_mask"]
+    res_v = res_m = None
+    wa = wb = 1.0
+    if add is not None:
+        res_v, res_m = residual
+        if tuple(res_v.shape) != tuple(out.shape):
+            return None
+        if not _matches(add.out, res_v):
+            add.out = torch.empty_like(res_v)
+        if not _matches(add.mask_out, res_m):
+            add.mask_out = torch.empty_like(res_m)
+        out, out_mask, wa, wb = add.out, add.mask_out, add.weight_a, add.weight_b
+    done = hk.sparse_project_expand(
+        x, mask, packed_p, plan_p["g"], res_v, res_m, out, out_mask, packed_e, act_e.prev_out, act_e.out_truncated,
+        act_e.activation_int, plan_e["out"], plan_e["out_mask"], plan_d["g"], act_d.activation_int,
+        act_d.truncation_mode.value, wa, wb)
+    if not done:
+        return None
+    DCConv2d.conv_idx += 1  # the projection's own forward call; the expansion counts when it is finished
+    project.frame_idx += 1
+    return (out, out_mask), OpenExpansion(expand, depthwise)
+
+
+def expand_depthwise(expand, depthwise, input, opened=None):
+    """``depthwise(expand(input))`` for a 1x1 expansion DCConv2d and a 3x3 stride-1 depthwise
+    DCConv2d, both with a truncating activation, as TWO launches instead of three on frames
+    after the first: the expansion's convolution leaves its keep decision to the depthwise
+    kernel (``dc_expand_depthwise``).  Returns the depthwise layer's ``(delta, mask)`` -- exactly
+    what the separate layer calls return, all layer states included -- or ``None`` when the
+    layers are not in a state or of a shape the kernels take; nothing has happened then and the
+    caller runs the layers one by one.  Switch: ``DCConv2d.fuse_expansion``.
+
+    ``opened``: the :class:`OpenExpansion` of a :func:`project_expand` call that has already run
+    the expansion's convolution on ``input``; only the depthwise launch remains, and it cannot be
+    declined any more."""
+    if opened is not None:
+        if opened.expand is not expand or opened.depthwise is not depthwise:
+            raise RuntimeError("an open expansion has to be finished by the layers it was opened for")
+    elif not DCConv2d.fuse_expansion or isinstance(input, Tensor):
+        return None
+    x, mask = input
+    acts = _closing_pair(expand, depthwise, x.dtype)
+    if acts is None:
+        if opened is not None:
+            raise RuntimeError("the layers of an open expansion changed state before it was finished")
+        return None
+    act_e, act_d = acts
     plan_e = expand._plan_for(x.shape, x.dtype, x.device)
     packed = expand._packed_filter()
     if packed is None or plan_e["out"] is None:
@@ -599,8 +681,11 @@ def expand_depthwise(expand, depthwise, input):
     done = hk.sparse_expand_depthwise(
         x, mask, packed, act_e.prev_out, act_e.out_truncated, DCThreshold.get(act_e), act_e.activation_int,
         plan_e["out"], plan_e["out_mask"], depthwise.weight, plan_d["g"], act_d.prev_out, act_d.out_truncated,
-        DCThreshold.get(act_d), act_d.activation_int, act_d.truncation_mode.value, plan_d["out"], plan_d["out_mask"])
+        DCThreshold.get(act_d), act_d.activation_int, act_d.truncation_mode.value, plan_d["out"], plan_d["out_mask"],
+        opened=opened is not None)
     if not done:
+        if opened is not None:
+            raise RuntimeError("dc_expand_depthwise declined to finish an expansion that dc_project_expand left open")
         return None
     for conv in (expand, depthwise):
         DCConv2d.conv_idx += 1  # what the layers' own forward calls would have counted

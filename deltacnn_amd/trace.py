@@ -227,12 +227,26 @@ class Tracer:
                 flops = 2 * ci * ch * n_in
                 shape = f"{ci}->{ch} k1 s1 @{g.in_h}x{g.in_w} (open)"
                 dens = (n_in / p_px, n_in / p_px)
-                ms = ms / 2  # the call's two launches share its time
-                extra = {"kernel": r["kernels"][1], "call": op, "shape": f"dw{ch} k3 s1 @{g.in_h}x{g.in_w} (closing)",
+                opened = meta.get("opened", False)  # the expansion ran in a project_expand call: one launch here
+                if not opened:
+                    ms = ms / 2  # the call's two launches share its time
+                extra = {"kernel": r["kernels"][-1], "call": op, "shape": f"dw{ch} k3 s1 @{g.in_h}x{g.in_w} (closing)",
                          "ms": ms,
                          "bytes": p_px * m + n_in * 3 * ch * s + 9 * ch * s + n_out * 2 * ch * s
                                   + n_in * 2 * ch * s + n_out * 3 * ch * s + p_px * m,
                          "flops": 2 * 9 * ch * n_out, "density_in": n_in / p_px, "density_out": n_out / p_px}
+            elif op == "project_expand":  # projection (+ residual sum) and the next expansion, activation left open
+                g = meta["g"]
+                ch, cm, ce = g.in_c, g.out_c, meta["Ce"]
+                p_px = g.batch * g.in_h * g.in_w
+                n_res = n_in_b or 0
+                rd = p_px * m + n_in * ch * s + ch * cm * s + cm * ce * s + n_out * 2 * ce * s
+                if n_in_b is not None:
+                    rd += p_px * m + n_res * cm * s
+                wr = n_out * cm * s + n_out * 2 * ce * s + 2 * p_px * m
+                flops = 2 * ch * cm * n_in + 2 * cm * ce * n_out
+                shape = f"{ch}->{cm}->{ce} k1 s1 @{g.in_h}x{g.in_w} (pair, open)"
+                dens = (n_in / p_px, n_out / p_px)
             elif op == "pool_densify":  # the map's updated pixels in, accumulator in and out, dense copy out
                 g = meta["g"]
                 p_in = g.batch * g.in_h * g.in_w
@@ -292,8 +306,9 @@ class Tracer:
                 else:  # mul_add
                     rd, wr = P * m + n_in * C * s + C * s, n_in * C * s
                     dens = (n_in / P, n_in / P)
-            out.append({"kernel": r["kernels"][0] or op, "call": op, "shape": shape, "ms": ms,
-                        "bytes": rd + wr, "flops": flops, "density_in": dens[0], "density_out": dens[1]})
+            if not (op == "expand_dw" and meta.get("opened", False)):
+                out.append({"kernel": r["kernels"][0] or op, "call": op, "shape": shape, "ms": ms,
+                            "bytes": rd + wr, "flops": flops, "density_in": dens[0], "density_out": dens[1]})
             if extra is not None:
                 out.append(extra)
         self.records = []

@@ -189,7 +189,7 @@ typedef struct dc_expand_dw_args {
     /* A: 1x1 expansion expand_in_channels -> C (the depthwise layer's channels) + activation/truncation */
     const void *input;              /* [B][H][W][expand_in_channels] delta */
     const int32_t *mask;            /* its update mask */
-    const void *expand_packed_filter;
+    const void *expand_packed_filter; /* NULL: dc_project_expand already ran the convolution (input, mask unused) */
     int32_t expand_in_channels;
     void *expand_prev_out;          /* [P][C] activation state of the expansion, in place */
     void *expand_truncated;
@@ -225,6 +225,47 @@ typedef struct dc_expand_dw_args {
  * to its first frame, which takes the separate calls).  No counterpart in the reference, which
  * launches every layer and every activation on its own (sparse_layers.py:636-638). */
 int dc_expand_depthwise(const dc_geometry *g, const dc_expand_dw_args *args, int dtype, void *stream);
+
+/* Operands of dc_project_expand beyond the projection's 1x1 geometry. */
+typedef struct dc_project_expand_args {
+    /* A: 1x1 projection in_c -> out_c of the geometry argument, no activation */
+    const void *input;              /* [P][in_c] delta (the block's depthwise output) */
+    const int32_t *mask;            /* its update mask */
+    const void *project_packed_filter;
+    const void *residual;           /* [P][out_c] delta added to the projection (DCAdd without activation), or NULL */
+    const int32_t *residual_mask;
+    float weight_residual, weight_conv;
+    void *out;                      /* [P][out_c] block output delta, written where out_mask is 1 */
+    int32_t *out_mask;              /* [P] = mask | residual_mask, written for every pixel */
+    /* B: 1x1 expansion out_c -> expand_channels of the next block, activation left open */
+    const void *expand_packed_filter;
+    int32_t expand_channels;
+    void *expand_prev_out;          /* [P][expand_channels] accumulated values: read only in this call */
+    void *expand_truncated;         /* receives T = truncated + v on updated pixels */
+    int32_t expand_activation;      /* DC_ACT_RELU or DC_ACT_RELU6 */
+    void *expand_out;               /* [P][expand_channels] receives D = act(T + prev) - act(prev) on updated pixels */
+    int32_t *expand_out_mask;       /* [P] receives the update mask (= out_mask) */
+    /* C: the depthwise layer that will finish the expansion (checked, not run) */
+    const dc_geometry *dw_geometry;
+    int32_t dw_activation;
+    int32_t dw_truncation_mode;
+} dc_project_expand_args;
+
+/* The 1x1 projection that ends an inverted-residual block (with the block's residual sum) and the
+ * 1x1 expansion that starts the next block in ONE launch, for the small maps where launches are
+ * the cost.  The expansion's activation is left open exactly as the first launch of
+ * dc_expand_depthwise leaves it (D and T stored, accumulated values untouched); the NEXT call on
+ * these buffers has to be dc_expand_depthwise with expand_packed_filter == NULL, which runs only
+ * its second launch -- the depthwise kernel that takes the keep decision and commits the
+ * expansion's state.  This call verifies that that call will be accepted (dw_geometry,
+ * dw_activation, dw_truncation_mode) and returns DC_ERR_UNSUPPORTED before any launch otherwise,
+ * as for shapes outside its own range: block output channels in multiples of 32 up to 96, a
+ * projection filter of at most 128 KB (every workgroup streams it), layers small enough that the
+ * stand-alone pointwise kernel would split the projection's reduction over four wavefronts and
+ * the expansion's over none.  Together the two calls are identical, bit for bit, to
+ * dc_conv / dc_conv_add(projection), dc_conv_act(expansion), dc_conv_act(depthwise).  16-bit
+ * types; no bias.  No counterpart in the reference (sparse_layers.py:636-638). */
+int dc_project_expand(const dc_geometry *g, const dc_project_expand_args *args, int dtype, void *stream);
 
 /* Number of bytes dc_pack_filter writes for this geometry (0 if the shape has no packed
  * form).  One-time weight relayout for the MFMA kernels, fp16 or bfloat16, un-swizzled, in fragment order

@@ -100,7 +100,8 @@ def test_mobilenet_open_expansions_keep_every_layer_state(lib):
     """MobileNetV2 224x224, 6 frames: the model whose expansions leave their activation to the
     depthwise kernels against the model that issues every layer call on its own -- logits and
     every activation layer's cached state equal bit for bit; nine blocks of every frame after
-    the first take the two-launch form (the 14x14 and 7x7 blocks with a stride-1 depthwise layer)."""
+    the first take the two-launch form (the 14x14 and 7x7 blocks with a stride-1 depthwise layer),
+    six of them with the expansion's convolution inside the previous block's projection launch."""
     from deltacnn_amd import hip_kernels as hk
     from deltacnn_amd import sparse_layers as SL
     from deltacnn_amd.video import moving_rectangles_video
@@ -115,7 +116,15 @@ def test_mobilenet_open_expansions_keep_every_layer_state(lib):
         done = original(*a, **k)
         launches.append(done)
         return done
+    pairs = []
+    original_pair = hk.sparse_project_expand
+
+    def counted_pair(*a, **k):
+        done = original_pair(*a, **k)
+        pairs.append(done)
+        return done
     hk.sparse_expand_depthwise = counted
+    hk.sparse_project_expand = counted_pair
     try:
         with torch.no_grad():
             for t in range(video.shape[0]):
@@ -134,6 +143,9 @@ def test_mobilenet_open_expansions_keep_every_layer_state(lib):
                 n += 1
         assert n == 35
         assert sum(launches) == 9 * (video.shape[0] - 1), (len(launches), sum(launches))
+        # ... and six projections carry the next block's expansion (the 14x14 blocks of 64 and 96 channels)
+        assert sum(pairs) == 6 * (video.shape[0] - 1), (len(pairs), sum(pairs))
     finally:
         SL.DCConv2d.fuse_expansion = SL.DCConv2d.fuse_blocks = True
         hk.sparse_expand_depthwise = original
+        hk.sparse_project_expand = original_pair

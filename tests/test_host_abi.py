@@ -299,3 +299,61 @@ def test_expand_depthwise_arguments_are_checked_before_any_launch(lib):
     assert lib.dc_expand_depthwise(ctypes.byref(g), None, 1, None) == -4
     assert call(g, args(out=None)) == -4 and call(g, args(expand_truncated=None)) == -4
     assert call(g, args(input=p + 2)) == -5 and call(g, args(dw_prev_out=p + 8)) == -5
+
+
+def test_project_expand_arguments_are_checked_before_any_launch(lib):
+    """dc_project_expand: shapes without the one-launch form, or whose expansion the depthwise
+    layer behind it could not finish -> -3 (the caller issues the separate calls), missing
+    operands -> -4, misaligned pointers -> -5; nothing touches a device.  dc_expand_depthwise
+    accepts a missing expansion filter (the convolution has run already) but no missing state."""
+    from deltacnn_amd._lib import ExpandDwArgs, ProjectExpandArgs
+    buf = (ctypes.c_char * 8192)()
+    p = (ctypes.addressof(buf) + 255) // 256 * 256
+    one = dict(kernel_h=1, kernel_w=1, pad_top=0, pad_left=0, pad_bottom=0, pad_right=0)
+    g = _geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=384, out_c=64, **one)
+    gd = _geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=384, out_c=384, groups=384)
+
+    def args(dw=gd, **kw):
+        a = ProjectExpandArgs()
+        for name in ("input", "mask", "project_packed_filter", "residual", "residual_mask", "out", "out_mask",
+                     "expand_packed_filter", "expand_prev_out", "expand_truncated", "expand_out", "expand_out_mask"):
+            setattr(a, name, p)
+        a.weight_residual = a.weight_conv = 1.0
+        a.expand_channels, a.expand_activation, a.dw_activation, a.dw_truncation_mode = 384, 2, 2, 0
+        a.dw_geometry = ctypes.pointer(dw) if dw is not None else None
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+
+    def call(geom, a, dtype=1):
+        return lib.dc_project_expand(ctypes.byref(geom), ctypes.byref(a), dtype, None)
+
+    assert call(g, args(), dtype=0) == -3 and b"16-bit" in lib.dc_last_error()
+    assert call(g, args(), dtype=9) == -1
+    assert call(g, args(expand_channels=0)) == -2
+    assert call(g, args(expand_activation=3)) == -3                        # leaky ReLU has no open form
+    assert call(_geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=384, out_c=48, **one), args()) == -3   # 48 channels
+    assert call(_geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=960, out_c=160, **one), args()) == -3  # too wide
+    assert call(_geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=384, out_c=64), args()) == -3          # 3x3
+    strided = _geom(in_h=14, in_w=14, out_h=7, out_w=7, in_c=384, out_c=384, groups=384, stride_h=2, stride_w=2)
+    assert call(g, args(dw=strided)) == -3 and b"depthwise" in lib.dc_last_error()
+    other = _geom(in_h=7, in_w=7, out_h=7, out_w=7, in_c=384, out_c=384, groups=384)
+    assert call(g, args(dw=other)) == -2                                   # not on the expansion's output map
+    assert call(g, args(dw=None)) == -4
+    assert lib.dc_project_expand(None, ctypes.byref(args()), 1, None) == -4
+    assert lib.dc_project_expand(ctypes.byref(g), None, 1, None) == -4
+    assert call(g, args(out=None)) == -4 and call(g, args(expand_truncated=None)) == -4
+    assert call(g, args(residual_mask=None)) == -4                         # a residual needs its mask
+    assert call(g, args(input=p + 2)) == -5 and call(g, args(expand_prev_out=p + 8)) == -5
+
+    # the second call of the pair: no expansion filter, no input, but every state tensor
+    b = ExpandDwArgs()
+    for name in ("expand_prev_out", "expand_truncated", "expand_out", "expand_out_mask", "dw_filter", "dw_prev_out",
+                 "dw_truncated", "out", "out_mask"):
+        setattr(b, name, p)
+    b.expand_in_channels, b.expand_threshold, b.expand_activation, b.expand_truncation_mode = 64, 0.05, 2, 0
+    b.dw_threshold, b.dw_activation, b.dw_truncation_mode = 0.05, 2, 0
+    b.expand_truncated = None
+    assert lib.dc_expand_depthwise(ctypes.byref(gd), ctypes.byref(b), 1, None) == -4
+    b.expand_truncated, b.dw_truncated = p, p + 8
+    assert lib.dc_expand_depthwise(ctypes.byref(gd), ctypes.byref(b), 1, None) == -5
