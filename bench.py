@@ -278,11 +278,18 @@ def _trace_calls(fn, alt_inputs=None):
 
 
 def _row_report(rows):
-    return [{"kernel": r["kernel"], "us": round(r["ms"] * 1e3, 3),
-             "alg_GBps": round(r["bytes"] / (r["ms"] * 1e-3) / 1e9, 1),
-             "hbm_frac": round(r["bytes"] / (r["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-             "alg_TFLOPs": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2),
-             "mfma_frac": round(r["flops"] / (r["ms"] * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 5)} for r in rows]
+    """Per-launch report rows.  A launch whose share of a two-kernel call was measured as zero
+    (the difference of two replays of a few microseconds, e.g. under a profiler) gets no rates."""
+    out = []
+    for r in rows:
+        sec = r["ms"] * 1e-3
+        rate = (lambda v, scale, digits: round(v / sec / scale, digits)) if sec > 0 else (lambda v, scale, digits: None)
+        gbps, tflops = rate(r["bytes"], 1e9, 1), rate(r["flops"], 1e12, 2)
+        out.append({"kernel": r["kernel"], "us": round(r["ms"] * 1e3, 3), "alg_GBps": gbps,
+                    "hbm_frac": None if gbps is None else round(r["bytes"] / sec / 1e9 / HBM_PEAK_GBS, 4),
+                    "alg_TFLOPs": tflops,
+                    "mfma_frac": None if tflops is None else round(r["flops"] / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 5)})
+    return out
 
 
 def micro_bench():
@@ -317,7 +324,7 @@ def micro_bench():
             out.append({"op": name, "density": rho, "us": round(sum(r["ms"] for r in rows) * 1e3, 3),
                         "kernels": _row_report(rows)})
             log(f"  micro {name:18s} density {rho:4.2f}: " +
-                "  ".join(f"{r['kernel']} {r['us']:.2f} us {r['alg_GBps']:.0f} GB/s {r['alg_TFLOPs']:.1f} TF/s"
+                "  ".join(f"{r['kernel']} {r['us']:.2f} us {r['alg_GBps'] or 0:.0f} GB/s {r['alg_TFLOPs'] or 0:.1f} TF/s"
                           for r in out[-1]["kernels"]))
     return out
 
@@ -377,7 +384,7 @@ def scaled_bench():
             rep = _row_report(rows)
             out.append({"op": name, "density": rho, "kernels": rep})
             log(f"  scaled {name:20s} density {rho:4.2f}: " +
-                "  ".join(f"{r['kernel']} {r['us']:.1f} us {r['alg_GBps']:.0f} GB/s ({100 * r['hbm_frac']:.1f} % of HBM peak)"
+                "  ".join(f"{r['kernel']} {r['us']:.1f} us {r['alg_GBps'] or 0:.0f} GB/s ({100 * (r['hbm_frac'] or 0):.1f} % of HBM peak)"
                           for r in rep))
     return out
 
