@@ -352,6 +352,8 @@ def scaled_bench():
     from deltacnn_amd.filter_conversion import convert_half_filter
     wpw = convert_half_filter((torch.randn(C, C, 1, 1, generator=torch.Generator().manual_seed(8)) / C ** 0.5).half()).cuda()
     wpw_packed = hk.pack_filter(wpw, C, C, 1)
+    w33 = convert_half_filter((torch.randn(C, C, 3, 3, generator=torch.Generator().manual_seed(9)) / (9 * C) ** 0.5).half()).cuda()
+    w33_packed = hk.pack_filter(w33, C, C, 1)
     for rho in (0.1, 1.0):
         mask = (torch.rand(B, 1, H, W, device="cuda", generator=gen) < rho).to(torch.int32)
         mask2 = mask.clone()
@@ -375,6 +377,9 @@ def scaled_bench():
             "pointwise64->64+relu": (lambda: hk.sparse_conv_activation(a, wpw, mask, None, b, c, 0.0, 1, 0, (1, 1), (0, 0),
                                                                          (1, 1), 1, C, out=d, out_mask=mask2,
                                                                          packed_filter=wpw_packed), None),
+            # the K x K contraction at this size sits at the ridge (288 flop per byte): its row is read against both peaks
+            "conv3x3_64->64": (lambda: hk.sparse_conv(a, w33, mask, None, (1, 1), (1, 1), (1, 1), 1, c_out=C, out=d,
+                                                        out_mask=mask2, packed_filter=w33_packed), None),
         })
         qmask_in = (torch.rand(B, 1, H // 2, W // 2, device="cuda", generator=gen) < rho).to(torch.int32)
         if rho < 1:
@@ -384,7 +389,8 @@ def scaled_bench():
             rep = _row_report(rows)
             out.append({"op": name, "density": rho, "kernels": rep})
             log(f"  scaled {name:20s} density {rho:4.2f}: " +
-                "  ".join(f"{r['kernel']} {r['us']:.1f} us {r['alg_GBps'] or 0:.0f} GB/s ({100 * (r['hbm_frac'] or 0):.1f} % of HBM peak)"
+                "  ".join(f"{r['kernel']} {r['us']:.1f} us {r['alg_GBps'] or 0:.0f} GB/s ({100 * (r['hbm_frac'] or 0):.1f} % of HBM peak"
+                          + (f", {100 * (r['mfma_frac'] or 0):.1f} % of the MFMA peak)" if (r['alg_TFLOPs'] or 0) >= 50 else ")")
                           for r in rep))
     return out
 

@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB = os.path.join(PKG, "libdeltacnn_hip.so")
-SOURCES = ["dc_abi.cpp", "elementwise.hip", "conv.hip", "pwconv.hip", "pwpair.hip", "pool.hip", "block.hip", "linear.hip"]
+SOURCES = ["dc_abi.cpp", "elementwise.hip", "conv.hip", "convres.hip", "pwconv.hip", "pwpair.hip", "pool.hip", "block.hip", "linear.hip"]
 HEADERS = ["common.hpp", "tile.hpp", "epilogue.hpp", os.path.join("..", "..", "include", "deltacnn_hip.h")]
 # -ffp-contract=off: every operation of the bit-exact elementwise operators rounds on its own.
 # packed-fp32-ops disabled: hipcc must not form v_pk_*_f32 from ordinary float code.

@@ -2387,7 +2387,13 @@ hipError_t launch_conv_t(const dc_geometry &g, const void *in, const void *filte
         // Larger layers: halo staged in LDS (see conv_lds_mfma_kernel).
         const LdsPlan lp = lds_plan(g, transposed);
         if (lp.ok) {
-            hipError_t le = launch_lds_conv<E16>(g, p, lp, in, packed, bias, out, mask, out_mask, transposed, nullptr, s);
+            // thin layers on large maps: the filter stays in registers while a workgroup walks over tiles
+            const bool resident = !transposed &&
+                resident_conv_eligible(g, lp.hal_h, lp.hal_w, lp.ltx, lp.lty, lp.kcc, lp.rl, lp.ksl, lp.ncw);
+            hipError_t le = resident
+                ? launch_resident_conv(g, p, lp.hal_h, lp.hal_w, lp.ltx, lp.lty, lp.kcc, lp.rl, lp.ksl, lp.ncw, in, packed,
+                                       bias, out, mask, out_mask, dtype, s)
+                : launch_lds_conv<E16>(g, p, lp, in, packed, bias, out, mask, out_mask, transposed, nullptr, s);
             if (le != hipSuccess || epi == nullptr) return le;
             return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
                                             epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);

@@ -133,4 +133,12 @@ __device__ __forceinline__ int tile_front(const ConvP &p, const int32_t *__restr
     return *s_n;
 }
 
+// The resident-filter form of the LDS-halo kernel (convres.hip): thin layers on large maps.  The
+// arguments after the geometry are the launch plan of conv_lds_mfma_kernel for the layer.
+bool resident_conv_eligible(const dc_geometry &g, int hal_h, int hal_w, int ltx, int lty, int kcc, int rl,
+                            int ksl, int ncw);
+hipError_t launch_resident_conv(const dc_geometry &g, const ConvP &p, int hal_h, int hal_w, int ltx, int lty, int kcc,
+                                int rl, int ksl, int ncw, const void *in, const void *packed, const void *bias,
+                                void *out, const int32_t *mask, int32_t *out_mask, int dtype, hipStream_t s);
+
 }  // namespace dc

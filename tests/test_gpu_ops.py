@@ -417,11 +417,42 @@ def test_conv(lib, dtype, cfg, density, use_bias, packed):
     _check_conv(dtype, out, want, want_mask)
 
 
+RESIDENT = [  # Cin, Cout, K, stride, padding, dilation, groups, H, W (batch 2): at least 2048 output tiles
+    (64, 64, 3, 1, 1, 1, 1, 256, 250),   # two channel tiles per wavefront, two reduction slices
+    (64, 32, 3, 1, 1, 1, 1, 256, 256),   # four reduction slices
+    (48, 64, 3, 2, 1, 1, 1, 512, 500),   # stride 2: 17 x 17 halo; input channels that do not fill the second step
+    (64, 32, 3, 1, 2, 2, 1, 256, 257),   # dilation 2
+    (40, 24, 3, 1, 1, 1, 1, 256, 256),   # channels that fill neither a reduction step nor the last channel tile
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["float16", "bfloat16"])
+@pytest.mark.parametrize("cfg", RESIDENT, ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("density", [0.02, 0.3, 1.0])
+def test_conv_resident_filter(lib, dtype, cfg, density):
+    """The resident-filter form of the K x K MFMA kernel (a workgroup walks over many tiles with
+    the filter fragments in registers) against the oracle, with a bias on the dense case."""
+    from deltacnn_amd import _lib
+    groups, Cin, Cout = cfg[6], cfg[0], cfg[1]
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 900 + Cin + Cout, density)
+    use_bias = density == 1.0
+    want, want_mask = ops.conv(x, mask, wt, bias if use_bias else None, s, p, d, groups)
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, Cin, Cout, groups)
+    out, om = hk().sparse_conv(cl(poison(x, mask)), d_filt, cl(mask), bias.to(DEV) if use_bias else None,
+                               s, p, d, groups, c_out=Cout, create_out_mask=True, packed_filter=pk)
+    assert _lib.load().dc_last_kernels().decode() == "conv_res_mfma_kernel"
+    assert torch.equal(om.cpu(), want_mask)
+    _check_conv(dtype, out, want, want_mask)
+
+
 @pytest.mark.parametrize("cfg,kernel", [
     ((32, 32, 3, 1, 1, 1, 1, 16, 16), "conv_patch_mfma_kernel"),
     ((64, 64, 3, 1, 1, 1, 1, 72, 70), "conv_lds_mfma_kernel"),
     ((16, 64, 3, 1, 1, 1, 1, 120, 120), "conv_lds_mfma_kernel"),
     ((320, 32, 3, 1, 1, 1, 1, 40, 40), "conv_lds_mfma_kernel"),
+    ((64, 64, 3, 1, 1, 1, 1, 256, 250), "conv_res_mfma_kernel"),   # thin layers on >= 2048 tiles: resident filter
+    ((16, 32, 3, 2, 1, 1, 1, 520, 500), "conv_lds_mfma_kernel"),   # one channel step: the per-tile kernel stays
     ((64, 256, 1, 1, 0, 1, 1, 20, 20), "pw_mfma_kernel"),
     ((32, 32, 3, 1, 1, 1, 32, 15, 18), "conv_dw_kernel"),
     ((16, 16, 3, 1, 1, 1, 16, 726, 727), "conv_dw_scan_kernel"),
