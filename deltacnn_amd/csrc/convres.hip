@@ -8,10 +8,13 @@
 // over tiles (tile = blockIdx.x, blockIdx.x + gridDim.x, ...): the filter fragments of each
 // wavefront's reduction steps (at most RES_MAX_STEPS steps x R channel tiles) are loaded before
 // the loop and stay in registers, the step table is built once, and per tile only the mask words,
-// the halo and the outputs move.  The mask words and halo rows of the NEXT tile are requested
-// before the reduction of the current one (unconditionally, from clamped addresses, and selected
-// by the mask afterwards), so the memory round trips of a tile hide behind the previous tile's
-// matrix instructions instead of heading its dependency chain.
+// the halo and the outputs move.  The loop is a two-stage pipeline with ONE barrier per tile:
+// the mask words and halo rows of the NEXT tile are requested before the reduction of the current
+// one (unconditionally, from clamped addresses, and selected by the mask afterwards) and staged
+// into the second of two LDS halo buffers right after it; every wavefront dilates and compacts
+// the tile's mask for itself; the partial sums of the reduction slices alternate between two
+// buffers as well, so the wavefronts that finish and store tile i never hold up the ones that
+// already contract tile i + 1.
 //
 // Everything else is the algorithm of conv_lds_mfma_kernel for a plain (not transposed)
 // convolution whose input channels fit one LDS chunk: halo staged in LDS with inactive and
@@ -21,6 +24,7 @@
 // one rounding after the bias.  An output element is accumulated by the same instruction sequence
 // in both kernels, so they agree bit for bit.
 #include <algorithm>
+#include <atomic>
 #include <type_traits>
 
 #include "epilogue.hpp"
@@ -30,7 +34,7 @@ namespace dc {
 namespace {
 
 constexpr int RES_MAX_STEPS = 10;   // reduction steps per wavefront that stay in registers
-constexpr int RES_MAX_HALO = 1024;  // halo pixels (table in LDS)
+constexpr int RES_MAX_HALO = 512;   // halo pixels (two tables in LDS)
 constexpr int RES_MAX_TABLE = 96;   // reduction steps of a tile (taps x channel steps)
 
 struct ResP {
@@ -47,11 +51,12 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
     typedef typename Elem16<E>::v4 E4;
     typedef typename Elem16<E>::v8 E8;
     constexpr int NT = 4;
-    extern __shared__ __align__(16) unsigned char s_halo[];
-    __shared__ int s_hpix[RES_MAX_HALO];
+    // dynamic LDS: two halo buffers (tile i is contracted out of one while tile i + 1 is staged
+    // into the other), then two buffers for the partial sums of the reduction slices
+    extern __shared__ __align__(16) unsigned char s_dyn[];
+    __shared__ int s_hpix[2][RES_MAX_HALO];
     __shared__ int2 s_step[RES_MAX_TABLE];
-    __shared__ int s_list[TILE_PX];
-    __shared__ int s_n;
+    __shared__ int s_wlist[8][TILE_PX];  // per wavefront: the tile's compacted updated pixels
     const int cb = blockIdx.y;
     const int tid = threadIdx.x, nthr = blockDim.x, nw = nthr / WAVE;
     const int wv = wave_id(), lane = lane_id();
@@ -63,6 +68,9 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
     const int K2 = p.Kh * p.Kw;
     const int nsteps = K2 * ksteps;
     const int row = q.kcc * 64 + 16;  // bytes per staged halo pixel
+    const int halo_bytes = hal_h * q.pitch * row;
+    unsigned char *s_part0 = s_dyn + 2 * halo_bytes;
+    const int PART_BYTES = (KS - 1) * ncw * R * NT * WAVE * 16;  // (KS - 1) slices x ncw groups x R x NT tiles
     auto tap_off = [&](int a, int b2) { return a * p.dh * hal_w + b2 * p.dw; };        // in the pixel table
     auto tap_lds = [&](int a, int b2) { return a * p.dh * q.pitch + b2 * p.dw; };      // in the staged halo
 
@@ -123,93 +131,110 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
             val[u] = *reinterpret_cast<const E8 *>(inb + (unsigned)(px * p.Ci));
         }
     };
-    if ((int)blockIdx.x < q.tiles) request(blockIdx.x);
-
-    for (int tile = blockIdx.x; tile < q.tiles; tile += gridDim.x) {
-        const int b = tile / tiles_per_map, tr = tile - b * tiles_per_map;
-        const int ty0 = (tr / q.ltx) * TILE, tx0 = (tr % q.ltx) * TILE;
-        __syncthreads();  // the previous tile's readers of the halo, the table and the list are done
-        {   // what was requested for this tile: table entry (first lane of a pixel) and halo bytes
-            const bool vok = sv < q.kcc * 4 && sv * 8 < p.Ci;
+    // what was requested goes into halo buffer `buf`: table entry (first lane of a pixel) and bytes
+    auto stage = [&](int buf) {
+        const bool vok = sv < q.kcc * 4 && sv * 8 < p.Ci;
+        unsigned char *halo = s_dyn + buf * halo_bytes;
 #pragma unroll
-            for (int u = 0; u < SU; ++u) {
-                const int hp = (tid >> q.lgv) + u * hstep;
-                const bool on = hpixel[u] >= 0 && word[u] != 0;
-                if (hp < hpx) {
-                    if (sv == 0) s_hpix[hp] = on ? hpixel[u] : -1;
-                    if (sv < q.kcc * 4)
-                        *reinterpret_cast<E8 *>(s_halo + ((hyx[u] >> 16) * q.pitch + (hyx[u] & 0xffff)) * row + sv * 16) =
-                            keep8(val[u], vok && on);
-                }
+        for (int u = 0; u < SU; ++u) {
+            const int hp = (tid >> q.lgv) + u * hstep;
+            const bool on = hpixel[u] >= 0 && word[u] != 0;
+            if (hp < hpx) {
+                if (sv == 0) s_hpix[buf][hp] = on ? hpixel[u] : -1;
+                if (sv < q.kcc * 4)
+                    *reinterpret_cast<E8 *>(halo + ((hyx[u] >> 16) * q.pitch + (hyx[u] & 0xffff)) * row + sv * 16) =
+                        keep8(val[u], vok && on);
             }
         }
-        __syncthreads();
-        if (tid < WAVE) {  // dilate the mask over the window, compact the updated pixels
-            const int ly = tid >> 3, lx = tid & 7;
+    };
+    if ((int)blockIdx.x < q.tiles) {
+        request(blockIdx.x);
+        stage(0);
+    }
+    __syncthreads();
+
+    // One barrier per tile.  Every wavefront dilates and compacts the tile's mask for itself (the
+    // first one writes the output mask); the partial sums of tile i and the staged halo of tile
+    // i + 1 become visible at the same barrier, behind which the finishing wavefronts store.
+    int it = 0;
+    for (int tile = blockIdx.x; tile < q.tiles; tile += gridDim.x, ++it) {
+        const int cur = it & 1;
+        const int b = tile / tiles_per_map, tr = tile - b * tiles_per_map;
+        const int ty0 = (tr / q.ltx) * TILE, tx0 = (tr % q.ltx) * TILE;
+        const bool has_next = tile + (int)gridDim.x < q.tiles;
+        if (has_next) request(tile + gridDim.x);  // travels while this tile is contracted
+        const unsigned char *halo = s_dyn + cur * halo_bytes;
+        int n;
+        {
+            const int ly = lane >> 3, lx = lane & 7;
             const int oy = ty0 + ly, ox = tx0 + lx;
             const bool inside = oy < p.Ho && ox < p.Wo;
             bool upd = false;
             const int base = ly * p.sh * hal_w + lx * p.sw;
-            for (int ta = 0; ta < p.Kh; ++ta)
-                for (int tb = 0; tb < p.Kw; ++tb) upd |= s_hpix[base + tap_off(ta, tb)] >= 0;
-            upd = upd && inside;
-            if (inside && cb == 0) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = upd ? 1 : 0;
-            int n;
-            const int rank = wave_rank(upd, n);
-            if (upd) s_list[rank] = tid;
-            if (tid == 0) s_n = n;
-        }
-        __syncthreads();
-        const int n = s_n;
-        // the next tile's mask words and halo rows travel while this one is contracted
-        if (tile + (int)gridDim.x < q.tiles) request(tile + gridDim.x);
-        if (n == 0) continue;  // the same for every wavefront
-
-        const int n_tiles = (n + 15) >> 4;
-        int hbase[NT];
+            if (p.Kh == 3 && p.Kw == 3) {  // the common window: nine independent reads
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const int slot = nt * 16 + l16;
-            const int loc = slot < n ? s_list[slot] : 0;
-            hbase[nt] = ((loc >> 3) * p.sh * q.pitch + (loc & 7) * p.sw) * row + kq * 16;
+                for (int t = 0; t < 9; ++t) upd |= s_hpix[cur][base + tap_off(t / 3, t % 3)] >= 0;
+            } else {
+                for (int ta = 0; ta < p.Kh; ++ta)
+                    for (int tb = 0; tb < p.Kw; ++tb) upd |= s_hpix[cur][base + tap_off(ta, tb)] >= 0;
+            }
+            upd = upd && inside;
+            if (wv == 0 && inside && cb == 0) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = upd ? 1 : 0;
+            const int rank = wave_rank(upd, n);
+            if (upd) s_wlist[wv][rank] = lane;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
         float4_t acc[R][NT];
+        int loc[NT];
+        if (n > 0) {  // the same for every wavefront
+            const int n_tiles = (n + 15) >> 4;
+            int hbase[NT];
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) acc[r][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
-        auto reduce = [&](auto nta_tag) {
-            constexpr int NTA = decltype(nta_tag)::value;
-#pragma unroll
-            for (int i = 0; i < NSW; ++i) {
-                if (i * KS + kz >= nsteps) break;  // wave-uniform
-                E8 x[NTA];
-#pragma unroll
-                for (int nt = 0; nt < NTA; ++nt) x[nt] = *reinterpret_cast<const E8 *>(s_halo + hbase[nt] + xoff[i]);
-#pragma unroll
-                for (int nt = 0; nt < NTA; ++nt)
-#pragma unroll
-                    for (int r = 0; r < R; ++r) acc[r][nt] = Elem16<E>::mfma(a[i][r], x[nt], acc[r][nt]);
+            for (int nt = 0; nt < NT; ++nt) {
+                const int slot = nt * 16 + l16;
+                loc[nt] = slot < n ? s_wlist[wv][slot] : 0;
+                hbase[nt] = ((loc[nt] >> 3) * p.sh * q.pitch + (loc[nt] & 7) * p.sw) * row + kq * 16;
             }
-        };
-        switch (n_tiles) {
-            case 1: reduce(std::integral_constant<int, 1>{}); break;
-            case 2: reduce(std::integral_constant<int, 2>{}); break;
-            case 3: reduce(std::integral_constant<int, 3>{}); break;
-            default: reduce(std::integral_constant<int, 4>{}); break;
-        }
-        if (KS > 1) {  // partial sums of the reduction slices meet in LDS (the halo is no longer needed)
-            float4_t *s_part = reinterpret_cast<float4_t *>(s_halo);
-            __syncthreads();
-            if (kz > 0) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[r][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+            auto reduce = [&](auto nta_tag) {
+                constexpr int NTA = decltype(nta_tag)::value;
+#pragma unroll
+                for (int i = 0; i < NSW; ++i) {
+                    if (i * KS + kz >= nsteps) break;  // wave-uniform
+                    E8 x[NTA];
+#pragma unroll
+                    for (int nt = 0; nt < NTA; ++nt) x[nt] = *reinterpret_cast<const E8 *>(halo + hbase[nt] + xoff[i]);
+#pragma unroll
+                    for (int nt = 0; nt < NTA; ++nt)
+#pragma unroll
+                        for (int r = 0; r < R; ++r) acc[r][nt] = Elem16<E>::mfma(a[i][r], x[nt], acc[r][nt]);
+                }
+            };
+            switch (n_tiles) {
+                case 1: reduce(std::integral_constant<int, 1>{}); break;
+                case 2: reduce(std::integral_constant<int, 2>{}); break;
+                case 3: reduce(std::integral_constant<int, 3>{}); break;
+                default: reduce(std::integral_constant<int, 4>{}); break;
+            }
+            if (KS > 1 && kz > 0) {
+                float4_t *s_part = reinterpret_cast<float4_t *>(s_part0 + cur * PART_BYTES);
 #pragma unroll
                 for (int r = 0; r < R; ++r)
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt)
                         s_part[((((kz - 1) * ncw + cw) * R + r) * NT + nt) * WAVE + lane] = acc[r][nt];
             }
-            __syncthreads();
-            if (kz > 0) continue;  // these wavefronts wait at the top of the next tile
+        }
+        if (has_next) stage(cur ^ 1);
+        __syncthreads();
+        if (n == 0 || kz > 0) continue;
+        if (KS > 1) {
+            const float4_t *s_part = reinterpret_cast<const float4_t *>(s_part0 + cur * PART_BYTES);
 #pragma unroll
             for (int s = 1; s < KS; ++s)  // ascending slice order
 #pragma unroll
@@ -226,10 +251,8 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
             const int co = ct * 16 + kq * 4;  // lane holds channels co .. co + 3 of pixel (nt, l16)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const int pix = nt * 16 + l16;
-                if (pix >= n) continue;
-                const int loc = s_list[pix];
-                E *o = otile + (unsigned)(((loc >> 3) * p.Wo + (loc & 7)) * p.Co + co);
+                if (nt * 16 + l16 >= n) continue;
+                E *o = otile + (unsigned)(((loc[nt] >> 3) * p.Wo + (loc[nt] & 7)) * p.Co + co);
                 E4 v;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) v[i] = E(acc[r][nt][i] + float(bv[r][i]));
@@ -247,14 +270,22 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
 
 }  // namespace
 
-// Pixels per halo row in LDS.  A 16-pixel tile of a dense output tile is two rows of eight
-// pixels; with a staged pixel of 16 bytes x an odd count, its 16 fragment reads hit distinct
-// bank groups when the second row starts 8 (mod 16) pixels behind the first.
-static int halo_pitch(const dc_geometry &g, int hal_w) {
-    if (g.stride_w != 1) return hal_w;
-    int pitch = hal_w;
-    while (pitch % 16 != 8) ++pitch;
-    return pitch;
+// Dynamic LDS of a launch: two halo buffers and two buffers of partial sums.
+static size_t resident_lds(int hpx, int kcc, int rl, int ksl, int ncw) {
+    return 2 * (size_t)hpx * (kcc * 64 + 16) + 2 * (size_t)(ksl - 1) * ncw * rl * 4 * 1024;
+}
+
+// Raises a kernel's dynamic LDS limit, once per kernel and device; a plain host call.
+template <typename K>
+static hipError_t allow_lds(K *kernel) {
+    static std::atomic<uint64_t> done{0};  // one bit per device; devices past 63 ask every time
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 64 && ((done.load(std::memory_order_relaxed) >> dev) & 1ull)) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 112 << 10);
+    if (e == hipSuccess && dev < 64) done.fetch_or(1ull << dev, std::memory_order_relaxed);
+    return e;
 }
 
 // Layers the resident-filter kernel takes, given the arrangement conv_lds_mfma_kernel would use
@@ -268,20 +299,23 @@ bool resident_conv_eligible(const dc_geometry &g, int hal_h, int hal_w, int ltx,
     const int nsteps = g.kernel_h * g.kernel_w * ksteps;
     const int co_tiles = ceil_div(g.out_c, 16);
     const int cbl = ceil_div(co_tiles, ncw * rl);
-    // Measured on 8 x 512 x 512 maps against conv_lds_mfma_kernel: 17-20 % faster where the filter
-    // takes two channel steps (64 -> 64: 399 -> 319 us, 64 -> 32: 352 -> 280 us), no gain or a loss
+    // Measured on 8 x 512 x 512 maps against conv_lds_mfma_kernel: 3 x 3 64 -> 64, whose filter takes
+    // two channel steps, 399 -> 289 us at full density and 345 -> 239 us at 10 %; no gain or a loss
     // for a single channel step, whose filter of a few KB was never the cost (32 -> 64 stride 2:
     // 67 -> 70 us; 16 -> 16 on 544 x 960: 19.6 -> 22.8 us).
     if (kcc < 2) return false;
-    // (four slices x two channel tiles x ten steps of fragments would not fit the register file)
-    if (kcc != ksteps || nsteps > RES_MAX_TABLE || ceil_div(nsteps, ksl) > (ksl == 4 ? 5 : RES_MAX_STEPS)) return false;
-    if (!((rl == 1 && ksl == 1) || (rl == 2 && (ksl == 1 || ksl == 2 || ksl == 4)))) return false;
+    if (kcc != ksteps || nsteps > RES_MAX_TABLE || ceil_div(nsteps, ksl) > RES_MAX_STEPS) return false;
+    if (!((rl == 1 && ksl == 1) || (rl == 2 && ksl == 2))) return false;  // the arrangements that occur in this range
     const int hpx = hal_h * hal_w;
     if (hpx > RES_MAX_HALO) return false;
-    const size_t lds = std::max((size_t)hal_h * halo_pitch(g, hal_w) * (kcc * 64 + 16), (size_t)(ksl - 1) * ncw * rl * 4 * 1024);
-    if (lds > (48u << 10)) return false;  // + 5 KB of tables: within the 64 KB a workgroup gets without asking
+    // two workgroups per compute unit (with one, the form loses to the per-tile kernel: 64 -> 32 with
+    // four reduction slices, whose partial sums take 48 KB, 397 us against 352 us)
+    if (resident_lds(hpx, kcc, rl, ksl, ncw) > (72u << 10)) return false;
     const int hstep = (ncw * ksl * WAVE) >> log2i(pow2_ceil(kcc * 4));
-    if (ceil_div(hpx, hstep) > 12) return false;  // halo rows a lane keeps in flight
+    const int su = ceil_div(hpx, hstep);  // halo rows a lane keeps in flight
+    const int nsw = ceil_div(nsteps, ksl);
+    // (instances that would spill registers are not offered)
+    if (su > 12 || (rl == 2 && su > (nsw > 5 ? 4 : 8))) return false;
     // (offsets within one map of the batch are computed in 32 bits)
     if ((int64_t)g.in_h * g.in_w * g.in_c >= (1ll << 31) || (int64_t)g.out_h * g.out_w * g.out_c >= (1ll << 31)) return false;
     return (int64_t)ltx * lty * g.batch * cbl >= 2048;
@@ -299,8 +333,8 @@ static hipError_t resident_t(const dc_geometry &g, const ConvP &p, int hal_h, in
     q.hal_h = hal_h; q.hal_w = hal_w; q.kcc = kcc;
     q.lgv = log2i(pow2_ceil(kcc * 4));
     q.ltx = ltx; q.lty = lty; q.tiles = ltx * lty * g.batch;
-    q.pitch = halo_pitch(g, hal_w);
-    const size_t lds = std::max((size_t)hal_h * q.pitch * (kcc * 64 + 16), (size_t)(ksl - 1) * ncw * rl * 4 * 1024);
+    q.pitch = hal_w;
+    const size_t lds = resident_lds(hpx, kcc, rl, ksl, ncw);
     const int nwv = ncw * ksl;
     // workgroups per compute unit: what registers and LDS allow, so that the memory round trips
     // of one workgroup's tile hide behind the others' reductions
@@ -311,8 +345,12 @@ static hipError_t resident_t(const dc_geometry &g, const ConvP &p, int hal_h, in
     note_kernel("conv_res_mfma_kernel");
     const int su = ceil_div(hpx, (nwv * WAVE) >> q.lgv);
 #define DC_RES_S(RV, KV, NV, SV)                                                                             \
-    conv_res_mfma_kernel<E, RV, KV, NV, SV><<<grid, nwv * WAVE, lds, s>>>(p, q, (const E *)in, (const E *)packed, \
-                                                                          (const E *)bias, (E *)out, mask, out_mask)
+    do {                                                                                                     \
+        const hipError_t big = allow_lds(&conv_res_mfma_kernel<E, RV, KV, NV, SV>);                          \
+        if (big != hipSuccess) return big;                                                                   \
+        conv_res_mfma_kernel<E, RV, KV, NV, SV><<<grid, nwv * WAVE, lds, s>>>(p, q, (const E *)in, (const E *)packed, \
+                                                                              (const E *)bias, (E *)out, mask, out_mask); \
+    } while (0)
 #define DC_RES(RV, KV, NV)                                                                                   \
     do {                                                                                                     \
         if (su <= 4) DC_RES_S(RV, KV, NV, 4);                                                                \
@@ -325,9 +363,7 @@ static hipError_t resident_t(const dc_geometry &g, const ConvP &p, int hal_h, in
         else DC_RES(RV, KV, RES_MAX_STEPS);                                                                  \
     } while (0)
     if (rl == 1) DC_RES_N(1, 1);
-    else if (ksl == 1) DC_RES_N(2, 1);
-    else if (ksl == 2) DC_RES_N(2, 2);
-    else DC_RES(2, 4, 5);
+    else DC_RES_N(2, 2);
 #undef DC_RES_N
 #undef DC_RES
 #undef DC_RES_S

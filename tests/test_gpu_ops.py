@@ -419,10 +419,9 @@ def test_conv(lib, dtype, cfg, density, use_bias, packed):
 
 RESIDENT = [  # Cin, Cout, K, stride, padding, dilation, groups, H, W (batch 2): at least 2048 output tiles
     (64, 64, 3, 1, 1, 1, 1, 256, 250),   # two channel tiles per wavefront, two reduction slices
-    (64, 32, 3, 1, 1, 1, 1, 256, 256),   # four reduction slices
-    (48, 64, 3, 2, 1, 1, 1, 512, 500),   # stride 2: 17 x 17 halo; input channels that do not fill the second step
-    (64, 32, 3, 1, 2, 2, 1, 256, 257),   # dilation 2
-    (40, 24, 3, 1, 1, 1, 1, 256, 256),   # channels that fill neither a reduction step nor the last channel tile
+    (64, 96, 3, 1, 1, 1, 1, 256, 256),   # two channel blocks
+    (40, 64, 3, 1, 1, 1, 1, 250, 256),   # input channels that do not fill the second reduction step
+    (56, 80, 3, 1, 1, 1, 1, 256, 250),   # a last channel block with one tile
 ]
 
 
