@@ -417,11 +417,12 @@ def test_conv(lib, dtype, cfg, density, use_bias, packed):
     _check_conv(dtype, out, want, want_mask)
 
 
-RESIDENT = [  # Cin, Cout, K, stride, padding, dilation, groups, H, W (batch 2): at least 2048 output tiles
+RESIDENT = [  # Cin, Cout, K, stride, padding, dilation, groups, H, W (batch 2): at least 1024 output tiles
     (64, 64, 3, 1, 1, 1, 1, 256, 250),   # two channel tiles per wavefront, two reduction slices
     (64, 96, 3, 1, 1, 1, 1, 256, 256),   # two channel blocks
     (40, 64, 3, 1, 1, 1, 1, 250, 256),   # input channels that do not fill the second reduction step
     (56, 80, 3, 1, 1, 1, 1, 256, 250),   # a last channel block with one tile
+    (64, 64, 3, 1, 1, 1, 1, 192, 184),   # 1104 tiles: just above the threshold
 ]
 
 
@@ -450,7 +451,7 @@ def test_conv_resident_filter(lib, dtype, cfg, density):
     ((64, 64, 3, 1, 1, 1, 1, 72, 70), "conv_lds_mfma_kernel"),
     ((16, 64, 3, 1, 1, 1, 1, 120, 120), "conv_lds_mfma_kernel"),
     ((320, 32, 3, 1, 1, 1, 1, 40, 40), "conv_lds_mfma_kernel"),
-    ((64, 64, 3, 1, 1, 1, 1, 256, 250), "conv_res_mfma_kernel"),   # thin layers on >= 2048 tiles: resident filter
+    ((64, 64, 3, 1, 1, 1, 1, 256, 250), "conv_res_mfma_kernel"),   # thin layers on >= 1024 tiles: resident filter
     ((16, 32, 3, 2, 1, 1, 1, 520, 500), "conv_lds_mfma_kernel"),   # one channel step: the per-tile kernel stays
     ((64, 256, 1, 1, 0, 1, 1, 20, 20), "pw_mfma_kernel"),
     ((32, 32, 3, 1, 1, 1, 32, 15, 18), "conv_dw_kernel"),
