@@ -6,7 +6,7 @@
 // of input halo and 8 KB of output.  On a map of thousands of tiles that stream is most of the
 // kernel's traffic and time.  Here a workgroup is launched once per compute-unit slot and loops
 // over tiles (tile = blockIdx.x, blockIdx.x + gridDim.x, ...): the filter fragments of each
-// wavefront's reduction steps (at most RES_MAX_STEPS steps x R channel tiles) are loaded before
+// wavefront's reduction steps (RES_STEPS steps x R channel tiles) are loaded before
 // the loop and stay in registers, the step table is built once, and per tile only the mask words,
 // the halo and the outputs move.  The loop is a two-stage pipeline with ONE barrier per tile:
 // the mask words and halo rows of the NEXT tile are requested before the reduction of the current
@@ -33,7 +33,7 @@
 namespace dc {
 namespace {
 
-constexpr int RES_MAX_STEPS = 10;   // reduction steps per wavefront that stay in registers
+constexpr int RES_STEPS = 9;        // reduction steps per wavefront: their filter fragments stay in registers
 constexpr int RES_MAX_HALO = 512;   // halo pixels (two tables in LDS)
 constexpr int RES_MAX_TABLE = 96;   // reduction steps of a tile (taps x channel steps)
 
@@ -88,7 +88,7 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
 #pragma unroll
     for (int i = 0; i < NSW; ++i) {
         const int2 e = s_step[min(i * KS + kz, nsteps - 1)];
-        xoff[i] = e.x;
+        xoff[i] = __builtin_amdgcn_readfirstlane(e.x);  // the same in every lane of the wavefront
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const unsigned wfrag = (unsigned)min((cb * ncw + cw) * R + r, co_tiles - 1) * K2 * ksteps * 512 + lane * 8;
@@ -201,18 +201,29 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
             for (int r = 0; r < R; ++r)
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) acc[r][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+            // NSW steps for every wavefront (host: taps x channel steps == NSW * KS), one
+            // branch-free block; the input fragments of a step are read from LDS while the matrix
+            // instructions of the step before run
             auto reduce = [&](auto nta_tag) {
                 constexpr int NTA = decltype(nta_tag)::value;
+                E8 x[2][NTA];
+#pragma unroll
+                for (int nt = 0; nt < NTA; ++nt) x[0][nt] = *reinterpret_cast<const E8 *>(halo + hbase[nt] + xoff[0]);
 #pragma unroll
                 for (int i = 0; i < NSW; ++i) {
-                    if (i * KS + kz >= nsteps) break;  // wave-uniform
-                    E8 x[NTA];
+                    if (i + 1 < NSW) {
 #pragma unroll
-                    for (int nt = 0; nt < NTA; ++nt) x[nt] = *reinterpret_cast<const E8 *>(halo + hbase[nt] + xoff[i]);
+                        for (int nt = 0; nt < NTA; ++nt)
+                            x[(i + 1) & 1][nt] = *reinterpret_cast<const E8 *>(halo + hbase[nt] + xoff[i + 1]);
+                    }
+                    // the reads above are issued before the matrix instructions below: left to
+                    // itself the scheduler sinks every read to just before its use and waits for it
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int nt = 0; nt < NTA; ++nt)
 #pragma unroll
-                        for (int r = 0; r < R; ++r) acc[r][nt] = Elem16<E>::mfma(a[i][r], x[nt], acc[r][nt]);
+                        for (int r = 0; r < R; ++r) acc[r][nt] = Elem16<E>::mfma(a[i][r], x[i & 1][nt], acc[r][nt]);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             };
             switch (n_tiles) {
@@ -290,9 +301,9 @@ static hipError_t allow_lds(K *kernel) {
 
 // Layers the resident-filter kernel takes, given the arrangement conv_lds_mfma_kernel would use
 // (R channel tiles per wavefront, KS reduction slices, ncw channel groups, kcc channel steps per
-// LDS chunk): all input channels in one chunk of at least two steps, at most RES_MAX_STEPS
-// reduction steps per wavefront, LDS within the default limit, and enough tiles that walking
-// over them pays.
+// LDS chunk): 3 x 3 taps over two channel steps (33-64 input channels) with two channel tiles per
+// wavefront and two reduction slices, LDS for two workgroups per compute unit, and enough tiles
+// that walking over them pays.
 bool resident_conv_eligible(const dc_geometry &g, int hal_h, int hal_w, int ltx, int lty, int kcc, int rl,
                             int ksl, int ncw) {
     const int ksteps = (g.in_c + 31) / 32;
@@ -300,12 +311,14 @@ bool resident_conv_eligible(const dc_geometry &g, int hal_h, int hal_w, int ltx,
     const int co_tiles = ceil_div(g.out_c, 16);
     const int cbl = ceil_div(co_tiles, ncw * rl);
     // Measured on 8 x 512 x 512 maps against conv_lds_mfma_kernel: 3 x 3 64 -> 64, whose filter takes
-    // two channel steps, 399 -> 289 us at full density and 345 -> 239 us at 10 %; no gain or a loss
+    // two channel steps, 399 -> 279 us at full density and 345 -> 224 us at 10 %; no gain or a loss
     // for a single channel step, whose filter of a few KB was never the cost (32 -> 64 stride 2:
     // 67 -> 70 us; 16 -> 16 on 544 x 960: 19.6 -> 22.8 us).
     if (kcc < 2) return false;
-    if (kcc != ksteps || nsteps > RES_MAX_TABLE || ceil_div(nsteps, ksl) > RES_MAX_STEPS) return false;
-    if (!((rl == 1 && ksl == 1) || (rl == 2 && ksl == 2))) return false;  // the arrangements that occur in this range
+    // the arrangement that occurs in this range: two channel tiles per wavefront, two reduction
+    // slices, nine steps each (3 x 3 taps x two channel steps); the reduction is one branch-free
+    // block of exactly that many steps
+    if (kcc != ksteps || nsteps > RES_MAX_TABLE || rl != 2 || ksl != 2 || nsteps != 2 * RES_STEPS) return false;
     const int hpx = hal_h * hal_w;
     if (hpx > RES_MAX_HALO) return false;
     // two workgroups per compute unit (with one, the form loses to the per-tile kernel: 64 -> 32 with
@@ -313,9 +326,7 @@ bool resident_conv_eligible(const dc_geometry &g, int hal_h, int hal_w, int ltx,
     if (resident_lds(hpx, kcc, rl, ksl, ncw) > (72u << 10)) return false;
     const int hstep = (ncw * ksl * WAVE) >> log2i(pow2_ceil(kcc * 4));
     const int su = ceil_div(hpx, hstep);  // halo rows a lane keeps in flight
-    const int nsw = ceil_div(nsteps, ksl);
-    // (instances that would spill registers are not offered)
-    if (su > 12 || (rl == 2 && su > (nsw > 5 ? 4 : 8))) return false;
+    if (su > 4) return false;  // (more halo rows in flight per lane would spill registers)
     // (offsets within one map of the batch are computed in 32 bits)
     if ((int64_t)g.in_h * g.in_w * g.in_c >= (1ll << 31) || (int64_t)g.out_h * g.out_w * g.out_c >= (1ll << 31)) return false;
     // (64 -> 64 on 136 x 240, 510 tiles per image: 10.4 against 9.9 us for one image, 15.3 against
@@ -343,32 +354,12 @@ static hipError_t resident_t(const dc_geometry &g, const ConvP &p, int hal_h, in
     const int per_cu = std::max(1, 8 / nwv);
     const int slots = 256 * per_cu;
     dim3 grid((unsigned)std::min(q.tiles, std::max(1, slots / cbl)), cbl);
-    const int nsw = ceil_div(g.kernel_h * g.kernel_w * kcc, ksl);
     note_kernel("conv_res_mfma_kernel");
-    const int su = ceil_div(hpx, (nwv * WAVE) >> q.lgv);
-#define DC_RES_S(RV, KV, NV, SV)                                                                             \
-    do {                                                                                                     \
-        const hipError_t big = allow_lds(&conv_res_mfma_kernel<E, RV, KV, NV, SV>);                          \
-        if (big != hipSuccess) return big;                                                                   \
-        conv_res_mfma_kernel<E, RV, KV, NV, SV><<<grid, nwv * WAVE, lds, s>>>(p, q, (const E *)in, (const E *)packed, \
-                                                                              (const E *)bias, (E *)out, mask, out_mask); \
-    } while (0)
-#define DC_RES(RV, KV, NV)                                                                                   \
-    do {                                                                                                     \
-        if (su <= 4) DC_RES_S(RV, KV, NV, 4);                                                                \
-        else if (su <= 8) DC_RES_S(RV, KV, NV, 8);                                                           \
-        else DC_RES_S(RV, KV, NV, 12);                                                                       \
-    } while (0)
-#define DC_RES_N(RV, KV)                                                                                     \
-    do {                                                                                                     \
-        if (nsw <= 5) DC_RES(RV, KV, 5);                                                                     \
-        else DC_RES(RV, KV, RES_MAX_STEPS);                                                                  \
-    } while (0)
-    if (rl == 1) DC_RES_N(1, 1);
-    else DC_RES_N(2, 2);
-#undef DC_RES_N
-#undef DC_RES
-#undef DC_RES_S
+    (void)rl;
+    const hipError_t big = allow_lds(&conv_res_mfma_kernel<E, 2, 2, RES_STEPS, 4>);
+    if (big != hipSuccess) return big;
+    conv_res_mfma_kernel<E, 2, 2, RES_STEPS, 4><<<grid, nwv * WAVE, lds, s>>>(p, q, (const E *)in, (const E *)packed,
+                                                                              (const E *)bias, (E *)out, mask, out_mask);
     return hipGetLastError();
 }
 
