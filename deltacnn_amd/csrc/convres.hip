@@ -39,7 +39,6 @@ constexpr int RES_MAX_TABLE = 96;   // reduction steps of a tile (taps x channel
 
 struct ResP {
     int ci_p, hal_h, hal_w, kcc, lgv;
-    int pitch;  // pixels per halo row in LDS (>= hal_w)
     int ltx, lty, tiles;  // tiles per row / column of a map, tiles in all (batch included)
 };
 
@@ -68,18 +67,17 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
     const int K2 = p.Kh * p.Kw;
     const int nsteps = K2 * ksteps;
     const int row = q.kcc * 64 + 16;  // bytes per staged halo pixel
-    const int halo_bytes = hal_h * q.pitch * row;
+    const int halo_bytes = hpx * row;
     unsigned char *s_part0 = s_dyn + 2 * halo_bytes;
     const int PART_BYTES = (KS - 1) * ncw * R * NT * WAVE * 16;  // (KS - 1) slices x ncw groups x R x NT tiles
-    auto tap_off = [&](int a, int b2) { return a * p.dh * hal_w + b2 * p.dw; };        // in the pixel table
-    auto tap_lds = [&](int a, int b2) { return a * p.dh * q.pitch + b2 * p.dw; };      // in the staged halo
+    auto tap_off = [&](int a, int b2) { return a * p.dh * hal_w + b2 * p.dw; };  // in halo pixels
 
     // step table: LDS byte offset of a step's input fragment relative to a pixel's halo origin
     // and its fragment offset in the packed filter; the same for every tile
     for (int j = tid; j < nsteps; j += nthr) {
         const int tap = j / ksteps, ks = j - tap * ksteps;
         const int ta = tap / p.Kw, tb = tap - ta * p.Kw;
-        s_step[j] = int2{tap_lds(ta, tb) * row + ks * 64, (tap * ksteps + ks) * 512};
+        s_step[j] = int2{tap_off(ta, tb) * row + ks * 64, (tap * ksteps + ks) * 512};
     }
     __syncthreads();
     // the wavefront's filter fragments, resident for the whole kernel
@@ -142,8 +140,7 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
             if (hp < hpx) {
                 if (sv == 0) s_hpix[buf][hp] = on ? hpixel[u] : -1;
                 if (sv < q.kcc * 4)
-                    *reinterpret_cast<E8 *>(halo + ((hyx[u] >> 16) * q.pitch + (hyx[u] & 0xffff)) * row + sv * 16) =
-                        keep8(val[u], vok && on);
+                    *reinterpret_cast<E8 *>(halo + hp * row + sv * 16) = keep8(val[u], vok && on);
             }
         }
     };
@@ -195,7 +192,7 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
             for (int nt = 0; nt < NT; ++nt) {
                 const int slot = nt * 16 + l16;
                 loc[nt] = slot < n ? s_wlist[wv][slot] : 0;
-                hbase[nt] = ((loc[nt] >> 3) * p.sh * q.pitch + (loc[nt] & 7) * p.sw) * row + kq * 16;
+                hbase[nt] = ((loc[nt] >> 3) * p.sh * hal_w + (loc[nt] & 7) * p.sw) * row + kq * 16;
             }
 #pragma unroll
             for (int r = 0; r < R; ++r)
@@ -346,7 +343,6 @@ static hipError_t resident_t(const dc_geometry &g, const ConvP &p, int hal_h, in
     q.hal_h = hal_h; q.hal_w = hal_w; q.kcc = kcc;
     q.lgv = log2i(pow2_ceil(kcc * 4));
     q.ltx = ltx; q.lty = lty; q.tiles = ltx * lty * g.batch;
-    q.pitch = hal_w;
     const size_t lds = resident_lds(hpx, kcc, rl, ksl, ncw);
     const int nwv = ncw * ksl;
     // workgroups per compute unit: what registers and LDS allow, so that the memory round trips

@@ -28,7 +28,7 @@ constexpr int PAIR_NW = 8;   // wavefronts per workgroup
 
 struct PairP {
     int P;                  // pixels
-    int Ch, ch_p, ksteps1;  // projection input channels, padded to 32, reduction steps
+    int Ch, ksteps1;        // projection input channels, reduction steps of 32
     int Cm, cm_tiles;       // block output channels (projection out = expansion in), tiles of 16
     int ksteps2;            // Cm / 32
     int Ce, ce_tiles;       // expansion output channels, tiles of 16
@@ -288,8 +288,7 @@ hipError_t launch_pointwise_pair(const dc_geometry &gp, const void *in, const in
     PairP p;
     p.P = gp.batch * gp.out_h * gp.out_w;
     p.Ch = gp.in_c;
-    p.ch_p = ceil_div(gp.in_c, 32) * 32;
-    p.ksteps1 = p.ch_p >> 5;
+    p.ksteps1 = ceil_div(gp.in_c, 32);
     p.Cm = gp.out_c;
     p.cm_tiles = ceil_div(p.Cm, 16);
     p.ksteps2 = p.Cm >> 5;
