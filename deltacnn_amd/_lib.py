@@ -64,6 +64,19 @@ class ProjectExpandArgs(ctypes.Structure):
         ("dw_geometry", POINTER(Geometry)), ("dw_activation", c_int32), ("dw_truncation_mode", c_int32)]
 
 
+class ConvItem(ctypes.Structure):
+    """struct dc_conv_item."""
+    _fields_ = [
+        ("geometry", Geometry), ("input", c_void_p), ("mask", c_void_p), ("packed_filter", c_void_p),
+        ("bias", c_void_p), ("out", c_void_p), ("out_mask", c_void_p),
+        ("residual", c_void_p), ("residual_mask", c_void_p), ("weight_residual", c_float), ("weight_conv", c_float),
+        ("sum_prev_out", c_void_p), ("sum_activation", c_int32),
+        ("prev_out", c_void_p), ("truncated", c_void_p), ("threshold", c_float), ("activation", c_int32),
+        ("truncation_mode", c_int32)]
+
+
+CONV_GROUP_MAX = 8
+
 _P = c_void_p
 _G = POINTER(Geometry)
 _SIGNATURES = {
@@ -78,6 +91,7 @@ _SIGNATURES = {
     "dc_block": (c_int, [_G, POINTER(BlockArgs), c_int, _P]),
     "dc_expand_depthwise": (c_int, [_G, POINTER(ExpandDwArgs), c_int, _P]),
     "dc_project_expand": (c_int, [_G, POINTER(ProjectExpandArgs), c_int, _P]),
+    "dc_conv_group": (c_int, [POINTER(ConvItem), c_int32, c_int, _P]),
     "dc_packed_filter_bytes": (c_int64, [_G, c_int, c_int]),
     "dc_pack_filter": (c_int, [_G, _P, _P, c_int, c_int, _P]),
     "dc_deconv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),

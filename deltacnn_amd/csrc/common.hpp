@@ -333,6 +333,34 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
                             const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
                             const ActEpilogue *epi, bool *epilogue_done, const Residual *res,
                             int dtype, hipStream_t s);
+
+// Independent small 3x3 layers launched together (dc_conv_group): each a plain convolution, a
+// convolution + residual sum (res) or a convolution + activation/truncation (epi).
+constexpr int CONV_GROUP_MAX = 8;
+struct ConvGroupItem {
+    dc_geometry g;
+    const void *in;
+    const int32_t *mask;
+    const void *packed, *bias;
+    void *out;
+    int32_t *out_mask;
+    const Residual *res;
+    const ActEpilogue *epi;
+};
+bool conv_group_item_eligible(const ConvGroupItem &c, int dtype);
+// the convolution kernel finishes the item's activation itself (otherwise it needs an ActGroupItem)
+bool conv_group_activation_fused(const ConvGroupItem &c);
+hipError_t launch_conv_group(const ConvGroupItem *items, int n, int dtype, hipStream_t s);
+
+// Activation / truncation (maximum norm) of several tensors in one launch.
+struct ActGroupItem {
+    void *delta, *prev, *trunc;
+    int32_t *mask;
+    float thr;
+    int32_t P, C;
+};
+bool act_group_eligible(const ActGroupItem *items, int n, int act, int mode, int dtype);
+hipError_t launch_activate_truncate_group(const ActGroupItem *items, int n, int act, int dtype, hipStream_t s);
 hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *packed, int dtype,
                               bool transposed, hipStream_t s);
 int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed);

@@ -508,6 +508,83 @@ int dc_project_expand(const dc_geometry *g, const dc_project_expand_args *args, 
                   "dc_project_expand");
 }
 
+int dc_conv_group(const dc_conv_item *items, int32_t count, int dtype, void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_conv_group");
+    DC_REQUIRE_PTR("dc_conv_group", items);
+    if (count < 2 || count > DC_CONV_GROUP_MAX)
+        return fail(DC_ERR_SHAPE, "dc_conv_group: count=%d outside 2..%d", count, int(DC_CONV_GROUP_MAX));
+    dc::ConvGroupItem conv[DC_CONV_GROUP_MAX];
+    dc::Residual res[DC_CONV_GROUP_MAX];
+    dc::ActEpilogue epi[DC_CONV_GROUP_MAX];
+    dc::ActGroupItem act[DC_CONV_GROUP_MAX];
+    int n_act = 0, act_kind = 0;
+    for (int i = 0; i < count; ++i) {
+        const dc_conv_item &it = items[i];
+        int rc = check_conv("dc_conv_group", &it.geometry, it.input, it.packed_filter, it.out, it.mask, it.out_mask,
+                            dtype, false);
+        if (rc != DC_OK) return rc;
+        DC_REQUIRE_ALIGNED("dc_conv_group", it.input, 16);
+        DC_REQUIRE_ALIGNED("dc_conv_group", it.packed_filter, 16);
+        DC_REQUIRE_ALIGNED("dc_conv_group", it.out, 8);
+        DC_REQUIRE_ALIGNED("dc_conv_group", it.bias, 8);
+        const dc_geometry &g = it.geometry;
+        conv[i] = dc::ConvGroupItem{g, it.input, it.mask, it.packed_filter, it.bias, it.out, it.out_mask, nullptr, nullptr};
+        if (it.residual != nullptr) {
+            if (it.prev_out != nullptr)
+                return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: item %d has a residual sum and an activation", i);
+            if (it.sum_activation < 0 || it.sum_activation > DC_ACT_SWISH)
+                return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: item %d: activation %d", i, it.sum_activation);
+            DC_REQUIRE_PTR("dc_conv_group", it.residual_mask);
+            if (it.sum_activation > 0) DC_REQUIRE_PTR("dc_conv_group", it.sum_prev_out);
+            DC_REQUIRE_ALIGNED("dc_conv_group", it.residual, 8);
+            DC_REQUIRE_ALIGNED("dc_conv_group", it.sum_prev_out, 8);
+            res[i] = dc::Residual{it.residual, it.residual_mask, it.weight_residual, it.weight_conv, it.sum_prev_out,
+                                  it.sum_activation};
+            conv[i].res = &res[i];
+        } else if (it.prev_out != nullptr) {
+            DC_REQUIRE_PTR("dc_conv_group", it.truncated);
+            if (it.activation > DC_ACT_SWISH || it.truncation_mode != DC_TRUNC_MAX)
+                return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: item %d: activation %d / truncation mode %d", i,
+                            it.activation, it.truncation_mode);
+            epi[i] = dc::ActEpilogue{it.prev_out, it.truncated, it.threshold, it.activation, it.truncation_mode};
+            conv[i].epi = &epi[i];
+        }
+        if (!dc::conv_group_item_eligible(conv[i], dtype))
+            return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: item %d is not a 16-bit 3x3 layer of the 4x4-patch kernel "
+                                            "(Cin %% 8 == 0, patches * channel tiles * steps <= 32768)", i);
+        if (conv[i].epi != nullptr && !dc::conv_group_activation_fused(conv[i])) {
+            const int kind = it.activation < 0 ? 0 : it.activation;
+            if (n_act > 0 && kind != act_kind)
+                return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: activations %d and %d in one group", act_kind, kind);
+            act_kind = kind;
+            act[n_act++] = dc::ActGroupItem{it.out, it.prev_out, it.truncated, it.out_mask, it.threshold,
+                                            g.batch * g.out_h * g.out_w, g.out_c};
+        }
+    }
+    // no item may write what another reads or writes
+    for (int i = 0; i < count; ++i)
+        for (int j = 0; j < count; ++j) {
+            if (i == j) continue;
+            const dc_conv_item &a = items[i], &b = items[j];
+            if (a.out == b.out || a.out == b.input || a.out == b.residual || a.out_mask == b.out_mask ||
+                a.out_mask == b.mask || a.out_mask == b.residual_mask ||
+                (a.prev_out != nullptr && (a.prev_out == b.prev_out || a.truncated == b.truncated)) ||
+                (a.sum_prev_out != nullptr && a.sum_prev_out == b.sum_prev_out))
+                return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: items %d and %d share a buffer one of them writes", i, j);
+        }
+    if (n_act > 1 && !dc::act_group_eligible(act, n_act, act_kind, DC_TRUNC_MAX, dtype))
+        return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: an activation outside the grouped kernel's range "
+                                        "(out_c %% 8 == 0, out_c <= 2048, tensor <= 1 MB, 16-byte aligned)");
+    hipError_t e = dc::launch_conv_group(conv, count, dtype, (hipStream_t)stream);
+    if (e == hipSuccess && n_act == 1)
+        e = dc::launch_activate_truncate(act[0].delta, act[0].prev, act[0].trunc, act[0].mask, act[0].thr, act_kind,
+                                         DC_TRUNC_MAX, act[0].P, act[0].C, dtype, (hipStream_t)stream);
+    else if (e == hipSuccess && n_act > 1)
+        e = dc::launch_activate_truncate_group(act, n_act, act_kind, dtype, (hipStream_t)stream);
+    return finish(e, "dc_conv_group");
+}
+
 int dc_pool_densify(const dc_geometry *g, const void *input, const int32_t *mask, void *prev_out,
                     void *out, int dtype, void *stream) {
     dc::kernel_log_reset();

@@ -135,6 +135,58 @@ act_trunc_vec_kernel(T *__restrict__ delta, T *__restrict__ prev, T *__restrict_
                                    T(thr_f), mode);
 }
 
+// The activation / truncation of several small tensors in one launch (the branches of a
+// multi-resolution network): a workgroup looks up the tensor its number falls into and runs the
+// eager form above on it.  Maximum norm only -- its keep decision does not depend on how the
+// channels of a pixel are spread over lanes, so the results are those of the separate launches.
+template <typename T>
+struct ActItemD {
+    T *delta, *prev, *trunc;
+    int32_t *mask;
+    float thr;
+    int P, C, lg, iters, first;
+};
+
+template <typename T>
+struct ActGroupD {
+    int n;
+    ActItemD<T> it[CONV_GROUP_MAX];
+};
+
+template <typename T, int ITERS, int ACT>
+__device__ __forceinline__ void act_trunc_group_item(const ActItemD<T> &it, int gid) {
+    constexpr int N = Vec16<T>::N;
+    const int G = 1 << it.lg, P = it.P, C = it.C;
+    const int p = gid >> it.lg, gl = gid & (G - 1);
+    Vec<T, N> dl[ITERS], q[ITERS], tr[ITERS];
+    const size_t row = (size_t)min(p, P - 1) * C;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+        const int c = min((i * G + gl) * N, C - N);
+        dl[i] = vload<T, N>(it.delta + row + c);
+        q[i] = vload<T, N>(it.prev + row + c);
+        tr[i] = vload<T, N>(it.trunc + row + c);
+    }
+    const bool valid = p < P && it.mask[min(p, P - 1)] != 0;
+    if (ballot(valid) == 0) return;
+    act_trunc_pixel<T, ITERS, ACT>(dl, q, tr, valid, (size_t)p, gl, G, C, it.delta, it.prev, it.trunc, it.mask,
+                                   T(it.thr), DC_TRUNC_MAX);
+}
+
+template <typename T, int ACT>
+__global__ void __launch_bounds__(256)
+act_trunc_group_kernel(ActGroupD<T> g) {
+    int idx = 0;
+#pragma unroll
+    for (int i = 1; i < CONV_GROUP_MAX; ++i)
+        if (i < g.n && (int)blockIdx.x >= g.it[i].first) idx = i;
+    const ActItemD<T> &it = g.it[idx];
+    const int gid = (blockIdx.x - it.first) * 256 + threadIdx.x;
+    if (it.iters == 1) act_trunc_group_item<T, 1, ACT>(it, gid);
+    else if (it.iters == 2) act_trunc_group_item<T, 2, ACT>(it, gid);
+    else act_trunc_group_item<T, 4, ACT>(it, gid);
+}
+
 // Large maps: a wavefront scans the mask words of 64 consecutive pixels in one coalesced read,
 // compacts the active ones by ballot and then works through them 64 / G pixels at a time.  With
 // one group per pixel a sparse map costs a wavefront launch per 64 / G pixels, most of which
@@ -957,6 +1009,63 @@ hipError_t launch_activate_truncate(void *delta, void *prev, void *trunc, int32_
     if (dtype == DC_BF16)
         return act_trunc_t<bf16_t>((bf16_t *)delta, (bf16_t *)prev, (bf16_t *)trunc, mask, thr, act, mode, P, C, s);
     return act_trunc_t<half_t>((half_t *)delta, (half_t *)prev, (half_t *)trunc, mask, thr, act, mode, P, C, s);
+}
+
+// 16-byte rows, at most four vectors per lane of a 64-lane group, tensors of at most 1 MB (the
+// eager form reads every pixel's row).
+bool act_group_eligible(const ActGroupItem *items, int n, int act, int mode, int dtype) {
+    if (n < 1 || n > CONV_GROUP_MAX || mode != DC_TRUNC_MAX || act > DC_ACT_SWISH) return false;
+    if (dtype != DC_F16 && dtype != DC_BF16) return false;
+    for (int i = 0; i < n; ++i) {
+        const ActGroupItem &a = items[i];
+        if (a.P <= 0 || a.C <= 0 || a.C % 8 != 0 || a.C / 8 > WAVE * 4) return false;
+        if ((int64_t)a.P * a.C * 2 > (1 << 20)) return false;
+        for (const void *q : {(const void *)a.delta, (const void *)a.prev, (const void *)a.trunc})
+            if (q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15u) != 0) return false;
+        if (a.mask == nullptr) return false;
+    }
+    return true;
+}
+
+namespace {
+template <typename T>
+hipError_t act_group_t(const ActGroupItem *items, int n, int act, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    ActGroupD<T> ag;
+    ag.n = n;
+    int blocks = 0;
+    for (int i = 0; i < n; ++i) {
+        const ActGroupItem &a = items[i];
+        ActItemD<T> &it = ag.it[i];
+        const int nvec = a.C / N;
+        const int G = pick_group(nvec, a.P, 4);
+        it.delta = (T *)a.delta; it.prev = (T *)a.prev; it.trunc = (T *)a.trunc; it.mask = a.mask;
+        it.thr = a.thr; it.P = a.P; it.C = a.C;
+        it.lg = log2i(G);
+        const int iters = ceil_div(nvec, G);
+        it.iters = iters <= 1 ? 1 : iters <= 2 ? 2 : 4;
+        it.first = blocks;
+        blocks += (int)ceil_div64((int64_t)a.P * G, 256);
+    }
+    for (int i = n; i < CONV_GROUP_MAX; ++i) ag.it[i] = ag.it[0];
+    note_kernel("act_trunc_group_kernel");
+    const dim3 grid((unsigned)blocks);
+    if (act < 0) act = 0;
+    switch (act) {
+        case DC_ACT_RELU: act_trunc_group_kernel<T, DC_ACT_RELU><<<grid, 256, 0, s>>>(ag); break;
+        case DC_ACT_RELU6: act_trunc_group_kernel<T, DC_ACT_RELU6><<<grid, 256, 0, s>>>(ag); break;
+        case DC_ACT_LEAKY: act_trunc_group_kernel<T, DC_ACT_LEAKY><<<grid, 256, 0, s>>>(ag); break;
+        case DC_ACT_SIGMOID: act_trunc_group_kernel<T, DC_ACT_SIGMOID><<<grid, 256, 0, s>>>(ag); break;
+        case DC_ACT_SWISH: act_trunc_group_kernel<T, DC_ACT_SWISH><<<grid, 256, 0, s>>>(ag); break;
+        default: act_trunc_group_kernel<T, DC_ACT_LINEAR><<<grid, 256, 0, s>>>(ag); break;
+    }
+    return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_activate_truncate_group(const ActGroupItem *items, int n, int act, int dtype, hipStream_t s) {
+    if (dtype == DC_BF16) return act_group_t<bf16_t>(items, n, act, s);
+    return act_group_t<half_t>(items, n, act, s);
 }
 
 template <typename T>

@@ -313,6 +313,59 @@ def sparse_project_expand(x, mask, project_packed, project_geometry, residual, r
     return True
 
 
+def sparse_conv_group(items) -> bool:
+    """Independent small 3x3 layers in ONE launch (``dc_conv_group``), plus one for the
+    activations that their convolutions cannot finish themselves.  ``items``: 2 .. 8 dicts with
+    ``x, mask, packed_filter, geometry, out, out_mask`` (and optionally ``bias``) and at most one of
+    ``residual = (values, mask, weight_residual, weight_conv, prev_out or None, activation)`` --
+    the operands of :func:`sparse_conv_add` -- and ``activation = (prev_out, truncated, threshold,
+    activation, truncation_mode)`` -- those of :func:`sparse_conv_activation`.  Every item's
+    results are identical, bit for bit, to the separate call's.  Returns ``False`` (nothing
+    launched) when the group has no such form."""
+    lib = _lib.load()
+    n = len(items)
+    if n < 2 or n > _lib.CONV_GROUP_MAX:
+        return False
+    dtype = items[0]["x"].dtype
+    if dtype not in (torch.float16, torch.bfloat16):
+        return False
+    arr = (_lib.ConvItem * n)()
+    metas, keep = [], []
+    for a, it in zip(arr, items):
+        x, packed = _nhwc(it["x"], "x"), it["packed_filter"]
+        if packed is None or x.dtype != dtype:
+            return False
+        a.geometry = it["geometry"]
+        a.input, a.mask, a.packed_filter = x.data_ptr(), _mask(it["mask"], "mask").data_ptr(), packed.data_ptr()
+        a.bias = _ptr(it.get("bias"))
+        a.out, a.out_mask = it["out"].data_ptr(), it["out_mask"].data_ptr()
+        meta = dict(g=it["geometry"], in_mask=it["mask"], in_mask_b=None, out_mask=it["out_mask"], kind="conv")
+        res, act = it.get("residual"), it.get("activation")
+        if res is not None:
+            values, rmask, wa, wb, prev, activation = res
+            a.residual, a.residual_mask = _nhwc(values, "residual").data_ptr(), _mask(rmask, "residual mask").data_ptr()
+            a.weight_residual, a.weight_conv = float(wa), float(wb)
+            a.sum_prev_out, a.sum_activation = _ptr(prev), max(int(activation), 0)
+            meta.update(kind="conv_add", in_mask_b=rmask)
+            keep.append((values, prev))
+        elif act is not None:
+            prev, truncated, threshold, activation, mode = act
+            a.prev_out, a.truncated = prev.data_ptr(), _ptr(truncated)
+            a.threshold, a.activation, a.truncation_mode = float(threshold), int(activation), int(mode)
+            meta.update(kind="conv_act")
+            keep.append((prev, truncated))
+        metas.append(meta)
+        keep.append((x, packed, it.get("bias")))
+    try:
+        _call("conv_group", lib.dc_conv_group, (arr, n, _DTYPES[dtype], _stream()), items=metas,
+              esize=items[0]["x"].element_size(), keep=(arr, keep))
+    except _lib.DeltaCNNError as e:
+        if e.code == -3:
+            return False
+        raise
+    return True
+
+
 def sparse_deconv(x, filter, mask=None, bias=None, stride=(1, 1), padding=(0, 0), dilation=(1, 1),
                   groups=1, c_out: int = None, create_out_mask=False, sub_tile_sparsity=True,
                   out_mask=None, out_shape=None, *, packed_filter=None, out=None, geometry=None):

@@ -420,6 +420,8 @@ class _HRModule(nn.Module):
     def __init__(self, L, channels, blocks=4, multi_scale_output=True):
         super().__init__()
         n = len(channels)
+        self._conv_group = getattr(L, "conv_group", None)
+        self._residual_group = getattr(L, "residual_group", None)
         self.branches = nn.ModuleList(
             nn.Sequential(*[_BasicBlock(L, c, c) for _ in range(blocks)]) for c in channels)
         n_out = n if multi_scale_output else 1
@@ -442,8 +444,21 @@ class _HRModule(nn.Module):
             self.adds.append(nn.ModuleList(L.DCAdd(activation="relu" if k == n - 2 else None)
                                            for k in range(n - 1)))
 
+    def _run_branches(self, xs):
+        """The branches side by side: block k of every branch before block k + 1 of any, so that
+        a layer namespace with ``conv_group`` / ``residual_group`` can launch the same layer of
+        all branches together.  On a model's first frame -- layers take their numbers in call
+        order -- and for namespaces without those functions: branch after branch."""
+        steady = all(getattr(m, "frame_idx", 0) >= 0 for b in self.branches for m in b.modules())
+        if self._conv_group is None or not steady or len(self.branches) < 2:
+            return [b(x) for b, x in zip(self.branches, xs)]
+        for blocks in zip(*self.branches):
+            mids = self._conv_group([blk.conv1 for blk in blocks], xs)
+            xs = self._residual_group([blk.add for blk in blocks], xs, [blk.conv2 for blk in blocks], mids)
+        return xs
+
     def forward(self, xs):
-        xs = [b(x) for b, x in zip(self.branches, xs)]
+        xs = self._run_branches(xs)
         outs = []
         for row, adds in zip(self.fuse, self.adds):
             y = row[0](xs[0])

@@ -375,6 +375,7 @@ class DCConv2d(_DeltaConvBase, nn.Conv2d, DCModule):
     fuse_expansion = True  # expand_depthwise(): 1x1 expansion + activation -> depthwise 3x3 + activation in two launches
     fuse_projection = True  # project_expand(): projection (+ residual sum) + next expansion (left open) in one launch
     fuse_blocks = True  # fused_block(): depthwise -> projection (-> expansion) in one launch
+    fuse_groups = True  # conv_group() / residual_group(): the same layer of several parallel branches in one launch
     # ... while the two 1x1 filters together stay below this many bytes: every 16-pixel workgroup
     # of that launch reads both in full, and one compute unit pulls only a few GB/s out of the
     # far caches, so larger layers are faster as separate launches that spread their filter over
@@ -759,6 +760,91 @@ def fused_block(dw_input, depthwise, project, add=None, residual=None, expand=No
         DCConv2d.conv_idx += 1  # what the layers' own forward calls would have counted
         conv.frame_idx += 1
     return (out, out_mask), ((ex[6], ex[7]) if ex is not None else None)
+
+
+def _group_ready(conv, input) -> bool:
+    """A 16-bit delta convolution past its first frame (no bias any more) on a delta input."""
+    return (DCConv2d.fuse_groups and isinstance(conv, DCConv2d) and conv.backend == DCBackend.deltacnn
+            and conv.frame_idx >= 0 and conv.filters_processed and not conv.dense_out
+            and conv.weight.dtype in (torch.float16, torch.bfloat16) and not isinstance(input, Tensor))
+
+
+def _group_item(conv, input):
+    """The convolution part of a dc_conv_group item, or None if the layer has no packed filter."""
+    x, mask, plan, packed, _, _ = conv._prepare(input)
+    if packed is None:
+        return None, None
+    g = plan["g"]
+    return dict(x=x, mask=mask, packed_filter=packed, geometry=g), plan
+
+
+def conv_group(convs, inputs):
+    """``[conv(x) for conv, x in zip(convs, inputs)]`` for layers that do not depend on each other
+    -- the same layer of several parallel branches -- as ONE launch (+ one for the activations the
+    convolution kernel cannot finish) where ``dc_conv_group`` takes them; the separate layer calls
+    otherwise.  Results are identical either way.  Switch: ``DCConv2d.fuse_groups``."""
+    items, results = [], []
+    ok = len(convs) >= 2 and all(_group_ready(c, x) for c, x in zip(convs, inputs))
+    if ok:
+        for conv, x in zip(convs, inputs):
+            item, plan = _group_item(conv, x)
+            act = conv.activation_layer
+            if item is None or (conv.activation is not None and (_steady_activation(conv) is None
+                                                                 or not DCConv2d.fuse_activation)):
+                ok = False
+                break
+            g = plan["g"]
+            out = plan["out"] if plan["out"] is not None else hk.new_features(
+                g.batch, g.out_c, g.out_h, g.out_w, item["x"].dtype, item["x"].device)
+            out_mask = plan["out_mask"] if plan["out_mask"] is not None else hk.new_mask(
+                g.batch, g.out_h, g.out_w, item["x"].device)
+            item.update(out=out, out_mask=out_mask)
+            if act is not None:
+                item["activation"] = (act.prev_out, act.out_truncated, DCThreshold.get(act), act.activation_int,
+                                      act.truncation_mode.value)
+            items.append(item)
+            results.append((out, out_mask))
+    if ok and hk.sparse_conv_group(items):
+        for conv in convs:
+            DCConv2d.conv_idx += 1
+            conv.frame_idx += 1
+        return results
+    return [conv(x) for conv, x in zip(convs, inputs)]
+
+
+def residual_group(adds, residuals, convs, conv_inputs):
+    """``[add(r, conv(x)) for ...]`` for independent (DCAdd, residual, convolution without
+    activation, input) quadruples -- the block ends of several parallel branches -- as ONE
+    launch where ``dc_conv_group`` takes them; ``add.after_conv`` per branch otherwise.  Results
+    are identical either way.  Switch: ``DCConv2d.fuse_groups``."""
+    items, results = [], []
+    ok = len(convs) >= 2 and DCAdd.fuse_into_conv and all(
+        _group_ready(c, x) and c.activation is None and not isinstance(r, Tensor) and not a.first_iter
+        and not a.dense_out for a, r, c, x in zip(adds, residuals, convs, conv_inputs))
+    if ok:
+        for add, res, conv, x in zip(adds, residuals, convs, conv_inputs):
+            item, plan = _group_item(conv, x)
+            val, mask = res
+            g = plan["g"] if plan is not None else None
+            if item is None or tuple(val.shape) != (g.batch, g.out_c, g.out_h, g.out_w):
+                ok = False
+                break
+            if not _matches(add.out, val):
+                add.out = torch.empty_like(val)
+            if not _matches(add.mask_out, mask):
+                add.mask_out = torch.empty_like(mask)
+            with_act = add.activation is not None
+            item.update(out=add.out, out_mask=add.mask_out,
+                        residual=(val, mask, add.weight_a, add.weight_b, add.prev_out if with_act else None,
+                                  add.activation_int if with_act else 0))
+            items.append(item)
+            results.append((add.out, add.mask_out))
+    if ok and hk.sparse_conv_group(items):
+        for conv in convs:
+            DCConv2d.conv_idx += 1
+            conv.frame_idx += 1
+        return results
+    return [a.after_conv(r, c, x) for a, r, c, x in zip(adds, residuals, convs, conv_inputs)]
 
 
 class DCConcatenate(DCModule):

@@ -56,6 +56,10 @@ class Tracer:
 
     def run(self, op, fn, args, meta):
         rec = {"op": op, "meta": meta}
+        if op == "conv_group":  # one set of counts per layer of the group
+            rec["items"] = [{"n_in": self._count(i["in_mask"]), "n_in_b": self._count(i["in_mask_b"]),
+                             "pairs": self._pairs(i["g"], i["in_mask"], False) if self.count_pairs else None}
+                            for i in meta["items"]]
         rec["n_in"] = self._count(meta.get("in_mask"))
         rec["n_in_b"] = self._count(meta.get("in_mask_b"))
         if self.count_pairs and op in ("conv", "deconv", "conv_act", "conv_add", "block"):
@@ -70,6 +74,8 @@ class Tracer:
         rec["kernels"] = _lib.load().dc_last_kernels().decode().split("+")
         rec["n_out"] = self._count(meta.get("out_mask"))
         rec["n_ex"] = self._count(meta.get("ex_mask"))
+        for it, im in zip(rec.get("items", []), meta.get("items", [])):
+            it["n_out"] = self._count(im["out_mask"])
         if op == "pool" and meta.get("mode") == 0:
             rec["n_cov"] = self._covered(meta["g"], meta["out_mask"])
         rec["call"] = (fn, args)
@@ -127,6 +133,18 @@ class Tracer:
                 times[i] = max(timed([pcall, call]) - timed([pcall]), 0.0)
             else:
                 times[i] = timed([call])
+            if rec["op"] == "conv_group" and len(rec["kernels"]) == 2:
+                # the grouped convolution on its own: the same items without the activations that
+                # need the second launch; that launch gets the remainder
+                fn, a = rec["call"]
+                items = a[0]
+                bare = type(items)(*items)
+                for it, needs_second in zip(bare, self._second_launch(rec)):
+                    if needs_second:
+                        it.prev_out = None
+                t_conv = min(timed([("conv_group", fn, (bare,) + tuple(a[1:]))]), times[i])
+                rec["split_us"] = [t_conv, times[i] - t_conv]
+                rec["bare"] = bare
             if rec["op"] == "conv_act" and len(rec["kernels"]) == 2:
                 # the convolution launch of a two-launch call on its own: dc_conv with the same
                 # operands runs the same kernel; the activation kernel gets the remainder
@@ -135,6 +153,22 @@ class Tracer:
                 t_conv = min(timed([conv_only]), times[i])
                 rec["split_us"] = [t_conv, times[i] - t_conv]
         return times
+
+    @staticmethod
+    def _second_launch(rec):
+        """Per item of a conv_group record: does its activation run in the group's second launch
+        (the convolution kernel finishes it only where one wavefront holds all output channels of
+        a pixel: up to 32 channels and a reduction of at most 12 steps)."""
+        flags = []
+        for im in rec["meta"]["items"]:
+            g = im["g"]
+            steps = g.kernel_h * g.kernel_w * ((g.in_c + 31) // 32)
+            patches = ((g.out_w + 3) // 4) * ((g.out_h + 3) // 4) * g.batch
+            tiles = (g.out_c + 15) // 16
+            rv = 2 if tiles >= 2 and patches * tiles >= 512 else 1
+            one_wave = steps <= 12 and (tiles + rv - 1) // rv == 1 and g.out_c % 4 == 0
+            flags.append(im["kind"] == "conv_act" and not one_wave)
+        return flags
 
     @staticmethod
     def _covered(g, out_mask):
@@ -200,6 +234,40 @@ class Tracer:
                     extra = {"kernel": r["kernels"][1], "call": op, "shape": f"C{C} P{p_out}", "ms": t_act * 1e-3,
                              "bytes": p_out * m + n_mid * 3 * C * s + n_out * 3 * C * s + (n_mid - n_out) * (C * s + m),
                              "flops": 0, "density_in": n_mid / p_out, "density_out": n_out / p_out}
+            elif op == "conv_group":  # the conv / conv_add / conv_act formulas above, summed over the layers
+                rd = wr = 0
+                act_bytes = act_in = act_out = act_px = 0
+                second = self._second_launch(r)
+                p_in_all = p_out_all = n_in_all = n_out_all = 0
+                names = []
+                for it, im, late in zip(r["items"], meta["items"], second):
+                    g = im["g"]
+                    p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
+                    ni, no = int(it["n_in"]), int(it["n_out"])
+                    n_mid = int(it["pairs"][1]) if it["pairs"] is not None else no
+                    rd += p_in * m + ni * g.in_c * s + 9 * g.in_c * g.out_c * s
+                    wr += (n_mid if late else no) * g.out_c * s + p_out * m
+                    if im["kind"] == "conv_add":
+                        rd += p_out * m + int(it["n_in_b"]) * g.out_c * s
+                    if im["kind"] == "conv_act" and not late:
+                        rd += n_mid * 2 * g.out_c * s
+                        wr += no * 2 * g.out_c * s + (n_mid - no) * g.out_c * s
+                    if late:
+                        C = g.out_c
+                        act_bytes += p_out * m + n_mid * 3 * C * s + no * 3 * C * s + (n_mid - no) * (C * s + m)
+                        act_in, act_out, act_px = act_in + n_mid, act_out + no, act_px + p_out
+                    if it["pairs"] is not None:
+                        flops += 2 * g.in_c * g.out_c * int(it["pairs"][0])
+                    p_in_all, p_out_all, n_in_all, n_out_all = p_in_all + p_in, p_out_all + p_out, n_in_all + ni, n_out_all + no
+                    names.append(f"{g.in_c}->{g.out_c}@{g.in_h}x{g.in_w}")
+                kinds = {im["kind"] for im in meta["items"]}
+                shape = f"{'/'.join(sorted(kinds))} k3 x{len(names)}: " + " ".join(names)
+                dens = (n_in_all / p_in_all, n_out_all / p_out_all)
+                if len(r["kernels"]) == 2:
+                    t_conv, t_act = r.get("split_us", [ms * 1e3 / 2, ms * 1e3 / 2])
+                    ms = t_conv * 1e-3
+                    extra = {"kernel": r["kernels"][1], "call": op, "shape": f"x{sum(second)} P{act_px}", "ms": t_act * 1e-3,
+                             "bytes": act_bytes, "flops": 0, "density_in": act_in / act_px, "density_out": act_out / act_px}
             elif op == "block":
                 g = meta["g"]
                 ch, cp, ce = g.in_c, meta["Cp"], meta["Ce"]

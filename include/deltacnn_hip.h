@@ -267,6 +267,45 @@ typedef struct dc_project_expand_args {
  * types; no bias.  No counterpart in the reference (sparse_layers.py:636-638). */
 int dc_project_expand(const dc_geometry *g, const dc_project_expand_args *args, int dtype, void *stream);
 
+/* One layer of a dc_conv_group call. */
+typedef struct dc_conv_item {
+    dc_geometry geometry;           /* 3x3 convolution, groups == 1 */
+    const void *input;              /* [B][in_h][in_w][in_c] delta */
+    const int32_t *mask;            /* its update mask */
+    const void *packed_filter;      /* from dc_pack_filter */
+    const void *bias;               /* [out_c] or NULL */
+    void *out;                      /* [B][out_h][out_w][out_c] */
+    int32_t *out_mask;              /* [B][out_h][out_w] */
+    /* the residual sum of dc_conv_add behind the convolution; residual == NULL: none */
+    const void *residual;
+    const int32_t *residual_mask;
+    float weight_residual, weight_conv;
+    void *sum_prev_out;             /* accumulated sum of a DCAdd with activation (sum_activation > 0) */
+    int32_t sum_activation;
+    /* the activation / truncation of dc_conv_act behind the convolution; prev_out == NULL: none.
+     * Not together with a residual sum. */
+    void *prev_out;
+    void *truncated;
+    float threshold;
+    int32_t activation;
+    int32_t truncation_mode;        /* DC_TRUNC_MAX */
+} dc_conv_item;
+
+enum { DC_CONV_GROUP_MAX = 8 };
+
+/* 2 .. DC_CONV_GROUP_MAX independent small 3x3 layers -- the parallel branches of a
+ * multi-resolution network, whose layers the reference (and dc_conv / dc_conv_act / dc_conv_add)
+ * launch one after the other -- in ONE launch, plus one more for the activation / truncation of
+ * those items whose convolution cannot finish it itself.  Each item is what one call of dc_conv,
+ * dc_conv_act or dc_conv_add would be given, and its results are identical, bit for bit, to that
+ * call's.  The items must not depend on each other (no item's output or state is another's
+ * operand).  Accepted: 16-bit types, 3x3 kernels on layers small enough for the library's
+ * 4x4-patch kernel, activations with maximum-norm truncation, all of one kind where they need
+ * the second launch; anything else returns DC_ERR_UNSUPPORTED before any launch so that the
+ * caller can issue the separate calls.  No counterpart in the reference
+ * (sparse_layers.py:425-470 runs one layer per call). */
+int dc_conv_group(const dc_conv_item *items, int32_t count, int dtype, void *stream);
+
 /* Number of bytes dc_pack_filter writes for this geometry (0 if the shape has no packed
  * form).  One-time weight relayout for the MFMA kernels, fp16 or bfloat16, un-swizzled, in fragment order
  * [Cout tile of 16][Kh][Kw][Cin step of 32][lane 0..63][8] (lane kq*16+r holds input channels

@@ -357,3 +357,53 @@ def test_project_expand_arguments_are_checked_before_any_launch(lib):
     assert lib.dc_expand_depthwise(ctypes.byref(gd), ctypes.byref(b), 1, None) == -4
     b.expand_truncated, b.dw_truncated = p, p + 8
     assert lib.dc_expand_depthwise(ctypes.byref(gd), ctypes.byref(b), 1, None) == -5
+
+
+def test_conv_group_arguments_are_checked_before_any_launch(lib):
+    """dc_conv_group: a count outside 2..8 -> -2; an item the 4x4-patch kernel does not take, an
+    item with both a residual sum and an activation, activations of two kinds for the second
+    launch, items that share a buffer one of them writes -> -3 (the caller issues the separate
+    calls); missing operands -> -4; misaligned pointers -> -5; nothing touches a device."""
+    from deltacnn_amd._lib import ConvItem
+    buf = (ctypes.c_char * 65536)()
+    base = (ctypes.addressof(buf) + 255) // 256 * 256
+
+    def item(k, geom=None, **kw):
+        it = ConvItem()
+        it.geometry = geom if geom is not None else _geom(in_h=16, in_w=16, out_h=16, out_w=16, in_c=64, out_c=64)
+        p = base + k * 4096  # every item its own buffers
+        for j, name in enumerate(("input", "mask", "packed_filter", "out", "out_mask")):
+            setattr(it, name, p + j * 256)
+        it.weight_residual = it.weight_conv = 1.0
+        for name, v in kw.items():
+            setattr(it, name, v)
+        return it
+
+    def call(items, dtype=1, count=None):
+        arr = (ConvItem * len(items))(*items)
+        return lib.dc_conv_group(arr, len(items) if count is None else count, dtype, None)
+
+    def act(k, a=1):
+        p = base + k * 4096
+        return dict(prev_out=p + 2048, truncated=p + 2304, threshold=0.05, activation=a, truncation_mode=0)
+
+    assert call([item(0), item(1)], dtype=9) == -1
+    assert call([item(0), item(1)], dtype=0) == -3                          # fp32
+    assert call([item(0)]) == -2 and call([item(k) for k in range(9)]) == -2
+    assert lib.dc_conv_group(None, 2, 1, None) == -4
+    assert call([item(0), item(1, out=None)]) == -4
+    assert call([item(0), item(1, input=base + 4096 + 2)]) == -5
+    big = _geom(in_h=136, in_w=240, out_h=136, out_w=240, in_c=64, out_c=64)
+    assert call([item(0), item(1, geom=big)]) == -3 and b"item 1" in lib.dc_last_error()
+    one = _geom(in_h=16, in_w=16, out_h=16, out_w=16, in_c=64, out_c=64, kernel_h=1, kernel_w=1, pad_top=0, pad_left=0,
+                pad_bottom=0, pad_right=0)
+    assert call([item(0, geom=one), item(1)]) == -3                          # the pointwise kernels' layer
+    both = dict(act(1), residual=base + 4096 + 1024, residual_mask=base + 4096 + 1280)
+    assert call([item(0), item(1, **both)]) == -3 and b"residual sum and an activation" in lib.dc_last_error()
+    assert call([item(0, **act(0)), item(1, **dict(act(1), truncation_mode=1))]) == -3   # norm truncation
+    assert call([item(0, **act(0)), item(1, **dict(act(1), truncated=None))]) == -4
+    assert call([item(0, **act(0, 1)), item(1, **act(1, 3))]) == -3 and b"activations" in lib.dc_last_error()
+    assert call([item(0), item(1, out=base + 3 * 256)]) == -3 and b"share" in lib.dc_last_error()
+    assert call([item(0), item(1, input=base + 3 * 256)]) == -3            # item 1 reads what item 0 writes
+    assert call([item(0, residual=base + 1024)]) == -2                       # still one item
+    assert call([item(0), item(1, residual=base + 4096 + 1024)]) == -4       # a residual needs its mask
