@@ -2354,7 +2354,15 @@ PatchPlan patch_plan(const dc_geometry &g) {
     const int64_t patches = (int64_t)ceil_div(g.out_w, 4) * ceil_div(g.out_h, 4) * g.batch;
     PatchPlan pp;
     pp.kwv = steps <= 12 ? 1 : steps <= 48 ? 4 : 8;
-    pp.rv = (co_tiles >= 2 && patches * co_tiles >= 512) ? 2 : 1;
+    // Two channel tiles per wavefront (they are independent: the summation order of an output does
+    // not depend on it) halve the workgroups and the input reads: on many patches; for reductions
+    // split over wavefronts while a workgroup's filter slice stays below 40 KB (measured on 64 -> 64
+    // ... 256, 64 .. 1024 patches: 4.4 - 4.6 -> 3.7 - 3.9 us; with 128 input channels it loses); and
+    // where it puts all channels of a 32-channel layer into one wavefront, which can then finish
+    // the layer's activation itself (3.8 + 2.0 -> 4.4 us; without an activation it costs 0.3 us).
+    pp.rv = 1;
+    if (co_tiles >= 2 && (patches * co_tiles >= 512 || (pp.kwv >= 4 && g.in_c <= 64) || (pp.kwv == 1 && co_tiles == 2)))
+        pp.rv = 2;
     pp.cbk = ceil_div(co_tiles, pp.rv);
     return pp;
 }

@@ -163,10 +163,7 @@ class Tracer:
         for im in rec["meta"]["items"]:
             g = im["g"]
             steps = g.kernel_h * g.kernel_w * ((g.in_c + 31) // 32)
-            patches = ((g.out_w + 3) // 4) * ((g.out_h + 3) // 4) * g.batch
-            tiles = (g.out_c + 15) // 16
-            rv = 2 if tiles >= 2 and patches * tiles >= 512 else 1
-            one_wave = steps <= 12 and (tiles + rv - 1) // rv == 1 and g.out_c % 4 == 0
+            one_wave = steps <= 12 and g.out_c <= 32 and g.out_c % 4 == 0
             flags.append(im["kind"] == "conv_act" and not one_wave)
         return flags
 
