@@ -15,6 +15,8 @@ m = 4-byte mask word, P pixels, n_x = number of active pixels of mask x):
                      truncation; conv_act in two launches: a conv row and an activate_truncate row)
                      flops = 2*(Cin/g)*Cout*N_pairs, N_pairs = sum over updated outputs of the
                      active inputs in their window (computed exactly from the masks)
+                     (conv_group: the conv / conv_add / conv_act terms of its layers added up, one row
+                     for the grouped convolution launch and one for the grouped activation launch)
   pool               R = P_in*m + n_in*C*s [max: + n_cov*C*s]   W = n_out*C*s + P_out*m
                      (the maximum of an updated window needs the cached input of EVERY pixel of the
                      window, updated or not: n_cov = input pixels covered by updated windows)
