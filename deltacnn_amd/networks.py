@@ -447,31 +447,53 @@ class _HRModule(nn.Module):
     def _run_branches(self, xs):
         """The branches side by side: block k of every branch before block k + 1 of any, so that
         a layer namespace with ``conv_group`` / ``residual_group`` can launch the same layer of
-        all branches together.  On a model's first frame -- layers take their numbers in call
-        order -- and for namespaces without those functions: branch after branch."""
-        steady = all(getattr(m, "frame_idx", 0) >= 0 for b in self.branches for m in b.modules())
-        if self._conv_group is None or not steady or len(self.branches) < 2:
-            return [b(x) for b, x in zip(self.branches, xs)]
+        all branches together."""
         for blocks in zip(*self.branches):
             mids = self._conv_group([blk.conv1 for blk in blocks], xs)
             xs = self._residual_group([blk.add for blk in blocks], xs, [blk.conv2 for blk in blocks], mids)
         return xs
 
+    def _run_strided_chains(self, xs):
+        """The strided 3x3 convolutions of the exchange, as far as they depend on the branch
+        outputs only: chain (i, j) brings branch j down to the resolution of output i in i - j
+        steps; all but its last step -- and the last one too for j == 0, where it starts the sum
+        of output i instead of joining it -- run level by level, the steps of one level as a group.
+        Returns ``{(i, j): tensor}``: the start of output i's sum for j == 0, otherwise the input
+        of the chain's last convolution."""
+        chains = {(i, j): list(row[j]) for i, row in enumerate(self.fuse) for j in range(min(i, len(xs)))}
+        cur = {key: xs[key[1]] for key in chains}
+        pos = dict.fromkeys(chains, 0)
+        while True:
+            ready = [k for k, steps in chains.items() if pos[k] < len(steps) - (1 if k[1] > 0 else 0)]
+            if not ready:
+                return cur
+            done = self._conv_group([chains[k][pos[k]] for k in ready], [cur[k] for k in ready])
+            for k, y in zip(ready, done):
+                cur[k], pos[k] = y, pos[k] + 1
+
     def forward(self, xs):
-        xs = self._run_branches(xs)
+        # Layers of parallel paths side by side where the layer namespace can launch them together;
+        # on a model's first frame -- layers take their numbers in call order -- and for namespaces
+        # without those functions: path after path.
+        grouped = self._conv_group is not None and len(xs) > 1 and all(
+            getattr(m, "frame_idx", 0) >= 0 for m in self.modules())
+        xs = self._run_branches(xs) if grouped else [b(x) for b, x in zip(self.branches, xs)]
+        ahead = self._run_strided_chains(xs) if grouped else {}
         outs = []
-        for row, adds in zip(self.fuse, self.adds):
-            y = row[0](xs[0])
+        for i, (row, adds) in enumerate(zip(self.fuse, self.adds)):
+            y = ahead[(i, 0)] if (i, 0) in ahead else row[0](xs[0])
             for j in range(1, len(xs)):
                 add, branch = adds[j - 1], row[j]
-                if j > len(outs) and hasattr(add, "after_upsample"):
+                if j > i and hasattr(add, "after_upsample"):
                     # 1x1 convolution + upsampling: the upsampling is folded into the sum
                     y = add.after_upsample(y, branch[0](xs[j]), branch[1])
                 elif isinstance(branch, nn.Sequential):
                     # strided 3x3 convolutions: the sum rides in the last one's kernel where it can
-                    mid = xs[j]
-                    for step in list(branch)[:-1]:
-                        mid = step(mid)
+                    mid = ahead.get((i, j))
+                    if mid is None:
+                        mid = xs[j]
+                        for step in list(branch)[:-1]:
+                            mid = step(mid)
                     y = _residual_sum(add, y, branch[-1], mid)
                 else:
                     y = add(y, branch(xs[j]))

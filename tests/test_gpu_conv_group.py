@@ -159,23 +159,24 @@ def test_conv_group_declines_what_it_cannot_do(lib):
 
 
 def test_hrnet_branches_side_by_side_change_nothing(lib):
-    """HRNet-W32 at 128x128 (one exchange module per stage), 5 frames: the model that launches the
-    same layer of all branches together against the model that runs branch after branch -- heat
-    maps and every layer's cached state equal bit for bit; and the groups are really taken."""
+    """HRNet-W32 at 128x128 (1 / 1 / 2 exchange modules), 5 frames: the model that launches the
+    same layer of all branches -- and the strided convolutions of an exchange level by level --
+    together against the model that runs path after path: heat maps and every layer's cached
+    state equal bit for bit; and the groups are really taken."""
     from deltacnn_amd import hip_kernels as hk
     from deltacnn_amd import sparse_layers as SL
     from deltacnn_amd.networks import DenseLayers, HRNet, fold_data_statistics
     from deltacnn_amd.video import moving_rectangles_video
     video = moving_rectangles_video(frames=5, height=128, width=128, n_rect=2, min_size=20, max_size=60)
     torch.manual_seed(0)
-    dense = HRNet(DenseLayers, modules=(1, 2, 1)).eval().to(DEV, memory_format=torch.channels_last)
+    dense = HRNet(DenseLayers, modules=(1, 1, 2)).eval().to(DEV, memory_format=torch.channels_last)
     with torch.no_grad():
         fold_data_statistics(dense, cl(video[:2]))
     state = {k: v.clone() for k, v in dense.state_dict().items()}
     SL.DCThreshold.t_default = 0.05
 
     def build():
-        m = HRNet(SL, modules=(1, 2, 1)).eval()
+        m = HRNet(SL, modules=(1, 1, 2)).eval()
         m.load_state_dict(state)
         m = m.to(DEV, memory_format=torch.channels_last).half()
         m.process_filters()
@@ -210,6 +211,7 @@ def test_hrnet_branches_side_by_side_change_nothing(lib):
                 assert torch.equal(a, b), f"{name}.{attr}"
                 n += 1
     assert n > 100
-    # 4 modules x 4 blocks x (conv + activation, conv + sum) on every frame after the first
-    assert len(calls) == 4 * 4 * 2 * (video.shape[0] - 1) and all(done for done, _ in calls), calls[:8]
+    # on every frame after the first: 4 modules x 4 blocks x (conv + activation, conv + sum), and of
+    # the exchanges' strided convolutions one group of 2 on three resolutions, 4 + 2 on four
+    assert len(calls) == (4 * 4 * 2 + 3) * (video.shape[0] - 1) and all(done for done, _ in calls), calls[:8]
     assert {k for _, k in calls} == {2, 3, 4}
