@@ -351,6 +351,9 @@ bool conv_group_item_eligible(const ConvGroupItem &c, int dtype);
 // the convolution kernel finishes the item's activation itself (otherwise it needs an ActGroupItem)
 bool conv_group_activation_fused(const ConvGroupItem &c);
 hipError_t launch_conv_group(const ConvGroupItem *items, int n, int dtype, hipStream_t s);
+// ... and independent small pointwise layers (plain convolutions) likewise
+bool pointwise_group_item_eligible(const ConvGroupItem &c, int dtype);
+hipError_t launch_pointwise_group(const ConvGroupItem *items, int n, int dtype, hipStream_t s);
 
 // Activation / truncation (maximum norm) of several tensors in one launch.
 struct ActGroupItem {

@@ -519,6 +519,7 @@ int dc_conv_group(const dc_conv_item *items, int32_t count, int dtype, void *str
     dc::ActEpilogue epi[DC_CONV_GROUP_MAX];
     dc::ActGroupItem act[DC_CONV_GROUP_MAX];
     int n_act = 0, act_kind = 0;
+    bool pointwise = false;
     for (int i = 0; i < count; ++i) {
         const dc_conv_item &it = items[i];
         int rc = check_conv("dc_conv_group", &it.geometry, it.input, it.packed_filter, it.out, it.mask, it.out_mask,
@@ -550,9 +551,14 @@ int dc_conv_group(const dc_conv_item *items, int32_t count, int dtype, void *str
             epi[i] = dc::ActEpilogue{it.prev_out, it.truncated, it.threshold, it.activation, it.truncation_mode};
             conv[i].epi = &epi[i];
         }
-        if (!dc::conv_group_item_eligible(conv[i], dtype))
-            return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: item %d is not a 16-bit 3x3 layer of the 4x4-patch kernel "
-                                            "(Cin %% 8 == 0, patches * channel tiles * steps <= 32768)", i);
+        const bool pw = dc::pointwise_group_item_eligible(conv[i], dtype);
+        if (!pw && !dc::conv_group_item_eligible(conv[i], dtype))
+            return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: item %d is neither a 16-bit 3x3 layer of the 4x4-patch kernel "
+                                            "(Cin %% 8 == 0, patches * channel tiles * steps <= 32768) nor a plain 1x1 "
+                                            "convolution of the one-tile pointwise arrangement", i);
+        if (i > 0 && pw != pointwise)
+            return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: 1x1 and 3x3 layers in one group");
+        pointwise = pw;
         if (conv[i].epi != nullptr && !dc::conv_group_activation_fused(conv[i])) {
             const int kind = it.activation < 0 ? 0 : it.activation;
             if (n_act > 0 && kind != act_kind)
@@ -576,6 +582,8 @@ int dc_conv_group(const dc_conv_item *items, int32_t count, int dtype, void *str
     if (n_act > 1 && !dc::act_group_eligible(act, n_act, act_kind, DC_TRUNC_MAX, dtype))
         return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: an activation outside the grouped kernel's range "
                                         "(out_c %% 8 == 0, out_c <= 2048, tensor <= 1 MB, 16-byte aligned)");
+    if (pointwise)
+        return finish(dc::launch_pointwise_group(conv, count, dtype, (hipStream_t)stream), "dc_conv_group");
     hipError_t e = dc::launch_conv_group(conv, count, dtype, (hipStream_t)stream);
     if (e == hipSuccess && n_act == 1)
         e = dc::launch_activate_truncate(act[0].delta, act[0].prev, act[0].trunc, act[0].mask, act[0].thr, act_kind,

@@ -72,29 +72,24 @@ struct ResP {
 // the state.  A workgroup holds a slice of a pixel's channels, so it cannot decide itself.
 // ACTC >= 0: the activation of MODE 2 / 3 as a compile-time constant (a run-time id costs a chain
 // of scalar branches per element, half a microsecond in a kernel of this size); -1: rp.act.
+// (bx, by): the workgroup's pixel group and channel group; s_red: KW * CBW * NBW * R * NTW * WAVE
+// partial sums in LDS (KW > 1).
 template <typename E, int KW, int CBW, int NBW, int R, int NTW, int S, int MODE, bool EAGER, int ACTC = -1>
-__global__ void __launch_bounds__(KW * CBW * NBW * WAVE)
-pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
-               const E *__restrict__ bias, E *__restrict__ out,
-               const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, ResP<E> rp) {
+__device__ __forceinline__ void
+pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
+             const E *__restrict__ bias, E *__restrict__ out,
+             const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, const ResP<E> &rp,
+             int bx, int by, float4_t *s_red) {
     typedef typename Elem16<E>::v4 E4;
     typedef typename Elem16<E>::v8 E8;
     static_assert(NBW * NTW <= 4, "a workgroup covers at most 64 pixels");
     constexpr bool ADD = MODE == 1 || MODE == 2, ADDACT = MODE == 2, OPEN = MODE == 3;
     constexpr int NW = KW * CBW * NBW, TILES = R * NTW, FT = (TILES + KW - 1) / KW;
     constexpr int PXW = NBW * NTW * 16;  // pixels per workgroup
-    __shared__ float4_t s_red[KW > 1 ? NW * TILES * WAVE : 1];
     const int wave = wave_id(), lane = lane_id();
     const int l16 = lane & 15, kq = lane >> 4;
     const int kw = wave % KW, tw = wave / KW, cw = tw % CBW, nw = tw / CBW;
     const int ksteps = p.ci_p >> 5;
-    int bx = blockIdx.x, by = blockIdx.y;
-    if (p.xcd) {
-        const int slot = blockIdx.x >> 3;
-        by = (blockIdx.x & 7) + 8 * (slot / p.nx);
-        bx = slot % p.nx;
-        if (by >= p.ny) return;  // padding of the channel groups to a multiple of 8
-    }
     const int pbase = bx * PXW;
 
     // the mask words of the workgroup's pixels, one per lane, together with the first chunk
@@ -299,6 +294,64 @@ pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
         }
         *reinterpret_cast<E4 *>(out + (size_t)(pbase + bit) * p.Co + co) = o;
     }
+}
+
+template <typename E, int KW, int CBW, int NBW, int R, int NTW, int S, int MODE, bool EAGER, int ACTC = -1>
+__global__ void __launch_bounds__(KW * CBW * NBW * WAVE)
+pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
+               const E *__restrict__ bias, E *__restrict__ out,
+               const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, ResP<E> rp) {
+    __shared__ float4_t s_red[KW > 1 ? KW * CBW * NBW * R * NTW * WAVE : 1];
+    int bx = blockIdx.x, by = blockIdx.y;
+    if (p.xcd) {
+        const int slot = blockIdx.x >> 3;
+        by = (blockIdx.x & 7) + 8 * (slot / p.nx);
+        bx = slot % p.nx;
+        if (by >= p.ny) return;  // padding of the channel groups to a multiple of 8
+    }
+    pw_mfma_body<E, KW, CBW, NBW, R, NTW, S, MODE, EAGER, ACTC>(p, in, wp, bias, out, mask, out_mask, rp, bx, by, s_red);
+}
+
+// Several independent small pointwise layers in ONE launch (the 1x1 convolutions of a
+// multi-resolution exchange): a workgroup looks up the layer its number falls into and runs the
+// one-tile, one-wavefront arrangement of pw_mfma_kernel on it unchanged, so the results are those
+// of the separate launches bit for bit.  Plain convolutions whose own launch would use that
+// arrangement only.
+template <typename E>
+struct PwItem {
+    PwP p;
+    const E *in, *wp, *bias;
+    E *out;
+    const int32_t *mask;
+    int32_t *out_mask;
+    int steps;  // fragment loads in flight together: 1, 2 or 4 reduction steps
+    int nx;     // pixel tiles
+    int first;  // number of this layer's first workgroup
+};
+
+template <typename E>
+struct PwGroup {
+    int n;
+    PwItem<E> it[CONV_GROUP_MAX];
+};
+
+template <typename E>
+__global__ void __launch_bounds__(WAVE)
+pw_group_kernel(PwGroup<E> g) {
+    int idx = 0;
+#pragma unroll
+    for (int i = 1; i < CONV_GROUP_MAX; ++i)
+        if (i < g.n && (int)blockIdx.x >= g.it[i].first) idx = i;
+    const PwItem<E> &it = g.it[idx];
+    const int local = blockIdx.x - it.first;
+    const int bx = local % it.nx, by = local / it.nx;
+    const ResP<E> none{nullptr, nullptr, 1.f, 1.f, nullptr, 0};
+    if (it.steps == 1)
+        pw_mfma_body<E, 1, 1, 1, 1, 1, 1, 0, true>(it.p, it.in, it.wp, it.bias, it.out, it.mask, it.out_mask, none, bx, by, nullptr);
+    else if (it.steps == 2)
+        pw_mfma_body<E, 1, 1, 1, 1, 1, 2, 0, true>(it.p, it.in, it.wp, it.bias, it.out, it.mask, it.out_mask, none, bx, by, nullptr);
+    else
+        pw_mfma_body<E, 1, 1, 1, 1, 1, 4, 0, true>(it.p, it.in, it.wp, it.bias, it.out, it.mask, it.out_mask, none, bx, by, nullptr);
 }
 
 // --------------------------------------------------------------- fused conv + act/trunc
@@ -1078,6 +1131,58 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     if (dtype == DC_BF16)
         return launch_pointwise_t<bf16_t>(g, in, packed, bias, out, mask, out_mask, epi, epilogue_done, res, s);
     return launch_pointwise_t<half_t>(g, in, packed, bias, out, mask, out_mask, epi, epilogue_done, res, s);
+}
+
+// A plain pointwise convolution whose own launch is one wavefront per 16 x 16 output tile:
+// what pw_group_kernel runs.
+bool pointwise_group_item_eligible(const ConvGroupItem &c, int dtype) {
+    if (c.packed == nullptr || c.res != nullptr || c.epi != nullptr || !pointwise_eligible(c.g, dtype)) return false;
+    PwP p;
+    p.P = c.g.batch * c.g.in_h * c.g.in_w;
+    p.Ci = c.g.in_c;
+    p.Co = c.g.out_c;
+    p.ci_p = (c.g.in_c + 31) / 32 * 32;
+    p.co_tiles = ceil_div(c.g.out_c, 16);
+    p.xcd = p.nx = p.ny = 0;
+    const int ksteps = p.ci_p / 32;
+    const auto al8 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 7u) == 0; };
+    return p.P < (1 << 16) && pick_config(p, ksteps) == 0 && al8(c.out) && al8(c.bias);
+}
+
+namespace {
+template <typename E>
+hipError_t launch_pointwise_group_t(const ConvGroupItem *items, int n, hipStream_t s) {
+    PwGroup<E> pg;
+    pg.n = n;
+    int blocks = 0;
+    for (int i = 0; i < n; ++i) {
+        const ConvGroupItem &c = items[i];
+        PwItem<E> &it = pg.it[i];
+        it.p.P = c.g.batch * c.g.in_h * c.g.in_w;
+        it.p.Ci = c.g.in_c;
+        it.p.Co = c.g.out_c;
+        it.p.ci_p = (c.g.in_c + 31) / 32 * 32;
+        it.p.co_tiles = ceil_div(c.g.out_c, 16);
+        it.p.xcd = 0;
+        it.p.nx = it.nx = ceil_div(it.p.P, 16);
+        it.p.ny = it.p.co_tiles;
+        it.in = (const E *)c.in; it.wp = (const E *)c.packed; it.bias = (const E *)c.bias;
+        it.out = (E *)c.out; it.mask = c.mask; it.out_mask = c.out_mask;
+        const int ksteps = it.p.ci_p / 32;
+        it.steps = ksteps <= 1 ? 1 : ksteps <= 2 ? 2 : 4;
+        it.first = blocks;
+        blocks += it.nx * it.p.co_tiles;
+    }
+    for (int i = n; i < CONV_GROUP_MAX; ++i) pg.it[i] = pg.it[0];
+    note_kernel("pw_group_kernel");
+    pw_group_kernel<E><<<dim3((unsigned)blocks), WAVE, 0, s>>>(pg);
+    return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_pointwise_group(const ConvGroupItem *items, int n, int dtype, hipStream_t s) {
+    if (dtype == DC_BF16) return launch_pointwise_group_t<bf16_t>(items, n, s);
+    return launch_pointwise_group_t<half_t>(items, n, s);
 }
 
 // ReLU and ReLU6 (what the layers in front of depthwise convolutions use) are instantiated.

@@ -471,6 +471,14 @@ class _HRModule(nn.Module):
             for k, y in zip(ready, done):
                 cur[k], pos[k] = y, pos[k] + 1
 
+    def _run_pointwise(self, xs):
+        """The 1x1 convolutions of the exchange (branch j up to the resolution of output i < j,
+        in front of the upsampling): all of them depend on the branch outputs only and run as one
+        group.  Returns ``{(i, j): tensor}``."""
+        keys = [(i, j) for i in range(len(self.fuse)) for j in range(i + 1, len(xs))]
+        done = self._conv_group([self.fuse[i][j][0] for i, j in keys], [xs[j] for _, j in keys]) if keys else []
+        return dict(zip(keys, done))
+
     def forward(self, xs):
         # Layers of parallel paths side by side where the layer namespace can launch them together;
         # on a model's first frame -- layers take their numbers in call order -- and for namespaces
@@ -479,6 +487,7 @@ class _HRModule(nn.Module):
             getattr(m, "frame_idx", 0) >= 0 for m in self.modules())
         xs = self._run_branches(xs) if grouped else [b(x) for b, x in zip(self.branches, xs)]
         ahead = self._run_strided_chains(xs) if grouped else {}
+        narrow = self._run_pointwise(xs) if grouped and hasattr(self.adds[0][0], "after_upsample") else {}
         outs = []
         for i, (row, adds) in enumerate(zip(self.fuse, self.adds)):
             y = ahead[(i, 0)] if (i, 0) in ahead else row[0](xs[0])
@@ -486,7 +495,7 @@ class _HRModule(nn.Module):
                 add, branch = adds[j - 1], row[j]
                 if j > i and hasattr(add, "after_upsample"):
                     # 1x1 convolution + upsampling: the upsampling is folded into the sum
-                    y = add.after_upsample(y, branch[0](xs[j]), branch[1])
+                    y = add.after_upsample(y, narrow[(i, j)] if (i, j) in narrow else branch[0](xs[j]), branch[1])
                 elif isinstance(branch, nn.Sequential):
                     # strided 3x3 convolutions: the sum rides in the last one's kernel where it can
                     mid = ahead.get((i, j))

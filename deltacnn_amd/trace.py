@@ -244,7 +244,7 @@ class Tracer:
                     p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
                     ni, no = int(it["n_in"]), int(it["n_out"])
                     n_mid = int(it["pairs"][1]) if it["pairs"] is not None else no
-                    rd += p_in * m + ni * g.in_c * s + 9 * g.in_c * g.out_c * s
+                    rd += p_in * m + ni * g.in_c * s + g.kernel_h * g.kernel_w * g.in_c * g.out_c * s
                     wr += (n_mid if late else no) * g.out_c * s + p_out * m
                     if im["kind"] == "conv_add":
                         rd += p_out * m + int(it["n_in_b"]) * g.out_c * s
@@ -260,7 +260,7 @@ class Tracer:
                     p_in_all, p_out_all, n_in_all, n_out_all = p_in_all + p_in, p_out_all + p_out, n_in_all + ni, n_out_all + no
                     names.append(f"{g.in_c}->{g.out_c}@{g.in_h}x{g.in_w}")
                 kinds = {im["kind"] for im in meta["items"]}
-                shape = f"{'/'.join(sorted(kinds))} k3 x{len(names)}: " + " ".join(names)
+                shape = f"{'/'.join(sorted(kinds))} k{meta['items'][0]['g'].kernel_h} x{len(names)}: " + " ".join(names)
                 dens = (n_in_all / p_in_all, n_out_all / p_out_all)
                 if len(r["kernels"]) == 2:
                     t_conv, t_act = r.get("split_us", [ms * 1e3 / 2, ms * 1e3 / 2])

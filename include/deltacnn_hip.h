@@ -269,7 +269,7 @@ int dc_project_expand(const dc_geometry *g, const dc_project_expand_args *args, 
 
 /* One layer of a dc_conv_group call. */
 typedef struct dc_conv_item {
-    dc_geometry geometry;           /* 3x3 convolution, groups == 1 */
+    dc_geometry geometry;           /* 3x3 or 1x1 convolution, groups == 1 */
     const void *input;              /* [B][in_h][in_w][in_c] delta */
     const int32_t *mask;            /* its update mask */
     const void *packed_filter;      /* from dc_pack_filter */
@@ -293,15 +293,18 @@ typedef struct dc_conv_item {
 
 enum { DC_CONV_GROUP_MAX = 8 };
 
-/* 2 .. DC_CONV_GROUP_MAX independent small 3x3 layers -- the parallel branches of a
+/* 2 .. DC_CONV_GROUP_MAX independent small layers -- the parallel branches of a
  * multi-resolution network, whose layers the reference (and dc_conv / dc_conv_act / dc_conv_add)
  * launch one after the other -- in ONE launch, plus one more for the activation / truncation of
  * those items whose convolution cannot finish it itself.  Each item is what one call of dc_conv,
  * dc_conv_act or dc_conv_add would be given, and its results are identical, bit for bit, to that
  * call's.  The items must not depend on each other (no item's output or state is another's
- * operand).  Accepted: 16-bit types, 3x3 kernels on layers small enough for the library's
- * 4x4-patch kernel, activations with maximum-norm truncation, all of one kind where they need
- * the second launch; anything else returns DC_ERR_UNSUPPORTED before any launch so that the
+ * operand).  Accepted, for the 16-bit types: either 3x3 kernels on layers small enough for the
+ * library's 4x4-patch kernel, with activations of maximum-norm truncation, all of one kind where
+ * they need the second launch; or plain 1x1 stride-1 convolutions (no residual sum, no
+ * activation) on maps below 2^16 pixels with a reduction of at most 10 steps of 32 channels (or
+ * 1024 output tiles of 16 x 16 and more), the layers the library runs one wavefront per tile.
+ * Anything else, and a mix of the two, returns DC_ERR_UNSUPPORTED before any launch so that the
  * caller can issue the separate calls.  No counterpart in the reference
  * (sparse_layers.py:425-470 runs one layer per call). */
 int dc_conv_group(const dc_conv_item *items, int32_t count, int dtype, void *stream);

@@ -10,8 +10,12 @@ from util import DEV, assert_masked_equal, cl, poison, rand_mask
 
 pytestmark = pytest.mark.gpu
 
-# items: (kind, Cin, Cout, H, W, batch, stride); kinds: conv, act (activation/truncation), add, addact
+# items: (kind, Cin, Cout, H, W, batch, stride); kinds: conv, act (activation/truncation), add, addact: 3x3;
+# pw: a plain 1x1 convolution
 GROUPS = {
+    "hrnet-exchange-pw": [("pw", 64, 32, 32, 32, 1, 1), ("pw", 128, 32, 16, 16, 1, 1), ("pw", 256, 32, 8, 8, 1, 1),
+                          ("pw", 128, 64, 16, 16, 1, 1), ("pw", 256, 64, 8, 8, 1, 1), ("pw", 256, 128, 8, 8, 1, 1)],
+    "pw-ragged": [("pw", 8, 4, 5, 7, 3, 1), ("pw", 40, 20, 13, 9, 1, 1), ("pw", 320, 72, 3, 3, 2, 1), ("pw", 32, 200, 6, 6, 1, 1)],
     "hrnet4-act": [("act", 32, 32, 64, 64, 1, 1), ("act", 64, 64, 32, 32, 1, 1), ("act", 128, 128, 16, 16, 1, 1),
                    ("act", 256, 256, 8, 8, 1, 1)],
     "hrnet4-addact": [("addact", 32, 32, 64, 64, 1, 1), ("addact", 64, 64, 32, 32, 1, 1),
@@ -41,10 +45,11 @@ def _item(dtype, spec, density, gen):
     x = torch.randn(B, cin, H, W, generator=gen)
     # half of the updates are small: some outputs stay below the activation's threshold
     x = (x * torch.where(torch.rand(B, 1, H, W, generator=gen) < 0.5, 1.0, 2e-2)).to(dtype)
-    w = (torch.randn(cout, cin, 3, 3, generator=gen) / (3 * cin ** 0.5)).to(dtype)
+    k = 1 if kind == "pw" else 3
+    w = (torch.randn(cout, cin, k, k, generator=gen) / (k * cin ** 0.5)).to(dtype)
     f = _filter(dtype, w)
     it = dict(kind=kind, x=cl(poison(x, mask)), mask=cl(mask), filter=f, packed=hk.pack_filter(f, cin, cout, 1),
-              geometry=hk.conv_geometry((B, cin, H, W), (3, 3), cout, (stride, stride), (1, 1), (1, 1), 1),
+              geometry=hk.conv_geometry((B, cin, H, W), (k, k), cout, (stride, stride), (k // 2, k // 2), (1, 1), 1),
               shape=(B, cout, Ho, Wo), stride=stride, cout=cout, host_mask=mask)
     if kind in ("add", "addact"):
         rmask = rand_mask(gen, B, Ho, Wo, 0.5 * density + 0.1)
@@ -67,7 +72,10 @@ def _separate(hk, it, dtype, act_id):
     """The item through the library's single-layer calls: (out, out_mask, states)."""
     prev, trunc = (cl(t) for t in it["states"])
     s = (it["stride"], it["stride"])
-    if it["kind"] == "conv":
+    if it["kind"] == "pw":
+        out, om = hk.sparse_conv(it["x"], it["filter"], it["mask"], None, s, (0, 0), (1, 1), 1, it["cout"],
+                                 create_out_mask=True, packed_filter=it["packed"])
+    elif it["kind"] == "conv":
         out, om = hk.sparse_conv(it["x"], it["filter"], it["mask"], None, s, (1, 1), (1, 1), 1, it["cout"],
                                  create_out_mask=True, packed_filter=it["packed"])
     elif it["kind"] == "act":
@@ -110,7 +118,10 @@ def test_conv_group_equals_separate_calls(lib, dtype, group, density, act_id):
     rows, got = _group_items(items, dtype, act_id)
     assert hk.sparse_conv_group(rows) is True
     kernels = _lib.load().dc_last_kernels().decode().split("+")
-    assert kernels[0] == "conv_patch_group_kernel" and len(kernels) <= 2
+    if GROUPS[group][0][0] == "pw":
+        assert kernels == ["pw_group_kernel"]
+    else:
+        assert kernels[0] == "conv_patch_group_kernel" and len(kernels) <= 2
     if len(kernels) == 2:
         assert kernels[1] in ("act_trunc_group_kernel", "act_trunc_vec_kernel")
     for spec, (o1, m1, p1, t1), (o2, m2, p2, t2) in zip(GROUPS[group], want, got):
@@ -150,6 +161,13 @@ def test_conv_group_declines_what_it_cannot_do(lib):
     # one output buffer for two items
     rows, outs = _group_items(small[:2] + small[:1], dtype, 1)
     rows[2]["out"] = rows[0]["out"]
+    assert hk.sparse_conv_group(rows) is False and untouched(outs)
+    # 1x1 and 3x3 layers together; a 1x1 layer with an activation
+    pws = [_item(dtype, spec, 0.5, gen) for spec in GROUPS["hrnet-exchange-pw"][:2]]
+    rows, outs = _group_items(small[:1] + pws[:1], dtype, 1)
+    assert hk.sparse_conv_group(rows) is False and untouched(outs)
+    rows, outs = _group_items(pws, dtype, 1)
+    rows[1]["activation"] = (outs[1][2], outs[1][3], THR, 1, 0)
     assert hk.sparse_conv_group(rows) is False and untouched(outs)
     # fp32 has no such form
     rows, outs = _group_items(small[:2], dtype, 1)
@@ -211,7 +229,8 @@ def test_hrnet_branches_side_by_side_change_nothing(lib):
                 assert torch.equal(a, b), f"{name}.{attr}"
                 n += 1
     assert n > 100
-    # on every frame after the first: 4 modules x 4 blocks x (conv + activation, conv + sum), and of
-    # the exchanges' strided convolutions one group of 2 on three resolutions, 4 + 2 on four
-    assert len(calls) == (4 * 4 * 2 + 3) * (video.shape[0] - 1) and all(done for done, _ in calls), calls[:8]
-    assert {k for _, k in calls} == {2, 3, 4}
+    # on every frame after the first: 4 modules x 4 blocks x (conv + activation, conv + sum); of the
+    # exchanges' strided convolutions one group of 2 on three resolutions, 4 + 2 on four; and the 1x1
+    # convolutions of each exchange but the first (which has one) as one group of 3, 6, 3
+    assert len(calls) == (4 * 4 * 2 + 3 + 3) * (video.shape[0] - 1) and all(done for done, _ in calls), calls[:8]
+    assert {k for _, k in calls} == {2, 3, 4, 6}
