@@ -75,6 +75,15 @@ class ConvItem(ctypes.Structure):
         ("truncation_mode", c_int32)]
 
 
+class AddItem(ctypes.Structure):
+    """struct dc_add_item."""
+    _fields_ = [
+        ("a", c_void_p), ("b", c_void_p), ("prev_out", c_void_p), ("out", c_void_p),
+        ("mask_a", c_void_p), ("mask_b", c_void_p), ("mask_out", c_void_p),
+        ("weight_a", c_float), ("weight_b", c_float), ("activation", c_int32),
+        ("batch", c_int32), ("height", c_int32), ("width", c_int32), ("channels", c_int32), ("scale", c_int32)]
+
+
 CONV_GROUP_MAX = 8
 
 _P = c_void_p
@@ -92,6 +101,7 @@ _SIGNATURES = {
     "dc_expand_depthwise": (c_int, [_G, POINTER(ExpandDwArgs), c_int, _P]),
     "dc_project_expand": (c_int, [_G, POINTER(ProjectExpandArgs), c_int, _P]),
     "dc_conv_group": (c_int, [POINTER(ConvItem), c_int32, c_int, _P]),
+    "dc_add_group": (c_int, [POINTER(AddItem), c_int32, c_int, _P]),
     "dc_packed_filter_bytes": (c_int64, [_G, c_int, c_int]),
     "dc_pack_filter": (c_int, [_G, _P, _P, c_int, c_int, _P]),
     "dc_deconv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),

@@ -364,6 +364,19 @@ struct ActGroupItem {
 };
 bool act_group_eligible(const ActGroupItem *items, int n, int act, int mode, int dtype);
 hipError_t launch_activate_truncate_group(const ActGroupItem *items, int n, int act, int dtype, hipStream_t s);
+
+// Independent sums of delta tensors in one launch (dc_add_group); S > 1: the second operand is read
+// through nearest upsampling from a map S times smaller.
+struct AddGroupItem {
+    const void *a, *b;
+    void *prev, *out;
+    const int32_t *ma, *mb;
+    int32_t *mo;
+    float wa, wb;
+    int32_t act, B, H, W, C, S;
+};
+bool add_group_eligible(const AddGroupItem *items, int n, int dtype);
+hipError_t launch_add_group(const AddGroupItem *items, int n, int dtype, hipStream_t s);
 hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *packed, int dtype,
                               bool transposed, hipStream_t s);
 int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed);

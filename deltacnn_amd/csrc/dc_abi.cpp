@@ -593,6 +593,55 @@ int dc_conv_group(const dc_conv_item *items, int32_t count, int dtype, void *str
     return finish(e, "dc_conv_group");
 }
 
+int dc_add_group(const dc_add_item *items, int32_t count, int dtype, void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_add_group");
+    DC_REQUIRE_PTR("dc_add_group", items);
+    if (count < 2 || count > DC_CONV_GROUP_MAX)
+        return fail(DC_ERR_SHAPE, "dc_add_group: count=%d outside 2..%d", count, int(DC_CONV_GROUP_MAX));
+    dc::AddGroupItem sums[DC_CONV_GROUP_MAX];
+    for (int i = 0; i < count; ++i) {
+        const dc_add_item &it = items[i];
+        if (it.batch <= 0 || it.height <= 0 || it.width <= 0 || it.scale <= 0)
+            return fail(DC_ERR_SHAPE, "dc_add_group: item %d: batch, height, width and scale must be positive", i);
+        if (it.height % it.scale != 0 || it.width % it.scale != 0)
+            return fail(DC_ERR_SHAPE, "dc_add_group: item %d: %d x %d is not a multiple of scale %d", i, it.height,
+                        it.width, it.scale);
+        if ((int64_t)it.batch * it.height * it.width > INT32_MAX)
+            return fail(DC_ERR_SHAPE, "dc_add_group: item %d: more than 2^31 pixels", i);
+        int rc = check_pc("dc_add_group", it.batch * it.height * it.width, it.channels);
+        if (rc != DC_OK) return rc;
+        if (it.activation > DC_ACT_SWISH)
+            return fail(DC_ERR_UNSUPPORTED, "dc_add_group: item %d: activation id %d", i, it.activation);
+        DC_REQUIRE_PTR("dc_add_group", it.a);
+        DC_REQUIRE_PTR("dc_add_group", it.b);
+        DC_REQUIRE_PTR("dc_add_group", it.out);
+        DC_REQUIRE_PTR("dc_add_group", it.mask_a);
+        DC_REQUIRE_PTR("dc_add_group", it.mask_b);
+        DC_REQUIRE_PTR("dc_add_group", it.mask_out);
+        if (it.activation > 0) DC_REQUIRE_PTR("dc_add_group", it.prev_out);
+        DC_REQUIRE_ALIGNED("dc_add_group", it.a, esize(dtype));
+        DC_REQUIRE_ALIGNED("dc_add_group", it.b, esize(dtype));
+        DC_REQUIRE_ALIGNED("dc_add_group", it.out, esize(dtype));
+        DC_REQUIRE_ALIGNED("dc_add_group", it.prev_out, esize(dtype));
+        sums[i] = dc::AddGroupItem{it.a, it.b, it.activation > 0 ? it.prev_out : nullptr, it.out, it.mask_a, it.mask_b,
+                                   it.mask_out, it.weight_a, it.weight_b, it.activation, it.batch, it.height, it.width,
+                                   it.channels, it.scale};
+    }
+    for (int i = 0; i < count; ++i)
+        for (int j = 0; j < count; ++j) {
+            if (i == j) continue;
+            const dc_add_item &a = items[i], &b = items[j];
+            if (a.out == b.out || a.out == b.a || a.out == b.b || a.mask_out == b.mask_out || a.mask_out == b.mask_a ||
+                a.mask_out == b.mask_b || (a.activation > 0 && b.activation > 0 && a.prev_out == b.prev_out))
+                return fail(DC_ERR_UNSUPPORTED, "dc_add_group: items %d and %d share a buffer one of them writes", i, j);
+        }
+    if (!dc::add_group_eligible(sums, count, dtype))
+        return fail(DC_ERR_UNSUPPORTED, "dc_add_group: 16-bit types, channels %% 8 == 0, 16-byte aligned operands and "
+                                        "maps below 2^18 pixels only");
+    return finish(dc::launch_add_group(sums, count, dtype, (hipStream_t)stream), "dc_add_group");
+}
+
 int dc_pool_densify(const dc_geometry *g, const void *input, const int32_t *mask, void *prev_out,
                     void *out, int dtype, void *stream) {
     dc::kernel_log_reset();

@@ -425,6 +425,75 @@ add_up_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ 
     }
 }
 
+// Several independent sums in one launch (the sums of one level of a multi-resolution exchange):
+// a workgroup looks up the sum its number falls into; a plain sum is an upsampled one of scale 1.
+// The arithmetic is add_up_kernel's, element by element.
+template <typename T>
+struct AddItemD {
+    const T *a, *b;
+    T *prev, *out;
+    const int32_t *ma, *mb;
+    int32_t *mo;
+    float wa, wb;
+    int act, B, H, W, C, S, lg, first;
+};
+
+template <typename T>
+struct AddGroupD {
+    int n;
+    AddItemD<T> it[CONV_GROUP_MAX];
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+add_group_kernel(AddGroupD<T> g) {
+    constexpr int N = Vec16<T>::N;
+    int idx = 0;
+#pragma unroll
+    for (int i = 1; i < CONV_GROUP_MAX; ++i)
+        if (i < g.n && (int)blockIdx.x >= g.it[i].first) idx = i;
+    const AddItemD<T> &it = g.it[idx];
+    const T wa = T(it.wa), wb = T(it.wb);
+    const int G = 1 << it.lg, H = it.H, W = it.W, C = it.C, S = it.S, P = it.B * H * W;
+    const int gid = (blockIdx.x - it.first) * 256 + threadIdx.x;
+    const int p = gid >> it.lg, gl = gid & (G - 1);
+    if (p >= P) return;
+    const int row = p / W, x = p - row * W;  // row = image * H + y
+    const int img = row / H, y = row - img * H;
+    const size_t pb = ((size_t)img * (H / S) + y / S) * (W / S) + x / S;
+    const bool aa = it.ma[p] != 0, ab = it.mb[pb] != 0;
+    if (gl == 0) it.mo[p] = (aa || ab) ? 1 : 0;
+    if (!(aa || ab)) return;
+    const int act = it.act;
+    for (int c = gl * N; c < C; c += G * N) {
+        const size_t off = (size_t)p * C + c;
+        Vec<T, N> s;
+#pragma unroll
+        for (int j = 0; j < N; ++j) s.v[j] = T(0);
+        if (aa) {
+            Vec<T, N> va = vload<T, N>(it.a + off);
+#pragma unroll
+            for (int j = 0; j < N; ++j) s.v[j] = va.v[j] * wa;
+        }
+        if (ab) {
+            Vec<T, N> vb = vload<T, N>(it.b + pb * C + c);
+#pragma unroll
+            for (int j = 0; j < N; ++j) s.v[j] = fma_t(vb.v[j], wb, s.v[j]);
+        }
+        if (act > 0) {
+            Vec<T, N> q = vload<T, N>(it.prev + off);
+            Vec<T, N> n;
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                n.v[j] = s.v[j] + q.v[j];
+                s.v[j] = act_apply<T>(n.v[j], act) - act_apply<T>(q.v[j], act);
+            }
+            vstore<T, N>(it.prev + off, n);
+        }
+        vstore<T, N>(it.out + off, s);
+    }
+}
+
 // add_kernel for large maps: mask scan and compaction per wavefront (see act_trunc_scan_kernel).
 template <typename T, int N>
 __global__ void __launch_bounds__(256)
@@ -1116,6 +1185,49 @@ hipError_t launch_add_upsampled(const void *a, const void *b, void *prev, void *
     if (dtype == DC_BF16)
         return add_up_t<bf16_t>((const bf16_t *)a, (const bf16_t *)b, (bf16_t *)prev, (bf16_t *)out, ma, mb, mo, wa, wb, act, B, H, W, C, scale, s);
     return add_up_t<half_t>((const half_t *)a, (const half_t *)b, (half_t *)prev, (half_t *)out, ma, mb, mo, wa, wb, act, B, H, W, C, scale, s);
+}
+
+// Sums the grouped kernel takes: 16-bit, 16-byte rows and operands, maps below the scanning kernels' size.
+bool add_group_eligible(const AddGroupItem *items, int n, int dtype) {
+    if (n < 2 || n > CONV_GROUP_MAX || (dtype != DC_F16 && dtype != DC_BF16)) return false;
+    for (int i = 0; i < n; ++i) {
+        const AddGroupItem &a = items[i];
+        if (a.C % 8 != 0 || (int64_t)a.B * a.H * a.W >= SCAN_MIN_PIXELS) return false;
+        for (const void *q : {a.a, a.b, (const void *)a.prev, (const void *)a.out})
+            if ((reinterpret_cast<uintptr_t>(q) & 15u) != 0) return false;
+    }
+    return true;
+}
+
+namespace {
+template <typename T>
+hipError_t add_group_t(const AddGroupItem *items, int n, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    AddGroupD<T> ag;
+    ag.n = n;
+    int blocks = 0;
+    for (int i = 0; i < n; ++i) {
+        const AddGroupItem &a = items[i];
+        AddItemD<T> &it = ag.it[i];
+        const int P = a.B * a.H * a.W;
+        it.a = (const T *)a.a; it.b = (const T *)a.b; it.prev = (T *)a.prev; it.out = (T *)a.out;
+        it.ma = a.ma; it.mb = a.mb; it.mo = a.mo;
+        it.wa = a.wa; it.wb = a.wb; it.act = a.act < 0 ? 0 : a.act;
+        it.B = a.B; it.H = a.H; it.W = a.W; it.C = a.C; it.S = a.S;
+        it.lg = log2i(pick_group(a.C / N, P, 4));
+        it.first = blocks;
+        blocks += (int)ceil_div64((int64_t)P << it.lg, 256);
+    }
+    for (int i = n; i < CONV_GROUP_MAX; ++i) ag.it[i] = ag.it[0];
+    note_kernel("add_group_kernel");
+    add_group_kernel<T><<<dim3((unsigned)blocks), 256, 0, s>>>(ag);
+    return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_add_group(const AddGroupItem *items, int n, int dtype, hipStream_t s) {
+    if (dtype == DC_BF16) return add_group_t<bf16_t>(items, n, s);
+    return add_group_t<half_t>(items, n, s);
 }
 
 hipError_t launch_add(const void *a, const void *b, void *prev, void *out, const int32_t *ma,

@@ -540,6 +540,47 @@ def sparse_add_upsampled(a, b, prev_out, out, mask_a, mask_b, mask_out, weight_a
           with_prev=prev_out is not None, dense_out=False, b_scale=scale)
 
 
+def sparse_add_group(items) -> bool:
+    """Independent sums in ONE launch (``dc_add_group``).  ``items``: 2 .. 8 tuples ``(a, b,
+    prev_out, out, mask_a, mask_b, mask_out, weight_a, weight_b, activation, scale)`` -- the
+    arguments of :func:`sparse_add_upsampled`; scale 1: those of :func:`sparse_add_tensors`
+    without ``dense_out``.  Every item's results are identical, bit for bit, to the separate
+    call's.  Returns ``False`` (nothing launched) when the group has no such form."""
+    lib = _lib.load()
+    n = len(items)
+    if n < 2 or n > _lib.CONV_GROUP_MAX:
+        return False
+    dtype = items[0][0].dtype
+    if dtype not in (torch.float16, torch.bfloat16):
+        return False
+    arr = (_lib.AddItem * n)()
+    metas = []
+    for it, (a, b, prev_out, out, mask_a, mask_b, mask_out, wa, wb, activation, scale) in zip(arr, items):
+        _nhwc(a, "a")
+        _nhwc(b, "b")
+        bt, c, h, w = a.shape
+        scale = int(scale)
+        if a.dtype != dtype or b.dtype != dtype:
+            return False
+        if tuple(b.shape) != (bt, c, h // scale, w // scale) or h % scale or w % scale:
+            raise _lib.DeltaCNNError(-2, f"sparse_add_group: {tuple(b.shape)} x{scale} does not give {tuple(a.shape)}")
+        it.a, it.b, it.prev_out, it.out = a.data_ptr(), b.data_ptr(), _ptr(prev_out), out.data_ptr()
+        it.mask_a, it.mask_b = _mask(mask_a, "mask_a").data_ptr(), _mask(mask_b, "mask_b").data_ptr()
+        it.mask_out = mask_out.data_ptr()
+        it.weight_a, it.weight_b, it.activation = float(wa), float(wb), int(activation)
+        it.batch, it.height, it.width, it.channels, it.scale = bt, h, w, c, scale
+        metas.append(dict(P=_pixels(a), C=c, in_mask=mask_a, in_mask_b=mask_b, out_mask=mask_out,
+                          with_prev=prev_out is not None, b_scale=scale))
+    try:
+        _call("add_group", lib.dc_add_group, (arr, n, _DTYPES[dtype], _stream()), items=metas,
+              esize=items[0][0].element_size(), keep=(arr, items))
+    except _lib.DeltaCNNError as e:
+        if e.code == -3:
+            return False
+        raise
+    return True
+
+
 def sparse_add_to_dense_tensor(a, b, mask_a, activation=0):
     """cuda_kernels.py:144-145: ``b[px] += a[px]`` on active pixels."""
     lib = _lib.load()

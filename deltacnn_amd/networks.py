@@ -422,6 +422,7 @@ class _HRModule(nn.Module):
         n = len(channels)
         self._conv_group = getattr(L, "conv_group", None)
         self._residual_group = getattr(L, "residual_group", None)
+        self._add_group = getattr(L, "add_group", None)
         self.branches = nn.ModuleList(
             nn.Sequential(*[_BasicBlock(L, c, c) for _ in range(blocks)]) for c in channels)
         n_out = n if multi_scale_output else 1
@@ -479,6 +480,29 @@ class _HRModule(nn.Module):
         done = self._conv_group([self.fuse[i][j][0] for i, j in keys], [xs[j] for _, j in keys]) if keys else []
         return dict(zip(keys, done))
 
+    def _exchange_by_levels(self, xs):
+        """The exchange with everything that is independent launched together: the strided and
+        the 1x1 convolutions first (they depend on the branch outputs only), then the sums level
+        by level -- term j of every output before term j + 1 of any: the sums of one level belong
+        to different outputs and run as one group, each output still adds its terms in order."""
+        ahead, narrow = self._run_strided_chains(xs), self._run_pointwise(xs)
+        ys = [ahead[(i, 0)] if (i, 0) in ahead else row[0](xs[0]) for i, row in enumerate(self.fuse)]
+        for j in range(1, len(xs)):
+            sums = []
+            for i, (row, adds) in enumerate(zip(self.fuse, self.adds)):
+                add, branch = adds[j - 1], row[j]
+                if j > i:    # 1x1 convolution (done) + upsampling, folded into the sum
+                    sums.append((i, add, narrow[(i, j)], branch[1]))
+                elif j == i:
+                    sums.append((i, add, xs[j], None))
+                else:        # the last strided convolution carries the sum
+                    ys[i] = _residual_sum(add, ys[i], branch[-1], ahead[(i, j)])
+            done = self._add_group([a for _, a, _, _ in sums], [ys[i] for i, _, _, _ in sums],
+                                   [b for _, _, b, _ in sums], [up for _, _, _, up in sums])
+            for (i, _, _, _), y in zip(sums, done):
+                ys[i] = y
+        return ys
+
     def forward(self, xs):
         # Layers of parallel paths side by side where the layer namespace can launch them together;
         # on a model's first frame -- layers take their numbers in call order -- and for namespaces
@@ -486,6 +510,8 @@ class _HRModule(nn.Module):
         grouped = self._conv_group is not None and len(xs) > 1 and all(
             getattr(m, "frame_idx", 0) >= 0 for m in self.modules())
         xs = self._run_branches(xs) if grouped else [b(x) for b, x in zip(self.branches, xs)]
+        if grouped and self._add_group is not None:
+            return self._exchange_by_levels(xs)
         ahead = self._run_strided_chains(xs) if grouped else {}
         narrow = self._run_pointwise(xs) if grouped and hasattr(self.adds[0][0], "after_upsample") else {}
         outs = []

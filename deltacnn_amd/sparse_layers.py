@@ -847,6 +847,34 @@ def residual_group(adds, residuals, convs, conv_inputs):
     return [a.after_conv(r, c, x) for a, r, c, x in zip(adds, residuals, convs, conv_inputs)]
 
 
+def add_group(adds, firsts, seconds, upsamples):
+    """``[add(a, b) if up is None else add.after_upsample(a, b, up) for ...]`` for DCAdd layers
+    that do not depend on each other -- the sums of one level of a multi-resolution exchange -- as
+    ONE launch where ``dc_add_group`` takes them; the separate layer calls otherwise.  Results are
+    identical either way.  Switch: ``DCConv2d.fuse_groups``."""
+    def separate():
+        return [add(a, b) if up is None else add.after_upsample(a, b, up)
+                for add, a, b, up in zip(adds, firsts, seconds, upsamples)]
+    ok = (DCConv2d.fuse_groups and len(adds) >= 2 and DCAdd.fuse_into_conv
+          and all(not isinstance(a, Tensor) and not isinstance(b, Tensor) and not add.first_iter and not add.dense_out
+                  and (up is None or isinstance(up, DCUpsamplingNearest2d))
+                  for add, a, b, up in zip(adds, firsts, seconds, upsamples)))
+    if not ok:
+        return separate()
+    items, results = [], []
+    for add, (val_a, mask_a), (val_b, mask_b), up in zip(adds, firsts, seconds, upsamples):
+        if not _matches(add.out, val_a):
+            add.out = torch.empty_like(val_a)
+        if not _matches(add.mask_out, mask_a):
+            add.mask_out = torch.empty_like(mask_a)
+        with_act = add.activation is not None
+        items.append((val_a, val_b, add.prev_out if with_act else None, add.out, mask_a, mask_b, add.mask_out,
+                      add.weight_a, add.weight_b, add.activation_int if with_act else 0,
+                      1 if up is None else up.scale_factor))
+        results.append((add.out, add.mask_out))
+    return results if hk.sparse_add_group(items) else separate()
+
+
 class DCConcatenate(DCModule):
     """Channel concatenation of two delta tensors (sparse_layers.py:1185-1194)."""
 

@@ -58,6 +58,9 @@ class Tracer:
 
     def run(self, op, fn, args, meta):
         rec = {"op": op, "meta": meta}
+        if op == "add_group":
+            rec["items"] = [{"n_in": self._count(i["in_mask"]), "n_in_b": self._count(i["in_mask_b"]), "pairs": None}
+                            for i in meta["items"]]
         if op == "conv_group":  # one set of counts per layer of the group
             rec["items"] = [{"n_in": self._count(i["in_mask"]), "n_in_b": self._count(i["in_mask_b"]),
                              "pairs": self._pairs(i["g"], i["in_mask"], False) if self.count_pairs else None}
@@ -267,6 +270,18 @@ class Tracer:
                     ms = t_conv * 1e-3
                     extra = {"kernel": r["kernels"][1], "call": op, "shape": f"x{sum(second)} P{act_px}", "ms": t_act * 1e-3,
                              "bytes": act_bytes, "flops": 0, "density_in": act_in / act_px, "density_out": act_out / act_px}
+            elif op == "add_group":  # the add formula, summed over the sums of the group
+                rd = wr = 0
+                p_all = act_all = out_all = 0
+                for it, im in zip(r["items"], meta["items"]):
+                    P, C, bs = im["P"], im["C"], im["b_scale"] ** 2
+                    ni, nb, no = int(it["n_in"]), int(it["n_in_b"]), int(it["n_out"])
+                    ext = no * C * s if im["with_prev"] else 0
+                    rd += (P + P // bs) * m + (ni + nb) * C * s + ext
+                    wr += no * C * s + ext + P * m
+                    p_all, act_all, out_all = p_all + 2 * P, act_all + ni + nb * bs, out_all + no
+                shape = f"x{len(meta['items'])}: " + " ".join(f"C{im['C']}P{im['P']}" for im in meta["items"])
+                dens = (act_all / p_all, 2 * out_all / p_all)
             elif op == "block":
                 g = meta["g"]
                 ch, cp, ce = g.in_c, meta["Cp"], meta["Ce"]

@@ -309,6 +309,29 @@ enum { DC_CONV_GROUP_MAX = 8 };
  * (sparse_layers.py:425-470 runs one layer per call). */
 int dc_conv_group(const dc_conv_item *items, int32_t count, int dtype, void *stream);
 
+/* One sum of a dc_add_group call: the arguments of dc_add_upsampled (scale 1: those of dc_add
+ * without dense_out). */
+typedef struct dc_add_item {
+    const void *a;                  /* [B][H][W][C] delta */
+    const void *b;                  /* [B][H/scale][W/scale][C] delta */
+    void *prev_out;                 /* accumulated sum (activation > 0), or NULL */
+    void *out;                      /* [B][H][W][C] */
+    const int32_t *mask_a, *mask_b;
+    int32_t *mask_out;              /* [B][H][W] = mask_a | upsampled mask_b */
+    float weight_a, weight_b;
+    int32_t activation;
+    int32_t batch, height, width, channels, scale;
+} dc_add_item;
+
+/* 2 .. DC_CONV_GROUP_MAX independent sums -- those of one level of a multi-resolution exchange,
+ * which the reference launches one after the other (sparse_layers.py:1086-1182) -- in ONE launch.
+ * Each item's results are identical, bit for bit, to dc_add_upsampled's (dc_add's for scale 1).
+ * No item's output, mask or accumulated sum may be another's operand.  For the 16-bit types,
+ * channels in multiples of 8, 16-byte aligned operands and maps below 2^18 pixels; anything else
+ * returns DC_ERR_UNSUPPORTED before any launch so that the caller can issue the separate calls.
+ * No counterpart in the reference. */
+int dc_add_group(const dc_add_item *items, int32_t count, int dtype, void *stream);
+
 /* Number of bytes dc_pack_filter writes for this geometry (0 if the shape has no packed
  * form).  One-time weight relayout for the MFMA kernels, fp16 or bfloat16, un-swizzled, in fragment order
  * [Cout tile of 16][Kh][Kw][Cin step of 32][lane 0..63][8] (lane kq*16+r holds input channels

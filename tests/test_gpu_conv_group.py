@@ -208,6 +208,14 @@ def test_hrnet_branches_side_by_side_change_nothing(lib):
         calls.append((done, len(items)))
         return done
     hk.sparse_conv_group = counted
+    sums = []
+    original_sums = hk.sparse_add_group
+
+    def counted_sums(items):
+        done = original_sums(items)
+        sums.append((done, len(items)))
+        return done
+    hk.sparse_add_group = counted_sums
     try:
         with torch.no_grad():
             for t in range(video.shape[0]):
@@ -220,6 +228,7 @@ def test_hrnet_branches_side_by_side_change_nothing(lib):
     finally:
         SL.DCConv2d.fuse_groups = True
         hk.sparse_conv_group = original
+        hk.sparse_add_group = original_sums
     gm, pm = dict(grouped.named_modules()), dict(plain.named_modules())
     n = 0
     for name, mod in gm.items():
@@ -234,3 +243,6 @@ def test_hrnet_branches_side_by_side_change_nothing(lib):
     # convolutions of each exchange but the first (which has one) as one group of 3, 6, 3
     assert len(calls) == (4 * 4 * 2 + 3 + 3) * (video.shape[0] - 1) and all(done for done, _ in calls), calls[:8]
     assert {k for _, k in calls} == {2, 3, 4, 6}
+    # the sums of an exchange level by level: 2 on two resolutions, 2 + 3 on three, 2 + 3 + 4 on four
+    assert len(sums) == 6 * (video.shape[0] - 1) and all(done for done, _ in sums), sums[:8]
+    assert sorted(k for _, k in sums[:6]) == [2, 2, 2, 3, 3, 4]

@@ -407,3 +407,40 @@ def test_conv_group_arguments_are_checked_before_any_launch(lib):
     assert call([item(0), item(1, input=base + 3 * 256)]) == -3            # item 1 reads what item 0 writes
     assert call([item(0, residual=base + 1024)]) == -2                       # still one item
     assert call([item(0), item(1, residual=base + 4096 + 1024)]) == -4       # a residual needs its mask
+
+
+def test_add_group_arguments_are_checked_before_any_launch(lib):
+    """dc_add_group: a count outside 2..8 or a map that is no multiple of the scale -> -2; channel
+    counts off the vector size, fp32, sums that share a buffer one of them writes -> -3; missing
+    operands -> -4; nothing touches a device."""
+    from deltacnn_amd._lib import AddItem
+    buf = (ctypes.c_char * 65536)()
+    base = (ctypes.addressof(buf) + 255) // 256 * 256
+
+    def item(k, **kw):
+        it = AddItem()
+        p = base + k * 4096
+        for j, name in enumerate(("a", "b", "prev_out", "out", "mask_a", "mask_b", "mask_out")):
+            setattr(it, name, p + j * 256)
+        it.weight_a = it.weight_b = 1.0
+        it.batch, it.height, it.width, it.channels, it.scale = 1, 8, 8, 32, 2
+        for name, v in kw.items():
+            setattr(it, name, v)
+        return it
+
+    def call(items, dtype=1):
+        arr = (AddItem * len(items))(*items)
+        return lib.dc_add_group(arr, len(items), dtype, None)
+
+    assert call([item(0), item(1)], dtype=9) == -1
+    assert call([item(0), item(1)], dtype=0) == -3
+    assert call([item(0)]) == -2 and call([item(k) for k in range(9)]) == -2
+    assert lib.dc_add_group(None, 2, 1, None) == -4
+    assert call([item(0), item(1, height=7)]) == -2 and b"multiple of scale" in lib.dc_last_error()
+    assert call([item(0), item(1, channels=12)]) == -3
+    assert call([item(0), item(1, a=base + 4096 + 2)]) == -3                 # not a 16-byte aligned row
+    assert call([item(0), item(1, out=None)]) == -4
+    assert call([item(0), item(1, activation=1, prev_out=None)]) == -4
+    assert call([item(0), item(1, activation=9)]) == -3
+    assert call([item(0), item(1, out=base + 3 * 256)]) == -3 and b"share" in lib.dc_last_error()
+    assert call([item(0), item(1, b=base + 3 * 256)]) == -3                  # item 1 reads what item 0 writes
