@@ -315,7 +315,8 @@ def sparse_project_expand(x, mask, project_packed, project_geometry, residual, r
 
 def sparse_conv_group(items) -> bool:
     """Independent small 3x3 layers in ONE launch (``dc_conv_group``), plus one for the
-    activations that their convolutions cannot finish themselves.  ``items``: 2 .. 8 dicts with
+    activations that their convolutions cannot finish themselves; or independent plain 1x1
+    convolutions in one launch.  ``items``: 2 .. 8 dicts with
     ``x, mask, packed_filter, geometry, out, out_mask`` (and optionally ``bias``) and at most one of
     ``residual = (values, mask, weight_residual, weight_conv, prev_out or None, activation)`` --
     the operands of :func:`sparse_conv_add` -- and ``activation = (prev_out, truncated, threshold,
