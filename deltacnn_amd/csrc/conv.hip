@@ -1678,13 +1678,13 @@ conv_patch_group_kernel(PatchGroup<E> g) {
         else DC_GROUP_BODY(KWV, RV, SV, 0);                \
     } while (0)
     if (it.kwv == 1) {
-        if (it.mode == 2) { if (it.rv == 2) DC_GROUP_BODY(1, 2, 6, 2); else DC_GROUP_BODY(1, 1, 12, 2); }
-        else if (it.rv == 2) DC_GROUP_MODE(1, 2, 6);
-        else DC_GROUP_MODE(1, 1, 12);
+        if (it.mode == 2) { if (it.rv == 2) DC_GROUP_BODY(1, 2, 9, 2); else DC_GROUP_BODY(1, 1, 9, 2); }
+        else if (it.rv == 2) DC_GROUP_MODE(1, 2, 9);
+        else DC_GROUP_MODE(1, 1, 9);
     } else if (it.kwv == 4) {
-        if (it.rv == 2) DC_GROUP_MODE(4, 2, 6); else DC_GROUP_MODE(4, 1, 12);
+        if (it.rv == 2) DC_GROUP_MODE(4, 2, 5); else DC_GROUP_MODE(4, 1, 9);
     } else {
-        if (it.rv == 2) DC_GROUP_MODE(8, 2, 6); else DC_GROUP_MODE(8, 1, 12);
+        if (it.rv == 2) DC_GROUP_MODE(8, 2, 6); else DC_GROUP_MODE(8, 1, 9);
     }
 #undef DC_GROUP_MODE
 #undef DC_GROUP_BODY
@@ -2402,13 +2402,13 @@ hipError_t launch_patch_conv_t(const dc_geometry &g, const void *in, const void 
     } while (0)
 #define DC_PATCH(TRF, AV)                                                                       \
     do {                                                                                        \
-        if (kwv == 1) { if (rv == 2) DC_PATCH_L(TRF, 1, 2, 6, AV); else DC_PATCH_L(TRF, 1, 1, 12, AV); } \
-        else if (kwv == 4) { if (rv == 2) DC_PATCH_L(TRF, 4, 2, 6, AV); else DC_PATCH_L(TRF, 4, 1, 12, AV); } \
-        else { if (rv == 2) DC_PATCH_L(TRF, 8, 2, 6, AV); else DC_PATCH_L(TRF, 8, 1, 12, AV); } \
+        if (kwv == 1) { if (rv == 2) DC_PATCH_L(TRF, 1, 2, 9, AV); else DC_PATCH_L(TRF, 1, 1, 9, AV); } \
+        else if (kwv == 4) { if (rv == 2) DC_PATCH_L(TRF, 4, 2, 5, AV); else DC_PATCH_L(TRF, 4, 1, 9, AV); } \
+        else { if (rv == 2) DC_PATCH_L(TRF, 8, 2, 6, AV); else DC_PATCH_L(TRF, 8, 1, 9, AV); } \
     } while (0)
     if (res != nullptr) DC_PATCH(false, 1);  // the fused sum exists for plain convolutions only
     else if (transposed) DC_PATCH(true, 0);
-    else if (fuse) { if (rv == 2) DC_PATCH_L(false, 1, 2, 6, 2); else DC_PATCH_L(false, 1, 1, 12, 2); }
+    else if (fuse) { if (rv == 2) DC_PATCH_L(false, 1, 2, 9, 2); else DC_PATCH_L(false, 1, 1, 9, 2); }
     else DC_PATCH(false, 0);
 #undef DC_PATCH
 #undef DC_PATCH_L
