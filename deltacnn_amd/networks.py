@@ -488,7 +488,7 @@ class _HRModule(nn.Module):
         ahead, narrow = self._run_strided_chains(xs), self._run_pointwise(xs)
         ys = [ahead[(i, 0)] if (i, 0) in ahead else row[0](xs[0]) for i, row in enumerate(self.fuse)]
         for j in range(1, len(xs)):
-            sums = []
+            sums, carried = [], []
             for i, (row, adds) in enumerate(zip(self.fuse, self.adds)):
                 add, branch = adds[j - 1], row[j]
                 if j > i:    # 1x1 convolution (done) + upsampling, folded into the sum
@@ -496,10 +496,12 @@ class _HRModule(nn.Module):
                 elif j == i:
                     sums.append((i, add, xs[j], None))
                 else:        # the last strided convolution carries the sum
-                    ys[i] = _residual_sum(add, ys[i], branch[-1], ahead[(i, j)])
-            done = self._add_group([a for _, a, _, _ in sums], [ys[i] for i, _, _, _ in sums],
-                                   [b for _, _, b, _ in sums], [up for _, _, _, up in sums])
-            for (i, _, _, _), y in zip(sums, done):
+                    carried.append((i, add, branch[-1], ahead[(i, j)]))
+            done = self._residual_group([a for _, a, _, _ in carried], [ys[i] for i, _, _, _ in carried],
+                                        [c for _, _, c, _ in carried], [m for _, _, _, m in carried])
+            done += self._add_group([a for _, a, _, _ in sums], [ys[i] for i, _, _, _ in sums],
+                                    [b for _, _, b, _ in sums], [up for _, _, _, up in sums])
+            for (i, _, _, _), y in zip(carried + sums, done):
                 ys[i] = y
         return ys
 

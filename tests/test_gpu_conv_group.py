@@ -240,8 +240,9 @@ def test_hrnet_branches_side_by_side_change_nothing(lib):
     assert n > 100
     # on every frame after the first: 4 modules x 4 blocks x (conv + activation, conv + sum); of the
     # exchanges' strided convolutions one group of 2 on three resolutions, 4 + 2 on four; and the 1x1
-    # convolutions of each exchange but the first (which has one) as one group of 3, 6, 3
-    assert len(calls) == (4 * 4 * 2 + 3 + 3) * (video.shape[0] - 1) and all(done for done, _ in calls), calls[:8]
+    # convolutions of each exchange but the first (which has one) as one group of 3, 6, 3; and the two
+    # sum-carrying strided convolutions of the first level on four resolutions
+    assert len(calls) == (4 * 4 * 2 + 3 + 3 + 1) * (video.shape[0] - 1) and all(done for done, _ in calls), calls[:8]
     assert {k for _, k in calls} == {2, 3, 4, 6}
     # the sums of an exchange level by level: 2 on two resolutions, 2 + 3 on three, 2 + 3 + 4 on four
     assert len(sums) == 6 * (video.shape[0] - 1) and all(done for done, _ in sums), sums[:8]
