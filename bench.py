@@ -20,6 +20,9 @@ the result; a section that fails is named under "errors" and the run goes on).  
                    C=512, each + ReLU/truncation) over the update densities
   scaled           the memory-bound operators at 512x512, batch 8 (working set beyond the caches)
   cpu_baseline     the CPU oracle of the delta path timed on this host's cores (bounded sample)
+  networks         MobileNetV2 on the 64-frame moving-rectangles clip, HRNet-W32 at 256x256 and
+                   DLA-34/CenterNet at 544x960: frames/sec, the dense model on the same GPU,
+                   launches per frame, mean update density, dominant kernel and its roofline fraction
 """
 from __future__ import annotations
 
@@ -395,7 +398,38 @@ def scaled_bench():
     return out
 
 
-def network_bench(which, steps, warmup):
+def _network_report(name, size, delta, dense, frames, steps, warmup, clip):
+    """Frames/s of the delta path and of the dense model (eager and graph) on one clip, launches
+    per frame, mean update density of the library calls, per-kernel device times and the kernel
+    with the largest share of the frame with its fraction of the HBM (or fp16 MFMA) peak."""
+    sec = run_delta(delta, frames, warmup, steps, "graph")
+    dense_eager, dense_graph = run_dense(dense, frames, warmup, steps)
+    agg, rows = trace_kernels(delta, frames)
+    dom_name = max(agg, key=lambda k: agg[k]["ms"])
+    dom = agg[dom_name]
+    hbm, mfma = dom["GBps"] / HBM_PEAK_GBS, dom["TFLOPs"] / MFMA_F16_PEAK_TFLOPS
+    return {
+        "network": name, "input": list(size), "clip": clip, "value": round(1 / sec, 1), "unit": "frames/s",
+        "ms_per_step": round(sec * 1e3, 4), "steps": steps, "warmup": warmup,
+        "dense_gpu": {"eager_fps": round(1 / dense_eager, 1), "graph_fps": round(1 / dense_graph, 1),
+                      "speedup_vs_dense_gpu": round(min(dense_eager, dense_graph) / sec, 3)},
+        "library_launches_per_frame": sum(a["launches"] for a in agg.values()),
+        "mean_input_density_of_library_calls": round(sum(r["density_in"] for r in rows) / len(rows), 3),
+        "frame_alg_GBps": round(sum(a["bytes"] for a in agg.values()) / sec / 1e9, 2),
+        "dominant_kernel": {"kernel": dom_name, "launches_per_frame": dom["launches"],
+                            "us_per_launch": round(dom["us_per_launch"], 3),
+                            "share_of_kernel_time": round(dom["ms"] / sum(a["ms"] for a in agg.values()), 3),
+                            "bound": "mfma" if mfma > hbm else "hbm",
+                            "achieved": round(dom["TFLOPs"], 2) if mfma > hbm else round(dom["GBps"], 1),
+                            "unit": "TFLOP/s" if mfma > hbm else "GB/s", "frac": round(max(hbm, mfma), 4)},
+        "kernels": {k: {"launches_per_frame": a["launches"], "us_per_launch": round(a["us_per_launch"], 3),
+                        "ms_per_frame": round(a["ms_per_frame"], 4), "alg_GBps": round(a["GBps"], 1),
+                        "alg_TFLOPs": round(a["TFLOPs"], 2)}
+                    for k, a in sorted(agg.items(), key=lambda kv: -kv[1]["ms"])},
+    }
+
+
+def network_bench(which, steps, warmup, only_delta=False):
     """The two larger configurations (parity cases, not the headline): HRNet-W32 pose network at
     256x256 and the DLA-34 CenterNet detector at 544x960, fp16, batch 1, random-init weights
     rescaled on two frames, threshold 0.05; synthetic static-camera clips (one large moving blob /
@@ -422,20 +456,13 @@ def network_bench(which, steps, warmup):
     delta = delta.to("cuda", memory_format=torch.channels_last).half()
     delta.process_filters()
     frames = gpu_frames(video)
-    sec = run_delta(delta, frames, warmup, steps, "graph")
-    dense_eager, dense_graph = run_dense(dense, frames, warmup, steps)
-    agg, rows = trace_kernels(delta, frames)
-    return {
-        "network": which, "input": list(size), "value": round(1 / sec, 1), "unit": "frames/s",
-        "ms_per_step": round(sec * 1e3, 4), "steps": steps, "warmup": warmup,
-        "dense_gpu": {"eager_fps": round(1 / dense_eager, 1), "graph_fps": round(1 / dense_graph, 1),
-                      "speedup_vs_dense_gpu": round(min(dense_eager, dense_graph) / sec, 3)},
-        "mean_input_density_of_library_calls": round(sum(r["density_in"] for r in rows) / len(rows), 3),
-        "kernels": {k: {"launches_per_frame": a["launches"], "us_per_launch": round(a["us_per_launch"], 3),
-                        "ms_per_frame": round(a["ms_per_frame"], 4), "alg_GBps": round(a["GBps"], 1),
-                        "alg_TFLOPs": round(a["TFLOPs"], 2)}
-                    for k, a in sorted(agg.items(), key=lambda kv: -kv[1]["ms"])},
-    }
+    clip = (f"static background, {kw['n_rect']} textured rectangle(s) of {kw['min_size']}-{kw['max_size']} px moving "
+            f"{kw['min_speed']}-{kw['max_speed']} px/frame, no sensor noise")
+    if only_delta:  # for profiling runs: nothing but the delta path's kernels
+        sec = run_delta(delta, frames, warmup, steps, "graph")
+        return {"network": which, "value": round(1 / sec, 1), "unit": "frames/s", "ms_per_step": round(sec * 1e3, 4),
+                "steps": steps}
+    return _network_report(which, size, delta, dense, frames, steps, warmup, clip)
 
 
 def cpu_baseline(state, video, n_frames, threads):
@@ -475,6 +502,9 @@ def main():
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-micro", action="store_true", help="skip the single-layer and scaled-shape sections")
+    ap.add_argument("--no-networks", action="store_true",
+                    help="skip the closing section that times MobileNetV2 on the moving-rectangles clip, HRNet-W32 "
+                         "256x256 and DLA-34/CenterNet 544x960")
     ap.add_argument("--only-delta", action="store_true",
                     help="time the delta path only and print a short JSON line (for profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -505,7 +535,8 @@ def main():
         print(json.dumps({"micro": micro_bench(), "scaled": scaled_bench()}), flush=True)
         return
     if args.network != "mobilenetv2":
-        print(json.dumps(network_bench(args.network, min(args.steps, 64), min(args.warmup, 16))), flush=True)
+        print(json.dumps(network_bench(args.network, min(args.steps, 64), min(args.warmup, 16), args.only_delta)),
+              flush=True)
         return
 
     plan = launch_plan(args.steps, args.warmup)
@@ -579,14 +610,18 @@ def main():
         result["library_launches_per_frame"] = sum(a["launches"] for a in agg.values())
         result["frame_alg_GBps"] = round(sum(a["bytes"] for a in agg.values()) / sec / 1e9, 2)
         result["kernel_time_sum_ms"] = round(sum(a["ms"] for a in agg.values()), 4)
-        traffic = None
+        traffic = traffic_source = None
         tpath = os.path.join(ROOT, "profiles", "pmc_traffic.json")
         if os.path.exists(tpath):  # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
             with open(tpath) as f:
                 traffic = json.load(f).get(dom_name, {}).get("bytes_per_launch")
+            traffic_source = ("not measured by this run: read from profiles/pmc_traffic.json, the summary of two "
+                              "separate rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of `bench.py --only-delta "
+                              "--calibrate-copy`; commands in profiles/mobilenetv2_224_delta_frame_traffic.txt")
         result["roofline"] = {
             "bound": "hbm", "kernel": dom_name, "achieved": round(dom["GBps"], 2), "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": round(dom["GBps"] / HBM_PEAK_GBS, 5), "traffic": traffic,
+            "traffic_source": traffic_source,
             "bytes_per_launch": round(dom["bytes_per_launch"], 1),
             "us_per_launch": round(dom["us_per_launch"], 3),
             "duration_source": "live: every library call of one traced frame replayed back to back from a HIP "
@@ -671,6 +706,29 @@ def main():
             result["scaled"] = scaled_bench()
         section("scaled", scaled_section)
         emit()
+
+    # -- the other configurations, each on its own clip (after the headline has been emitted) --
+    if not args.no_networks:
+        nets = result["networks"] = []
+        nw_steps, nw_warm = min(args.steps, 48), min(args.warmup, 8)
+
+        def config3_section():
+            # MobileNetV2 on the clip its configuration names: 64 frames, smooth-noise background,
+            # three textured rectangles of 20-60 px moving 1-4 px/frame, sensor noise sigma 0.01
+            clip = gpu_frames(moving_rectangles_video(frames=max(64, clip_frames(nw_steps, nw_warm))))
+            nets.append(_network_report("mobilenetv2", (224, 224), delta, dense, clip, nw_steps, nw_warm,
+                                        "64-frame synthetic video: static smooth-noise background, 3 textured rectangles "
+                                        "of 20-60 px moving 1-4 px/frame, Gaussian sensor noise sigma 0.01"))
+            log(f"MobileNetV2 on the moving-rectangles clip: {nets[-1]['value']:.0f} frames/s")
+        section("networks.mobilenetv2_clip", config3_section)
+        emit()
+        for which in ("hrnet", "dla34"):
+            def net_section(which=which):
+                nets.append(network_bench(which, nw_steps, nw_warm))
+                log(f"{which}: {nets[-1]['value']:.0f} frames/s, dense graph {nets[-1]['dense_gpu']['graph_fps']:.0f}, "
+                    f"{nets[-1]['library_launches_per_frame']} launches per frame")
+            section(f"networks.{which}", net_section)
+            emit()
 
 
 if __name__ == "__main__":

@@ -34,6 +34,13 @@ inline size_t esize(int dtype) { return dtype == DC_F32 ? 4 : 2; }
     if ((p) != nullptr && (reinterpret_cast<uintptr_t>(p) % (a)) != 0) \
         return fail(DC_ERR_ALIGN, fn ": " #p " is not aligned to %d bytes", int(a))
 
+// A buffer as a byte range; a NULL pointer is an empty range.
+struct Span {
+    uintptr_t lo, hi;
+    Span(const void *p, size_t bytes) : lo(reinterpret_cast<uintptr_t>(p)), hi(p == nullptr ? 0 : reinterpret_cast<uintptr_t>(p) + bytes) {}
+    bool meets(const Span &o) const { return lo < hi && o.lo < o.hi && lo < o.hi && o.lo < hi; }
+};
+
 int check_pc(const char *fn, int32_t pixels, int32_t channels) {
     if (pixels <= 0 || channels <= 0)
         return fail(DC_ERR_SHAPE, "%s: pixels=%d channels=%d must be positive", fn, pixels, channels);
@@ -404,7 +411,7 @@ int dc_expand_depthwise(const dc_geometry *g, const dc_expand_dw_args *args, int
     const bool opened = a.expand_packed_filter == nullptr;  // dc_project_expand ran the convolution
     if (!opened && !dc::pointwise_open_eligible(ge, dtype, a.expand_activation))
         return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: the expansion needs input channels in multiples of 8, "
-                                        "output channels in multiples of 4 and ReLU or ReLU6");
+                                        "output channels in multiples of 8 and ReLU or ReLU6");
     dc::ActEpilogue dw_epi{a.dw_prev_out, a.dw_truncated, a.dw_threshold, a.dw_activation, a.dw_truncation_mode};
     if (!dc::depthwise_closing_eligible(*g, &dw_epi, dtype))
         return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: needs a depthwise 3x3 convolution with stride 1 and "
@@ -496,6 +503,29 @@ int dc_project_expand(const dc_geometry *g, const dc_project_expand_args *args, 
             return fail(DC_ERR_UNSUPPORTED, "dc_project_expand: the depthwise layer behind the expansion cannot finish "
                                             "its activation (needs 3x3, stride 1, padding 1 on a small map)");
     }
+    {
+        // Several workgroups per pixel tile read every input of this call and repeat the projection
+        // while one of them stores it: nothing the call writes may overlap anything it reads or
+        // anything else it writes (expand_truncated is read and written by the same lanes).
+        const size_t P = (size_t)g->batch * g->out_h * g->out_w, es = esize(dtype);
+        const Span wr[] = {Span(a.out, P * g->out_c * es), Span(a.out_mask, P * 4), Span(a.expand_out_mask, P * 4),
+                           Span(a.expand_out, P * a.expand_channels * es), Span(a.expand_truncated, P * a.expand_channels * es)};
+        const Span rd[] = {Span(a.input, P * g->in_c * es), Span(a.mask, P * 4), Span(a.residual, P * g->out_c * es),
+                           Span(a.residual_mask, P * 4), Span(a.expand_prev_out, P * a.expand_channels * es),
+                           Span(a.project_packed_filter, (size_t)dc_packed_filter_bytes(g, dtype, 0)),
+                           Span(a.expand_packed_filter, (size_t)((g->out_c + 31) / 32 * 32) * ((a.expand_channels + 15) / 16 * 16) * es)};
+        for (size_t i = 0; i < sizeof(wr) / sizeof(wr[0]); ++i) {
+            for (size_t j = 0; j < sizeof(rd) / sizeof(rd[0]); ++j)
+                if (wr[i].meets(rd[j]))
+                    return fail(DC_ERR_UNSUPPORTED, "dc_project_expand: an output buffer overlaps an input of the call "
+                                                    "(no in-place sums: out, out_mask, expand_out, expand_out_mask and "
+                                                    "expand_truncated must be separate from input, mask, residual, "
+                                                    "residual_mask, expand_prev_out and the filters)");
+            for (size_t j = i + 1; j < sizeof(wr) / sizeof(wr[0]); ++j)
+                if (wr[i].meets(wr[j]))
+                    return fail(DC_ERR_UNSUPPORTED, "dc_project_expand: two output buffers of the call overlap");
+        }
+    }
     dc::Residual res{a.residual, a.residual_mask, a.weight_residual, a.weight_conv};
     dc::OpenAct open;
     open.prev = a.expand_prev_out;
@@ -568,16 +598,26 @@ int dc_conv_group(const dc_conv_item *items, int32_t count, int dtype, void *str
                                             g.batch * g.out_h * g.out_w, g.out_c};
         }
     }
-    // no item may write what another reads or writes
+    // All items run side by side in one launch: no item may write bytes that another reads or
+    // writes (byte ranges, so views into one allocation are seen too).
     for (int i = 0; i < count; ++i)
         for (int j = 0; j < count; ++j) {
             if (i == j) continue;
             const dc_conv_item &a = items[i], &b = items[j];
-            if (a.out == b.out || a.out == b.input || a.out == b.residual || a.out_mask == b.out_mask ||
-                a.out_mask == b.mask || a.out_mask == b.residual_mask ||
-                (a.prev_out != nullptr && (a.prev_out == b.prev_out || a.truncated == b.truncated)) ||
-                (a.sum_prev_out != nullptr && a.sum_prev_out == b.sum_prev_out))
-                return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: items %d and %d share a buffer one of them writes", i, j);
+            const size_t es = esize(dtype);
+            const size_t pa = (size_t)a.geometry.batch * a.geometry.out_h * a.geometry.out_w, ca = a.geometry.out_c;
+            const size_t pb = (size_t)b.geometry.batch * b.geometry.out_h * b.geometry.out_w, cb = b.geometry.out_c;
+            const size_t pbi = (size_t)b.geometry.batch * b.geometry.in_h * b.geometry.in_w;
+            const Span wr[] = {Span(a.out, pa * ca * es), Span(a.out_mask, pa * 4), Span(a.prev_out, pa * ca * es),
+                               Span(a.truncated, pa * ca * es), Span(a.sum_prev_out, pa * ca * es)};
+            const Span other[] = {Span(b.input, pbi * b.geometry.in_c * es), Span(b.mask, pbi * 4),
+                                  Span(b.residual, pb * cb * es), Span(b.residual_mask, pb * 4), Span(b.bias, cb * es),
+                                  Span(b.out, pb * cb * es), Span(b.out_mask, pb * 4), Span(b.prev_out, pb * cb * es),
+                                  Span(b.truncated, pb * cb * es), Span(b.sum_prev_out, pb * cb * es)};
+            for (const Span &w : wr)
+                for (const Span &o : other)
+                    if (w.meets(o))
+                        return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: items %d and %d share a buffer one of them writes", i, j);
         }
     if (n_act > 1 && !dc::act_group_eligible(act, n_act, act_kind, DC_TRUNC_MAX, dtype))
         return fail(DC_ERR_UNSUPPORTED, "dc_conv_group: an activation outside the grouped kernel's range "

@@ -79,7 +79,7 @@ __device__ __forceinline__ void
 pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
              const E *__restrict__ bias, E *__restrict__ out,
              const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, const ResP<E> &rp,
-             int bx, int by, float4_t *s_red) {
+             int bx, int by, float4_t *s_red, E *s_open = nullptr) {
     typedef typename Elem16<E>::v4 E4;
     typedef typename Elem16<E>::v8 E8;
     static_assert(NBW * NTW <= 4, "a workgroup covers at most 64 pixels");
@@ -262,6 +262,35 @@ pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
         if (t >= TILES) continue;
         const int r = t / NTW, j = t % NTW;
         const int ct = ct0 + r, co = ct * 16 + kq * 4;  // Cout % 4 == 0: a lane's 4 channels are all in or all out
+        if (OPEN) {
+            // D and T of the tile go through a wavefront-private LDS tile and leave as pieces of
+            // pixel rows, 16 bytes per lane (Cout % 8 == 0): lanes 0..31 store D, lanes 32..63 T,
+            // two neighbouring lanes one pixel's 16 channels.
+            if (ct >= p.co_tiles) continue;  // the same for the whole wavefront
+            const float4_t v = fin[m] + float4_t{float(bh[m][0]), float(bh[m][1]), float(bh[m][2]), float(bh[m][3])};
+            E4 d, tq;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                tq[i] = res[m][i] + E(v[i]);
+                const E sm = tq[i] + qv[m][i];
+                d[i] = act_apply<E>(sm, act) - act_apply<E>(qv[m][i], act);
+            }
+            E *st = s_open + wave * 512;
+            *reinterpret_cast<E4 *>(st + l16 * 16 + kq * 4) = d;
+            *reinterpret_cast<E4 *>(st + 256 + l16 * 16 + kq * 4) = tq;
+            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            const int which = lane >> 5, pr = (lane & 31) >> 1, hf = lane & 1;
+            const int pbit = (nw * NTW + j) * 16 + pr, ch = ct * 16 + hf * 8;
+            const E8 piece = *reinterpret_cast<const E8 *>(st + which * 256 + pr * 16 + hf * 8);
+            if (((bm >> pbit) & 1) && ch < p.Co)
+                *reinterpret_cast<E8 *>((which ? rp.tmp : out) + (size_t)(pbase + pbit) * p.Co + ch) = piece;
+            if (FT > 1) {  // the tile is written again for the wavefront's next tile
+                __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+            }
+            continue;
+        }
         if (ct >= p.co_tiles || co >= p.Co) continue;
         const int bit = (nw * NTW + j) * 16 + l16;
         const bool on = (bm >> bit) & 1, on_r = (br >> bit) & 1;
@@ -282,16 +311,6 @@ pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
             }
             if (ADDACT) *reinterpret_cast<E4 *>(rp.prev + (size_t)(pbase + bit) * p.Co + co) = qn;
         }
-        if (OPEN) {
-            E4 tq;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                tq[i] = res[m][i] + o[i];
-                const E sm = tq[i] + qv[m][i];
-                o[i] = act_apply<E>(sm, act) - act_apply<E>(qv[m][i], act);
-            }
-            *reinterpret_cast<E4 *>(rp.tmp + (size_t)(pbase + bit) * p.Co + co) = tq;
-        }
         *reinterpret_cast<E4 *>(out + (size_t)(pbase + bit) * p.Co + co) = o;
     }
 }
@@ -302,6 +321,8 @@ pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
                const E *__restrict__ bias, E *__restrict__ out,
                const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, ResP<E> rp) {
     __shared__ float4_t s_red[KW > 1 ? KW * CBW * NBW * R * NTW * WAVE : 1];
+    // MODE 3: per wavefront one 16 x 16 tile each of D and T on their way into pixel rows
+    __shared__ __align__(16) E s_open[MODE == 3 ? KW * CBW * NBW * 512 : 8];
     int bx = blockIdx.x, by = blockIdx.y;
     if (p.xcd) {
         const int slot = blockIdx.x >> 3;
@@ -309,7 +330,8 @@ pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
         bx = slot % p.nx;
         if (by >= p.ny) return;  // padding of the channel groups to a multiple of 8
     }
-    pw_mfma_body<E, KW, CBW, NBW, R, NTW, S, MODE, EAGER, ACTC>(p, in, wp, bias, out, mask, out_mask, rp, bx, by, s_red);
+    pw_mfma_body<E, KW, CBW, NBW, R, NTW, S, MODE, EAGER, ACTC>(p, in, wp, bias, out, mask, out_mask, rp, bx, by, s_red,
+                                                                 s_open);
 }
 
 // Several independent small pointwise layers in ONE launch (the 1x1 convolutions of a
@@ -1185,9 +1207,10 @@ hipError_t launch_pointwise_group(const ConvGroupItem *items, int n, int dtype, 
     return launch_pointwise_group_t<half_t>(items, n, s);
 }
 
-// ReLU and ReLU6 (what the layers in front of depthwise convolutions use) are instantiated.
+// ReLU and ReLU6 (what the layers in front of depthwise convolutions use) are instantiated; output
+// channels in multiples of 8: D and T leave as 16-byte pieces of pixel rows.
 bool pointwise_open_eligible(const dc_geometry &g, int dtype, int activation) {
-    return pointwise_eligible(g, dtype) && (activation == DC_ACT_RELU || activation == DC_ACT_RELU6);
+    return pointwise_eligible(g, dtype) && g.out_c % 8 == 0 && (activation == DC_ACT_RELU || activation == DC_ACT_RELU6);
 }
 
 // The pointwise convolution of a layer whose activation / truncation is left open (MODE 3 of

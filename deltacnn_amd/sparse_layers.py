@@ -625,6 +625,10 @@ def project_expand(project, add, residual, expand, depthwise, input):
     if plan_e["out"] is None:
         return None
     plan_d = depthwise._plan_for(plan_e["out"].shape, x.dtype, x.device)
+    # everything the closing call will need, before the launch that cannot be taken back
+    if plan_d["out"] is None or any(not _matches(t, plan_e["out"]) for t in (act_e.prev_out, act_e.out_truncated)) \
+            or any(not _matches(t, plan_d["out"]) for t in (act_d.prev_out, act_d.out_truncated)):
+        return None
     out, out_mask = plan_p["out"], plan_p["out_mask"]
     res_v = res_m = None
     wa = wb = 1.0
@@ -674,10 +678,10 @@ def expand_depthwise(expand, depthwise, input, opened=None):
     act_e, act_d = acts
     plan_e = expand._plan_for(x.shape, x.dtype, x.device)
     packed = expand._packed_filter()
-    if packed is None or plan_e["out"] is None:
-        return None
-    plan_d = depthwise._plan_for(plan_e["out"].shape, x.dtype, x.device)
-    if plan_d["out"] is None:
+    plan_d = None if plan_e["out"] is None else depthwise._plan_for(plan_e["out"].shape, x.dtype, x.device)
+    if packed is None or plan_d is None or plan_d["out"] is None:
+        if opened is not None:  # the expansion's state already holds T: there is no way back
+            raise RuntimeError("the layers of an open expansion lost their buffers before it was finished")
         return None
     done = hk.sparse_expand_depthwise(
         x, mask, packed, act_e.prev_out, act_e.out_truncated, DCThreshold.get(act_e), act_e.activation_int,

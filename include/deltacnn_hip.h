@@ -221,7 +221,8 @@ typedef struct dc_expand_dw_args {
  * the pixels it keeps are meaningful (as always), and expand_out_mask receives its convolution's
  * update mask rather than the keep mask.  For the small maps where launches are the cost:
  * shapes outside the range (see dc_last_error) return DC_ERR_UNSUPPORTED before any launch so
- * that the caller can issue the separate calls.  16-bit types; no bias (a layer's bias belongs
+ * that the caller can issue the separate calls.  16-bit types, the expansion's output channels in
+ * multiples of 8; no bias (a layer's bias belongs
  * to its first frame, which takes the separate calls).  No counterpart in the reference, which
  * launches every layer and every activation on its own (sparse_layers.py:636-638). */
 int dc_expand_depthwise(const dc_geometry *g, const dc_expand_dw_args *args, int dtype, void *stream);
@@ -264,7 +265,11 @@ typedef struct dc_project_expand_args {
  * stand-alone pointwise kernel would split the projection's reduction over four wavefronts and
  * the expansion's over none.  Together the two calls are identical, bit for bit, to
  * dc_conv / dc_conv_add(projection), dc_conv_act(expansion), dc_conv_act(depthwise).  16-bit
- * types; no bias.  No counterpart in the reference (sparse_layers.py:636-638). */
+ * types; no bias.  Several workgroups per pixel tile read every input of the call while one of
+ * them stores the block output, so nothing is summed in place: out, out_mask, expand_out,
+ * expand_out_mask and expand_truncated must not overlap input, mask, residual, residual_mask,
+ * expand_prev_out, the filters or one another (DC_ERR_UNSUPPORTED otherwise).  No counterpart in
+ * the reference (sparse_layers.py:636-638). */
 int dc_project_expand(const dc_geometry *g, const dc_project_expand_args *args, int dtype, void *stream);
 
 /* One layer of a dc_conv_group call. */

@@ -346,6 +346,22 @@ def test_project_expand_arguments_are_checked_before_any_launch(lib):
     assert call(g, args(residual_mask=None)) == -4                         # a residual needs its mask
     assert call(g, args(input=p + 2)) == -5 and call(g, args(expand_prev_out=p + 8)) == -5
 
+    # nothing is summed in place: several workgroups read every input while one stores the outputs
+    big = (ctypes.c_char * (4 << 20))()
+    q = (ctypes.addressof(big) + 255) // 256 * 256
+    names = ("input", "mask", "project_packed_filter", "residual", "residual_mask", "out", "out_mask",
+             "expand_packed_filter", "expand_prev_out", "expand_truncated", "expand_out", "expand_out_mask")
+    apart = {n: q + i * (256 << 10) for i, n in enumerate(names)}      # 256 KB each: larger than any operand
+    for written, read in (("out", "residual"), ("out", "input"), ("out_mask", "mask"), ("expand_out_mask", "residual_mask"),
+                          ("out_mask", "residual_mask"), ("expand_out", "out"), ("expand_truncated", "expand_prev_out"),
+                          ("expand_out", "expand_truncated"), ("out_mask", "expand_out_mask")):
+        alias = dict(apart)
+        alias[written] = apart[read]
+        assert call(g, args(**alias)) == -3 and b"overlap" in lib.dc_last_error(), (written, read)
+    partly = dict(apart)
+    partly["out"] = apart["residual"] + 1024                               # a view into the same allocation
+    assert call(g, args(**partly)) == -3 and b"overlap" in lib.dc_last_error()
+
     # the second call of the pair: no expansion filter, no input, but every state tensor
     b = ExpandDwArgs()
     for name in ("expand_prev_out", "expand_truncated", "expand_out", "expand_out_mask", "dw_filter", "dw_prev_out",
@@ -405,6 +421,21 @@ def test_conv_group_arguments_are_checked_before_any_launch(lib):
     assert call([item(0, **act(0, 1)), item(1, **act(1, 3))]) == -3 and b"activations" in lib.dc_last_error()
     assert call([item(0), item(1, out=base + 3 * 256)]) == -3 and b"share" in lib.dc_last_error()
     assert call([item(0), item(1, input=base + 3 * 256)]) == -3            # item 1 reads what item 0 writes
+    # byte ranges, not pointers: views into one allocation, and every buffer an item writes
+    wide = (ctypes.c_char * (4 << 20))()
+    w0 = (ctypes.addressof(wide) + 255) // 256 * 256
+
+    def roomy(k, **kw):  # 16 x 16 x 64 channels = 32 KB per tensor, 64 KB apart
+        names = ("input", "mask", "packed_filter", "out", "out_mask", "prev_out", "truncated")
+        d = {n: w0 + (k * 8 + j) * (64 << 10) for j, n in enumerate(names)}
+        d.update(threshold=0.05, activation=1, truncation_mode=0)
+        d.update(kw)
+        return item(k, **d)
+
+    for kw in (dict(out=w0 + 3 * (64 << 10) + 512), dict(input=w0 + 5 * (64 << 10) + 64),
+               dict(prev_out=w0 + 3 * (64 << 10)), dict(truncated=w0 + 0 * (64 << 10) + 4096),
+               dict(out_mask=w0 + 1 * (64 << 10) + 16)):
+        assert call([roomy(0), roomy(1, **kw)]) == -3 and b"share" in lib.dc_last_error(), kw
     assert call([item(0, residual=base + 1024)]) == -2                       # still one item
     assert call([item(0), item(1, residual=base + 4096 + 1024)]) == -4       # a residual needs its mask
 
