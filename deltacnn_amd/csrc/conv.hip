@@ -979,11 +979,14 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
     typedef typename Elem16<E>::v4 E4;
     typedef typename Elem16<E>::v8 E8;
     constexpr int NT = 4;
+    constexpr int TPW = R * NT / KS;  // output tiles of 16 x 16 a wavefront finishes
+    static_assert(TPW * KS == R * NT, "the reduction slices of a channel group share its tiles evenly");
     extern __shared__ __align__(16) unsigned char s_halo[];
     __shared__ int s_hpix[LDS_MAX_HALO];
     __shared__ int2 s_step[LDS_MAX_STEPS];
-    __shared__ int s_list[TILE_PX];  // compacted tile pixels: index | 64 if updated | 128 if the residual is
-    __shared__ int s_n, s_nupd;
+    // compacted tile pixels (index | 64 if updated | 128 if the residual is), one copy per wavefront:
+    // every wavefront dilates and compacts the mask itself
+    __shared__ int s_list[8][TILE_PX];
     const int b = blockIdx.z / co_blocks, cb = blockIdx.z % co_blocks;
     // TR (transposed, dilation 1): the outputs of one stride phase (py, px) form an ordinary
     // convolution of the input with the A x Bt filter taps ky = ry + a * stride, kx = rx + b * stride:
@@ -1040,19 +1043,54 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
         }
         return;
     }
-    // halo table: global pixel index of every active in-bounds halo pixel, -1 otherwise.  The
-    // mask word of a thread's first halo pixel is requested before the step table is built, so
-    // the table's arithmetic runs while it travels.
-    auto halo_pixel = [&](int i, bool &ok) {
+    // Front end.  Nothing in it waits for anything it does not need: the mask word of halo pixel
+    // `tid` and the halo ROWS of this lane's staging slots are requested first, the rows from
+    // addresses that follow from the tile's coordinates alone (what an inactive pixel returns is
+    // zeroed when it is stored); the step table is built while they travel; the filter chunks are
+    // requested behind the rows, so that the rows are not queued behind them.
+    auto halo_pixel = [&](int i, bool &ok) {  // position in the input map (clamped into it), and whether it lies inside
         const int hy = i / hal_w, hx = i - hy * hal_w;
         const int iy = iy0 + hy, ix = ix0 + hx;
         ok = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
-        return ok ? iy * p.Wi + ix : 0;
+        return min(max(iy, 0), p.Hi - 1) * p.Wi + min(max(ix, 0), p.Wi - 1);
     };
     bool ok0;
     const int hpix0 = halo_pixel(min(tid, hpx - 1), ok0);
     const int hword0 = mb[hpix0];
+    // Staging of channels [kbase * 32, (kbase + kcur) * 32) of the halo: 2^lgv lanes per pixel, SU
+    // pixels per lane in flight (a 10 x 10 halo is one pass); inactive pixels are stored as zeros.
+    constexpr int SU = 8;
+    const E *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
+    const int sv = tid & ((1 << lgv) - 1), hstep = nthr >> lgv;
+    E8 val0[SU];
+    {
+        const int c = min(sv * 8, p.Ci - 8);
+        // slot u of this lane lies hstep halo pixels behind slot u - 1: row and column follow from
+        // one division
+        const int dy = hstep / hal_w, dx = hstep - dy * hal_w;  // uniform
+        int hy = (tid >> lgv) / hal_w, hx = (tid >> lgv) - hy * hal_w;
+#pragma unroll
+        for (int u = 0; u < SU; ++u) {
+            const bool in_halo = hy < hal_h;  // past the halo: the last pixel again, not stored
+            const int iy = iy0 + (in_halo ? hy : hal_h - 1), ix = ix0 + (in_halo ? hx : hal_w - 1);
+            const int px = min(max(iy, 0), p.Hi - 1) * p.Wi + min(max(ix, 0), p.Wi - 1);
+            val0[u] = *reinterpret_cast<const E8 *>(inb + (size_t)px * p.Ci + c);
+            hx += dx;
+            hy += dy;
+            if (hx >= hal_w) {
+                hx -= hal_w;
+                ++hy;
+            }
+        }
+    }
+    // the tile pixel of this lane (every wavefront dilates the mask for all 64 pixels itself)
+    const int ly = lane >> 3, lx = lane & 7;
+    const int oy = out_y(ly), ox = out_x(lx);
+    const bool inside = oy < p.Ho && ox < p.Wo;
+    int rword = 0;  // ADD: the residual's mask word
+    if (ADD) rword = rs.mask[((size_t)b * p.Ho + min(oy, p.Ho - 1)) * p.Wo + min(ox, p.Wo - 1)];
     build_steps(0, min(kcc, ksteps));
+    // mask words -> pixel table: global pixel index of every active in-bounds halo pixel, else -1
     if (tid < hpx) s_hpix[tid] = (ok0 && hword0 != 0) ? hpix0 : -1;
     for (int i = tid + nthr; i < hpx; i += nthr) {
         bool ok;
@@ -1085,21 +1123,15 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
     };
 #pragma unroll
     for (int d = 0; d < D; ++d) load_chunk(a[d], xo[d]);
-    E bv[R][4];  // bias of the lane's four channels per tile, requested early as well
+    // bias of the lane's four channels for the tiles this wavefront finishes: tiles
+    // [kz * TPW, (kz + 1) * TPW) of its channel group, tile t = (channel tile t / NT, pixel tile t % NT)
+    E bv[TPW][4];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int co = ((cb * ncw + cw) * R + r) * 16 + kq * 4;
+    for (int q = 0; q < TPW; ++q) {
+        const int co = ((cb * ncw + cw) * R + (kz * TPW + q) / NT) * 16 + kq * 4;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) bv[r][i] = bias != nullptr ? bias[min(co + i, p.Co - 1)] : E(0);
+        for (int i = 0; i < 4; ++i) bv[q][i] = bias != nullptr ? bias[min(co + i, p.Co - 1)] : E(0);
     }
-
-    // Staging of channels [kbase * 32, (kbase + kcur) * 32) of the halo: 2^lgv lanes per pixel, SU
-    // pixels per lane in flight (a 10 x 10 halo is one pass); inactive pixels read one shared
-    // dummy address and are stored as zeros.  The first pass of the first channel chunk is
-    // requested here, so that it travels while the first wavefront dilates the mask.
-    constexpr int SU = 8;
-    const E *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci;
-    const int sv = tid & ((1 << lgv) - 1), hstep = nthr >> lgv;
     auto stage_load = [&](int kbase, int h0, E8 (&val)[SU], int (&px)[SU]) {
         const int c = min((kbase << 5) + sv * 8, p.Ci - 8);
 #pragma unroll
@@ -1117,16 +1149,12 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
                 *reinterpret_cast<E8 *>(s_halo + hp * row + sv * 16) = keep8(val[u], vok && px[u] >= 0);
         }
     };
-    E8 val0[SU];
-    int px0[SU];
-    stage_load(0, tid >> lgv, val0, px0);
 
-    if (tid < WAVE) {  // dilate the mask over the window, compact the updated pixels
-        const int ly = tid >> 3, lx = tid & 7;
-        const int oy = out_y(ly), ox = out_x(lx);
-        const bool inb = oy < p.Ho && ox < p.Wo;
-        int rword = 0;  // ADD: the residual's mask word, requested before the window is examined
-        if (ADD) rword = rs.mask[((size_t)b * p.Ho + min(oy, p.Ho - 1)) * p.Wo + min(ox, p.Wo - 1)];
+    // dilate the mask over the window and compact the updated pixels: by every wavefront for itself
+    // (the same table, hence the same list in all of them), while the halo rows are still travelling
+    int n;
+    bool tile_upd;
+    {
         bool upd = false;
         const int base = ly * vsy * hal_w + lx * vsx;
         if (!TR && p.Kh == 3 && p.Kw == 3) {  // the common window: nine independent reads
@@ -1136,56 +1164,55 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
             for (int ta = 0; ta < A; ++ta)
                 for (int tb = 0; tb < Bt; ++tb) upd |= s_hpix[base + tap_off(ta, tb)] >= 0;
         }
-        upd = upd && inb;
-        const bool radd = ADD && inb && rword != 0;
+        upd = upd && inside;
+        const bool radd = ADD && inside && rword != 0;
         const bool any = upd || radd;  // ADD: the union of both masks is written and compacted
-        if (inb && cb == 0) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = any ? 1 : 0;
-        int n;
+        if (inside && cb == 0 && wv == 0) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = any ? 1 : 0;
         const int rank = wave_rank(any, n);
-        if (any) s_list[rank] = tid | (upd ? 64 : 0) | (radd ? 128 : 0);
-        const bool tile_upd = ballot(upd) != 0;
-        if (tid == 0) {
-            s_n = n;
-            s_nupd = tile_upd ? 1 : 0;
-        }
+        if (any) s_list[wv][rank] = lane | (upd ? 64 : 0) | (radd ? 128 : 0);
+        tile_upd = ballot(upd) != 0;
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
     }
-    stage_store(0, min(kcc, ksteps), tid >> lgv, val0, px0);
+    if (n == 0) return;  // the same in every wavefront
+    {   // the rows requested at the start: into LDS, those of inactive pixels as zeros
+        int px0[SU];
+#pragma unroll
+        for (int u = 0; u < SU; ++u) px0[u] = s_hpix[min((tid >> lgv) + u * hstep, hpx - 1)];
+        stage_store(0, min(kcc, ksteps), tid >> lgv, val0, px0);
+    }
     __syncthreads();
-    const int n = s_n;
-    if (n == 0) return;
 
     const int n_tiles = (n + 15) >> 4;
     int hbase[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int slot = nt * 16 + l16;
-        const int loc = slot < n ? (s_list[slot] & 63) : 0;
+        const int loc = slot < n ? (s_list[wv][slot] & 63) : 0;
         hbase[nt] = ((loc >> 3) * vsy * hal_w + (loc & 7) * vsx) * row + kq * 16;
     }
-    // ADD: the operands of the sum for all tiles of this lane, requested before the reduction,
-    // which they overlap
-    E4 rv[ADD ? R : 1][ADD ? NT : 1];
-    if (ADD && kz == 0) {
+    // ADD: the operands of the sum for the tiles this wavefront finishes, requested before the
+    // reduction, which they overlap
+    E4 rv[ADD ? TPW : 1];
+    if (ADD) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int co = ((cb * ncw + cw) * R + r) * 16 + kq * 4;
+        for (int q = 0; q < TPW; ++q) {
+            const int t = kz * TPW + q, nt = t % NT;
+            const int co = ((cb * ncw + cw) * R + t / NT) * 16 + kq * 4;
             const bool vec = co + 3 < p.Co && (p.Co & 3) == 0;
+            rv[q] = zero4<E>();
+            const int pix = nt * 16 + l16;
+            if (pix >= n || co >= p.Co) continue;
+            const int code = s_list[wv][pix], loc = code & 63;
+            const size_t off = (((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7)) * p.Co;
+            const bool radd = (code & 128) != 0;
+            if (vec) {
+                if (radd) rv[q] = *reinterpret_cast<const E4 *>(rs.values + off + co);
+            } else {
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                rv[r][nt] = zero4<E>();
-                const int pix = nt * 16 + l16;
-                if (pix >= n || co >= p.Co) continue;
-                const int code = s_list[pix], loc = code & 63;
-                const size_t off = (((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7)) * p.Co;
-                const bool radd = (code & 128) != 0;
-                if (vec) {
-                    if (radd) rv[r][nt] = *reinterpret_cast<const E4 *>(rs.values + off + co);
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int c = min(co + i, p.Co - 1);
-                        if (radd) rv[r][nt][i] = rs.values[off + c];
-                    }
+                for (int i = 0; i < 4; ++i) {
+                    const int c = min(co + i, p.Co - 1);
+                    if (radd) rv[q][i] = rs.values[off + c];
                 }
             }
         }
@@ -1197,7 +1224,7 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
         for (int nt = 0; nt < NT; ++nt) acc[r][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // ADD: a tile reached by the residual only has nothing to contract (uniform)
-    const int kend = (ADD && s_nupd == 0) ? 0 : ksteps;
+    const int kend = (ADD && !tile_upd) ? 0 : ksteps;
     for (int kbase = 0; kbase < kend; kbase += kcc) {
         const int kcur = min(kcc, ksteps - kbase);
         if (kbase > 0) {
@@ -1275,60 +1302,62 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
         }
     }
 
-    if (KS > 1) {  // partial sums of the reduction slices meet in LDS (the halo is no longer needed)
+    // The partial sums of the reduction slices meet in LDS (the halo is no longer needed), added in
+    // ascending slice order; the KS wavefronts of a channel group share the finishing of its R * NT
+    // tiles, TPW each.
+    float4_t fin[TPW];
+    if (KS > 1) {
         float4_t *s_part = reinterpret_cast<float4_t *>(s_halo);
         __syncthreads();
-        if (kz > 0) {
 #pragma unroll
-            for (int r = 0; r < R; ++r)
+        for (int r = 0; r < R; ++r)
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    s_part[((((kz - 1) * ncw + cw) * R + r) * NT + nt) * WAVE + lane] = acc[r][nt];
-        }
+            for (int nt = 0; nt < NT; ++nt)
+                s_part[(((kz * ncw + cw) * R + r) * NT + nt) * WAVE + lane] = acc[r][nt];
         __syncthreads();
-        if (kz > 0) return;
 #pragma unroll
-        for (int q = 1; q < KS; ++q)  // ascending slice order
+        for (int q = 0; q < TPW; ++q) {
+            const int t = kz * TPW + q;  // r * NT + nt
+            fin[q] = s_part[((0 * ncw + cw) * R * NT + t) * WAVE + lane];
 #pragma unroll
-            for (int r = 0; r < R; ++r)
+            for (int z = 1; z < KS; ++z) fin[q] += s_part[((z * ncw + cw) * R * NT + t) * WAVE + lane];
+        }
+    } else {
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    acc[r][nt] += s_part[((((q - 1) * ncw + cw) * R + r) * NT + nt) * WAVE + lane];
+        for (int q = 0; q < TPW; ++q) fin[q] = acc[q / NT][q % NT];
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int ct = (cb * ncw + cw) * R + r;
+    for (int q = 0; q < TPW; ++q) {
+        const int t = kz * TPW + q, nt = t % NT;
+        const int ct = (cb * ncw + cw) * R + t / NT;
         if (ct >= co_tiles) continue;
         const int co = ct * 16 + kq * 4;  // lane holds channels co .. co + 3 of pixel (nt, l16)
+        const int pix = nt * 16 + l16;
+        if (pix >= n) continue;
+        const int code = s_list[wv][pix], loc = code & 63;
+        const size_t opix = ((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7);
+        E *o = out + opix * p.Co + co;
+        const bool vec = co + 3 < p.Co && (p.Co & 3) == 0;
+        E4 v;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const int pix = nt * 16 + l16;
-            if (pix >= n) continue;
-            const int code = s_list[pix], loc = code & 63;
-            const size_t opix = ((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7);
-            E *o = out + opix * p.Co + co;
-            const bool vec = co + 3 < p.Co && (p.Co & 3) == 0;
-            E4 v;
+        for (int i = 0; i < 4; ++i) v[i] = E(fin[q][i] + float(bv[q][i]));
+        if (ADD) {  // add_kernel's sequence on the rounded convolution result: s = a * wa; s = fma(b, wb, s)
+            const bool upd = (code & 64) != 0, radd = (code & 128) != 0;
+            const E wa = E(rs.wa), wb = E(rs.wb);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = E(acc[r][nt][i] + float(bv[r][i]));
-            if (ADD) {  // add_kernel's sequence on the rounded convolution result: s = a * wa; s = fma(b, wb, s)
-                const bool upd = (code & 64) != 0, radd = (code & 128) != 0;
-                const E wa = E(rs.wa), wb = E(rs.wb);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    E sum = E(0);
-                    if (radd) sum = rv[r][nt][i] * wa;
-                    if (upd) sum = fma_t(v[i], wb, sum);
-                    v[i] = sum;
-                }
+            for (int i = 0; i < 4; ++i) {
+                E sum = E(0);
+                if (radd) sum = rv[q][i] * wa;
+                if (upd) sum = fma_t(v[i], wb, sum);
+                v[i] = sum;
             }
-            if (vec) {
-                *reinterpret_cast<E4 *>(o) = v;
-            } else {
+        }
+        if (vec) {
+            *reinterpret_cast<E4 *>(o) = v;
+        } else {
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (co + i < p.Co) o[i] = v[i];
-            }
+            for (int i = 0; i < 4; ++i)
+                if (co + i < p.Co) o[i] = v[i];
         }
     }
 }
@@ -2309,7 +2338,7 @@ hipError_t launch_lds_conv(const dc_geometry &g, const ConvP &p, const LdsPlan &
     const int kcc = lp.kcc, hal_h = lp.hal_h, hal_w = lp.hal_w;
     const int nwv = lp.ncw * lp.ksl;  // wavefronts per workgroup
     const int cbl = ceil_div(co_tiles, lp.ncw * lp.rl);
-    const size_t lds = std::max((size_t)hpx * (kcc * 64 + 16), (size_t)(lp.ksl - 1) * lp.ncw * lp.rl * 4 * 1024);
+    const size_t lds = std::max((size_t)hpx * (kcc * 64 + 16), lp.ksl > 1 ? (size_t)lp.ksl * lp.ncw * lp.rl * 4 * 1024 : 0);
     const int lgv = log2i(pow2_ceil(kcc * 4));  // lanes per halo pixel while staging
     dim3 lgrid(lp.ltx, lp.lty, g.batch * cbl);
     PatchRes<E> rs{nullptr, nullptr, nullptr, 0.f, 0.f, 0};
