@@ -105,7 +105,10 @@ _SIGNATURES = {
     "dc_packed_filter_bytes": (c_int64, [_G, c_int, c_int]),
     "dc_pack_filter": (c_int, [_G, _P, _P, c_int, c_int, _P]),
     "dc_deconv": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_int, _P]),
+    "dc_deconv_add": (c_int, [_G, _P, _P, _P, _P, _P, _P, _P, c_float, c_float, c_int, _P]),
     "dc_pool": (c_int, [_G, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P]),
+    "dc_pool_update": (c_int, [_G, _P, _P, _P, _P, _P, c_int, _P]),
+    "dc_concat_conv": (c_int, [_G, c_int, _P, _P, _P, _P, _P, _P, c_int, _P]),
     "dc_densify": (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int, _P]),
     "dc_pool_densify": (c_int, [_G, _P, _P, _P, _P, c_int, _P]),
     "dc_linear": (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int32, c_int, _P]),

@@ -309,6 +309,10 @@ bool depthwise_closing_eligible(const dc_geometry &g, const ActEpilogue *epi, in
 hipError_t launch_depthwise_closing(const dc_geometry &g, const void *in, const void *filter, void *out,
                                     const int32_t *mask, int32_t *out_mask, const ActEpilogue *epi,
                                     const OpenAct &open, int dtype, hipStream_t s);
+bool pointwise_concat_eligible(const dc_geometry &g, const int32_t *channels, int n, int dtype);
+hipError_t launch_pointwise_concat(const dc_geometry &g, const void *const *inputs, const int32_t *const *masks,
+                                   const int32_t *channels, int n, const void *packed, void *out, int32_t *out_mask,
+                                   int dtype, hipStream_t s);
 bool pointwise_open_eligible(const dc_geometry &g, int dtype, int activation);
 hipError_t launch_pointwise_open(const dc_geometry &g, const void *in, const void *packed, void *out,
                                  const int32_t *mask, int32_t *out_mask, const OpenAct &open, int dtype,
@@ -321,10 +325,10 @@ hipError_t launch_pointwise_pair(const dc_geometry &gp, const void *in, const in
                                  void *expand_out, int32_t *expand_out_mask, int dtype, hipStream_t s);
 bool pointwise_eligible(const dc_geometry &g, int dtype);
 bool patch_eligible(const dc_geometry &g, int dtype);
-bool lds_add_eligible(const dc_geometry &g, int dtype, int activation);
+bool lds_add_eligible(const dc_geometry &g, int dtype, int activation, bool transposed = false);
 hipError_t launch_lds_conv_add(const dc_geometry &g, const void *in, const void *packed, const void *bias,
                                void *out, const int32_t *mask, int32_t *out_mask, const Residual *res,
-                               int dtype, hipStream_t s);
+                               int dtype, hipStream_t s, bool transposed = false);
 hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *packed,
                              const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
                              bool transposed, const Residual *res, int dtype, hipStream_t s,
@@ -382,6 +386,9 @@ hipError_t launch_pack_filter(const dc_geometry &g, const void *filter, void *pa
 int64_t packed_filter_bytes(const dc_geometry &g, int dtype, bool transposed);
 hipError_t launch_densify(const void *delta, void *prev, void *out, const int32_t *mask, int P, int C,
                           int dtype, hipStream_t s);
+bool pool_update_eligible(const dc_geometry &g, const void *in, const void *prev, const void *out, int dtype);
+hipError_t launch_pool_update(const dc_geometry &g, const void *in, void *prev, void *out, const int32_t *mask,
+                              int32_t *out_mask, int dtype, hipStream_t s);
 hipError_t launch_pool(const dc_geometry &g, const void *in, const void *prev, void *out,
                        const int32_t *mask, int32_t *out_mask, int mode, int dtype, bool out_f32,
                        hipStream_t s);

@@ -975,7 +975,7 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
     // ADD: the sum of a DCAdd without activation rides on the accumulators.  (With an activation the
     // accumulated sum has to be read and written as well; in this kernel's 8-byte-per-lane epilogue
     // that costs what the separate add kernel costs -- measured -- so that form is not offered.)
-    static_assert(!(ADD && TR), "the fused sum exists for plain convolutions only");
+    // ADD && TR: a transposed convolution whose every stride phase has taps (window >= stride).
     typedef typename Elem16<E>::v4 E4;
     typedef typename Elem16<E>::v8 E8;
     constexpr int NT = 4;
@@ -2355,7 +2355,8 @@ hipError_t launch_lds_conv(const dc_geometry &g, const ConvP &p, const LdsPlan &
     } while (0)
 #define DC_LDS_L(RV, SV, DV, KV)                                                                            \
     do {                                                                                                    \
-        if (res != nullptr) DC_LDS_K(RV, SV, DV, KV, false, true);                                          \
+        if (res != nullptr && transposed) DC_LDS_K(RV, SV, DV, KV, true, true);                             \
+        else if (res != nullptr) DC_LDS_K(RV, SV, DV, KV, false, true);                                     \
         else if (transposed) DC_LDS_K(RV, SV, DV, KV, true, false);                                         \
         else DC_LDS_K(RV, SV, DV, KV, false, false);                                                        \
     } while (0)
@@ -2446,20 +2447,23 @@ hipError_t launch_patch_conv_t(const dc_geometry &g, const void *in, const void 
 }
 }  // namespace
 
-// Layers of the LDS-halo kernel (larger K x K convolutions) have the fused residual sum too, for a
-// DCAdd without activation.
-bool lds_add_eligible(const dc_geometry &g, int dtype, int activation) {
+// Layers of the LDS-halo kernel (larger K x K convolutions, plain or transposed) have the fused
+// residual sum too, for a DCAdd without activation.
+bool lds_add_eligible(const dc_geometry &g, int dtype, int activation, bool transposed) {
+    // transposed: every stride phase of the output needs at least one tap (window >= stride), so
+    // that every output tile runs the reduction kernel's epilogue
+    if (transposed && (g.kernel_h < g.stride_h || g.kernel_w < g.stride_w)) return false;
     return activation <= 0 && mfma_eligible(g, dtype) && g.kernel_h * g.kernel_w <= MFMA_MAX_TAPS && !patch_eligible(g, dtype) &&
-           lds_plan(g, false).ok;
+           lds_plan(g, transposed).ok;
 }
 
 hipError_t launch_lds_conv_add(const dc_geometry &g, const void *in, const void *packed, const void *bias,
                                void *out, const int32_t *mask, int32_t *out_mask, const Residual *res,
-                               int dtype, hipStream_t s) {
+                               int dtype, hipStream_t s, bool transposed) {
     const ConvP p = make_params(g, DC_F16);  // the packed filter's layout does not depend on the type
-    const LdsPlan lp = lds_plan(g, false);
-    if (dtype == DC_BF16) return launch_lds_conv<bf16_t>(g, p, lp, in, packed, bias, out, mask, out_mask, false, res, s);
-    return launch_lds_conv<half_t>(g, p, lp, in, packed, bias, out, mask, out_mask, false, res, s);
+    const LdsPlan lp = lds_plan(g, transposed);
+    if (dtype == DC_BF16) return launch_lds_conv<bf16_t>(g, p, lp, in, packed, bias, out, mask, out_mask, transposed, res, s);
+    return launch_lds_conv<half_t>(g, p, lp, in, packed, bias, out, mask, out_mask, transposed, res, s);
 }
 
 hipError_t launch_patch_conv(const dc_geometry &g, const void *in, const void *packed,

@@ -282,6 +282,45 @@ int dc_deconv(const dc_geometry *g, const void *input, const void *filter,
                                   dtype, true, nullptr, (hipStream_t)stream), "dc_deconv");
 }
 
+int dc_deconv_add(const dc_geometry *g, const void *input, const void *packed_filter, const int32_t *mask,
+                  const void *residual, const int32_t *mask_residual, void *out, int32_t *out_mask,
+                  float weight_residual, float weight_conv, int dtype, void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_deconv_add");
+    int rc = check_geometry("dc_deconv_add", g, true, false);
+    if (rc != DC_OK) return rc;
+    if (!dc::lds_add_eligible(*g, dtype, 0, true))
+        return fail(DC_ERR_UNSUPPORTED, "dc_deconv_add: only 16-bit transposed convolutions of the LDS-halo kernel "
+                                        "(Cin %% 8 == 0, groups 1, dilation 1, window >= stride, too large for the "
+                                        "4x4-patch kernel) have the fused form");
+    DC_REQUIRE_PTR("dc_deconv_add", input);
+    DC_REQUIRE_PTR("dc_deconv_add", packed_filter);
+    DC_REQUIRE_PTR("dc_deconv_add", mask);
+    DC_REQUIRE_PTR("dc_deconv_add", residual);
+    DC_REQUIRE_PTR("dc_deconv_add", mask_residual);
+    DC_REQUIRE_PTR("dc_deconv_add", out);
+    DC_REQUIRE_PTR("dc_deconv_add", out_mask);
+    DC_REQUIRE_ALIGNED("dc_deconv_add", input, 16);
+    DC_REQUIRE_ALIGNED("dc_deconv_add", packed_filter, 16);
+    DC_REQUIRE_ALIGNED("dc_deconv_add", residual, 8);
+    DC_REQUIRE_ALIGNED("dc_deconv_add", out, 8);
+    {
+        // every output tile reads the residual of its pixels and other tiles' workgroups may have
+        // stored theirs by then: the sum is not taken in place
+        const size_t po = (size_t)g->batch * g->out_h * g->out_w, es = esize(dtype);
+        const Span o(out, po * g->out_c * es), om(out_mask, po * 4);
+        const Span rd[] = {Span(residual, po * g->out_c * es), Span(mask_residual, po * 4),
+                           Span(input, (size_t)g->batch * g->in_h * g->in_w * g->in_c * es),
+                           Span(mask, (size_t)g->batch * g->in_h * g->in_w * 4)};
+        for (const Span &r : rd)
+            if (o.meets(r) || om.meets(r))
+                return fail(DC_ERR_UNSUPPORTED, "dc_deconv_add: out / out_mask overlap an input of the call");
+    }
+    dc::Residual res{residual, mask_residual, weight_residual, weight_conv, nullptr, 0};
+    return finish(dc::launch_lds_conv_add(*g, input, packed_filter, nullptr, out, mask, out_mask, &res, dtype,
+                                          (hipStream_t)stream, true), "dc_deconv_add");
+}
+
 int dc_pool(const dc_geometry *g, const void *input, const void *prev_input, void *out,
             const int32_t *mask, int32_t *out_mask, int pooling_mode, int dtype,
             int global_out_dtype, void *stream) {
@@ -311,6 +350,72 @@ int dc_pool(const dc_geometry *g, const void *input, const void *prev_input, voi
     DC_REQUIRE_ALIGNED("dc_pool", out, (global && out_f32) ? 4 : esize(dtype));
     return finish(dc::launch_pool(*g, input, prev_input, out, mask, out_mask, pooling_mode, dtype,
                                   out_f32, (hipStream_t)stream), "dc_pool");
+}
+
+int dc_concat_conv(const dc_geometry *g, int32_t count, const void *const *inputs, const int32_t *const *masks,
+                   const int32_t *channels, const void *packed_filter, void *out, int32_t *out_mask, int dtype,
+                   void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_concat_conv");
+    int rc = check_geometry("dc_concat_conv", g, false, false);
+    if (rc != DC_OK) return rc;
+    if (count < 2 || count > 4)
+        return fail(DC_ERR_SHAPE, "dc_concat_conv: count=%d outside 2..4", count);
+    DC_REQUIRE_PTR("dc_concat_conv", inputs);
+    DC_REQUIRE_PTR("dc_concat_conv", masks);
+    DC_REQUIRE_PTR("dc_concat_conv", channels);
+    if (!dc::pointwise_concat_eligible(*g, channels, count, dtype))
+        return fail(DC_ERR_UNSUPPORTED, "dc_concat_conv: needs a 16-bit 1x1 stride-1 convolution without padding "
+                                        "(Cout %% 4 == 0) over tensors with channels in multiples of 32 that add up "
+                                        "to in_c");
+    DC_REQUIRE_PTR("dc_concat_conv", packed_filter);
+    DC_REQUIRE_PTR("dc_concat_conv", out);
+    DC_REQUIRE_PTR("dc_concat_conv", out_mask);
+    DC_REQUIRE_ALIGNED("dc_concat_conv", packed_filter, 16);
+    DC_REQUIRE_ALIGNED("dc_concat_conv", out, 8);
+    const size_t P = (size_t)g->batch * g->in_h * g->in_w, es = esize(dtype);
+    const Span o(out, P * g->out_c * es), om(out_mask, P * 4);
+    for (int i = 0; i < count; ++i) {
+        if (inputs[i] == nullptr || masks[i] == nullptr)
+            return fail(DC_ERR_NULL, "dc_concat_conv: input %d or its mask is NULL", i);
+        if (reinterpret_cast<uintptr_t>(inputs[i]) % 16 != 0)
+            return fail(DC_ERR_ALIGN, "dc_concat_conv: input %d is not aligned to 16 bytes", i);
+        const Span in(inputs[i], P * channels[i] * es), im(masks[i], P * 4);
+        if (o.meets(in) || o.meets(im) || om.meets(in) || om.meets(im))
+            return fail(DC_ERR_UNSUPPORTED, "dc_concat_conv: out / out_mask overlap input %d", i);
+    }
+    return finish(dc::launch_pointwise_concat(*g, inputs, masks, channels, count, packed_filter, out, out_mask, dtype,
+                                              (hipStream_t)stream), "dc_concat_conv");
+}
+
+int dc_pool_update(const dc_geometry *g, const void *input, void *prev_input, void *out, const int32_t *mask,
+                   int32_t *out_mask, int dtype, void *stream) {
+    dc::kernel_log_reset();
+    DC_REQUIRE_DTYPE("dc_pool_update");
+    int rc = check_geometry("dc_pool_update", g, false, true);
+    if (rc != DC_OK) return rc;
+    DC_REQUIRE_PTR("dc_pool_update", input);
+    DC_REQUIRE_PTR("dc_pool_update", prev_input);
+    DC_REQUIRE_PTR("dc_pool_update", out);
+    DC_REQUIRE_PTR("dc_pool_update", mask);
+    DC_REQUIRE_PTR("dc_pool_update", out_mask);
+    if (!dc::pool_update_eligible(*g, input, prev_input, out, dtype))
+        return fail(DC_ERR_UNSUPPORTED, "dc_pool_update: needs 2x2 or 3x3 windows that tile the map exactly (window == "
+                                        "stride, no padding, no dilation, input = output * stride), channels in whole "
+                                        "16-byte vectors, 16-byte aligned tensors and at most 2^20 lanes");
+    {
+        const size_t pi = (size_t)g->batch * g->in_h * g->in_w, po = (size_t)g->batch * g->out_h * g->out_w, es = esize(dtype);
+        const Span wr[] = {Span(prev_input, pi * g->in_c * es), Span(out, po * g->in_c * es), Span(out_mask, po * 4)};
+        const Span rd[] = {Span(input, pi * g->in_c * es), Span(mask, pi * 4)};
+        for (size_t i = 0; i < 3; ++i) {
+            for (const Span &r : rd)
+                if (wr[i].meets(r)) return fail(DC_ERR_UNSUPPORTED, "dc_pool_update: an output overlaps an input of the call");
+            for (size_t j = i + 1; j < 3; ++j)
+                if (wr[i].meets(wr[j])) return fail(DC_ERR_UNSUPPORTED, "dc_pool_update: two outputs of the call overlap");
+        }
+    }
+    return finish(dc::launch_pool_update(*g, input, prev_input, out, mask, out_mask, dtype, (hipStream_t)stream),
+                  "dc_pool_update");
 }
 
 int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_t *mask_a,

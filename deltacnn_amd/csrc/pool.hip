@@ -12,6 +12,8 @@
 // pool_global_kernel  1x1 output (float32 [B][C]); every workgroup owns a slice of channels
 //                     and walks all input pixels, so the sum has a fixed order and needs no
 //                     atomics
+#include <type_traits>
+
 #include "tile.hpp"
 
 namespace dc {
@@ -271,9 +273,13 @@ pool_scan_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restrict
 // and (for the maximum) the cached inputs of all taps at once from clamped addresses and selects
 // afterwards -- one memory round trip, no workgroup barrier, no serial walk over a tile's pixels.
 // Same operations in the same order as pool_window_kernel.
-template <typename T, int N, bool MAX, int K>
+// UPD (maximum, windows that tile the map exactly: window == stride, no padding, no dilation): the
+// cached input follows the input in the same launch -- prev += delta on the window's updated
+// pixels, each of which belongs to this group's window alone -- what dc_add_to_dense does behind
+// dc_pool otherwise.
+template <typename T, int N, bool MAX, int K, bool UPD = false>
 __global__ void __launch_bounds__(256)
-pool_pixel_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restrict__ prev,
+pool_pixel_kernel(ConvP p, PoolQ q, const T *__restrict__ in, typename std::conditional<UPD, T, const T>::type *prev,
                   T *__restrict__ out, const int32_t *__restrict__ mask,
                   int32_t *__restrict__ out_mask, int lg) {
     constexpr int KK = K * K;
@@ -362,6 +368,16 @@ pool_pixel_kernel(ConvP p, PoolQ q, const T *__restrict__ in, const T *__restric
 #pragma unroll
         for (int j = 0; j < N; ++j) r.v[j] = MAX ? T(hi[j] - hp[j]) : T(hi[j] / area);
         vstore<T, N>(out + (size_t)po * C + c0, r);
+        if (UPD) {
+#pragma unroll
+            for (int t = 0; t < KK; ++t) {
+                if (!((taps >> t) & 1)) continue;
+                Vec<T, N> nv;
+#pragma unroll
+                for (int j = 0; j < N; ++j) nv.v[j] = pp[t].v[j] + pd[t].v[j];
+                vstore<T, N>(const_cast<T *>(prev) + ip[t] * C + c0, nv);  // UPD: prev is not const
+            }
+        }
     }
 }
 
@@ -604,6 +620,56 @@ hipError_t pool_t(const dc_geometry &g, const T *in, const T *prev, void *out, c
 }
 
 }  // namespace
+
+// dc_pool_update: maximum pooling whose windows tile the map exactly, on a map of the per-pixel
+// kernel's range, channels in whole 16-byte vectors.
+bool pool_update_eligible(const dc_geometry &g, const void *in, const void *prev, const void *out, int dtype) {
+    const int n = dtype == DC_F32 ? 4 : 8;
+    const bool sq = g.kernel_h == g.kernel_w && (g.kernel_h == 2 || g.kernel_h == 3);
+    const bool tiles = g.stride_h == g.kernel_h && g.stride_w == g.kernel_w && g.dilation_h == 1 && g.dilation_w == 1 &&
+                       g.pad_top == 0 && g.pad_left == 0 && g.pad_bottom == 0 && g.pad_right == 0 &&
+                       g.in_h == g.out_h * g.stride_h && g.in_w == g.out_w * g.stride_w;
+    const bool vec = g.in_c % n == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)prev & 15) == 0;
+    int G = pow2_ceil(g.in_c / std::max(n, 1));
+    if (G > WAVE) G = WAVE;
+    const int64_t po = (int64_t)g.batch * g.out_h * g.out_w;
+    return sq && tiles && vec && g.in_c / n <= WAVE && po * G <= (1 << 20) && (int64_t)g.batch * g.in_h * g.in_w < (1ll << 31);
+}
+
+namespace {
+template <typename T>
+hipError_t pool_update_t(const dc_geometry &g, const T *in, T *prev, T *out, const int32_t *mask, int32_t *out_mask,
+                         hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    ConvP p;
+    p.B = g.batch; p.Hi = g.in_h; p.Wi = g.in_w; p.Ci = g.in_c;
+    p.Ho = g.out_h; p.Wo = g.out_w; p.Co = g.in_c;
+    p.Kh = g.kernel_h; p.Kw = g.kernel_w; p.sh = g.stride_h; p.sw = g.stride_w;
+    p.dh = p.dw = 1; p.pt = p.pl = 0;
+    p.ci_g = p.co_g = 1; p.w_co = 0; p.swz = 0;
+    PoolQ q;
+    q.pb = q.pr = 0;
+    q.zero_bottom = q.zero_right = false;
+    int G = pow2_ceil(g.in_c / N);
+    if (G > WAVE) G = WAVE;
+    const int64_t lanes = (int64_t)g.batch * g.out_h * g.out_w * G;
+    const int block = lanes <= 2048 * WAVE ? WAVE : 256;
+    const dim3 pgrid((unsigned)ceil_div64(lanes, block));
+    int lg = 0;
+    while ((1 << lg) < G) ++lg;
+    note_kernel("pool_pixel_kernel");
+    if (g.kernel_h == 2) pool_pixel_kernel<T, N, true, 2, true><<<pgrid, block, 0, s>>>(p, q, in, prev, out, mask, out_mask, lg);
+    else pool_pixel_kernel<T, N, true, 3, true><<<pgrid, block, 0, s>>>(p, q, in, prev, out, mask, out_mask, lg);
+    return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_pool_update(const dc_geometry &g, const void *in, void *prev, void *out, const int32_t *mask,
+                              int32_t *out_mask, int dtype, hipStream_t s) {
+    if (dtype == DC_F32) return pool_update_t<float>(g, (const float *)in, (float *)prev, (float *)out, mask, out_mask, s);
+    if (dtype == DC_BF16) return pool_update_t<bf16_t>(g, (const bf16_t *)in, (bf16_t *)prev, (bf16_t *)out, mask, out_mask, s);
+    return pool_update_t<half_t>(g, (const half_t *)in, (half_t *)prev, (half_t *)out, mask, out_mask, s);
+}
 
 bool pool_global_casts(const dc_geometry &g, const void *in, const void *prev, int dtype) {
     const int n = dtype == DC_F32 ? 4 : 8;

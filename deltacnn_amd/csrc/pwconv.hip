@@ -51,6 +51,23 @@ struct ResP {
     E *tmp = nullptr;  // MODE 3: the layer's truncated values again, which receive T = truncated + v
 };
 
+// MODE 4: the input is the concatenation, along the channels, of up to four delta tensors with
+// masks of their own (a DCConcatenate chain in front of the convolution, which then never
+// runs): reduction step s belongs to the tensor whose step range holds it, a pixel's fragment
+// counts only where that tensor's mask is set, and the output mask is the union -- the products
+// a concatenated tensor's zero-filled halves would add are exact zeros, so the result equals the
+// convolution of the concatenation bit for bit.  Unused entries repeat entry 0 with a step range
+// that is never reached.
+constexpr int PW_MAX_SEGS = 4;
+template <typename E>
+struct PwSegs {
+    const E *in[PW_MAX_SEGS];
+    const int32_t *mask[PW_MAX_SEGS];
+    int C[PW_MAX_SEGS];          // channels, multiples of 32
+    int step0[PW_MAX_SEGS];      // first reduction step
+    int n;
+};
+
 // A workgroup takes 64 consecutive pixels (4 pixel tiles of 16) x CBW * R channel tiles of 16.
 // Its KW * CBW * NBW wavefronts are arranged as
 //   KW  slices of the reduction (wavefront kw takes steps kw, kw + KW, ...; the partial sums
@@ -79,11 +96,11 @@ __device__ __forceinline__ void
 pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
              const E *__restrict__ bias, E *__restrict__ out,
              const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, const ResP<E> &rp,
-             int bx, int by, float4_t *s_red, E *s_open = nullptr) {
+             int bx, int by, float4_t *s_red, E *s_open = nullptr, const PwSegs<E> *sgp = nullptr) {
     typedef typename Elem16<E>::v4 E4;
     typedef typename Elem16<E>::v8 E8;
     static_assert(NBW * NTW <= 4, "a workgroup covers at most 64 pixels");
-    constexpr bool ADD = MODE == 1 || MODE == 2, ADDACT = MODE == 2, OPEN = MODE == 3;
+    constexpr bool ADD = MODE == 1 || MODE == 2, ADDACT = MODE == 2, OPEN = MODE == 3, SEG = MODE == 4;
     constexpr int NW = KW * CBW * NBW, TILES = R * NTW, FT = (TILES + KW - 1) / KW;
     constexpr int PXW = NBW * NTW * 16;  // pixels per workgroup
     const int wave = wave_id(), lane = lane_id();
@@ -96,9 +113,28 @@ pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
     // of filter fragments (which do not depend on the masks)
     const int mp = pbase + lane;
     const bool mine = lane < PXW && mp < p.P;
-    const int mword = mask[min(mp, p.P - 1)];
+    int mword = 0, sword[PW_MAX_SEGS] = {0, 0, 0, 0};
+    if (SEG) {
+#pragma unroll
+        for (int g = 0; g < PW_MAX_SEGS; ++g) sword[g] = sgp->mask[g][min(mp, p.P - 1)];
+    } else {
+        mword = mask[min(mp, p.P - 1)];
+    }
     int rword = 0;
     if (ADD) rword = rp.mask[min(mp, p.P - 1)];
+    // SEG: tensor, first step and channel count of reduction step s (uniform selects: an indexed
+    // read of the argument block would move it to scratch memory)
+    auto seg_of = [&](int st) { return SEG ? (st >= sgp->step0[1]) + (st >= sgp->step0[2]) + (st >= sgp->step0[3]) : 0; };
+    auto seg_in = [&](int g) { return g == 0 ? sgp->in[0] : g == 1 ? sgp->in[1] : g == 2 ? sgp->in[2] : sgp->in[3]; };
+    auto seg_c = [&](int g) { return g == 0 ? sgp->C[0] : g == 1 ? sgp->C[1] : g == 2 ? sgp->C[2] : sgp->C[3]; };
+    auto seg_s0 = [&](int g) { return g == 0 ? sgp->step0[0] : g == 1 ? sgp->step0[1] : g == 2 ? sgp->step0[2] : sgp->step0[3]; };
+    // SEG: the input fragment of step st for pixel tile j of this wavefront (clamped pixel; what an
+    // inactive pixel returns is zeroed before it is used)
+    auto seg_x = [&](int st, int j) {
+        const int g = seg_of(st);
+        const size_t pix = (size_t)min(pbase + (nw * NTW + j) * 16 + l16, p.P - 1);
+        return *reinterpret_cast<const E8 *>(seg_in(g) + pix * seg_c(g) + ((st - seg_s0(g)) << 5) + kq * 8);
+    };
     const int ct0 = (by * CBW + cw) * R;
     const E *wrow[R];  // fragment order: one contiguous KB per (channel tile, step)
 #pragma unroll
@@ -119,13 +155,13 @@ pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
     if (EAGER) {
 #pragma unroll
         for (int j = 0; j < NTW; ++j)
-            xrow[j] = in + (size_t)min(pbase + (nw * NTW + j) * 16 + l16, p.P - 1) * p.Ci;
+            xrow[j] = SEG ? nullptr : in + (size_t)min(pbase + (nw * NTW + j) * 16 + l16, p.P - 1) * p.Ci;
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             const int s = min(kw + i * KW, ksteps - 1);
             const int k = min((s << 5) + kq * 8, p.Ci - 8);
 #pragma unroll
-            for (int j = 0; j < NTW; ++j) x[i][j] = *reinterpret_cast<const E8 *>(xrow[j] + k);
+            for (int j = 0; j < NTW; ++j) x[i][j] = SEG ? seg_x(s, j) : *reinterpret_cast<const E8 *>(xrow[j] + k);
         }
     }
     // tiles this wavefront finishes: all of its own (KW == 1) or tiles kw, kw + KW, ... of
@@ -142,11 +178,17 @@ pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
             qv[m] = *reinterpret_cast<const E4 *>(rp.prev + off);
         }
     }
-    const uint64_t bm = ballot(mine && mword != 0);
+    uint64_t bseg[PW_MAX_SEGS] = {0, 0, 0, 0};
+    if (SEG) {
+#pragma unroll
+        for (int g = 0; g < PW_MAX_SEGS; ++g) bseg[g] = g < sgp->n ? ballot(mine && sword[g] != 0) : 0;
+    }
+    const uint64_t bm = SEG ? (bseg[0] | bseg[1] | bseg[2] | bseg[3]) : ballot(mine && mword != 0);
     const uint64_t br = ADD ? ballot(mine && rword != 0) : 0;
     const uint64_t bo = bm | br;
     if (by == 0 && wave == 0 && mine) out_mask[mp] = int((bo >> lane) & 1);
     if (bo == 0) return;  // the same for every wavefront of the workgroup
+    auto seg_bits = [&](int g) { return g == 0 ? bseg[0] : g == 1 ? bseg[1] : g == 2 ? bseg[2] : bseg[3]; };
     if (OPEN && EAGER) {  // requested above, arrived with the mask words: not to be moved down to the epilogue
 #pragma unroll
         for (int m = 0; m < FT; ++m) {
@@ -193,7 +235,7 @@ pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
         nt_on[j] = ((bm >> bit) & 0xffffu) != 0;
         wave_on |= nt_on[j];
         // inactive pixels all point at pixel 0, so their (discarded) loads share one cache line
-        if (!EAGER) xrow[j] = in + (size_t)(((bm >> (bit + l16)) & 1) ? pbase + bit + l16 : 0) * p.Ci;
+        if (!EAGER && !SEG) xrow[j] = in + (size_t)(((bm >> (bit + l16)) & 1) ? pbase + bit + l16 : 0) * p.Ci;
     }
 
     if (wave_on) {
@@ -213,7 +255,7 @@ pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
                     const int s = min(s0 + i * KW, ksteps - 1);
                     const int k = min((s << 5) + kq * 8, p.Ci - 8);
 #pragma unroll
-                    for (int j = 0; j < NTW; ++j) x[i][j] = *reinterpret_cast<const E8 *>(xrow[j] + k);
+                    for (int j = 0; j < NTW; ++j) x[i][j] = SEG ? seg_x(s, j) : *reinterpret_cast<const E8 *>(xrow[j] + k);
                 }
             }
             // No zero-fill is needed: columns of inactive pixels are never stored, and where a
@@ -222,12 +264,14 @@ pw_mfma_body(const PwP &p, const E *__restrict__ in, const E *__restrict__ wp,
 #pragma unroll
             for (int i = 0; i < S; ++i) {
                 if (s0 + i * KW < ksteps) {  // wave-uniform
+                    const uint64_t sb = SEG ? seg_bits(seg_of(s0 + i * KW)) : 0;  // the step's tensor: its mask
 #pragma unroll
                     for (int j = 0; j < NTW; ++j)
                         if (nt_on[j]) {  // wave-uniform
+                            const E8 xz = SEG ? keep8(x[i][j], (sb >> ((nw * NTW + j) * 16 + l16)) & 1) : x[i][j];
 #pragma unroll
                             for (int r = 0; r < R; ++r)
-                                acc[r][j] = Elem16<E>::mfma(a[i][r], x[i][j], acc[r][j]);
+                                acc[r][j] = Elem16<E>::mfma(a[i][r], xz, acc[r][j]);
                         }
                 }
             }
@@ -319,7 +363,7 @@ template <typename E, int KW, int CBW, int NBW, int R, int NTW, int S, int MODE,
 __global__ void __launch_bounds__(KW * CBW * NBW * WAVE)
 pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
                const E *__restrict__ bias, E *__restrict__ out,
-               const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, ResP<E> rp) {
+               const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, ResP<E> rp, PwSegs<E> sg) {
     __shared__ float4_t s_red[KW > 1 ? KW * CBW * NBW * R * NTW * WAVE : 1];
     // MODE 3: per wavefront one 16 x 16 tile each of D and T on their way into pixel rows
     __shared__ __align__(16) E s_open[MODE == 3 ? KW * CBW * NBW * 512 : 8];
@@ -331,7 +375,7 @@ pw_mfma_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
         if (by >= p.ny) return;  // padding of the channel groups to a multiple of 8
     }
     pw_mfma_body<E, KW, CBW, NBW, R, NTW, S, MODE, EAGER, ACTC>(p, in, wp, bias, out, mask, out_mask, rp, bx, by, s_red,
-                                                                 s_open);
+                                                                 s_open, &sg);
 }
 
 // Several independent small pointwise layers in ONE launch (the 1x1 convolutions of a
@@ -974,7 +1018,7 @@ template <typename E>
 hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *packed,
                               const void *bias, void *out, const int32_t *mask, int32_t *out_mask,
                               const ActEpilogue *epi, bool *epilogue_done, const Residual *res,
-                              hipStream_t s, const OpenAct *open = nullptr) {
+                              hipStream_t s, const OpenAct *open = nullptr, const PwSegs<E> *segs = nullptr) {
     PwP p;
     p.P = g.batch * g.in_h * g.in_w;
     p.Ci = g.in_c;
@@ -989,7 +1033,7 @@ hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *
     // Large maps: active-pixel gather, with the activation / truncation as its epilogue where the
     // layer has one with maximum-norm truncation.
     const auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
-    const int gct = (res == nullptr && open == nullptr && al16(in) && al16(out) && al16(packed)) ? gather_tiles(p, ksteps) : 0;
+    const int gct = (res == nullptr && open == nullptr && segs == nullptr && al16(in) && al16(out) && al16(packed)) ? gather_tiles(p, ksteps) : 0;
     if (gct > 0 && gather_lds(p, ksteps, gct) <= (64u << 10)) {
         const bool with_act = epi != nullptr && epi->mode == DC_TRUNC_MAX && epi->trunc != nullptr && al16(epi->prev) &&
                               al16(epi->trunc);
@@ -1096,6 +1140,8 @@ hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *
         if (ctw == 2) DC_GO(16, 2);  // 32 KB of filter: at most 32 channel tiles
 #undef DC_GO
     }
+    PwSegs<E> sg{};
+    if (segs != nullptr) sg = *segs;
     ResP<E> rp{nullptr, nullptr, 1.f, 1.f, nullptr, 0};
     if (res != nullptr) rp = ResP<E>{(const E *)res->values, res->mask, res->wa, res->wb, (E *)res->prev, res->act};
     if (open != nullptr)
@@ -1109,24 +1155,27 @@ hipError_t launch_pointwise_t(const dc_geometry &g, const void *in, const void *
         /* filter bytes dominate and the plain order would spread a channel group over XCDs */      \
         p.xcd = (p.nx % 8 != 0 && p.ny > 1 && (int64_t)p.ci_p * p.Co > (int64_t)p.P * p.Ci) ? 1 : 0; \
         dim3 grid(p.xcd ? p.nx * ((p.ny + 7) / 8 * 8) : p.nx, p.xcd ? 1 : p.ny);                     \
-        if (open != nullptr && open->act == DC_ACT_RELU6)                                            \
+        if (segs != nullptr)                                                                         \
+            pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 4, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp, sg); \
+        else if (open != nullptr && open->act == DC_ACT_RELU6)                                       \
             pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 3, EA, DC_ACT_RELU6><<<grid, KW * CBW * NBW * WAVE, 0, s>>>( \
-                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp, sg); \
         else if (open != nullptr)                                                                    \
             pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 3, EA, DC_ACT_RELU><<<grid, KW * CBW * NBW * WAVE, 0, s>>>( \
-                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp, sg); \
         else if (res != nullptr && res->act == DC_ACT_RELU)                                          \
             pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 2, EA, DC_ACT_RELU><<<grid, KW * CBW * NBW * WAVE, 0, s>>>( \
-                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp, sg); \
         else if (res != nullptr && res->act > 0)                                                     \
             pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 2, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
-                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp, sg); \
         else if (res != nullptr)                                                                     \
             pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 1, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
-                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp, sg); \
         else                                                                                         \
             pw_mfma_kernel<E, KW, CBW, NBW, R, NTW, SS, 0, EA><<<grid, KW * CBW * NBW * WAVE, 0, s>>>(     \
-                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp); \
+                p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, rp, sg); \
     } while (0)
 #define DC_PW(ID, KW, CBW, NBW, R, NTW, EA)                                                          \
     case ID: {                                                                                       \
@@ -1153,6 +1202,48 @@ hipError_t launch_pointwise(const dc_geometry &g, const void *in, const void *pa
     if (dtype == DC_BF16)
         return launch_pointwise_t<bf16_t>(g, in, packed, bias, out, mask, out_mask, epi, epilogue_done, res, s);
     return launch_pointwise_t<half_t>(g, in, packed, bias, out, mask, out_mask, epi, epilogue_done, res, s);
+}
+
+// The pointwise convolution of a concatenation of n (2..4) delta tensors that is never formed
+// (MODE 4 of pw_mfma_kernel): `g` describes the convolution of the concatenated tensor, whose
+// arrangement -- and hence summation order -- the launch takes.
+bool pointwise_concat_eligible(const dc_geometry &g, const int32_t *channels, int n, int dtype) {
+    if (!pointwise_eligible(g, dtype) || n < 2 || n > PW_MAX_SEGS) return false;
+    int total = 0;
+    for (int i = 0; i < n; ++i) {
+        if (channels[i] <= 0 || channels[i] % 32 != 0) return false;
+        total += channels[i];
+    }
+    return total == g.in_c;
+}
+
+namespace {
+template <typename E>
+hipError_t pointwise_concat_t(const dc_geometry &g, const void *const *inputs, const int32_t *const *masks,
+                              const int32_t *channels, int n, const void *packed, void *out, int32_t *out_mask,
+                              hipStream_t s) {
+    PwSegs<E> sg;
+    int step = 0;
+    for (int i = 0; i < PW_MAX_SEGS; ++i) {
+        const int k = i < n ? i : 0;
+        sg.in[i] = (const E *)inputs[k];
+        sg.mask[i] = masks[k];
+        sg.C[i] = channels[k];
+        sg.step0[i] = i < n ? step : (1 << 30);  // never reached
+        if (i < n) step += channels[i] / 32;
+    }
+    sg.n = n;
+    bool unused = false;
+    return launch_pointwise_t<E>(g, inputs[0], packed, nullptr, out, masks[0], out_mask, nullptr, &unused, nullptr, s,
+                                 nullptr, &sg);
+}
+}  // namespace
+
+hipError_t launch_pointwise_concat(const dc_geometry &g, const void *const *inputs, const int32_t *const *masks,
+                                   const int32_t *channels, int n, const void *packed, void *out, int32_t *out_mask,
+                                   int dtype, hipStream_t s) {
+    if (dtype == DC_BF16) return pointwise_concat_t<bf16_t>(g, inputs, masks, channels, n, packed, out, out_mask, s);
+    return pointwise_concat_t<half_t>(g, inputs, masks, channels, n, packed, out, out_mask, s);
 }
 
 // A plain pointwise convolution whose own launch is one wavefront per 16 x 16 output tile:

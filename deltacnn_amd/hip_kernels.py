@@ -191,6 +191,30 @@ def sparse_conv_add(x, packed_filter, mask, bias, residual, mask_residual, geome
     return out, out_mask
 
 
+def sparse_deconv_add(x, packed_filter, mask, residual, mask_residual, geometry, out, out_mask,
+                      weight_residual=1.0, weight_conv=1.0):
+    """``sparse_add_tensors(residual, sparse_deconv(x))`` (no activation) in the transposed
+    convolution's launch (``dc_deconv_add``), for 16-bit layers with a packed filter that the
+    LDS-halo kernel takes.  Returns ``None`` (nothing launched) when the shape has no fused form,
+    so the caller can issue the two separate calls."""
+    lib = _lib.load()
+    _nhwc(x, "x")
+    _nhwc(residual, "residual")
+    if packed_filter is None or x.dtype not in (torch.float16, torch.bfloat16):
+        return None
+    args = (geometry, x.data_ptr(), packed_filter.data_ptr(), _mask(mask, "mask").data_ptr(), residual.data_ptr(),
+            _mask(mask_residual, "mask_residual").data_ptr(), out.data_ptr(), out_mask.data_ptr(),
+            float(weight_residual), float(weight_conv), _dtype(x), _stream())
+    meta = dict(g=geometry, esize=2, in_mask=mask, in_mask_b=mask_residual, out_mask=out_mask, mfma=True)
+    try:
+        _call("deconv_add", lib.dc_deconv_add, args, **meta)
+    except _lib.DeltaCNNError as e:
+        if e.code == -3:
+            return None
+        raise
+    return out, out_mask
+
+
 def sparse_block(x, mask, dw_filter, dw_geometry, dw_prev_out, dw_truncated, dw_threshold, dw_activation,
                  project_packed, project_channels, out, out_mask, residual=None, residual_mask=None,
                  weight_residual=1.0, weight_conv=1.0, expand=None, truncation_mode=0, late_loads=False):
@@ -430,6 +454,59 @@ def sparse_pooling(x, prev_x, kernel_size, mask=None, stride=(1, 1), padding=(0,
     if create_out_mask:
         return out, out_mask
     return out
+
+
+def sparse_concat_conv(inputs, packed_filter, geometry, out, out_mask):
+    """A 1x1 convolution over the channel concatenation of 2..4 delta tensors ``inputs = [(x,
+    mask), ...]`` that is never formed (``dc_concat_conv``): identical to chained
+    :func:`sparse_concatenate` calls followed by :func:`sparse_conv`.  ``geometry`` describes the
+    convolution of the concatenated tensor.  Returns ``None`` (nothing launched) when the shapes
+    have no fused form, so the caller can issue the separate calls."""
+    lib = _lib.load()
+    n = len(inputs)
+    if packed_filter is None or not 2 <= n <= 4 or inputs[0][0].dtype not in (torch.float16, torch.bfloat16):
+        return None
+    for x, _ in inputs:
+        _nhwc(x, "input")
+    ptrs = (ctypes.c_void_p * n)(*[x.data_ptr() for x, _ in inputs])
+    mptrs = (ctypes.c_void_p * n)(*[_mask(m, "mask").data_ptr() for _, m in inputs])
+    chans = (ctypes.c_int32 * n)(*[x.shape[1] for x, _ in inputs])
+    args = (geometry, n, ctypes.cast(ptrs, ctypes.c_void_p), ctypes.cast(mptrs, ctypes.c_void_p),
+            ctypes.cast(chans, ctypes.c_void_p), packed_filter.data_ptr(), out.data_ptr(), out_mask.data_ptr(),
+            _dtype(inputs[0][0]), _stream())
+    try:
+        _call("concat_conv", lib.dc_concat_conv, args, g=geometry, esize=2, in_mask=inputs[0][1], out_mask=out_mask,
+              seg_masks=[m for _, m in inputs], seg_channels=[x.shape[1] for x, _ in inputs], mfma=True,
+              keep=(ptrs, mptrs, chans, [x for x, _ in inputs]))
+    except _lib.DeltaCNNError as e:
+        if e.code == -3:
+            return None
+        raise
+    return out, out_mask
+
+
+def sparse_max_pooling_update(x, prev_x, kernel_size, mask, stride, out=None, out_mask=None):
+    """Maximum pooling and the update of the layer's cached input (``prev_x[mask] += x``) in one
+    launch (``dc_pool_update``), for windows that tile the map exactly.  Returns ``(out,
+    out_mask)``, or ``None`` (nothing launched) for other shapes: the caller then issues
+    :func:`sparse_pooling` and :func:`sparse_add_to_dense_tensor`."""
+    lib = _lib.load()
+    _nhwc(x, "x")
+    g = conv_geometry(x.shape, kernel_size, x.shape[1], stride, (0, 0), (1, 1), 1, False, None)
+    if out is None:
+        out = new_features(g.batch, x.shape[1], g.out_h, g.out_w, x.dtype, x.device)
+    if out_mask is None:
+        out_mask = new_mask(g.batch, g.out_h, g.out_w, x.device)
+    try:
+        _call("pool_update", lib.dc_pool_update,
+              (g, x.data_ptr(), prev_x.data_ptr(), out.data_ptr(), _mask(mask, "mask").data_ptr(), out_mask.data_ptr(),
+               _dtype(x), _stream()),
+              g=g, esize=x.element_size(), in_mask=mask, out_mask=out_mask, mode=0, keep=(x, prev_x, out))
+    except _lib.DeltaCNNError as e:
+        if e.code == -3:
+            return None
+        raise
+    return out, out_mask
 
 
 def sparse_activation(x, prev_x, truncated, mask, threshold, activation, truncation_mode):

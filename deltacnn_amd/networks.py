@@ -581,8 +581,13 @@ class _Root(nn.Module):
         super().__init__()
         self.cats = nn.ModuleList(L.DCConcatenate() for _ in range(n_inputs - 1))
         self.conv = _conv_act(L, in_channels, out_channels, 1)
+        self._concat_conv = getattr(L, "concat_conv", None)  # the convolution reads the children where they lie
 
     def forward(self, xs):
+        if self._concat_conv is not None:
+            y = self._concat_conv(self.conv, xs)
+            if y is not None:
+                return y
         y = xs[0]
         for cat, x in zip(self.cats, xs[1:]):
             y = cat(y, x)
@@ -656,8 +661,14 @@ class _IDAUp(nn.Module):
     def forward(self, layers, start, end):
         for i in range(start + 1, end):
             k = i - start - 1
-            up = self.up[k](self.proj[k](layers[i]))
-            layers[i] = self.node[k](self.add[k](up, layers[i - 1]))
+            # add(up(proj(x)), previous level): a layer namespace whose DCAdd has ``conv_first`` may
+            # run the sum inside the transposed convolution's kernel
+            fused = getattr(self.add[k], "conv_first", None)
+            if fused is None:
+                merged = self.add[k](self.up[k](self.proj[k](layers[i])), layers[i - 1])
+            else:
+                merged = fused(self.up[k], self.proj[k](layers[i]), layers[i - 1])
+            layers[i] = self.node[k](merged)
 
 
 class DLA34CenterNet(_Net):

@@ -510,6 +510,31 @@ class DCAdd(DCModule):
                     return res
         return self(a, conv(conv_input))
 
+    def conv_first(self, conv, conv_input, b):
+        """``self(conv(conv_input), b)`` for a transposed convolution ``conv`` without activation:
+        the addition runs in the convolution's kernel (``dc_deconv_add``) when this layer has unit
+        weights, no activation and no dense_out -- the sum is then commutative bit for bit, and
+        the kernel takes ``b`` as its residual operand; otherwise exactly the two layer calls."""
+        fusable = (DCAdd.fuse_into_conv and type(b) != Tensor and type(conv_input) != Tensor and not self.first_iter
+                   and not self.dense_out and self.activation is None and self.weight_a == 1.0 and self.weight_b == 1.0
+                   and isinstance(conv, DCConvTranspose2d) and conv.activation is None and not conv.dense_out
+                   and conv.backend == DCBackend.deltacnn and conv.frame_idx >= 0)
+        if fusable:
+            val_b, mask_b = b
+            x, mask, plan, packed, _, _ = conv._prepare(conv_input)
+            g = plan["g"]
+            if packed is not None and tuple(val_b.shape) == (g.batch, g.out_c, g.out_h, g.out_w):
+                if not _matches(self.out, val_b):
+                    self.out = torch.empty_like(val_b)
+                if not _matches(self.mask_out, mask_b):
+                    self.mask_out = torch.empty_like(mask_b)
+                res = hk.sparse_deconv_add(x, packed, mask, val_b, mask_b, g, self.out, self.mask_out)
+                if res is not None:
+                    DCConv2d.conv_idx += 1
+                    conv.frame_idx += 1
+                    return res
+        return self(conv(conv_input), b)
+
     def after_upsample(self, a, b, upsample):
         """``self(a, upsample(b))`` with the nearest upsampling folded into the addition's kernel
         (the upsampled tensor is never stored) when both operands are delta tensors and this
@@ -650,6 +675,40 @@ def project_expand(project, add, residual, expand, depthwise, input):
     DCConv2d.conv_idx += 1  # the projection's own forward call; the expansion counts when it is finished
     project.frame_idx += 1
     return (out, out_mask), OpenExpansion(expand, depthwise)
+
+
+def concat_conv(conv, inputs):
+    """``conv(cat(inputs))`` for a 1x1 DCConv2d (with or without activation) over the channel
+    concatenation of 2..4 delta tensors, on frames after the first: the convolution reads the
+    tensors where they lie (``dc_concat_conv``), no DCConcatenate launch runs, and the layer's own
+    activation follows as in its forward call.  Returns what the layer returns, or ``None`` when
+    the layer is not in a state or of a shape the kernel takes; nothing has happened then and the
+    caller concatenates and calls the layer.  Switch: ``DCConcatenate.fuse_into_conv``."""
+    if not DCConcatenate.fuse_into_conv or any(isinstance(x, Tensor) for x in inputs) or not 2 <= len(inputs) <= 4:
+        return None
+    x0 = inputs[0][0]
+    if not (isinstance(conv, DCConv2d) and not conv._transposed and conv.backend == DCBackend.deltacnn
+            and conv.frame_idx >= 0 and conv.conv_idx >= 0 and conv.filters_processed and not conv.dense_out
+            and conv.weight.dtype == x0.dtype
+            and (conv.kernel_size, conv.stride, conv.padding, conv.groups) == ((1, 1), (1, 1), (0, 0), 1)):
+        return None
+    act = conv.activation_layer
+    if act is not None and act.first_iter:
+        return None
+    b, _, h, w = x0.shape
+    if any(x.shape[0] != b or x.shape[2:] != x0.shape[2:] or x.dtype != x0.dtype for x, _ in inputs):
+        return None
+    total = sum(x.shape[1] for x, _ in inputs)
+    plan = conv._plan_for((b, total, h, w), x0.dtype, x0.device)
+    packed = conv._packed_filter()
+    if packed is None or plan["out"] is None:
+        return None
+    done = hk.sparse_concat_conv(list(inputs), packed, plan["g"], plan["out"], plan["out_mask"])
+    if done is None:
+        return None
+    DCConv2d.conv_idx += 1  # what the layer's own forward call would have counted
+    conv.frame_idx += 1
+    return done if act is None else act(done)
 
 
 def expand_depthwise(expand, depthwise, input, opened=None):
@@ -881,6 +940,7 @@ def add_group(adds, firsts, seconds, upsamples):
 
 class DCConcatenate(DCModule):
     """Channel concatenation of two delta tensors (sparse_layers.py:1185-1194)."""
+    fuse_into_conv = True  # a 1x1 convolution behind a chain of concatenations reads the tensors where they lie
 
     def __init__(self, name=""):
         super().__init__()
@@ -1139,6 +1199,8 @@ class DCMaxPooling(nn.MaxPool2d, DCModule):
     ``padding`` may be a pair or (left, right, top, bottom) as torch.nn.functional.pad takes it
     (:1439-1441)."""
 
+    fuse_cache_update = True  # windows that tile the map: pooling and cache update in one launch
+
     def __init__(self, kernel_size, stride=(1, 1), padding=(0, 0), dilation=(1, 1)):
         kernel_size, stride, padding, dilation = to_tuple(kernel_size, stride, padding, dilation)
         nn.MaxPool2d.__init__(self, kernel_size, stride=stride, padding=padding, dilation=dilation)
@@ -1161,6 +1223,11 @@ class DCMaxPooling(nn.MaxPool2d, DCModule):
         if self.first_iter:
             self.first_iter = False
             self.prev_in = self._cache(torch.zeros_like(delta))
+        if (DCMaxPooling.fuse_cache_update and tuple(self.kernel_size) == tuple(self.stride) and not any(self.padding)
+                and tuple(self.dilation) == (1, 1)):
+            pooled = hk.sparse_max_pooling_update(delta, self.prev_in, self.kernel_size, mask, self.stride)
+            if pooled is not None:  # the pooling kernel has moved the cache along as well
+                return pooled
         pooled = hk.sparse_pooling(delta, self.prev_in, self.kernel_size, mask, self.stride, self.padding,
                                    self.dilation, create_out_mask=True, pooling_mode_int=0)
         hk.sparse_add_to_dense_tensor(delta, self.prev_in, mask)  # the cache follows the input

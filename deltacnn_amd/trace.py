@@ -9,7 +9,7 @@ m = 4-byte mask word, P pixels, n_x = number of active pixels of mask x):
   densify            R = P*m + n*2*C*s                    W = n*C*s   (+ dense copy: R += (P-n)*C*s, W += P*C*s)
   add                R = 2*P*m + (n_a+n_b)*C*s [+n_out*C*s]  W = n_out*C*s [+n_out*C*s] + P*m
   conv / deconv      R = P_in*m + n_in*Cin*s + K*K*(Cin/g)*Cout*s   W = n_out*Cout*s + P_out*m
-                     (conv_add: + P_out*m + n_res*Cout*s for the residual; conv_act in one launch:
+                     (conv_add, deconv_add: + P_out*m + n_res*Cout*s for the residual; conv_act in one launch:
                      + the activate_truncate state traffic R += n_mid*2*Cout*s,
                      W += n_out*2*Cout*s + (n_mid-n_out)*Cout*s, n_mid = updated outputs before
                      truncation; conv_act in two launches: a conv row and an activate_truncate row)
@@ -18,11 +18,15 @@ m = 4-byte mask word, P pixels, n_x = number of active pixels of mask x):
                      (conv_group: the conv / conv_add / conv_act terms of its layers added up, one row
                      for the grouped convolution launch and one for the grouped activation launch)
   pool               R = P_in*m + n_in*C*s [max: + n_cov*C*s]   W = n_out*C*s + P_out*m
+                     (pool_update, the maximum with the layer's cache update in its launch: W += n_in*C*s)
                      (the maximum of an updated window needs the cached input of EVERY pixel of the
                      window, updated or not: n_cov = input pixels covered by updated windows)
   add_to_dense       R = P*m + 2*n*C*s                    W = n*C*s
   upsample           R = P*m + n*C*s                      W = S*S*(n*C*s + P*m)
   concat             R = 2*P*m + (n_a*Ca + n_b*Cb)*s      W = n_out*(Ca+Cb)*s + P*m
+  concat_conv        (a 1x1 convolution over k tensors that are never concatenated)
+                     R = sum_i (P*m + n_i*C_i*s) + Cin*Cout*s   W = n_out*Cout*s + P*m
+                     flops = 2*Cout*sum_i n_i*C_i
   mul_add            R = P*m + n*C*s + C*s                W = n*C*s
   block              (depthwise 3x3 + activation -> projection (+ residual) -> expansion + activation in
                      one launch; Ch hidden, Cp projection, Ce expansion channels; n_mid = updated
@@ -65,10 +69,12 @@ class Tracer:
             rec["items"] = [{"n_in": self._count(i["in_mask"]), "n_in_b": self._count(i["in_mask_b"]),
                              "pairs": self._pairs(i["g"], i["in_mask"], False) if self.count_pairs else None}
                             for i in meta["items"]]
+        if op == "concat_conv":
+            rec["n_seg"] = [self._count(m) for m in meta["seg_masks"]]
         rec["n_in"] = self._count(meta.get("in_mask"))
         rec["n_in_b"] = self._count(meta.get("in_mask_b"))
-        if self.count_pairs and op in ("conv", "deconv", "conv_act", "conv_add", "block"):
-            rec["pairs"], rec["n_mid"] = self._pairs(meta["g"], meta["in_mask"], op == "deconv")
+        if self.count_pairs and op in ("conv", "deconv", "deconv_add", "conv_act", "conv_add", "block"):
+            rec["pairs"], rec["n_mid"] = self._pairs(meta["g"], meta["in_mask"], op in ("deconv", "deconv_add"))
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
         rc = fn(*args)
@@ -81,7 +87,7 @@ class Tracer:
         rec["n_ex"] = self._count(meta.get("ex_mask"))
         for it, im in zip(rec.get("items", []), meta.get("items", [])):
             it["n_out"] = self._count(im["out_mask"])
-        if op == "pool" and meta.get("mode") == 0:
+        if op in ("pool", "pool_update") and meta.get("mode") == 0:
             rec["n_cov"] = self._covered(meta["g"], meta["out_mask"])
         rec["call"] = (fn, args)
         self.records.append(rec)
@@ -212,7 +218,7 @@ class Tracer:
             flops = 0
             extra = None  # second kernel of a two-launch call
             ms = r.get("ms", r["events"][0].elapsed_time(r["events"][1]))
-            if op in ("conv", "deconv", "conv_act", "conv_add"):
+            if op in ("conv", "deconv", "deconv_add", "conv_act", "conv_add"):
                 g = meta["g"]
                 p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
                 wbytes = g.kernel_h * g.kernel_w * (g.in_c // g.groups) * g.out_c * s
@@ -220,7 +226,7 @@ class Tracer:
                 two = op == "conv_act" and len(r["kernels"]) == 2
                 rd = p_in * m + n_in * g.in_c * s + wbytes
                 wr = (n_mid if two else n_out) * g.out_c * s + p_out * m
-                if op == "conv_add":  # + the residual operand of the fused add
+                if op in ("conv_add", "deconv_add"):  # + the residual operand of the fused add
                     rd += p_out * m + n_in_b * g.out_c * s
                 if op == "conv_act" and not two:  # fused epilogue: cached state of every updated output
                     rd += n_mid * 2 * g.out_c * s
@@ -342,13 +348,24 @@ class Tracer:
                 flops = 2 * rows * fi * fo
                 shape = f"{fi}->{fo} rows {rows}"
                 dens = (1.0, 1.0)
-            elif op == "pool":
+            elif op == "concat_conv":  # a 1x1 convolution over tensors that are never concatenated
+                g = meta["g"]
+                P = g.batch * g.in_h * g.in_w
+                n_seg = [int(v) for v in r["n_seg"]]
+                rd = sum(P * m + n * c * s for n, c in zip(n_seg, meta["seg_channels"])) + g.in_c * g.out_c * s
+                wr = n_out * g.out_c * s + P * m
+                flops = 2 * g.out_c * sum(n * c for n, c in zip(n_seg, meta["seg_channels"]))
+                shape = f"{'+'.join(str(c) for c in meta['seg_channels'])}->{g.out_c} k1 @{g.in_h}x{g.in_w}"
+                dens = (sum(n_seg) / (P * len(n_seg)), n_out / P)
+            elif op in ("pool", "pool_update"):
                 g = meta["g"]
                 p_in, p_out = g.batch * g.in_h * g.in_w, g.batch * g.out_h * g.out_w
                 rd = p_in * m + n_in * g.in_c * s
                 if meta["mode"] == 0:  # + the cached input of every pixel under an updated window
                     rd += int(r["n_cov"]) * g.in_c * s if "n_cov" in r else n_in * g.in_c * s
                 wr = n_out * g.in_c * s + p_out * m
+                if op == "pool_update":  # + the cached input of the updated pixels, written back
+                    wr += n_in * g.in_c * s
                 shape = f"C{g.in_c} k{g.kernel_h} @{g.in_h}x{g.in_w}"
                 dens = (n_in / p_in, n_out / p_out)
             else:

@@ -358,6 +358,20 @@ int dc_deconv(const dc_geometry *g, const void *input, const void *filter,
               const void *packed_filter, const void *bias, void *out, const int32_t *mask,
               int32_t *out_mask, int dtype, void *stream);
 
+/* dc_deconv followed by dc_add(deconv, residual) -- the DCAdd (sparse_layers.py:1086-1182, no
+ * activation, no dense_out) that merges an up-sampled level into the next one -- in the transposed
+ * convolution's launch: out = weight_residual * residual [mask_residual] + weight_conv *
+ * deconv(input) [updated pixels], out_mask = the union, with the arithmetic of dc_conv_add
+ * (activation 0), whose results it equals bit for bit.  16-bit types, groups 1, dilation 1,
+ * Cin % 8 == 0, a window at least as large as the stride, layers beyond the 4 x 4-patch kernel's
+ * range (the other transposed layers return DC_ERR_UNSUPPORTED before any launch, and the caller
+ * issues the two calls); no bias (it belongs to the first frame).  out and out_mask must not
+ * overlap the operands.  No counterpart in the reference, which launches deconv_kernel.cu's
+ * kernel and the addition separately (sparse_layers.py:1101-1174). */
+int dc_deconv_add(const dc_geometry *g, const void *input, const void *packed_filter, const int32_t *mask,
+                  const void *residual, const int32_t *mask_residual, void *out, int32_t *out_mask,
+                  float weight_residual, float weight_conv, int dtype, void *stream);
+
 /* Replaces sparse_pooling_wrapper_masked (conv_torch_wrapper.cpp:213-293).  `prev_input` is
  * required for DC_POOL_MAX.  When out_h == out_w == 1, `out` is [B][C], fully overwritten, of
  * type `global_out_dtype`: DC_F32 is the reference's protocol (a float32 accumulator,
@@ -367,6 +381,34 @@ int dc_deconv(const dc_geometry *g, const void *input, const void *filter,
 int dc_pool(const dc_geometry *g, const void *input, const void *prev_input, void *out,
             const int32_t *mask, int32_t *out_mask, int pooling_mode, int dtype,
             int global_out_dtype, void *stream);
+
+/* A 1x1 convolution (stride 1, no padding, no bias) over the concatenation, along the channels,
+ * of `count` (2..4) delta tensors that is never formed: DCConcatenate (sparse_layers.py:1185-1194,
+ * other_nn_layers.cu:3601-3771) chained count - 1 times, then dc_conv, in the convolution's
+ * launch.  `g` describes the convolution of the concatenated tensor (in_c = the sum of
+ * `channels`); inputs[i] is [B][H][W][channels[i]] with update mask masks[i].  A pixel takes part
+ * in the reduction steps of tensor i only where masks[i] is set -- where the concatenation would
+ * hold zeros -- and out_mask is the union of the masks, so out and out_mask equal those of the
+ * separate calls bit for bit (the launch uses the arrangement, and hence the summation order,
+ * dc_conv picks for the concatenated layer).  16-bit types, channels[i] in multiples of 32,
+ * out_c % 4 == 0, a packed filter of the whole layer; anything else returns DC_ERR_UNSUPPORTED
+ * before any launch so that the caller can issue the separate calls.  No counterpart in the
+ * reference, which launches every concatenation (sparse_layers.py:1185-1194). */
+int dc_concat_conv(const dc_geometry *g, int32_t count, const void *const *inputs, const int32_t *const *masks,
+                   const int32_t *channels, const void *packed_filter, void *out, int32_t *out_mask, int dtype,
+                   void *stream);
+
+/* Maximum pooling of a DCMaxPooling layer together with the update of its cached input
+ * (sparse_layers.py:1466-1468: the pooling call, then prev_in[mask] += delta) in ONE launch:
+ * dc_pool(DC_POOL_MAX) followed by dc_add_to_dense(input, prev_input, mask), with identical
+ * results.  For windows that tile the map exactly -- 2x2 or 3x3, stride == window, no padding,
+ * no dilation, input size = output size * stride -- so that every input pixel belongs to one
+ * window and its owner can update it; channels in whole 16-byte vectors, 16-byte aligned
+ * tensors, at most 2^20 lanes (output pixels x lanes per pixel).  Other shapes return
+ * DC_ERR_UNSUPPORTED before any launch and the caller issues the two calls.  prev_input is
+ * updated in place; out and out_mask must not overlap it or the inputs. */
+int dc_pool_update(const dc_geometry *g, const void *input, void *prev_input, void *out, const int32_t *mask,
+                   int32_t *out_mask, int dtype, void *stream);
 
 /* Replaces sparse_add_tensors_wrapper (conv_torch_wrapper.cpp:387-444). */
 int dc_add(const void *a, const void *b, void *prev_out, void *out, const int32_t *mask_a,

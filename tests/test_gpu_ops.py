@@ -800,6 +800,105 @@ def test_conv_add_fused_small_layers(lib, cfg, act, weights, dtype):
         assert_masked_close(p1, want_prev, torch.ones_like(want_mask), 0, tol, "prev_out")
 
 
+@pytest.mark.parametrize("cfg", [(64, 48, 4, 2, 1, 1, 1, 37, 41), (64, 64, 4, 2, 1, 1, 1, 34, 60),
+                                 (128, 128, 4, 2, 1, 1, 1, 17, 30), (32, 32, 8, 4, 2, 1, 1, 20, 23),
+                                 (40, 24, 3, 2, 1, 1, 1, 66, 60)], ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("density", [0.05, 0.6])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["float16", "bfloat16"])
+def test_deconv_add_fused(lib, cfg, density, dtype):
+    """dc_deconv_add == DCAdd(deconv(x), residual) of the oracle, and bit-identical to dc_deconv
+    followed by dc_add with the transposed convolution as FIRST operand (unit weights: the sum is
+    commutative), on pixels reached by one operand only and by both."""
+    from deltacnn_amd import _lib
+    from deltacnn_amd.hip_kernels import conv_geometry
+    Cin, Cout = cfg[0], cfg[1]
+    tol = 2e-2 if dtype == torch.float16 else 8e-2
+    x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(dtype, cfg, 95, density, True)
+    want_conv, want_cm = ops.deconv(x, mask, wt, None, s, p, d, groups)
+    B, _, Ho, Wo = want_conv.shape
+    g = _gen(96)
+    mres = rand_mask(g, B, Ho, Wo, 0.3)
+    res = torch.randn(B, Cout, Ho, Wo, generator=g).to(dtype)
+    want, want_mask = ops.add(want_conv, want_cm, res, mres, None, 1.0, 1.0, 0, False)
+    if density < 0.5:
+        assert 0 < int((want_cm & (1 - mres)).sum()) and 0 < int(((1 - want_cm) & mres).sum())
+    d_filt = filt.to(DEV)
+    pk = hk().pack_filter(d_filt, Cin, Cout, 1, transposed=True)
+    dx, dm, dres, dmres = cl(poison(x, mask)), cl(mask), cl(poison(res, mres)), cl(mres)
+    geo = conv_geometry(x.shape, K, Cout, s, p, d, 1, transposed=True)
+    out = torch.full((B, Cout, Ho, Wo), float("nan"), dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+    om = torch.full((B, 1, Ho, Wo), -5, dtype=torch.int32, device=DEV)
+    got = hk().sparse_deconv_add(dx, pk, dm, dres, dmres, geo, out, om)
+    assert got is not None and _lib.load().dc_last_kernels().decode() == "conv_lds_mfma_kernel"
+    assert torch.equal(om.cpu(), want_mask)
+    assert_masked_close(out, want, want_mask, 0, tol, "out")
+    c_out, c_mask = hk().sparse_deconv(dx, d_filt, dm, None, s, p, d, 1, c_out=Cout, create_out_mask=True, packed_filter=pk)
+    two, two_mask = torch.empty_like(out), torch.empty_like(om)
+    hk().sparse_add_tensors(c_out, dres, None, two, c_mask, dmres, two_mask, 1.0, 1.0, 0, False)
+    assert torch.equal(two_mask, om)
+    assert_masked_equal(out, two.cpu(), want_mask, "fused vs two calls")
+
+
+def test_deconv_add_declines_what_it_cannot_do(lib):
+    """Small transposed layers (the 4x4-patch kernel's), windows smaller than the stride and fp32:
+    None, nothing launched."""
+    from deltacnn_amd.hip_kernels import conv_geometry
+    for cfg, dtype in (((16, 8, 4, 2, 1, 1, 1, 9, 11), torch.float16), ((16, 16, 2, 3, 0, 1, 1, 30, 31), torch.float16),
+                       ((64, 48, 4, 2, 1, 1, 1, 37, 41), torch.float32)):
+        Cin, Cout = cfg[0], cfg[1]
+        x, mask, wt, bias, filt, (K, s, p, d, groups) = _conv_case(torch.float16, cfg, 97, 0.5, True)
+        want_conv, _ = ops.deconv(x, mask, wt, None, s, p, d, groups)
+        B, _, Ho, Wo = want_conv.shape
+        pk = hk().pack_filter(filt.to(DEV), Cin, Cout, 1, transposed=True)
+        geo = conv_geometry(x.shape, K, Cout, s, p, d, 1, transposed=True)
+        out = torch.zeros((B, Cout, Ho, Wo), dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+        om = torch.zeros((B, 1, Ho, Wo), dtype=torch.int32, device=DEV)
+        res = torch.ones_like(out)
+        assert hk().sparse_deconv_add(cl(x).to(dtype), pk, cl(mask), res, torch.ones_like(om), geo, out, om) is None
+        assert not bool(out.any()) and not bool(om.any())
+
+
+@pytest.mark.parametrize("cfg", [((64, 64), 64, 37, 41, 2), ((64, 64), 64, 136, 240, 1), ((128, 128, 64, 128), 128, 20, 23, 1),
+                                 ((256, 256), 256, 17, 30, 1), ((512, 256, 128), 256, 9, 11, 1),
+                                 ((512, 512, 256), 512, 6, 7, 1), ((32, 96), 40, 50, 50, 1), ((64, 32, 32, 64), 256, 64, 64, 1)],
+                         ids=lambda c: "-".join(str(v).replace(" ", "") for v in c))
+@pytest.mark.parametrize("density", [0.1, 0.7])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["float16", "bfloat16"])
+def test_concat_conv_fused(lib, cfg, density, dtype):
+    """dc_concat_conv == the oracle's chained concatenation + 1x1 convolution, and bit-identical
+    to dc_concat (chained) followed by dc_conv, with every tensor active on its own pixels."""
+    from deltacnn_amd import _lib
+    from deltacnn_amd.filter_conversion import convert_filter_out_channels_last, convert_half_filter
+    from deltacnn_amd.hip_kernels import conv_geometry
+    chans, Cout, H, W, B = cfg
+    g = _gen(1300 + sum(chans) + Cout)
+    xs = [torch.randn(B, c, H, W, generator=g).to(dtype) for c in chans]
+    ms = [rand_mask(g, B, H, W, density * (0.5 + 0.5 * i / len(chans))) for i in range(len(chans))]
+    wt = (torch.randn(Cout, sum(chans), 1, 1, generator=g) / sum(chans) ** 0.5).to(dtype)
+    cat, cm = xs[0], ms[0]
+    for x, m in zip(xs[1:], ms[1:]):
+        cat, cm = ops.concatenate(cat, cm, x, m)
+    want, want_mask = ops.conv(cat, cm, wt, None, (1, 1), (0, 0), (1, 1), 1)
+    filt = (convert_half_filter(wt) if dtype == torch.float16 else convert_filter_out_channels_last(wt)).to(DEV)
+    pk = hk().pack_filter(filt, sum(chans), Cout, 1)
+    dxs = [(cl(poison(x, m)), cl(m)) for x, m in zip(xs, ms)]
+    geo = conv_geometry((B, sum(chans), H, W), (1, 1), Cout, (1, 1), (0, 0), (1, 1), 1)
+    out = torch.full((B, Cout, H, W), float("nan"), dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last)
+    om = torch.full((B, 1, H, W), -5, dtype=torch.int32, device=DEV)
+    got = hk().sparse_concat_conv(dxs, pk, geo, out, om)
+    assert got is not None and _lib.load().dc_last_kernels().decode() == "pw_mfma_kernel"
+    assert torch.equal(om.cpu(), want_mask)
+    _check_conv(dtype, out, want, want_mask)
+    dcat = dxs[0]
+    for d in dxs[1:]:
+        dcat = hk().sparse_concatenate(dcat, d)
+    two, two_mask = hk().sparse_conv(dcat[0], filt, dcat[1], None, (1, 1), (0, 0), (1, 1), 1, c_out=Cout, create_out_mask=True,
+                                     packed_filter=pk)
+    assert _lib.load().dc_last_kernels().decode() in ("pw_mfma_kernel", "pw_gather_kernel")
+    assert torch.equal(two_mask, om)
+    assert_masked_equal(out, two.cpu(), want_mask, "fused vs separate calls")
+
+
 # ------------------------------------------------------------------ nothing active / all active
 @pytest.mark.parametrize("fill", [0, 1], ids=["all-inactive", "all-active"])
 @pytest.mark.parametrize("cfg", [
@@ -889,6 +988,51 @@ def test_pool(lib, dtype, cfg, mode, density):
                                   pooling_mode_int=mode)
     assert torch.equal(om.cpu(), want_mask)
     assert_masked_equal(out, want, want_mask, "out")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", [(32, 2, 12, 14, 2), (64, 2, 34, 60, 1), (128, 2, 68, 120, 1), (24, 3, 12, 15, 2),
+                                 (512, 2, 6, 8, 1), (1024, 2, 4, 4, 1)], ids=lambda c: "-".join(str(v) for v in c))
+@pytest.mark.parametrize("density", [0.0, 0.1, 0.7])
+def test_pool_update_fused(lib, dtype, cfg, density):
+    """dc_pool_update == the oracle's maximum pooling followed by its cache update, and
+    bit-identical (pooled delta, mask and the cached input) to dc_pool + dc_add_to_dense."""
+    from deltacnn_amd import _lib
+    C, K, H, W, B = cfg
+    g = _gen(1100 + C)
+    mask = rand_mask(g, B, H, W, density)
+    x = torch.randn(B, C, H, W, generator=g).to(dtype)
+    prev = torch.randn(B, C, H, W, generator=g).to(dtype)
+    want, want_mask = ops.pool(x, prev, mask, (K, K), (K, K), (0, 0), (1, 1), 0)
+    want_prev = prev.clone()
+    ops.add_to_dense(torch.where(mask != 0, x, torch.zeros_like(x)), want_prev, mask)
+    dx, dm = cl(poison(x, mask)), cl(mask)
+    p1 = cl(prev)
+    got = hk().sparse_max_pooling_update(dx, p1, (K, K), dm, (K, K))
+    if C * x.element_size() > 64 * 16:  # more than 64 vectors of 16 bytes per pixel: the two calls
+        assert got is None
+        return
+    assert got is not None and _lib.load().dc_last_kernels().decode() == "pool_pixel_kernel"
+    out, om = got
+    assert torch.equal(om.cpu(), want_mask)
+    assert_masked_equal(out, want, want_mask, "out")
+    assert torch.equal(p1.cpu(), want_prev), "cached input"
+    p2 = cl(prev)
+    out2, om2 = hk().sparse_pooling(dx, p2, (K, K), dm, (K, K), (0, 0), (1, 1), pooling_mode_int=0)
+    hk().sparse_add_to_dense_tensor(dx, p2, dm)
+    assert torch.equal(om2, om) and torch.equal(p1, p2)
+    assert_masked_equal(out, out2.cpu(), want_mask, "fused vs two calls")
+
+
+def test_pool_update_declines_other_shapes(lib):
+    """Windows that overlap, leave pixels over or are padded, channel counts off the vector size:
+    None, nothing launched, nothing touched."""
+    for C, K, s, H, W in ((32, 3, 2, 13, 13), (32, 2, 2, 13, 14), (20, 2, 2, 12, 12), (32, 2, 1, 12, 12)):
+        x = torch.randn(1, C, H, W).half().to(DEV).contiguous(memory_format=torch.channels_last)
+        prev = torch.zeros_like(x)
+        mask = torch.ones(1, 1, H, W, dtype=torch.int32, device=DEV)
+        assert hk().sparse_max_pooling_update(x, prev, (K, K), mask, (s, s)) is None
+        assert not bool(prev.any())
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

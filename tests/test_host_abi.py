@@ -375,6 +375,61 @@ def test_project_expand_arguments_are_checked_before_any_launch(lib):
     assert lib.dc_expand_depthwise(ctypes.byref(gd), ctypes.byref(b), 1, None) == -5
 
 
+def test_deconv_add_arguments_are_checked_before_any_launch(lib):
+    """dc_deconv_add: layers without the fused form -> -3 (the caller issues the two calls), a
+    sum taken in place -> -3, missing operands -> -4, misaligned pointers -> -5; nothing touches
+    a device."""
+    big = (ctypes.c_char * (8 << 20))()
+    q = (ctypes.addressof(big) + 255) // 256 * 256
+    names = ("input", "packed_filter", "mask", "residual", "mask_residual", "out", "out_mask")
+    g = _geom(in_h=34, in_w=60, out_h=68, out_w=120, in_c=64, out_c=64, kernel_h=4, kernel_w=4, stride_h=2, stride_w=2)
+
+    def call(geom=g, dtype=1, **kw):
+        a = {n: q + i * (1 << 20) for i, n in enumerate(names)}  # 1 MB apart: 68 * 120 * 64 * 2 = 1.04e6 bytes fit
+        a.update(kw)
+        return lib.dc_deconv_add(ctypes.byref(geom), *[a[n] for n in names], 1.0, 1.0, dtype, None)
+
+    assert call(dtype=9) == -1
+    assert call(dtype=0) == -3 and b"16-bit" in lib.dc_last_error()
+    small = _geom(in_h=9, in_w=11, out_h=18, out_w=22, in_c=16, out_c=8, kernel_h=4, kernel_w=4, stride_h=2, stride_w=2)
+    assert call(geom=small) == -3                                           # the 4x4-patch kernel's layer
+    gap = _geom(in_h=30, in_w=31, out_h=89, out_w=92, in_c=64, out_c=64, kernel_h=2, kernel_w=2, stride_h=3, stride_w=3,
+                pad_top=0, pad_left=0, pad_bottom=0, pad_right=0)
+    assert call(geom=gap) == -3                                             # stride phases without a tap
+    assert call(geom=_geom(in_h=34, in_w=60, out_h=70, out_w=120, in_c=64, out_c=64, kernel_h=4, kernel_w=4,
+                           stride_h=2, stride_w=2)) == -2                   # output size does not match
+    assert lib.dc_deconv_add(None, q, q, q, q, q, q, q, 1.0, 1.0, 1, None) == -4
+    assert call(residual=None) == -4 and call(out_mask=None) == -4
+    assert call(input=q + 2) == -5 and call(out=q + 5 * (1 << 20) + 4) == -5
+    assert call(out=q + 3 * (1 << 20)) == -3 and b"overlap" in lib.dc_last_error()          # summed in place
+    assert call(out_mask=q + 2 * (1 << 20) + 64) == -3 and b"overlap" in lib.dc_last_error()
+
+
+def test_pool_update_arguments_are_checked_before_any_launch(lib):
+    """dc_pool_update: windows that do not tile the map, channels off the vector size -> -3 (the
+    caller issues dc_pool and dc_add_to_dense), outputs that overlap the operands -> -3, missing
+    operands -> -4; nothing touches a device."""
+    big = (ctypes.c_char * (4 << 20))()
+    q = (ctypes.addressof(big) + 255) // 256 * 256
+    names = ("input", "prev_input", "out", "mask", "out_mask")
+    two = dict(kernel_h=2, kernel_w=2, stride_h=2, stride_w=2, pad_top=0, pad_left=0, pad_bottom=0, pad_right=0)
+    g = _geom(in_h=34, in_w=60, out_h=17, out_w=30, in_c=64, out_c=64, **two)
+
+    def call(geom=g, dtype=1, **kw):
+        a = {n: q + i * (512 << 10) for i, n in enumerate(names)}  # 34 * 60 * 64 * 2 = 261 120 bytes fit
+        a.update(kw)
+        return lib.dc_pool_update(ctypes.byref(geom), *[a[n] for n in names], dtype, None)
+
+    assert call(dtype=9) == -1
+    assert call(geom=_geom(in_h=35, in_w=60, out_h=17, out_w=30, in_c=64, out_c=64, **two)) == -3   # a row left over
+    assert call(geom=_geom(in_h=34, in_w=60, out_h=17, out_w=30, in_c=20, out_c=20, **two)) == -3   # 20 channels
+    over = dict(two, kernel_h=3, kernel_w=3, pad_top=1, pad_left=1, pad_bottom=1, pad_right=1)
+    assert call(geom=_geom(in_h=34, in_w=60, out_h=17, out_w=30, in_c=64, out_c=64, **over)) == -3  # overlapping windows
+    assert call(prev_input=None) == -4 and call(out_mask=None) == -4
+    assert call(out=q + (512 << 10) + 4096) == -3 and b"overlap" in lib.dc_last_error()
+    assert call(prev_input=q) == -3 and b"overlap" in lib.dc_last_error()
+
+
 def test_conv_group_arguments_are_checked_before_any_launch(lib):
     """dc_conv_group: a count outside 2..8 -> -2; an item the 4x4-patch kernel does not take, an
     item with both a residual sum and an activation, activations of two kinds for the second
