@@ -1125,10 +1125,12 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
     for (int d = 0; d < D; ++d) load_chunk(a[d], xo[d]);
     // bias of the lane's four channels for the tiles this wavefront finishes: tiles
     // [kz * TPW, (kz + 1) * TPW) of its channel group, tile t = (channel tile t / NT, pixel tile t % NT)
-    E bv[TPW][4];
+    // (the TPW tiles lie in BR channel tiles: all R of them without reduction slices, else one)
+    constexpr int BR = TPW > NT ? TPW / NT : 1;
+    E bv[BR][4];
 #pragma unroll
-    for (int q = 0; q < TPW; ++q) {
-        const int co = ((cb * ncw + cw) * R + (kz * TPW + q) / NT) * 16 + kq * 4;
+    for (int q = 0; q < BR; ++q) {
+        const int co = ((cb * ncw + cw) * R + (kz * TPW) / NT + q) * 16 + kq * 4;
 #pragma unroll
         for (int i = 0; i < 4; ++i) bv[q][i] = bias != nullptr ? bias[min(co + i, p.Co - 1)] : E(0);
     }
@@ -1340,7 +1342,7 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
         const bool vec = co + 3 < p.Co && (p.Co & 3) == 0;
         E4 v;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = E(fin[q][i] + float(bv[q][i]));
+        for (int i = 0; i < 4; ++i) v[i] = E(fin[q][i] + float(bv[q / NT][i]));
         if (ADD) {  // add_kernel's sequence on the rounded convolution result: s = a * wa; s = fma(b, wb, s)
             const bool upd = (code & 64) != 0, radd = (code & 128) != 0;
             const E wa = E(rs.wa), wb = E(rs.wb);
@@ -1912,6 +1914,197 @@ conv_stem_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ w
     }
 }
 
+// ------------------------------------------------------- thin layers on the matrix cores
+// K x K convolutions (window up to 3 x 3, stride <= 2) with 8 or 16 input channels and up to 64
+// output channels on large maps, where the LDS-halo kernel spends a whole reduction step of 32 on
+// every tap and stores in 8-byte pieces.  Here a reduction step holds 32 / CIN TAPS: lane
+// (pixel, kq) of the input fragment reads the 16 bytes of tap s * TPS + kq * 8 / CIN, channels
+// (kq * 8) % CIN .. + 7, straight from the staged halo -- 5 steps instead of 9 for 16 channels,
+// 3 for 8 -- and the filter fragments (gathered once per wavefront from the packed filter, whose
+// fragment (channel tile, tap) holds the same 16 bytes in lane (ci / 8) * 16 + co) stay in registers.
+// Workgroup = 8 x 8 output pixels, wavefront w = rows 2w, 2w + 1 x all R channel tiles.  The
+// rounded result goes through a wavefront-private LDS tile into pixel rows; output and, MODE 2,
+// the activation / maximum-norm truncation of the layer work on rows in 16-byte pieces (the
+// operations and roundings of act_trunc_pixel; the keep decision of a pixel through an LDS flag),
+// the cached state requested before the contraction.  lazy (maps of 2^18 pixels and more): only
+// updated pixels are read at all.  MODE 0: convolution only.
+template <typename E, int CIN, int R, int MODE, int ACT>
+__global__ void __launch_bounds__(256)
+conv_thin_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp,
+                      const E *__restrict__ bias, E *__restrict__ out,
+                      const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask, EpiP epi,
+                      int hal_h, int hal_w, int lazy) {
+    typedef typename Elem16<E>::v4 E4;
+    typedef typename Elem16<E>::v8 E8;
+    static_assert(CIN == 8 || CIN == 16, "8 or 16 input channels");
+    constexpr int TPS = 32 / CIN;            // taps per reduction step
+    constexpr int NS = (9 + TPS - 1) / TPS;  // reduction steps of a window of up to nine taps
+    constexpr int CV = CIN / 8;              // 16-byte pieces per staged pixel
+    constexpr int ROWB = R * 32 + 16;        // bytes of a staged output row: padded, rows start in different banks
+    constexpr int PIECES = (16 * R * 2 + WAVE - 1) / WAVE;
+    extern __shared__ __align__(16) unsigned char s_mem[];
+    E *s_x = reinterpret_cast<E *>(s_mem);                                     // [hal_h * hal_w][CIN]
+    unsigned char *s_v = s_mem + hal_h * hal_w * CIN * 2 + wave_id() * 16 * ROWB;  // [4 wavefronts][16][ROWB]
+    unsigned *s_row = reinterpret_cast<unsigned *>(s_mem + hal_h * hal_w * CIN * 2 + 4 * 16 * ROWB);  // [hal_h]
+    __shared__ int s_keep[4][16];
+    const int b = blockIdx.z, ty0 = blockIdx.y * TILE, tx0 = blockIdx.x * TILE;
+    const int tid = threadIdx.x, wave = wave_id(), lane = lane_id();
+    const int l16 = lane & 15, kq = lane >> 4;
+    const int iy0 = ty0 * p.sh - p.pt, ix0 = tx0 * p.sw - p.pl;
+    const int K2 = p.Kh * p.Kw;
+    const int co_tiles = (p.Co + 15) >> 4;
+    const int rc = p.Co >> 3;  // 16-byte pieces of an output row (Cout % 8 == 0)
+    // this lane's tap and 8-channel piece in reduction step st
+    const int tsub = CIN == 16 ? kq >> 1 : kq, c8 = CIN == 16 ? kq & 1 : 0;
+    E8 a[R][NS];
+    auto load_filter = [&]() {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int st = 0; st < NS; ++st) {
+                const int t = st * TPS + tsub;
+                const E8 w = *reinterpret_cast<const E8 *>(
+                    wp + ((size_t)(min(r, co_tiles - 1) * K2 + min(t, K2 - 1)) * WAVE + c8 * 16 + l16) * 8);
+                a[r][st] = keep8(w, t < K2);  // taps past the window meet zero weights
+            }
+    };
+    if (!lazy) load_filter();  // lazy: a tile without an update does not fetch the filter
+    E4 bv[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        bv[r] = zero4<E>();
+        if (bias != nullptr) bv[r] = *reinterpret_cast<const E4 *>(bias + min(r * 16 + kq * 4, p.Co - 4));
+    }
+    if (tid < hal_h) s_row[tid] = 0;
+    __syncthreads();
+    const E *inb = in + (size_t)b * p.Hi * p.Wi * CIN;
+    const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
+    for (int hp = tid; hp < hal_h * hal_w; hp += 256) {
+        const int hy = hp / hal_w, hx = hp - hy * hal_w;
+        const int iy = iy0 + hy, ix = ix0 + hx;
+        const bool ok = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
+        const size_t pix = ok ? (size_t)iy * p.Wi + ix : 0;
+        const int word = mb[pix];
+        const bool m = ok && word != 0;
+        E8 v[CV] = {};
+        // small maps: the pixel is requested together with its mask word (one round trip);
+        // lazy: only updated pixels are read
+        if (!lazy || m) {
+#pragma unroll
+            for (int c = 0; c < CV; ++c) v[c] = *reinterpret_cast<const E8 *>(inb + pix * CIN + c * 8);
+        }
+#pragma unroll
+        for (int c = 0; c < CV; ++c) *reinterpret_cast<E8 *>(s_x + hp * CIN + c * 8) = keep8(v[c], m);
+        if (m) atomicOr(&s_row[hy], 1u << hx);
+    }
+    __syncthreads();
+
+    const int ly = wave * 2 + (l16 >> 3), lx = l16 & 7;
+    const int oy = ty0 + ly, ox = tx0 + lx;
+    const bool inside = oy < p.Ho && ox < p.Wo;
+    unsigned any = 0;
+    for (int ky = 0; ky < p.Kh; ++ky) any |= (s_row[ly * p.sh + ky] >> (lx * p.sw)) & ((1u << p.Kw) - 1u);
+    const bool upd = inside && any != 0;
+    const size_t po = ((size_t)b * p.Ho + oy) * p.Wo + ox;
+    if (inside && kq == 0 && (MODE == 0 || !upd)) out_mask[po] = upd ? 1 : 0;
+    const uint64_t bu = ballot(upd);
+    if (bu == 0) return;
+    if (lazy) load_filter();
+
+    // the row pieces this lane finishes: piece c = lane + i * 64 of the wavefront's 16 rows is piece
+    // c % rc of pixel c / rc; the cached state is requested now, before the contraction
+    int ppix[PIECES], pcol[PIECES];
+    bool pon[PIECES];
+    size_t poff[PIECES], ppo[PIECES];
+    E8 qrow[MODE == 2 ? PIECES : 1], trow[MODE == 2 ? PIECES : 1];
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+        const int c = lane + i * WAVE;
+        const int r = min(c / rc, 15), cc = c - (c / rc) * rc;
+        ppix[i] = r;
+        pcol[i] = cc * 8;
+        pon[i] = c < 16 * rc && ((bu >> r) & 1);
+        const int ry = ty0 + wave * 2 + (r >> 3), rx = tx0 + (r & 7);
+        ppo[i] = pon[i] ? ((size_t)b * p.Ho + ry) * p.Wo + rx : 0;
+        poff[i] = ppo[i] * p.Co + (pon[i] ? pcol[i] : 0);
+        if (MODE == 2) {
+            qrow[i] = *reinterpret_cast<const E8 *>((const E *)epi.prev + poff[i]);
+            trow[i] = *reinterpret_cast<const E8 *>((const E *)epi.trunc + poff[i]);
+        }
+    }
+    float4_t acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < NS; ++st) {
+        if (st * TPS < K2) {  // uniform
+            const int t = min(st * TPS + tsub, K2 - 1);
+            const int ky = t / p.Kw, kx = t - ky * p.Kw;
+            const E8 x = *reinterpret_cast<const E8 *>(s_x + ((ly * p.sh + ky) * hal_w + lx * p.sw + kx) * CIN + c8 * 8);
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = Elem16<E>::mfma(a[r][st], x, acc[r]);
+        }
+    }
+    // rounded result into the wavefront's LDS tile, pixel rows contiguous
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        E4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = E(acc[r][i] + float(bv[r][i]));
+        *reinterpret_cast<E4 *>(s_v + l16 * ROWB + r * 32 + kq * 8) = v;
+    }
+    if (MODE == 2 && lane < 16) s_keep[wave][lane] = 0;
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    E8 vrow[PIECES];
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) vrow[i] = *reinterpret_cast<const E8 *>(s_v + ppix[i] * ROWB + pcol[i] * 2);
+    if (MODE == 0) {
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i)
+            if (pon[i]) *reinterpret_cast<E8 *>(out + poff[i]) = vrow[i];
+        return;
+    }
+    constexpr int ACTC = ACT < 0 ? 0 : ACT;
+    const E thr = E(epi.thr);
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+        bool hit = false;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const E t = trow[i][j] + vrow[i][j];
+            const E sm = t + qrow[i][j];
+            const E d = act_apply<E>(sm, ACTC) - act_apply<E>(qrow[i][j], ACTC);
+            hit |= tabs(d) > thr;
+        }
+        if (pon[i] && hit) s_keep[wave][ppix[i]] = 1;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    // second pass: T, S, D again (a handful of operations, cheaper than holding them)
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+        if (!pon[i]) continue;
+        const bool keep = s_keep[wave][ppix[i]] != 0;
+        if (pcol[i] == 0) out_mask[ppo[i]] = keep ? 1 : 0;
+        E8 tv, sv, dv, z;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            tv[j] = trow[i][j] + vrow[i][j];
+            sv[j] = tv[j] + qrow[i][j];
+            dv[j] = act_apply<E>(sv[j], ACTC) - act_apply<E>(qrow[i][j], ACTC);
+            z[j] = E(0);
+        }
+        if (keep) {
+            *reinterpret_cast<E8 *>((E *)epi.prev + poff[i]) = sv;
+            *reinterpret_cast<E8 *>(out + poff[i]) = dv;
+            *reinterpret_cast<E8 *>((E *)epi.trunc + poff[i]) = z;
+        } else {
+            *reinterpret_cast<E8 *>((E *)epi.trunc + poff[i]) = tv;
+        }
+    }
+}
+
 // Filter of conv_stem_mfma_kernel: fragment (channel tile, ky) holds, for lane (l16, kq) and
 // element e, W[co = tile * 16 + l16][ky][kx = (kq * 8 + e) / 4][ci = (kq * 8 + e) % 4], zero past
 // Kw, Cin and Cout.  Reads the processed fp16 layout (rows swizzled by the output parity) or,
@@ -2211,6 +2404,64 @@ bool try_stem_mfma(const dc_geometry &g, const ConvP &p, const E *in, const E *p
     return true;
 }
 
+// Shapes conv_thin_mfma_kernel takes (16-bit types).
+inline bool thin_shape(const dc_geometry &g) {
+    return g.groups == 1 && (g.in_c == 8 || g.in_c == 16) && g.kernel_h <= 3 && g.kernel_w <= 3 &&
+           g.kernel_h * g.kernel_w >= 2 && g.dilation_h == 1 && g.dilation_w == 1 && g.stride_h <= 2 && g.stride_w <= 2 &&
+           g.out_c % 8 == 0 && g.out_c <= 64 &&
+           (int64_t)g.batch * g.out_h * g.out_w >= 32768 &&  // small maps: latency, not bandwidth, is the cost
+           !patch_eligible(g, DC_F16);                       // ... and the 4x4-patch kernel's layers stay with it
+}
+
+// Thin K x K layers of large maps on the matrix cores (see conv_thin_mfma_kernel).  Returns 0 if
+// the shape, the operands' alignment or the map size do not qualify (nothing launched), 1 if the
+// layer is done, 2 if the convolution is done and the caller has to launch the activation /
+// truncation `epi` describes (anything but the maximum norm): the layer keeps this kernel's
+// summation order whatever follows it.
+template <typename E>
+int try_thin_mfma(const dc_geometry &g, const ConvP &p, const E *in, const E *packed, const E *bias, E *out,
+                  const int32_t *mask, int32_t *out_mask, const ActEpilogue *epi, hipStream_t s) {
+    const auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (packed == nullptr || !thin_shape(g)) return 0;
+    if (!al16(in) || !al16(out) || !al16(packed) || (bias && (reinterpret_cast<uintptr_t>(bias) & 7u) != 0)) return 0;
+    const ActEpilogue *pending = nullptr;
+    if (epi && (epi->mode != DC_TRUNC_MAX || epi->trunc == nullptr || !al16(epi->prev) || !al16(epi->trunc))) {
+        pending = epi;
+        epi = nullptr;
+    }
+    const int hal_h = (TILE - 1) * g.stride_h + g.kernel_h, hal_w = (TILE - 1) * g.stride_w + g.kernel_w;
+    const int co_tiles = ceil_div(g.out_c, 16);
+    const int R = co_tiles <= 1 ? 1 : co_tiles <= 2 ? 2 : 4;
+    const size_t lds = (size_t)hal_h * hal_w * g.in_c * 2 + (size_t)4 * 16 * (R * 32 + 16) + (size_t)hal_h * 4;
+    dim3 grid(ceil_div(g.out_w, TILE), ceil_div(g.out_h, TILE), g.batch);
+    EpiP e{epi ? epi->prev : nullptr, epi ? epi->trunc : nullptr, epi ? epi->thr : 0.f, epi ? epi->mode : 0};
+    const int act = epi ? (epi->act < 0 ? 0 : epi->act) : -1;
+    const int lazy = (int64_t)g.batch * g.in_h * g.in_w >= (1 << 18) ? 1 : 0;
+    note_kernel("conv_thin_mfma_kernel");
+#define DC_TH_R(CI, M, A)                                                                                            \
+    do {                                                                                                             \
+        if (R == 1) conv_thin_mfma_kernel<E, CI, 1, M, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_w, lazy); \
+        else if (R == 2) conv_thin_mfma_kernel<E, CI, 2, M, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_w, lazy); \
+        else conv_thin_mfma_kernel<E, CI, 4, M, A><<<grid, 256, lds, s>>>(p, in, packed, bias, out, mask, out_mask, e, hal_h, hal_w, lazy); \
+    } while (0)
+#define DC_TH(M, A)                                                                                                  \
+    do {                                                                                                             \
+        if (g.in_c == 16) DC_TH_R(16, M, A); else DC_TH_R(8, M, A);                                                  \
+    } while (0)
+    switch (act) {
+        case DC_ACT_LINEAR: DC_TH(2, DC_ACT_LINEAR); break;
+        case DC_ACT_RELU: DC_TH(2, DC_ACT_RELU); break;
+        case DC_ACT_RELU6: DC_TH(2, DC_ACT_RELU6); break;
+        case DC_ACT_LEAKY: DC_TH(2, DC_ACT_LEAKY); break;
+        case DC_ACT_SIGMOID: DC_TH(2, DC_ACT_SIGMOID); break;
+        case DC_ACT_SWISH: DC_TH(2, DC_ACT_SWISH); break;
+        default: DC_TH(0, 0); break;
+    }
+#undef DC_TH
+#undef DC_TH_R
+    return pending != nullptr ? 2 : 1;
+}
+
 template <typename T>
 bool try_fewcin(const dc_geometry &g, const ConvP &p, const T *in, const T *filter, const T *bias,
                 T *out, const int32_t *mask, int32_t *out_mask, const ActEpilogue *epi,
@@ -2453,6 +2704,8 @@ bool lds_add_eligible(const dc_geometry &g, int dtype, int activation, bool tran
     // transposed: every stride phase of the output needs at least one tap (window >= stride), so
     // that every output tile runs the reduction kernel's epilogue
     if (transposed && (g.kernel_h < g.stride_h || g.kernel_w < g.stride_w)) return false;
+    // a layer of the thin-layer kernel keeps that kernel's summation order: no fused sum
+    if (!transposed && thin_shape(g)) return false;
     return activation <= 0 && mfma_eligible(g, dtype) && g.kernel_h * g.kernel_w <= MFMA_MAX_TAPS && !patch_eligible(g, dtype) &&
            lds_plan(g, transposed).ok;
 }
@@ -2556,6 +2809,14 @@ hipError_t launch_conv_t(const dc_geometry &g, const void *in, const void *filte
         if (dtype != DC_F32 && try_stem_mfma<E16>(g, p, (const E16 *)in, (const E16 *)packed, (const E16 *)bias,
                                                   (E16 *)out, mask, out_mask, epi, s))
             return hipGetLastError();
+        const int thin = dtype == DC_F32 ? 0 : try_thin_mfma<E16>(g, p, (const E16 *)in, (const E16 *)packed, (const E16 *)bias,
+                                                                  (E16 *)out, mask, out_mask, epi, s);
+        if (thin != 0) {
+            const hipError_t te = hipGetLastError();
+            if (te != hipSuccess || thin == 1) return te;
+            return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
+                                            epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
+        }
         const bool few = dtype == DC_F32
             ? try_fewcin<float>(g, p, (const float *)in, (const float *)filter, (const float *)bias, (float *)out, mask, out_mask, epi, s)
             : dtype == DC_BF16

@@ -340,6 +340,14 @@ CONVS = [
     (64, 48, 3, 1, 2, 2, 1, 80, 81),        # dilation 2
     (32, 64, 5, 1, 2, 1, 1, 64, 66),        # 5x5
     (24, 40, 3, 1, 1, 1, 1, 128, 130),      # partial reduction step and partial channel tile
+    # thin layers (8 or 16 input channels) on large maps: several taps per reduction step
+    (16, 16, 3, 1, 1, 1, 1, 200, 190),      # five steps, one channel tile
+    (16, 32, 3, 2, 1, 1, 1, 520, 500),      # stride 2 on a map of 2^18 pixels and more: only updated pixels are staged
+    (8, 24, 3, 1, 1, 1, 1, 130, 131),       # three steps, a partial channel tile
+    (16, 64, 3, 1, 1, 1, 1, 160, 170),      # four channel tiles per wavefront
+    (8, 8, 3, 2, 1, 1, 1, 400, 401),        # half a channel tile
+    (16, 40, 2, 2, 0, 1, 1, 300, 300),      # 2 x 2 window
+    (8, 48, (1, 3), 1, (0, 1), 1, 1, 150, 160),  # one window row
     (16, 16, 3, 1, 1, 1, 16, 726, 727),     # depthwise on a very large map: mask scan and compaction per wavefront
     (24, 24, 3, 1, 1, 1, 24, 600, 601),     # ... with idle lanes in the group
     (16, 16, 3, 2, 1, 1, 16, 600, 521),     # ... with a stride
@@ -452,7 +460,9 @@ def test_conv_resident_filter(lib, dtype, cfg, density):
     ((16, 64, 3, 1, 1, 1, 1, 120, 120), "conv_lds_mfma_kernel"),
     ((320, 32, 3, 1, 1, 1, 1, 40, 40), "conv_lds_mfma_kernel"),
     ((64, 64, 3, 1, 1, 1, 1, 256, 250), "conv_res_mfma_kernel"),   # thin layers on >= 1024 tiles: resident filter
-    ((16, 32, 3, 2, 1, 1, 1, 520, 500), "conv_lds_mfma_kernel"),   # one channel step: the per-tile kernel stays
+    ((32, 32, 3, 2, 1, 1, 1, 520, 500), "conv_lds_mfma_kernel"),   # one channel step: the per-tile kernel stays
+    ((16, 32, 3, 2, 1, 1, 1, 520, 500), "conv_thin_mfma_kernel"),  # 8 / 16 input channels on a large map
+    ((8, 24, 3, 1, 1, 1, 1, 130, 131), "conv_thin_mfma_kernel"),
     ((64, 256, 1, 1, 0, 1, 1, 20, 20), "pw_mfma_kernel"),
     ((32, 32, 3, 1, 1, 1, 32, 15, 18), "conv_dw_kernel"),
     ((16, 16, 3, 1, 1, 1, 16, 726, 727), "conv_dw_scan_kernel"),
@@ -558,6 +568,10 @@ FUSED = [
     (64, 64, 3, 1, 1, 1, 64, 180, 181),     # large map: strips of four pixels per lane group
     (144, 144, 3, 1, 1, 1, 144, 130, 131),  # ... wide rows, filter through LDS
     (16, 96, 1, 1, 0, 1, 1, 110, 111),      # pointwise on a large map: convolution and activation as two launches
+    (16, 16, 3, 1, 1, 1, 1, 200, 190),      # thin layer on a large map: epilogue on pixel rows in the kernel
+    (16, 32, 3, 2, 1, 1, 1, 520, 500),      # ... stride 2, only updated pixels staged
+    (8, 24, 3, 1, 1, 1, 1, 130, 131),       # ... 8 input channels, a partial channel tile
+    (16, 64, 3, 1, 1, 1, 1, 160, 170),      # ... four channel tiles: two passes over the row pieces
 ]
 
 
