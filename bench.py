@@ -722,6 +722,29 @@ def main():
             log(f"MobileNetV2 on the moving-rectangles clip: {nets[-1]['value']:.0f} frames/s")
         section("networks.mobilenetv2_clip", config3_section)
         emit()
+
+        def default_init_section():
+            # the same network and clip with PyTorch's own initialisation left as it is (no rescaling
+            # of the weights on data): activations shrink from layer to layer, so threshold 0.05
+            # truncates far more than in a trained network -- the other end of the range
+            from deltacnn_amd import sparse_layers as SL
+            from deltacnn_amd.networks import DenseLayers, MobileNetV2
+            torch.manual_seed(0)
+            d0 = MobileNetV2(DenseLayers).eval().to("cuda", memory_format=torch.channels_last)
+            st = {k: v.clone() for k, v in d0.state_dict().items()}
+            d0 = d0.half()
+            SL.DCThreshold.t_default = THRESHOLD
+            m0 = MobileNetV2(SL).eval()
+            m0.load_state_dict(st)
+            m0 = m0.to("cuda", memory_format=torch.channels_last).half()
+            m0.process_filters()
+            clip = gpu_frames(moving_rectangles_video(frames=max(64, clip_frames(nw_steps, nw_warm))))
+            nets.append(_network_report("mobilenetv2 (PyTorch default initialisation, weights not rescaled)", (224, 224), m0, d0,
+                                        clip, nw_steps, nw_warm, "as above"))
+            log(f"MobileNetV2, default initialisation: {nets[-1]['value']:.0f} frames/s, mean density "
+                f"{nets[-1]['mean_input_density_of_library_calls']}")
+        section("networks.mobilenetv2_default_init", default_init_section)
+        emit()
         for which in ("hrnet", "dla34"):
             def net_section(which=which):
                 nets.append(network_bench(which, nw_steps, nw_warm))
