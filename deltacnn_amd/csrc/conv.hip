@@ -966,12 +966,66 @@ struct PatchRes {  // DCAdd fused behind the convolution: a = residual, b = conv
 constexpr int LDS_MAX_HALO = 1024;
 constexpr int LDS_MAX_STEPS = 1024;
 
-template <typename E, int R, int S, int D, int KS, bool TR, bool ADD>
+// The layer's activation / truncation finished in the convolution's launch (FIN), for layers whose
+// workgroups hold all output channels of their pixels (the keep decision of a pixel needs them
+// all): the wavefronts put their rounded sums into LDS as pixel rows and the workgroup runs
+// act_trunc_pixel over the rows, 2^lg lanes per pixel; the cached state of the first pass is
+// requested before the reduction.  `out` receives the activated differences of the kept pixels
+// only.  Offered where the launch has at most one workgroup per compute unit: the finishing stores
+// three tensors, which a workgroup that is followed by another on its compute unit only delays
+// (measured on 64 -> 64 at 136 x 240, 510 workgroups: 8.3 + 4.6 us as two launches, 13.5 us as
+// one; 128 -> 64 at 68 x 120, 135 workgroups: 7.7 + 2.9 -> 9.1 us).
+template <typename E>
+struct LdsFin {
+    E *prev, *trunc;
+    float thr;
+    int mode, act;
+    int lg, iters;  // 2^lg lanes per pixel, `iters` 16-byte vectors per lane
+};
+
+// The finishing passes: 2^lg lanes per pixel over the compacted list `list` of `n` tile pixels
+// (`opix`: tile pixel -> pixel index in the output map).  The sums lie in LDS, row `slot` at
+// rows + slot * row_b; q0 / tr0 hold the state of the first pass.
+template <typename E, int ITERS, int ACT, typename PixelOf>
+__device__ __forceinline__ void lds_finish(const LdsFin<E> &f, const int *list, int n, int tid, int nthr, int Co,
+                                           E *__restrict__ out, int32_t *__restrict__ out_mask, PixelOf opix,
+                                           const unsigned char *rows, int row_b,
+                                           const Vec<E, Vec16<E>::N> (&q0)[2], const Vec<E, Vec16<E>::N> (&tr0)[2]) {
+    constexpr int N = Vec16<E>::N;
+    const int G = 1 << f.lg, gl = tid & (G - 1), groups = nthr >> f.lg;
+    for (int s0 = 0; s0 < n; s0 += groups) {  // the same number of passes in every wavefront
+        const int slot = min(s0 + (tid >> f.lg), n - 1);
+        const bool valid = s0 + (tid >> f.lg) < n;
+        const size_t px = opix(list[slot] & 63);
+        Vec<E, N> dl[ITERS], q[ITERS], tr[ITERS];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {  // later passes request their state here
+            const int c = min((it * G + gl) * N, Co - N);
+            const size_t off = px * Co + c;
+            dl[it] = *reinterpret_cast<const Vec<E, N> *>(rows + slot * row_b + c * (int)sizeof(E));
+            if (s0 == 0) {
+                q[it] = q0[it];
+                tr[it] = tr0[it];
+            } else {
+                q[it] = vload<E, N>(f.prev + off);
+                tr[it] = vload<E, N>(f.trunc + off);
+            }
+        }
+        const bool keep = act_trunc_pixel<E, ITERS, ACT>(dl, q, tr, valid, px, gl, G, Co, out, f.prev, f.trunc,
+                                                         out_mask, E(f.thr), f.mode);
+        if (valid && keep && gl == 0) out_mask[px] = 1;
+    }
+}
+
+template <typename E, int R, int S, int D, int KS, bool TR, bool ADD, bool FIN = false>
 __global__ void __launch_bounds__(8 * WAVE)
 conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp,
                      const E *__restrict__ bias, E *__restrict__ out,
                      const int32_t *__restrict__ mask, int32_t *__restrict__ out_mask,
-                     int co_blocks, int ci_p, int hal_h, int hal_w, int kcc, int lgv, PatchRes<E> rs) {
+                     int co_blocks, int ci_p, int hal_h, int hal_w, int kcc, int lgv, PatchRes<E> rs,
+                     LdsFin<E> fin_args) {
+    static_assert(!(FIN && (TR || ADD)), "the finishing pass exists for plain convolutions");
+    // FIN: launched with co_blocks == 1
     // ADD: the sum of a DCAdd without activation rides on the accumulators.  (With an activation the
     // accumulated sum has to be read and written as well; in this kernel's 8-byte-per-lane epilogue
     // that costs what the separate add kernel costs -- measured -- so that form is not offered.)
@@ -1155,7 +1209,7 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
     // dilate the mask over the window and compact the updated pixels: by every wavefront for itself
     // (the same table, hence the same list in all of them), while the halo rows are still travelling
     int n;
-    bool tile_upd;
+    bool tile_upd, any_px;
     {
         bool upd = false;
         const int base = ly * vsy * hal_w + lx * vsx;
@@ -1169,8 +1223,11 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
         upd = upd && inside;
         const bool radd = ADD && inside && rword != 0;
         const bool any = upd || radd;  // ADD: the union of both masks is written and compacted
-        if (inside && cb == 0 && wv == 0) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = any ? 1 : 0;
+        any_px = any;
+        // FIN: the finishing workgroup writes the mask; a tile without updates has none
         const int rank = wave_rank(any, n);
+        if (inside && cb == 0 && wv == 0 && (!FIN || n == 0))
+            out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = any ? 1 : 0;
         if (any) s_list[wv][rank] = lane | (upd ? 64 : 0) | (radd ? 128 : 0);
         tile_upd = ballot(upd) != 0;
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
@@ -1216,6 +1273,22 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
                     const int c = min(co + i, p.Co - 1);
                     if (radd) rv[q][i] = rs.values[off + c];
                 }
+            }
+        }
+    }
+    // FIN, all channels in this workgroup: the cached state of the first finishing pass, requested
+    // before the reduction, which it overlaps
+    auto opix = [&](int loc) { return ((size_t)b * p.Ho + out_y(loc >> 3)) * p.Wo + out_x(loc & 7); };
+    Vec<E, Vec16<E>::N> fq[2], ftr[2];
+    if (FIN) {
+        const int slot = min(tid >> fin_args.lg, n - 1), gl = tid & ((1 << fin_args.lg) - 1);
+        const size_t row = opix(s_list[wv][slot] & 63) * p.Co;
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            if (it < fin_args.iters) {
+                const int c = min(((it << fin_args.lg) + gl) * 8, p.Co - 8);
+                fq[it] = vload<E, 8>(fin_args.prev + row + c);
+                ftr[it] = vload<E, 8>(fin_args.trunc + row + c);
             }
         }
     }
@@ -1328,6 +1401,11 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
 #pragma unroll
         for (int q = 0; q < TPW; ++q) fin[q] = acc[q / NT][q % NT];
     }
+    // FIN: the sums go to LDS as pixel rows, behind the partial sums
+    constexpr bool to_rows = FIN;
+    unsigned char *s_rows = s_halo + (KS > 1 ? KS * ncw * R * NT * WAVE * 16 : 0);
+    const int row_b = p.Co * (int)sizeof(E) + 16;
+    if (FIN && KS == 1) __syncthreads();  // the halo is still being read by slower wavefronts
 #pragma unroll
     for (int q = 0; q < TPW; ++q) {
         const int t = kz * TPW + q, nt = t % NT;
@@ -1354,13 +1432,29 @@ conv_lds_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ wp
                 v[i] = sum;
             }
         }
-        if (vec) {
+        if (to_rows) {  // (Co % 8 == 0: whole vectors)
+            if (co < p.Co) *reinterpret_cast<E4 *>(s_rows + pix * row_b + co * (int)sizeof(E)) = v;
+        } else if (vec) {
             *reinterpret_cast<E4 *>(o) = v;
         } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
                 if (co + i < p.Co) o[i] = v[i];
         }
+    }
+    if (FIN) {
+        __syncthreads();
+        if (wv == 0 && inside && !any_px) out_mask[((size_t)b * p.Ho + oy) * p.Wo + ox] = 0;
+#define DC_FIN_ACT(IT)                                                                                          \
+    switch (fin_args.act) {                                                                                     \
+        case DC_ACT_RELU: lds_finish<E, IT, DC_ACT_RELU>(fin_args, s_list[wv], n, tid, nthr, p.Co, out, out_mask, opix, s_rows, row_b, fq, ftr); break;   \
+        case DC_ACT_RELU6: lds_finish<E, IT, DC_ACT_RELU6>(fin_args, s_list[wv], n, tid, nthr, p.Co, out, out_mask, opix, s_rows, row_b, fq, ftr); break; \
+        case DC_ACT_LEAKY: lds_finish<E, IT, DC_ACT_LEAKY>(fin_args, s_list[wv], n, tid, nthr, p.Co, out, out_mask, opix, s_rows, row_b, fq, ftr); break; \
+        default: lds_finish<E, IT, DC_ACT_LINEAR>(fin_args, s_list[wv], n, tid, nthr, p.Co, out, out_mask, opix, s_rows, row_b, fq, ftr); break;          \
+    }
+        if (fin_args.iters == 1) DC_FIN_ACT(1)
+        else DC_FIN_ACT(2)
+#undef DC_FIN_ACT
     }
 }
 
@@ -2579,37 +2673,67 @@ LdsPlan lds_plan(const dc_geometry &g, bool transposed) {
 
 // res != nullptr (plain convolutions only): the DCAdd behind the convolution runs on the
 // accumulators, see conv_lds_mfma_kernel.
+// Can the layer's activation / truncation be finished in the convolution's launch?  One workgroup
+// holds all channels of its pixels, rows of 16-byte vectors, at most two per lane of a wavefront,
+// and no more workgroups than compute units (see LdsFin).
+bool lds_finishes_activation(const dc_geometry &g, const LdsPlan &lp, bool transposed, const Residual *res,
+                             const void *out, const ActEpilogue *epi) {
+    const auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (epi == nullptr || transposed || res != nullptr || epi->mode < 0 || epi->trunc == nullptr || epi->prev == nullptr)
+        return false;
+    if (epi->act != DC_ACT_LINEAR && epi->act != DC_ACT_RELU && epi->act != DC_ACT_RELU6 && epi->act != DC_ACT_LEAKY)
+        return false;
+    if (g.out_c % 8 != 0 || g.out_c > 1024 || !al16(epi->prev) || !al16(epi->trunc) || !al16(out)) return false;
+    return ceil_div(ceil_div(g.out_c, 16), lp.ncw * lp.rl) == 1 && (int64_t)lp.ltx * lp.lty * g.batch <= 256;
+}
+
+// epi + fused: the layer's activation / truncation, finished in this launch where
+// lds_finishes_activation allows (then *fused = true), else left to the caller.
 template <typename E>
 hipError_t launch_lds_conv(const dc_geometry &g, const ConvP &p, const LdsPlan &lp, const void *in, const void *packed,
                            const void *bias, void *out, const int32_t *mask, int32_t *out_mask, bool transposed,
-                           const Residual *res, hipStream_t s) {
+                           const Residual *res, hipStream_t s, const ActEpilogue *epi = nullptr,
+                           bool *fused = nullptr) {
     const int co_tiles = ceil_div(g.out_c, 16);
     const int ci_p = round_up(g.in_c, 32);
     const int hpx = lp.hal_h * lp.hal_w;
     const int kcc = lp.kcc, hal_h = lp.hal_h, hal_w = lp.hal_w;
     const int nwv = lp.ncw * lp.ksl;  // wavefronts per workgroup
     const int cbl = ceil_div(co_tiles, lp.ncw * lp.rl);
-    const size_t lds = std::max((size_t)hpx * (kcc * 64 + 16), lp.ksl > 1 ? (size_t)lp.ksl * lp.ncw * lp.rl * 4 * 1024 : 0);
+    size_t lds = std::max((size_t)hpx * (kcc * 64 + 16), lp.ksl > 1 ? (size_t)lp.ksl * lp.ncw * lp.rl * 4 * 1024 : 0);
     const int lgv = log2i(pow2_ceil(kcc * 4));  // lanes per halo pixel while staging
     dim3 lgrid(lp.ltx, lp.lty, g.batch * cbl);
     PatchRes<E> rs{nullptr, nullptr, nullptr, 0.f, 0.f, 0};
     if (res != nullptr) rs = PatchRes<E>{(const E *)res->values, res->mask, (E *)res->prev, res->wa, res->wb, res->act};
+    const bool fin = fused != nullptr && lds_finishes_activation(g, lp, transposed, res, out, epi);
+    if (fused != nullptr) *fused = fin;
+    LdsFin<E> lf{nullptr, nullptr, 0.f, 0, 0, 0, 1};
+    if (fin) {
+        const int nvec = g.out_c / 8;
+        const int iters = nvec > WAVE ? 2 : 1;
+        lf = LdsFin<E>{(E *)epi->prev, (E *)epi->trunc, epi->thr, epi->mode, epi->act,
+                       log2i(pow2_ceil(ceil_div(nvec, iters))), iters};
+        // the tile's sums as pixel rows behind the partial sums of the reduction slices
+        lds = std::max(lds, (lp.ksl > 1 ? (size_t)lp.ksl * lp.ncw * lp.rl * 4 * 1024 : 0) +
+                                (size_t)TILE_PX * (g.out_c * 2 + 16));
+    }
     note_kernel("conv_lds_mfma_kernel");
-#define DC_LDS_ARGS (p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv, rs)
-#define DC_LDS_K(RV, SV, DV, KV, TV, AV)                                                                    \
+#define DC_LDS_ARGS (p, (const E *)in, (const E *)packed, (const E *)bias, (E *)out, mask, out_mask, cbl, ci_p, hal_h, hal_w, kcc, lgv, rs, lf)
+#define DC_LDS_K(RV, SV, DV, KV, TV, AV, FV)                                                                \
     do {                                                                                                    \
         if (lds > (48u << 10)) {                                                                            \
-            const hipError_t big = allow_large_lds(&conv_lds_mfma_kernel<E, RV, SV, DV, KV, TV, AV>);       \
+            const hipError_t big = allow_large_lds(&conv_lds_mfma_kernel<E, RV, SV, DV, KV, TV, AV, FV>);   \
             if (big != hipSuccess) return big;                                                              \
         }                                                                                                   \
-        conv_lds_mfma_kernel<E, RV, SV, DV, KV, TV, AV><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS;          \
+        conv_lds_mfma_kernel<E, RV, SV, DV, KV, TV, AV, FV><<<lgrid, nwv * WAVE, lds, s>>> DC_LDS_ARGS;      \
     } while (0)
 #define DC_LDS_L(RV, SV, DV, KV)                                                                            \
     do {                                                                                                    \
-        if (res != nullptr && transposed) DC_LDS_K(RV, SV, DV, KV, true, true);                             \
-        else if (res != nullptr) DC_LDS_K(RV, SV, DV, KV, false, true);                                     \
-        else if (transposed) DC_LDS_K(RV, SV, DV, KV, true, false);                                         \
-        else DC_LDS_K(RV, SV, DV, KV, false, false);                                                        \
+        if (res != nullptr && transposed) DC_LDS_K(RV, SV, DV, KV, true, true, false);                      \
+        else if (res != nullptr) DC_LDS_K(RV, SV, DV, KV, false, true, false);                              \
+        else if (transposed) DC_LDS_K(RV, SV, DV, KV, true, false, false);                                  \
+        else if (fin) DC_LDS_K(RV, SV, DV, KV, false, false, true);                                         \
+        else DC_LDS_K(RV, SV, DV, KV, false, false, false);                                                 \
     } while (0)
     if (lp.rl == 1) DC_LDS_L(1, 2, 3, 1);
     else if (lp.ksl == 1) DC_LDS_L(2, 2, 3, 1);
@@ -2849,11 +2973,12 @@ hipError_t launch_conv_t(const dc_geometry &g, const void *in, const void *filte
             // thin layers on large maps: the filter stays in registers while a workgroup walks over tiles
             const bool resident = !transposed &&
                 resident_conv_eligible(g, lp.hal_h, lp.hal_w, lp.ltx, lp.lty, lp.kcc, lp.rl, lp.ksl, lp.ncw);
+            bool fused = false;
             hipError_t le = resident
                 ? launch_resident_conv(g, p, lp.hal_h, lp.hal_w, lp.ltx, lp.lty, lp.kcc, lp.rl, lp.ksl, lp.ncw, in, packed,
                                        bias, out, mask, out_mask, dtype, s)
-                : launch_lds_conv<E16>(g, p, lp, in, packed, bias, out, mask, out_mask, transposed, nullptr, s);
-            if (le != hipSuccess || epi == nullptr) return le;
+                : launch_lds_conv<E16>(g, p, lp, in, packed, bias, out, mask, out_mask, transposed, nullptr, s, epi, &fused);
+            if (le != hipSuccess || epi == nullptr || fused) return le;
             return launch_activate_truncate(out, epi->prev, epi->trunc, out_mask, epi->thr, epi->act,
                                             epi->mode, g.batch * g.out_h * g.out_w, g.out_c, dtype, s);
         }

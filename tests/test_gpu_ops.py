@@ -572,7 +572,14 @@ FUSED = [
     (16, 32, 3, 2, 1, 1, 1, 520, 500),      # ... stride 2, only updated pixels staged
     (8, 24, 3, 1, 1, 1, 1, 130, 131),       # ... 8 input channels, a partial channel tile
     (16, 64, 3, 1, 1, 1, 1, 160, 170),      # ... four channel tiles: two passes over the row pieces
+    (64, 64, 3, 1, 1, 1, 1, 70, 66),        # halo kernel, one workgroup holds all channels: it finishes the activation
+    (128, 64, 3, 1, 1, 1, 1, 72, 61),       # ... four reduction slices
+    (32, 64, 3, 2, 1, 1, 1, 176, 175),      # ... stride 2
+    (64, 56, 3, 1, 1, 1, 1, 70, 66),        # ... a partial channel tile
+    (32, 24, 5, 1, 2, 1, 1, 90, 77),        # ... 5x5
+    (64, 64, 3, 1, 1, 1, 1, 136, 120),      # ... more workgroups than compute units: two launches
 ]
+HALO_FINISHED = FUSED[-6:-1]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -598,6 +605,8 @@ def test_conv_activation_fused(lib, dtype, cfg, act, mode):
     p2, t2 = cl(prev), cl(trunc)
     out2, om2 = hk().sparse_conv_activation(dx, d_filt, dm, None, p2, t2, 0.3, act, mode, s, p, d, groups, Cout,
                                             packed_filter=pk)
+    if cfg in HALO_FINISHED and dtype != torch.float32 and act != 5:
+        assert _last_kernel() == "conv_lds_mfma_kernel"   # one launch
     assert torch.equal(om1, om2)
     assert 0 < int(om1.sum()) and (mode != 0 or int(om1.sum()) < int(want_mask.sum()))
     assert torch.equal(p1, p2) and torch.equal(t1, t2)
