@@ -107,9 +107,6 @@ pw_pair_kernel(PairP p, PairPtr<E> q) {
 #pragma unroll
         for (int s = 0; s < S2; ++s)
             a2[j][s] = *reinterpret_cast<const E8 *>(q.w2 + ((size_t)ct * p.ksteps2 + min(s, p.ksteps2 - 1)) * 512 + lane * 8);
-        const size_t off = (size_t)pix * p.Ce + min(ct * 16 + kq * 4, p.Ce - 4);
-        tr2[j] = *reinterpret_cast<const E4 *>(q.trunc2 + off);
-        pv2[j] = *reinterpret_cast<const E4 *>(q.prev2 + off);
     }
     // the residual's values for the tile this wavefront finishes (tile `wave` of the projection)
     E4 rv = zero4<E>();
@@ -123,10 +120,15 @@ pw_pair_kernel(PairP p, PairPtr<E> q) {
         q.out_mask2[mp] = int((bo >> lane) & 1);
     }
     if (bo == 0) return;  // the same for every wavefront of the workgroup
+    // the expansion's cached state, for workgroups with an update: needed two barriers from here
+#pragma unroll
+    for (int j = 0; j < CT2; ++j) {
+        const size_t off = (size_t)pix * p.Ce + min(min(ct2[j], p.ce_tiles - 1) * 16 + kq * 4, p.Ce - 4);
+        tr2[j] = *reinterpret_cast<const E4 *>(q.trunc2 + off);
+        pv2[j] = *reinterpret_cast<const E4 *>(q.prev2 + off);
+    }
 #pragma unroll
     for (int j = 0; j < CT2; ++j) {  // arrived with the mask words: not to be moved down to the epilogue
-        DC_PIN(tr2[j]);
-        DC_PIN(pv2[j]);
 #pragma unroll
         for (int s = 0; s < S2; ++s) DC_PIN(a2[j][s]);
     }
