@@ -13,8 +13,11 @@
 // one (unconditionally, from clamped addresses, and selected by the mask afterwards) and staged
 // into the second of two LDS halo buffers right after it; every wavefront dilates and compacts
 // the tile's mask for itself; the partial sums of the reduction slices alternate between two
-// buffers as well, so the wavefronts that finish and store tile i never hold up the ones that
-// already contract tile i + 1.
+// buffers as well, so a wavefront that still finishes and stores tile i never holds up one that
+// already contracts tile i + 1.  The slices of a channel group share the finishing of its tiles
+// (each adds the partial sums of its share in ascending slice order, rounds and stores), and the
+// walk from tile to tile is carried in (map, tile row, tile column) so that no tile costs a
+// division; tiles whose halo lies inside the map skip the clamping of the row addresses.
 //
 // Everything else is the algorithm of conv_lds_mfma_kernel for a plain (not transposed)
 // convolution whose input channels fit one LDS chunk: halo staged in LDS with inactive and
@@ -50,6 +53,8 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
     typedef typename Elem16<E>::v4 E4;
     typedef typename Elem16<E>::v8 E8;
     constexpr int NT = 4;
+    constexpr int TPW = R * NT / KS;  // output tiles of 16 x 16 a wavefront finishes
+    static_assert(TPW * KS == R * NT, "the reduction slices of a channel group share its tiles evenly");
     // dynamic LDS: two halo buffers (tile i is contracted out of one while tile i + 1 is staged
     // into the other), then two buffers for the partial sums of the reduction slices
     extern __shared__ __align__(16) unsigned char s_dyn[];
@@ -69,7 +74,8 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
     const int row = q.kcc * 64 + 16;  // bytes per staged halo pixel
     const int halo_bytes = hpx * row;
     unsigned char *s_part0 = s_dyn + 2 * halo_bytes;
-    const int PART_BYTES = (KS - 1) * ncw * R * NT * WAVE * 16;  // (KS - 1) slices x ncw groups x R x NT tiles
+    // every wavefront leaves the partial sums of the (KS - 1) * TPW tiles that other slices finish
+    const int PART_BYTES = nw * (KS - 1) * TPW * WAVE * 16;
     auto tap_off = [&](int a, int b2) { return a * p.dh * hal_w + b2 * p.dw; };  // in halo pixels
 
     // step table: LDS byte offset of a step's input fragment relative to a pixel's halo origin
@@ -107,30 +113,69 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
     E8 val[SU];
     int word[SU], hpixel[SU];  // mask word; pixel index in the map, -1 outside of it
     int hyx[SU];               // the lane's halo pixels (row << 16 | column): the same for every tile
+    int hrel[SU];              // ... and their pixel offset from the halo's first pixel in the map
 #pragma unroll
     for (int u = 0; u < SU; ++u) {
         const int hp = min((tid >> q.lgv) + u * hstep, hpx - 1);
         const int hy = hp / hal_w;
         hyx[u] = (hy << 16) | (hp - hy * hal_w);
+        hrel[u] = hy * p.Wi + (hp - hy * hal_w);
     }
     const int cst = min(sv * 8, p.Ci - 8);
-    auto request = [&](int tile) {
-        const int b = tile / tiles_per_map, tr = tile - b * tiles_per_map;
-        const int iy0 = (tr / q.ltx) * TILE * p.sh - p.pt, ix0 = (tr % q.ltx) * TILE * p.sw - p.pl;
-        const int32_t *mb = mask + (size_t)b * p.Hi * p.Wi;
-        const E *inb = in + (size_t)b * p.Hi * p.Wi * p.Ci + cst;
+    // A tile is (map b, tile row ty, tile column tx); the walk from tile to tile + gridDim.x is
+    // carried in these coordinates, so that no tile costs a division.
+    struct TilePos {
+        int b, ty, tx;
+    };
+    const int gstep_b = (int)gridDim.x / tiles_per_map, gstep_r = (int)gridDim.x - gstep_b * tiles_per_map;
+    const int gstep_y = gstep_r / q.ltx, gstep_x = gstep_r - gstep_y * q.ltx;
+    auto advance = [&](TilePos t) {
+        t.tx += gstep_x;
+        t.ty += gstep_y;
+        t.b += gstep_b;
+        if (t.tx >= q.ltx) {
+            t.tx -= q.ltx;
+            ++t.ty;
+        }
+        if (t.ty >= q.lty) {
+            t.ty -= q.lty;
+            ++t.b;
+        }
+        return t;
+    };
+    auto request = [&](const TilePos &t) {
+        const int iy0 = t.ty * TILE * p.sh - p.pt, ix0 = t.tx * TILE * p.sw - p.pl;
+        const int32_t *mb = mask + (size_t)t.b * p.Hi * p.Wi;
+        const E *inb = in + (size_t)t.b * p.Hi * p.Wi * p.Ci + cst;
+        if (iy0 >= 0 && ix0 >= 0 && iy0 + hal_h <= p.Hi && ix0 + hal_w <= p.Wi) {  // uniform: nothing to clamp
+            const int base = iy0 * p.Wi + ix0;
 #pragma unroll
-        for (int u = 0; u < SU; ++u) {
-            const int iy = iy0 + (hyx[u] >> 16), ix = ix0 + (hyx[u] & 0xffff);
-            const bool ok = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
-            const int px = min(max(iy, 0), p.Hi - 1) * p.Wi + min(max(ix, 0), p.Wi - 1);
-            hpixel[u] = ok ? px : -1;
-            word[u] = mb[px];
-            val[u] = *reinterpret_cast<const E8 *>(inb + (unsigned)(px * p.Ci));
+            for (int u = 0; u < SU; ++u) {
+                const int px = base + hrel[u];
+                hpixel[u] = px;
+                word[u] = mb[px];
+                val[u] = *reinterpret_cast<const E8 *>(inb + (unsigned)(px * p.Ci));
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < SU; ++u) {
+                const int iy = iy0 + (hyx[u] >> 16), ix = ix0 + (hyx[u] & 0xffff);
+                const bool ok = iy >= 0 && iy < p.Hi && ix >= 0 && ix < p.Wi;
+                const int px = min(max(iy, 0), p.Hi - 1) * p.Wi + min(max(ix, 0), p.Wi - 1);
+                hpixel[u] = ok ? px : -1;
+                word[u] = mb[px];
+                val[u] = *reinterpret_cast<const E8 *>(inb + (unsigned)(px * p.Ci));
+            }
         }
     };
     // what was requested goes into halo buffer `buf`: table entry (first lane of a pixel) and bytes
     auto stage = [&](int buf) {
+        // What was requested has to have arrived here, for every lane: said once and without a
+        // condition (s_waitcnt vmcnt(0)).  The stores below sit under per-lane tests, and a wait
+        // that the compiler places inside them leaves it with a path on which the requests are
+        // still in flight -- it then guards later writes of the same registers with waits that, at
+        // run time, wait for the previous tile's output stores.
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         const bool vok = sv < q.kcc * 4 && sv * 8 < p.Ci;
         unsigned char *halo = s_dyn + buf * halo_bytes;
 #pragma unroll
@@ -144,22 +189,41 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
             }
         }
     };
+    TilePos pos;
+    {
+        const int t0 = min((int)blockIdx.x, q.tiles - 1);
+        pos.b = t0 / tiles_per_map;
+        const int tr = t0 - pos.b * tiles_per_map;
+        pos.ty = tr / q.ltx;
+        pos.tx = tr - pos.ty * q.ltx;
+    }
+    TilePos nxt = advance(pos);
     if ((int)blockIdx.x < q.tiles) {
-        request(blockIdx.x);
+        request(pos);
         stage(0);
     }
+    // Everything requested so far has arrived -- said explicitly (s_waitcnt vmcnt(0)): the compiler
+    // cannot see it on every path into the loop and would otherwise wait for the resident filter
+    // fragments in front of each matrix instruction of EVERY tile, where the count it waits on is
+    // that of the next tile's rows, i.e. the reduction would stall until its prefetch has landed.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
 
     // One barrier per tile.  Every wavefront dilates and compacts the tile's mask for itself (the
     // first one writes the output mask); the partial sums of tile i and the staged halo of tile
     // i + 1 become visible at the same barrier, behind which the finishing wavefronts store.
     int it = 0;
-    for (int tile = blockIdx.x; tile < q.tiles; tile += gridDim.x, ++it) {
+    for (int tile = blockIdx.x; tile < q.tiles; tile += gridDim.x, ++it, pos = nxt, nxt = advance(nxt)) {
         const int cur = it & 1;
-        const int b = tile / tiles_per_map, tr = tile - b * tiles_per_map;
-        const int ty0 = (tr / q.ltx) * TILE, tx0 = (tr % q.ltx) * TILE;
+        const int b = pos.b;
+        const int ty0 = pos.ty * TILE, tx0 = pos.tx * TILE;
+        // The next tile's mask words and rows travel while this tile is contracted.  Requested and
+        // staged without a condition (behind the last tile: this tile once more, into the buffer
+        // nobody reads): with the two under separate tests the compiler sees a path on which the
+        // requests are never consumed and waits for ALL memory traffic -- the previous tile's
+        // stores included -- at the head of every iteration.
         const bool has_next = tile + (int)gridDim.x < q.tiles;
-        if (has_next) request(tile + gridDim.x);  // travels while this tile is contracted
+        request(has_next ? nxt : pos);
         const unsigned char *halo = s_dyn + cur * halo_bytes;
         int n;
         {
@@ -194,6 +258,7 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
                 loc[nt] = slot < n ? s_wlist[wv][slot] : 0;
                 hbase[nt] = ((loc[nt] >> 3) * p.sh * hal_w + (loc[nt] & 7) * p.sw) * row + kq * 16;
             }
+            // (the tiles in use start from the first step's product; the others stay zero)
 #pragma unroll
             for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -219,7 +284,8 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
 #pragma unroll
                     for (int nt = 0; nt < NTA; ++nt)
 #pragma unroll
-                        for (int r = 0; r < R; ++r) acc[r][nt] = Elem16<E>::mfma(a[i][r], x[i & 1][nt], acc[r][nt]);
+                        for (int r = 0; r < R; ++r)
+                            acc[r][nt] = Elem16<E>::mfma(a[i][r], x[i & 1][nt], i == 0 ? float4_t{0.f, 0.f, 0.f, 0.f} : acc[r][nt]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             };
@@ -229,48 +295,52 @@ conv_res_mfma_kernel(ConvP p, ResP q, const E *__restrict__ in, const E *__restr
                 case 3: reduce(std::integral_constant<int, 3>{}); break;
                 default: reduce(std::integral_constant<int, 4>{}); break;
             }
-            if (KS > 1 && kz > 0) {
-                float4_t *s_part = reinterpret_cast<float4_t *>(s_part0 + cur * PART_BYTES);
+            if (KS > 1) {  // the tiles other slices finish: tile t of this wavefront in slot t (- TPW behind its own)
+                float4_t *s_part = reinterpret_cast<float4_t *>(s_part0 + cur * PART_BYTES) + wv * (KS - 1) * TPW * WAVE;
 #pragma unroll
-                for (int r = 0; r < R; ++r)
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
-                        s_part[((((kz - 1) * ncw + cw) * R + r) * NT + nt) * WAVE + lane] = acc[r][nt];
+                for (int t = 0; t < R * NT; ++t) {
+                    if (t / TPW == kz) continue;  // uniform
+                    s_part[(t < kz * TPW ? t : t - TPW) * WAVE + lane] = acc[t / NT][t % NT];
+                }
             }
         }
-        if (has_next) stage(cur ^ 1);
+        stage(cur ^ 1);
         __syncthreads();
-        if (n == 0 || kz > 0) continue;
-        if (KS > 1) {
-            const float4_t *s_part = reinterpret_cast<const float4_t *>(s_part0 + cur * PART_BYTES);
-#pragma unroll
-            for (int s = 1; s < KS; ++s)  // ascending slice order
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
-                        acc[r][nt] += s_part[((((s - 1) * ncw + cw) * R + r) * NT + nt) * WAVE + lane];
-        }
+        if (n == 0) continue;
+        // The slices of a channel group share the finishing of its R * NT tiles: slice kz takes tiles
+        // [kz * TPW, (kz + 1) * TPW), t = channel tile * NT + pixel tile, and adds the slices' partial
+        // sums in ascending slice order (its own from registers).
+        const float4_t *s_part = reinterpret_cast<const float4_t *>(s_part0 + cur * PART_BYTES);
         E *otile = out + (((size_t)b * p.Ho + ty0) * p.Wo + tx0) * p.Co;  // the tile's first output pixel
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
+        for (int t = 0; t < R * NT; ++t) {
+            if (KS > 1 && t / TPW != kz) continue;  // uniform
+            const int r = t / NT, nt = t % NT;
+            float4_t sum = acc[r][nt];
+            if (KS > 1) {
+#pragma unroll
+                for (int z = 0; z < KS; ++z) {
+                    // slice z's copy of tile t: in its wavefront's block, slot t (- TPW behind its own tiles)
+                    float4_t term = acc[r][nt];
+                    if (z != kz)  // uniform
+                        term = s_part[(((z * ncw + cw) * (KS - 1) * TPW) + (t < z * TPW ? t : t - TPW)) * WAVE + lane];
+                    sum = z == 0 ? term : sum + term;
+                }
+            }
             const int ct = (cb * ncw + cw) * R + r;
             if (ct >= co_tiles) continue;
             const int co = ct * 16 + kq * 4;  // lane holds channels co .. co + 3 of pixel (nt, l16)
+            if (nt * 16 + l16 >= n) continue;
+            E *o = otile + (unsigned)(((loc[nt] >> 3) * p.Wo + (loc[nt] & 7)) * p.Co + co);
+            E4 v;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                if (nt * 16 + l16 >= n) continue;
-                E *o = otile + (unsigned)(((loc[nt] >> 3) * p.Wo + (loc[nt] & 7)) * p.Co + co);
-                E4 v;
+            for (int i = 0; i < 4; ++i) v[i] = E(sum[i] + float(bv[r][i]));
+            if (co + 3 < p.Co && (p.Co & 3) == 0) {
+                *reinterpret_cast<E4 *>(o) = v;
+            } else {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v[i] = E(acc[r][nt][i] + float(bv[r][i]));
-                if (co + 3 < p.Co && (p.Co & 3) == 0) {
-                    *reinterpret_cast<E4 *>(o) = v;
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        if (co + i < p.Co) o[i] = v[i];
-                }
+                for (int i = 0; i < 4; ++i)
+                    if (co + i < p.Co) o[i] = v[i];
             }
         }
     }
