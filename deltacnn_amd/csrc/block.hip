@@ -408,8 +408,15 @@ block_eager_kernel(BlockP p) {
     const int pc = min(po, P - 1);
     const int c = gl * N;
     const int cc = min(c, p.Ch - N);
-    half8_t x[9], w[9], qa, tra;
-    {
+    // (Requests are made only by lanes and wavefronts that will use what they ask for -- the pixel
+    // slots of this workgroup that hold a pixel, the wavefronts that own a projection or expansion
+    // tile, the reduction steps that exist: a compute unit issues 64 bytes of requests per clock,
+    // and the rows, filters and fragments of a workgroup are 60-250 KB of them.)
+    const half8_t zero8 = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    half8_t x[9], w[9], qa = zero8, tra = zero8;
+#pragma unroll
+    for (int t = 0; t < 9; ++t) x[t] = w[t] = zero8;
+    if (po < P && c < p.Ch) {
         const int b = pc / (p.Ho * p.Wo);
         const int r = pc - b * p.Ho * p.Wo;
         const int oy = r / p.Wo, ox = r - oy * p.Wo;
@@ -430,20 +437,23 @@ block_eager_kernel(BlockP p) {
     const size_t pxl = (size_t)min(p0 + l16, P - 1);
     half8_t afr[KPS_E];
 #pragma unroll
-    for (int s = 0; s < KPS_E; ++s)
-        afr[s] = *reinterpret_cast<const half8_t *>(
-            p.wpj + ((size_t)ct_b * p.kp_steps + min(s, p.kp_steps - 1)) * 512 + lane * 8);
+    for (int s = 0; s < KPS_E; ++s) {
+        afr[s] = zero8;
+        if (wave < p.cp_tiles && s < p.kp_steps)  // uniform
+            afr[s] = *reinterpret_cast<const half8_t *>(p.wpj + ((size_t)ct_b * p.kp_steps + s) * 512 + lane * 8);
+    }
     const int co_b = min(ct_b * 16 + kq * 4, p.Cp - 4);
     half4_t rv = half4_t{0, 0, 0, 0};
-    if (p.res != nullptr) rv = *reinterpret_cast<const half4_t *>(p.res + pxl * p.Cp + co_b);
+    if (p.res != nullptr && wave < p.cp_tiles) rv = *reinterpret_cast<const half4_t *>(p.res + pxl * p.Cp + co_b);
     // stage C: filter fragments (one step) and cached state of this wavefront's tiles
     half8_t efr[CTW_E];
     half4_t qc[CTW_E], trc[CTW_E];
     if (p.Ce > 0) {
 #pragma unroll
         for (int j = 0; j < CTW_E; ++j) {
-            const int ct = min(wave + j * NW, p.ce_tiles - 1);
-            efr[j] = *reinterpret_cast<const half8_t *>(p.wex + (size_t)ct * 512 + lane * 8);
+            efr[j] = zero8;
+            if (wave + j * NW < p.ce_tiles)  // uniform
+                efr[j] = *reinterpret_cast<const half8_t *>(p.wex + (size_t)(wave + j * NW) * 512 + lane * 8);
         }
     }
     // all of the above is in flight before anything is waited for
@@ -483,7 +493,9 @@ block_eager_kernel(BlockP p) {
     if (p.Ce > 0) {
 #pragma unroll
         for (int j = 0; j < CTW_E; ++j) {
-            const int ct = min(wave + j * NW, p.ce_tiles - 1);
+            qc[j] = trc[j] = half4_t{0, 0, 0, 0};
+            const int ct = wave + j * NW;
+            if (ct >= p.ce_tiles) continue;  // uniform
             const int co = min(ct * 16 + kq * 4, p.Ce - 4);
             qc[j] = *reinterpret_cast<const half4_t *>(p.prev_c + pxl * p.Ce + co);
             trc[j] = *reinterpret_cast<const half4_t *>(p.trunc_c + pxl * p.Ce + co);
