@@ -228,26 +228,48 @@ def streams_bench(delta, dense, batch=8, steps=64, warmup=16, density=0.10, with
     return out
 
 
-def trace_kernels(delta, frames):
+def streams_profile(delta, batch, density, isolated=True):
+    """For profiling runs (`--only-streams N`): the graph-replayed step of N streams as a batch, and
+    beside it the sum of the same step's library calls each replayed on its own -- the two figures
+    whose difference is what a kernel loses by running behind another kernel's output."""
+    import torch
+    from deltacnn_amd.video import controlled_density_video
+    out = streams_bench(delta, None, batch=batch, steps=64, warmup=16, density=density, with_dense=False)
+    if not isolated:
+        return out
+    clip = gpu_frames(controlled_density_video(frames=(batch - 1) * STREAM_STRIDE + 5, density=density))
+    steps = torch.cat([clip[torch.arange(batch) * STREAM_STRIDE + i] for i in range(4)]).contiguous(
+        memory_format=torch.channels_last)
+    agg, rows = trace_kernels(delta, steps, batch=batch)
+    delta.reset_layers()
+    out["library_launches_per_step"] = len(rows)
+    out["isolated_replays_sum_ms"] = round(sum(r["ms"] for r in rows), 4)
+    out["kernels_isolated"] = {k: {"launches_per_step": a["launches"], "us_per_launch": round(a["us_per_launch"], 3)}
+                               for k, a in sorted(agg.items(), key=lambda kv: -kv[1]["ms"])}
+    return out
+
+
+def trace_kernels(delta, frames, batch=1):
     """Device time per call and algorithmic bytes / flops of every library call of one delta
-    frame.  The calls are recorded during an eager pass; each is then timed on the device by
-    replaying it back to back from a HIP graph on the masks of that frame (see
-    Tracer.replay_times), free of the host-side event overhead that dwarfs a few-microsecond
-    kernel."""
+    frame (of `batch` streams: frames[i * batch:(i + 1) * batch] is step i).  The calls are recorded
+    during an eager pass; each is then timed on the device by replaying it back to back from a HIP
+    graph on the masks of that frame (see Tracer.replay_times), free of the host-side event overhead
+    that dwarfs a few-microsecond kernel."""
     import torch
     from deltacnn_amd import hip_kernels as hk
     from deltacnn_amd.trace import Tracer, summarise
     delta.reset_layers()
+    step = lambda i: frames[i * batch:(i + 1) * batch]
     with torch.no_grad():
         for i in range(3):
-            delta(frames[i:i + 1])
+            delta(step(i))
         tr = Tracer()
         hk.set_tracer(tr)
         try:
-            delta(frames[3:4])
+            delta(step(3))
         finally:
             hk.set_tracer(None)
-        times = tr.replay_times(alt_inputs=[frames[2:3].data_ptr(), frames[3:4].data_ptr()])
+        times = tr.replay_times(alt_inputs=[step(2).data_ptr(), step(3).data_ptr()])
         for rec, us in zip(tr.records, times):
             rec["ms"] = us * 1e-3
         rows = tr.finish()
@@ -512,6 +534,11 @@ def main():
                          "reference that hardware traffic counters of a profiling run are scaled by")
     ap.add_argument("--network", choices=["mobilenetv2", "hrnet", "dla34"], default="mobilenetv2",
                     help="hrnet / dla34: time that configuration instead and print a short JSON line")
+    ap.add_argument("--only-streams", type=int, default=0, metavar="N",
+                    help="time the step of N video streams as one batch only and print a short JSON line with the "
+                         "sum of the step's library calls replayed one by one beside it (for profiling runs; with "
+                         "--no-sweep the step alone, so that a kernel trace of the run holds no other launches of "
+                         "the library than the eager frames and the step)")
     ap.add_argument("--only-micro", action="store_true",
                     help="run the single-layer and scaled-shape sections only (for profiling runs)")
     ap.add_argument("--cpu-frames", type=int, default=200,
@@ -545,6 +572,9 @@ def main():
     dense, delta, state = build_models(stats_video.to("cuda").contiguous(memory_format=torch.channels_last))
     frames = gpu_frames(video)
 
+    if args.only_streams > 0:
+        print(json.dumps(streams_profile(delta, args.only_streams, args.density, isolated=not args.no_sweep)), flush=True)
+        return
     sec = run_delta(delta, frames, args.warmup, args.steps, args.mode)
     fps = 1.0 / sec
     log(f"delta path: {fps:.1f} frames/s ({sec * 1e3:.3f} ms/frame, mode={args.mode})")
