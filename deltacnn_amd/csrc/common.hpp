@@ -98,6 +98,18 @@ __device__ __forceinline__ float vec_absmax(const Vec<T, N> &x) {
     return m;
 }
 
+// Is any bit of a 16-byte vector set?
+template <typename T, int N>
+__device__ __forceinline__ bool any_bits(const Vec<T, N> &x) {
+    static_assert(sizeof(Vec<T, N>) == 16, "16-byte vectors only");
+    union {
+        Vec<T, N> v;
+        uint32_t u[4];
+    } c;
+    c.v = x;
+    return ((c.u[0] | c.u[1]) | (c.u[2] | c.u[3])) != 0u;
+}
+
 // A 16-byte vector kept if `on`, else all-zero bits: four 32-bit selects whatever the element
 // type (a per-element select on halves costs twice as many instructions).
 template <typename T, int N>

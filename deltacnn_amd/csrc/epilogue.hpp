@@ -99,7 +99,8 @@ __device__ __forceinline__ bool act_trunc_pixel(Vec<T, Vec16<T>::N> (&dl)[ITERS]
                     for (int j = 0; j < N; ++j) z.v[j] = T(0);
                     vstore<T, N>(prev + off, s[it]);
                     vstore<T, N>(delta + off, dl[it]);
-                    vstore<T, N>(trunc + off, z);
+                    // (a remainder that is zero already -- the pixel was kept last time too -- is not stored again)
+                    if (any_bits(tr[it])) vstore<T, N>(trunc + off, z);
                 } else {
                     vstore<T, N>(trunc + off, t[it]);
                 }
