@@ -26,6 +26,21 @@
 
 namespace dc {
 namespace {
+// Is any bit of a 16-byte / 8-byte vector set?  (A truncated remainder that is zero already need
+// not be stored as zero again.)
+template <typename V>
+__device__ __forceinline__ bool bits_set16(const V &x) {
+    static_assert(sizeof(V) == 16, "16-byte vectors");
+    const u32x4_t u = __builtin_bit_cast(u32x4_t, x);
+    return ((u[0] | u[1]) | (u[2] | u[3])) != 0u;
+}
+template <typename V>
+__device__ __forceinline__ bool bits_set8(const V &x) {
+    static_assert(sizeof(V) == 8, "8-byte vectors");
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    const u32x2_t u = __builtin_bit_cast(u32x2_t, x);
+    return (u[0] | u[1]) != 0u;
+}
 
 struct PwP {
     int P, Ci, Co, ci_p, co_tiles;
@@ -481,7 +496,7 @@ __device__ __forceinline__ void pw_epilogue_store(const typename Elem16<E>::v4 (
         if (keep) {
             *reinterpret_cast<E4 *>(prev + off) = s;
             *reinterpret_cast<E4 *>(out + off) = d;
-            *reinterpret_cast<E4 *>(trunc + off) = zero4<E>();
+            if (bits_set8(tr[j])) *reinterpret_cast<E4 *>(trunc + off) = zero4<E>();  // else zero already
         } else {
             *reinterpret_cast<E4 *>(trunc + off) = t;
         }
@@ -754,7 +769,7 @@ pw_rows_act_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp,
         if (keep) {
             *reinterpret_cast<E8 *>(prev + poff[i]) = sv;
             *reinterpret_cast<E8 *>(out + poff[i]) = dv;
-            *reinterpret_cast<E8 *>(trunc + poff[i]) = z;
+            if (bits_set16(trow[i])) *reinterpret_cast<E8 *>(trunc + poff[i]) = z;  // else zero already
         } else {
             *reinterpret_cast<E8 *>(trunc + poff[i]) = tv;
         }
@@ -922,7 +937,7 @@ pw_gather_kernel(PwP p, const E *__restrict__ in, const E *__restrict__ wp, cons
                 if (keep) {
                     *reinterpret_cast<E8 *>(prev + off) = sv;
                     *reinterpret_cast<E8 *>(out + off) = dv;
-                    *reinterpret_cast<E8 *>(trunc + off) = z;
+                    if (bits_set16(trow[i])) *reinterpret_cast<E8 *>(trunc + off) = z;  // else zero already
                 } else {
                     *reinterpret_cast<E8 *>(trunc + off) = tv;
                 }
