@@ -1678,7 +1678,7 @@ conv_patch_body(const ConvP &p, const E *__restrict__ in, const E *__restrict__ 
                 if (keep) {
                     *reinterpret_cast<E4 *>(ep.prev + off) = sm[r];
                     *reinterpret_cast<E4 *>(out + off) = d[r];
-                    *reinterpret_cast<E4 *>(ep.trunc + off) = zero4<E>();
+                    if (bits_set8(etr[r])) *reinterpret_cast<E4 *>(ep.trunc + off) = zero4<E>();  // else zero already
                 } else {
                     *reinterpret_cast<E4 *>(ep.trunc + off) = t[r];
                 }
@@ -2001,7 +2001,7 @@ conv_stem_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ w
         if (keep) {
             *reinterpret_cast<E4 *>((E *)epi.prev + off) = sm[r];
             *reinterpret_cast<E4 *>(out + off) = d[r];
-            *reinterpret_cast<E4 *>((E *)epi.trunc + off) = zero4<E>();
+            if (bits_set8(tr[r])) *reinterpret_cast<E4 *>((E *)epi.trunc + off) = zero4<E>();  // else zero already
         } else {
             *reinterpret_cast<E4 *>((E *)epi.trunc + off) = t[r];
         }
@@ -2192,7 +2192,7 @@ conv_thin_mfma_kernel(ConvP p, const E *__restrict__ in, const E *__restrict__ w
         if (keep) {
             *reinterpret_cast<E8 *>((E *)epi.prev + poff[i]) = sv;
             *reinterpret_cast<E8 *>(out + poff[i]) = dv;
-            *reinterpret_cast<E8 *>((E *)epi.trunc + poff[i]) = z;
+            if (bits_set16(trow[i])) *reinterpret_cast<E8 *>((E *)epi.trunc + poff[i]) = z;  // else zero already
         } else {
             *reinterpret_cast<E8 *>((E *)epi.trunc + poff[i]) = tv;
         }

@@ -26,21 +26,6 @@
 
 namespace dc {
 namespace {
-// Is any bit of a 16-byte / 8-byte vector set?  (A truncated remainder that is zero already need
-// not be stored as zero again.)
-template <typename V>
-__device__ __forceinline__ bool bits_set16(const V &x) {
-    static_assert(sizeof(V) == 16, "16-byte vectors");
-    const u32x4_t u = __builtin_bit_cast(u32x4_t, x);
-    return ((u[0] | u[1]) | (u[2] | u[3])) != 0u;
-}
-template <typename V>
-__device__ __forceinline__ bool bits_set8(const V &x) {
-    static_assert(sizeof(V) == 8, "8-byte vectors");
-    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-    const u32x2_t u = __builtin_bit_cast(u32x2_t, x);
-    return (u[0] | u[1]) != 0u;
-}
 
 struct PwP {
     int P, Ci, Co, ci_p, co_tiles;
