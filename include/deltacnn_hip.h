@@ -102,8 +102,11 @@ int dc_conv(const dc_geometry *g, const void *input, const void *filter,
 
 /* Conv + activation/truncation in one call: dc_conv followed by dc_activate_truncate on the
  * conv output.  Depthwise, few-input-channel, mid-size pointwise and small KxK shapes of up
- * to 32 output channels run as ONE launch
- * (the epilogue works on the accumulators, the conv output never travels through memory);
+ * to 32 output channels, K x K layers with 8 / 16 input channels on large maps, and larger K x K
+ * layers of up to 64 output channels on at most 256 output tiles of 8 x 8 run as ONE launch
+ * (the epilogue works on the accumulators, the conv output never travels through memory; `out`
+ * then holds the activated difference of the pixels whose out_mask word is set and is undefined
+ * elsewhere, as after the two calls);
  * every other shape runs the two kernels back to back inside the call.  No counterpart in
  * the reference (it launches the two kernels separately, sparse_layers.py:636-638); results
  * are identical to the two-call sequence bit for bit. */
