@@ -116,15 +116,16 @@ struct OpenActP {
 // EAGER (3x3 only, small maps): the nine input rows, the filter and the cached state are
 // requested before the mask words have arrived -- their addresses depend on coordinates only --
 // so the whole kernel is one memory round trip; what is loaded for inactive pixels is dropped.
-// FIN (EAGER, stride 1, padding 1): the producing layer's activation / truncation is finished
-// here, which saves that layer's activation launch.  A window pixel counts as updated only if
-// the producer's keep decision holds for it -- any |D| above the producer's threshold over all
-// channels, which this lane group sees since it reads the pixel's whole row anyway -- and the
-// group commits the producer's cached state of its CENTRE pixel (every pixel is the centre of
-// exactly one group): kept: prev += T, truncated = 0; dropped: truncated = T, which it holds
-// already.  Neighbouring groups read D and the update mask only, never that state, so nothing
-// races.
-template <typename T, int ITERS, int ACT, bool K3, bool EAGER, bool FIN = false>
+// FIN (EAGER, padding 1; 1: stride 1, 2: stride 2): the producing layer's activation / truncation
+// is finished here, which saves that layer's activation launch.  A window pixel counts as updated
+// only if the producer's keep decision holds for it -- any |D| above the producer's threshold over
+// all channels, which this lane group sees since it reads the pixel's whole row anyway -- and the
+// group commits the producer's cached state of the input pixels it OWNS: with stride 1 its centre
+// pixel, with stride 2 the 2 x 2 block (2 oy + {0, 1}, 2 ox + {0, 1}), taps (1, 1) .. (2, 2) of its
+// window -- every input pixel is owned by exactly one group.  Kept: prev += T, truncated = 0;
+// dropped: truncated = T, which it holds already.  Neighbouring groups read D and the update mask
+// only, never that state, so nothing races.
+template <typename T, int ITERS, int ACT, bool K3, bool EAGER, int FIN = 0>
 __global__ void __launch_bounds__(256)
 conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
                const T *__restrict__ bias, T *__restrict__ out, const int32_t *__restrict__ mask,
@@ -173,17 +174,24 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
             }
         }
     }
-    // FIN: T and the accumulated value of the centre pixel (stride 1, padding 1: input pixel
-    // (oy, ox)), requested with everything else
-    Vec<T, N> ft[FIN ? ITERS : 1], fq[FIN ? ITERS : 1];
-    const size_t centre = ((size_t)b * p.Hi + oy) * p.Wi + ox;
+    // FIN: T and the accumulated value of the owned input pixels (padding 1: tap (1 + dy, 1 + dx) of
+    // the window is input pixel (oy * stride + dy, ox * stride + dx)), requested with everything else
+    constexpr int NOWN = FIN == 2 ? 4 : 1;
+    Vec<T, N> ft[FIN ? NOWN : 1][FIN ? ITERS : 1], fq[FIN ? NOWN : 1][FIN ? ITERS : 1];
+    size_t own[NOWN];
+#pragma unroll
+    for (int o = 0; o < NOWN; ++o)  // (past the map's edge: the edge pixel again; its tap is never set)
+        own[o] = ((size_t)b * p.Hi + min(oy * (FIN == 2 ? 2 : 1) + (o >> 1), p.Hi - 1)) * p.Wi +
+                 min(ox * (FIN == 2 ? 2 : 1) + (o & 1), p.Wi - 1);
     if (FIN) {
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            const int c = min((it * G + gl) * N, C - N);
-            ft[it] = vload<T, N>((const T *)fin.trunc + centre * C + c);
-            fq[it] = vload<T, N>((const T *)fin.prev + centre * C + c);
-        }
+        for (int o = 0; o < NOWN; ++o)
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int c = min((it * G + gl) * N, C - N);
+                ft[o][it] = vload<T, N>((const T *)fin.trunc + own[o] * C + c);
+                fq[o][it] = vload<T, N>((const T *)fin.prev + own[o] * C + c);
+            }
     }
 
     uint64_t taps = 0;
@@ -202,10 +210,12 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
         // (the centre pixel's state was requested with everything else and has arrived with the
         // mask words: keep the compiler from moving those requests down to the commit below)
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            pin_vec(ft[it]);
-            pin_vec(fq[it]);
-        }
+        for (int o = 0; o < NOWN; ++o)
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                pin_vec(ft[o][it]);
+                pin_vec(fq[o][it]);
+            }
         // the producer's keep decision for the nine window pixels: this lane's share first (what
         // was loaded for a pixel without update is dropped), then the group's, straight-line
         const float fthr = float(T(fin.thr));
@@ -233,21 +243,25 @@ conv_dw_kernel(ConvP p, const T *__restrict__ in, const T *__restrict__ filter,
             kept = 0;
             for (int w = 0; w < (int)(blockDim.x / WAVE); ++w) kept |= s_kept[w];
         }
-        const bool centre_updated = (taps >> 4) & 1ull;
+        // (a tap that was not updated is clear in `taps`, one that was not kept in `kept`)
         taps &= kept;
-        if (valid && centre_updated && ((taps >> 4) & 1ull)) {  // kept
 #pragma unroll
-            for (int it = 0; it < ITERS; ++it) {
-                const int c = (it * G + gl) * N;
-                if (c < C) {
-                    Vec<T, N> z, sum;
+        for (int o = 0; o < NOWN; ++o) {
+            const int tap = (1 + (o >> 1)) * 3 + 1 + (o & 1);  // 4; stride 2: 4, 5, 7, 8
+            if (valid && ((taps >> tap) & 1ull)) {  // updated and kept
 #pragma unroll
-                    for (int j = 0; j < N; ++j) {
-                        z.v[j] = T(0);
-                        sum.v[j] = ft[it].v[j] + fq[it].v[j];
+                for (int it = 0; it < ITERS; ++it) {
+                    const int c = (it * G + gl) * N;
+                    if (c < C) {
+                        Vec<T, N> z, sum;
+#pragma unroll
+                        for (int j = 0; j < N; ++j) {
+                            z.v[j] = T(0);
+                            sum.v[j] = ft[o][it].v[j] + fq[o][it].v[j];
+                        }
+                        vstore<T, N>((T *)fin.prev + own[o] * C + c, sum);
+                        vstore<T, N>((T *)fin.trunc + own[o] * C + c, z);
                     }
-                    vstore<T, N>((T *)fin.prev + centre * C + c, sum);
-                    vstore<T, N>((T *)fin.trunc + centre * C + c, z);
                 }
             }
         }
@@ -2409,7 +2423,7 @@ bool try_depthwise(const dc_geometry &g, const ConvP &p, const T *in, const T *f
 }
 
 // The depthwise layer that finishes its producer's open activation (conv_dw_kernel<FIN>): 3x3,
-// stride 1, padding 1, on maps small enough for the eager per-pixel form (where launches, not
+// stride 1 or 2, padding 1, on maps small enough for the eager per-pixel form (where launches, not
 // bytes, are the cost).  Returns false if the shape does not qualify; nothing is launched then.
 template <typename T>
 bool try_depthwise_closing(const dc_geometry &g, const ConvP &p, const T *in, const T *filter, T *out,
@@ -2418,9 +2432,12 @@ bool try_depthwise_closing(const dc_geometry &g, const ConvP &p, const T *in, co
     constexpr int N = Vec16<T>::N;
     const auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     if (g.groups != g.in_c || g.groups != g.out_c || g.groups == 1) return false;
-    if (g.kernel_h != 3 || g.kernel_w != 3 || g.stride_h != 1 || g.stride_w != 1 || g.dilation_h != 1 ||
-        g.dilation_w != 1 || g.pad_top != 1 || g.pad_left != 1 || g.pad_bottom != 1 || g.pad_right != 1)
+    if (g.kernel_h != 3 || g.kernel_w != 3 || g.stride_h != g.stride_w || (g.stride_h != 1 && g.stride_h != 2) ||
+        g.dilation_h != 1 || g.dilation_w != 1 || g.pad_top != 1 || g.pad_left != 1 || g.pad_bottom != 1 ||
+        g.pad_right != 1)
         return false;
+    // (stride 2: every input pixel lies in the 2 x 2 block of exactly one output pixel)
+    if (g.stride_h == 2 && (2 * g.out_h < g.in_h || 2 * g.out_w < g.in_w)) return false;
     if (g.in_c % N != 0 || g.in_c / N > WAVE * 4) return false;
     if (epi == nullptr || epi->trunc == nullptr || epi->mode < 0) return false;
     const int64_t P_out = (int64_t)g.batch * g.out_h * g.out_w;
@@ -2429,7 +2446,9 @@ bool try_depthwise_closing(const dc_geometry &g, const ConvP &p, const T *in, co
     const int wide = epi->mode == DC_TRUNC_MAX ? wide_group(nvec, P_out) : 0;
     const int G = wide ? wide : pick_group(nvec, P_out, 4);
     const int iters = ceil_div(nvec, G);
-    if (iters > 2 || P_out * g.in_c * (int64_t)sizeof(T) > (2 << 20)) return false;  // the eager form only
+    // the eager form only (its input at most 2 MB); stride 2: one vector per lane, the state of four pixels
+    if (iters > (g.stride_h == 2 ? 1 : 2) || (int64_t)g.batch * g.in_h * g.in_w * g.in_c * (int64_t)sizeof(T) > (2 << 20))
+        return false;
     if (!launch) return true;
     if (!al(in) || !al(filter) || !al(out) || !al(epi->prev) || !al(epi->trunc) || !al(open.prev) || !al(open.trunc))
         return false;
@@ -2442,8 +2461,9 @@ bool try_depthwise_closing(const dc_geometry &g, const ConvP &p, const T *in, co
     const int lg = log2i(G);
 #define DC_DWF(A)                                                                                                      \
     do {                                                                                                               \
-        if (iters == 1) conv_dw_kernel<T, 1, A, true, true, true><<<grid, block, 0, s>>>(p, in, filter, nullptr, out, mask, out_mask, e, lg, f); \
-        else conv_dw_kernel<T, 2, A, true, true, true><<<grid, block, 0, s>>>(p, in, filter, nullptr, out, mask, out_mask, e, lg, f); \
+        if (g.stride_h == 2) conv_dw_kernel<T, 1, A, true, true, 2><<<grid, block, 0, s>>>(p, in, filter, nullptr, out, mask, out_mask, e, lg, f); \
+        else if (iters == 1) conv_dw_kernel<T, 1, A, true, true, 1><<<grid, block, 0, s>>>(p, in, filter, nullptr, out, mask, out_mask, e, lg, f); \
+        else conv_dw_kernel<T, 2, A, true, true, 1><<<grid, block, 0, s>>>(p, in, filter, nullptr, out, mask, out_mask, e, lg, f); \
     } while (0)
     switch (act) {
         case DC_ACT_RELU: DC_DWF(DC_ACT_RELU); break;

@@ -519,9 +519,10 @@ int dc_expand_depthwise(const dc_geometry *g, const dc_expand_dw_args *args, int
                                         "output channels in multiples of 8 and ReLU or ReLU6");
     dc::ActEpilogue dw_epi{a.dw_prev_out, a.dw_truncated, a.dw_threshold, a.dw_activation, a.dw_truncation_mode};
     if (!dc::depthwise_closing_eligible(*g, &dw_epi, dtype))
-        return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: needs a depthwise 3x3 convolution with stride 1 and "
+        return fail(DC_ERR_UNSUPPORTED, "dc_expand_depthwise: needs a depthwise 3x3 convolution with stride 1 or 2 and "
                                         "padding 1 on a map small enough for the per-pixel kernel (input of at "
-                                        "most 2 MB, at most two 16-byte vectors per lane) with a truncating activation");
+                                        "most 2 MB, at most two 16-byte vectors per lane, one with stride 2) with a "
+                                        "truncating activation");
     if (!opened) {
         DC_REQUIRE_PTR("dc_expand_depthwise", a.input);
         DC_REQUIRE_PTR("dc_expand_depthwise", a.mask);
@@ -606,7 +607,7 @@ int dc_project_expand(const dc_geometry *g, const dc_project_expand_args *args, 
         dc::ActEpilogue probe{a.expand_prev_out, a.expand_truncated, 0.f, a.dw_activation, a.dw_truncation_mode};
         if (!dc::depthwise_closing_eligible(gd, &probe, dtype))
             return fail(DC_ERR_UNSUPPORTED, "dc_project_expand: the depthwise layer behind the expansion cannot finish "
-                                            "its activation (needs 3x3, stride 1, padding 1 on a small map)");
+                                            "its activation (needs 3x3, stride 1 or 2, padding 1 on a small map)");
     }
     {
         // Several workgroups per pixel tile read every input of this call and repeat the projection

@@ -263,7 +263,7 @@ def sparse_expand_depthwise(x, mask, expand_packed, expand_prev_out, expand_trun
                             dw_truncated, dw_threshold, dw_activation, dw_truncation_mode, out, out_mask,
                             opened: bool = False):
     """A 1x1 expansion with activation / maximum-norm truncation followed by a depthwise 3x3
-    (stride 1, padding 1) with activation / truncation as TWO launches instead of three
+    (stride 1 or 2, padding 1) with activation / truncation as TWO launches instead of three
     (``dc_expand_depthwise``): the expansion leaves its keep decision to the depthwise kernel,
     which reads whole pixel rows anyway and commits the expansion's cached state.  Layer states
     and the depthwise output are identical, bit for bit, to the separate calls.  Returns ``False``

@@ -712,8 +712,8 @@ def concat_conv(conv, inputs):
 
 
 def expand_depthwise(expand, depthwise, input, opened=None):
-    """``depthwise(expand(input))`` for a 1x1 expansion DCConv2d and a 3x3 stride-1 depthwise
-    DCConv2d, both with a truncating activation, as TWO launches instead of three on frames
+    """``depthwise(expand(input))`` for a 1x1 expansion DCConv2d and a 3x3 depthwise DCConv2d
+    (stride 1 or 2), both with a truncating activation, as TWO launches instead of three on frames
     after the first: the expansion's convolution leaves its keep decision to the depthwise
     kernel (``dc_expand_depthwise``).  Returns the depthwise layer's ``(delta, mask)`` -- exactly
     what the separate layer calls return, all layer states included -- or ``None`` when the

@@ -201,7 +201,7 @@ typedef struct dc_expand_dw_args {
     int32_t expand_truncation_mode; /* DC_TRUNC_MAX */
     void *expand_out;               /* [P][C] the expansion's output delta, valid on the pixels it keeps */
     int32_t *expand_out_mask;       /* [P] receives the UPDATE mask of the expansion's convolution (= mask) */
-    /* B: depthwise 3x3, stride 1, padding 1 (geometry argument) + activation/truncation */
+    /* B: depthwise 3x3, stride 1 or 2, padding 1 (geometry argument) + activation/truncation */
     const void *dw_filter;          /* reference depthwise layout [3][3][C] */
     void *dw_prev_out;              /* [P][C], in place */
     void *dw_truncated;
@@ -213,12 +213,13 @@ typedef struct dc_expand_dw_args {
 } dc_expand_dw_args;
 
 /* A 1x1 expansion with activation / maximum-norm truncation followed by a depthwise 3x3
- * (stride 1, padding 1) with activation / truncation, as two launches instead of three: the
+ * (stride 1 or 2, padding 1) with activation / truncation, as two launches instead of three: the
  * expansion's convolution computes T = truncated + v, S = T + prev, D = act(S) - act(prev) for
  * every updated pixel, stores D and T, and leaves the keep decision -- any |D| of a pixel's
  * channels above the threshold, which no workgroup of that kernel can see -- to the depthwise
  * kernel, whose lane groups read whole pixel rows anyway: a window pixel counts only if the
- * decision holds for it, and every group commits the expansion's state of its centre pixel.
+ * decision holds for it, and every group commits the expansion's state of the input pixels it
+ * owns (stride 1: its centre pixel; stride 2: the 2 x 2 block at twice its output coordinates).
  * All layer states and the depthwise output are identical, bit for bit, to
  * dc_conv_act(expansion) followed by dc_conv_act(depthwise); of the expansion's own output only
  * the pixels it keeps are meaningful (as always), and expand_out_mask receives its convolution's

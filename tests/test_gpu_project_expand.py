@@ -10,14 +10,19 @@ from util import DEV, assert_masked_equal, cl, poison, rand_mask
 
 pytestmark = pytest.mark.gpu
 
-CASES = [  # hidden channels, block channels, next hidden channels, H, W, batch
+CASES = [  # hidden channels, block channels, next hidden channels, H, W, batch (, stride of the closing depthwise layer)
     (384, 64, 384, 14, 14, 1), (384, 96, 576, 14, 14, 1), (576, 96, 576, 14, 14, 1), (576, 96, 576, 10, 13, 2),
     (384, 64, 384, 20, 21, 1), (640, 32, 192, 9, 9, 1), (352, 64, 128, 7, 7, 3),
     (192, 64, 384, 14, 14, 1), (320, 96, 192, 7, 9, 2), (64, 32, 64, 12, 12, 1),  # projections without reduction slices
+    (576, 96, 576, 14, 14, 1, 2), (384, 64, 384, 15, 13, 2, 2), (192, 32, 192, 9, 9, 1, 2),  # closed by a stride-2 layer
 ]
 
 
-def _case(dtype, ch, cm, ce, H, W, B, density, seed, raw=False):
+def _stride(case):
+    return case[6] if len(case) > 6 else 1
+
+
+def _case(dtype, ch, cm, ce, H, W, B, density, seed, raw=False, stride=1):
     from deltacnn_amd.filter_conversion import convert_filter_out_channels_last, convert_half_filter
     g = torch.Generator().manual_seed(seed)
     mask = rand_mask(g, B, H, W, density)
@@ -34,7 +39,9 @@ def _case(dtype, ch, cm, ce, H, W, B, density, seed, raw=False):
         fp, fe, fd = convert_half_filter(wp), convert_half_filter(we), convert_half_filter(wd, pixel_wise=True)
     else:
         fp, fe, fd = (convert_filter_out_channels_last(w) for w in (wp, we, wd))
-    states = [torch.randn(B, ce, H, W, generator=g).to(dtype) * s for s in (1.0, 0.05, 1.0, 0.05)]
+    Ho, Wo = (H - 1) // stride + 1, (W - 1) // stride + 1
+    states = [torch.randn(B, ce, h, w, generator=g).to(dtype) * s
+              for (s, h, w) in ((1.0, H, W), (0.05, H, W), (1.0, Ho, Wo), (0.05, Ho, Wo))]
     if raw:
         return x, mask, r, rmask, fp.to(DEV), fe.to(DEV), fd.to(DEV), states, (wp, we, wd)
     return x, mask, r, rmask, fp.to(DEV), fe.to(DEV), fd.to(DEV), states
@@ -48,19 +55,20 @@ def _case(dtype, ch, cm, ce, H, W, B, density, seed, raw=False):
 def test_project_expand_equals_separate_calls(lib, dtype, case, density, residual, act):
     from deltacnn_amd import _lib
     from deltacnn_amd import hip_kernels as hk
-    ch, cm, ce, H, W, B = case
-    x, mask, r, rmask, fp, fe, fd, states = _case(dtype, ch, cm, ce, H, W, B, density, 2100 + ch + cm + ce)
+    ch, cm, ce, H, W, B = case[:6]
+    st = _stride(case)
+    x, mask, r, rmask, fp, fe, fd, states = _case(dtype, ch, cm, ce, H, W, B, density, 2100 + ch + cm + ce, stride=st)
     pkp, pke = hk.pack_filter(fp, ch, cm, 1), hk.pack_filter(fe, cm, ce, 1)
     dx, dm = cl(poison(x, mask)), cl(mask)
     dr, drm = cl(poison(r, rmask)), cl(rmask)
     gp = hk.conv_geometry((B, ch, H, W), (1, 1), cm, (1, 1), (0, 0), (1, 1), 1)
-    gd = hk.conv_geometry((B, ce, H, W), (3, 3), ce, (1, 1), (1, 1), (1, 1), ce)
+    gd = hk.conv_geometry((B, ce, H, W), (3, 3), ce, (st, st), (1, 1), (1, 1), ce)
     thr_e, thr_d = 0.9, 0.3
     nan = float("nan")
 
-    def fresh(c):
-        return (torch.full((B, c, H, W), nan, dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last),
-                torch.full((B, 1, H, W), -7, dtype=torch.int32, device=DEV))
+    def fresh(c, h=H, w=W):
+        return (torch.full((B, c, h, w), nan, dtype=dtype, device=DEV).contiguous(memory_format=torch.channels_last),
+                torch.full((B, 1, h, w), -7, dtype=torch.int32, device=DEV))
 
     # separate calls
     pe1, te1, pd1, td1 = (cl(t) for t in states)
@@ -73,13 +81,13 @@ def test_project_expand_equals_separate_calls(lib, dtype, case, density, residua
                                               packed_filter=pke)
     kept, reached = int(e_mask.sum()), int(ym1.sum())
     assert reached < 16 or 0 < kept < reached, (kept, reached)  # some kept, some truncated
-    d_out, d_mask = hk.sparse_conv_activation(e_out, fd, e_mask, None, pd1, td1, thr_d, 2, 0, (1, 1), (1, 1), (1, 1),
+    d_out, d_mask = hk.sparse_conv_activation(e_out, fd, e_mask, None, pd1, td1, thr_d, 2, 0, (st, st), (1, 1), (1, 1),
                                               ce, ce)
     # the pair launch + the closing depthwise launch
     pe2, te2, pd2, td2 = (cl(t) for t in states)
     y2, ym2 = fresh(cm)
     e2, em2 = fresh(ce)
-    out2, om2 = fresh(ce)
+    out2, om2 = fresh(ce, (H - 1) // st + 1, (W - 1) // st + 1)
     assert hk.sparse_project_expand(dx, dm, pkp, gp, dr if residual else None, drm if residual else None, y2, ym2, pke,
                                     pe2, te2, act, e2, em2, gd, 2, 0)
     assert _lib.load().dc_last_kernels().decode() == "pw_pair_kernel"
@@ -122,7 +130,7 @@ def test_project_expand_against_oracle_chain(lib, case, residual):
     from deltacnn_amd import hip_kernels as hk
     from oracle import delta_ops as ops
     dtype = torch.float16
-    ch, cm, ce, H, W, B = case
+    ch, cm, ce, H, W, B = case[:6]
     x, mask, r, rmask, fp, fe, fd, states, (wp, we, wd) = _case(dtype, ch, cm, ce, H, W, B, 0.4, 2300 + ch + cm + ce, raw=True)
     thr_e, thr_d, act = 0.9, 0.3, 2
     # oracle
@@ -168,11 +176,11 @@ def test_project_expand_against_oracle_chain(lib, case, residual):
 
 def test_project_expand_declines_what_it_cannot_do(lib):
     """Block channels outside multiples of 32 up to 96, projections of more than 20 reduction
-    steps, a depthwise layer that cannot finish the expansion (stride 2)
+    steps, a depthwise layer that cannot finish the expansion (stride 3)
     and fp32: False, nothing launched, nothing touched."""
     from deltacnn_amd import hip_kernels as hk
     dtype = torch.float16
-    for (ch, cm, ce, H, W, B, stride, dt) in [(384, 64, 384, 14, 14, 1, 2, dtype), (704, 64, 384, 14, 14, 1, 1, dtype),
+    for (ch, cm, ce, H, W, B, stride, dt) in [(384, 64, 384, 14, 14, 1, 3, dtype), (704, 64, 384, 14, 14, 1, 1, dtype),
                                               (384, 48, 288, 14, 14, 1, 1, dtype), (960, 160, 960, 7, 7, 1, 1, dtype),
                                               (384, 64, 384, 14, 14, 1, 1, torch.float32)]:
         x, mask, r, rmask, fp, fe, fd, states = _case(dtype, ch, cm, ce, H, W, B, 0.5, 2200 + ch)
