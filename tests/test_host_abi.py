@@ -291,8 +291,8 @@ def test_expand_depthwise_arguments_are_checked_before_any_launch(lib):
     assert call(g, args(expand_in_channels=20)) == -3                      # not a multiple of 8
     assert call(g, args(expand_truncation_mode=1)) == -3                   # norm truncation of the expansion
     assert call(g, args(dw_truncation_mode=-1)) == -3                      # a depthwise layer without truncation
-    assert call(_geom(in_h=14, in_w=14, out_h=7, out_w=7, in_c=384, out_c=384, groups=384, stride_h=2, stride_w=2),
-                args()) == -3                                              # strided
+    assert call(_geom(in_h=14, in_w=14, out_h=5, out_w=5, in_c=384, out_c=384, groups=384, stride_h=3, stride_w=3),
+                args()) == -3                                              # a stride beyond 2
     assert call(_geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=384, out_c=384, groups=1), args()) == -3  # not depthwise
     assert call(_geom(in_h=224, in_w=224, out_h=224, out_w=224, in_c=96, out_c=96, groups=96), args()) == -3  # too large
     assert lib.dc_expand_depthwise(None, ctypes.byref(args()), 1, None) == -4
@@ -335,7 +335,7 @@ def test_project_expand_arguments_are_checked_before_any_launch(lib):
     assert call(_geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=384, out_c=48, **one), args()) == -3   # 48 channels
     assert call(_geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=960, out_c=160, **one), args()) == -3  # too wide
     assert call(_geom(in_h=14, in_w=14, out_h=14, out_w=14, in_c=384, out_c=64), args()) == -3          # 3x3
-    strided = _geom(in_h=14, in_w=14, out_h=7, out_w=7, in_c=384, out_c=384, groups=384, stride_h=2, stride_w=2)
+    strided = _geom(in_h=14, in_w=14, out_h=5, out_w=5, in_c=384, out_c=384, groups=384, stride_h=3, stride_w=3)
     assert call(g, args(dw=strided)) == -3 and b"depthwise" in lib.dc_last_error()
     other = _geom(in_h=7, in_w=7, out_h=7, out_w=7, in_c=384, out_c=384, groups=384)
     assert call(g, args(dw=other)) == -2                                   # not on the expansion's output map
