@@ -84,7 +84,7 @@ def time_steps(step, warmup, steps):
     return (time.perf_counter() - t0) / steps
 
 
-UNROLL = 8  # frames per graph launch (processed one after the other)
+UNROLL = 16  # frames per graph launch (processed one after the other)
 
 
 def launch_plan(steps, warmup, unroll=UNROLL):
