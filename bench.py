@@ -317,6 +317,35 @@ def _row_report(rows):
     return out
 
 
+def dense_library_conv_us(batch, cin, cout, k, h, w, groups=1, reps=30):
+    """Device time of the vendor library's DENSE convolution of the same shape (PyTorch -> MIOpen, fp16,
+    channels-last, `reps` calls replayed from one HIP graph): what the delta kernels are up against on the
+    same GPU, reported beside their own times."""
+    import torch
+    x = torch.randn(batch, cin, h, w, device="cuda", dtype=torch.half).contiguous(memory_format=torch.channels_last)
+    wt = torch.randn(cout, cin // groups, k, k, device="cuda", dtype=torch.half).contiguous(memory_format=torch.channels_last)
+    fn = lambda: torch.nn.functional.conv2d(x, wt, padding=k // 2, groups=groups)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.no_grad(), torch.cuda.stream(side):
+        for _ in range(3):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.no_grad(), torch.cuda.graph(graph):
+        for _ in range(reps):
+            fn()
+    graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return round(e0.elapsed_time(e1) / reps * 1e3, 2)
+
+
 def micro_bench():
     """Single-layer sweeps on a 64x64 fp16 map: 3x3 256->256, 1x1 256->1024 and depthwise 3x3
     C=512, each followed by ReLU with truncation (threshold 0.05), update density 1..100 %.
@@ -336,6 +365,8 @@ def micro_bench():
         prev = torch.randn(1, cout, H, W, generator=gen).half().cuda().contiguous(memory_format=torch.channels_last)
         trunc = torch.zeros_like(prev)
         obuf, omask = torch.zeros_like(prev), torch.zeros(1, 1, H, W, dtype=torch.int32, device="cuda")
+        dense_us = dense_library_conv_us(1, cin, cout, k, H, W, groups)
+        log(f"  micro {name:18s} dense library convolution (no activation): {dense_us:.2f} us")
         for rho in SWEEP:
             n = max(1, round(rho * H * W))
             mask = torch.zeros(H * W, dtype=torch.int32)
@@ -347,7 +378,7 @@ def micro_bench():
                 x, filt, mask, None, prev, trunc, THRESHOLD, 1, 0, (1, 1), (k // 2, k // 2), (1, 1), groups, cout,
                 packed_filter=packed, out=obuf, out_mask=omask))
             out.append({"op": name, "density": rho, "us": round(sum(r["ms"] for r in rows) * 1e3, 3),
-                        "kernels": _row_report(rows)})
+                        "dense_library_conv_us": dense_us, "kernels": _row_report(rows)})
             log(f"  micro {name:18s} density {rho:4.2f}: " +
                 "  ".join(f"{r['kernel']} {r['us']:.2f} us {r['alg_GBps'] or 0:.0f} GB/s {r['alg_TFLOPs'] or 0:.1f} TF/s"
                           for r in out[-1]["kernels"]))
@@ -379,6 +410,9 @@ def scaled_bench():
     wpw_packed = hk.pack_filter(wpw, C, C, 1)
     w33 = convert_half_filter((torch.randn(C, C, 3, 3, generator=torch.Generator().manual_seed(9)) / (9 * C) ** 0.5).half()).cuda()
     w33_packed = hk.pack_filter(w33, C, C, 1)
+    dense_us = {"conv3x3_64->64": dense_library_conv_us(B, C, C, 3, H, W, reps=10),
+                "pointwise64->64": dense_library_conv_us(B, C, C, 1, H, W, reps=10),
+                "depthwise3x3+relu": dense_library_conv_us(B, C, C, 3, H, W, groups=C, reps=10)}
     for rho in (0.1, 1.0):
         mask = (torch.rand(B, 1, H, W, device="cuda", generator=gen) < rho).to(torch.int32)
         mask2 = mask.clone()
@@ -413,6 +447,9 @@ def scaled_bench():
             rows = _trace_calls(fn, alt_inputs=[a.data_ptr(), d.data_ptr()])
             rep = _row_report(rows)
             out.append({"op": name, "density": rho, "kernels": rep})
+            if name in dense_us:  # the vendor library's dense convolution of the same shape (without the activation)
+                out[-1]["dense_library_conv_us"] = dense_us[name]
+                log(f"  scaled {name:20s} dense library convolution: {dense_us[name]:.1f} us")
             log(f"  scaled {name:20s} density {rho:4.2f}: " +
                 "  ".join(f"{r['kernel']} {r['us']:.1f} us {r['alg_GBps'] or 0:.0f} GB/s ({100 * (r['hbm_frac'] or 0):.1f} % of HBM peak"
                           + (f", {100 * (r['mfma_frac'] or 0):.1f} % of the MFMA peak)" if (r['alg_TFLOPs'] or 0) >= 50 else ")")
